@@ -1,0 +1,65 @@
+"""ctypes binding of libfaith_amd.so (the C ABI declared in include/faith_amd.h).
+
+There is no fallback: if the library is missing or a symbol is absent, import
+of this module raises.  Build it with ``python -m faith_amd.build``.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libfaith_amd.so")
+
+OK = 0
+Q_1, Q_2, Q_INF = 1, 2, 0
+LAYOUT_NATURAL, LAYOUT_TRANSPOSED = 0, 1
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+
+# name -> argument types, in the order of include/faith_amd.h
+SIGNATURES = {
+    "faith_concretize": [_P] * 6 + [_I, _I, _I, _F, _I, _I, _I, _P],
+    "faith_relu_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
+    "faith_tanh_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
+    "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],
+    "faith_dot_product_verification_QK": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
+    "faith_convolution_verification": [_P] * 10 + [_I] * 9 + [_P],
+}
+
+
+class FaithError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+    def __init__(self, fn, code, msg):
+        super().__init__(f"{fn} failed with status {code}: {msg}")
+        self.code = code
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: the HIP library is not built "
+            "(run `python -m faith_amd.build`); there is no CPU fallback")
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.faith_last_error.restype = ctypes.c_char_p
+    lib.faith_last_error.argtypes = []
+    lib.faith_version.restype = _I
+    lib.faith_version.argtypes = []
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is missing
+        fn.restype = _I
+        fn.argtypes = argtypes
+    return lib
+
+
+lib = _load()
+
+
+def call(name, *args):
+    """Invoke an entry point; raise FaithError on a non-zero status."""
+    rc = getattr(lib, name)(*args)
+    if rc != OK:
+        raise FaithError(name, rc, lib.faith_last_error().decode())

@@ -1,0 +1,107 @@
+"""`Bounds`: the reference's operator surface for forward bound propagation, on HIP.
+
+Mirrors the constructor and the method names / return conventions of the
+reference class (Transformer_Verification_Code/Verifiers/Bounds.py:270-297) for
+the methods on the accelerated path:
+
+    concretize   Bounds.py:319-326        relu        :1163-1169 (ori_relu :921-963)
+    matmul       :1177-1199 (ori_matmul :397-413)     tanh        :1171-1175 (ori_tanh :1027-1103)
+    dense        :1016-1025               dot_product :833-841 (ori_dot_product :710-823)
+    add          :383-395                 conv2d      HandTunedKernels/convolution_verification.cu:219-239
+
+Every method launches hand-written HIP kernels through the C ABI; none has a
+PyTorch fallback.  Known defects of the reference are not reproduced: `dense`
+is `matmul(weight).add(bias)` (the reference line raises NameError), and the
+dot product uses the true upper constant term (the reference's CUDA adapter
+overwrites ub with lb, Bounds.py:1286).
+"""
+from __future__ import annotations
+
+from types import SimpleNamespace
+
+import torch
+
+from . import ops
+
+
+class Bounds:
+    def __init__(self, args, p, eps, w=None, b=None, lw=None, lb=None, uw=None, ub=None, clone=True):
+        self.args = args if args is not None else SimpleNamespace(perturbed_words=1)
+        self.p = p
+        self.eps = eps
+        self.perturbed_words = getattr(self.args, "perturbed_words", 1)
+        self.lw = lw if lw is not None else (w.clone() if clone else w)
+        self.uw = uw if uw is not None else (w.clone() if clone else w)
+        self.lb = lb if lb is not None else (b.clone() if clone else b)
+        self.ub = ub if ub is not None else (b.clone() if clone else b)
+        self.device = self.lw.device
+        self.update_shape()
+
+    def update_shape(self):
+        self.batch_size, self.length, self.dim_in, self.dim_out = self.lw.shape[:4]
+
+    def _like(self, lw, lb, uw, ub):
+        return Bounds(self.args, self.p, self.eps, lw=lw, lb=lb, uw=uw, ub=ub)
+
+    def _c(self):
+        return (self.lw.contiguous(), self.lb.contiguous(), self.uw.contiguous(), self.ub.contiguous())
+
+    # ---- Bounds.py:319-326
+    def concretize(self):
+        lw, lb, uw, ub = self._c()
+        return ops.concretize(lw, lb, uw, ub, self.p, self.eps, self.perturbed_words)
+
+    # ---- Bounds.py:383-395
+    def add(self, delta):
+        if isinstance(delta, Bounds):
+            return self._like(self.lw + delta.lw, self.lb + delta.lb, self.uw + delta.uw, self.ub + delta.ub)
+        return self._like(self.lw, self.lb + delta, self.uw, self.ub + delta)
+
+    # ---- Bounds.py:397-413, :1177-1199
+    def matmul(self, W, bias=None):
+        if isinstance(W, Bounds):
+            raise NotImplementedError("matmul with a Bounds operand is dot_product")
+        if W.dim() != 2:
+            raise NotImplementedError("only a 2-D weight has a kernel")
+        lw, lb, uw, ub = self._c()
+        return self._like(*ops.linear(lw, lb, uw, ub, W.contiguous(), bias))
+
+    # ---- Bounds.py:1016-1025 (bias fused into the same launch)
+    def dense(self, dense):
+        bias = getattr(dense, "bias", None)
+        return self.matmul(dense.weight.detach(), None if bias is None else bias.detach().contiguous())
+
+    # ---- Bounds.py:1163-1175
+    def relu(self):
+        return self._like(*ops.relu(*self._c(), self.p, self.eps, self.perturbed_words))
+
+    def tanh(self):
+        return self._like(*ops.tanh(*self._c(), self.p, self.eps, self.perturbed_words))
+
+    def act(self, act_name):
+        if act_name == "relu":
+            return self.relu()
+        if act_name == "tanh":
+            return self.tanh()
+        raise NotImplementedError(act_name)
+
+    # ---- Bounds.py:833-841 (scores path: self = query, other = key)
+    def dot_product(self, other):
+        return self._like(*ops.dot_product_qk(self._c(), other._c(), self.p, self.eps, self.perturbed_words))
+
+
+class ConvBounds:
+    """Bounds of an image-shaped activation: lw, uw [1, D_in, C, H, W]; lb, ub [1, C, H, W]."""
+
+    def __init__(self, p, eps, lw, lb, uw, ub):
+        self.p, self.eps = p, eps
+        self.lw, self.lb, self.uw, self.ub = lw, lb, uw, ub
+
+    def conv2d(self, weight, bias=None, stride=1, padding=0):
+        out = ops.conv2d(self.lw.contiguous(), self.lb.contiguous(), self.uw.contiguous(), self.ub.contiguous(),
+                         weight.contiguous(), bias, stride, padding)
+        return ConvBounds(self.p, self.eps, *out)
+
+    def concretize(self):
+        return ops.concretize_conv(self.lw.contiguous(), self.lb.contiguous(), self.uw.contiguous(),
+                                   self.ub.contiguous(), self.p, self.eps)

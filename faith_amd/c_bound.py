@@ -1,0 +1,94 @@
+"""Drop-in for the reference's pybind module (HandTunedKernels/kernel.cpp:297-304).
+
+Same function names, argument order and in-place output convention as the
+module the reference loads as ``c_bound`` (Bounds.py:14-26), so its
+``Bounds.cuda_*`` adapters (Bounds.py:1201-1343) can call this module
+unchanged.  As there, lw / uw arrive transposed ([.., dim_out, dim_in]) and
+every output tensor is pre-allocated by the caller.
+
+Two differences from the reference kernels, both towards the PyTorch
+semantics they were meant to reproduce: the dual norm follows ``p`` (module
+attribute, default 2; the CUDA kernels hard-wire q = 2) and ``words`` blocks
+are honoured.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib, ops
+from ._lib import LAYOUT_TRANSPOSED
+
+p = 2.0        # perturbation norm used by the calls below
+words = 1      # perturbed_words
+
+
+def _s(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _act(entry, src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw, length, dim_in, dim_out, epsilon):
+    for n, t in (("src_lb", src_lb), ("src_ub", src_ub), ("src_lw", src_lw), ("src_uw", src_uw),
+                 ("out_lb", out_lb), ("out_ub", out_ub), ("out_lw", out_lw), ("out_uw", out_uw)):
+        ops._check(n, t)
+    if src_lw.numel() != length * dim_in * dim_out or src_lb.numel() != length * dim_out:
+        raise ValueError("tensor sizes do not match length * dim_in * dim_out (batch must be 1)")
+    with torch.cuda.device(src_lw.device):
+        _lib.call(entry, src_lb.data_ptr(), src_ub.data_ptr(), src_lw.data_ptr(), src_uw.data_ptr(),
+                  out_lb.data_ptr(), out_ub.data_ptr(), out_lw.data_ptr(), out_uw.data_ptr(), None, None,
+                  length, dim_in, dim_out, float(epsilon), ops.q_code(p), words, LAYOUT_TRANSPOSED, _s(src_lw))
+
+
+def c_relu_verification(src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw,
+                        length, dim_in, dim_out, epsilon):
+    """kernel.cpp:69-99."""
+    _act("faith_relu_verification", src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw,
+         length, dim_in, dim_out, epsilon)
+
+
+def c_tanh_verification(src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw,
+                        length, dim_in, dim_out, epsilon):
+    """kernel.cpp:101-131."""
+    _act("faith_tanh_verification", src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw,
+         length, dim_in, dim_out, epsilon)
+
+
+def c_dot_product_verification_QK(x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
+                                  z_lb, z_ub, z_lw, z_uw, batch_size, length, dim_out, dim_in, epsilon):
+    """kernel.cpp:133-186.  x_lw .. y_uw are [B, L, dim_out, dim_in]; z_lw, z_uw are [B, L, L, dim_in].
+
+    The contraction kernel works on the natural layout, so this compatibility entry
+    re-lays the transposed operands out with torch copies before and after the call;
+    callers that keep the natural layout (faith_amd.Bounds) pay none of that.
+    """
+    nat = [t.transpose(2, 3).contiguous() for t in (x_lw, x_uw, y_lw, y_uw)]
+    zlw, zlb, zuw, zub, (xl, xu, yl, yu) = ops.dot_product_qk(
+        (nat[0], x_lb.contiguous(), nat[1], x_ub.contiguous()),
+        (nat[2], y_lb.contiguous(), nat[3], y_ub.contiguous()),
+        p, epsilon, words, return_intervals=True)
+    z_lw.copy_(zlw.transpose(2, 3)); z_uw.copy_(zuw.transpose(2, 3))
+    z_lb.copy_(zlb); z_ub.copy_(zub)
+    x_l.copy_(xl); x_u.copy_(xu); y_l.copy_(yl); y_u.copy_(yu)
+
+
+def c_matmul_verification(x_lb, x_ub, x_lw, x_uw, W, y_lb, y_ub, y_lw, y_uw,
+                          batch_size, length, dim_in, dim_out, dim_y_out):
+    """kernel.cpp:243-266 (commented out there; natural layout, no bias)."""
+    for n, t in (("x_lb", x_lb), ("x_ub", x_ub), ("x_lw", x_lw), ("x_uw", x_uw), ("W", W),
+                 ("y_lb", y_lb), ("y_ub", y_ub), ("y_lw", y_lw), ("y_uw", y_uw)):
+        ops._check(n, t)
+    with torch.cuda.device(x_lw.device):
+        _lib.call("faith_matmul_verification", x_lb.data_ptr(), x_ub.data_ptr(), x_lw.data_ptr(), x_uw.data_ptr(),
+                  W.data_ptr(), None, y_lb.data_ptr(), y_ub.data_ptr(), y_lw.data_ptr(), y_uw.data_ptr(),
+                  batch_size, length, dim_in, dim_out, dim_y_out, _s(x_lw))
+
+
+def c_convolution_verification(x_lb, x_ub, x_lw, x_uw, W, y_lb, y_ub, y_lw, y_uw,
+                               batch_size, Height, Width, CIN, COUT, K, Stride, padding_size, dim_in):
+    """kernel.cpp:268-295 (commented out there)."""
+    for n, t in (("x_lb", x_lb), ("x_ub", x_ub), ("x_lw", x_lw), ("x_uw", x_uw), ("W", W),
+                 ("y_lb", y_lb), ("y_ub", y_ub), ("y_lw", y_lw), ("y_uw", y_uw)):
+        ops._check(n, t)
+    with torch.cuda.device(x_lw.device):
+        _lib.call("faith_convolution_verification", x_lb.data_ptr(), x_ub.data_ptr(), x_lw.data_ptr(),
+                  x_uw.data_ptr(), W.data_ptr(), None, y_lb.data_ptr(), y_ub.data_ptr(), y_lw.data_ptr(),
+                  y_uw.data_ptr(), batch_size, Height, Width, CIN, COUT, K, Stride, padding_size, dim_in, _s(x_lw))

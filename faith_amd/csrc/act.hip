@@ -1,0 +1,488 @@
+// Concretization and the ReLU / tanh relaxations, each as ONE pass over HBM.
+//
+// Arithmetic follows the reference's PyTorch Bounds methods
+// (Transformer_Verification_Code/Verifiers/Bounds.py:311-326 concretize, :348-381 new /
+// add_linear, :921-963 ori_relu, :1027-1103 ori_tanh), not its CUDA kernels, which hard-wire
+// q = 2 and differ at the branch boundaries.
+//
+// Natural layout [rows, D_in, H] (the layout the reference's Python keeps its tensors in):
+//   a workgroup owns one row r and a tile of TH neighbouring neurons.  Lanes run along H, so
+//   every global access is a run of TH*4 contiguous bytes; the D_in rows of the tile are spread
+//   over the workgroup's threads and stay in registers between the norm reduction and the
+//   scaling, so lw / uw are read once and lw' / uw' written once.
+//   Per thread: partial q-norms of its rows -> LDS -> one thread per neuron finishes the norm,
+//   forms [l, u], derives the two lines (slope k, anchor x0, offset y0) -> LDS -> every thread
+//   scales what it holds and stores it.
+//
+// Transposed layout [rows, H, D_in] (what the reference's CUDA adapters hand over,
+// Bounds.py:1210-1211): D_in is contiguous, a wavefront owns a neuron and reduces with
+// cross-lane shuffles.
+//
+// This file is built with -ffp-contract=off: the reference rounds (b - x0) * k and the
+// following + y0 separately, and l = lb + (-eps * norm) likewise.
+#include "common.h"
+
+namespace {
+
+constexpr int WAVE = 64;
+constexpr float TINY = 1e-12f;   // Bounds.py:27
+
+enum Mode { CONCRETIZE = 0, RELU = 1, TANH = 2 };
+
+struct ActArgs {
+    const float *lb, *ub, *lw, *uw;
+    float *olb, *oub, *olw, *ouw;
+    float *l, *u;
+    int rows, D, H, words;
+    float eps;
+};
+
+// y = k * (v - x0) + y0
+struct Line {
+    float k, x0, y0;
+};
+
+// ------------------------------------------------------------------ q-norm pieces
+template <int Q>
+__device__ __forceinline__ float nacc(float acc, float v) {
+    if (Q == FAITH_Q_2) return acc + v * v;
+    if (Q == FAITH_Q_1) return acc + fabsf(v);
+    return fmaxf(acc, fabsf(v));
+}
+template <int Q>
+__device__ __forceinline__ float ncomb(float a, float b) {
+    return Q == FAITH_Q_INF ? fmaxf(a, b) : a + b;
+}
+template <int Q>
+__device__ __forceinline__ float nfin(float a) {
+    return Q == FAITH_Q_2 ? sqrtf(a) : a;
+}
+
+// ------------------------------------------------------------------ the relaxations
+// Bounds.py:921-963.  Strict comparisons: l == 0 or u == 0 is a straddling neuron.
+__device__ __forceinline__ void relu_lines(float l, float u, Line &lo, Line &up) {
+    if (u < 0.f) {
+        lo = {0.f, 0.f, 0.f};
+        up = {0.f, 0.f, 0.f};
+    } else if (l > 0.f) {
+        lo = {1.f, 0.f, 0.f};
+        up = {1.f, 0.f, 0.f};
+    } else {
+        up = {u / ((u - l) + TINY), l, 0.f};
+        lo = {fabsf(u) > fabsf(l) ? 1.f : 0.f, 0.f, 0.f};
+    }
+}
+
+// 1 / cosh^2 in double.
+__device__ __forceinline__ double sech2(double x) {
+    const double c = cosh(x);
+    return 1.0 / (c * c);
+}
+
+// Bounds.py:1027-1097.  Interval end points, bisection state and the results are fp32 as in
+// the reference; tanh / cosh and the quotients are evaluated in double and rounded once, so
+// that the only disagreement with an fp32 library left is that library's own rounding.
+__device__ void tanh_lines(float l, float u, Line &lo, Line &up) {
+    const double tl = tanh((double)l), tu = tanh((double)u);
+    if (u < 0.f || l > 0.f) {
+        const float m = (l + u) / 2;
+        const Line tangent = {(float)sech2((double)m), m, (float)tanh((double)m)};
+        const Line chord = {(float)((tu - tl) / (double)((u - l) + TINY)), l, (float)tl};
+        if (u < 0.f) {
+            lo = tangent;
+            up = chord;
+        } else {
+            lo = chord;
+            up = tangent;
+        }
+        return;
+    }
+    {   // lower line: tangent point d in [l, 0] whose tangent passes through (u, tanh u)
+        float d = l / 2, a = l, b = 0.f;
+        for (int it = 0; it < 10; ++it) {
+            const double v = (tu - tanh((double)d)) / (double)((u - d) + TINY) - sech2((double)d);
+            if (v > 0) {
+                a = d;
+                d = (d + b) / 2;
+            } else {
+                b = d;
+                d = (d + a) / 2;
+            }
+        }
+        const double td = tanh((double)d);
+        lo = {(float)((td - tu) / (double)((d - u) + TINY)), d, (float)td};
+    }
+    {   // upper line: tangent point d in [0, u] whose tangent passes through (l, tanh l)
+        float d = u / 2, a = 0.f, b = u;
+        for (int it = 0; it < 10; ++it) {
+            const double v = (tanh((double)d) - tl) / (double)((d - l) + TINY) - sech2((double)d);
+            if (v > 0) {
+                b = d;
+                d = (d + a) / 2;
+            } else {
+                a = d;
+                d = (d + b) / 2;
+            }
+        }
+        const double td = tanh((double)d);
+        up = {(float)((td - tl) / (double)((d - l) + TINY)), d, (float)td};
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void make_lines(float l, float u, Line &lo, Line &up) {
+    if (MODE == RELU)
+        relu_lines(l, u, lo, up);
+    else
+        tanh_lines(l, u, lo, up);
+}
+
+// Bounds.add_linear, constant term (Bounds.py:378, :381): a positive slope takes the same-side
+// bound, a non-positive one the opposite bound; three separate roundings.
+__device__ __forceinline__ float line_bias(const Line &ln, float same, float other) {
+    const float b = ln.k > 0.f ? same : other;
+    return (b - ln.x0) * ln.k + ln.y0;
+}
+
+// ------------------------------------------------------------------ vector access
+template <int VEC>
+struct Vec;
+template <>
+struct Vec<4> {
+    float4 v;
+    __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
+    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
+    __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
+    __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+    __device__ __forceinline__ void set(int i, float f) {
+        if (i == 0) v.x = f;
+        else if (i == 1) v.y = f;
+        else if (i == 2) v.z = f;
+        else v.w = f;
+    }
+};
+template <>
+struct Vec<1> {
+    float v;
+    __device__ __forceinline__ void load(const float *p) { v = *p; }
+    __device__ __forceinline__ void store(float *p) const { *p = v; }
+    __device__ __forceinline__ void zero() { v = 0.f; }
+    __device__ __forceinline__ float get(int) const { return v; }
+    __device__ __forceinline__ void set(int, float f) { v = f; }
+};
+
+// ------------------------------------------------------------------ natural layout
+// TPR threads cover one row of the tile (TH = TPR * VEC neurons); RG = NTHREADS / TPR rows are
+// in flight per step; a thread keeps RPT rows.  D_in <= RG * RPT is the register-resident case;
+// larger D_in is walked in chunks and read a second time for the scaling.
+template <int MODE, int Q, int VEC, int TPR, int NTHREADS, int RPT>
+__global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
+    constexpr int TH = TPR * VEC;
+    constexpr int RG = NTHREADS / TPR;
+    static_assert(TH <= NTHREADS, "one thread per neuron must exist");
+    extern __shared__ float smem[];
+    float *part = smem;                          // [words][RG][2][TH]
+    float *coef = smem + a.words * RG * 2 * TH;  // [2][TH] slopes
+
+    const int tiles = (a.H + TH - 1) / TH;
+    const int r = blockIdx.x / tiles;
+    const int col0 = (blockIdx.x % tiles) * TH;
+    const int tid = threadIdx.x;
+    const int c = tid % TPR, rg = tid / TPR;
+    const int col = col0 + c * VEC;
+    const bool col_ok = col < a.H;
+    const size_t base = (size_t)r * a.D * a.H + col;
+    const int blk = a.D / a.words;
+    constexpr int CHUNK = RG * RPT;
+    const int nchunks = (a.D + CHUNK - 1) / CHUNK;
+
+    Vec<VEC> dl[RPT], du[RPT];
+
+    for (int w = 0; w < a.words; ++w)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            part[((w * RG + rg) * 2 + 0) * TH + c * VEC + v] = 0.f;
+            part[((w * RG + rg) * 2 + 1) * TH + c * VEC + v] = 0.f;
+        }
+
+    for (int ch = 0; ch < nchunks; ++ch) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            const int row = ch * CHUNK + i * RG + rg;
+            if (col_ok && row < a.D) {
+                dl[i].load(a.lw + base + (size_t)row * a.H);
+                du[i].load(a.uw + base + (size_t)row * a.H);
+            } else {
+                dl[i].zero();
+                du[i].zero();
+            }
+        }
+        for (int w = 0; w < a.words; ++w) {
+            const int lo_row = w * blk, hi_row = lo_row + blk;
+            float pl[VEC], pu[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                const int row = ch * CHUNK + i * RG + rg;
+                if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        pl[v] = nacc<Q>(pl[v], dl[i].get(v));
+                        pu[v] = nacc<Q>(pu[v], du[i].get(v));
+                    }
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                float *sl = &part[((w * RG + rg) * 2 + 0) * TH + c * VEC + v];
+                float *su = &part[((w * RG + rg) * 2 + 1) * TH + c * VEC + v];
+                *sl = ncomb<Q>(*sl, pl[v]);
+                *su = ncomb<Q>(*su, pu[v]);
+            }
+        }
+    }
+    __syncthreads();
+
+    // one thread per neuron: finish the norms, concretize, derive the lines
+    if (tid < TH) {
+        const int column = col0 + tid;
+        if (column < a.H) {
+            const size_t bi = (size_t)r * a.H + column;
+            const float lb = a.lb[bi], ub = a.ub[bi];
+            float l = lb, u = ub;
+            for (int w = 0; w < a.words; ++w) {
+                float nl = 0.f, nu = 0.f;
+                for (int g = 0; g < RG; ++g) {
+                    nl = ncomb<Q>(nl, part[((w * RG + g) * 2 + 0) * TH + tid]);
+                    nu = ncomb<Q>(nu, part[((w * RG + g) * 2 + 1) * TH + tid]);
+                }
+                l += (-a.eps) * nfin<Q>(nl);
+                u += a.eps * nfin<Q>(nu);
+            }
+            if (a.l) a.l[bi] = l;
+            if (a.u) a.u[bi] = u;
+            if (MODE != CONCRETIZE) {
+                Line lo, up;
+                make_lines<MODE>(l, u, lo, up);
+                coef[tid] = lo.k;
+                coef[TH + tid] = up.k;
+                a.olb[bi] = line_bias(lo, lb, ub);
+                a.oub[bi] = line_bias(up, ub, lb);
+            }
+        }
+    }
+    if (MODE == CONCRETIZE) return;
+    __syncthreads();
+
+    if (!col_ok) return;
+    float klo[VEC], kup[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        klo[v] = coef[c * VEC + v];
+        kup[v] = coef[TH + c * VEC + v];
+    }
+    for (int ch = 0; ch < nchunks; ++ch) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            const int row = ch * CHUNK + i * RG + rg;
+            if (row < a.D) {
+                const size_t off = base + (size_t)row * a.H;
+                if (nchunks > 1) {
+                    dl[i].load(a.lw + off);
+                    du[i].load(a.uw + off);
+                }
+                Vec<VEC> ol, ou;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    const float xl = dl[i].get(v), xu = du[i].get(v);
+                    ol.set(v, (klo[v] > 0.f ? xl : xu) * klo[v]);
+                    ou.set(v, (kup[v] > 0.f ? xu : xl) * kup[v]);
+                }
+                ol.store(a.olw + off);
+                ou.store(a.ouw + off);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ transposed layout
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
+    return v;
+}
+
+// 256 threads, 64 neurons per workgroup: each wavefront reduces 16 neurons (lanes along D_in,
+// cross-lane butterfly), wavefront 0 then derives the 64 pairs of lines (one neuron per lane),
+// and each wavefront scales its 16 neurons (second read comes from L2).
+template <int MODE, int Q>
+__global__ void __launch_bounds__(256) act_transposed(const ActArgs a) {
+    constexpr int NPB = 64, NPW = NPB / 4;
+    __shared__ float s_l[NPB], s_u[NPB], s_klo[NPB], s_kup[NPB];
+    const long long total = (long long)a.rows * a.H;
+    const long long n0 = (long long)blockIdx.x * NPB;
+    const int lane = threadIdx.x % WAVE, wv = threadIdx.x / WAVE;
+    const int blk = a.D / a.words;
+
+    for (int i = 0; i < NPW; ++i) {
+        const int t = wv * NPW + i;
+        const long long n = n0 + t;
+        if (n >= total) break;
+        const float *pl = a.lw + (size_t)n * a.D, *pu = a.uw + (size_t)n * a.D;
+        float l = a.lb[n], u = a.ub[n];
+        for (int w = 0; w < a.words; ++w) {
+            float nl = 0.f, nu = 0.f;
+            for (int k = w * blk + lane; k < (w + 1) * blk; k += WAVE) {
+                nl = nacc<Q>(nl, pl[k]);
+                nu = nacc<Q>(nu, pu[k]);
+            }
+            nl = Q == FAITH_Q_INF ? wave_max(nl) : wave_sum(nl);
+            nu = Q == FAITH_Q_INF ? wave_max(nu) : wave_sum(nu);
+            l += (-a.eps) * nfin<Q>(nl);
+            u += a.eps * nfin<Q>(nu);
+        }
+        if (lane == 0) {
+            s_l[t] = l;
+            s_u[t] = u;
+            if (a.l) a.l[n] = l;
+            if (a.u) a.u[n] = u;
+        }
+    }
+    if (MODE == CONCRETIZE) return;
+    __syncthreads();
+    if (threadIdx.x < NPB && n0 + threadIdx.x < total) {
+        const long long n = n0 + threadIdx.x;
+        Line lo, up;
+        make_lines<MODE>(s_l[threadIdx.x], s_u[threadIdx.x], lo, up);
+        s_klo[threadIdx.x] = lo.k;
+        s_kup[threadIdx.x] = up.k;
+        const float lb = a.lb[n], ub = a.ub[n];
+        a.olb[n] = line_bias(lo, lb, ub);
+        a.oub[n] = line_bias(up, ub, lb);
+    }
+    __syncthreads();
+    for (int i = 0; i < NPW; ++i) {
+        const int t = wv * NPW + i;
+        const long long n = n0 + t;
+        if (n >= total) break;
+        const float klo = s_klo[t], kup = s_kup[t];
+        const size_t off = (size_t)n * a.D;
+        for (int k = lane; k < a.D; k += WAVE) {
+            const float xl = a.lw[off + k], xu = a.uw[off + k];
+            a.olw[off + k] = (klo > 0.f ? xl : xu) * klo;
+            a.ouw[off + k] = (kup > 0.f ? xu : xl) * kup;
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host dispatch
+template <int MODE, int Q, int VEC, int TPR, int NTHREADS, int RPT>
+void launch_natural(const ActArgs &a, hipStream_t st) {
+    constexpr int TH = TPR * VEC, RG = NTHREADS / TPR;
+    const int tiles = (a.H + TH - 1) / TH;
+    const size_t smem = ((size_t)a.words * RG * 2 * TH + 2 * TH) * sizeof(float);
+    hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles)),
+                       dim3(NTHREADS), smem, st, a);
+}
+
+template <int MODE, int Q>
+void dispatch_natural(const ActArgs &a, hipStream_t st) {
+    const bool vec4 = (a.H % 4 == 0) && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
+                      (MODE == CONCRETIZE || (faith::aligned(a.olw, 16) && faith::aligned(a.ouw, 16)));
+    if (MODE == CONCRETIZE) {
+        // nothing is kept: short chunks, many loads in flight
+        if (vec4)
+            launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);
+        else
+            launch_natural<MODE, Q, 1, 64, 256, 8>(a, st);
+        return;
+    }
+    if (!vec4) {
+        launch_natural<MODE, Q, 1, 64, 256, 16>(a, st);   // 64 neurons x 64 rows per chunk
+    } else if (a.D <= 128) {
+        launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);    // 64 neurons, D_in <= 128 in registers
+    } else if (a.D <= 256) {
+        launch_natural<MODE, Q, 4, 16, 256, 16>(a, st);   // D_in <= 256 in registers
+    } else {
+        launch_natural<MODE, Q, 4, 16, 512, 16>(a, st);   // D_in <= 512 in registers, chunks beyond
+    }
+}
+
+template <int MODE, int Q>
+void dispatch_layout(const ActArgs &a, int layout, hipStream_t st) {
+    if (layout == FAITH_LAYOUT_NATURAL) {
+        dispatch_natural<MODE, Q>(a, st);
+    } else {
+        const long long total = (long long)a.rows * a.H;
+        hipLaunchKernelGGL((act_transposed<MODE, Q>), dim3((unsigned)((total + 63) / 64)), dim3(256), 0, st, a);
+    }
+}
+
+template <int MODE>
+int run(const char *who, ActArgs a, int q, int layout, void *stream) {
+    FAITH_REQUIRE(a.rows > 0 && a.D > 0 && a.H > 0, FAITH_ERR_SHAPE,
+                  "%s: rows=%d dim_in=%d dim_out=%d must all be positive", who, a.rows, a.D, a.H);
+    FAITH_REQUIRE(a.words >= 1 && a.words <= 16 && a.D % a.words == 0, FAITH_ERR_SHAPE,
+                  "%s: words=%d must be in 1..16 and divide dim_in=%d", who, a.words, a.D);
+    FAITH_REQUIRE(q == FAITH_Q_1 || q == FAITH_Q_2 || q == FAITH_Q_INF, FAITH_ERR_UNSUPPORTED,
+                  "%s: q=%d is not one of FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF", who, q);
+    FAITH_REQUIRE(layout == FAITH_LAYOUT_NATURAL || layout == FAITH_LAYOUT_TRANSPOSED, FAITH_ERR_UNSUPPORTED,
+                  "%s: unknown layout %d", who, layout);
+    FAITH_REQUIRE((long long)a.rows * a.H * 1LL <= 0x7fffffffLL * 32, FAITH_ERR_SHAPE, "%s: problem too large", who);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (q) {
+        case FAITH_Q_1: dispatch_layout<MODE, FAITH_Q_1>(a, layout, st); break;
+        case FAITH_Q_2: dispatch_layout<MODE, FAITH_Q_2>(a, layout, st); break;
+        default: dispatch_layout<MODE, FAITH_Q_INF>(a, layout, st); break;
+    }
+    return faith::check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int faith_concretize(const float *lb, const float *ub, const float *lw, const float *uw, float *l,
+                                float *u, int rows, int dim_in, int dim_out, float eps, int q, int words,
+                                int layout, void *stream) {
+    FAITH_NOT_NULL(lb); FAITH_NOT_NULL(ub); FAITH_NOT_NULL(lw); FAITH_NOT_NULL(uw);
+    FAITH_NOT_NULL(l); FAITH_NOT_NULL(u);
+    FAITH_ALIGNED4(lb); FAITH_ALIGNED4(ub); FAITH_ALIGNED4(lw); FAITH_ALIGNED4(uw);
+    FAITH_ALIGNED4(l); FAITH_ALIGNED4(u);
+    ActArgs a{lb, ub, lw, uw, nullptr, nullptr, nullptr, nullptr, l, u, rows, dim_in, dim_out, words, eps};
+    return run<CONCRETIZE>("faith_concretize", a, q, layout, stream);
+}
+
+static int act_entry(const char *who, int mode, const float *src_lb, const float *src_ub, const float *src_lw,
+                     const float *src_uw, float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                     float *l_out, float *u_out, int length, int dim_in, int dim_out, float epsilon, int q,
+                     int words, int layout, void *stream) {
+    FAITH_NOT_NULL(src_lb); FAITH_NOT_NULL(src_ub); FAITH_NOT_NULL(src_lw); FAITH_NOT_NULL(src_uw);
+    FAITH_NOT_NULL(out_lb); FAITH_NOT_NULL(out_ub); FAITH_NOT_NULL(out_lw); FAITH_NOT_NULL(out_uw);
+    FAITH_ALIGNED4(src_lb); FAITH_ALIGNED4(src_ub); FAITH_ALIGNED4(src_lw); FAITH_ALIGNED4(src_uw);
+    FAITH_ALIGNED4(out_lb); FAITH_ALIGNED4(out_ub); FAITH_ALIGNED4(out_lw); FAITH_ALIGNED4(out_uw);
+    FAITH_ALIGNED4(l_out); FAITH_ALIGNED4(u_out);
+    ActArgs a{src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw, l_out, u_out,
+              length, dim_in, dim_out, words, epsilon};
+    return mode == RELU ? run<RELU>(who, a, q, layout, stream) : run<TANH>(who, a, q, layout, stream);
+}
+
+extern "C" int faith_relu_verification(const float *src_lb, const float *src_ub, const float *src_lw,
+                                       const float *src_uw, float *out_lb, float *out_ub, float *out_lw,
+                                       float *out_uw, float *l_out, float *u_out, int length, int dim_in,
+                                       int dim_out, float epsilon, int q, int words, int layout, void *stream) {
+    return act_entry("faith_relu_verification", RELU, src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw,
+                     out_uw, l_out, u_out, length, dim_in, dim_out, epsilon, q, words, layout, stream);
+}
+
+extern "C" int faith_tanh_verification(const float *src_lb, const float *src_ub, const float *src_lw,
+                                       const float *src_uw, float *out_lb, float *out_ub, float *out_lw,
+                                       float *out_uw, float *l_out, float *u_out, int length, int dim_in,
+                                       int dim_out, float epsilon, int q, int words, int layout, void *stream) {
+    return act_entry("faith_tanh_verification", TANH, src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw,
+                     out_uw, l_out, u_out, length, dim_in, dim_out, epsilon, q, words, layout, stream);
+}

@@ -1,0 +1,34 @@
+// Shared host-side helpers of the C ABI: status codes, error text, launch checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/faith_amd.h"
+
+namespace faith {
+
+// Thread-local message behind faith_last_error().
+void set_error(const char *fmt, ...);
+
+// Returns FAITH_OK or records the HIP error text and returns FAITH_ERR_LAUNCH.
+int check_launch(const char *what);
+
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline int ceil_div(long long a, long long b) { return static_cast<int>((a + b - 1) / b); }
+
+}  // namespace faith
+
+#define FAITH_REQUIRE(cond, code, ...)      \
+    do {                                    \
+        if (!(cond)) {                      \
+            faith::set_error(__VA_ARGS__);  \
+            return (code);                  \
+        }                                   \
+    } while (0)
+
+#define FAITH_NOT_NULL(p) FAITH_REQUIRE((p) != nullptr, FAITH_ERR_NULL, "%s: argument '%s' is NULL", __func__, #p)
+#define FAITH_ALIGNED4(p) \
+    FAITH_REQUIRE(faith::aligned((p), 4), FAITH_ERR_ALIGN, "%s: argument '%s' is not 4-byte aligned", __func__, #p)

@@ -1,0 +1,202 @@
+"""Tensor-level wrappers over the C ABI.
+
+Each function checks device / dtype / contiguity / shape on the host, allocates
+the outputs with torch (device memory plumbing only) and passes raw pointers
+plus the current HIP stream to libfaith_amd.so.  No arithmetic happens here.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+from ._lib import LAYOUT_NATURAL, LAYOUT_TRANSPOSED, Q_1, Q_2, Q_INF  # noqa: F401
+
+
+def q_code(p: float) -> int:
+    """Dual-norm selector for perturbation norm p (q = 1 / (1 - 1/p))."""
+    if p == 1:
+        return Q_INF
+    if p == 2:
+        return Q_2
+    if math.isinf(p) or p >= 10:      # the reference treats p >= 10 as infinity
+        return Q_1
+    raise ValueError(f"p={p}: only p in {{1, 2, inf}} has a kernel")
+
+
+def _check(name, t, shape=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: must live on the GPU (got {t.device}); there is no CPU path")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name}: must be float32, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _wb_shapes(lw, lb, layout):
+    if lw.dim() != 4 or lb.dim() != 3:
+        raise ValueError(f"lw must be 4-D and lb 3-D, got {tuple(lw.shape)} and {tuple(lb.shape)}")
+    B, L = lw.shape[0], lw.shape[1]
+    if layout == LAYOUT_NATURAL:
+        D, H = lw.shape[2], lw.shape[3]
+    else:
+        H, D = lw.shape[2], lw.shape[3]
+    if tuple(lb.shape) != (B, L, H):
+        raise ValueError(f"lb shape {tuple(lb.shape)} does not match lw shape {tuple(lw.shape)}")
+    return B, L, D, H
+
+
+def concretize(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL):
+    """Concrete interval [l, u] of every neuron.  Shapes as Bounds.concretize."""
+    B, L, D, H = _wb_shapes(lw, lb, layout)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    l = torch.empty_like(lb)
+    u = torch.empty_like(ub)
+    with torch.cuda.device(lw.device):
+        _lib.call("faith_concretize", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(l), _ptr(u),
+                  B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
+    return l, u
+
+
+def _activation(entry, lw, lb, uw, ub, p, eps, words, layout, return_interval, out=None):
+    B, L, D, H = _wb_shapes(lw, lb, layout)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    if out is None:
+        olw, olb, ouw, oub = (torch.empty_like(lw), torch.empty_like(lb),
+                              torch.empty_like(uw), torch.empty_like(ub))
+    else:
+        olw, olb, ouw, oub = out
+        _check("out lw", olw, lw.shape); _check("out uw", ouw, lw.shape)
+        _check("out lb", olb, lb.shape); _check("out ub", oub, lb.shape)
+    l = torch.empty_like(lb) if return_interval else None
+    u = torch.empty_like(ub) if return_interval else None
+    with torch.cuda.device(lw.device):
+        _lib.call(entry, _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
+                  _ptr(l), _ptr(u), B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
+    if return_interval:
+        return olw, olb, ouw, oub, l, u
+    return olw, olb, ouw, oub
+
+
+def relu(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
+    """ReLU relaxation; returns (lw', lb', uw', ub'[, l, u])."""
+    return _activation("faith_relu_verification", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
+
+
+def tanh(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
+    """tanh relaxation; returns (lw', lb', uw', ub'[, l, u])."""
+    return _activation("faith_tanh_verification", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
+
+
+def linear(lw, lb, uw, ub, weight, bias=None, out=None):
+    """Sign-split propagation through y = x @ weight.T + bias.  weight: [H_out, H]."""
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    _check("weight", weight)
+    if weight.dim() != 2 or weight.shape[1] != H:
+        raise ValueError(f"weight must be [H_out, {H}], got {tuple(weight.shape)}")
+    N = weight.shape[0]
+    if bias is not None:
+        _check("bias", bias, (N,))
+    if out is None:
+        olw = torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32)
+        ouw = torch.empty_like(olw)
+        olb = torch.empty(B, L, N, device=lw.device, dtype=torch.float32)
+        oub = torch.empty_like(olb)
+    else:
+        olw, olb, ouw, oub = out
+        _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
+        _check("out lb", olb, (B, L, N)); _check("out ub", oub, (B, L, N))
+    with torch.cuda.device(lw.device):
+        _lib.call("faith_matmul_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
+                  _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), B, L, D, H, N, _stream(lw))
+    return olw, olb, ouw, oub
+
+
+def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
+    """McCormick bounds of x . y^T.  x, y: (lw, lb, uw, ub) tuples with
+    lw [B, Lx|Ly, D, d]; returns (lw [B, Lx, D, Ly], lb [B, Lx, Ly], uw, ub)."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    B, Lx, D, d = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    B2, Ly, D2, d2 = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
+    if (B2, D2, d2) != (B, D, d):
+        raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} disagree in batch, dim_in or dim_out")
+    for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                    ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
+        _check(n, t, s)
+    dev = xlw.device
+    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
+    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
+    if out is None:
+        zlw = torch.empty(B, Lx, D, Ly, device=dev, dtype=torch.float32)
+        zuw = torch.empty_like(zlw)
+        zlb = torch.empty(B, Lx, Ly, device=dev, dtype=torch.float32)
+        zub = torch.empty_like(zlb)
+    else:
+        zlw, zlb, zuw, zub = out
+        _check("out lw", zlw, (B, Lx, D, Ly)); _check("out uw", zuw, (B, Lx, D, Ly))
+        _check("out lb", zlb, (B, Lx, Ly)); _check("out ub", zub, (B, Lx, Ly))
+    with torch.cuda.device(dev):
+        _lib.call("faith_dot_product_verification_QK", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
+                  _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
+                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Ly, d, D, float(eps), q_code(p), int(words),
+                  _stream(xlw))
+    if return_intervals:
+        return zlw, zlb, zuw, zub, (x_l, x_u, y_l, y_u)
+    return zlw, zlb, zuw, zub
+
+
+def conv2d(lw, lb, uw, ub, weight, bias=None, stride=1, padding=0, out=None):
+    """Sign-split propagation through a 2-D convolution.
+    lw, uw: [1, D_in, C_in, H, W]; lb, ub: [1, C_in, H, W]; weight: [C_out, C_in, K, K]."""
+    if lw.dim() != 5 or lb.dim() != 4 or lw.shape[0] != 1 or lb.shape[0] != 1:
+        raise ValueError(f"expected lw [1,D,C,H,W] and lb [1,C,H,W], got {tuple(lw.shape)}, {tuple(lb.shape)}")
+    _, D, C, Hh, Ww = lw.shape
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb, (1, C, Hh, Ww)); _check("ub", ub, lb.shape)
+    _check("weight", weight)
+    if weight.dim() != 4 or weight.shape[1] != C or weight.shape[2] != weight.shape[3]:
+        raise ValueError(f"weight must be [C_out, {C}, K, K], got {tuple(weight.shape)}")
+    Co, _, K, _ = weight.shape
+    if bias is not None:
+        _check("bias", bias, (Co,))
+    Ho = (Hh + 2 * padding - K) // stride + 1
+    Wo = (Ww + 2 * padding - K) // stride + 1
+    if Ho <= 0 or Wo <= 0:
+        raise ValueError("convolution output would be empty")
+    if out is None:
+        olw = torch.empty(1, D, Co, Ho, Wo, device=lw.device, dtype=torch.float32)
+        ouw = torch.empty_like(olw)
+        olb = torch.empty(1, Co, Ho, Wo, device=lw.device, dtype=torch.float32)
+        oub = torch.empty_like(olb)
+    else:
+        olw, olb, ouw, oub = out
+        _check("out lw", olw, (1, D, Co, Ho, Wo)); _check("out uw", ouw, (1, D, Co, Ho, Wo))
+        _check("out lb", olb, (1, Co, Ho, Wo)); _check("out ub", oub, (1, Co, Ho, Wo))
+    with torch.cuda.device(lw.device):
+        _lib.call("faith_convolution_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight),
+                  _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), 1, Hh, Ww, C, Co, K, int(stride),
+                  int(padding), D, _stream(lw))
+    return olw, olb, ouw, oub
+
+
+def concretize_conv(lw, lb, uw, ub, p, eps):
+    """Concretize conv-shaped bounds (norm over D_in): lw [1, D, C, H, W] -> l, u [1, C, H, W]."""
+    _, D, C, Hh, Ww = lw.shape
+    l, u = concretize(lw.view(1, 1, D, C * Hh * Ww), lb.view(1, 1, C * Hh * Ww),
+                      uw.view(1, 1, D, C * Hh * Ww), ub.view(1, 1, C * Hh * Ww), p, eps, 1)
+    return l.view(1, C, Hh, Ww), u.view(1, C, Hh, Ww)

@@ -1,0 +1,142 @@
+/*
+ * faith_amd.h -- C ABI of the MI355X (gfx950) forward bound-propagation kernels.
+ *
+ * Each entry point takes raw DEVICE pointers to contiguous fp32 arrays, plain
+ * ints / floats, and a HIP stream handle passed as void* (NULL = the default
+ * stream).  Launches are asynchronous on that stream.  Nothing is allocated or
+ * freed; the caller owns every buffer, inputs and outputs alike (as in the
+ * reference, Transformer_Verification_Code/Verifiers/Bounds.py:1270-1277).
+ *
+ * Return value: FAITH_OK (0) or a negative FAITH_ERR_* code.  Nothing aborts.
+ * faith_last_error() returns a thread-local message for the last failure.
+ *
+ * Conventions shared by all entry points
+ *   lw, uw   coefficient arrays; "natural" layout [rows, dim_in, dim_out]
+ *            (Bounds.py:293-297) or "transposed" layout [rows, dim_out, dim_in]
+ *            (what the reference's CUDA adapters pass, Bounds.py:1210-1211).
+ *   lb, ub   constant terms [rows, dim_out].
+ *   rows     batch * length; every op here is independent across rows.
+ *   q        dual-norm selector FAITH_Q_*  (q = 1/(1-1/p), Bounds.py:277).
+ *   words    number of equal blocks of dim_in that are normed separately and
+ *            summed (perturbed_words, Bounds.py:319-326).
+ */
+#ifndef FAITH_AMD_H
+#define FAITH_AMD_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FAITH_OK                0
+#define FAITH_ERR_NULL         -1   /* a required pointer is NULL                    */
+#define FAITH_ERR_SHAPE        -2   /* a dimension is non-positive or inconsistent   */
+#define FAITH_ERR_UNSUPPORTED  -3   /* valid request this build has no kernel for    */
+#define FAITH_ERR_ALIGN        -4   /* pointer not 4-byte aligned                    */
+#define FAITH_ERR_LAUNCH       -5   /* HIP reported an error at launch               */
+
+#define FAITH_Q_1    1   /* p = inf : sum of magnitudes  */
+#define FAITH_Q_2    2   /* p = 2   : Euclidean norm     */
+#define FAITH_Q_INF  0   /* p = 1   : largest magnitude  */
+
+#define FAITH_LAYOUT_NATURAL     0
+#define FAITH_LAYOUT_TRANSPOSED  1
+
+const char *faith_last_error(void);
+int faith_version(void);
+
+/*
+ * Dual-norm concretization.  Replaces Bounds.concretize (Bounds.py:311-326) and the
+ * CUDA `concretize` kernel (HandTunedKernels/dot_product_verification.cu:47-105).
+ *   l[r,j] = lb[r,j] - eps * sum_w ||lw[r, block w, j]||_q
+ *   u[r,j] = ub[r,j] + eps * sum_w ||uw[r, block w, j]||_q
+ */
+int faith_concretize(const float *lb, const float *ub, const float *lw, const float *uw,
+                     float *l, float *u,
+                     int rows, int dim_in, int dim_out,
+                     float eps, int q, int words, int layout, void *stream);
+
+/*
+ * ReLU relaxation fused with concretization.  Replaces call_relu_verification
+ * (HandTunedKernels/kernel.cpp:7-20, relu_verification.cu:134-147) with the arithmetic of
+ * Bounds.ori_relu (Bounds.py:921-963).  `epsilon` is the perturbation radius, as in the
+ * reference signature.  l_out / u_out may be NULL; when given they receive the concrete
+ * pre-activation interval the relaxation was built from.
+ */
+int faith_relu_verification(const float *src_lb, const float *src_ub,
+                            const float *src_lw, const float *src_uw,
+                            float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                            float *l_out, float *u_out,
+                            int length, int dim_in, int dim_out, float epsilon,
+                            int q, int words, int layout, void *stream);
+
+/*
+ * tanh relaxation fused with concretization.  Replaces call_tanh_verification
+ * (kernel.cpp:22-35, tanh_verification.cu:196-209) with the arithmetic of
+ * Bounds.ori_tanh (Bounds.py:1027-1103): tangent / chord lines and two 10-step bisections.
+ */
+int faith_tanh_verification(const float *src_lb, const float *src_ub,
+                            const float *src_lw, const float *src_uw,
+                            float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                            float *l_out, float *u_out,
+                            int length, int dim_in, int dim_out, float epsilon,
+                            int q, int words, int layout, void *stream);
+
+/*
+ * Sign-split affine propagation  y = x @ W^T (+ bias).  Replaces the (commented-out)
+ * call_matmul_verification (kernel.cpp:37-43, matmul_verification.cu:787-815) with the
+ * arithmetic of Bounds.ori_matmul + add (Bounds.py:397-413, :383-395).
+ *   x_lw, x_uw [batch*length, dim_in, dim_out]   natural layout
+ *   x_lb, x_ub [batch*length, dim_out]
+ *   W          [dim_y_out, dim_out]              nn.Linear layout
+ *   bias       [dim_y_out] or NULL
+ *   y_lw, y_uw [batch*length, dim_in, dim_y_out];  y_lb, y_ub [batch*length, dim_y_out]
+ */
+int faith_matmul_verification(const float *x_lb, const float *x_ub,
+                              const float *x_lw, const float *x_uw,
+                              const float *W, const float *bias,
+                              float *y_lb, float *y_ub, float *y_lw, float *y_uw,
+                              int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
+                              void *stream);
+
+/*
+ * McCormick bounds of the attention scores  z[i,j] = sum_k x[i,k] * y[j,k].  Replaces
+ * call_dot_product_verification_QK (kernel.cpp:45-51, dot_product_verification.cu:458-496)
+ * with the arithmetic of Bounds.ori_dot_product (Bounds.py:710-823).  Natural layout:
+ *   x_lw, x_uw [batch, length_x, dim_in, dim_out];  x_lb, x_ub [batch, length_x, dim_out]
+ *   y_lw, y_uw [batch, length_y, dim_in, dim_out];  y_lb, y_ub [batch, length_y, dim_out]
+ *   x_l, x_u   [batch, length_x, dim_out]  (out: concrete interval of x; caller's scratch)
+ *   y_l, y_u   [batch, length_y, dim_out]  (out: concrete interval of y)
+ *   z_lw, z_uw [batch, length_x, dim_in, length_y];  z_lb, z_ub [batch, length_x, length_y]
+ * The reference entry has one `length`; here x and y may differ in length.
+ */
+int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u,
+                                      const float *x_lb, const float *x_ub,
+                                      const float *y_lb, const float *y_ub,
+                                      const float *x_lw, const float *x_uw,
+                                      const float *y_lw, const float *y_uw,
+                                      float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                                      int batch_size, int length_x, int length_y,
+                                      int dim_out, int dim_in, float epsilon,
+                                      int q, int words, void *stream);
+
+/*
+ * Sign-split propagation through a 2-D convolution (NCHW).  Replaces the (commented-out)
+ * call_convolution_verification (kernel.cpp:62-67, convolution_verification.cu:219-239).
+ *   x_lw, x_uw [dim_in, CIN, Height, Width]   (dim_in plays the conv batch)
+ *   x_lb, x_ub [batch_size, CIN, Height, Width]
+ *   W          [COUT, CIN, K, K];  bias [COUT] or NULL (added to y_lb / y_ub only)
+ *   y_lw, y_uw [dim_in, COUT, Ho, Wo];  y_lb, y_ub [batch_size, COUT, Ho, Wo]
+ *   Ho = (Height + 2*padding_size - K) / Stride + 1, likewise Wo.
+ */
+int faith_convolution_verification(const float *x_lb, const float *x_ub,
+                                   const float *x_lw, const float *x_uw,
+                                   const float *W, const float *bias,
+                                   float *y_lb, float *y_ub, float *y_lw, float *y_uw,
+                                   int batch_size, int Height, int Width, int CIN, int COUT,
+                                   int K, int Stride, int padding_size, int dim_in,
+                                   void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FAITH_AMD_H */

@@ -52,19 +52,27 @@ def _apply(side, k, x0, y0, lw_col, lb, uw_col, ub):
     return np.asarray(w, dtype=np.float64) * k, (float(b) - x0) * k + y0
 
 
-def relu_neuron(lw_col, lb, uw_col, ub, p, eps, words=1):
-    """(lw', lb', uw', ub') of one neuron through ReLU (Bounds.py:921-963)."""
-    lo, hi = interval(lw_col, lb, uw_col, ub, p, eps, words)
-    zeros = np.zeros(len(lw_col))
-    if hi < 0:                       # dead
-        return zeros, 0.0, zeros, 0.0
+def relu_lines(lo, hi):
+    """(k, x0, y0) of the lower and the upper line of ReLU on [lo, hi] (Bounds.py:921-963)."""
+    if hi < 0:                       # dead: the zero line
+        return (0.0, 0.0, 0.0), (0.0, 0.0, 0.0)
     if lo > 0:                       # active: identity
-        return (np.asarray(lw_col, float), float(lb), np.asarray(uw_col, float), float(ub))
-    k_up = hi / (hi - lo + TINY)
-    uw2, ub2 = _apply("upper", k_up, lo, 0.0, lw_col, lb, uw_col, ub)
-    k_lo = 1.0 if abs(hi) > abs(lo) else 0.0
-    lw2, lb2 = _apply("lower", k_lo, 0.0, 0.0, lw_col, lb, uw_col, ub)
+        return (1.0, 0.0, 0.0), (1.0, 0.0, 0.0)
+    upper = (hi / (hi - lo + TINY), lo, 0.0)          # chord from (lo, 0) to (hi, hi)
+    lower = (1.0 if abs(hi) > abs(lo) else 0.0, 0.0, 0.0)
+    return lower, upper
+
+
+def lines_applied(lower, upper, lw_col, lb, uw_col, ub):
+    lw2, lb2 = _apply("lower", *lower, lw_col, lb, uw_col, ub)
+    uw2, ub2 = _apply("upper", *upper, lw_col, lb, uw_col, ub)
     return lw2, lb2, uw2, ub2
+
+
+def relu_neuron(lw_col, lb, uw_col, ub, p, eps, words=1):
+    """(lw', lb', uw', ub') of one neuron through ReLU."""
+    lo, hi = interval(lw_col, lb, uw_col, ub, p, eps, words)
+    return lines_applied(*relu_lines(lo, hi), lw_col, lb, uw_col, ub)
 
 
 def _sech2(v):
@@ -107,10 +115,7 @@ def tanh_lines(lo, hi, iters=10):
 
 def tanh_neuron(lw_col, lb, uw_col, ub, p, eps, words=1, iters=10):
     lo, hi = interval(lw_col, lb, uw_col, ub, p, eps, words)
-    lower, upper = tanh_lines(lo, hi, iters)
-    lw2, lb2 = _apply("lower", *lower, lw_col, lb, uw_col, ub)
-    uw2, ub2 = _apply("upper", *upper, lw_col, lb, uw_col, ub)
-    return lw2, lb2, uw2, ub2
+    return lines_applied(*tanh_lines(lo, hi, iters), lw_col, lb, uw_col, ub)
 
 
 def linear_brute(lw, lb, uw, ub, W, bias=None):

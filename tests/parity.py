@@ -1,0 +1,75 @@
+"""Parity harness for the activation relaxations (HIP path vs CPU oracle).
+
+The bar is rtol 1e-5 / atol 1e-6 (fp32).  A relaxation is a discontinuous
+function of the concrete interval [l, u]:
+
+  * ReLU and tanh switch formulas at l = 0 and at u = 0,
+  * ReLU's lower slope flips 0 <-> 1 at |u| = |l|,
+  * tanh's bisections branch on the sign of a quantity that passes through 0
+    at the tangent point.
+
+The GPU reduces the q-norm in a different order than the CPU, so l and u can
+differ in the last bits; a neuron sitting within a few ulps of such a switch
+may legitimately take the other branch.  The policy here never widens the
+tolerance:
+
+  1. l and u themselves are compared first, at the full bar.
+  2. Neurons whose outputs all meet the bar pass.
+  3. Every remaining neuron must be *explained*: the fp64 closed form,
+     evaluated from the GPU's own [l, u] for that neuron, must reproduce the
+     GPU's outputs (at a bar that allows for fp32 rounding of the inputs of
+     the closed form), AND the neuron must be a boundary case -- l, u or
+     |u| - |l| within `boundary_ulps` ulps of a switch, or (tanh only) a
+     straddling neuron, where a bisection step may flip.
+  4. The number of explained neurons is bounded (`max_explained_frac`) and
+     reported.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from oracle import closed_form as C
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def _bad(got, exp, rtol=RTOL, atol=ATOL):
+    got = got.detach().cpu().double()
+    exp = exp.detach().cpu().double()
+    return (got - exp).abs() > atol + rtol * exp.abs()
+
+
+def compare_activation(kind, x, got, exp, l_gpu, u_gpu, l_ref, u_ref,
+                       boundary_ulps=16, max_explained_frac=2e-4):
+    """x: oracle LinearBounds input (CPU); got / exp: (lw, lb, uw, ub) from the
+    HIP path / the oracle, natural layout; returns a small report dict."""
+    assert not _bad(l_gpu, l_ref).any(), "concrete lower bounds differ"
+    assert not _bad(u_gpu, u_ref).any(), "concrete upper bounds differ"
+    assert bool((l_gpu <= u_gpu).all()), "l <= u violated"
+
+    glw, glb, guw, gub = (t.detach().cpu() for t in got)
+    elw, elb, euw, eub = exp
+    bad_n = (_bad(glw, elw).any(dim=2) | _bad(guw, euw).any(dim=2) | _bad(glb, elb) | _bad(gub, eub))
+    idx = bad_n.nonzero().tolist()
+    total = bad_n.numel()
+    assert len(idx) <= max(2, int(max_explained_frac * total)), \
+        f"{len(idx)} of {total} neurons off the bar -- too many to be boundary cases"
+
+    lines = C.relu_lines if kind == "relu" else C.tanh_lines
+    ulp = float(np.finfo(np.float32).eps)
+    for b, r, j in idx:
+        lo, hi = float(l_gpu[b, r, j]), float(u_gpu[b, r, j])
+        scale = max(abs(lo), abs(hi), 1e-30)
+        near_switch = (abs(lo) <= boundary_ulps * ulp * scale or abs(hi) <= boundary_ulps * ulp * scale
+                       or abs(abs(hi) - abs(lo)) <= boundary_ulps * ulp * scale)
+        straddles = lo <= 0.0 <= hi
+        assert near_switch or (kind == "tanh" and straddles), \
+            f"neuron {(b, r, j)} with [l,u]=[{lo},{hi}] is off the bar and not a boundary case"
+        e = C.lines_applied(*lines(lo, hi), x.lw[b, r, :, j].double().numpy(), float(x.lb[b, r, j]),
+                            x.uw[b, r, :, j].double().numpy(), float(x.ub[b, r, j]))
+        np.testing.assert_allclose(glw[b, r, :, j].double().numpy(), e[0], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(float(glb[b, r, j]), e[1], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(guw[b, r, :, j].double().numpy(), e[2], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(float(gub[b, r, j]), e[3], rtol=1e-4, atol=1e-5)
+    return {"neurons": total, "explained_boundary_cases": len(idx)}

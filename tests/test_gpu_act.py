@@ -1,0 +1,170 @@
+"""HIP concretize / ReLU / tanh against the CPU oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import bounds_oracle as O
+from tests.helpers import rand_bounds, as_bounds, close, RTOL, ATOL
+from tests.parity import compare_activation
+
+pytestmark = pytest.mark.gpu
+INF = float("inf")
+PS = [1.0, 2.0, INF]
+
+
+def dev(*ts):
+    return [t.cuda().contiguous() for t in ts]
+
+
+def run_act(kind, x, p, eps, words, layout="natural"):
+    from faith_amd import ops
+    lw, lb, uw, ub = dev(*x.tensors())
+    fn = getattr(ops, kind)
+    if layout == "natural":
+        out = fn(lw, lb, uw, ub, p, eps, words, return_interval=True)
+        return out[:4], out[4], out[5]
+    lwt, uwt = lw.transpose(2, 3).contiguous(), uw.transpose(2, 3).contiguous()
+    olw, olb, ouw, oub, l, u = fn(lwt, lb, uwt, ub, p, eps, words, layout=ops.LAYOUT_TRANSPOSED,
+                                  return_interval=True)
+    return (olw.transpose(2, 3), olb, ouw.transpose(2, 3), oub), l, u
+
+
+def check(kind, x, p, eps, words, layout="natural"):
+    print(f"[case] {kind} shape={tuple(x.lw.shape)} p={p} eps={eps} words={words} layout={layout}", flush=True)
+    got, l, u = run_act(kind, x, p, eps, words, layout)
+    torch.cuda.synchronize()
+    exp = getattr(O, kind)(x, p, eps, words)
+    l_ref, u_ref = O.concretize(x, p, eps, words)
+    rep = compare_activation(kind, x, got, exp.tensors(), l.cpu(), u.cpu(), l_ref, u_ref)
+    print("   ", rep, flush=True)
+    return rep
+
+
+@pytest.mark.parametrize("p", PS)
+@pytest.mark.parametrize("words", [1, 2])
+@pytest.mark.parametrize("layout", ["natural", "transposed"])
+def test_concretize(p, words, layout):
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(5)
+    for (B, L, D, H) in [(1, 3, 64, 64), (2, 5, 96, 40), (1, 2, 600, 132), (1, 1, 6, 7)]:
+        x = rand_bounds(g, B, L, D, H, ordered=False)
+        lw, lb, uw, ub = dev(*x.tensors())
+        if layout == "natural":
+            l, u = ops.concretize(lw, lb, uw, ub, p, 0.3, words)
+        else:
+            l, u = ops.concretize(lw.transpose(2, 3).contiguous(), lb, uw.transpose(2, 3).contiguous(), ub,
+                                  p, 0.3, words, layout=ops.LAYOUT_TRANSPOSED)
+        el, eu = O.concretize(x, p, 0.3, words)
+        assert close(l, el) and close(u, eu), (B, L, D, H)
+
+
+@pytest.mark.parametrize("kind", ["relu", "tanh"])
+@pytest.mark.parametrize("p", PS)
+@pytest.mark.parametrize("layout", ["natural", "transposed"])
+def test_activation_small_shapes(kind, p, layout):
+    g = torch.Generator().manual_seed(6)
+    # register-resident, chunked (D_in > 512), ragged H (scalar path), tiny
+    for (L, D, H, words) in [(4, 64, 64, 1), (3, 128, 192, 2), (2, 256, 64, 2), (2, 512, 64, 1),
+                             (1, 1100, 72, 1), (2, 48, 37, 3), (1, 2, 5, 1)]:
+        x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+        check(kind, x, p, 0.05, words, layout)
+
+
+@pytest.mark.parametrize("kind", ["relu", "tanh"])
+def test_activation_reference_test_distribution(kind):
+    """Inputs drawn as the reference's own op test draws them
+    (kernel_test/transformer_forward_test_bound.py:746-754, p=2, eps=0.5):
+    lb ~ U(0,1), ub = lb + U(0,1), lw and uw independent U(-.5,.5)."""
+    g = torch.Generator().manual_seed(0)
+    for (L, D, H) in [(2, 64, 64), (8, 128, 64), (4, 64, 256)]:
+        lb = torch.rand(1, L, H, generator=g)
+        ub = lb + torch.rand(1, L, H, generator=g)
+        lw = torch.rand(1, L, D, H, generator=g) - 0.5
+        uw = torch.rand(1, L, D, H, generator=g) - 0.5
+        check(kind, O.LinearBounds(lw, lb, uw, ub), 2.0, 0.5, 1)
+
+
+def test_activation_branch_edges():
+    """Neurons exactly on the switches: l == 0, u == 0, |u| == |l|, and zero-width intervals."""
+    from faith_amd import ops
+    H, D = 64, 8
+    lw = torch.zeros(1, 1, D, H); uw = torch.zeros(1, 1, D, H)
+    lw[0, 0, 0, :] = 0.25; uw[0, 0, 0, :] = 0.5
+    lb = torch.linspace(-1, 1, H).view(1, 1, H).clone()
+    ub = lb.clone() + 0.5
+    lb[0, 0, 0] = 0.0; ub[0, 0, 0] = 1.0        # l == 0 exactly (eps = 0 below)
+    lb[0, 0, 1] = -1.0; ub[0, 0, 1] = 0.0       # u == 0 exactly
+    lb[0, 0, 2] = -0.5; ub[0, 0, 2] = 0.5       # |u| == |l|
+    lb[0, 0, 3] = 0.0; ub[0, 0, 3] = 0.0        # degenerate at 0
+    x = O.LinearBounds(lw, lb, uw, ub)
+    for kind in ("relu", "tanh"):
+        got, l, u = run_act(kind, x, 2.0, 0.0, 1)
+        exp = getattr(O, kind)(x, 2.0, 0.0, 1)
+        for a, b in zip(got, exp.tensors()):
+            assert close(a, b), kind
+
+
+@pytest.mark.parametrize("kind", ["relu", "tanh"])
+@pytest.mark.parametrize("p", PS)
+def test_activation_config1_reduced(kind, p):
+    """Benchmark configuration 1 at a quarter of its length (same D_in, H, words)."""
+    from faith_amd.workloads import make_config
+    c = make_config(1, scale=0.25)
+    rep = check(kind, as_bounds(c["x"]), p, c["eps"], c["words"])
+    assert rep["neurons"] == 32 * 512
+
+
+@pytest.mark.parametrize("kind", ["relu", "tanh"])
+def test_activation_config1_full_properties(kind):
+    """Full-size configuration 1: size-independent properties instead of the oracle.
+    (i) the concrete interval of the output bounds the activation of the input interval
+    end points; (ii) dead / active ReLU neurons are zero / identity; (iii) l <= u."""
+    from faith_amd import ops
+    from faith_amd.workloads import make_config
+    c = make_config(1)
+    lw, lb, uw, ub = dev(*(c["x"][k] for k in ("lw", "lb", "uw", "ub")))
+    for p in PS:
+        olw, olb, ouw, oub, l, u = getattr(ops, kind)(lw, lb, uw, ub, p, c["eps"], c["words"], return_interval=True)
+        assert bool((l <= u).all())
+        ol, ou = ops.concretize(olw, olb, ouw, oub, p, c["eps"], c["words"])
+        f = torch.relu if kind == "relu" else torch.tanh
+        assert bool((ol <= f(l) + 1e-4).all()) and bool((ou >= f(u) - 1e-4).all())
+        if kind == "relu":
+            dead, act = u < 0, l > 0
+            assert torch.count_nonzero(olw.transpose(2, 3)[dead]) == 0
+            assert torch.count_nonzero(ouw.transpose(2, 3)[dead]) == 0
+            assert torch.equal(olw.transpose(2, 3)[act], lw.transpose(2, 3)[act])
+            assert torch.equal(oub[act], ub[act])
+            frac_both = 1.0 - float(dead.float().mean()) - float(act.float().mean())
+            assert 0.2 < frac_both < 0.8
+
+
+def test_c_bound_shim_matches_reference_calling_convention():
+    """faith_amd.c_bound: reference names, transposed operands, caller-allocated outputs
+    (HandTunedKernels/kernel.cpp:69-131; adapter in Bounds.py:1201-1231)."""
+    from faith_amd import c_bound
+    g = torch.Generator().manual_seed(7)
+    L, D, H = 4, 64, 128
+    x = rand_bounds(g, 1, L, D, H, sw=0.2, gap_w=0.02, gap_b=0.5)
+    lw, lb, uw, ub = dev(*x.tensors())
+    for name, kind in (("c_relu_verification", "relu"), ("c_tanh_verification", "tanh")):
+        _lw = torch.zeros(1, L, H, D, device="cuda"); _uw = torch.zeros_like(_lw)
+        _lb = torch.zeros(1, L, H, device="cuda"); _ub = torch.zeros_like(_lb)
+        getattr(c_bound, name)(lb, ub, lw.transpose(2, 3).contiguous(), uw.transpose(2, 3).contiguous(),
+                               _lb, _ub, _lw, _uw, L, D, H, 0.05)
+        exp = getattr(O, kind)(x, 2.0, 0.05, 1)
+        assert close(_lw.transpose(2, 3), exp.lw) and close(_uw.transpose(2, 3), exp.uw)
+        assert close(_lb, exp.lb) and close(_ub, exp.ub)
+
+
+def test_bad_arguments_are_rejected_not_launched():
+    from faith_amd import ops, _lib
+    lw = torch.zeros(1, 2, 8, 4, device="cuda"); lb = torch.zeros(1, 2, 4, device="cuda")
+    with pytest.raises(_lib.FaithError) as e:
+        ops.relu(lw, lb, lw, lb, 2.0, 0.1, words=3)          # 3 does not divide 8
+    assert e.value.code == -2
+    with pytest.raises(ValueError):
+        ops.relu(lw, lb, lw, lb, 3.0, 0.1)                   # no kernel for q = 1.5
+    with pytest.raises(ValueError):
+        ops.relu(lw.cpu(), lb, lw, lb, 2.0, 0.1)             # CPU tensor: no fallback
+    with pytest.raises(TypeError):
+        ops.relu(lw.double(), lb, lw, lb, 2.0, 0.1)
