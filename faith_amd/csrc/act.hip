@@ -73,69 +73,6 @@ __device__ __forceinline__ void relu_lines(float l, float u, Line &lo, Line &up)
     }
 }
 
-// 1 / cosh^2 in double.
-__device__ __forceinline__ double sech2(double x) {
-    const double c = cosh(x);
-    return 1.0 / (c * c);
-}
-
-// Bounds.py:1027-1097.  Interval end points, bisection state and the results are fp32 as in
-// the reference; tanh / cosh and the quotients are evaluated in double and rounded once, so
-// that the only disagreement with an fp32 library left is that library's own rounding.
-__device__ void tanh_lines(float l, float u, Line &lo, Line &up) {
-    const double tl = tanh((double)l), tu = tanh((double)u);
-    if (u < 0.f || l > 0.f) {
-        const float m = (l + u) / 2;
-        const Line tangent = {(float)sech2((double)m), m, (float)tanh((double)m)};
-        const Line chord = {(float)((tu - tl) / (double)((u - l) + TINY)), l, (float)tl};
-        if (u < 0.f) {
-            lo = tangent;
-            up = chord;
-        } else {
-            lo = chord;
-            up = tangent;
-        }
-        return;
-    }
-    {   // lower line: tangent point d in [l, 0] whose tangent passes through (u, tanh u)
-        float d = l / 2, a = l, b = 0.f;
-        for (int it = 0; it < 10; ++it) {
-            const double v = (tu - tanh((double)d)) / (double)((u - d) + TINY) - sech2((double)d);
-            if (v > 0) {
-                a = d;
-                d = (d + b) / 2;
-            } else {
-                b = d;
-                d = (d + a) / 2;
-            }
-        }
-        const double td = tanh((double)d);
-        lo = {(float)((td - tu) / (double)((d - u) + TINY)), d, (float)td};
-    }
-    {   // upper line: tangent point d in [0, u] whose tangent passes through (l, tanh l)
-        float d = u / 2, a = 0.f, b = u;
-        for (int it = 0; it < 10; ++it) {
-            const double v = (tanh((double)d) - tl) / (double)((d - l) + TINY) - sech2((double)d);
-            if (v > 0) {
-                b = d;
-                d = (d + a) / 2;
-            } else {
-                a = d;
-                d = (d + b) / 2;
-            }
-        }
-        const double td = tanh((double)d);
-        up = {(float)((td - tl) / (double)((d - l) + TINY)), d, (float)td};
-    }
-}
-
-template <int MODE>
-__device__ __forceinline__ void make_lines(float l, float u, Line &lo, Line &up) {
-    if (MODE == RELU)
-        relu_lines(l, u, lo, up);
-    else
-        tanh_lines(l, u, lo, up);
-}
 
 // Bounds.add_linear, constant term (Bounds.py:378, :381): a positive slope takes the same-side
 // bound, a non-positive one the opposite bound; three separate roundings.
@@ -172,6 +109,63 @@ struct Vec<1> {
 };
 
 // ------------------------------------------------------------------ natural layout
+// exp-based pieces for the tanh lines, all in double: with t = exp(2x),
+// tanh x = (t - 1) / (t + 1) and 1 / cosh^2 x = 4 t / (t + 1)^2.  |x| is clamped at 20, where
+// tanh is 1 to 17 digits.
+struct TanhAt {
+    double th, s2;
+};
+__device__ __forceinline__ TanhAt tanh_at(float x) {
+    const double t = exp(2.0 * fmin(fmax((double)x, -20.0), 20.0));
+    const double r = 1.0 / (t + 1.0);
+    return {(t - 1.0) * r, 4.0 * t * r * r};
+}
+
+// Tangent point search of Bounds.py:1065-1075 (lower = true) and :1082-1092 (lower = false).
+// `anchor` is the far end of the interval (u for the lower line, l for the upper line).
+// v > 0 is decided on (tanh difference) - sech^2(d) * (distance), which has the sign of the
+// reference's quotient form because the distance (+1e-12) is positive.
+template <bool LOWER>
+__device__ __forceinline__ Line tanh_tangent_line(float l, float u) {
+    const float anchor = LOWER ? u : l;
+    const double ta = tanh_at(anchor).th;
+    float d = (LOWER ? l : u) / 2, a = LOWER ? l : 0.f, b = LOWER ? 0.f : u;
+    for (int it = 0; it < 10; ++it) {
+        const TanhAt f = tanh_at(d);
+        bool go;
+        if (LOWER)
+            go = (ta - f.th) - f.s2 * (double)((u - d) + TINY) > 0.0;
+        else
+            go = (f.th - ta) - f.s2 * (double)((d - l) + TINY) > 0.0;
+        if (LOWER == go) {   // lower & v>0, or upper & v<=0: move right
+            a = d;
+            d = (d + b) / 2;
+        } else {             // move left
+            b = d;
+            d = (d + a) / 2;
+        }
+    }
+    const double td = tanh_at(d).th;
+    if (LOWER) return {(float)((td - ta) / (double)((d - u) + TINY)), d, (float)td};
+    return {(float)((td - ta) / (double)((d - l) + TINY)), d, (float)td};
+}
+
+// One-signed interval: tangent at the midpoint and chord (Bounds.py:1037-1060).
+__device__ __forceinline__ void tanh_pure_lines(float l, float u, Line &lo, Line &up) {
+    const float m = (l + u) / 2;
+    const TanhAt fm = tanh_at(m);
+    const double tl = tanh_at(l).th, tu = tanh_at(u).th;
+    const Line tangent = {(float)fm.s2, m, (float)fm.th};
+    const Line chord = {(float)((tu - tl) / (double)((u - l) + TINY)), l, (float)tl};
+    if (u < 0.f) {
+        lo = tangent;
+        up = chord;
+    } else {
+        lo = chord;
+        up = tangent;
+    }
+}
+
 // TPR threads cover one row of the tile (TH = TPR * VEC neurons); RG = NTHREADS / TPR rows are
 // in flight per step; a thread keeps RPT rows.  D_in <= RG * RPT is the register-resident case;
 // larger D_in is walked in chunks and read a second time for the scaling.
@@ -179,15 +173,18 @@ template <int MODE, int Q, int VEC, int TPR, int NTHREADS, int RPT>
 __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     constexpr int TH = TPR * VEC;
     constexpr int RG = NTHREADS / TPR;
-    static_assert(TH <= NTHREADS, "one thread per neuron must exist");
+    constexpr int NW = NTHREADS / WAVE;
+    static_assert(TH <= WAVE && TPR <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
     extern __shared__ float smem[];
-    float *part = smem;                          // [words][RG][2][TH]
-    float *coef = smem + a.words * RG * 2 * TH;  // [2][TH] slopes
+    float *part = smem;                       // [words][NW][2][TH] per-wavefront partial norms
+    float *s_lu = part + a.words * NW * 2 * TH;   // [2][TH] concrete interval
+    float *s_ln = s_lu + 2 * TH;              // [2][3][TH] lower / upper line (k, x0, y0)
 
     const int tiles = (a.H + TH - 1) / TH;
     const int r = blockIdx.x / tiles;
     const int col0 = (blockIdx.x % tiles) * TH;
     const int tid = threadIdx.x;
+    const int lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid % TPR, rg = tid / TPR;
     const int col = col0 + c * VEC;
     const bool col_ok = col < a.H;
@@ -198,12 +195,14 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
 
     Vec<VEC> dl[RPT], du[RPT];
 
-    for (int w = 0; w < a.words; ++w)
+    if (nchunks > 1 && lane < TPR) {
+        for (int w = 0; w < a.words; ++w)
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-            part[((w * RG + rg) * 2 + 0) * TH + c * VEC + v] = 0.f;
-            part[((w * RG + rg) * 2 + 1) * TH + c * VEC + v] = 0.f;
-        }
+            for (int v = 0; v < VEC; ++v) {
+                part[((w * NW + wv) * 2 + 0) * TH + c * VEC + v] = 0.f;
+                part[((w * NW + wv) * 2 + 1) * TH + c * VEC + v] = 0.f;
+            }
+    }
 
     for (int ch = 0; ch < nchunks; ++ch) {
 #pragma unroll
@@ -233,54 +232,106 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
                     }
                 }
             }
+            // lanes of one wavefront that share a column: butterfly over the row groups
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-                float *sl = &part[((w * RG + rg) * 2 + 0) * TH + c * VEC + v];
-                float *su = &part[((w * RG + rg) * 2 + 1) * TH + c * VEC + v];
-                *sl = ncomb<Q>(*sl, pl[v]);
-                *su = ncomb<Q>(*su, pu[v]);
+            for (int m = TPR; m < WAVE; m <<= 1) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    pl[v] = ncomb<Q>(pl[v], __shfl_xor(pl[v], m, WAVE));
+                    pu[v] = ncomb<Q>(pu[v], __shfl_xor(pu[v], m, WAVE));
+                }
+            }
+            if (lane < TPR) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    float *sl = &part[((w * NW + wv) * 2 + 0) * TH + c * VEC + v];
+                    float *su = &part[((w * NW + wv) * 2 + 1) * TH + c * VEC + v];
+                    if (nchunks > 1) {
+                        *sl = ncomb<Q>(*sl, pl[v]);
+                        *su = ncomb<Q>(*su, pu[v]);
+                    } else {
+                        *sl = pl[v];
+                        *su = pu[v];
+                    }
+                }
             }
         }
     }
     __syncthreads();
 
-    // one thread per neuron: finish the norms, concretize, derive the lines
-    if (tid < TH) {
-        const int column = col0 + tid;
-        if (column < a.H) {
-            const size_t bi = (size_t)r * a.H + column;
+    // one lane per neuron (wavefront 0): finish the norms, concretize
+    const int column = col0 + lane;
+    const bool n_ok = lane < TH && column < a.H;
+    const size_t bi = (size_t)r * a.H + column;
+    if (wv == 0 && n_ok) {
+        float l = a.lb[bi], u = a.ub[bi];
+        for (int w = 0; w < a.words; ++w) {
+            float nl = 0.f, nu = 0.f;
+#pragma unroll
+            for (int g = 0; g < NW; ++g) {
+                nl = ncomb<Q>(nl, part[((w * NW + g) * 2 + 0) * TH + lane]);
+                nu = ncomb<Q>(nu, part[((w * NW + g) * 2 + 1) * TH + lane]);
+            }
+            l += (-a.eps) * nfin<Q>(nl);
+            u += a.eps * nfin<Q>(nu);
+        }
+        if (a.l) a.l[bi] = l;
+        if (a.u) a.u[bi] = u;
+        if (MODE == RELU) {
+            Line lo, up;
+            relu_lines(l, u, lo, up);
+            s_ln[lane] = lo.k;
+            s_ln[3 * TH + lane] = up.k;
             const float lb = a.lb[bi], ub = a.ub[bi];
-            float l = lb, u = ub;
-            for (int w = 0; w < a.words; ++w) {
-                float nl = 0.f, nu = 0.f;
-                for (int g = 0; g < RG; ++g) {
-                    nl = ncomb<Q>(nl, part[((w * RG + g) * 2 + 0) * TH + tid]);
-                    nu = ncomb<Q>(nu, part[((w * RG + g) * 2 + 1) * TH + tid]);
-                }
-                l += (-a.eps) * nfin<Q>(nl);
-                u += a.eps * nfin<Q>(nu);
-            }
-            if (a.l) a.l[bi] = l;
-            if (a.u) a.u[bi] = u;
-            if (MODE != CONCRETIZE) {
-                Line lo, up;
-                make_lines<MODE>(l, u, lo, up);
-                coef[tid] = lo.k;
-                coef[TH + tid] = up.k;
-                a.olb[bi] = line_bias(lo, lb, ub);
-                a.oub[bi] = line_bias(up, ub, lb);
-            }
+            a.olb[bi] = line_bias(lo, lb, ub);
+            a.oub[bi] = line_bias(up, ub, lb);
+        } else if (MODE == TANH) {
+            s_lu[lane] = l;
+            s_lu[TH + lane] = u;
         }
     }
     if (MODE == CONCRETIZE) return;
     __syncthreads();
 
+    if (MODE == TANH) {
+        // three wavefronts share the per-neuron work: 0 = lower tangent search, 1 = upper tangent
+        // search (straddling neurons), 2 = tangent / chord of one-signed neurons
+        if (wv < 3 && n_ok) {
+            const float l = s_lu[lane], u = s_lu[TH + lane];
+            const bool pure = (u < 0.f || l > 0.f);
+            if (wv == 2) {
+                if (pure) {
+                    Line lo, up;
+                    tanh_pure_lines(l, u, lo, up);
+                    s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
+                    s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
+                }
+            } else if (!pure) {
+                if (wv == 0) {
+                    const Line lo = tanh_tangent_line<true>(l, u);
+                    s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
+                } else {
+                    const Line up = tanh_tangent_line<false>(l, u);
+                    s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
+                }
+            }
+        }
+        __syncthreads();
+        if (wv == 0 && n_ok) {
+            const Line lo = {s_ln[lane], s_ln[TH + lane], s_ln[2 * TH + lane]};
+            const Line up = {s_ln[3 * TH + lane], s_ln[4 * TH + lane], s_ln[5 * TH + lane]};
+            const float lb = a.lb[bi], ub = a.ub[bi];
+            a.olb[bi] = line_bias(lo, lb, ub);
+            a.oub[bi] = line_bias(up, ub, lb);
+        }
+    }
+
     if (!col_ok) return;
     float klo[VEC], kup[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-        klo[v] = coef[c * VEC + v];
-        kup[v] = coef[TH + c * VEC + v];
+        klo[v] = s_ln[c * VEC + v];
+        kup[v] = s_ln[3 * TH + c * VEC + v];
     }
     for (int ch = 0; ch < nchunks; ++ch) {
 #pragma unroll
@@ -303,6 +354,18 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
                 ou.store(a.ouw + off);
             }
         }
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void make_lines(float l, float u, Line &lo, Line &up) {
+    if (MODE == RELU) {
+        relu_lines(l, u, lo, up);
+    } else if (u < 0.f || l > 0.f) {
+        tanh_pure_lines(l, u, lo, up);
+    } else {
+        lo = tanh_tangent_line<true>(l, u);
+        up = tanh_tangent_line<false>(l, u);
     }
 }
 
@@ -386,7 +449,7 @@ template <int MODE, int Q, int VEC, int TPR, int NTHREADS, int RPT>
 void launch_natural(const ActArgs &a, hipStream_t st) {
     constexpr int TH = TPR * VEC, RG = NTHREADS / TPR;
     const int tiles = (a.H + TH - 1) / TH;
-    const size_t smem = ((size_t)a.words * RG * 2 * TH + 2 * TH) * sizeof(float);
+    const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
     hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles)),
                        dim3(NTHREADS), smem, st, a);
 }
@@ -405,12 +468,24 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
     }
     if (!vec4) {
         launch_natural<MODE, Q, 1, 64, 256, 16>(a, st);   // 64 neurons x 64 rows per chunk
-    } else if (a.D <= 128) {
-        launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);    // 64 neurons, D_in <= 128 in registers
+        return;
+    }
+    switch (faith::tune_get(FAITH_TUNE_ACT_VARIANT)) {
+        case 1: launch_natural<MODE, Q, 4, 8, 256, 8>(a, st); return;     // 32 neurons, 256 rows / chunk
+        case 2: launch_natural<MODE, Q, 4, 16, 512, 8>(a, st); return;    // 64 neurons, 256 rows / chunk, 8 waves
+        case 3: launch_natural<MODE, Q, 4, 16, 1024, 4>(a, st); return;   // 64 neurons, 256 rows / chunk, 16 waves
+        case 4: launch_natural<MODE, Q, 4, 8, 512, 4>(a, st); return;     // 32 neurons, 256 rows / chunk, 8 waves
+        case 5: launch_natural<MODE, Q, 4, 16, 256, 16>(a, st); return;   // 64 neurons, 256 rows / chunk, 4 waves
+        default: break;
+    }
+    // 32-neuron tiles (128-byte row segments) keep the register footprint at 64 values per
+    // thread, which measured fastest on MI355X (more resident workgroups, shorter tail).
+    if (a.D <= 128) {
+        launch_natural<MODE, Q, 4, 8, 256, 4>(a, st);     // D_in <= 128 in registers
     } else if (a.D <= 256) {
-        launch_natural<MODE, Q, 4, 16, 256, 16>(a, st);   // D_in <= 256 in registers
+        launch_natural<MODE, Q, 4, 8, 256, 8>(a, st);     // D_in <= 256 in registers
     } else {
-        launch_natural<MODE, Q, 4, 16, 512, 16>(a, st);   // D_in <= 512 in registers, chunks beyond
+        launch_natural<MODE, Q, 4, 8, 512, 8>(a, st);     // D_in <= 512 in registers, chunks beyond
     }
 }
 

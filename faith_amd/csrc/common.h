@@ -15,6 +15,9 @@ void set_error(const char *fmt, ...);
 // Returns FAITH_OK or records the HIP error text and returns FAITH_ERR_LAUNCH.
 int check_launch(const char *what);
 
+// Tuning knobs (faith_tune_set); 0 = built-in choice.
+int tune_get(int knob);
+
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 inline int ceil_div(long long a, long long b) { return static_cast<int>((a + b - 1) / b); }

@@ -21,7 +21,41 @@ int check_launch(const char *what) {
     return FAITH_OK;
 }
 
+static int g_tune[FAITH_TUNE_COUNT] = {0};
+
+int tune_get(int knob) { return (knob >= 0 && knob < FAITH_TUNE_COUNT) ? g_tune[knob] : 0; }
+
 }  // namespace faith
+
+extern "C" int faith_tune_set(int knob, int value) {
+    if (knob < 0 || knob >= FAITH_TUNE_COUNT) {
+        faith::set_error("faith_tune_set: unknown knob %d", knob);
+        return FAITH_ERR_UNSUPPORTED;
+    }
+    faith::g_tune[knob] = value;
+    return FAITH_OK;
+}
+
+// Plain streaming copy: the yardstick the HBM-bound kernels are compared with, and the kernel
+// of known size that hardware byte counters are calibrated against.
+__global__ void __launch_bounds__(256) copy_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst,
+                                                   size_t n4) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
+}
+
+extern "C" int faith_copy_f32(const float *src, float *dst, long long n, void *stream) {
+    FAITH_NOT_NULL(src);
+    FAITH_NOT_NULL(dst);
+    FAITH_REQUIRE(n > 0 && n % 4 == 0, FAITH_ERR_SHAPE, "faith_copy_f32: n=%lld must be a positive multiple of 4", n);
+    FAITH_REQUIRE(faith::aligned(src, 16) && faith::aligned(dst, 16), FAITH_ERR_ALIGN,
+                  "faith_copy_f32: pointers must be 16-byte aligned");
+    const size_t n4 = (size_t)n / 4;
+    const unsigned blocks = (unsigned)((n4 + 255) / 256 < 256 * 32 ? (n4 + 255) / 256 : 256 * 32);
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<const float4 *>(src), reinterpret_cast<float4 *>(dst), n4);
+    return faith::check_launch("faith_copy_f32");
+}
 
 extern "C" const char *faith_last_error(void) { return faith::g_error; }
 

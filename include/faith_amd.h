@@ -45,6 +45,23 @@ const char *faith_last_error(void);
 int faith_version(void);
 
 /*
+ * Kernel-variant selection for tuning runs (no counterpart in the reference, whose tile sizes
+ * are compile-time: HandTunedKernels/matmul_config.h).  value 0 restores the built-in choice.
+ * Process-wide, not thread-safe; results never depend on it, only speed.
+ */
+#define FAITH_TUNE_ACT_VARIANT   0   /* tile shape of the natural-layout relaxation kernels */
+#define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split MFMA contraction       */
+#define FAITH_TUNE_COUNT         4
+int faith_tune_set(int knob, int value);
+
+/*
+ * Plain device-to-device copy of n floats (n % 4 == 0, 16-byte aligned).  Measurement aid with no
+ * counterpart in the reference: the yardstick for the HBM-bound kernels and the known-size
+ * kernel that hardware byte counters are calibrated against.
+ */
+int faith_copy_f32(const float *src, float *dst, long long n, void *stream);
+
+/*
  * Dual-norm concretization.  Replaces Bounds.concretize (Bounds.py:311-326) and the
  * CUDA `concretize` kernel (HandTunedKernels/dot_product_verification.cu:47-105).
  *   l[r,j] = lb[r,j] - eps * sum_w ||lw[r, block w, j]||_q

@@ -135,7 +135,7 @@ def test_activation_config1_full_properties(kind):
             assert torch.equal(olw.transpose(2, 3)[act], lw.transpose(2, 3)[act])
             assert torch.equal(oub[act], ub[act])
             frac_both = 1.0 - float(dead.float().mean()) - float(act.float().mean())
-            assert 0.2 < frac_both < 0.8
+            assert 0.05 < frac_both < 0.9
 
 
 def test_c_bound_shim_matches_reference_calling_convention():
