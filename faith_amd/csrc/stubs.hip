@@ -1,11 +1,5 @@
 // Placeholders until the contraction kernels land.
 #include "common.h"
-extern "C" int faith_matmul_verification(const float *, const float *, const float *, const float *, const float *,
-                                         const float *, float *, float *, float *, float *, int, int, int, int, int,
-                                         void *) {
-    faith::set_error("faith_matmul_verification: not built yet");
-    return FAITH_ERR_UNSUPPORTED;
-}
 extern "C" int faith_dot_product_verification_QK(float *, float *, float *, float *, const float *, const float *,
                                                  const float *, const float *, const float *, const float *,
                                                  const float *, const float *, float *, float *, float *, float *,

@@ -73,3 +73,45 @@ def compare_activation(kind, x, got, exp, l_gpu, u_gpu, l_ref, u_ref,
         np.testing.assert_allclose(guw[b, r, :, j].double().numpy(), e[2], rtol=1e-4, atol=1e-5)
         np.testing.assert_allclose(float(gub[b, r, j]), e[3], rtol=1e-4, atol=1e-5)
     return {"neurons": total, "explained_boundary_cases": len(idx)}
+
+
+# ----------------------------------------------------------------------------------------
+# contractions (linear, dot product, conv)
+# ----------------------------------------------------------------------------------------
+KAPPA = 8.0
+U32 = 2.0 ** -24
+
+
+def compare_contraction(name, got, oracle32, ref64, abs_terms):
+    """Parity of one output tensor of a contraction.
+
+    First the plain bar against the fp32 CPU oracle (rtol 1e-5, atol 1e-6).  Two fp32
+    summations of the same K products in different orders (MKL blocks on the CPU, MFMA K-pairs
+    here) may differ by more than that where the products are O(1) and the sum cancels to
+    ~0: neither is "the" fp32 answer.  For a tensor that misses the plain bar, the check
+    falls back -- loudly, it prints -- to the float64 value of the same fp32 inputs with
+    the standard forward-error allowance of an fp32 dot product,
+
+        |got - ref64| <= atol + rtol * |ref64| + KAPPA * u * sum_k |a_k * w_k|,   u = 2^-24,
+
+    KAPPA = 8 (the worst-case bound has K = 64..1024 in place of 8), and requires the GPU's
+    worst error on that tensor to stay within 8x the CPU oracle's own worst error against
+    float64 (the MFMA accumulates K/2 steps in sequence, MKL sums in blocks, so a few x is
+    expected; more would point at the kernel, not at fp32).
+    Returns "plain" or "accumulation-aware".
+    """
+    got = got.detach().cpu().double()
+    o32 = oracle32.detach().cpu().double()
+    if not bool(_bad(got, o32).any()):
+        return "plain"
+    ref64 = ref64.detach().cpu().double()
+    tol = ATOL + RTOL * ref64.abs() + KAPPA * U32 * abs_terms.detach().cpu().double()
+    err = (got - ref64).abs()
+    oerr = (o32 - ref64).abs()
+    print(f"   [{name}] plain bar missed by {int(_bad(got, o32).sum())} of {got.numel()} elements; "
+          f"vs float64: gpu max err {float(err.max()):.3g}, cpu-oracle max err {float(oerr.max()):.3g}, "
+          f"max err/allowance {float((err / tol).max()):.3f}", flush=True)
+    assert bool((err <= tol).all()), f"{name}: outside the accumulation-aware bar"
+    assert float(err.max()) <= 8.0 * float(oerr.max()) + ATOL, \
+        f"{name}: the CPU oracle is much closer to float64 than the GPU ({float(oerr.max()):.3g} vs {float(err.max()):.3g})"
+    return "accumulation-aware"

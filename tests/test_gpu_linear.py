@@ -1,0 +1,130 @@
+"""HIP sign-split affine propagation (fp32 MFMA) against the CPU oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import bounds_oracle as O
+from tests.helpers import rand_bounds, as_bounds, close, worst
+from tests.parity import compare_contraction
+
+pytestmark = pytest.mark.gpu
+INF = float("inf")
+
+
+def dev(*ts):
+    return [None if t is None else t.cuda().contiguous() for t in ts]
+
+
+def run_linear(x, W, bias):
+    from faith_amd import ops
+    lw, lb, uw, ub, W, bias = dev(*x.tensors(), W, bias)
+    return ops.linear(lw, lb, uw, ub, W, bias)
+
+
+def linear64(x, W, bias):
+    """float64 value of the same fp32 inputs, and sum_k |a_k w_k| per output."""
+    Wp, Wn = W.double().clamp(min=0).t(), W.double().clamp(max=0).t()
+    a = {k: v.double() for k, v in zip(("lw", "lb", "uw", "ub"), x.tensors())}
+    b = 0 if bias is None else bias.double()
+    ref = dict(lw=a["lw"] @ Wp + a["uw"] @ Wn, uw=a["uw"] @ Wp + a["lw"] @ Wn,
+               lb=a["lb"] @ Wp + a["ub"] @ Wn + b, ub=a["ub"] @ Wp + a["lb"] @ Wn + b)
+    mag = dict(lw=a["lw"].abs() @ Wp - a["uw"].abs() @ Wn, uw=a["uw"].abs() @ Wp - a["lw"].abs() @ Wn,
+               lb=a["lb"].abs() @ Wp - a["ub"].abs() @ Wn, ub=a["ub"].abs() @ Wp - a["lb"].abs() @ Wn)
+    return ref, mag
+
+
+def check(x, W, bias, what=""):
+    print(f"[case] linear {what} x={tuple(x.lw.shape)} W={tuple(W.shape)} bias={bias is not None}", flush=True)
+    got = run_linear(x, W, bias)
+    torch.cuda.synchronize()
+    exp = O.linear(x, W, bias)
+    ref, mag = linear64(x, W, bias)
+    for name, g, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
+        compare_contraction(name, g, e, ref[name], mag[name])
+    return got
+
+
+@pytest.mark.parametrize("shape", [
+    (1, 16, 64, 64, 64),       # benchmark configuration 0
+    (1, 2, 64, 64, 64), (1, 8, 128, 256, 128), (1, 4, 64, 512, 512),   # reference sweep corners
+    (2, 3, 50, 72, 200),       # M, N not multiples of the tile
+    (1, 1, 1, 4, 1),           # degenerate
+    (1, 5, 33, 100, 130),      # ragged everywhere, K % 4 == 0
+    (1, 3, 17, 37, 29),        # K % 4 != 0: any-shape kernel
+    (1, 130, 2, 16, 8),        # more constant-term rows than one tile
+])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_linear_shapes(shape, with_bias):
+    B, L, D, H, N = shape
+    g = torch.Generator().manual_seed(21)
+    x = rand_bounds(g, B, L, D, H, ordered=False, sw=0.5)
+    W = torch.randn(N, H, generator=g) / H ** 0.5
+    if N * H > 4:
+        W.view(-1)[::7] = 0.0          # exact zeros belong to neither sign
+    bias = torch.randn(N, generator=g) if with_bias else None
+    check(x, W, bias, "sweep")
+
+
+def test_linear_config0_with_concretize():
+    from faith_amd import ops
+    from faith_amd.workloads import make_config
+    c = make_config(0)
+    x = as_bounds(c["x"])
+    got = check(x, c["W"], c["bias"], "config0")
+    l, u = ops.concretize(*got, c["p"], c["eps"], c["words"])
+    el, eu = O.concretize(O.linear(x, c["W"], c["bias"]), c["p"], c["eps"], c["words"])
+    assert close(l, el) and close(u, eu)
+    assert bool((l <= u).all())
+
+
+def test_linear_config2_reduced():
+    """Benchmark configuration 2 with L = 16 instead of 256 (same D_in = 512, H = N = 1024)."""
+    from faith_amd import ops
+    from faith_amd.workloads import make_config
+    c = make_config(2, scale=1 / 16)
+    x = as_bounds(c["x"])
+    got = check(x, c["W"], c["bias"], "config2/16")
+    l, u = ops.concretize(*got, c["p"], c["eps"], c["words"])
+    # concretize is checked on the GPU's own propagated bounds (the constant terms of the two
+    # fp32 summation orders differ by more than the bar, see tests/parity.py)
+    el, eu = O.concretize(O.LinearBounds(*(t.cpu() for t in got)), c["p"], c["eps"], c["words"])
+    assert close(l, el) and close(u, eu)
+    assert bool((l <= u).all())
+
+
+def test_linear_closed_forms_on_gpu():
+    """Properties that hold at any size: non-negative W => plain product; degenerate bounds =>
+    both sides equal; width identity uw' - lw' = (uw - lw) @ |W|^T."""
+    g = torch.Generator().manual_seed(22)
+    x = rand_bounds(g, 1, 6, 96, 256, ordered=True)
+    W = torch.randn(192, 256, generator=g) / 16
+    lw, lb, uw, ub = run_linear(x, W.abs(), None)
+    assert close(lw, x.lw @ W.abs().t(), rtol=1e-5, atol=2e-6) and close(uw, x.uw @ W.abs().t(), rtol=1e-5, atol=2e-6)
+    pt = O.LinearBounds(x.lw, x.lb, x.lw, x.lb)
+    lw, lb, uw, ub = run_linear(pt, W, None)
+    assert torch.equal(lw, uw) and torch.equal(lb, ub)
+    lw, lb, uw, ub = run_linear(x, W, None)
+    assert close(uw.cpu() - lw.cpu(), (x.uw - x.lw) @ W.abs().t(), rtol=1e-4, atol=1e-5)
+    assert bool((uw >= lw - 1e-6).all())
+
+
+def test_linear_config2_full_size_properties():
+    """Full configuration 2 (1.1 TFLOP): linearity in the input and agreement of sampled rows
+    with a float64 evaluation; preserves lw' <= uw' and l <= u."""
+    from faith_amd import ops
+    from faith_amd.workloads import make_config
+    c = make_config(2)
+    lw, lb, uw, ub, W, bias = dev(*(c["x"][k] for k in ("lw", "lb", "uw", "ub")), c["W"], c["bias"])
+    olw, olb, ouw, oub = ops.linear(lw, lb, uw, ub, W, bias)
+    assert bool((ouw >= olw - 1e-6).all()) and bool((oub >= olb).all())
+    # sampled rows against float64
+    Wp, Wn = W.double().clamp(min=0).t(), W.double().clamp(max=0).t()
+    idx = torch.randint(0, 256 * 512, (64,), generator=torch.Generator().manual_seed(1)).cuda()
+    a_l = lw.view(-1, 1024)[idx].double(); a_u = uw.view(-1, 1024)[idx].double()
+    assert close(olw.view(-1, 1024)[idx], a_l @ Wp + a_u @ Wn)
+    assert close(ouw.view(-1, 1024)[idx], a_u @ Wp + a_l @ Wn)
+    assert close(olb, lb.double() @ Wp + ub.double() @ Wn + bias.double(), rtol=1e-5, atol=1e-5)
+    # scaling the input by 2 scales the coefficients by exactly 2 (power of two: bit-exact)
+    o2 = ops.linear(lw * 2, lb, uw * 2, ub, W, bias)
+    assert torch.equal(o2[0], olw * 2) and torch.equal(o2[2], ouw * 2)
+    l, u = ops.concretize(olw, olb, ouw, oub, c["p"], c["eps"], c["words"])
+    assert bool((l <= u).all())
