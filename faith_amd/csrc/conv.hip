@@ -1,0 +1,259 @@
+// Sign-split bound propagation through a 2-D convolution, as an implicit GEMM on fp32 MFMA.
+//
+// Semantics from the reference's verify_conv and its launcher
+// (HandTunedKernels/convolution_verification.cu:124-138, :219-239): a positive tap multiplies the
+// same-side bound, a non-positive tap the opposite one,
+//     y_l = conv(x_l, W+) + conv(x_u, W-)        y_u = conv(x_u, W+) + conv(x_l, W-)
+// applied to (lb, ub) with the real batch and to (lw, uw) with D_in as the batch.  NCHW,
+// W [C_out, C_in, K, K], zero padding.  (The reference kernel itself is unfinished -- it drops
+// the last K-tile, ignores the tile origin in its padding test and never stores; the arithmetic
+// above is what it sets out to compute.)
+//
+// Implicit GEMM:  C[co, p] = sum_k W[co, k] * X[k, p],  k = (ci, kh, kw),  p = output pixel.
+// MFMA rows are output channels (W is the sign-split operand), MFMA columns are pixels (x_l / x_u
+// is the paired operand), so lanes run along ow and every store is a contiguous run of a
+// channel plane -- NCHW needs no transposition.
+//
+// Workgroup = 4 wavefronts on 128 channels x (4 output rows x 32 output columns) of one image;
+// wavefront tile 64 channels x 2 rows.  The reduction walks C_in in chunks of 4 channels.  Per
+// chunk the LDS holds
+//   * the input patch of both bounds: [2][4][(4-1)*stride + K][(32-1)*stride + K], out-of-image
+//     positions stored as exact zeros (so padding contributes +0 to both products), each input
+//     element fetched from global memory once and reused by up to K*K taps;
+//   * the weight slab [128][4*K*K] (row padded to an odd length: conflict-free column reads).
+// No im2col matrix is ever formed: the B fragment of tap (kh, kw) is the patch read at a
+// shifted offset.  One MFMA K-pair is (ci, tap) on lanes 0-31 and (ci + 2, tap) on lanes 32-63,
+// which turns the half-wave distinction into a per-lane constant offset.
+//
+// The constant-term path (batch images, 1/D_in of the work, O(1) cancelling terms) runs in a
+// direct kernel that accumulates in double and adds the bias.
+#include "common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int TCO = 128;      // output channels per workgroup
+constexpr int TR = 4;         // output rows per workgroup
+constexpr int TC = 32;        // output columns per workgroup
+constexpr int CC = 4;         // input channels per reduction chunk
+constexpr int NTHREADS = 256;
+
+struct ConvArgs {
+    const float *xl, *xu;     // [N, Ci, H, W]
+    const float *w;           // [Co, Ci, K, K]
+    const float *bias;        // [Co] or nullptr
+    float *yl, *yu;           // [N, Co, Ho, Wo]
+    int N, Ci, H, W, Co, K, S, P, Ho, Wo;
+};
+
+__device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+conv_signsplit(const ConvArgs g) {
+    extern __shared__ float smem[];
+    const int KK = g.K * g.K;
+    const int prow = (TR - 1) * g.S + g.K, pcol = (TC - 1) * g.S + g.K;
+    const int PP = prow * pcol;                  // one channel plane of the patch
+    const int WS = (CC * KK) | 1;                // weight row length, odd
+    float *sXl = smem;                           // [CC][prow][pcol]
+    float *sXu = sXl + CC * PP;
+    float *sW = sXu + CC * PP;                   // [TCO][WS]
+
+    const int tcol = (g.Wo + TC - 1) / TC, trow = (g.Ho + TR - 1) / TR, tco = (g.Co + TCO - 1) / TCO;
+    int pid = blockIdx.x;
+    const int ow0 = (pid % tcol) * TC;  pid /= tcol;
+    const int oh0 = (pid % trow) * TR;  pid /= trow;
+    const int co0 = (pid % tco) * TCO;  pid /= tco;
+    const int n = pid;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wv = tid / 64;
+    const int wm = wv / 2, wn = wv % 2;          // wm: channel half, wn: row pair
+    const int fi = lane % 32, fh = lane / 32;
+
+    const int ih0 = oh0 * g.S - g.P, iw0 = ow0 * g.S - g.P;
+    const size_t img = (size_t)g.H * g.W;
+    const float *xl_n = g.xl + (size_t)n * g.Ci * img;
+    const float *xu_n = g.xu + (size_t)n * g.Ci * img;
+
+    // per-lane fragment offsets
+    int xoff[2], woff[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) xoff[b] = fh * (CC / 2) * PP + ((wn * 2 + b) * g.S) * pcol + fi * g.S;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) woff[a] = (wm * 64 + a * 32 + fi) * WS + fh * (CC / 2) * KK;
+
+    floatx16 cl[2][2], cu[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
+
+    for (int c0 = 0; c0 < g.Ci; c0 += CC) {
+        // ---- stage the patch: a wavefront per (channel, patch row), lanes along the row
+        for (int rr = wv; rr < CC * prow; rr += NTHREADS / 64) {
+            const int ci = c0 + rr / prow, pr = rr % prow;
+            const int ih = ih0 + pr;
+            const bool row_ok = ci < g.Ci && ih >= 0 && ih < g.H;
+            const size_t rbase = (size_t)ci * img + (size_t)ih * g.W;
+            for (int pc = lane; pc < pcol; pc += 64) {
+                const int iw = iw0 + pc;
+                const bool ok = row_ok && iw >= 0 && iw < g.W;
+                sXl[rr * pcol + pc] = ok ? xl_n[rbase + iw] : 0.f;
+                sXu[rr * pcol + pc] = ok ? xu_n[rbase + iw] : 0.f;
+            }
+        }
+        // ---- stage the weight slab: CC*KK contiguous floats per output channel
+        {
+            const int per = CC * KK;
+            for (int e = tid; e < TCO * per; e += NTHREADS) {
+                const int co = e / per, kk = e % per;
+                const bool ok = co0 + co < g.Co && c0 + kk / KK < g.Ci;
+                sW[co * WS + kk] = ok ? g.w[((size_t)(co0 + co) * g.Ci + c0) * KK + kk] : 0.f;
+            }
+        }
+        __syncthreads();
+
+        // ---- multiply: (CC/2) channel pairs x K*K taps, 16 MFMAs each
+        for (int cp = 0; cp < CC / 2; ++cp) {
+            int tap = 0;
+            for (int kh = 0; kh < g.K; ++kh) {
+                for (int kw = 0; kw < g.K; ++kw, ++tap) {
+                    const int xo = cp * PP + kh * pcol + kw;
+                    const int wo = cp * KK + tap;
+                    float wp[2], wq[2], xl[2], xu[2];
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+                        const float w = sW[woff[a] + wo];
+                        wp[a] = fmaxf(w, 0.f);
+                        wq[a] = fminf(w, 0.f);
+                    }
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        xl[b] = sXl[xoff[b] + xo];
+                        xu[b] = sXu[xoff[b] + xo];
+                    }
+#pragma unroll
+                    for (int a = 0; a < 2; ++a)
+#pragma unroll
+                        for (int b = 0; b < 2; ++b) {
+                            cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
+                            cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
+                        }
+#pragma unroll
+                    for (int a = 0; a < 2; ++a)
+#pragma unroll
+                        for (int b = 0; b < 2; ++b) {
+                            cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
+                            cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                        }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: register r of a block is channel 8*(r/4) + 4*(lane/32) + r%4, pixel lane%32
+    const int ow = ow0 + fi;
+    if (ow >= g.Wo) return;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int oh = oh0 + wn * 2 + b;
+        if (oh >= g.Ho) continue;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+                if (co < g.Co) {
+                    const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
+                    g.yl[o] = cl[a][b][r];
+                    g.yu[o] = cu[a][b][r];
+                }
+            }
+        }
+    }
+}
+
+// Direct convolution, one thread per output, products and sums in double; adds the bias.
+__global__ void __launch_bounds__(256) conv_direct(const ConvArgs g) {
+    const size_t total = (size_t)g.N * g.Co * g.Ho * g.Wo;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int ow = idx % g.Wo;
+    const int oh = (idx / g.Wo) % g.Ho;
+    const int co = (idx / ((size_t)g.Wo * g.Ho)) % g.Co;
+    const int n = idx / ((size_t)g.Wo * g.Ho * g.Co);
+    double sl = 0.0, su = 0.0;
+    for (int ci = 0; ci < g.Ci; ++ci) {
+        const float *xl = g.xl + ((size_t)n * g.Ci + ci) * g.H * g.W;
+        const float *xu = g.xu + ((size_t)n * g.Ci + ci) * g.H * g.W;
+        const float *w = g.w + ((size_t)co * g.Ci + ci) * g.K * g.K;
+        for (int kh = 0; kh < g.K; ++kh) {
+            const int ih = oh * g.S - g.P + kh;
+            if (ih < 0 || ih >= g.H) continue;
+            for (int kw = 0; kw < g.K; ++kw) {
+                const int iw = ow * g.S - g.P + kw;
+                if (iw < 0 || iw >= g.W) continue;
+                const float wv = w[kh * g.K + kw];
+                const double wp = fmaxf(wv, 0.f), wq = fminf(wv, 0.f);
+                const double a = xl[ih * g.W + iw], b = xu[ih * g.W + iw];
+                sl += wp * a + wq * b;
+                su += wp * b + wq * a;
+            }
+        }
+    }
+    const float add = g.bias ? g.bias[co] : 0.f;
+    g.yl[idx] = (float)sl + add;
+    g.yu[idx] = (float)su + add;
+}
+
+}  // namespace
+
+extern "C" int faith_convolution_verification(const float *x_lb, const float *x_ub, const float *x_lw,
+                                              const float *x_uw, const float *W, const float *bias, float *y_lb,
+                                              float *y_ub, float *y_lw, float *y_uw, int batch_size, int Height,
+                                              int Width, int CIN, int COUT, int K, int Stride, int padding_size,
+                                              int dim_in, void *stream) {
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(W);
+    FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_ALIGNED4(x_lb); FAITH_ALIGNED4(x_ub); FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(W);
+    FAITH_ALIGNED4(bias); FAITH_ALIGNED4(y_lb); FAITH_ALIGNED4(y_ub); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_REQUIRE(batch_size > 0 && Height > 0 && Width > 0 && CIN > 0 && COUT > 0 && K > 0 && Stride > 0 &&
+                      padding_size >= 0 && dim_in > 0,
+                  FAITH_ERR_SHAPE,
+                  "faith_convolution_verification: batch=%d H=%d W=%d CIN=%d COUT=%d K=%d stride=%d pad=%d dim_in=%d",
+                  batch_size, Height, Width, CIN, COUT, K, Stride, padding_size, dim_in);
+    const int Ho = (Height + 2 * padding_size - K) / Stride + 1, Wo = (Width + 2 * padding_size - K) / Stride + 1;
+    FAITH_REQUIRE(Height + 2 * padding_size >= K && Width + 2 * padding_size >= K && Ho > 0 && Wo > 0,
+                  FAITH_ERR_SHAPE, "faith_convolution_verification: kernel %d larger than the padded input", K);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    // coefficients: D_in images through the MFMA kernel
+    ConvArgs gw{x_lw, x_uw, W, nullptr, y_lw, y_uw, dim_in, CIN, Height, Width, COUT, K, Stride, padding_size, Ho, Wo};
+    const int prow = (TR - 1) * Stride + K, pcol = (TC - 1) * Stride + K;
+    const size_t smem = ((size_t)2 * CC * prow * pcol + (size_t)TCO * ((CC * K * K) | 1)) * sizeof(float);
+    FAITH_REQUIRE(smem <= 160 * 1024, FAITH_ERR_UNSUPPORTED,
+                  "faith_convolution_verification: K=%d stride=%d needs %zu bytes of LDS per workgroup (limit 163840)",
+                  K, Stride, smem);
+    if (smem > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(conv_signsplit),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        FAITH_REQUIRE(e == hipSuccess, FAITH_ERR_LAUNCH, "faith_convolution_verification: cannot reserve %zu bytes of LDS (%s)",
+                      smem, hipGetErrorString(e));
+    }
+    const long long grid = (long long)dim_in * ((COUT + TCO - 1) / TCO) * ((Ho + TR - 1) / TR) * ((Wo + TC - 1) / TC);
+    FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_convolution_verification: grid too large");
+    hipLaunchKernelGGL(conv_signsplit, dim3((unsigned)grid), dim3(NTHREADS), smem, st, gw);
+
+    // constant terms: batch images through the exact-accumulation kernel, bias added
+    ConvArgs gb{x_lb, x_ub, W, bias, y_lb, y_ub, batch_size, CIN, Height, Width, COUT, K, Stride, padding_size, Ho, Wo};
+    const long long nb = (long long)batch_size * COUT * Ho * Wo;
+    hipLaunchKernelGGL(conv_direct, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, st, gb);
+    return faith::check_launch("faith_convolution_verification");
+}

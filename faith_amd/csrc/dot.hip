@@ -1,0 +1,318 @@
+// McCormick bounds of the attention scores  z[i, j] = sum_k x[i, k] * y[j, k]  on fp32 MFMA.
+//
+// Arithmetic of the reference's Bounds.ori_dot_product with get_bounds_xy
+// (Transformer_Verification_Code/Verifiers/Bounds.py:666-688, :710-823).  With the concrete
+// intervals [l_x, u_x] of x and [l_y, u_y] of y, the planes are
+//     x*y >= a_l x + b y - a_l b,   x*y <= a_u x + b y - a_u b,   a_l = l_y, a_u = u_y, b = l_x
+// (b = l_x on both sides, as the reference has it), and each plane is pushed through the linear
+// bounds of x and y by the sign of its coefficient.  For a fixed perturbation coordinate m this
+// is one [Lx x Ly] tile with a reduction over d:
+//   z_lw[i,m,j] = sum_k  xlw[i,m,k] a_l+[j,k] + xuw[i,m,k] a_l-[j,k] + b+[i,k] ylw[j,m,k] + b-[i,k] yuw[j,m,k]
+//   z_uw[i,m,j] = sum_k  xuw[i,m,k] a_u+[j,k] + xlw[i,m,k] a_u-[j,k] + b+[i,k] yuw[j,m,k] + b-[i,k] ylw[j,m,k]
+// i.e. eight MFMA products per K-pair into two accumulators.  Rows (i) come from x and b, columns
+// (j) from a and y, so the accumulator tile is already laid out as z[i, m, j..]: lanes run along j
+// and every store is a 128-byte run.  Neither the [Lx, D, d, Ly] broadcast the PyTorch code
+// materialises nor the transposed add of its y-terms exists here.
+//
+// Tiling: workgroup = 4 wavefronts on a 128 x 128 (i x j) tile of one (head, m); wavefront tile
+// 64 x 64 (2 x 2 blocks of v_mfma_f32_32x32x2_f32, for each of z_lw and z_uw).  K-step 8:
+// seven operand tiles [128 x 8] per step (xlw, xuw, b | a_l, a_u, ylw, yuw) = 28 KB, double
+// buffered = 56 KB, so two workgroups share a CU.  Rows are 8 floats with the two 16-byte halves
+// swapped on every other group of four rows, which makes both the 16-byte stores and the 16-byte
+// fragment reads bank-conflict free without padding.  a / b are split by sign after the LDS
+// read (v_max / v_min); they are staged from the concretization results, unsplit.
+//
+// The constant terms z_lb / z_ub ([Lx, Ly] per head, 1/D_in of the work, O(1) cancelling terms)
+// are summed in double by a small kernel.
+#include "common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int TI = 128, TJ = 128, BK = 8;
+constexpr int NTHREADS = 256;
+constexpr int TILE = 128 * BK;            // floats per operand tile
+
+struct DotArgs {
+    const float *xlw, *xuw, *ylw, *yuw;   // [B, Lx, D, d], [B, Ly, D, d]
+    const float *xlb, *xub, *ylb, *yub;   // [B, Lx, d], [B, Ly, d]
+    const float *x_l, *y_l, *y_u;         // concrete intervals: b = x_l, a_l = y_l, a_u = y_u
+    float *zlw, *zuw;                     // [B, Lx, D, Ly]
+    float *zlb, *zub;                     // [B, Lx, Ly]
+    int B, Lx, Ly, D, d;
+};
+
+__device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 pos4(float4 v) {
+    return make_float4(fmaxf(v.x, 0.f), fmaxf(v.y, 0.f), fmaxf(v.z, 0.f), fmaxf(v.w, 0.f));
+}
+__device__ __forceinline__ float4 neg4(float4 v) {
+    return make_float4(fminf(v.x, 0.f), fminf(v.y, 0.f), fminf(v.z, 0.f), fminf(v.w, 0.f));
+}
+
+// position of 16-byte half `c` (0 / 1) of row `row` inside an [128 x 8] tile
+__device__ __forceinline__ int swz(int row, int c) { return row * BK + 4 * (c ^ ((row >> 2) & 1)); }
+
+enum { XL = 0, XU, BT, AL, AU, YL, YU, NOPS };
+
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+dot_qk_w(const DotArgs g) {
+    __shared__ float sm[2][NOPS][TILE];
+
+    const int ti = (g.Lx + TI - 1) / TI, tj = (g.Ly + TJ - 1) / TJ;
+    int pid = blockIdx.x;
+    const int j0 = (pid % tj) * TJ;  pid /= tj;
+    const int i0 = (pid % ti) * TI;  pid /= ti;
+    const int m = pid % g.D;
+    const int t = pid / g.D;
+    const int d = g.d;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wv = tid / 64;
+    const int wi = wv / 2, wj = wv % 2;
+
+    // ---- staging: one float4 per operand per thread per K-step
+    const int srow = tid / 2, sc = tid % 2;
+    const int irow = min(i0 + srow, g.Lx - 1), jrow = min(j0 + srow, g.Ly - 1);   // clamped rows are never stored
+    const float *src[NOPS];
+    src[XL] = g.xlw + ((size_t)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
+    src[XU] = g.xuw + ((size_t)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
+    src[BT] = g.x_l + (size_t)(t * g.Lx + irow) * d + sc * 4;
+    src[AL] = g.y_l + (size_t)(t * g.Ly + jrow) * d + sc * 4;
+    src[AU] = g.y_u + (size_t)(t * g.Ly + jrow) * d + sc * 4;
+    src[YL] = g.ylw + ((size_t)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
+    src[YU] = g.yuw + ((size_t)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
+    const int sdst = swz(srow, sc);
+    float4 pre[NOPS];
+    auto gload = [&](int kt) {
+        const int k = kt * BK;
+        const bool in = k + sc * 4 < d;            // d % 4 == 0
+#pragma unroll
+        for (int o = 0; o < NOPS; ++o) pre[o] = in ? ld4(src[o] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int o = 0; o < NOPS; ++o) *reinterpret_cast<float4 *>(&sm[buf][o][sdst]) = pre[o];
+    };
+
+    floatx16 cl[2][2], cu[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
+
+    const int fi = lane % 32, fh = lane / 32;
+    int fa[2], fb[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        fa[s] = swz(wi * 64 + s * 32 + fi, fh);
+        fb[s] = swz(wj * 64 + s * 32 + fi, fh);
+    }
+
+    const int nk = (d + BK - 1) / BK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload(kt + 1);
+        float4 xl[2], xu[2], bp[2], bn[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            xl[s] = *reinterpret_cast<const float4 *>(&sm[buf][XL][fa[s]]);
+            xu[s] = *reinterpret_cast<const float4 *>(&sm[buf][XU][fa[s]]);
+            const float4 bt = *reinterpret_cast<const float4 *>(&sm[buf][BT][fa[s]]);
+            bp[s] = pos4(bt);
+            bn[s] = neg4(bt);
+        }
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const float4 al = *reinterpret_cast<const float4 *>(&sm[buf][AL][fb[b]]);
+            const float4 au = *reinterpret_cast<const float4 *>(&sm[buf][AU][fb[b]]);
+            const float4 yl = *reinterpret_cast<const float4 *>(&sm[buf][YL][fb[b]]);
+            const float4 yu = *reinterpret_cast<const float4 *>(&sm[buf][YU][fb[b]]);
+            const float4 alp = pos4(al), aln = neg4(al), aup = pos4(au), aun = neg4(au);
+#define FAITH_DOT_STEP(c)                                   \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a][b] = mfma(xl[a].c, alp.c, cl[a][b]);          \
+        cu[a][b] = mfma(xu[a].c, aup.c, cu[a][b]);          \
+    }                                                       \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a][b] = mfma(xu[a].c, aln.c, cl[a][b]);          \
+        cu[a][b] = mfma(xl[a].c, aun.c, cu[a][b]);          \
+    }                                                       \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a][b] = mfma(bp[a].c, yl.c, cl[a][b]);           \
+        cu[a][b] = mfma(bp[a].c, yu.c, cu[a][b]);           \
+    }                                                       \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a][b] = mfma(bn[a].c, yu.c, cl[a][b]);           \
+        cu[a][b] = mfma(bn[a].c, yl.c, cu[a][b]);           \
+    }
+            FAITH_DOT_STEP(x)
+            FAITH_DOT_STEP(y)
+            FAITH_DOT_STEP(z)
+            FAITH_DOT_STEP(w)
+#undef FAITH_DOT_STEP
+        }
+        if (kt + 1 < nk) lstore(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: z[t, i, m, j]; register r of a block is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int j = j0 + wj * 64 + b * 32 + fi;
+        if (j >= g.Ly) continue;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + wi * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+                if (i < g.Lx) {
+                    const size_t o = ((size_t)(t * g.Lx + i) * g.D + m) * g.Ly + j;
+                    g.zlw[o] = cl[a][b][r];
+                    g.zuw[o] = cu[a][b][r];
+                }
+            }
+        }
+    }
+}
+
+// Any-shape coefficient kernel (d not a multiple of 4, unaligned pointers): one thread per
+// (i, m, j), products and sums in double.
+__global__ void __launch_bounds__(256) dot_qk_w_simple(const DotArgs g) {
+    const size_t total = (size_t)g.B * g.Lx * g.D * g.Ly;
+    for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+        const int j = idx % g.Ly;
+        const int m = (idx / g.Ly) % g.D;
+        const int i = (idx / ((size_t)g.Ly * g.D)) % g.Lx;
+        const int t = idx / ((size_t)g.Ly * g.D * g.Lx);
+        const float *xl = g.xlw + ((size_t)(t * g.Lx + i) * g.D + m) * g.d;
+        const float *xu = g.xuw + ((size_t)(t * g.Lx + i) * g.D + m) * g.d;
+        const float *yl = g.ylw + ((size_t)(t * g.Ly + j) * g.D + m) * g.d;
+        const float *yu = g.yuw + ((size_t)(t * g.Ly + j) * g.D + m) * g.d;
+        const float *bt = g.x_l + (size_t)(t * g.Lx + i) * g.d;
+        const float *al = g.y_l + (size_t)(t * g.Ly + j) * g.d;
+        const float *au = g.y_u + (size_t)(t * g.Ly + j) * g.d;
+        double sl = 0.0, su = 0.0;
+        for (int k = 0; k < g.d; ++k) {
+            const double bp = fmaxf(bt[k], 0.f), bn = fminf(bt[k], 0.f);
+            const double alp = fmaxf(al[k], 0.f), aln = fminf(al[k], 0.f);
+            const double aup = fmaxf(au[k], 0.f), aun = fminf(au[k], 0.f);
+            sl += xl[k] * alp + xu[k] * aln + bp * yl[k] + bn * yu[k];
+            su += xu[k] * aup + xl[k] * aun + bp * yu[k] + bn * yl[k];
+        }
+        g.zlw[idx] = (float)sl;
+        g.zuw[idx] = (float)su;
+    }
+}
+
+// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): one thread per (head, i, j).
+__global__ void __launch_bounds__(256) dot_qk_b(const DotArgs g) {
+    const size_t total = (size_t)g.B * g.Lx * g.Ly;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int j = idx % g.Ly;
+    const int i = (idx / g.Ly) % g.Lx;
+    const int t = idx / ((size_t)g.Ly * g.Lx);
+    const size_t xo = (size_t)(t * g.Lx + i) * g.d, yo = (size_t)(t * g.Ly + j) * g.d;
+    double sl = 0.0, su = 0.0;
+    for (int k = 0; k < g.d; ++k) {
+        const double bt = g.x_l[xo + k], al = g.y_l[yo + k], au = g.y_u[yo + k];
+        const double xlb = g.xlb[xo + k], xub = g.xub[xo + k], ylb = g.ylb[yo + k], yub = g.yub[yo + k];
+        const double bp = bt > 0 ? bt : 0, bn = bt < 0 ? bt : 0;
+        sl += -al * bt + (al > 0 ? al * xlb : al * xub) + bp * ylb + bn * yub;
+        su += -au * bt + (au > 0 ? au * xub : au * xlb) + bp * yub + bn * ylb;
+    }
+    g.zlb[idx] = (float)sl;
+    g.zub[idx] = (float)su;
+}
+
+// dim_in == 1: the reference switches to plain interval arithmetic on the constant terms and
+// returns zero coefficients (Bounds.py:711-721).
+__global__ void __launch_bounds__(256) dot_qk_interval(const DotArgs g) {
+    const size_t total = (size_t)g.B * g.Lx * g.Ly;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int j = idx % g.Ly;
+    const int i = (idx / g.Ly) % g.Lx;
+    const int t = idx / ((size_t)g.Ly * g.Lx);
+    const size_t xo = (size_t)(t * g.Lx + i) * g.d, yo = (size_t)(t * g.Ly + j) * g.d;
+    float lo = 0.f, hi = 0.f;
+    for (int k = 0; k < g.d; ++k) {
+        const float l1 = g.xlb[xo + k], u1 = g.xub[xo + k], l2 = g.ylb[yo + k], u2 = g.yub[yo + k];
+        const float c1 = l1 * l2, c2 = l1 * u2, c3 = u1 * l2, c4 = u1 * u2;
+        lo += fminf(fminf(c1, c2), fminf(c3, c4));
+        hi += fmaxf(fmaxf(c1, c2), fmaxf(c3, c4));
+    }
+    g.zlb[idx] = lo;
+    g.zub[idx] = hi;
+    g.zlw[idx] = 0.f;      // [B, Lx, 1, Ly] has the same linear index
+    g.zuw[idx] = 0.f;
+}
+
+}  // namespace
+
+extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
+                                                 const float *x_ub, const float *y_lb, const float *y_ub,
+                                                 const float *x_lw, const float *x_uw, const float *y_lw,
+                                                 const float *y_uw, float *z_lb, float *z_ub, float *z_lw,
+                                                 float *z_uw, int batch_size, int length_x, int length_y,
+                                                 int dim_out, int dim_in, float epsilon, int q, int words,
+                                                 void *stream) {
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
+    FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
+    FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_ALIGNED4(z_lw); FAITH_ALIGNED4(z_uw); FAITH_ALIGNED4(z_lb); FAITH_ALIGNED4(z_ub);
+    FAITH_REQUIRE(batch_size > 0 && length_x > 0 && length_y > 0 && dim_out > 0 && dim_in > 0, FAITH_ERR_SHAPE,
+                  "faith_dot_product_verification_QK: batch=%d length_x=%d length_y=%d dim_out=%d dim_in=%d "
+                  "must be positive", batch_size, length_x, length_y, dim_out, dim_in);
+    const long long nw = (long long)batch_size * length_x * dim_in * length_y;
+    FAITH_REQUIRE((long long)batch_size * (length_x > length_y ? length_x : length_y) * dim_in <= 0x7fffffffLL,
+                  FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: batch*length*dim_in exceeds 2^31");
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dim_in == 1) {
+        DotArgs gi{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub,
+                   batch_size, length_x, length_y, dim_in, dim_out};
+        const long long n = (long long)batch_size * length_x * length_y;
+        hipLaunchKernelGGL(dot_qk_interval, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gi);
+        return faith::check_launch("faith_dot_product_verification_QK");
+    }
+
+    // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the
+    // reference interface exposes it, the planes do not use it
+    int rc = faith_concretize(x_lb, x_ub, x_lw, x_uw, x_l, x_u, batch_size * length_x, dim_in, dim_out, epsilon, q,
+                              words, FAITH_LAYOUT_NATURAL, stream);
+    if (rc != FAITH_OK) return rc;
+    rc = faith_concretize(y_lb, y_ub, y_lw, y_uw, y_l, y_u, batch_size * length_y, dim_in, dim_out, epsilon, q,
+                          words, FAITH_LAYOUT_NATURAL, stream);
+    if (rc != FAITH_OK) return rc;
+
+    DotArgs g{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub,
+              batch_size, length_x, length_y, dim_in, dim_out};
+    const long long nb = (long long)batch_size * length_x * length_y;
+    hipLaunchKernelGGL(dot_qk_b, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, st, g);
+
+    const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
+                      faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
+                      faith::aligned(y_l, 16) && faith::aligned(y_u, 16);
+    if (fast) {
+        const long long grid = (long long)batch_size * dim_in * ((length_x + TI - 1) / TI) * ((length_y + TJ - 1) / TJ);
+        FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: grid too large");
+        hipLaunchKernelGGL(dot_qk_w, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
+    } else {
+        const long long blocks = (nw + 255) / 256;
+        hipLaunchKernelGGL(dot_qk_w_simple, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
+    }
+    return faith::check_launch("faith_dot_product_verification_QK");
+}
