@@ -1,0 +1,300 @@
+#!/usr/bin/env python3
+"""Benchmark of the forward bound-propagation hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only-headline]
+
+Prints ONE JSON line on stdout (a table for humans goes to stderr).
+
+Headline workload ("step"): benchmark configuration 1 -- the ReLU and the tanh relaxation of
+bounds lw/uw [1,128,256,512], lb/ub [1,128,512], two perturbed words, eps = 0.01, once for each
+p in {1, 2, inf}: six fused concretize+relax launches per step.  `value` is the algorithmic
+HBM traffic of a step (read lw, uw; write lw', uw'; read and write the constant terms:
+16*L*D*H + 16*L*H bytes per launch) divided by the step time, inputs resident in HBM.
+
+The same JSON line carries, under "ops", one entry per benchmark configuration (0..4) with
+latency, achieved TFLOP/s or GB/s, roofline fraction and the CPU baseline, because the metric
+is a per-op figure.
+
+`cpu_baseline` times the CPU oracle (a PyTorch restatement of the reference's Bounds methods,
+kind "port") on the host cores of the same machine; it is the checker being timed as a
+baseline, never part of the measured GPU path.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "bound-prop latency & TFLOP/s (matmul/dot/conv) or HBM GB/s (relu/tanh), % roofline"
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+INF = float("inf")
+
+# HBM bytes per launch of the dominant relaxation kernel from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE, scaled by the same counters on faith_copy_f32 of known size (see
+# profiles/act_natural_config1_pmc.md).  None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gpu_times_ms(fn, n, warmup):
+    """Per-launch durations from HIP events recorded on the launch stream (torch's current one)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for s, e in evs:
+        s.record()
+        fn()
+        e.record()
+    torch.cuda.synchronize()
+    return [s.elapsed_time(e) for s, e in evs]
+
+
+def cpu_time_s(fn, reps=1, warmup=0):
+    for _ in range(warmup):
+        fn()
+    ts = []
+    for _ in range(reps):
+        t = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t)
+    return statistics.median(ts)
+
+
+def to_dev(d):
+    return {k: v.cuda().contiguous() for k, v in d.items()}
+
+
+def quad(d):
+    return d["lw"], d["lb"], d["uw"], d["ub"]
+
+
+# ------------------------------------------------------------------------------------------
+# per-configuration measurements
+# ------------------------------------------------------------------------------------------
+def op_entry(name, kind, times_ms, work, cpu=None, extra=None):
+    """kind 'hbm': work in bytes -> GB/s; kind 'mfma': work in flop -> TFLOP/s."""
+    med = statistics.median(times_ms)
+    if kind == "hbm":
+        ach, peak, unit = work / med / 1e6, HBM_PEAK_GBS, "GB/s"
+    else:
+        ach, peak, unit = work / med / 1e9, MFMA_FP32_PEAK_TFLOPS, "TFLOP/s"
+    e = {"op": name, "latency_us": round(med * 1e3, 2), "latency_min_us": round(min(times_ms) * 1e3, 2),
+         "bound": kind, "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
+         "work": work}
+    if cpu is not None:
+        e["cpu_baseline"] = cpu
+    if extra:
+        e.update(extra)
+    return e
+
+
+def bench_config0(args, ops, O, wl):
+    c = wl.make_config(0)
+    x, W, b = to_dev(c["x"]), c["W"].cuda(), c["bias"].cuda()
+
+    def step():
+        y = ops.linear(*quad(x), W, b)
+        ops.concretize(*y, c["p"], c["eps"], 1)
+    flop = 4 * 2 * (16 * 64 + 16) * 64 * 64
+    t = gpu_times_ms(step, 200, 20)
+    cpu = None
+    if not args.no_cpu:
+        xo = O.LinearBounds(*quad(c["x"]))
+        s = cpu_time_s(lambda: O.concretize(O.linear(xo, c["W"], c["bias"]), c["p"], c["eps"]), reps=20, warmup=3)
+        cpu = {"latency_us": round(s * 1e6, 1), "value": round(flop / s / 1e12, 4), "unit": "TFLOP/s"}
+    return op_entry("config0 linear+concretize(p=inf) [1,16,64,64]x[64,64]", "mfma", t, flop, cpu,
+                    {"note": "34 MFLOP: launch-latency bound (3 launches), latency is the figure of merit"})
+
+
+def bench_config1(args, ops, O, wl, steps, warmup):
+    """Returns (headline dict, per-op entries)."""
+    import torch
+    c = wl.make_config(1)
+    x = to_dev(c["x"])
+    out = tuple(torch.empty_like(t) for t in quad(x))
+    nbytes = 16 * x["lw"].numel() + 16 * x["lb"].numel()
+    calls = [(kind, p) for kind in ("relu", "tanh") for p in c["ps"]]
+
+    def one(kind, p):
+        getattr(ops, kind)(*quad(x), p, c["eps"], c["words"], out=out)
+
+    def step():
+        for kind, p in calls:
+            one(kind, p)
+
+    # the timed region of the contract: W warm-up steps, then exactly K steps between syncs
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    entries, per_kernel = [], {}
+    for kind, p in calls:
+        t = gpu_times_ms(lambda: one(kind, p), max(steps, 50), 5)
+        per_kernel[(kind, p)] = t
+        entries.append(op_entry(f"config1 {kind} p={p:g} [1,128,256,512] words=2", "hbm", t, nbytes))
+    src = torch.empty(nbytes // 8, device="cuda")
+    dst = torch.empty_like(src)
+    from faith_amd import _lib
+    st = torch.cuda.current_stream().cuda_stream
+    tc = gpu_times_ms(lambda: _lib.call("faith_copy_f32", src.data_ptr(), dst.data_ptr(), src.numel(), st), 50, 5)
+    entries.append(op_entry("plain copy of the same byte count (yardstick, not a bound op)", "hbm", tc, nbytes))
+
+    dom = max(per_kernel, key=lambda k: statistics.mean(per_kernel[k]))
+    avg_ms = statistics.mean(per_kernel[dom])
+    roofline = {"bound": "hbm", "kernel": f"act_natural<{dom[0]}, p={dom[1]:g}>",
+                "achieved": round(nbytes / avg_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(nbytes / avg_ms / 1e6 / HBM_PEAK_GBS, 4),
+                "avg_launch_us": round(avg_ms * 1e3, 2), "bytes_per_launch": nbytes,
+                "traffic": TRAFFIC_BYTES_PER_LAUNCH}
+
+    cpu = None
+    if not args.no_cpu:
+        xo = O.LinearBounds(*quad(c["x"]))
+
+        def cpu_step():
+            for kind, p in calls:
+                getattr(O, kind)(xo, p, c["eps"], c["words"])
+        getattr(O, "relu")(xo, 2.0, c["eps"], c["words"])      # warm the allocator
+        s = cpu_time_s(cpu_step, reps=2)
+        cpu = {"value": round(len(calls) * nbytes / s / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+               "kind": "port", "sec_per_step": round(s, 3),
+               "sample": "2 full steps (6 calls each) on the identical tensors, median"}
+    head = {"value": round(len(calls) * nbytes / ms_per_step / 1e6, 1), "ms_per_step": round(ms_per_step, 4),
+            "roofline": roofline, "cpu_baseline": cpu,
+            "bytes_per_step": len(calls) * nbytes}
+    return head, entries
+
+
+def bench_config2(args, ops, O, wl):
+    import torch
+    c = wl.make_config(2)
+    x, W, b = to_dev(c["x"]), c["W"].cuda(), c["bias"].cuda()
+    L, D, H, N = 256, 512, 1024, 1024
+    out = (torch.empty(1, L, D, N, device="cuda"), torch.empty(1, L, N, device="cuda"),
+           torch.empty(1, L, D, N, device="cuda"), torch.empty(1, L, N, device="cuda"))
+    flop = 4 * 2 * (L * D + L) * H * N
+    t = gpu_times_ms(lambda: ops.linear(*quad(x), W, b, out=out), 10, 2)
+    tc = gpu_times_ms(lambda: ops.concretize(*out, c["p"], c["eps"], 1), 10, 2)
+    cpu = None
+    if not args.no_cpu:
+        # bounded sample: L = 32 of 256 rows (1/8 of the work), same D_in, H, N
+        xs = O.LinearBounds(*(t_[:, :32] for t_ in quad(c["x"])))
+        s = cpu_time_s(lambda: O.linear(xs, c["W"], c["bias"]), reps=3, warmup=1)
+        cpu = {"value": round(flop / 8 / s / 1e12, 4), "unit": "TFLOP/s", "sample": "L=32 of 256 rows, median of 3",
+               "sec_full_size_est": round(s * 8, 2)}
+    e = op_entry("config2 linear [1,256,512,1024]x[1024,1024]", "mfma", t, flop, cpu)
+    e2 = op_entry("config2 concretize(p=2) of the result", "hbm", tc, 8 * L * D * N + 16 * L * N)
+    return [e, e2]
+
+
+def bench_config3(args, ops, O, wl):
+    import torch
+    c = wl.make_config(3)
+    x, y = to_dev(c["x"]), to_dev(c["y"])
+    B, L, D, d = 4, 128, 256, 64
+    out = (torch.empty(B, L, D, L, device="cuda"), torch.empty(B, L, L, device="cuda"),
+           torch.empty(B, L, D, L, device="cuda"), torch.empty(B, L, L, device="cuda"))
+    flop = B * (8 * 2 * L * D * d * L + 8 * 2 * L * d * L)
+    t = gpu_times_ms(lambda: ops.dot_product_qk(quad(x), quad(y), c["p"], c["eps"], 1, out=out), 50, 5)
+    cpu = None
+    if not args.no_cpu:
+        xo, yo = O.LinearBounds(*quad(c["x"])), O.LinearBounds(*quad(c["y"]))
+        s = cpu_time_s(lambda: O.dot_product(xo, yo, c["p"], c["eps"]), reps=3, warmup=1)
+        cpu = {"value": round(flop / s / 1e12, 4), "unit": "TFLOP/s", "sample": "full size, median of 3",
+               "latency_ms": round(s * 1e3, 1)}
+    return op_entry("config3 dot_product QK 4 heads [4,128,256,64] (concretize + planes + contraction)",
+                    "mfma", t, flop, cpu)
+
+
+def bench_config4(args, ops, O, wl):
+    import torch
+    c = wl.make_config(4)
+    x, W, b = to_dev(c["x"]), c["W"].cuda(), c["bias"].cuda()
+    D, Ci, Co, Hh = 256, 64, 128, 32
+    out = (torch.empty(1, D, Co, Hh, Hh, device="cuda"), torch.empty(1, Co, Hh, Hh, device="cuda"),
+           torch.empty(1, D, Co, Hh, Hh, device="cuda"), torch.empty(1, Co, Hh, Hh, device="cuda"))
+    flop = 4 * 2 * (D + 1) * Co * Hh * Hh * Ci * 9
+    t = gpu_times_ms(lambda: ops.conv2d(*quad(x), W, b, 1, 1, out=out), 10, 2)
+    tc = gpu_times_ms(lambda: ops.concretize_conv(*out, c["p"], c["eps"]), 10, 2)
+    cpu = None
+    if not args.no_cpu:
+        xs = O.LinearBounds(c["x"]["lw"][:, :32], c["x"]["lb"], c["x"]["uw"][:, :32], c["x"]["ub"])
+        s = cpu_time_s(lambda: O.conv2d(xs, c["W"], c["bias"], 1, 1), reps=3, warmup=1)
+        cpu = {"value": round(4 * 2 * 33 * Co * Hh * Hh * Ci * 9 / s / 1e12, 4), "unit": "TFLOP/s",
+               "sample": "D_in=32 of 256, median of 3"}
+    e = op_entry("config4 conv3x3 64->128 [1,256,64,32,32]", "mfma", t, flop, cpu)
+    e2 = op_entry("config4 concretize(p=inf) of the result", "hbm", tc, 8 * D * Co * Hh * Hh + 16 * Co * Hh * Hh)
+    return [e, e2]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--only-headline", action="store_true", help="skip configurations 0, 2, 3, 4")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; every op is independent across the length axis and "
+              "nothing here uses a second GPU, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    from faith_amd import ops, workloads as wl
+    O = None
+    if not args.no_cpu:
+        from oracle import bounds_oracle as O     # cpu_baseline leg only
+
+    prop = torch.cuda.get_device_properties(0)
+    log(f"device: {prop.name}, {prop.multi_processor_count} CUs, host threads {torch.get_num_threads()}")
+
+    head, entries = bench_config1(args, ops, O, wl, args.steps, args.warmup)
+    if not args.only_headline:
+        entries = [bench_config0(args, ops, O, wl)] + entries
+        entries += bench_config2(args, ops, O, wl)
+        entries.append(bench_config3(args, ops, O, wl))
+        entries += bench_config4(args, ops, O, wl)
+
+    for e in entries:
+        cb = e.get("cpu_baseline")
+        log(f"{e['op']:<90s} {e['latency_us']:>10.1f} us  {e['achieved']:>9.1f} {e['unit']:<8s} "
+            f"{100 * e['frac']:5.1f}% of {e['peak']:g}" + (f"   cpu: {cb}" if cb else ""))
+
+    line = {
+        "metric": METRIC, "value": head["value"], "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config1: relu+tanh relaxation, lw/uw [1,128,256,512], words=2, eps=0.01, "
+                               "p in {1,2,inf} (6 launches per step)",
+                   "bytes_per_step": head["bytes_per_step"], "device": prop.name,
+                   "compute_units": prop.multi_processor_count},
+        "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "ops": entries,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -180,17 +180,23 @@ conv_signsplit(const ConvArgs g) {
     }
 }
 
-// Direct convolution, one thread per output, products and sums in double; adds the bias.
-__global__ void __launch_bounds__(256) conv_direct(const ConvArgs g) {
+// Direct convolution for the constant terms: 32 neighbouring outputs x 8 channel groups per
+// workgroup; a thread sums its share of the input channels in double (an fp32 x fp32 product is
+// exact there), the 8 partial sums meet in LDS, one rounding, then the bias.
+constexpr int DP = 32, DG = 8;
+__global__ void __launch_bounds__(DP * DG) conv_direct(const ConvArgs g) {
+    __shared__ double red[2][DG][DP];
     const size_t total = (size_t)g.N * g.Co * g.Ho * g.Wo;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    const int ow = idx % g.Wo;
-    const int oh = (idx / g.Wo) % g.Ho;
-    const int co = (idx / ((size_t)g.Wo * g.Ho)) % g.Co;
-    const int n = idx / ((size_t)g.Wo * g.Ho * g.Co);
+    const int px = threadIdx.x % DP, cg = threadIdx.x / DP;
+    const size_t idx = (size_t)blockIdx.x * DP + px;
+    const bool live = idx < total;
+    const size_t id = live ? idx : total - 1;
+    const int ow = id % g.Wo;
+    const int oh = (id / g.Wo) % g.Ho;
+    const int co = (id / ((size_t)g.Wo * g.Ho)) % g.Co;
+    const int n = id / ((size_t)g.Wo * g.Ho * g.Co);
     double sl = 0.0, su = 0.0;
-    for (int ci = 0; ci < g.Ci; ++ci) {
+    for (int ci = cg; ci < g.Ci; ci += DG) {
         const float *xl = g.xl + ((size_t)n * g.Ci + ci) * g.H * g.W;
         const float *xu = g.xu + ((size_t)n * g.Ci + ci) * g.H * g.W;
         const float *w = g.w + ((size_t)co * g.Ci + ci) * g.K * g.K;
@@ -208,9 +214,19 @@ __global__ void __launch_bounds__(256) conv_direct(const ConvArgs g) {
             }
         }
     }
-    const float add = g.bias ? g.bias[co] : 0.f;
-    g.yl[idx] = (float)sl + add;
-    g.yu[idx] = (float)su + add;
+    red[0][cg][px] = sl;
+    red[1][cg][px] = su;
+    __syncthreads();
+    if (cg == 0 && live) {
+#pragma unroll
+        for (int c = 1; c < DG; ++c) {
+            sl += red[0][c][px];
+            su += red[1][c][px];
+        }
+        const float add = g.bias ? g.bias[co] : 0.f;
+        g.yl[idx] = (float)sl + add;
+        g.yu[idx] = (float)su + add;
+    }
 }
 
 }  // namespace
@@ -254,6 +270,6 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
     // constant terms: batch images through the exact-accumulation kernel, bias added
     ConvArgs gb{x_lb, x_ub, W, bias, y_lb, y_ub, batch_size, CIN, Height, Width, COUT, K, Stride, padding_size, Ho, Wo};
     const long long nb = (long long)batch_size * COUT * Ho * Wo;
-    hipLaunchKernelGGL(conv_direct, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, st, gb);
+    hipLaunchKernelGGL(conv_direct, dim3((unsigned)((nb + DP - 1) / DP)), dim3(DP * DG), 0, st, gb);
     return faith::check_launch("faith_convolution_verification");
 }

@@ -214,25 +214,51 @@ __global__ void __launch_bounds__(256) dot_qk_w_simple(const DotArgs g) {
     }
 }
 
-// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): one thread per (head, i, j).
+// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns a 16 x 16 tile of
+// (i, j) of one head, stages the seven [16 x d-chunk] operand rows in LDS and sums in double.
+constexpr int BT_T = 16, BT_K = 64;
 __global__ void __launch_bounds__(256) dot_qk_b(const DotArgs g) {
-    const size_t total = (size_t)g.B * g.Lx * g.Ly;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
-    const int j = idx % g.Ly;
-    const int i = (idx / g.Ly) % g.Lx;
-    const int t = idx / ((size_t)g.Ly * g.Lx);
-    const size_t xo = (size_t)(t * g.Lx + i) * g.d, yo = (size_t)(t * g.Ly + j) * g.d;
+    __shared__ float sx[3][BT_T][BT_K + 1];     // b (= l_x), xlb, xub
+    __shared__ float sy[4][BT_T][BT_K + 1];     // a_l, a_u, ylb, yub
+    const int ti = (g.Lx + BT_T - 1) / BT_T, tj = (g.Ly + BT_T - 1) / BT_T;
+    int pid = blockIdx.x;
+    const int j0 = (pid % tj) * BT_T;  pid /= tj;
+    const int i0 = (pid % ti) * BT_T;  pid /= ti;
+    const int t = pid;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;     // output (i0 + ty, j0 + tx)
     double sl = 0.0, su = 0.0;
-    for (int k = 0; k < g.d; ++k) {
-        const double bt = g.x_l[xo + k], al = g.y_l[yo + k], au = g.y_u[yo + k];
-        const double xlb = g.xlb[xo + k], xub = g.xub[xo + k], ylb = g.ylb[yo + k], yub = g.yub[yo + k];
-        const double bp = bt > 0 ? bt : 0, bn = bt < 0 ? bt : 0;
-        sl += -al * bt + (al > 0 ? al * xlb : al * xub) + bp * ylb + bn * yub;
-        su += -au * bt + (au > 0 ? au * xub : au * xlb) + bp * yub + bn * ylb;
+    for (int k0 = 0; k0 < g.d; k0 += BT_K) {
+        for (int e = threadIdx.x; e < BT_T * BT_K; e += 256) {
+            const int r = e / BT_K, k = e % BT_K;
+            const bool kin = k0 + k < g.d;
+            const bool xin = kin && i0 + r < g.Lx, yin = kin && j0 + r < g.Ly;
+            const size_t xo = (size_t)(t * g.Lx + i0 + r) * g.d + k0 + k;
+            const size_t yo = (size_t)(t * g.Ly + j0 + r) * g.d + k0 + k;
+            sx[0][r][k] = xin ? g.x_l[xo] : 0.f;
+            sx[1][r][k] = xin ? g.xlb[xo] : 0.f;
+            sx[2][r][k] = xin ? g.xub[xo] : 0.f;
+            sy[0][r][k] = yin ? g.y_l[yo] : 0.f;
+            sy[1][r][k] = yin ? g.y_u[yo] : 0.f;
+            sy[2][r][k] = yin ? g.ylb[yo] : 0.f;
+            sy[3][r][k] = yin ? g.yub[yo] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int k = 0; k < BT_K; ++k) {
+            const double bt = sx[0][ty][k], xlb = sx[1][ty][k], xub = sx[2][ty][k];
+            const double al = sy[0][tx][k], au = sy[1][tx][k], ylb = sy[2][tx][k], yub = sy[3][tx][k];
+            const double bp = bt > 0 ? bt : 0, bn = bt < 0 ? bt : 0;
+            sl += -al * bt + (al > 0 ? al * xlb : al * xub) + bp * ylb + bn * yub;
+            su += -au * bt + (au > 0 ? au * xub : au * xlb) + bp * yub + bn * ylb;
+        }
+        __syncthreads();
     }
-    g.zlb[idx] = (float)sl;
-    g.zub[idx] = (float)su;
+    const int i = i0 + ty, j = j0 + tx;
+    if (i < g.Lx && j < g.Ly) {
+        const size_t o = ((size_t)t * g.Lx + i) * g.Ly + j;
+        g.zlb[o] = (float)sl;
+        g.zub[o] = (float)su;
+    }
 }
 
 // dim_in == 1: the reference switches to plain interval arithmetic on the constant terms and
@@ -301,7 +327,10 @@ extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *
     DotArgs g{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub,
               batch_size, length_x, length_y, dim_in, dim_out};
     const long long nb = (long long)batch_size * length_x * length_y;
-    hipLaunchKernelGGL(dot_qk_b, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, st, g);
+    (void)nb;
+    hipLaunchKernelGGL(dot_qk_b, dim3((unsigned)((long long)batch_size * ((length_x + BT_T - 1) / BT_T) *
+                                                 ((length_y + BT_T - 1) / BT_T))),
+                       dim3(256), 0, st, g);
 
     const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
                       faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
