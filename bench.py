@@ -40,7 +40,7 @@ INF = float("inf")
 # HBM bytes per launch of the dominant relaxation kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE, scaled by the same counters on faith_copy_f32 of known size (see
 # profiles/act_natural_config1_pmc.md).  None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = None
+TRAFFIC_BYTES_PER_LAUNCH = 269_750_000   # tanh kernel: (2.000 * 65,919 + 131,584) KiB
 
 
 def log(*a):

@@ -1,0 +1,88 @@
+"""C ABI checks that need no GPU: every function declared in include/faith_amd.h is exported by
+the built library, the Python binding lists the same set, and argument validation returns
+status codes (nothing is launched, nothing aborts)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "faith_amd.h")
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(faith_\w+)\s*\(", src)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from faith_amd import _lib
+    return _lib
+
+
+def test_header_declares_the_reference_surface():
+    names = declared_functions()
+    for fn in ("faith_relu_verification", "faith_tanh_verification", "faith_matmul_verification",
+               "faith_dot_product_verification_QK", "faith_convolution_verification", "faith_concretize"):
+        assert fn in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(lib.LIB_PATH)
+    for fn in declared_functions():
+        assert hasattr(raw, fn), f"{fn} is declared in include/faith_amd.h but not exported"
+
+
+def test_binding_covers_every_entry_point(lib):
+    bound = set(lib.SIGNATURES) | {"faith_last_error", "faith_version"}
+    assert set(declared_functions()) == bound
+
+
+def test_null_and_shape_errors_are_status_codes(lib):
+    L = lib.lib
+    buf = (ctypes.c_float * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)          # non-NULL host address; validation fails before any use
+    # NULL required pointer
+    assert L.faith_concretize(None, p, p, p, p, p, 1, 4, 4, 0.1, lib.Q_2, 1, 0, None) == -1
+    assert b"NULL" in L.faith_last_error()
+    # non-positive dimension
+    assert L.faith_concretize(p, p, p, p, p, p, 0, 4, 4, 0.1, lib.Q_2, 1, 0, None) == -2
+    # words must divide dim_in
+    assert L.faith_relu_verification(p, p, p, p, p, p, p, p, None, None, 1, 6, 4, 0.1, lib.Q_2, 4, 0, None) == -2
+    # unknown norm / layout
+    assert L.faith_tanh_verification(p, p, p, p, p, p, p, p, None, None, 1, 4, 4, 0.1, 7, 1, 0, None) == -3
+    assert L.faith_tanh_verification(p, p, p, p, p, p, p, p, None, None, 1, 4, 4, 0.1, lib.Q_1, 1, 9, None) == -3
+    # misaligned pointer
+    q = ctypes.c_void_p(p.value + 2)
+    assert L.faith_matmul_verification(q, p, p, p, p, None, p, p, p, p, 1, 1, 4, 4, 4, None) == -4
+    assert L.faith_matmul_verification(p, p, p, p, p, None, p, p, p, p, 1, 0, 4, 4, 4, None) == -2
+    assert L.faith_dot_product_verification_QK(p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, p,
+                                               1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, None) == -2
+    # kernel larger than the padded image
+    assert L.faith_convolution_verification(p, p, p, p, p, None, p, p, p, p, 1, 2, 2, 1, 1, 5, 1, 0, 1, None) == -2
+    assert L.faith_tune_set(99, 1) == -3
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+    from faith_amd import ops
+    lw = torch.zeros(1, 2, 4, 4)
+    lb = torch.zeros(1, 2, 4)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.relu(lw, lb, lw, lb, 2.0, 0.1)
+    with pytest.raises(ValueError):
+        ops.q_code(3.0)
+    assert ops.q_code(float("inf")) == ops.Q_1 and ops.q_code(1) == ops.Q_INF and ops.q_code(2) == ops.Q_2
+
+
+def test_workloads_are_reproducible():
+    import torch
+    from faith_amd.workloads import make_config
+    a, b = make_config(0), make_config(0)
+    assert torch.equal(a["x"]["lw"], b["x"]["lw"]) and torch.equal(a["W"], b["W"])
+    assert bool((a["x"]["uw"] >= a["x"]["lw"]).all()) and bool((a["x"]["ub"] >= a["x"]["lb"]).all())
+    c3 = make_config(3, scale=0.1)
+    assert c3["x"]["lw"].shape == (4, 13, 256, 64)
