@@ -180,6 +180,169 @@ conv_signsplit(const ConvArgs g) {
     }
 }
 
+// ------------------------------------------------------------------ 3x3, stride 1 fast path
+// Same tiling with every extent a compile-time constant (patch 6 x 34, weight rows of 36 + 1),
+// plus a register prefetch across chunks: the global loads of chunk c+1 are issued before the
+// MFMAs of chunk c and land in LDS after them, so their latency is covered by 288 MFMAs per
+// wavefront instead of being exposed at the head of every chunk.  Needs C_in % 4 == 0 and a
+// 16-byte aligned weight pointer (float4 weight loads).
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+conv_signsplit_k3s1(const ConvArgs g) {
+    constexpr int K = 3, KK = 9, PROW = TR - 1 + K, PCOL = TC - 1 + K, PP = PROW * PCOL;   // 6, 34, 204
+    constexpr int WS = CC * KK + 1;                      // 37
+    constexpr int NP = (CC * PP + NTHREADS - 1) / NTHREADS;          // patch elements per thread and bound: 4
+    constexpr int NW4 = (TCO * CC * KK / 4 + NTHREADS - 1) / NTHREADS;   // weight float4 per thread: 5
+    __shared__ float sXl[CC * PP];
+    __shared__ float sXu[CC * PP];
+    __shared__ float sW[TCO * WS];
+
+    const int tcol = (g.Wo + TC - 1) / TC, trow = (g.Ho + TR - 1) / TR, tco = (g.Co + TCO - 1) / TCO;
+    int pid = blockIdx.x;
+    const int ow0 = (pid % tcol) * TC;  pid /= tcol;
+    const int oh0 = (pid % trow) * TR;  pid /= trow;
+    const int co0 = (pid % tco) * TCO;  pid /= tco;
+    const int n = pid;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wv = tid / 64;
+    const int wm = wv / 2, wn = wv % 2;
+    const int fi = lane % 32, fh = lane / 32;
+
+    const int ih0 = oh0 - g.P, iw0 = ow0 - g.P;
+    const int img = g.H * g.W;
+    const float *xl_n = g.xl + (size_t)n * g.Ci * img;
+    const float *xu_n = g.xu + (size_t)n * g.Ci * img;
+
+    // ---- staging plan, fixed for the whole reduction
+    int poff[NP];                                        // offset inside a 4-channel slab, -1 = zero
+#pragma unroll
+    for (int u = 0; u < NP; ++u) {
+        const int e = tid + u * NTHREADS;
+        const int ci = e / PP, r2 = e % PP, pr = r2 / PCOL, pc = r2 % PCOL;
+        const int ih = ih0 + pr, iw = iw0 + pc;
+        const bool ok = e < CC * PP && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+        poff[u] = ok ? ci * img + ih * g.W + iw : -1;
+    }
+    int wsrc[NW4], wdst[NW4];
+#pragma unroll
+    for (int u = 0; u < NW4; ++u) {
+        const int e = tid + u * NTHREADS;
+        const int co = e / 9, f = e % 9;
+        const bool ok = e < TCO * 9;
+        wsrc[u] = ok ? min(co0 + co, g.Co - 1) * g.Ci * KK + f * 4 : -1;     // rows past C_out are never stored
+        wdst[u] = co * WS + f * 4;
+    }
+    float pxl[NP], pxu[NP];
+    float4 pw[NW4];
+    auto prefetch = [&](int c0) {
+        const float *xl = xl_n + (size_t)c0 * img, *xu = xu_n + (size_t)c0 * img;
+        const float *w = g.w + c0 * KK;
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            pxl[u] = poff[u] >= 0 ? xl[poff[u]] : 0.f;
+            pxu[u] = poff[u] >= 0 ? xu[poff[u]] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < NW4; ++u)
+            pw[u] = wsrc[u] >= 0 ? *reinterpret_cast<const float4 *>(w + wsrc[u]) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            const int e = tid + u * NTHREADS;
+            if (e < CC * PP) {
+                sXl[e] = pxl[u];
+                sXu[e] = pxu[u];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NW4; ++u) {
+            if (wsrc[u] >= 0) {
+                sW[wdst[u] + 0] = pw[u].x;
+                sW[wdst[u] + 1] = pw[u].y;
+                sW[wdst[u] + 2] = pw[u].z;
+                sW[wdst[u] + 3] = pw[u].w;
+            }
+        }
+    };
+
+    int xoff[2], woff[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) xoff[b] = fh * (CC / 2) * PP + (wn * 2 + b) * PCOL + fi;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) woff[a] = (wm * 64 + a * 32 + fi) * WS + fh * (CC / 2) * KK;
+
+    floatx16 cl[2][2], cu[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
+
+    prefetch(0);
+    for (int c0 = 0; c0 < g.Ci; c0 += CC) {
+        commit();
+        __syncthreads();
+        if (c0 + CC < g.Ci) prefetch(c0 + CC);
+#pragma unroll
+        for (int cp = 0; cp < CC / 2; ++cp) {
+#pragma unroll
+            for (int tap = 0; tap < KK; ++tap) {
+                const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
+                const int wo = cp * KK + tap;
+                float wp[2], wq[2], xl[2], xu[2];
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const float w = sW[woff[a] + wo];
+                    wp[a] = fmaxf(w, 0.f);
+                    wq[a] = fminf(w, 0.f);
+                }
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    xl[b] = sXl[xoff[b] + xo];
+                    xu[b] = sXu[xoff[b] + xo];
+                }
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
+                        cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
+                    }
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
+                        cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                    }
+            }
+        }
+        __syncthreads();
+    }
+
+    const int ow = ow0 + fi;
+    if (ow >= g.Wo) return;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int oh = oh0 + wn * 2 + b;
+        if (oh >= g.Ho) continue;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+                if (co < g.Co) {
+                    const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
+                    g.yl[o] = cl[a][b][r];
+                    g.yu[o] = cu[a][b][r];
+                }
+            }
+        }
+    }
+}
+
 // Direct convolution for the constant terms: 32 neighbouring outputs x 8 channel groups per
 // workgroup; a thread sums its share of the input channels in double (an fp32 x fp32 product is
 // exact there), the 8 partial sums meet in LDS, one rounding, then the bias.
@@ -265,7 +428,12 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
     }
     const long long grid = (long long)dim_in * ((COUT + TCO - 1) / TCO) * ((Ho + TR - 1) / TR) * ((Wo + TC - 1) / TC);
     FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_convolution_verification: grid too large");
-    hipLaunchKernelGGL(conv_signsplit, dim3((unsigned)grid), dim3(NTHREADS), smem, st, gw);
+    const bool k3s1 = K == 3 && Stride == 1 && CIN % 4 == 0 && faith::aligned(W, 16) &&
+                      (long long)CIN * Height * Width < 0x7fffffffLL && (long long)COUT * CIN * 9 < 0x7fffffffLL;
+    if (k3s1)
+        hipLaunchKernelGGL(conv_signsplit_k3s1, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
+    else
+        hipLaunchKernelGGL(conv_signsplit, dim3((unsigned)grid), dim3(NTHREADS), smem, st, gw);
 
     // constant terms: batch images through the exact-accumulation kernel, bias added
     ConvArgs gb{x_lb, x_ub, W, bias, y_lb, y_ub, batch_size, CIN, Height, Width, COUT, K, Stride, padding_size, Ho, Wo};
