@@ -82,13 +82,20 @@ __device__ __forceinline__ float line_bias(const Line &ln, float same, float oth
 }
 
 // ------------------------------------------------------------------ vector access
+// Stores are non-temporal: lw' / uw' are written once and not read again by this kernel, and
+// keeping them out of the cache's way measured 11 % faster at configuration 1 (loads are left
+// temporal: marking them non-temporal measured 15 % slower).
+typedef float v4f __attribute__((ext_vector_type(4)));
 template <int VEC>
 struct Vec;
 template <>
 struct Vec<4> {
     float4 v;
     __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
-    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
+    __device__ __forceinline__ void store(float *p) const {
+        const v4f t = {v.x, v.y, v.z, v.w};
+        __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
+    }
     __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
     __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
     __device__ __forceinline__ void set(int i, float f) {
@@ -102,7 +109,7 @@ template <>
 struct Vec<1> {
     float v;
     __device__ __forceinline__ void load(const float *p) { v = *p; }
-    __device__ __forceinline__ void store(float *p) const { *p = v; }
+    __device__ __forceinline__ void store(float *p) const { __builtin_nontemporal_store(v, p); }
     __device__ __forceinline__ void zero() { v = 0.f; }
     __device__ __forceinline__ float get(int) const { return v; }
     __device__ __forceinline__ void set(int, float f) { v = f; }

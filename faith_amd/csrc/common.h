@@ -15,6 +15,9 @@ void set_error(const char *fmt, ...);
 // Returns FAITH_OK or records the HIP error text and returns FAITH_ERR_LAUNCH.
 int check_launch(const char *what);
 
+// Compute units of the current device (queried once per device, then cached).
+int compute_units();
+
 // Tuning knobs (faith_tune_set); 0 = built-in choice.
 int tune_get(int knob);
 

@@ -21,6 +21,18 @@ int check_launch(const char *what) {
     return FAITH_OK;
 }
 
+int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 static int g_tune[FAITH_TUNE_COUNT] = {0};
 
 int tune_get(int knob) { return (knob >= 0 && knob < FAITH_TUNE_COUNT) ? g_tune[knob] : 0; }

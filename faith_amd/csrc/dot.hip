@@ -59,55 +59,62 @@ __device__ __forceinline__ int swz(int row, int c) { return row * BK + 4 * (c ^ 
 
 enum { XL = 0, XU, BT, AL, AU, YL, YU, NOPS };
 
+// Persistent: the grid is sized to the machine (two workgroups per CU) and every workgroup walks
+// tiles pid, pid + grid, ...  The walk is ONE software pipeline over (tile, K-step): the global
+// loads of the next step -- the first K-step of the next tile included -- are issued before the
+// MFMAs of the current step, and the accumulator stores of a finished tile are issued while
+// those loads are in flight, so neither the head nor the tail of a tile leaves the MFMA pipe idle.
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-dot_qk_w(const DotArgs g) {
+dot_qk_w(const DotArgs g, const int total_tiles) {
     __shared__ float sm[2][NOPS][TILE];
 
     const int ti = (g.Lx + TI - 1) / TI, tj = (g.Ly + TJ - 1) / TJ;
-    int pid = blockIdx.x;
-    const int j0 = (pid % tj) * TJ;  pid /= tj;
-    const int i0 = (pid % ti) * TI;  pid /= ti;
-    const int m = pid % g.D;
-    const int t = pid / g.D;
     const int d = g.d;
+    const int nk = (d + BK - 1) / BK;
 
     const int tid = threadIdx.x;
     const int lane = tid % 64, wv = tid / 64;
     const int wi = wv / 2, wj = wv % 2;
+    const int fi = lane % 32, fh = lane / 32;
 
     // ---- staging: one float4 per operand per thread per K-step
     const int srow = tid / 2, sc = tid % 2;
-    const int irow = min(i0 + srow, g.Lx - 1), jrow = min(j0 + srow, g.Ly - 1);   // clamped rows are never stored
-    const float *src[NOPS];
-    src[XL] = g.xlw + ((size_t)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
-    src[XU] = g.xuw + ((size_t)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
-    src[BT] = g.x_l + (size_t)(t * g.Lx + irow) * d + sc * 4;
-    src[AL] = g.y_l + (size_t)(t * g.Ly + jrow) * d + sc * 4;
-    src[AU] = g.y_u + (size_t)(t * g.Ly + jrow) * d + sc * 4;
-    src[YL] = g.ylw + ((size_t)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
-    src[YU] = g.yuw + ((size_t)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
     const int sdst = swz(srow, sc);
+    // element offsets of this thread's source rows (32-bit: the entry point checks the sizes);
+    // xlw / xuw share one, ylw / yuw share one, a_l / a_u share one
+    unsigned ox, oy, obt, oa;
     float4 pre[NOPS];
+    auto point_at = [&](int tile) {
+        int q = tile;
+        const int j0 = (q % tj) * TJ;  q /= tj;
+        const int i0 = (q % ti) * TI;  q /= ti;
+        const int m = q % g.D, t = q / g.D;
+        const int irow = min(i0 + srow, g.Lx - 1), jrow = min(j0 + srow, g.Ly - 1);   // clamped rows are never stored
+        ox = ((unsigned)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
+        oy = ((unsigned)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
+        obt = (unsigned)(t * g.Lx + irow) * d + sc * 4;
+        oa = (unsigned)(t * g.Ly + jrow) * d + sc * 4;
+    };
     auto gload = [&](int kt) {
         const int k = kt * BK;
-        const bool in = k + sc * 4 < d;            // d % 4 == 0
+        if (k + sc * 4 < d) {                      // d % 4 == 0: a float4 is all in or all out
+            pre[XL] = ld4(g.xlw + ox + k);
+            pre[XU] = ld4(g.xuw + ox + k);
+            pre[BT] = ld4(g.x_l + obt + k);
+            pre[AL] = ld4(g.y_l + oa + k);
+            pre[AU] = ld4(g.y_u + oa + k);
+            pre[YL] = ld4(g.ylw + oy + k);
+            pre[YU] = ld4(g.yuw + oy + k);
+        } else {
 #pragma unroll
-        for (int o = 0; o < NOPS; ++o) pre[o] = in ? ld4(src[o] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int o = 0; o < NOPS; ++o) pre[o] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     };
     auto lstore = [&](int buf) {
 #pragma unroll
         for (int o = 0; o < NOPS; ++o) *reinterpret_cast<float4 *>(&sm[buf][o][sdst]) = pre[o];
     };
 
-    floatx16 cl[2][2], cu[2][2];
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
-
-    const int fi = lane % 32, fh = lane / 32;
     int fa[2], fb[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -115,29 +122,47 @@ dot_qk_w(const DotArgs g) {
         fb[s] = swz(wj * 64 + s * 32 + fi, fh);
     }
 
-    const int nk = (d + BK - 1) / BK;
+    floatx16 cl[2][2], cu[2][2];
+    int tile = blockIdx.x;
+    if (tile >= total_tiles) return;
+    point_at(tile);
     gload(0);
     lstore(0);
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) gload(kt + 1);
-        float4 xl[2], xu[2], bp[2], bn[2];
+    int buf = 0;
+    for (; tile < total_tiles; tile += gridDim.x) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            xl[s] = *reinterpret_cast<const float4 *>(&sm[buf][XL][fa[s]]);
-            xu[s] = *reinterpret_cast<const float4 *>(&sm[buf][XU][fa[s]]);
-            const float4 bt = *reinterpret_cast<const float4 *>(&sm[buf][BT][fa[s]]);
-            bp[s] = pos4(bt);
-            bn[s] = neg4(bt);
-        }
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const float4 al = *reinterpret_cast<const float4 *>(&sm[buf][AL][fb[b]]);
-            const float4 au = *reinterpret_cast<const float4 *>(&sm[buf][AU][fb[b]]);
-            const float4 yl = *reinterpret_cast<const float4 *>(&sm[buf][YL][fb[b]]);
-            const float4 yu = *reinterpret_cast<const float4 *>(&sm[buf][YU][fb[b]]);
-            const float4 alp = pos4(al), aln = neg4(al), aup = pos4(au), aun = neg4(au);
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
+        const int next_tile = tile + gridDim.x;
+        const bool has_next = next_tile < total_tiles;
+        for (int kt = 0; kt < nk; ++kt) {
+            const bool last = kt + 1 == nk;
+            if (!last) {
+                gload(kt + 1);
+            } else if (has_next) {
+                point_at(next_tile);
+                gload(0);
+            }
+            float4 xl[2], xu[2], bp[2], bn[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                xl[s] = *reinterpret_cast<const float4 *>(&sm[buf][XL][fa[s]]);
+                xu[s] = *reinterpret_cast<const float4 *>(&sm[buf][XU][fa[s]]);
+                const float4 bt = *reinterpret_cast<const float4 *>(&sm[buf][BT][fa[s]]);
+                bp[s] = pos4(bt);
+                bn[s] = neg4(bt);
+            }
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const float4 al = *reinterpret_cast<const float4 *>(&sm[buf][AL][fb[b]]);
+                const float4 au = *reinterpret_cast<const float4 *>(&sm[buf][AU][fb[b]]);
+                const float4 yl = *reinterpret_cast<const float4 *>(&sm[buf][YL][fb[b]]);
+                const float4 yu = *reinterpret_cast<const float4 *>(&sm[buf][YU][fb[b]]);
+                const float4 alp = pos4(al), aln = neg4(al), aup = pos4(au), aun = neg4(au);
 #define FAITH_DOT_STEP(c)                                   \
     _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
         cl[a][b] = mfma(xl[a].c, alp.c, cl[a][b]);          \
@@ -155,33 +180,48 @@ dot_qk_w(const DotArgs g) {
         cl[a][b] = mfma(bn[a].c, yu.c, cl[a][b]);           \
         cu[a][b] = mfma(bn[a].c, yl.c, cu[a][b]);           \
     }
-            FAITH_DOT_STEP(x)
-            FAITH_DOT_STEP(y)
-            FAITH_DOT_STEP(z)
-            FAITH_DOT_STEP(w)
+                FAITH_DOT_STEP(x)
+                FAITH_DOT_STEP(y)
+                FAITH_DOT_STEP(z)
+                FAITH_DOT_STEP(w)
 #undef FAITH_DOT_STEP
+            }
+            if (!last) {
+                lstore(buf ^ 1);
+                __syncthreads();
+                buf ^= 1;
+            }
         }
-        if (kt + 1 < nk) lstore(buf ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue: z[t, i, m, j]; register r of a block is row 8*(r/4) + 4*(lane/32) + r%4
+        {
+            // ---- z[t, i, m, j]; register r of a block is row 8*(r/4) + 4*(lane/32) + r%4.
+            // Issued while the first K-step of the next tile is on its way.
+            int q = tile;
+            const int j0 = (q % tj) * TJ;  q /= tj;
+            const int i0 = (q % ti) * TI;  q /= ti;
+            const int m = q % g.D, t = q / g.D;
+            const unsigned rs = (unsigned)g.D * g.Ly;                     // one step in i
+            const int ib = i0 + wi * 64 + 4 * fh;
+            const unsigned ob = ((unsigned)(t * g.Lx + ib) * g.D + m) * g.Ly + j0 + wj * 64 + fi;
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        const int j = j0 + wj * 64 + b * 32 + fi;
-        if (j >= g.Ly) continue;
+            for (int b = 0; b < 2; ++b) {
+                if (j0 + wj * 64 + b * 32 + fi >= g.Ly) continue;
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+                for (int a = 0; a < 2; ++a) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int i = i0 + wi * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
-                if (i < g.Lx) {
-                    const size_t o = ((size_t)(t * g.Lx + i) * g.D + m) * g.Ly + j;
-                    g.zlw[o] = cl[a][b][r];
-                    g.zuw[o] = cu[a][b][r];
+                    for (int r = 0; r < 16; ++r) {
+                        const int di = a * 32 + 8 * (r / 4) + (r % 4);
+                        if (ib + di < g.Lx) {
+                            const unsigned o = ob + di * rs + b * 32;
+                            g.zlw[o] = cl[a][b][r];
+                            g.zuw[o] = cu[a][b][r];
+                        }
+                    }
                 }
             }
         }
+        if (has_next) lstore(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
     }
 }
 
@@ -336,9 +376,14 @@ extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *
                       faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
                       faith::aligned(y_l, 16) && faith::aligned(y_u, 16);
     if (fast) {
-        const long long grid = (long long)batch_size * dim_in * ((length_x + TI - 1) / TI) * ((length_y + TJ - 1) / TJ);
-        FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: grid too large");
-        hipLaunchKernelGGL(dot_qk_w, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
+        FAITH_REQUIRE(nw < 0xffffffffLL && (long long)batch_size * (length_x > length_y ? length_x : length_y) *
+                                              dim_in * dim_out < 0xffffffffLL,
+                      FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: tensors beyond 2^32 elements");
+        const long long tiles = (long long)batch_size * dim_in * ((length_x + TI - 1) / TI) * ((length_y + TJ - 1) / TJ);
+        FAITH_REQUIRE(tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: too many tiles");
+        const long long resident = 2LL * faith::compute_units();      // 56 KB of LDS each: two per CU
+        hipLaunchKernelGGL(dot_qk_w, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(NTHREADS), 0, st, g,
+                           (int)tiles);
     } else {
         const long long blocks = (nw + 255) / 256;
         hipLaunchKernelGGL(dot_qk_w_simple, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
