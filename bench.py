@@ -252,6 +252,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only-headline", action="store_true", help="skip configurations 0, 2, 3, 4")
+    ap.add_argument("--configs", default="0,2,3,4", help="extra configurations to report under 'ops'")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every op is independent across the length axis and "
@@ -272,10 +273,14 @@ def main():
     log(f"device: {prop.name}, {prop.multi_processor_count} CUs, host threads {torch.get_num_threads()}")
 
     head, entries = bench_config1(args, ops, O, wl, args.steps, args.warmup)
-    if not args.only_headline:
+    extra = set() if args.only_headline else {int(c) for c in args.configs.split(",") if c.strip()}
+    if 0 in extra:
         entries = [bench_config0(args, ops, O, wl)] + entries
+    if 2 in extra:
         entries += bench_config2(args, ops, O, wl)
+    if 3 in extra:
         entries.append(bench_config3(args, ops, O, wl))
+    if 4 in extra:
         entries += bench_config4(args, ops, O, wl)
 
     for e in entries:

@@ -172,8 +172,8 @@ conv_signsplit(const ConvArgs g) {
                 const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (co < g.Co) {
                     const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
-                    g.yl[o] = cl[a][b][r];
-                    g.yu[o] = cu[a][b][r];
+                    __builtin_nontemporal_store(cl[a][b][r], &g.yl[o]);
+                    __builtin_nontemporal_store(cu[a][b][r], &g.yu[o]);
                 }
             }
         }
@@ -335,8 +335,8 @@ conv_signsplit_k3s1(const ConvArgs g) {
                 const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (co < g.Co) {
                     const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
-                    g.yl[o] = cl[a][b][r];
-                    g.yu[o] = cu[a][b][r];
+                    __builtin_nontemporal_store(cl[a][b][r], &g.yl[o]);
+                    __builtin_nontemporal_store(cu[a][b][r], &g.yu[o]);
                 }
             }
         }

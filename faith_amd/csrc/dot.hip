@@ -212,8 +212,8 @@ dot_qk_w(const DotArgs g, const int total_tiles) {
                         const int di = a * 32 + 8 * (r / 4) + (r % 4);
                         if (ib + di < g.Lx) {
                             const unsigned o = ob + di * rs + b * 32;
-                            g.zlw[o] = cl[a][b][r];
-                            g.zuw[o] = cu[a][b][r];
+                            __builtin_nontemporal_store(cl[a][b][r], &g.zlw[o]);
+                            __builtin_nontemporal_store(cu[a][b][r], &g.zuw[o]);
                         }
                     }
                 }

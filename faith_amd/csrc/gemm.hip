@@ -179,8 +179,8 @@ signsplit_gemm(const GemmArgs g) {
                 const int row = m0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (row < M) {
                     const size_t o = (size_t)row * g.N + col;
-                    Cl[o] = cl[a][b][r] + add;
-                    Cu[o] = cu[a][b][r] + add;
+                    __builtin_nontemporal_store(cl[a][b][r] + add, &Cl[o]);
+                    __builtin_nontemporal_store(cu[a][b][r] + add, &Cu[o]);
                 }
             }
         }
