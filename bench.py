@@ -50,8 +50,14 @@ def log(*a):
 def gpu_times_ms(fn, n, warmup):
     """Per-launch durations from HIP events recorded on the launch stream (torch's current one)."""
     import torch
-    for _ in range(warmup):
+    # warm up by count AND by time: clocks and caches settle only after ~0.2 s of sustained work
+    t0 = time.perf_counter()
+    done = 0
+    while done < warmup or time.perf_counter() - t0 < 0.25:
         fn()
+        done += 1
+        if done % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
     for s, e in evs:

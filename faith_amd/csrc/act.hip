@@ -35,6 +35,10 @@ struct ActArgs {
     float *l, *u;
     int rows, D, H, words;
     float eps;
+    // optional second bound object of the same D, H (concretize only): one launch covers both
+    const float *lb2 = nullptr, *ub2 = nullptr, *lw2 = nullptr, *uw2 = nullptr;
+    float *l2 = nullptr, *u2 = nullptr;
+    int rows2 = 0;
 };
 
 // y = k * (v - x0) + y0
@@ -188,8 +192,13 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     float *s_ln = s_lu + 2 * TH;              // [2][3][TH] lower / upper line (k, x0, y0)
 
     const int tiles = (a.H + TH - 1) / TH;
-    const int r = blockIdx.x / tiles;
-    const int col0 = (blockIdx.x % tiles) * TH;
+    const bool second = MODE == CONCRETIZE && (int)blockIdx.x >= a.rows * tiles;
+    const int bid = second ? blockIdx.x - a.rows * tiles : blockIdx.x;
+    const float *__restrict__ p_lw = second ? a.lw2 : a.lw, *__restrict__ p_uw = second ? a.uw2 : a.uw;
+    const float *__restrict__ p_lb = second ? a.lb2 : a.lb, *__restrict__ p_ub = second ? a.ub2 : a.ub;
+    float *__restrict__ p_l = second ? a.l2 : a.l, *__restrict__ p_u = second ? a.u2 : a.u;
+    const int r = bid / tiles;
+    const int col0 = (bid % tiles) * TH;
     const int tid = threadIdx.x;
     const int lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid % TPR, rg = tid / TPR;
@@ -216,8 +225,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
         for (int i = 0; i < RPT; ++i) {
             const int row = ch * CHUNK + i * RG + rg;
             if (col_ok && row < a.D) {
-                dl[i].load(a.lw + base + (size_t)row * a.H);
-                du[i].load(a.uw + base + (size_t)row * a.H);
+                dl[i].load(p_lw + base + (size_t)row * a.H);
+                du[i].load(p_uw + base + (size_t)row * a.H);
             } else {
                 dl[i].zero();
                 du[i].zero();
@@ -271,7 +280,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     const bool n_ok = lane < TH && column < a.H;
     const size_t bi = (size_t)r * a.H + column;
     if (wv == 0 && n_ok) {
-        float l = a.lb[bi], u = a.ub[bi];
+        float l = p_lb[bi], u = p_ub[bi];
         for (int w = 0; w < a.words; ++w) {
             float nl = 0.f, nu = 0.f;
 #pragma unroll
@@ -282,14 +291,14 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
             l += (-a.eps) * nfin<Q>(nl);
             u += a.eps * nfin<Q>(nu);
         }
-        if (a.l) a.l[bi] = l;
-        if (a.u) a.u[bi] = u;
+        if (p_l) p_l[bi] = l;
+        if (p_u) p_u[bi] = u;
         if (MODE == RELU) {
             Line lo, up;
             relu_lines(l, u, lo, up);
             s_ln[lane] = lo.k;
             s_ln[3 * TH + lane] = up.k;
-            const float lb = a.lb[bi], ub = a.ub[bi];
+            const float lb = p_lb[bi], ub = p_ub[bi];
             a.olb[bi] = line_bias(lo, lb, ub);
             a.oub[bi] = line_bias(up, ub, lb);
         } else if (MODE == TANH) {
@@ -327,7 +336,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
         if (wv == 0 && n_ok) {
             const Line lo = {s_ln[lane], s_ln[TH + lane], s_ln[2 * TH + lane]};
             const Line up = {s_ln[3 * TH + lane], s_ln[4 * TH + lane], s_ln[5 * TH + lane]};
-            const float lb = a.lb[bi], ub = a.ub[bi];
+            const float lb = p_lb[bi], ub = p_ub[bi];
             a.olb[bi] = line_bias(lo, lb, ub);
             a.oub[bi] = line_bias(up, ub, lb);
         }
@@ -347,8 +356,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
             if (row < a.D) {
                 const size_t off = base + (size_t)row * a.H;
                 if (nchunks > 1) {
-                    dl[i].load(a.lw + off);
-                    du[i].load(a.uw + off);
+                    dl[i].load(p_lw + off);
+                    du[i].load(p_uw + off);
                 }
                 Vec<VEC> ol, ou;
 #pragma unroll
@@ -457,18 +466,25 @@ void launch_natural(const ActArgs &a, hipStream_t st) {
     constexpr int TH = TPR * VEC, RG = NTHREADS / TPR;
     const int tiles = (a.H + TH - 1) / TH;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
-    hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles)),
+    hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)((a.rows + a.rows2) * tiles)),
                        dim3(NTHREADS), smem, st, a);
 }
 
 template <int MODE, int Q>
 void dispatch_natural(const ActArgs &a, hipStream_t st) {
     const bool vec4 = (a.H % 4 == 0) && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
+                      faith::aligned(a.lw2, 16) && faith::aligned(a.uw2, 16) &&
                       (MODE == CONCRETIZE || (faith::aligned(a.olw, 16) && faith::aligned(a.ouw, 16)));
     if (MODE == CONCRETIZE) {
-        // nothing is kept: short chunks, many loads in flight
-        if (vec4)
+        // nothing is kept, so what counts is bytes in flight: 64-neuron tiles, 16 wavefronts, 256 rows
+        // per pass measured best or equal on every shape tried (wide and narrow H alike)
+        const int pick = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
+        if (vec4 && pick == 11)
             launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);
+        else if (vec4 && pick == 13)
+            launch_natural<MODE, Q, 4, 8, 256, 8>(a, st);
+        else if (vec4)
+            launch_natural<MODE, Q, 4, 16, 1024, 4>(a, st);
         else
             launch_natural<MODE, Q, 1, 64, 256, 8>(a, st);
         return;
@@ -527,6 +543,17 @@ int run(const char *who, ActArgs a, int q, int layout, void *stream) {
 }
 
 }  // namespace
+
+// Concretizes two bound objects of equal dim_in / dim_out in ONE launch (the dot product needs
+// the intervals of both operands before it can start).  Natural layout.
+int faith::concretize_pair(const float *lb, const float *ub, const float *lw, const float *uw, float *l, float *u,
+                           int rows, const float *lb2, const float *ub2, const float *lw2, const float *uw2,
+                           float *l2, float *u2, int rows2, int dim_in, int dim_out, float eps, int q, int words,
+                           void *stream) {
+    ActArgs a{lb, ub, lw, uw, nullptr, nullptr, nullptr, nullptr, l, u, rows, dim_in, dim_out, words, eps};
+    a.lb2 = lb2; a.ub2 = ub2; a.lw2 = lw2; a.uw2 = uw2; a.l2 = l2; a.u2 = u2; a.rows2 = rows2;
+    return run<CONCRETIZE>("faith_concretize", a, q, FAITH_LAYOUT_NATURAL, stream);
+}
 
 extern "C" int faith_concretize(const float *lb, const float *ub, const float *lw, const float *uw, float *l,
                                 float *u, int rows, int dim_in, int dim_out, float eps, int q, int words,

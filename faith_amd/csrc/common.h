@@ -15,6 +15,11 @@ void set_error(const char *fmt, ...);
 // Returns FAITH_OK or records the HIP error text and returns FAITH_ERR_LAUNCH.
 int check_launch(const char *what);
 
+// One-launch concretization of two bound objects (defined with the relaxation kernels).
+int concretize_pair(const float *lb, const float *ub, const float *lw, const float *uw, float *l, float *u, int rows,
+                    const float *lb2, const float *ub2, const float *lw2, const float *uw2, float *l2, float *u2,
+                    int rows2, int dim_in, int dim_out, float eps, int q, int words, void *stream);
+
 // Compute units of the current device (queried once per device, then cached).
 int compute_units();
 

@@ -357,11 +357,9 @@ extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *
 
     // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the
     // reference interface exposes it, the planes do not use it
-    int rc = faith_concretize(x_lb, x_ub, x_lw, x_uw, x_l, x_u, batch_size * length_x, dim_in, dim_out, epsilon, q,
-                              words, FAITH_LAYOUT_NATURAL, stream);
-    if (rc != FAITH_OK) return rc;
-    rc = faith_concretize(y_lb, y_ub, y_lw, y_uw, y_l, y_u, batch_size * length_y, dim_in, dim_out, epsilon, q,
-                          words, FAITH_LAYOUT_NATURAL, stream);
+    const int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, batch_size * length_x, y_lb, y_ub, y_lw,
+                                          y_uw, y_l, y_u, batch_size * length_y, dim_in, dim_out, epsilon, q, words,
+                                          stream);
     if (rc != FAITH_OK) return rc;
 
     DotArgs g{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub,

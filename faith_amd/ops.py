@@ -47,6 +47,24 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _NoGuard:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on(device):
+    """Device guard for the launch; free when the tensor already lives on the current device."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
 def _wb_shapes(lw, lb, layout):
     if lw.dim() != 4 or lb.dim() != 3:
         raise ValueError(f"lw must be 4-D and lb 3-D, got {tuple(lw.shape)} and {tuple(lb.shape)}")
@@ -66,7 +84,7 @@ def concretize(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL):
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
     l = torch.empty_like(lb)
     u = torch.empty_like(ub)
-    with torch.cuda.device(lw.device):
+    with _on(lw.device):
         _lib.call("faith_concretize", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(l), _ptr(u),
                   B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
     return l, u
@@ -84,7 +102,7 @@ def _activation(entry, lw, lb, uw, ub, p, eps, words, layout, return_interval, o
         _check("out lb", olb, lb.shape); _check("out ub", oub, lb.shape)
     l = torch.empty_like(lb) if return_interval else None
     u = torch.empty_like(ub) if return_interval else None
-    with torch.cuda.device(lw.device):
+    with _on(lw.device):
         _lib.call(entry, _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
                   _ptr(l), _ptr(u), B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
     if return_interval:
@@ -121,7 +139,7 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
         olw, olb, ouw, oub = out
         _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
         _check("out lb", olb, (B, L, N)); _check("out ub", oub, (B, L, N))
-    with torch.cuda.device(lw.device):
+    with _on(lw.device):
         _lib.call("faith_matmul_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
                   _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), B, L, D, H, N, _stream(lw))
     return olw, olb, ouw, oub
@@ -151,7 +169,7 @@ def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
         zlw, zlb, zuw, zub = out
         _check("out lw", zlw, (B, Lx, D, Ly)); _check("out uw", zuw, (B, Lx, D, Ly))
         _check("out lb", zlb, (B, Lx, Ly)); _check("out ub", zub, (B, Lx, Ly))
-    with torch.cuda.device(dev):
+    with _on(dev):
         _lib.call("faith_dot_product_verification_QK", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Ly, d, D, float(eps), q_code(p), int(words),
@@ -187,7 +205,7 @@ def conv2d(lw, lb, uw, ub, weight, bias=None, stride=1, padding=0, out=None):
         olw, olb, ouw, oub = out
         _check("out lw", olw, (1, D, Co, Ho, Wo)); _check("out uw", ouw, (1, D, Co, Ho, Wo))
         _check("out lb", olb, (1, Co, Ho, Wo)); _check("out ub", oub, (1, Co, Ho, Wo))
-    with torch.cuda.device(lw.device):
+    with _on(lw.device):
         _lib.call("faith_convolution_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight),
                   _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), 1, Hh, Ww, C, Co, K, int(stride),
                   int(padding), D, _stream(lw))
