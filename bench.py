@@ -36,11 +36,12 @@ METRIC = "bound-prop latency & TFLOP/s (matmul/dot/conv) or HBM GB/s (relu/tanh)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 INF = float("inf")
+WARM_SECONDS = 0.25            # minimum warm-up per measurement; --profile sets it to 0
 
 # HBM bytes per launch of the dominant relaxation kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE, scaled by the same counters on faith_copy_f32 of known size (see
-# profiles/act_natural_config1_pmc.md).  None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = 269_750_000   # tanh kernel: (2.000 * 65,919 + 131,584) KiB
+# profiles/hbm_traffic_pmc.md).  None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = 270_180_000   # tanh kernel: (2.000 * 65,906 + 132,036) KiB
 
 
 def log(*a):
@@ -53,7 +54,7 @@ def gpu_times_ms(fn, n, warmup):
     # warm up by count AND by time: clocks and caches settle only after ~0.2 s of sustained work
     t0 = time.perf_counter()
     done = 0
-    while done < warmup or time.perf_counter() - t0 < 0.25:
+    while done < warmup or time.perf_counter() - t0 < WARM_SECONDS:
         fn()
         done += 1
         if done % 8 == 0:
@@ -259,7 +260,12 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only-headline", action="store_true", help="skip configurations 0, 2, 3, 4")
     ap.add_argument("--configs", default="0,2,3,4", help="extra configurations to report under 'ops'")
+    ap.add_argument("--profile", action="store_true",
+                    help="for runs under rocprofv3: warm up by count only, so the trace stays small")
     args = ap.parse_args()
+    if args.profile:
+        global WARM_SECONDS
+        WARM_SECONDS = 0.0
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every op is independent across the length axis and "
               "nothing here uses a second GPU, so --gpus must be 1", file=sys.stderr)
