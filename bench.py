@@ -227,8 +227,18 @@ def bench_config3(args, ops, O, wl):
         s = cpu_time_s(lambda: O.dot_product(xo, yo, c["p"], c["eps"]), reps=3, warmup=1)
         cpu = {"value": round(flop / s / 1e12, 4), "unit": "TFLOP/s", "sample": "full size, median of 3",
                "latency_ms": round(s * 1e3, 1)}
-    return op_entry("config3 dot_product QK 4 heads [4,128,256,64] (concretize + planes + contraction)",
-                    "mfma", t, flop, cpu)
+    e = op_entry("config3 dot_product QK 4 heads [4,128,256,64] (concretize + planes + contraction)",
+                 "mfma", t, flop, cpu)
+    # the second half of attention on the same shapes (not one of the five configurations): context =
+    # probabilities [4,128,256,128] . values [4,128,256,64]; the scores bounds just computed serve as
+    # the probability operand
+    probs = tuple(out)
+    outv = (torch.empty(B, L, D, d, device="cuda"), torch.empty(B, L, d, device="cuda"),
+            torch.empty(B, L, D, d, device="cuda"), torch.empty(B, L, d, device="cuda"))
+    flopv = B * (8 * 2 * L * D * L * d + 8 * 2 * L * L * d)
+    tv = gpu_times_ms(lambda: ops.dot_product_v(probs, quad(y), c["p"], c["eps"], 1, out=outv), 50, 5)
+    ev = op_entry("extra: context (probs.value) 4 heads [4,128,256,128].[4,128,256,64]", "mfma", tv, flopv)
+    return [e, ev]
 
 
 def bench_config4(args, ops, O, wl):
@@ -291,7 +301,7 @@ def main():
     if 2 in extra:
         entries += bench_config2(args, ops, O, wl)
     if 3 in extra:
-        entries.append(bench_config3(args, ops, O, wl))
+        entries += bench_config3(args, ops, O, wl)
     if 4 in extra:
         entries += bench_config4(args, ops, O, wl)
 

@@ -7,6 +7,7 @@ the methods on the accelerated path:
     concretize   Bounds.py:319-326        relu        :1163-1169 (ori_relu :921-963)
     matmul       :1177-1199 (ori_matmul :397-413)     tanh        :1171-1175 (ori_tanh :1027-1103)
     dense        :1016-1025               dot_product :833-841 (ori_dot_product :710-823)
+    t / context  :335-346, :843-850
     add          :383-395                 conv2d      HandTunedKernels/convolution_verification.cu:219-239
 
 Every method launches hand-written HIP kernels through the C ABI; none has a
@@ -85,9 +86,26 @@ class Bounds:
             return self.tanh()
         raise NotImplementedError(act_name)
 
-    # ---- Bounds.py:833-841 (scores path: self = query, other = key)
+    # ---- Bounds.py:335-346.  The transposed object is a pair of views that remembers where it came
+    # from, so that dot_product can read the original layout instead of materialising it.
+    def t(self):
+        r = self._like(self.lw.transpose(1, 3), self.lb.transpose(1, 2),
+                       self.uw.transpose(1, 3), self.ub.transpose(1, 2))
+        r._transpose_of = self
+        return r
+
+    # ---- Bounds.py:833-841.  Scores path: self = query, other = key.  Context path: other is the
+    # transposed value object (the reference tells the two apart by the shape of self.lb; here the
+    # transposed object says so itself).
     def dot_product(self, other):
+        src = getattr(other, "_transpose_of", None)
+        if src is not None:
+            return self._like(*ops.dot_product_v(self._c(), src._c(), self.p, self.eps, self.perturbed_words))
         return self._like(*ops.dot_product_qk(self._c(), other._c(), self.p, self.eps, self.perturbed_words))
+
+    # ---- Bounds.py:843-850
+    def context(self, value):
+        return self.dot_product(value.t())
 
 
 class ConvBounds:

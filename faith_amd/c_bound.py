@@ -70,6 +70,24 @@ def c_dot_product_verification_QK(x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_
     x_l.copy_(xl); x_u.copy_(xu); y_l.copy_(yl); y_u.copy_(yu)
 
 
+def c_dot_product_verification_V(x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
+                                 z_lb, z_ub, z_lw, z_uw, batch_size, length, dim_out, dim_in, epsilon):
+    """kernel.cpp:188-241; adapter Bounds.py:1306-1343.  x_* is the probability object with lw transposed
+    to [B, L, L, dim_in]; y_* is the TRANSPOSED value object (lb [B, dim_out, L], lw [B, dim_out, L, dim_in]);
+    z_lw, z_uw are [B, L, dim_out, dim_in].  The kernel reads values in their natural layout, so this
+    compatibility entry re-lays the operands out with torch copies, as the QK entry does."""
+    xn = [t.transpose(2, 3).contiguous() for t in (x_lw, x_uw)]                    # [B, L, dim_in, L]
+    yn = [t.permute(0, 2, 3, 1).contiguous() for t in (y_lw, y_uw)]                # [B, L, dim_in, dim_out]
+    ylb, yub = y_lb.transpose(1, 2).contiguous(), y_ub.transpose(1, 2).contiguous()  # [B, L, dim_out]
+    zlw, zlb, zuw, zub, (xl, xu, yl, yu) = ops.dot_product_v(
+        (xn[0], x_lb.contiguous(), xn[1], x_ub.contiguous()), (yn[0], ylb, yn[1], yub),
+        p, epsilon, words, return_intervals=True)
+    z_lw.copy_(zlw.transpose(2, 3)); z_uw.copy_(zuw.transpose(2, 3))
+    z_lb.copy_(zlb); z_ub.copy_(zub)
+    x_l.copy_(xl); x_u.copy_(xu)
+    y_l.copy_(yl.transpose(1, 2)); y_u.copy_(yu.transpose(1, 2))
+
+
 def c_matmul_verification(x_lb, x_ub, x_lw, x_uw, W, y_lb, y_ub, y_lw, y_uw,
                           batch_size, length, dim_in, dim_out, dim_y_out):
     """kernel.cpp:243-266 (commented out there; natural layout, no bias)."""

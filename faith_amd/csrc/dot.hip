@@ -64,8 +64,15 @@ enum { XL = 0, XU, BT, AL, AU, YL, YU, NOPS };
 // loads of the next step -- the first K-step of the next tile included -- are issued before the
 // MFMAs of the current step, and the accumulator stores of a finished tile are issued while
 // those loads are in flight, so neither the head nor the tail of a tile leaves the MFMA pipe idle.
+//
+// VP = false: scores path, y is [B, Ly, D, d] (reduction axis contiguous, like x).
+// VP = true : context path (probs . value): y is the value bound object in its own natural layout
+//   [B, d, D, Ly] -- the reduction axis (key position) is the slow one and j is contiguous --
+//   and so are its concrete bounds [B, d, Ly].  The y-side tiles are then staged as [k][j]
+//   (16-byte loads along j, conflict-free) and their fragments read with four 4-byte LDS reads.
+template <bool VP>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-dot_qk_w(const DotArgs g, const int total_tiles) {
+dot_w(const DotArgs g, const int total_tiles) {
     __shared__ float sm[2][NOPS][TILE];
 
     const int ti = (g.Lx + TI - 1) / TI, tj = (g.Ly + TJ - 1) / TJ;
@@ -80,47 +87,70 @@ dot_qk_w(const DotArgs g, const int total_tiles) {
     // ---- staging: one float4 per operand per thread per K-step
     const int srow = tid / 2, sc = tid % 2;
     const int sdst = swz(srow, sc);
+    const int vk = tid / 32, vj = (tid % 32) * 4;          // VP: this thread's (k, j..j+3) of a y-side tile
+    const int ydst = VP ? vk * TJ + vj : sdst;
     // element offsets of this thread's source rows (32-bit: the entry point checks the sizes);
     // xlw / xuw share one, ylw / yuw share one, a_l / a_u share one
     unsigned ox, oy, obt, oa;
+    bool y_in = true;                                      // VP: columns past Ly are staged as zeros
     float4 pre[NOPS];
     auto point_at = [&](int tile) {
         int q = tile;
         const int j0 = (q % tj) * TJ;  q /= tj;
         const int i0 = (q % ti) * TI;  q /= ti;
         const int m = q % g.D, t = q / g.D;
-        const int irow = min(i0 + srow, g.Lx - 1), jrow = min(j0 + srow, g.Ly - 1);   // clamped rows are never stored
+        const int irow = min(i0 + srow, g.Lx - 1);         // clamped rows are never stored
         ox = ((unsigned)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
-        oy = ((unsigned)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
         obt = (unsigned)(t * g.Lx + irow) * d + sc * 4;
-        oa = (unsigned)(t * g.Ly + jrow) * d + sc * 4;
+        if (VP) {
+            y_in = j0 + vj < g.Ly;                         // Ly % 4 == 0
+            oy = ((unsigned)(t * d + vk) * g.D + m) * g.Ly + j0 + vj;
+            oa = (unsigned)(t * d + vk) * g.Ly + j0 + vj;
+        } else {
+            const int jrow = min(j0 + srow, g.Ly - 1);
+            oy = ((unsigned)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
+            oa = (unsigned)(t * g.Ly + jrow) * d + sc * 4;
+        }
     };
     auto gload = [&](int kt) {
         const int k = kt * BK;
-        if (k + sc * 4 < d) {                      // d % 4 == 0: a float4 is all in or all out
-            pre[XL] = ld4(g.xlw + ox + k);
-            pre[XU] = ld4(g.xuw + ox + k);
-            pre[BT] = ld4(g.x_l + obt + k);
-            pre[AL] = ld4(g.y_l + oa + k);
-            pre[AU] = ld4(g.y_u + oa + k);
-            pre[YL] = ld4(g.ylw + oy + k);
-            pre[YU] = ld4(g.yuw + oy + k);
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+        const bool x_ok = k + sc * 4 < d;                  // d % 4 == 0: a float4 is all in or all out
+        pre[XL] = x_ok ? ld4(g.xlw + ox + k) : zero;
+        pre[XU] = x_ok ? ld4(g.xuw + ox + k) : zero;
+        pre[BT] = x_ok ? ld4(g.x_l + obt + k) : zero;
+        if (VP) {
+            const bool y_ok = y_in && k + vk < d;
+            const unsigned ky = (unsigned)k * g.D * g.Ly, ka = (unsigned)k * g.Ly;
+            pre[AL] = y_ok ? ld4(g.y_l + oa + ka) : zero;
+            pre[AU] = y_ok ? ld4(g.y_u + oa + ka) : zero;
+            pre[YL] = y_ok ? ld4(g.ylw + oy + ky) : zero;
+            pre[YU] = y_ok ? ld4(g.yuw + oy + ky) : zero;
         } else {
-#pragma unroll
-            for (int o = 0; o < NOPS; ++o) pre[o] = make_float4(0.f, 0.f, 0.f, 0.f);
+            pre[AL] = x_ok ? ld4(g.y_l + oa + k) : zero;
+            pre[AU] = x_ok ? ld4(g.y_u + oa + k) : zero;
+            pre[YL] = x_ok ? ld4(g.ylw + oy + k) : zero;
+            pre[YU] = x_ok ? ld4(g.yuw + oy + k) : zero;
         }
     };
     auto lstore = [&](int buf) {
 #pragma unroll
-        for (int o = 0; o < NOPS; ++o) *reinterpret_cast<float4 *>(&sm[buf][o][sdst]) = pre[o];
+        for (int o = 0; o < NOPS; ++o)
+            *reinterpret_cast<float4 *>(&sm[buf][o][(o == XL || o == XU || o == BT) ? sdst : ydst]) = pre[o];
+    };
+    // y-side fragment of block b: four K values of column j; [j][k] tile -> one 16-byte read,
+    // [k][j] tile (VP) -> four 4-byte reads, lanes along j
+    auto yfrag = [&](int buf, int o, int b) -> float4 {
+        if (VP) {
+            const float *p = &sm[buf][o][(4 * fh) * TJ + wj * 64 + b * 32 + fi];
+            return make_float4(p[0], p[TJ], p[2 * TJ], p[3 * TJ]);
+        }
+        return *reinterpret_cast<const float4 *>(&sm[buf][o][swz(wj * 64 + b * 32 + fi, fh)]);
     };
 
-    int fa[2], fb[2];
+    int fa[2];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        fa[s] = swz(wi * 64 + s * 32 + fi, fh);
-        fb[s] = swz(wj * 64 + s * 32 + fi, fh);
-    }
+    for (int s = 0; s < 2; ++s) fa[s] = swz(wi * 64 + s * 32 + fi, fh);
 
     floatx16 cl[2][2], cu[2][2];
     int tile = blockIdx.x;
@@ -158,10 +188,8 @@ dot_qk_w(const DotArgs g, const int total_tiles) {
             }
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
-                const float4 al = *reinterpret_cast<const float4 *>(&sm[buf][AL][fb[b]]);
-                const float4 au = *reinterpret_cast<const float4 *>(&sm[buf][AU][fb[b]]);
-                const float4 yl = *reinterpret_cast<const float4 *>(&sm[buf][YL][fb[b]]);
-                const float4 yu = *reinterpret_cast<const float4 *>(&sm[buf][YU][fb[b]]);
+                const float4 al = yfrag(buf, AL, b), au = yfrag(buf, AU, b);
+                const float4 yl = yfrag(buf, YL, b), yu = yfrag(buf, YU, b);
                 const float4 alp = pos4(al), aln = neg4(al), aup = pos4(au), aun = neg4(au);
 #define FAITH_DOT_STEP(c)                                   \
     _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
@@ -227,7 +255,8 @@ dot_qk_w(const DotArgs g, const int total_tiles) {
 
 // Any-shape coefficient kernel (d not a multiple of 4, unaligned pointers): one thread per
 // (i, m, j), products and sums in double.
-__global__ void __launch_bounds__(256) dot_qk_w_simple(const DotArgs g) {
+template <bool VP>
+__global__ void __launch_bounds__(256) dot_w_simple(const DotArgs g) {
     const size_t total = (size_t)g.B * g.Lx * g.D * g.Ly;
     for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
         const int j = idx % g.Ly;
@@ -236,18 +265,21 @@ __global__ void __launch_bounds__(256) dot_qk_w_simple(const DotArgs g) {
         const int t = idx / ((size_t)g.Ly * g.D * g.Lx);
         const float *xl = g.xlw + ((size_t)(t * g.Lx + i) * g.D + m) * g.d;
         const float *xu = g.xuw + ((size_t)(t * g.Lx + i) * g.D + m) * g.d;
-        const float *yl = g.ylw + ((size_t)(t * g.Ly + j) * g.D + m) * g.d;
-        const float *yu = g.yuw + ((size_t)(t * g.Ly + j) * g.D + m) * g.d;
+        // y element (j, m, k): scores path [t, j, m, k]; context path [t, k, m, j]
+        const size_t ybase = VP ? ((size_t)t * g.d * g.D + m) * g.Ly + j : ((size_t)(t * g.Ly + j) * g.D + m) * g.d;
+        const size_t ystep = VP ? (size_t)g.D * g.Ly : 1;
+        const size_t abase = VP ? (size_t)t * g.d * g.Ly + j : (size_t)(t * g.Ly + j) * g.d;
+        const size_t astep = VP ? g.Ly : 1;
         const float *bt = g.x_l + (size_t)(t * g.Lx + i) * g.d;
-        const float *al = g.y_l + (size_t)(t * g.Ly + j) * g.d;
-        const float *au = g.y_u + (size_t)(t * g.Ly + j) * g.d;
         double sl = 0.0, su = 0.0;
         for (int k = 0; k < g.d; ++k) {
+            const float yl = g.ylw[ybase + k * ystep], yu = g.yuw[ybase + k * ystep];
+            const float al = g.y_l[abase + k * astep], au = g.y_u[abase + k * astep];
             const double bp = fmaxf(bt[k], 0.f), bn = fminf(bt[k], 0.f);
-            const double alp = fmaxf(al[k], 0.f), aln = fminf(al[k], 0.f);
-            const double aup = fmaxf(au[k], 0.f), aun = fminf(au[k], 0.f);
-            sl += xl[k] * alp + xu[k] * aln + bp * yl[k] + bn * yu[k];
-            su += xu[k] * aup + xl[k] * aun + bp * yu[k] + bn * yl[k];
+            const double alp = fmaxf(al, 0.f), aln = fminf(al, 0.f);
+            const double aup = fmaxf(au, 0.f), aun = fminf(au, 0.f);
+            sl += xl[k] * alp + xu[k] * aln + bp * yl + bn * yu;
+            su += xu[k] * aup + xl[k] * aun + bp * yu + bn * yl;
         }
         g.zlw[idx] = (float)sl;
         g.zuw[idx] = (float)su;
@@ -257,7 +289,8 @@ __global__ void __launch_bounds__(256) dot_qk_w_simple(const DotArgs g) {
 // Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns a 16 x 16 tile of
 // (i, j) of one head, stages the seven [16 x d-chunk] operand rows in LDS and sums in double.
 constexpr int BT_T = 16, BT_K = 64;
-__global__ void __launch_bounds__(256) dot_qk_b(const DotArgs g) {
+template <bool VP>
+__global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
     __shared__ float sx[3][BT_T][BT_K + 1];     // b (= l_x), xlb, xub
     __shared__ float sy[4][BT_T][BT_K + 1];     // a_l, a_u, ylb, yub
     const int ti = (g.Lx + BT_T - 1) / BT_T, tj = (g.Ly + BT_T - 1) / BT_T;
@@ -273,7 +306,7 @@ __global__ void __launch_bounds__(256) dot_qk_b(const DotArgs g) {
             const bool kin = k0 + k < g.d;
             const bool xin = kin && i0 + r < g.Lx, yin = kin && j0 + r < g.Ly;
             const size_t xo = (size_t)(t * g.Lx + i0 + r) * g.d + k0 + k;
-            const size_t yo = (size_t)(t * g.Ly + j0 + r) * g.d + k0 + k;
+            const size_t yo = VP ? (size_t)(t * g.d + k0 + k) * g.Ly + j0 + r : (size_t)(t * g.Ly + j0 + r) * g.d + k0 + k;
             sx[0][r][k] = xin ? g.x_l[xo] : 0.f;
             sx[1][r][k] = xin ? g.xlb[xo] : 0.f;
             sx[2][r][k] = xin ? g.xub[xo] : 0.f;
@@ -303,17 +336,19 @@ __global__ void __launch_bounds__(256) dot_qk_b(const DotArgs g) {
 
 // dim_in == 1: the reference switches to plain interval arithmetic on the constant terms and
 // returns zero coefficients (Bounds.py:711-721).
-__global__ void __launch_bounds__(256) dot_qk_interval(const DotArgs g) {
+template <bool VP>
+__global__ void __launch_bounds__(256) dot_interval(const DotArgs g) {
     const size_t total = (size_t)g.B * g.Lx * g.Ly;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int j = idx % g.Ly;
     const int i = (idx / g.Ly) % g.Lx;
     const int t = idx / ((size_t)g.Ly * g.Lx);
-    const size_t xo = (size_t)(t * g.Lx + i) * g.d, yo = (size_t)(t * g.Ly + j) * g.d;
+    const size_t xo = (size_t)(t * g.Lx + i) * g.d;
+    const size_t yo = VP ? (size_t)t * g.d * g.Ly + j : (size_t)(t * g.Ly + j) * g.d, ys = VP ? g.Ly : 1;
     float lo = 0.f, hi = 0.f;
     for (int k = 0; k < g.d; ++k) {
-        const float l1 = g.xlb[xo + k], u1 = g.xub[xo + k], l2 = g.ylb[yo + k], u2 = g.yub[yo + k];
+        const float l1 = g.xlb[xo + k], u1 = g.xub[xo + k], l2 = g.ylb[yo + k * ys], u2 = g.yub[yo + k * ys];
         const float c1 = l1 * l2, c2 = l1 * u2, c3 = u1 * l2, c4 = u1 * u2;
         lo += fminf(fminf(c1, c2), fminf(c3, c4));
         hi += fmaxf(fmaxf(c1, c2), fmaxf(c3, c4));
@@ -322,6 +357,73 @@ __global__ void __launch_bounds__(256) dot_qk_interval(const DotArgs g) {
     g.zub[idx] = hi;
     g.zlw[idx] = 0.f;      // [B, Lx, 1, Ly] has the same linear index
     g.zuw[idx] = 0.f;
+}
+
+// Shared body of the two entry points.  For the context path (VP) `d` is the number of key positions
+// (the reduction length) and `Ly` the width of the value vectors; y_* are the value bounds in their
+// natural layout [B, d, D, Ly] / [B, d, Ly].
+template <bool VP>
+int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb, const float *x_ub,
+              const float *y_lb, const float *y_ub, const float *x_lw, const float *x_uw, const float *y_lw,
+              const float *y_uw, float *z_lb, float *z_ub, float *z_lw, float *z_uw, int B, int Lx, int Ly, int d, int D,
+              float epsilon, int q, int words, void *stream) {
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
+    FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
+    FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_ALIGNED4(z_lw); FAITH_ALIGNED4(z_uw); FAITH_ALIGNED4(z_lb); FAITH_ALIGNED4(z_ub);
+    FAITH_REQUIRE(B > 0 && Lx > 0 && Ly > 0 && d > 0 && D > 0, FAITH_ERR_SHAPE,
+                  "%s: batch=%d rows of x=%d columns of z=%d reduction length=%d dim_in=%d must be positive", who, B,
+                  Lx, Ly, d, D);
+    const long long nw = (long long)B * Lx * D * Ly;
+    const long long nx = (long long)B * Lx * D * d, ny = (long long)B * Ly * D * d;
+    FAITH_REQUIRE((long long)B * (Lx > Ly ? Lx : Ly) * D <= 0x7fffffffLL && (long long)B * d * D <= 0x7fffffffLL,
+                  FAITH_ERR_SHAPE, "%s: batch*length*dim_in exceeds 2^31", who);
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DotArgs g{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub, B, Lx, Ly, D, d};
+    if (D == 1) {
+        const long long n = (long long)B * Lx * Ly;
+        hipLaunchKernelGGL(dot_interval<VP>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, g);
+        return faith::check_launch(who);
+    }
+
+    // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the reference
+    // interface exposes it, the planes do not use it.  One launch when both objects have the same
+    // [D, H] shape (always on the scores path).
+    const int y_rows = VP ? B * d : B * Ly, y_h = VP ? Ly : d;
+    int rc;
+    if (y_h == d) {
+        rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, B * Lx, y_lb, y_ub, y_lw, y_uw, y_l, y_u, y_rows,
+                                    D, d, epsilon, q, words, stream);
+    } else {
+        rc = faith_concretize(x_lb, x_ub, x_lw, x_uw, x_l, x_u, B * Lx, D, d, epsilon, q, words,
+                              FAITH_LAYOUT_NATURAL, stream);
+        if (rc == FAITH_OK)
+            rc = faith_concretize(y_lb, y_ub, y_lw, y_uw, y_l, y_u, y_rows, D, y_h, epsilon, q, words,
+                                  FAITH_LAYOUT_NATURAL, stream);
+    }
+    if (rc != FAITH_OK) return rc;
+
+    hipLaunchKernelGGL(dot_b<VP>, dim3((unsigned)((long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T))),
+                       dim3(256), 0, st, g);
+
+    const bool fast = (d % 4 == 0) && (!VP || Ly % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
+                      faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
+                      faith::aligned(y_l, 16) && faith::aligned(y_u, 16) && nw < 0xffffffffLL && nx < 0xffffffffLL &&
+                      ny < 0xffffffffLL;
+    if (fast) {
+        const long long tiles = (long long)B * D * ((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ);
+        FAITH_REQUIRE(tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: too many tiles", who);
+        const long long resident = 2LL * faith::compute_units();      // 56 KB of LDS each: two per CU
+        hipLaunchKernelGGL(dot_w<VP>, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(NTHREADS), 0, st, g,
+                           (int)tiles);
+    } else {
+        const long long blocks = (nw + 255) / 256;
+        hipLaunchKernelGGL(dot_w_simple<VP>, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
+    }
+    return faith::check_launch(who);
 }
 
 }  // namespace
@@ -333,58 +435,18 @@ extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *
                                                  float *z_uw, int batch_size, int length_x, int length_y,
                                                  int dim_out, int dim_in, float epsilon, int q, int words,
                                                  void *stream) {
-    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
-    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
-    FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
-    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
-    FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
-    FAITH_ALIGNED4(z_lw); FAITH_ALIGNED4(z_uw); FAITH_ALIGNED4(z_lb); FAITH_ALIGNED4(z_ub);
-    FAITH_REQUIRE(batch_size > 0 && length_x > 0 && length_y > 0 && dim_out > 0 && dim_in > 0, FAITH_ERR_SHAPE,
-                  "faith_dot_product_verification_QK: batch=%d length_x=%d length_y=%d dim_out=%d dim_in=%d "
-                  "must be positive", batch_size, length_x, length_y, dim_out, dim_in);
-    const long long nw = (long long)batch_size * length_x * dim_in * length_y;
-    FAITH_REQUIRE((long long)batch_size * (length_x > length_y ? length_x : length_y) * dim_in <= 0x7fffffffLL,
-                  FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: batch*length*dim_in exceeds 2^31");
+    return dot_entry<false>("faith_dot_product_verification_QK", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
+                            y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, length_y, dim_out, dim_in, epsilon,
+                            q, words, stream);
+}
 
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dim_in == 1) {
-        DotArgs gi{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub,
-                   batch_size, length_x, length_y, dim_in, dim_out};
-        const long long n = (long long)batch_size * length_x * length_y;
-        hipLaunchKernelGGL(dot_qk_interval, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gi);
-        return faith::check_launch("faith_dot_product_verification_QK");
-    }
-
-    // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the
-    // reference interface exposes it, the planes do not use it
-    const int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, batch_size * length_x, y_lb, y_ub, y_lw,
-                                          y_uw, y_l, y_u, batch_size * length_y, dim_in, dim_out, epsilon, q, words,
-                                          stream);
-    if (rc != FAITH_OK) return rc;
-
-    DotArgs g{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub,
-              batch_size, length_x, length_y, dim_in, dim_out};
-    const long long nb = (long long)batch_size * length_x * length_y;
-    (void)nb;
-    hipLaunchKernelGGL(dot_qk_b, dim3((unsigned)((long long)batch_size * ((length_x + BT_T - 1) / BT_T) *
-                                                 ((length_y + BT_T - 1) / BT_T))),
-                       dim3(256), 0, st, g);
-
-    const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
-                      faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
-                      faith::aligned(y_l, 16) && faith::aligned(y_u, 16);
-    if (fast) {
-        FAITH_REQUIRE(nw < 0xffffffffLL && (long long)batch_size * (length_x > length_y ? length_x : length_y) *
-                                              dim_in * dim_out < 0xffffffffLL,
-                      FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: tensors beyond 2^32 elements");
-        const long long tiles = (long long)batch_size * dim_in * ((length_x + TI - 1) / TI) * ((length_y + TJ - 1) / TJ);
-        FAITH_REQUIRE(tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_dot_product_verification_QK: too many tiles");
-        const long long resident = 2LL * faith::compute_units();      // 56 KB of LDS each: two per CU
-        hipLaunchKernelGGL(dot_qk_w, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(NTHREADS), 0, st, g,
-                           (int)tiles);
-    } else {
-        const long long blocks = (nw + 255) / 256;
-        hipLaunchKernelGGL(dot_qk_w_simple, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
-    }
-    return faith::check_launch("faith_dot_product_verification_QK");
+extern "C" int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
+                                                const float *x_ub, const float *y_lb, const float *y_ub,
+                                                const float *x_lw, const float *x_uw, const float *y_lw,
+                                                const float *y_uw, float *z_lb, float *z_ub, float *z_lw,
+                                                float *z_uw, int batch_size, int length_x, int length_k, int dim_out,
+                                                int dim_in, float epsilon, int q, int words, void *stream) {
+    return dot_entry<true>("faith_dot_product_verification_V", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
+                           y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, dim_out, length_k, dim_in, epsilon,
+                           q, words, stream);
 }

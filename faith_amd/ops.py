@@ -179,6 +179,43 @@ def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
     return zlw, zlb, zuw, zub
 
 
+def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
+    """McCormick bounds of the attention context x . y (probabilities times values).
+
+    x: (lw [B, Lx, D, Lk], lb [B, Lx, Lk], uw, ub);  y: the VALUE bounds in their natural layout
+    (lw [B, Lk, D, dv], lb [B, Lk, dv], uw, ub) -- no transposed copy is needed.
+    Returns (lw [B, Lx, D, dv], lb [B, Lx, dv], uw, ub)."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    B, Lx, D, Lk = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    B2, Lk2, D2, dv = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
+    if (B2, Lk2, D2) != (B, Lk, D):
+        raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} disagree in batch, key length or dim_in")
+    for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                    ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
+        _check(n, t, s)
+    dev = xlw.device
+    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
+    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
+    if out is None:
+        zlw = torch.empty(B, Lx, D, dv, device=dev, dtype=torch.float32)
+        zuw = torch.empty_like(zlw)
+        zlb = torch.empty(B, Lx, dv, device=dev, dtype=torch.float32)
+        zub = torch.empty_like(zlb)
+    else:
+        zlw, zlb, zuw, zub = out
+        _check("out lw", zlw, (B, Lx, D, dv)); _check("out uw", zuw, (B, Lx, D, dv))
+        _check("out lb", zlb, (B, Lx, dv)); _check("out ub", zub, (B, Lx, dv))
+    with _on(dev):
+        _lib.call("faith_dot_product_verification_V", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
+                  _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
+                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Lk, dv, D, float(eps), q_code(p), int(words),
+                  _stream(xlw))
+    if return_intervals:
+        return zlw, zlb, zuw, zub, (x_l, x_u, y_l, y_u)
+    return zlw, zlb, zuw, zub
+
+
 def conv2d(lw, lb, uw, ub, weight, bias=None, stride=1, padding=0, out=None):
     """Sign-split propagation through a 2-D convolution.
     lw, uw: [1, D_in, C_in, H, W]; lb, ub: [1, C_in, H, W]; weight: [C_out, C_in, K, K]."""

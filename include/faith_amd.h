@@ -137,6 +137,27 @@ int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float 
                                       int q, int words, void *stream);
 
 /*
+ * McCormick bounds of the attention context  z[i,j] = sum_k x[i,k] * y[k,j]  (probabilities times
+ * values).  Replaces call_dot_product_verification_V (kernel.cpp:53-60,
+ * dot_product_verification.cu:498-535) with the arithmetic of Bounds.context -> ori_dot_product
+ * (Bounds.py:843-850, :710-823).  The value bounds are taken in their own natural layout: the
+ * transposed views that Bounds.t() builds (Bounds.py:335-346) are never materialised.
+ *   x_lw, x_uw [batch, length_x, dim_in, length_k];  x_lb, x_ub [batch, length_x, length_k]
+ *   y_lw, y_uw [batch, length_k, dim_in, dim_out];   y_lb, y_ub [batch, length_k, dim_out]
+ *   x_l, x_u   [batch, length_x, length_k];  y_l, y_u [batch, length_k, dim_out]   (out / scratch)
+ *   z_lw, z_uw [batch, length_x, dim_in, dim_out];   z_lb, z_ub [batch, length_x, dim_out]
+ */
+int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *y_u,
+                                     const float *x_lb, const float *x_ub,
+                                     const float *y_lb, const float *y_ub,
+                                     const float *x_lw, const float *x_uw,
+                                     const float *y_lw, const float *y_uw,
+                                     float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                                     int batch_size, int length_x, int length_k,
+                                     int dim_out, int dim_in, float epsilon,
+                                     int q, int words, void *stream);
+
+/*
  * Sign-split propagation through a 2-D convolution (NCHW).  Replaces the (commented-out)
  * call_convolution_verification (kernel.cpp:62-67, convolution_verification.cu:219-239).
  *   x_lw, x_uw [dim_in, CIN, Height, Width]   (dim_in plays the conv batch)

@@ -27,6 +27,8 @@ Parity status of each function (what pins it, see tests/test_oracle_*.py):
                and nvcc at import time).
   dot_product  pinned: brute-force five-deep loop on tiny shapes, einsum
                restatement, sampled soundness of the McCormick planes.
+  context      the same function on transposed views; pinned by the brute-force loop
+               fed with explicitly transposed numpy arrays.
   conv         pinned: brute-force loops, 1x1 conv == linear, F.conv2d
                linearity.  The reference has NO Python conv bound; semantics
                come from HandTunedKernels/convolution_verification.cu:124-138
@@ -287,6 +289,21 @@ def dot_product(x: LinearBounds, y: LinearBounds, p: float, eps: float, words: i
         y_term_b(ub, y.ub, b_lu, torch.gt)
         y_term_b(ub, y.lb, b_lu, torch.lt)
     return LinearBounds(lw, lb, uw, ub)
+
+
+def transpose_bounds(v: LinearBounds) -> LinearBounds:
+    """Bounds.t (Bounds.py:335-346): swap the length and the hidden axis (views, no copy)."""
+    return LinearBounds(v.lw.transpose(1, 3), v.lb.transpose(1, 2), v.uw.transpose(1, 3), v.ub.transpose(1, 2))
+
+
+def context(probs: LinearBounds, value: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.context (Bounds.py:843-850): z[i, j] = sum_k probs[i, k] * value[k, j].
+
+    probs: lw [B, L, D, L], lb [B, L, L];  value: lw [B, L, D, dim_out], lb [B, L, dim_out]
+    -> lw [B, L, D, dim_out], lb [B, L, dim_out].  It is the dot product of probs with the
+    transposed value bounds.
+    """
+    return dot_product(probs, transpose_bounds(value), p, eps, words)
 
 
 # --------------------------------------------------------------------------

@@ -118,3 +118,103 @@ def test_dot_config3_full_size_properties():
     tol = lambda r, m: 1e-6 + 1e-5 * r.abs() + 8 * 2.0 ** -24 * m
     assert bool(((zlw[t].cpu().double() - ref["lw"][0]).abs() <= tol(ref["lw"][0], mag["lw"][0])).all())
     assert bool(((zub[t].cpu().double() - ref["ub"][0]).abs() <= tol(ref["ub"][0], mag["ub"][0])).all())
+
+
+# ------------------------------------------------------------------ context path (probs . value)
+def check_v(probs, value, p, eps, words, what=""):
+    from faith_amd import ops
+    print(f"[case] context {what} probs={tuple(probs.lw.shape)} value={tuple(value.lw.shape)} p={p} eps={eps}", flush=True)
+    zlw, zlb, zuw, zub, (xl, xu, yl, yu) = ops.dot_product_v(dev(probs), dev(value), p, eps, words,
+                                                             return_intervals=True)
+    torch.cuda.synchronize()
+    exp = O.context(probs, value, p, eps, words)
+    if probs.lw.shape[2] == 1:
+        for g, e in zip((zlw, zlb, zuw, zub), exp.tensors()):
+            assert close(g, e)
+        return
+    el, eu = O.concretize(value, p, eps, words)
+    assert close(yl, el) and close(yu, eu)
+    ref, mag = dot64(probs, O.transpose_bounds(value), p, eps, words)
+    for name, g, e in zip(("lw", "lb", "uw", "ub"), (zlw, zlb, zuw, zub), exp.tensors()):
+        assert g.shape == e.shape
+        compare_contraction(name, g, e, ref[name], mag[name])
+
+
+@pytest.mark.parametrize("shape", [
+    # B, L (queries = keys), D, dim_out of the values
+    (1, 2, 64, 16), (2, 16, 64, 64), (2, 32, 32, 20),
+    (1, 130, 12, 72),      # L off the tile in both roles
+    (2, 8, 5, 12),         # tiny
+    (1, 6, 4, 10),         # value width % 4 != 0: any-shape kernel
+    (1, 5, 3, 8),          # key length % 4 != 0: any-shape kernel
+    (2, 4, 1, 8),          # dim_in == 1: interval shortcut
+])
+@pytest.mark.parametrize("p", [1.0, 2.0, INF])
+def test_context_shapes(shape, p):
+    B, L, D, dv = shape
+    g = torch.Generator().manual_seed(33)
+    probs = rand_bounds(g, B, L, D, L, ordered=False, sw=0.2, sb=0.5)
+    value = rand_bounds(g, B, L, D, dv, ordered=False, sw=0.3, sb=1.0)
+    check_v(probs, value, p, 0.1, 1, "sweep")
+
+
+def test_context_rectangular_and_two_words():
+    """More keys than queries, two perturbed words."""
+    g = torch.Generator().manual_seed(34)
+    probs = rand_bounds(g, 2, 12, 64, 40, sw=0.2, sb=0.5)      # 12 queries over 40 keys
+    value = rand_bounds(g, 2, 40, 64, 32, sw=0.2)
+    check_v(probs, value, 2.0, 0.05, 2, "Lx != Lk, words=2")
+
+
+def test_bounds_class_dispatches_context_to_the_native_kernel():
+    """Bounds.context(value) == dot_product(value.t()) and matches the oracle; the transposed
+    object is never materialised (reference: Bounds.py:833-850)."""
+    from faith_amd import Bounds
+    g = torch.Generator().manual_seed(35)
+    probs = rand_bounds(g, 2, 16, 32, 16, sw=0.2, sb=0.5)
+    value = rand_bounds(g, 2, 16, 32, 24, sw=0.2)
+    bp = Bounds(None, 2.0, 0.05, lw=probs.lw.cuda(), lb=probs.lb.cuda(), uw=probs.uw.cuda(), ub=probs.ub.cuda())
+    bv = Bounds(None, 2.0, 0.05, lw=value.lw.cuda(), lb=value.lb.cuda(), uw=value.uw.cuda(), ub=value.ub.cuda())
+    z = bp.context(bv)
+    exp = O.context(probs, value, 2.0, 0.05)
+    ref, mag = dot64(probs, O.transpose_bounds(value), 2.0, 0.05, 1)
+    for name, g_, e in zip(("lw", "lb", "uw", "ub"), (z.lw, z.lb, z.uw, z.ub), exp.tensors()):
+        compare_contraction(name, g_, e, ref[name], mag[name])
+    # scores path through the class as well
+    s = bp.dot_product(bp)
+    es = O.dot_product(probs, probs, 2.0, 0.05)
+    rs, ms = dot64(probs, probs, 2.0, 0.05, 1)
+    for name, g_, e in zip(("lw", "lb", "uw", "ub"), (s.lw, s.lb, s.uw, s.ub), es.tensors()):
+        compare_contraction(name, g_, e, rs[name], ms[name])
+
+
+def test_c_bound_dot_shims():
+    """Reference calling convention of the two dot-product entries (kernel.cpp:133-241): transposed
+    operands, caller-allocated outputs, z_lw as [B, L, L|dim_out, dim_in]."""
+    from faith_amd import c_bound
+    g = torch.Generator().manual_seed(36)
+    B, L, D, d = 2, 8, 16, 12
+    x = rand_bounds(g, B, L, D, d, sw=0.2); y = rand_bounds(g, B, L, D, d, sw=0.2)
+    T = lambda t_: t_.cuda().transpose(2, 3).contiguous()
+    z = lambda *s_: torch.zeros(*s_, device="cuda")
+    x_l, y_l, x_u, y_u = z(B, L, d), z(B, L, d), z(B, L, d), z(B, L, d)
+    zlb, zub, zlw, zuw = z(B, L, L), z(B, L, L), z(B, L, L, D), z(B, L, L, D)
+    c_bound.p, c_bound.words = 2.0, 1
+    c_bound.c_dot_product_verification_QK(x_l, y_l, x_u, y_u, x.lb.cuda(), x.ub.cuda(), y.lb.cuda(), y.ub.cuda(),
+                                          T(x.lw), T(x.uw), T(y.lw), T(y.uw), zlb, zub, zlw, zuw, B, L, d, D, 0.05)
+    e = O.dot_product(x, y, 2.0, 0.05)
+    assert close(zlw.transpose(2, 3), e.lw, rtol=1e-5, atol=2e-6) and close(zub, e.ub, rtol=1e-5, atol=2e-6)
+    # context: probs [B, L, D, L], value [B, L, D, dv] handed over as the reference's adapter does
+    dv = 20
+    probs = rand_bounds(g, B, L, D, L, sw=0.2, sb=0.5); value = rand_bounds(g, B, L, D, dv, sw=0.2)
+    vt = O.transpose_bounds(value)                         # lw [B, dv, D, L], lb [B, dv, L]
+    x_l, x_u = z(B, L, L), z(B, L, L)
+    y_l, y_u = z(B, dv, L), z(B, dv, L)
+    zlb, zub, zlw, zuw = z(B, L, dv), z(B, L, dv), z(B, L, dv, D), z(B, L, dv, D)
+    c_bound.c_dot_product_verification_V(x_l, y_l, x_u, y_u, probs.lb.cuda(), probs.ub.cuda(),
+                                         vt.lb.cuda().contiguous(), vt.ub.cuda().contiguous(),
+                                         T(probs.lw), T(probs.uw), T(vt.lw), T(vt.uw),
+                                         zlb, zub, zlw, zuw, B, L, dv, D, 0.05)
+    e = O.context(probs, value, 2.0, 0.05)
+    assert close(zlw.transpose(2, 3), e.lw, rtol=1e-5, atol=2e-6) and close(zlb, e.lb, rtol=1e-5, atol=2e-6)
+    assert close(zuw.transpose(2, 3), e.uw, rtol=1e-5, atol=2e-6) and close(zub, e.ub, rtol=1e-5, atol=2e-6)

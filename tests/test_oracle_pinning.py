@@ -359,3 +359,22 @@ def test_conv_concretize_soundness():
     for t in (0.0, 0.5, 1.0):
         v = torch.nn.functional.conv2d(xin_l + t * (xin_u - xin_l), W.double(), None, 1, 1)
         assert (v >= lo.double() - 1e-5).all() and (v <= hi.double() + 1e-5).all()
+
+
+# -------------------------------------------------------------------- context
+@pytest.mark.parametrize("p", PS)
+def test_context_vs_brute_force(p):
+    """probs . value with the value object transposed by hand in numpy (no torch views)."""
+    g = gen(21)
+    L, D, dv = 4, 3, 5
+    probs = rand_bounds(g, 2, L, D, L, ordered=False)
+    value = rand_bounds(g, 2, L, D, dv, ordered=False)
+    z = O.context(probs, value, p, 0.2)
+    assert z.lw.shape == (2, L, D, dv) and z.lb.shape == (2, L, dv)
+    for t in range(2):
+        y = [np.ascontiguousarray(f64(a)[t].transpose(2, 1, 0)) for a in (value.lw, value.uw)]     # [dv, D, L]
+        yb = [np.ascontiguousarray(f64(a)[t].T) for a in (value.lb, value.ub)]                      # [dv, L]
+        e = C.dot_brute(f64(probs.lw)[t], f64(probs.lb)[t], f64(probs.uw)[t], f64(probs.ub)[t],
+                        y[0], yb[0], y[1], yb[1], p, 0.2, 1)
+        for got, exp in zip((z.lw, z.lb, z.uw, z.ub), e):
+            np.testing.assert_allclose(f64(got)[t], exp, rtol=1e-5, atol=2e-6)
