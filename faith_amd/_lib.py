@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(HERE, "libfaith_amd.so")
 OK = 0
 Q_1, Q_2, Q_INF = 1, 2, 0
 LAYOUT_NATURAL, LAYOUT_TRANSPOSED = 0, 1
+OP_RELU, OP_TANH, OP_EXP, OP_RECIPROCAL, OP_SQR, OP_SQRT = 1, 2, 3, 4, 5, 6
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int
@@ -26,6 +27,7 @@ SIGNATURES = {
     "faith_concretize": [_P] * 6 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_relu_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_tanh_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
+    "faith_unary_verification": [_I] + [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],
     "faith_dot_product_verification_QK": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_dot_product_verification_V": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],

@@ -7,7 +7,7 @@ the methods on the accelerated path:
     concretize   Bounds.py:319-326        relu        :1163-1169 (ori_relu :921-963)
     matmul       :1177-1199 (ori_matmul :397-413)     tanh        :1171-1175 (ori_tanh :1027-1103)
     dense        :1016-1025               dot_product :833-841 (ori_dot_product :710-823)
-    t / context  :335-346, :843-850
+    t / context  :335-346, :843-850       exp / sqr / sqrt / reciprocal  :970-1003, :860-919, :1136-1161
     add          :383-395                 conv2d      HandTunedKernels/convolution_verification.cu:219-239
 
 Every method launches hand-written HIP kernels through the C ABI; none has a
@@ -78,6 +78,25 @@ class Bounds:
 
     def tanh(self):
         return self._like(*ops.tanh(*self._c(), self.p, self.eps, self.perturbed_words))
+
+    # ---- Bounds.py:970-1003, :860-890
+    def exp(self):
+        return self._like(*ops.exp(*self._c(), self.p, self.eps, self.perturbed_words))
+
+    def sqr(self):
+        return self._like(*ops.sqr(*self._c(), self.p, self.eps, self.perturbed_words))
+
+    # ---- Bounds.py:892-919, :1136-1161.  Both assert a positive interval in the reference; the
+    # check reads the concrete lower bound back from the kernel (one synchronisation).
+    def sqrt(self):
+        out = ops.sqrt(*self._c(), self.p, self.eps, self.perturbed_words, return_interval=True)
+        assert float(out[4].min()) > 0, "sqrt of a bound that reaches zero"
+        return self._like(*out[:4])
+
+    def reciprocal(self):
+        out = ops.reciprocal(*self._c(), self.p, self.eps, self.perturbed_words, return_interval=True)
+        assert float(out[4].min()) >= 1e-12, "reciprocal of a bound that reaches zero"
+        return self._like(*out[:4])
 
     def act(self, act_name):
         if act_name == "relu":

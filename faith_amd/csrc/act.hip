@@ -27,7 +27,8 @@ namespace {
 constexpr int WAVE = 64;
 constexpr float TINY = 1e-12f;   // Bounds.py:27
 
-enum Mode { CONCRETIZE = 0, RELU = 1, TANH = 2 };
+enum Mode { CONCRETIZE = 0, RELU = FAITH_OP_RELU, TANH = FAITH_OP_TANH, EXP = FAITH_OP_EXP, RECIP = FAITH_OP_RECIPROCAL,
+            SQR = FAITH_OP_SQR, SQRT = FAITH_OP_SQRT };
 
 struct ActArgs {
     const float *lb, *ub, *lw, *uw;
@@ -78,11 +79,63 @@ __device__ __forceinline__ void relu_lines(float l, float u, Line &lo, Line &up)
 }
 
 
+// exp with the reference's cap (Bounds.py:984-989): the tangent at 12 above 12.  In double.
+__device__ __forceinline__ double exp_capped(float x) {
+    return x < 12.f ? exp((double)x) : exp(12.0) * ((double)(x - 12.f) + 1.0);
+}
+
 // Bounds.add_linear, constant term (Bounds.py:378, :381): a positive slope takes the same-side
 // bound, a non-positive one the opposite bound; three separate roundings.
 __device__ __forceinline__ float line_bias(const Line &ln, float same, float other) {
     const float b = ln.k > 0.f ? same : other;
     return (b - ln.x0) * ln.k + ln.y0;
+}
+
+// Slopes and constant terms of every relaxation whose per-neuron work is a handful of operations
+// (everything but tanh).  fp32 operation order follows the reference line by line; exp itself is
+// taken in double and rounded once.
+template <int MODE>
+__device__ __forceinline__ void relax_point(float l, float u, float lb, float ub, float &klo, float &kup, float &olb,
+                                            float &oub) {
+    if (MODE == EXP) {                       // Bounds.py:970-1003
+        const float m = fminf((l + u) / 2, l + 0.99f);
+        klo = (float)exp((double)fminf(m, 12.f));
+        olb = klo * ((lb - m) + 1.f);
+        const double el = exp_capped(l), eu = exp_capped(u);
+        kup = (float)((eu - el) / (double)((u - l) + TINY));
+        oub = (ub * kup - kup * l) + (float)el;
+    } else if (MODE == RECIP) {              // Bounds.py:1136-1161 (positive intervals)
+        const float m = (l + u) / 2;
+        klo = -1.f / (m * m);
+        olb = ub * klo + 2.f / m;
+        kup = -1.f / (l * u);
+        oub = (lb * kup - kup * l) + 1.f / l;
+    } else {
+        Line lo, up;
+        if (MODE == RELU) {
+            relu_lines(l, u, lo, up);
+        } else if (MODE == SQR) {            // Bounds.py:860-890
+            up = {u + l, l, l * l};
+            if (u < 0.f) {
+                const float m = fmaxf((l + u) / 2, 2 * u);
+                lo = {2 * m, m, m * m};
+            } else if (l > 0.f) {
+                const float m = fminf((l + u) / 2, 2 * l);
+                lo = {2 * m, m, m * m};
+            } else {
+                lo = {0.f, 0.f, 0.f};
+            }
+        } else {                             // SQRT, Bounds.py:892-919 (positive intervals)
+            // the chord slope cancels when u - l is small: the difference is taken in double
+            lo = {(float)((sqrt((double)u) - sqrt((double)l)) / (double)((u - l) + TINY)), l, sqrtf(l)};
+            const float m = (l + u) / 2;
+            up = {0.5f / sqrtf(m), m, sqrtf(m)};
+        }
+        klo = lo.k;
+        kup = up.k;
+        olb = line_bias(lo, lb, ub);
+        oub = line_bias(up, ub, lb);
+    }
 }
 
 // ------------------------------------------------------------------ vector access
@@ -293,14 +346,13 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
         }
         if (p_l) p_l[bi] = l;
         if (p_u) p_u[bi] = u;
-        if (MODE == RELU) {
-            Line lo, up;
-            relu_lines(l, u, lo, up);
-            s_ln[lane] = lo.k;
-            s_ln[3 * TH + lane] = up.k;
-            const float lb = p_lb[bi], ub = p_ub[bi];
-            a.olb[bi] = line_bias(lo, lb, ub);
-            a.oub[bi] = line_bias(up, ub, lb);
+        if (MODE != TANH && MODE != CONCRETIZE) {
+            float klo, kup, olb, oub;
+            relax_point<MODE>(l, u, p_lb[bi], p_ub[bi], klo, kup, olb, oub);
+            s_ln[lane] = klo;
+            s_ln[3 * TH + lane] = kup;
+            a.olb[bi] = olb;
+            a.oub[bi] = oub;
         } else if (MODE == TANH) {
             s_lu[lane] = l;
             s_lu[TH + lane] = u;
@@ -373,15 +425,24 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     }
 }
 
+// All modes, one neuron per lane (used by the transposed-layout kernel).
 template <int MODE>
-__device__ __forceinline__ void make_lines(float l, float u, Line &lo, Line &up) {
-    if (MODE == RELU) {
-        relu_lines(l, u, lo, up);
-    } else if (u < 0.f || l > 0.f) {
-        tanh_pure_lines(l, u, lo, up);
+__device__ __forceinline__ void relax_any(float l, float u, float lb, float ub, float &klo, float &kup, float &olb,
+                                          float &oub) {
+    if (MODE == TANH) {
+        Line lo, up;
+        if (u < 0.f || l > 0.f) {
+            tanh_pure_lines(l, u, lo, up);
+        } else {
+            lo = tanh_tangent_line<true>(l, u);
+            up = tanh_tangent_line<false>(l, u);
+        }
+        klo = lo.k;
+        kup = up.k;
+        olb = line_bias(lo, lb, ub);
+        oub = line_bias(up, ub, lb);
     } else {
-        lo = tanh_tangent_line<true>(l, u);
-        up = tanh_tangent_line<false>(l, u);
+        relax_point<MODE>(l, u, lb, ub, klo, kup, olb, oub);
     }
 }
 
@@ -437,13 +498,12 @@ __global__ void __launch_bounds__(256) act_transposed(const ActArgs a) {
     __syncthreads();
     if (threadIdx.x < NPB && n0 + threadIdx.x < total) {
         const long long n = n0 + threadIdx.x;
-        Line lo, up;
-        make_lines<MODE>(s_l[threadIdx.x], s_u[threadIdx.x], lo, up);
-        s_klo[threadIdx.x] = lo.k;
-        s_kup[threadIdx.x] = up.k;
-        const float lb = a.lb[n], ub = a.ub[n];
-        a.olb[n] = line_bias(lo, lb, ub);
-        a.oub[n] = line_bias(up, ub, lb);
+        float klo, kup, olb, oub;
+        relax_any<MODE>(s_l[threadIdx.x], s_u[threadIdx.x], a.lb[n], a.ub[n], klo, kup, olb, oub);
+        s_klo[threadIdx.x] = klo;
+        s_kup[threadIdx.x] = kup;
+        a.olb[n] = olb;
+        a.oub[n] = oub;
     }
     __syncthreads();
     for (int i = 0; i < NPW; ++i) {
@@ -577,7 +637,17 @@ static int act_entry(const char *who, int mode, const float *src_lb, const float
     FAITH_ALIGNED4(l_out); FAITH_ALIGNED4(u_out);
     ActArgs a{src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw, l_out, u_out,
               length, dim_in, dim_out, words, epsilon};
-    return mode == RELU ? run<RELU>(who, a, q, layout, stream) : run<TANH>(who, a, q, layout, stream);
+    switch (mode) {
+        case RELU: return run<RELU>(who, a, q, layout, stream);
+        case TANH: return run<TANH>(who, a, q, layout, stream);
+        case EXP: return run<EXP>(who, a, q, layout, stream);
+        case RECIP: return run<RECIP>(who, a, q, layout, stream);
+        case SQR: return run<SQR>(who, a, q, layout, stream);
+        case SQRT: return run<SQRT>(who, a, q, layout, stream);
+        default:
+            faith::set_error("%s: unknown relaxation %d", who, mode);
+            return FAITH_ERR_UNSUPPORTED;
+    }
 }
 
 extern "C" int faith_relu_verification(const float *src_lb, const float *src_ub, const float *src_lw,
@@ -594,4 +664,12 @@ extern "C" int faith_tanh_verification(const float *src_lb, const float *src_ub,
                                        int dim_out, float epsilon, int q, int words, int layout, void *stream) {
     return act_entry("faith_tanh_verification", TANH, src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw,
                      out_uw, l_out, u_out, length, dim_in, dim_out, epsilon, q, words, layout, stream);
+}
+
+extern "C" int faith_unary_verification(int op, const float *src_lb, const float *src_ub, const float *src_lw,
+                                        const float *src_uw, float *out_lb, float *out_ub, float *out_lw,
+                                        float *out_uw, float *l_out, float *u_out, int length, int dim_in,
+                                        int dim_out, float epsilon, int q, int words, int layout, void *stream) {
+    return act_entry("faith_unary_verification", op, src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw,
+                     l_out, u_out, length, dim_in, dim_out, epsilon, q, words, layout, stream);
 }

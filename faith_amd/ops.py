@@ -90,6 +90,10 @@ def concretize(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL):
     return l, u
 
 
+_UNARY = {"relu": _lib.OP_RELU, "tanh": _lib.OP_TANH, "exp": _lib.OP_EXP, "reciprocal": _lib.OP_RECIPROCAL,
+          "sqr": _lib.OP_SQR, "sqrt": _lib.OP_SQRT}
+
+
 def _activation(entry, lw, lb, uw, ub, p, eps, words, layout, return_interval, out=None):
     B, L, D, H = _wb_shapes(lw, lb, layout)
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
@@ -103,8 +107,13 @@ def _activation(entry, lw, lb, uw, ub, p, eps, words, layout, return_interval, o
     l = torch.empty_like(lb) if return_interval else None
     u = torch.empty_like(ub) if return_interval else None
     with _on(lw.device):
-        _lib.call(entry, _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
-                  _ptr(l), _ptr(u), B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
+        if entry in _UNARY:
+            _lib.call("faith_unary_verification", _UNARY[entry], _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb),
+                      _ptr(oub), _ptr(olw), _ptr(ouw), _ptr(l), _ptr(u), B * L, D, H, float(eps), q_code(p),
+                      int(words), layout, _stream(lw))
+        else:
+            _lib.call(entry, _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
+                      _ptr(l), _ptr(u), B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
     if return_interval:
         return olw, olb, ouw, oub, l, u
     return olw, olb, ouw, oub
@@ -118,6 +127,26 @@ def relu(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval
 def tanh(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
     """tanh relaxation; returns (lw', lb', uw', ub'[, l, u])."""
     return _activation("faith_tanh_verification", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
+
+
+def exp(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
+    """exp relaxation (tangent below, chord above, capped at 12 as in the reference)."""
+    return _activation("exp", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
+
+
+def reciprocal(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
+    """1/x relaxation; the concrete lower bound must be positive."""
+    return _activation("reciprocal", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
+
+
+def sqr(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
+    """x^2 relaxation."""
+    return _activation("sqr", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
+
+
+def sqrt(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval=False, out=None):
+    """sqrt relaxation; the concrete lower bound must be positive."""
+    return _activation("sqrt", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
 
 
 def linear(lw, lb, uw, ub, weight, bias=None, out=None):

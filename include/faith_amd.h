@@ -99,6 +99,27 @@ int faith_tanh_verification(const float *src_lb, const float *src_ub,
                             int q, int words, int layout, void *stream);
 
 /*
+ * Any unary relaxation, selected by `op`; same arguments as the two entries above.  The reference
+ * has no CUDA entry for the last four: they replace the PyTorch methods Bounds.exp
+ * (Bounds.py:970-1003), Bounds.reciprocal (:1136-1161), Bounds.sqr (:860-890) and Bounds.sqrt
+ * (:892-919).  reciprocal and sqrt need strictly positive intervals (the reference asserts it);
+ * here the caller checks l_out if it needs the guarantee.
+ */
+#define FAITH_OP_RELU        1
+#define FAITH_OP_TANH        2
+#define FAITH_OP_EXP         3
+#define FAITH_OP_RECIPROCAL  4
+#define FAITH_OP_SQR         5
+#define FAITH_OP_SQRT        6
+int faith_unary_verification(int op,
+                             const float *src_lb, const float *src_ub,
+                             const float *src_lw, const float *src_uw,
+                             float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                             float *l_out, float *u_out,
+                             int length, int dim_in, int dim_out, float epsilon,
+                             int q, int words, int layout, void *stream);
+
+/*
  * Sign-split affine propagation  y = x @ W^T (+ bias).  Replaces the (commented-out)
  * call_matmul_verification (kernel.cpp:37-43, matmul_verification.cu:787-815) with the
  * arithmetic of Bounds.ori_matmul + add (Bounds.py:397-413, :383-395).

@@ -25,6 +25,9 @@ Parity status of each function (what pins it, see tests/test_oracle_*.py):
                soundness.  The bisection update order is pinned by text only
                (Bounds.py:1063-1097 cannot be imported: the module needs tvm
                and nvcc at import time).
+  exp, reciprocal, sqr, sqrt
+               pinned: independent fp64 per-neuron closed forms, sampled soundness
+               (lower line <= f <= upper line on [l, u]).
   dot_product  pinned: brute-force five-deep loop on tiny shapes, einsum
                restatement, sampled soundness of the McCormick planes.
   context      the same function on transposed views; pinned by the brute-force loop
@@ -215,6 +218,72 @@ def tanh(x: LinearBounds, p: float, eps: float, words: int = 1, iters: int = 10)
         d = (d + right) / 2 * (1 - go) + (d + left) / 2 * go
     k = (torch.tanh(d) - torch.tanh(lo)) / (d - lo + EPSILON)
     _add_line(x, is_both, out.uw, out.ub, "upper", k, d, torch.tanh(d))
+    return out
+
+
+# --------------------------------------------------------------------------
+# further unary relaxations on the same skeleton
+# --------------------------------------------------------------------------
+EXP_THRESHOLD = 12.0   # Bounds.py:984
+
+
+def _exp_capped(v):
+    """exp below the threshold, its tangent at the threshold above it (Bounds.py:986-989)."""
+    thres = torch.tensor(EXP_THRESHOLD)
+    below = torch.lt(v, thres).to(torch.float32)
+    return below * torch.exp(torch.min(v, thres)) + (1 - below) * (torch.exp(thres) * (v - thres + 1))
+
+
+def exp(x: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.exp (Bounds.py:970-1003): tangent below (at min(mid, l + 0.99)), chord above."""
+    lo, hi = concretize(x, p, eps, words)
+    thres = torch.tensor(EXP_THRESHOLD)
+    m = torch.min((lo + hi) / 2, lo + 0.99)
+    kl = torch.exp(torch.min(m, thres))
+    lw = x.lw * kl.unsqueeze(2)
+    lb = kl * (x.lb - m + 1)
+    ku = (_exp_capped(hi) - _exp_capped(lo)) / (hi - lo + EPSILON)
+    uw = x.uw * ku.unsqueeze(2)
+    ub = x.ub * ku - ku * lo + _exp_capped(lo)
+    return LinearBounds(lw, lb, uw, ub)
+
+
+def reciprocal(x: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.reciprocal (Bounds.py:1136-1161); needs l >= 1e-12 everywhere."""
+    lo, hi = concretize(x, p, eps, words)
+    assert torch.min(lo) >= EPSILON
+    m = (lo + hi) / 2
+    kl = -1 / m.pow(2)
+    lw = x.uw * kl.unsqueeze(2)
+    lb = x.ub * kl + 2 / m
+    ku = -1.0 / (lo * hi)
+    uw = x.lw * ku.unsqueeze(2)
+    ub = x.lb * ku - ku * lo + 1 / lo
+    return LinearBounds(lw, lb, uw, ub)
+
+
+def sqr(x: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.sqr (Bounds.py:860-890): chord above; tangent below for one-signed neurons, zero
+    for straddling ones."""
+    lo, hi, is_pos, is_neg, _is_both, out = _fresh(x, p, eps, words)
+    _add_line(x, torch.ones_like(lo), out.uw, out.ub, "upper", hi + lo, lo, lo.pow(2))
+    m = torch.max((lo + hi) / 2, 2 * hi)
+    _add_line(x, is_neg, out.lw, out.lb, "lower", 2 * m, m, m.pow(2))
+    m = torch.min((lo + hi) / 2, 2 * lo)
+    _add_line(x, is_pos, out.lw, out.lb, "lower", 2 * m, m, m.pow(2))
+    return out
+
+
+def sqrt(x: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.sqrt (Bounds.py:892-919): chord below, tangent at the midpoint above; needs l > 0."""
+    lo, hi, _p, _n, _b, out = _fresh(x, p, eps, words)
+    assert torch.min(lo) > 0
+    one = torch.ones_like(lo)
+    k = (torch.sqrt(hi) - torch.sqrt(lo)) / (hi - lo + EPSILON)
+    _add_line(x, one, out.lw, out.lb, "lower", k, lo, torch.sqrt(lo))
+    m = (lo + hi) / 2
+    k = 0.5 / torch.sqrt(m)
+    _add_line(x, one, out.uw, out.ub, "upper", k, m, torch.sqrt(m))
     return out
 
 

@@ -118,6 +118,81 @@ def tanh_neuron(lw_col, lb, uw_col, ub, p, eps, words=1, iters=10):
     return lines_applied(*tanh_lines(lo, hi, iters), lw_col, lb, uw_col, ub)
 
 
+def _exp_capped(v, thres=12.0):
+    return math.exp(v) if v < thres else math.exp(thres) * (v - thres + 1.0)
+
+
+def exp_neuron(lw_col, lb, uw_col, ub, p, eps, words=1):
+    return exp_outputs(*interval(lw_col, lb, uw_col, ub, p, eps, words), lw_col, lb, uw_col, ub)
+
+
+def exp_outputs(lo, hi, lw_col, lb, uw_col, ub):
+    """Bounds.py:970-1003.  Lower: tangent of exp at m = min(mid, lo + 0.99); upper: chord."""
+    m = min(0.5 * (lo + hi), lo + 0.99)
+    kl = math.exp(min(m, 12.0))
+    ku = (_exp_capped(hi) - _exp_capped(lo)) / (hi - lo + TINY)
+    lw = np.asarray(lw_col, float) * kl
+    uw = np.asarray(uw_col, float) * ku
+    return lw, kl * (float(lb) - m + 1.0), uw, float(ub) * ku - ku * lo + _exp_capped(lo)
+
+
+def reciprocal_neuron(lw_col, lb, uw_col, ub, p, eps, words=1):
+    return reciprocal_outputs(*interval(lw_col, lb, uw_col, ub, p, eps, words), lw_col, lb, uw_col, ub)
+
+
+def reciprocal_outputs(lo, hi, lw_col, lb, uw_col, ub):
+    """Bounds.py:1136-1161 for a positive interval.  1/x is convex and decreasing: the tangent at
+    the midpoint bounds it from below and takes the UPPER input bound (negative slope), the chord
+    bounds it from above and takes the LOWER input bound."""
+    m = 0.5 * (lo + hi)
+    kl = -1.0 / (m * m)
+    ku = -1.0 / (lo * hi)
+    return (np.asarray(uw_col, float) * kl, float(ub) * kl + 2.0 / m,
+            np.asarray(lw_col, float) * ku, float(lb) * ku - ku * lo + 1.0 / lo)
+
+
+def sqr_lines(lo, hi):
+    """Bounds.py:860-890: (lower, upper) lines of x^2 on [lo, hi]."""
+    upper = (hi + lo, lo, lo * lo)                       # chord through (lo, lo^2), (hi, hi^2)
+    if hi < 0:
+        m = max(0.5 * (lo + hi), 2 * hi)
+        lower = (2 * m, m, m * m)
+    elif lo > 0:
+        m = min(0.5 * (lo + hi), 2 * lo)
+        lower = (2 * m, m, m * m)
+    else:
+        lower = (0.0, 0.0, 0.0)
+    return lower, upper
+
+
+def sqrt_lines(lo, hi):
+    """Bounds.py:892-919: chord below, tangent at the midpoint above."""
+    m = 0.5 * (lo + hi)
+    lower = ((math.sqrt(hi) - math.sqrt(lo)) / (hi - lo + TINY), lo, math.sqrt(lo))
+    upper = (0.5 / math.sqrt(m), m, math.sqrt(m))
+    return lower, upper
+
+
+def sqr_neuron(lw_col, lb, uw_col, ub, p, eps, words=1):
+    lo, hi = interval(lw_col, lb, uw_col, ub, p, eps, words)
+    return lines_applied(*sqr_lines(lo, hi), lw_col, lb, uw_col, ub)
+
+
+def sqrt_neuron(lw_col, lb, uw_col, ub, p, eps, words=1):
+    lo, hi = interval(lw_col, lb, uw_col, ub, p, eps, words)
+    return lines_applied(*sqrt_lines(lo, hi), lw_col, lb, uw_col, ub)
+
+
+def outputs_from_interval(kind, lo, hi, lw_col, lb, uw_col, ub):
+    """(lw', lb', uw', ub') of one neuron of relaxation `kind`, given its concrete interval."""
+    if kind == "exp":
+        return exp_outputs(lo, hi, lw_col, lb, uw_col, ub)
+    if kind == "reciprocal":
+        return reciprocal_outputs(lo, hi, lw_col, lb, uw_col, ub)
+    lines = {"relu": relu_lines, "tanh": tanh_lines, "sqr": sqr_lines, "sqrt": sqrt_lines}[kind]
+    return lines_applied(*lines(lo, hi), lw_col, lb, uw_col, ub)
+
+
 def linear_brute(lw, lb, uw, ub, W, bias=None):
     """Triple-loop sign-split affine map; arrays [L, D, H], [L, H], W [N, H]."""
     L, D, H = lw.shape

@@ -378,3 +378,58 @@ def test_context_vs_brute_force(p):
                         y[0], yb[0], y[1], yb[1], p, 0.2, 1)
         for got, exp in zip((z.lw, z.lb, z.uw, z.ub), e):
             np.testing.assert_allclose(f64(got)[t], exp, rtol=1e-5, atol=2e-6)
+
+
+# ------------------------------------------------- exp / reciprocal / sqr / sqrt
+def _unary_input(kind, g, ordered=True):
+    x = rand_bounds(g, 1, 3, 8, 24, ordered=ordered, sw=0.1, sb=1.5, gap_w=0.02, gap_b=0.5)
+    if kind in ("reciprocal", "sqrt"):          # strictly positive pre-activations
+        x = O.LinearBounds(x.lw, x.lb.abs() + 1.0, x.uw, x.lb.abs() + 1.0 + (x.ub - x.lb))
+    return x
+
+
+@pytest.mark.parametrize("kind", ["exp", "reciprocal", "sqr", "sqrt"])
+@pytest.mark.parametrize("p", PS)
+@pytest.mark.parametrize("words", [1, 2])
+def test_unary_vs_per_neuron_closed_form(kind, p, words):
+    x = _unary_input(kind, gen(22))
+    y = getattr(O, kind)(x, p, 0.2, words)
+    fn = getattr(C, kind + "_neuron")
+    lw, lb, uw, ub = (f64(t)[0] for t in x.tensors())
+    for l in range(3):
+        for j in range(24):
+            e = fn(lw[l, :, j], lb[l, j], uw[l, :, j], ub[l, j], p, 0.2, words)
+            tol = dict(rtol=2e-5, atol=1e-5)
+            np.testing.assert_allclose(f64(y.lw)[0, l, :, j], e[0], **tol)
+            np.testing.assert_allclose(f64(y.lb)[0, l, j], e[1], **tol)
+            np.testing.assert_allclose(f64(y.uw)[0, l, :, j], e[2], **tol)
+            np.testing.assert_allclose(f64(y.ub)[0, l, j], e[3], **tol)
+
+
+@pytest.mark.parametrize("kind", ["exp", "reciprocal", "sqr", "sqrt"])
+@pytest.mark.parametrize("p", PS)
+def test_unary_soundness(kind, p):
+    g = gen(23)
+    x = _unary_input(kind, g)
+    x.ub += 0.1
+    eps = 0.3
+    y = getattr(O, kind)(x, p, eps, 1)
+    fn = {"exp": torch.exp, "reciprocal": torch.reciprocal, "sqr": torch.square, "sqrt": torch.sqrt}[kind]
+    delta = _sample_delta(g, 8, p, eps, 300)
+    lo_in, hi_in = _eval(x.lw[0], x.lb[0], delta), _eval(x.uw[0], x.ub[0], delta)
+    lo_out, hi_out = _eval(y.lw[0], y.lb[0], delta), _eval(y.uw[0], y.ub[0], delta)
+    for t in (0.0, 0.4, 1.0):
+        v = fn(lo_in + t * (hi_in - lo_in))
+        assert (v >= lo_out - 1e-5 * (1 + v.abs())).all()
+        assert (v <= hi_out + 1e-5 * (1 + v.abs())).all()
+
+
+def test_exp_saturates_above_threshold():
+    """Above 12 the reference switches exp to its tangent (Bounds.py:984-989)."""
+    lw = torch.zeros(1, 1, 2, 3); lb = torch.tensor([[[11.0, 12.5, 20.0]]]); ub = lb + 1.0
+    y = O.exp(O.LinearBounds(lw, lb, lw, ub), 2.0, 0.1)
+    e12 = math.exp(12.0)
+    for j, (lo, hi) in enumerate([(11.0, 12.0), (12.5, 13.5), (20.0, 21.0)]):
+        cap = lambda v: math.exp(v) if v < 12 else e12 * (v - 11.0)
+        ku = (cap(hi) - cap(lo)) / (hi - lo)
+        assert abs(y.ub[0, 0, j].item() - (hi * ku - ku * lo + cap(lo))) / cap(hi) < 1e-5
