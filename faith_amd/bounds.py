@@ -8,6 +8,7 @@ the methods on the accelerated path:
     matmul       :1177-1199 (ori_matmul :397-413)     tanh        :1171-1175 (ori_tanh :1027-1103)
     dense        :1016-1025               dot_product :833-841 (ori_dot_product :710-823)
     t / context  :335-346, :843-850       exp / sqr / sqrt / reciprocal  :970-1003, :860-919, :1136-1161
+    multiply / divide / softmax / layer_norm  :594-664, :825-830, :1005-1014, :1111-1131
     add          :383-395                 conv2d      HandTunedKernels/convolution_verification.cu:219-239
 
 Every method launches hand-written HIP kernels through the C ABI; none has a
@@ -55,8 +56,43 @@ class Bounds:
     # ---- Bounds.py:383-395
     def add(self, delta):
         if isinstance(delta, Bounds):
-            return self._like(self.lw + delta.lw, self.lb + delta.lb, self.uw + delta.uw, self.ub + delta.ub)
-        return self._like(self.lw, self.lb + delta, self.uw, self.ub + delta)
+            return self._like(*ops.add(self._c(), delta._c()))
+        lb, ub = ops.shift(self.lb.contiguous(), self.ub.contiguous(), delta)
+        return self._like(self.lw, lb, self.uw, ub)
+
+    # ---- Bounds.py:594-664: by a float, by a per-neuron tensor, or by another bound object
+    def multiply(self, W):
+        if isinstance(W, Bounds):
+            return self._like(*ops.multiply(self._c(), W._c(), self.p, self.eps, self.perturbed_words))
+        return self._like(*ops.scale(*self._c(), W))
+
+    # ---- Bounds.py:825-830
+    def divide(self, W):
+        if not isinstance(W, Bounds):
+            raise NotImplementedError
+        return self.multiply(W.reciprocal())
+
+    # ---- Bounds.py:1005-1014
+    def softmax(self):
+        e = self.exp()
+        total = self._like(ops.rowsum_broadcast(e.lw), ops.rowsum_broadcast(e.lb),
+                           ops.rowsum_broadcast(e.uw), ops.rowsum_broadcast(e.ub))
+        return e.divide(total)
+
+    # ---- Bounds.py:1111-1131
+    def layer_norm(self, normalizer, layer_norm):
+        if layer_norm == "no":
+            return self
+        H = self.dim_out
+        w_avg = torch.full((H, H), 1.0 / H, device=self.device, dtype=torch.float32)
+        minus_mu = self.add(self.matmul(w_avg).multiply(-1.0))
+        if layer_norm == "standard":
+            variance = minus_mu.sqr().matmul(w_avg)
+            normalized = minus_mu.divide(variance.add(1e-12).sqrt())
+        else:
+            assert layer_norm == "no_var"
+            normalized = minus_mu
+        return normalized.multiply(normalizer.weight.detach().contiguous()).add(normalizer.bias.detach().contiguous())
 
     # ---- Bounds.py:397-413, :1177-1199
     def matmul(self, W, bias=None):

@@ -28,6 +28,7 @@ COMMON = [
 EXTRA = {
     # the relaxations round (b - x0) * k and + y0 separately, as the PyTorch path does
     "act.hip": ["-ffp-contract=off"],
+    "mul.hip": ["-ffp-contract=off"],
 }
 
 

@@ -20,12 +20,9 @@
 //
 // This file is built with -ffp-contract=off: the reference rounds (b - x0) * k and the
 // following + y0 separately, and l = lb + (-eps * norm) likewise.
-#include "common.h"
+#include "relax_common.h"
 
 namespace {
-
-constexpr int WAVE = 64;
-constexpr float TINY = 1e-12f;   // Bounds.py:27
 
 enum Mode { CONCRETIZE = 0, RELU = FAITH_OP_RELU, TANH = FAITH_OP_TANH, EXP = FAITH_OP_EXP, RECIP = FAITH_OP_RECIPROCAL,
             SQR = FAITH_OP_SQR, SQRT = FAITH_OP_SQRT };
@@ -46,22 +43,6 @@ struct ActArgs {
 struct Line {
     float k, x0, y0;
 };
-
-// ------------------------------------------------------------------ q-norm pieces
-template <int Q>
-__device__ __forceinline__ float nacc(float acc, float v) {
-    if (Q == FAITH_Q_2) return acc + v * v;
-    if (Q == FAITH_Q_1) return acc + fabsf(v);
-    return fmaxf(acc, fabsf(v));
-}
-template <int Q>
-__device__ __forceinline__ float ncomb(float a, float b) {
-    return Q == FAITH_Q_INF ? fmaxf(a, b) : a + b;
-}
-template <int Q>
-__device__ __forceinline__ float nfin(float a) {
-    return Q == FAITH_Q_2 ? sqrtf(a) : a;
-}
 
 // ------------------------------------------------------------------ the relaxations
 // Bounds.py:921-963.  Strict comparisons: l == 0 or u == 0 is a straddling neuron.
@@ -137,40 +118,6 @@ __device__ __forceinline__ void relax_point(float l, float u, float lb, float ub
         oub = line_bias(up, ub, lb);
     }
 }
-
-// ------------------------------------------------------------------ vector access
-// Stores are non-temporal: lw' / uw' are written once and not read again by this kernel, and
-// keeping them out of the cache's way measured 11 % faster at configuration 1 (loads are left
-// temporal: marking them non-temporal measured 15 % slower).
-typedef float v4f __attribute__((ext_vector_type(4)));
-template <int VEC>
-struct Vec;
-template <>
-struct Vec<4> {
-    float4 v;
-    __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
-    __device__ __forceinline__ void store(float *p) const {
-        const v4f t = {v.x, v.y, v.z, v.w};
-        __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
-    }
-    __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
-    __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
-    __device__ __forceinline__ void set(int i, float f) {
-        if (i == 0) v.x = f;
-        else if (i == 1) v.y = f;
-        else if (i == 2) v.z = f;
-        else v.w = f;
-    }
-};
-template <>
-struct Vec<1> {
-    float v;
-    __device__ __forceinline__ void load(const float *p) { v = *p; }
-    __device__ __forceinline__ void store(float *p) const { __builtin_nontemporal_store(v, p); }
-    __device__ __forceinline__ void zero() { v = 0.f; }
-    __device__ __forceinline__ float get(int) const { return v; }
-    __device__ __forceinline__ void set(int, float f) { v = f; }
-};
 
 // ------------------------------------------------------------------ natural layout
 // exp-based pieces for the tanh lines, all in double: with t = exp(2x),

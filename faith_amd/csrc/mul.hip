@@ -1,0 +1,291 @@
+// Elementwise operations on bound objects: product of two bounded quantities (McCormick planes),
+// per-column scaling, sum of two objects, and the row sum that softmax needs.  All HBM bound.
+//
+// Arithmetic of the reference's PyTorch methods: Bounds.multiply (Bounds.py:594-664) with
+// get_bounds_xy (:666-688), Bounds.add (:383-395), and the sum / repeat of Bounds.softmax
+// (:1005-1014).  The reference has no CUDA kernels for these.
+//
+// Product of two objects x, y of one shape [rows, D_in, H]: with the concrete intervals
+// [l_x, u_x], [l_y, u_y] the planes are  a_l = l_y, a_u = u_y, b = l_x  (b on both sides, as the
+// reference has it) and
+//   z_lw = (a_l > 0 ? x.lw : x.uw) a_l + (b > 0 ? y.lw : y.uw) b
+//   z_uw = (a_u > 0 ? x.uw : x.lw) a_u + (b > 0 ? y.uw : y.lw) b
+//   z_lb = ((a_l > 0 ? x.lb : x.ub) a_l - a_l b) + (b > 0 ? y.lb : y.ub) b          (z_ub alike)
+// The kernel has the shape of the relaxation kernels: a workgroup owns (row, 32 neurons), the
+// D_in rows of the tile of ALL FOUR coefficient tensors stay in registers between the two norm
+// reductions and the combination, so every input is read once: 24 bytes per coefficient element.
+//
+// Built with -ffp-contract=off (the reference rounds every product and sum separately).
+#include "relax_common.h"
+
+namespace {
+
+struct MulArgs {
+    const float *xlb, *xub, *xlw, *xuw;
+    const float *ylb, *yub, *ylw, *yuw;
+    float *zlb, *zub, *zlw, *zuw;
+    int rows, D, H, words;
+    float eps;
+};
+
+template <int Q, int VEC, int TPR, int NTHREADS, int RPT>
+__global__ void __launch_bounds__(NTHREADS) mul_natural(const MulArgs a) {
+    constexpr int TH = TPR * VEC;
+    constexpr int RG = NTHREADS / TPR;
+    constexpr int NW = NTHREADS / WAVE;
+    static_assert(TH <= WAVE, "one lane per neuron in wavefront 0");
+    extern __shared__ float smem[];
+    float *part = smem;                          // [words][NW][4][TH]: x.lw, x.uw, y.lw, y.uw partial norms
+    float *coef = part + a.words * NW * 4 * TH;  // [3][TH]: a_l, a_u, b
+
+    const int tiles = (a.H + TH - 1) / TH;
+    const int r = blockIdx.x / tiles;
+    const int col0 = (blockIdx.x % tiles) * TH;
+    const int tid = threadIdx.x;
+    const int lane = tid % WAVE, wv = tid / WAVE;
+    const int c = tid % TPR, rg = tid / TPR;
+    const int col = col0 + c * VEC;
+    const bool col_ok = col < a.H;
+    const size_t base = (size_t)r * a.D * a.H + col;
+    const int blk = a.D / a.words;
+    constexpr int CHUNK = RG * RPT;
+    const int nchunks = (a.D + CHUNK - 1) / CHUNK;
+    const float *src[4] = {a.xlw, a.xuw, a.ylw, a.yuw};
+
+    Vec<VEC> d[4][RPT];
+
+    if (nchunks > 1 && lane < TPR)
+        for (int w = 0; w < a.words; ++w)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) part[((w * NW + wv) * 4 + t) * TH + c * VEC + v] = 0.f;
+
+    for (int ch = 0; ch < nchunks; ++ch) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            const int row = ch * CHUNK + i * RG + rg;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                if (col_ok && row < a.D)
+                    d[t][i].load(src[t] + base + (size_t)row * a.H);
+                else
+                    d[t][i].zero();
+            }
+        }
+        for (int w = 0; w < a.words; ++w) {
+            const int lo_row = w * blk, hi_row = lo_row + blk;
+            float pn[4][VEC];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) pn[t][v] = 0.f;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                const int row = ch * CHUNK + i * RG + rg;
+                if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v));
+                }
+            }
+#pragma unroll
+            for (int m = TPR; m < WAVE; m <<= 1)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) pn[t][v] = ncomb<Q>(pn[t][v], __shfl_xor(pn[t][v], m, WAVE));
+            if (lane < TPR) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        float *sl = &part[((w * NW + wv) * 4 + t) * TH + c * VEC + v];
+                        *sl = nchunks > 1 ? ncomb<Q>(*sl, pn[t][v]) : pn[t][v];
+                    }
+            }
+        }
+    }
+    __syncthreads();
+
+    // one lane per neuron: both concretizations (Bounds.py:611-612), planes, constant terms
+    const int column = col0 + lane;
+    if (wv == 0 && lane < TH && column < a.H) {
+        const size_t bi = (size_t)r * a.H + column;
+        const float xlb = a.xlb[bi], xub = a.xub[bi], ylb = a.ylb[bi], yub = a.yub[bi];
+        float lx = xlb, ly = ylb, uy = yub;
+        for (int w = 0; w < a.words; ++w) {
+            float n[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int g = 0; g < NW; ++g)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) n[t] = ncomb<Q>(n[t], part[((w * NW + g) * 4 + t) * TH + lane]);
+            lx += (-a.eps) * nfin<Q>(n[0]);
+            ly += (-a.eps) * nfin<Q>(n[2]);
+            uy += a.eps * nfin<Q>(n[3]);
+        }
+        const float al = ly, au = uy, bt = lx;
+        coef[lane] = al;
+        coef[TH + lane] = au;
+        coef[2 * TH + lane] = bt;
+        // Bounds.py:631-646: ((b_src - 0) * k + gamma) then + ((b_src - 0) * k + 0)
+        const float gl = -al * bt, gu = -au * bt;
+        a.zlb[bi] = ((al > 0.f ? xlb : xub) * al + gl) + (bt > 0.f ? ylb : yub) * bt;
+        a.zub[bi] = ((au > 0.f ? xub : xlb) * au + gu) + (bt > 0.f ? yub : ylb) * bt;
+    }
+    __syncthreads();
+
+    if (!col_ok) return;
+    float al[VEC], au[VEC], bt[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        al[v] = coef[c * VEC + v];
+        au[v] = coef[TH + c * VEC + v];
+        bt[v] = coef[2 * TH + c * VEC + v];
+    }
+    for (int ch = 0; ch < nchunks; ++ch) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            const int row = ch * CHUNK + i * RG + rg;
+            if (row < a.D) {
+                const size_t off = base + (size_t)row * a.H;
+                if (nchunks > 1) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) d[t][i].load(src[t] + off);
+                }
+                Vec<VEC> ol, ou;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    const float xl = d[0][i].get(v), xu = d[1][i].get(v), yl = d[2][i].get(v), yu = d[3][i].get(v);
+                    ol.set(v, (al[v] > 0.f ? xl : xu) * al[v] + (bt[v] > 0.f ? yl : yu) * bt[v]);
+                    ou.set(v, (au[v] > 0.f ? xu : xl) * au[v] + (bt[v] > 0.f ? yu : yl) * bt[v]);
+                }
+                ol.store(a.zlw + off);
+                ou.store(a.zuw + off);
+            }
+        }
+    }
+}
+
+template <int Q, int VEC, int TPR, int NTHREADS, int RPT>
+void launch_mul(const MulArgs &a, hipStream_t st) {
+    constexpr int TH = TPR * VEC;
+    const int tiles = (a.H + TH - 1) / TH;
+    const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 4 * TH + 3 * TH) * sizeof(float);
+    hipLaunchKernelGGL((mul_natural<Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles)), dim3(NTHREADS), smem,
+                       st, a);
+}
+
+template <int Q>
+void dispatch_mul(const MulArgs &a, hipStream_t st) {
+    const bool vec4 = a.H % 4 == 0 && faith::aligned(a.xlw, 16) && faith::aligned(a.xuw, 16) &&
+                      faith::aligned(a.ylw, 16) && faith::aligned(a.yuw, 16) && faith::aligned(a.zlw, 16) &&
+                      faith::aligned(a.zuw, 16);
+    if (!vec4)
+        launch_mul<Q, 1, 64, 256, 8>(a, st);      // 64 neurons x 32 rows per pass
+    else if (a.D <= 128)
+        launch_mul<Q, 4, 8, 256, 4>(a, st);       // 32 neurons, D_in <= 128 in registers (64 values per thread)
+    else
+        launch_mul<Q, 4, 8, 256, 8>(a, st);       // D_in <= 256 in registers (128 values per thread), passes beyond
+}
+
+// ------------------------------------------------------------------ plain elementwise kernels
+// out = a * s+ + a' * s-  per column (Bounds.multiply with a float or a tensor, Bounds.py:595-607, :653-664),
+// optionally followed by + b (Bounds.add, :383-395).  inner = elements per scale entry cycle:
+// element e uses scale[(e % H)].
+__global__ void __launch_bounds__(256) scale_add_kernel(const float *__restrict__ lo, const float *__restrict__ up,
+                                                        const float *__restrict__ scale, float scalar,
+                                                        const float *__restrict__ add_lo,
+                                                        const float *__restrict__ add_up,
+                                                        const float *__restrict__ shift, float *__restrict__ out_lo,
+                                                        float *__restrict__ out_up, size_t n, int H) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+        float l = lo[e], u = up[e];
+        if (scale || scalar != 1.f) {
+            const float s = scale ? scale[e % H] : scalar;
+            const float sp = s > 0.f ? s : 0.f * s;      // W * (W > 0): zero keeps the sign rule of the product
+            const float sn = s - sp;
+            const float nl = l * sp + u * sn, nu = l * sn + u * sp;
+            l = nl;
+            u = nu;
+        }
+        if (add_lo) {
+            l += add_lo[e];
+            u += add_up[e];
+        }
+        if (shift) {
+            const float t = shift[e % H];
+            l += t;
+            u += t;
+        }
+        out_lo[e] = l;
+        out_up[e] = u;
+    }
+}
+
+// dst[r, :] = sum_h src[r, h] for every h (torch.sum(dim=-1, keepdim=True).repeat, Bounds.py:1009-1012):
+// a wavefront per row, cross-lane butterfly, broadcast store.
+__global__ void __launch_bounds__(256) rowsum_broadcast_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                               long long rows, int H) {
+    const long long r = (long long)blockIdx.x * 4 + threadIdx.x / WAVE;
+    if (r >= rows) return;
+    const int lane = threadIdx.x % WAVE;
+    const float *p = src + (size_t)r * H;
+    float s = 0.f;
+    for (int h = lane; h < H; h += WAVE) s += p[h];
+#pragma unroll
+    for (int m = WAVE / 2; m > 0; m >>= 1) s += __shfl_xor(s, m, WAVE);
+    float *q = dst + (size_t)r * H;
+    for (int h = lane; h < H; h += WAVE) q[h] = s;
+}
+
+}  // namespace
+
+extern "C" int faith_multiply_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
+                                           const float *y_lb, const float *y_ub, const float *y_lw, const float *y_uw,
+                                           float *z_lb, float *z_ub, float *z_lw, float *z_uw, int length, int dim_in,
+                                           int dim_out, float epsilon, int q, int words, void *stream) {
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw);
+    FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
+    FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_ALIGNED4(z_lw); FAITH_ALIGNED4(z_uw);
+    FAITH_REQUIRE(length > 0 && dim_in > 0 && dim_out > 0, FAITH_ERR_SHAPE,
+                  "faith_multiply_verification: length=%d dim_in=%d dim_out=%d must be positive", length, dim_in, dim_out);
+    FAITH_REQUIRE(words >= 1 && words <= 16 && dim_in % words == 0, FAITH_ERR_SHAPE,
+                  "faith_multiply_verification: words=%d must be in 1..16 and divide dim_in=%d", words, dim_in);
+    FAITH_REQUIRE(q == FAITH_Q_1 || q == FAITH_Q_2 || q == FAITH_Q_INF, FAITH_ERR_UNSUPPORTED,
+                  "faith_multiply_verification: q=%d is not one of FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF", q);
+    MulArgs a{x_lb, x_ub, x_lw, x_uw, y_lb, y_ub, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, length, dim_in, dim_out, words,
+              epsilon};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (q == FAITH_Q_1) dispatch_mul<FAITH_Q_1>(a, st);
+    else if (q == FAITH_Q_2) dispatch_mul<FAITH_Q_2>(a, st);
+    else dispatch_mul<FAITH_Q_INF>(a, st);
+    return faith::check_launch("faith_multiply_verification");
+}
+
+extern "C" int faith_scale_add(const float *lo, const float *up, const float *scale, float scalar,
+                               const float *add_lo, const float *add_up, const float *shift, float *out_lo,
+                               float *out_up, long long n, int period, void *stream) {
+    FAITH_NOT_NULL(lo); FAITH_NOT_NULL(up); FAITH_NOT_NULL(out_lo); FAITH_NOT_NULL(out_up);
+    FAITH_REQUIRE(n > 0 && period > 0, FAITH_ERR_SHAPE, "faith_scale_add: n=%lld period=%d must be positive", n, period);
+    FAITH_REQUIRE((add_lo == nullptr) == (add_up == nullptr), FAITH_ERR_NULL,
+                  "faith_scale_add: add_lo and add_up must be given together");
+    const long long blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(scale_add_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), lo, up, scale, scalar, add_lo, add_up, shift, out_lo, out_up,
+                       (size_t)n, period);
+    return faith::check_launch("faith_scale_add");
+}
+
+extern "C" int faith_rowsum_broadcast(const float *src, float *dst, long long rows, int dim_out, void *stream) {
+    FAITH_NOT_NULL(src); FAITH_NOT_NULL(dst);
+    FAITH_REQUIRE(rows > 0 && dim_out > 0 && (rows + 3) / 4 <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "faith_rowsum_broadcast: rows=%lld dim_out=%d out of range", rows, dim_out);
+    hipLaunchKernelGGL(rowsum_broadcast_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), src, dst, rows, dim_out);
+    return faith::check_launch("faith_rowsum_broadcast");
+}

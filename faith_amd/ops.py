@@ -149,6 +149,83 @@ def sqrt(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL, return_interval
     return _activation("sqrt", lw, lb, uw, ub, p, eps, words, layout, return_interval, out)
 
 
+def multiply(x, y, p, eps, words=1, out=None):
+    """Product of two bound objects of one shape; x, y: (lw, lb, uw, ub)."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    B, L, D, H = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    for n, t, s_ in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                     ("y.lw", ylw, xlw.shape), ("y.uw", yuw, xlw.shape), ("y.lb", ylb, xlb.shape),
+                     ("y.ub", yub, xlb.shape)):
+        _check(n, t, s_)
+    if out is None:
+        out = (torch.empty_like(xlw), torch.empty_like(xlb), torch.empty_like(xlw), torch.empty_like(xlb))
+    zlw, zlb, zuw, zub = out
+    _check("out lw", zlw, xlw.shape); _check("out uw", zuw, xlw.shape)
+    _check("out lb", zlb, xlb.shape); _check("out ub", zub, xlb.shape)
+    with _on(xlw.device):
+        _lib.call("faith_multiply_verification", _ptr(xlb), _ptr(xub), _ptr(xlw), _ptr(xuw), _ptr(ylb), _ptr(yub),
+                  _ptr(ylw), _ptr(yuw), _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B * L, D, H, float(eps),
+                  q_code(p), int(words), _stream(xlw))
+    return zlw, zlb, zuw, zub
+
+
+def _scale_add_pair(lo, up, scale, scalar, add_lo, add_up, shift, period):
+    out_lo, out_up = torch.empty_like(lo), torch.empty_like(up)
+    with _on(lo.device):
+        _lib.call("faith_scale_add", _ptr(lo), _ptr(up), _ptr(scale), float(scalar), _ptr(add_lo), _ptr(add_up),
+                  _ptr(shift), _ptr(out_lo), _ptr(out_up), lo.numel(), int(period), _stream(lo))
+    return out_lo, out_up
+
+
+def scale(lw, lb, uw, ub, W):
+    """Bounds.multiply with a float or a per-neuron tensor W [H] (sign-split elementwise scaling)."""
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    H = lw.shape[-1]
+    if isinstance(W, torch.Tensor):
+        _check("W", W, (H,))
+        vec, scalar = W, 1.0
+    else:
+        vec, scalar = None, float(W)
+    olw, ouw = _scale_add_pair(lw, uw, vec, scalar, None, None, None, H)
+    olb, oub = _scale_add_pair(lb, ub, vec, scalar, None, None, None, H)
+    return olw, olb, ouw, oub
+
+
+def add(x, y):
+    """Bounds.add with a Bounds argument: elementwise sum of two objects."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    for n, t, s_ in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                     ("y.lw", ylw, xlw.shape), ("y.uw", yuw, xlw.shape), ("y.lb", ylb, xlb.shape),
+                     ("y.ub", yub, xlb.shape)):
+        _check(n, t, s_)
+    H = xlw.shape[-1]
+    olw, ouw = _scale_add_pair(xlw, xuw, None, 1.0, ylw, yuw, None, H)
+    olb, oub = _scale_add_pair(xlb, xub, None, 1.0, ylb, yub, None, H)
+    return olw, olb, ouw, oub
+
+
+def shift(lb, ub, delta):
+    """Bounds.add with a float or a tensor [H]: moves the constant terms only."""
+    _check("lb", lb); _check("ub", ub, lb.shape)
+    H = lb.shape[-1]
+    if not isinstance(delta, torch.Tensor):
+        delta = torch.full((H,), float(delta), device=lb.device, dtype=torch.float32)
+    _check("delta", delta, (H,))
+    return _scale_add_pair(lb, ub, None, 1.0, None, None, delta, H)
+
+
+def rowsum_broadcast(t):
+    """sum over the last axis, written to every position of that axis."""
+    _check("t", t)
+    out = torch.empty_like(t)
+    H = t.shape[-1]
+    with _on(t.device):
+        _lib.call("faith_rowsum_broadcast", _ptr(t), _ptr(out), t.numel() // H, H, _stream(t))
+    return out
+
+
 def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     """Sign-split propagation through y = x @ weight.T + bias.  weight: [H_out, H]."""
     B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)

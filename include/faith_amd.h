@@ -120,6 +120,36 @@ int faith_unary_verification(int op,
                              int q, int words, int layout, void *stream);
 
 /*
+ * Product of two bound objects of one shape (McCormick planes).  No CUDA counterpart in the
+ * reference: replaces the PyTorch method Bounds.multiply with a Bounds argument
+ * (Bounds.py:608-651, planes from get_bounds_xy :666-688); Bounds.divide (:825-830) is this after
+ * a reciprocal.  Natural layout, all twelve arrays shaped like x: [length, dim_in, dim_out] and
+ * [length, dim_out].
+ */
+int faith_multiply_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
+                                const float *y_lb, const float *y_ub, const float *y_lw, const float *y_uw,
+                                float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                                int length, int dim_in, int dim_out, float epsilon,
+                                int q, int words, void *stream);
+
+/*
+ * out_lo[e] = lo[e] * s+ + up[e] * s- (+ add_lo[e]) (+ shift[e % period]),  out_up mirrored, with
+ * s = scale[e % period] when scale is given, else `scalar`;  s+ = s * (s > 0), s- = s - s+.
+ * One kernel behind Bounds.multiply with a float or a tensor (Bounds.py:595-607, :653-664) and
+ * Bounds.add (:383-395); called once for (lw, uw) and once for (lb, ub).  scale, add_lo / add_up and
+ * shift may be NULL; out may alias the inputs.
+ */
+int faith_scale_add(const float *lo, const float *up, const float *scale, float scalar,
+                    const float *add_lo, const float *add_up, const float *shift,
+                    float *out_lo, float *out_up, long long n, int period, void *stream);
+
+/*
+ * dst[r, :] = sum over h of src[r, h], written to every h: the sum / repeat pair of Bounds.softmax
+ * (Bounds.py:1009-1012) without the intermediate.
+ */
+int faith_rowsum_broadcast(const float *src, float *dst, long long rows, int dim_out, void *stream);
+
+/*
  * Sign-split affine propagation  y = x @ W^T (+ bias).  Replaces the (commented-out)
  * call_matmul_verification (kernel.cpp:37-43, matmul_verification.cu:787-815) with the
  * arithmetic of Bounds.ori_matmul + add (Bounds.py:397-413, :383-395).

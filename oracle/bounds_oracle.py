@@ -28,6 +28,12 @@ Parity status of each function (what pins it, see tests/test_oracle_*.py):
   exp, reciprocal, sqr, sqrt
                pinned: independent fp64 per-neuron closed forms, sampled soundness
                (lower line <= f <= upper line on [l, u]).
+  scale, add   one-line tensor identities (checked against their definition).
+  multiply     pinned: the brute-force McCormick loop with a reduction of length 1.
+  divide, softmax, layer_norm
+               compositions of pinned parts, in the reference's order; pinned as wholes
+               by sampled soundness (the true softmax / layer norm of any admissible
+               input lies between the propagated lines).
   dot_product  pinned: brute-force five-deep loop on tiny shapes, einsum
                restatement, sampled soundness of the McCormick planes.
   context      the same function on transposed views; pinned by the brute-force loop
@@ -285,6 +291,75 @@ def sqrt(x: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
     k = 0.5 / torch.sqrt(m)
     _add_line(x, one, out.uw, out.ub, "upper", k, m, torch.sqrt(m))
     return out
+
+
+# --------------------------------------------------------------------------
+# elementwise algebra and the composites built from it
+# --------------------------------------------------------------------------
+def scale(x: LinearBounds, W) -> LinearBounds:
+    """Bounds.multiply with a float (Bounds.py:595-607) or a tensor [H] (:653-664)."""
+    if isinstance(W, float):
+        if W > 0:
+            return LinearBounds(x.lw * W, x.lb * W, x.uw * W, x.ub * W)
+        return LinearBounds(x.uw * W, x.ub * W, x.lw * W, x.lb * W)
+    w_pos = W * torch.gt(W, 0).to(torch.float32)
+    w_neg = W - w_pos
+    return LinearBounds(x.lw * w_pos + x.uw * w_neg, x.lb * w_pos + x.ub * w_neg,
+                        x.lw * w_neg + x.uw * w_pos, x.lb * w_neg + x.ub * w_pos)
+
+
+def add(x: LinearBounds, delta) -> LinearBounds:
+    """Bounds.add (Bounds.py:383-395)."""
+    if isinstance(delta, LinearBounds):
+        return LinearBounds(x.lw + delta.lw, x.lb + delta.lb, x.uw + delta.uw, x.ub + delta.ub)
+    return LinearBounds(x.lw, x.lb + delta, x.uw, x.ub + delta)
+
+
+def multiply(x: LinearBounds, y: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.multiply with a Bounds argument (Bounds.py:608-651): McCormick planes
+    a_l = l_y, a_u = u_y, b = l_x (both sides), pushed through x and y by sign."""
+    lx, _ux = concretize(x, p, eps, words)
+    ly, uy = concretize(y, p, eps, words)
+    out = LinearBounds(torch.zeros_like(x.lw), torch.zeros_like(x.lb), torch.zeros_like(x.uw), torch.zeros_like(x.ub))
+    every = torch.ones_like(lx)
+    _add_line(x, every, out.lw, out.lb, "lower", ly, 0, -ly * lx)
+    _add_line(y, every, out.lw, out.lb, "lower", lx, 0, 0)
+    _add_line(x, every, out.uw, out.ub, "upper", uy, 0, -uy * lx)
+    _add_line(y, every, out.uw, out.ub, "upper", lx, 0, 0)
+    return out
+
+
+def divide(x: LinearBounds, y: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.divide (Bounds.py:825-830)."""
+    return multiply(x, reciprocal(y, p, eps, words), p, eps, words)
+
+
+def softmax(x: LinearBounds, p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.softmax (Bounds.py:1005-1014): exp, then division by the (repeated) sum over H."""
+    e = exp(x, p, eps, words)
+    H = x.lw.shape[-1]
+    total = LinearBounds(torch.sum(e.lw, dim=-1, keepdim=True).repeat(1, 1, 1, H),
+                         torch.sum(e.lb, dim=-1, keepdim=True).repeat(1, 1, H),
+                         torch.sum(e.uw, dim=-1, keepdim=True).repeat(1, 1, 1, H),
+                         torch.sum(e.ub, dim=-1, keepdim=True).repeat(1, 1, H))
+    return divide(e, total, p, eps, words)
+
+
+def layer_norm(x: LinearBounds, weight: torch.Tensor, bias: torch.Tensor, mode: str,
+               p: float, eps: float, words: int = 1) -> LinearBounds:
+    """Bounds.layer_norm (Bounds.py:1111-1131); mode in {"no", "no_var", "standard"}."""
+    if mode == "no":
+        return x
+    H = x.lw.shape[-1]
+    w_avg = torch.ones(H, H) * (1.0 / H)
+    minus_mu = add(x, scale(linear(x, w_avg), -1.0))
+    if mode == "standard":
+        variance = linear(sqr(minus_mu, p, eps, words), w_avg)
+        normalized = divide(minus_mu, sqrt(add(variance, EPSILON), p, eps, words), p, eps, words)
+    else:
+        assert mode == "no_var"
+        normalized = minus_mu
+    return add(scale(normalized, weight), bias)
 
 
 # --------------------------------------------------------------------------

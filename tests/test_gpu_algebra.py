@@ -1,0 +1,103 @@
+"""HIP elementwise algebra (multiply / divide / scale / add) and the composites built from it
+(softmax, layer_norm) against the CPU oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import bounds_oracle as O
+from tests.helpers import rand_bounds, close, worst
+
+pytestmark = pytest.mark.gpu
+INF = float("inf")
+PS = [1.0, 2.0, INF]
+
+
+def dev(x):
+    return tuple(t.cuda().contiguous() for t in x.tensors())
+
+
+def gpu_bounds(x, p, eps, words=1):
+    from faith_amd import Bounds
+    from types import SimpleNamespace
+    lw, lb, uw, ub = dev(x)
+    return Bounds(SimpleNamespace(perturbed_words=words), p, eps, lw=lw, lb=lb, uw=uw, ub=ub)
+
+
+def assert_bounds_close(got, exp, rtol=1e-5, atol=1e-6, what=""):
+    for name, g_, e in zip(("lw", "lb", "uw", "ub"), (got.lw, got.lb, got.uw, got.ub), exp.tensors()):
+        assert g_.shape == e.shape, (what, name, g_.shape, e.shape)
+        assert close(g_, e, rtol=rtol, atol=atol), f"{what} {name}: {worst(g_, e)}"
+
+
+@pytest.mark.parametrize("p", PS)
+@pytest.mark.parametrize("words", [1, 2])
+def test_multiply_shapes(p, words):
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(61)
+    for (L, D, H) in [(4, 64, 64), (3, 128, 96), (2, 256, 64), (1, 600, 40), (2, 12, 37), (1, 2, 5)]:
+        x = rand_bounds(g, 1, L, D, H, ordered=False, sw=0.1)
+        y = rand_bounds(g, 1, L, D, H, ordered=False, sw=0.1)
+        print(f"[case] multiply {L,D,H} p={p} words={words}", flush=True)
+        z = ops.multiply(dev(x), dev(y), p, 0.05, words)
+        e = O.multiply(x, y, p, 0.05, words)
+        # constant terms are sums of O(1) products of concrete bounds: allow for the ulp-level
+        # difference between the two norm reductions that feed them
+        for name, g_, ee, tol in zip(("lw", "lb", "uw", "ub"), z, e.tensors(), (1e-6, 4e-6, 1e-6, 4e-6)):
+            assert close(g_, ee, rtol=1e-5, atol=tol), f"{name}: {worst(g_, ee)}"
+
+
+def test_scale_add_shift_are_exact():
+    """One rounding per operation on both sides: these must agree bit for bit."""
+    g = torch.Generator().manual_seed(62)
+    x = rand_bounds(g, 2, 3, 16, 24, ordered=False)
+    y = rand_bounds(g, 2, 3, 16, 24, ordered=False)
+    bx, by = gpu_bounds(x, 2.0, 0.1), gpu_bounds(y, 2.0, 0.1)
+    W = torch.randn(24, generator=g)
+    W[3] = 0.0
+    for got, exp in ((bx.multiply(2.5), O.scale(x, 2.5)), (bx.multiply(-0.75), O.scale(x, -0.75)),
+                     (bx.multiply(W.cuda()), O.scale(x, W)), (bx.add(by), O.add(x, y)),
+                     (bx.add(W.cuda()), O.add(x, W)), (bx.add(0.25), O.add(x, 0.25))):
+        for a, b in zip((got.lw, got.lb, got.uw, got.ub), exp.tensors()):
+            assert torch.equal(a.cpu(), b)
+
+
+@pytest.mark.parametrize("p", PS)
+def test_divide_and_softmax(p):
+    g = torch.Generator().manual_seed(63)
+    x = rand_bounds(g, 2, 6, 32, 16, sw=0.05, sb=1.0, gap_w=0.005, gap_b=0.1)
+    pos = rand_bounds(g, 2, 6, 32, 16, sw=0.02, sb=0.5, gap_w=0.005, gap_b=0.1)
+    pos = O.LinearBounds(pos.lw, pos.lb.abs() + 1.0, pos.uw, pos.lb.abs() + 1.0 + (pos.ub - pos.lb))
+    eps = 0.05
+    bx, bp = gpu_bounds(x, p, eps), gpu_bounds(pos, p, eps)
+    assert_bounds_close(bx.divide(bp), O.divide(x, pos, p, eps), rtol=2e-5, atol=4e-6, what="divide")
+    assert_bounds_close(bx.softmax(), O.softmax(x, p, eps), rtol=5e-5, atol=4e-6, what="softmax")
+    # a row of probability bounds brackets a distribution
+    lo, hi = bx.softmax().concretize()
+    assert bool((lo.sum(-1) <= 1 + 1e-4).all()) and bool((hi.sum(-1) >= 1 - 1e-4).all())
+
+
+@pytest.mark.parametrize("mode", ["no", "no_var", "standard"])
+@pytest.mark.parametrize("p", [2.0, INF])
+def test_layer_norm(mode, p):
+    g = torch.Generator().manual_seed(64)
+    H = 64
+    x = rand_bounds(g, 1, 8, 32, H, sw=0.02, sb=1.0, gap_w=0.002, gap_b=0.02)
+    weight, bias = torch.randn(H, generator=g), torch.randn(H, generator=g)
+
+    class Norm:
+        pass
+    n = Norm()
+    n.weight, n.bias = weight.cuda(), bias.cuda()
+    got = gpu_bounds(x, p, 0.01).layer_norm(n, mode)
+    exp = O.layer_norm(x, weight, bias, mode, p, 0.01)
+    # a chain of six to ten operators: rounding differences compound
+    assert_bounds_close(got, exp, rtol=1e-4, atol=2e-5, what=f"layer_norm/{mode}")
+
+
+def test_rowsum_broadcast():
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(65)
+    for shape in [(2, 3, 7, 64), (1, 5, 100), (3, 1, 2, 5)]:
+        t = torch.randn(*shape, generator=g)
+        out = ops.rowsum_broadcast(t.cuda())
+        exp = t.sum(-1, keepdim=True).expand_as(t)
+        assert close(out, exp, rtol=1e-5, atol=2e-6)

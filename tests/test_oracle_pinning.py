@@ -433,3 +433,84 @@ def test_exp_saturates_above_threshold():
         cap = lambda v: math.exp(v) if v < 12 else e12 * (v - 11.0)
         ku = (cap(hi) - cap(lo)) / (hi - lo)
         assert abs(y.ub[0, 0, j].item() - (hi * ku - ku * lo + cap(lo))) / cap(hi) < 1e-5
+
+
+# ------------------------------------ scale / add / multiply / divide / softmax / layer_norm
+def test_scale_and_add_definitions():
+    x = rand_bounds(gen(24), 1, 2, 4, 6, ordered=False)
+    y = rand_bounds(gen(25), 1, 2, 4, 6, ordered=False)
+    s = O.scale(x, 2.5)
+    assert torch.equal(s.lw, x.lw * 2.5) and torch.equal(s.ub, x.ub * 2.5)
+    s = O.scale(x, -2.0)                                   # negative factor swaps the sides
+    assert torch.equal(s.lw, x.uw * -2.0) and torch.equal(s.lb, x.ub * -2.0) and torch.equal(s.uw, x.lw * -2.0)
+    W = torch.tensor([1.0, -2.0, 0.0, 0.5, -0.25, 3.0])
+    s = O.scale(x, W)
+    for j, w in enumerate(W.tolist()):
+        a, b = (x.lw, x.uw) if w > 0 else (x.uw, x.lw)
+        assert torch.allclose(s.lw[..., j], a[..., j] * w) and torch.allclose(s.uw[..., j], b[..., j] * w)
+    z = O.add(x, y)
+    assert torch.equal(z.lw, x.lw + y.lw) and torch.equal(z.ub, x.ub + y.ub)
+    z = O.add(x, 0.5)
+    assert torch.equal(z.lw, x.lw) and torch.equal(z.lb, x.lb + 0.5)
+
+
+@pytest.mark.parametrize("p", PS)
+@pytest.mark.parametrize("words", [1, 2])
+def test_multiply_vs_brute_force(p, words):
+    """An elementwise product is a dot product with a reduction of length one."""
+    g = gen(26)
+    x = rand_bounds(g, 1, 3, 4, 7, ordered=False)
+    y = rand_bounds(g, 1, 3, 4, 7, ordered=False)
+    z = O.multiply(x, y, p, 0.3, words)
+    for l in range(3):
+        for j in range(7):
+            col = lambda t_: f64(t_)[0, l, :, j].reshape(1, 4, 1)
+            sc = lambda t_: f64(t_)[0, l, j].reshape(1, 1)
+            e = C.dot_brute(col(x.lw), sc(x.lb), col(x.uw), sc(x.ub), col(y.lw), sc(y.lb), col(y.uw), sc(y.ub),
+                            p, 0.3, words)
+            np.testing.assert_allclose(f64(z.lw)[0, l, :, j], e[0][0, :, 0], rtol=1e-5, atol=2e-6)
+            np.testing.assert_allclose(f64(z.lb)[0, l, j], e[1][0, 0], rtol=1e-5, atol=2e-6)
+            np.testing.assert_allclose(f64(z.uw)[0, l, :, j], e[2][0, :, 0], rtol=1e-5, atol=2e-6)
+            np.testing.assert_allclose(f64(z.ub)[0, l, j], e[3][0, 0], rtol=1e-5, atol=2e-6)
+
+
+def _bounded_between(fn, x, y, g, D, p, eps, slack=1e-4):
+    delta = _sample_delta(g, D, p, eps, 200)
+    lo_in, hi_in = _eval(x.lw[0], x.lb[0], delta), _eval(x.uw[0], x.ub[0], delta)
+    lo_out, hi_out = _eval(y.lw[0], y.lb[0], delta), _eval(y.uw[0], y.ub[0], delta)
+    for t in (0.0, 0.35, 1.0):
+        v = fn(lo_in + t * (hi_in - lo_in))
+        assert (v >= lo_out - slack * (1 + v.abs())).all(), float((lo_out - v).max())
+        assert (v <= hi_out + slack * (1 + v.abs())).all(), float((v - hi_out).max())
+
+
+@pytest.mark.parametrize("p", PS)
+def test_softmax_soundness(p):
+    g = gen(27)
+    x = rand_bounds(g, 1, 3, 5, 8, sw=0.1, sb=1.0, gap_w=0.01, gap_b=0.05)
+    x.ub += 0.02
+    y = O.softmax(x, p, 0.1)
+    _bounded_between(lambda v: torch.softmax(v, dim=-1), x, y, g, 5, p, 0.1)
+    # the bounds of one row of probabilities must bracket a distribution: sum l <= 1 <= sum u
+    lo, hi = O.concretize(y, p, 0.1)
+    assert (lo.sum(-1) <= 1 + 1e-5).all() and (hi.sum(-1) >= 1 - 1e-5).all()
+
+
+@pytest.mark.parametrize("p", PS)
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+def test_layer_norm_soundness(p, mode):
+    g = gen(28)
+    H = 8
+    x = rand_bounds(g, 1, 3, 5, H, sw=0.05, sb=1.0, gap_w=0.005, gap_b=0.02)
+    x.ub += 0.01
+    weight = torch.randn(H, generator=g)
+    bias = torch.randn(H, generator=g)
+    y = O.layer_norm(x, weight, bias, mode, p, 0.05)
+
+    def true_ln(v):
+        c = v - v.mean(-1, keepdim=True)
+        if mode == "standard":
+            c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + 1e-12)
+        return c * weight.double() + bias.double()
+    _bounded_between(true_ln, x, y, g, 5, p, 0.05)
+    assert O.layer_norm(x, weight, bias, "no", p, 0.05) is x
