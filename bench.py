@@ -157,6 +157,17 @@ def bench_config1(args, ops, O, wl, steps, warmup):
         t = gpu_times_ms(lambda: one(kind, p), max(steps, 50), 5)
         per_kernel[(kind, p)] = t
         entries.append(op_entry(f"config1 {kind} p={p:g} [1,128,256,512] words=2", "hbm", t, nbytes))
+    # the other relaxations on the same skeleton and the product of two objects, same shape, p = 2
+    # (not among the five configurations; reciprocal and sqrt get strictly positive pre-activations)
+    xp = {k: v.clone() for k, v in x.items()}       # distinct memory: the product must read both objects
+    xp["lb"] = x["lb"].abs() + 2.0
+    xp["ub"] = xp["lb"] + (x["ub"] - x["lb"])
+    for kind, src_x in (("exp", x), ("sqr", x), ("sqrt", xp), ("reciprocal", xp)):
+        t = gpu_times_ms(lambda: getattr(ops, kind)(*quad(src_x), 2.0, c["eps"], c["words"], out=out), 50, 5)
+        entries.append(op_entry(f"extra: {kind} p=2 [1,128,256,512] words=2", "hbm", t, nbytes))
+    t = gpu_times_ms(lambda: ops.multiply(quad(x), quad(xp), 2.0, c["eps"], c["words"], out=out), 50, 5)
+    entries.append(op_entry("extra: multiply(Bounds, Bounds) p=2 [1,128,256,512] words=2", "hbm", t,
+                            24 * x["lw"].numel() + 24 * x["lb"].numel()))
     src = torch.empty(nbytes // 8, device="cuda")
     dst = torch.empty_like(src)
     from faith_amd import _lib

@@ -1,0 +1,99 @@
+"""One Transformer encoder layer end to end: embeddings -> layer norm -> self-attention -> feed
+forward -> pooling -> classifier, driven by faith_amd/forward.py.
+
+CPU: the pipeline on the oracle is sound (the true network output of sampled perturbations lies
+inside the propagated bounds).  GPU: the same pipeline on faith_amd.Bounds reproduces the oracle's
+bounds and is sound as well.  Mirrors VerifierForward.verify_safety (VerifierForward.py:93-125)."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from faith_amd import forward as F
+from tests.oracle_bounds import OracleBounds, random_layer, to_device, true_layer
+
+HIDDEN, HEADS, INTER, LENGTH = 32, 4, 64, 6
+
+
+def build(seed, mode):
+    g = torch.Generator().manual_seed(seed)
+    layer = random_layer(g, HIDDEN, HEADS, INTER)
+    embed_norm = SimpleNamespace(weight=1.0 + 0.1 * torch.randn(HIDDEN, generator=g),
+                                 bias=0.05 * torch.randn(HIDDEN, generator=g))
+    pooler = SimpleNamespace(weight=torch.randn(HIDDEN, HIDDEN, generator=g) / HIDDEN ** 0.5,
+                             bias=0.05 * torch.randn(HIDDEN, generator=g))
+    classifier = SimpleNamespace(weight=torch.randn(2, HIDDEN, generator=g) / HIDDEN ** 0.5,
+                                 bias=0.05 * torch.randn(2, generator=g))
+    emb = torch.randn(1, LENGTH, HIDDEN, generator=g)
+    return layer, embed_norm, pooler, classifier, emb
+
+
+def propagate(make, emb, parts, mode, p, eps, index):
+    layer, embed_norm, pooler, classifier = parts
+    x = F.bound_input(make, emb, index, eps, 1, p, embed_norm, mode)
+    scores, probs, out = F.bound_layer(x, layer, mode, "relu")
+    pooled = F.bound_pooling(out, pooler, make)
+    safe, l, u = F.bound_classifier(pooled, classifier, 0)
+    return out, l, u, safe
+
+
+def check_sound(out_l, out_u, l, u, emb, parts, mode, p, eps, index, g):
+    layer, embed_norm, pooler, classifier = parts
+    d = torch.randn(64, HIDDEN, generator=g, dtype=torch.float64)
+    if p == float("inf"):
+        d = torch.sign(d) * eps
+    else:
+        d = d / torch.linalg.vector_norm(d, ord=p, dim=1, keepdim=True) * eps
+    x = emb.double().repeat(64, 1, 1)
+    x[:, index] += d
+    out, margin = true_layer(x, layer, embed_norm, mode, pooler, classifier)
+    slack = 1e-4
+    assert bool((out >= out_l.double() - slack).all()) and bool((out <= out_u.double() + slack).all())
+    lo, hi = l.double()[0, 0, 0], u.double()[0, 0, 0]        # output 0 of the margin classifier
+    assert bool((margin >= lo - slack).all()) and bool((margin <= hi + slack).all())
+
+
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+@pytest.mark.parametrize("p", [2.0, float("inf")])
+def test_pipeline_on_the_oracle_is_sound(mode, p):
+    layer, embed_norm, pooler, classifier, emb = build(7, mode)
+    eps, index = 0.02, 2
+    make = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)
+    out, l, u, _ = propagate(make, emb, (layer, embed_norm, pooler, classifier), mode, p, eps, index)
+    ol, ou = out.concretize()
+    assert bool((l <= u).all()) and bool((ol <= ou).all())
+    check_sound(ol, ou, l, u, emb, (layer, embed_norm, pooler, classifier), mode, p, eps, index,
+                torch.Generator().manual_seed(8))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+@pytest.mark.parametrize("p", [2.0, float("inf")])
+def test_pipeline_on_hip_matches_the_oracle_and_is_sound(mode, p):
+    from faith_amd import Bounds
+    layer, embed_norm, pooler, classifier, emb = build(7, mode)
+    eps, index = 0.02, 2
+    parts = (layer, embed_norm, pooler, classifier)
+    omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)
+    o_out, o_l, o_u, o_safe = propagate(omake, emb, parts, mode, p, eps, index)
+
+    gparts = tuple(to_device(x, "cuda") for x in parts)
+    gmake = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    g_out, g_l, g_u, g_safe = propagate(gmake, emb.cuda(), gparts, mode, p, eps, index)
+    torch.cuda.synchronize()
+
+    # ~25 chained operators: compare at a tolerance that allows rounding to compound, relative to the
+    # size of the quantities involved
+    def near(a, b, what, rel=2e-4):
+        a, b = a.cpu().double(), b.double()
+        err = float((a - b).abs().max())
+        scale = float(b.abs().max())
+        assert err <= rel * max(scale, 1.0), f"{what}: max err {err:.3g} at scale {scale:.3g}"
+    near(g_out.lw, o_out.lw, "output lw"); near(g_out.uw, o_out.uw, "output uw")
+    near(g_out.lb, o_out.lb, "output lb"); near(g_out.ub, o_out.ub, "output ub")
+    # behind the pooler's tanh the chord slopes divide by interval widths of ~1e-2, which amplifies
+    # the accumulated differences once more
+    near(g_l, o_l, "margin l", 1e-3); near(g_u, o_u, "margin u", 1e-3)
+    gl, gu = g_out.concretize()
+    check_sound(gl.cpu(), gu.cpu(), g_l.cpu(), g_u.cpu(), emb, parts, mode, p, eps, index,
+                torch.Generator().manual_seed(9))
