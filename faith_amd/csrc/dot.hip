@@ -14,13 +14,26 @@
 // and every store is a 128-byte run.  Neither the [Lx, D, d, Ly] broadcast the PyTorch code
 // materialises nor the transposed add of its y-terms exists here.
 //
-// Tiling: workgroup = 4 wavefronts on a 128 x 128 (i x j) tile of one (head, m); wavefront tile
-// 64 x 64 (2 x 2 blocks of v_mfma_f32_32x32x2_f32, for each of z_lw and z_uw).  K-step 8:
-// seven operand tiles [128 x 8] per step (xlw, xuw, b | a_l, a_u, ylw, yuw) = 28 KB, double
-// buffered = 56 KB, so two workgroups share a CU.  Rows are 8 floats with the two 16-byte halves
-// swapped on every other group of four rows, which makes both the 16-byte stores and the 16-byte
-// fragment reads bank-conflict free without padding.  a / b are split by sign after the LDS
-// read (v_max / v_min); they are staged from the concretization results, unsplit.
+// Tiling: workgroup = 4 wavefronts on a 128 x 64 (i x j) tile of one (head, m); wavefront tile
+// 64 x 32 (two v_mfma_f32_32x32x2_f32 blocks along i, for each of z_lw and z_uw).  K-step 8:
+// operand tiles xlw, xuw, b+, b- [128 x 8] and a_l+, a_l-, a_u+, a_u-, ylw, yuw [64 x 8] = 28 KB,
+// double buffered, two workgroups per CU.  Rows are 8 floats with the two 16-byte halves swapped
+// on every other group of four rows, which makes both the 16-byte stores and the 16-byte fragment
+// reads bank-conflict free without padding.
+//
+// On this part every vector-ALU instruction a wavefront issues takes its slot from the MFMA pipe
+// (measured: 48 v_max / v_min per 64 MFMAs cost 5 % of the MFMA rate, more when interleaved), so
+// the K-loop is written to issue almost none:
+//   * a / b are split by sign ONCE, by the thread that stages them, not by every wavefront that
+//     reads them;
+//   * global addresses are a wave-uniform 64-bit base (scalar ALU) plus a per-thread 32-bit offset
+//     that only changes from tile to tile; the K-step advances the scalar base;
+//   * tiles are numbered in mixed radix and walked with scalar adds and carries (no division);
+//   * bounds predicates exist only on the paths for ragged tiles and a ragged last K-step.
+//
+// The reduction is short (d = 64 is eight K-steps), so a tile's 64 KB of results would otherwise
+// leave in a burst during which no MFMA issues.  Each wavefront therefore holds TWO accumulator
+// sets: while tile n accumulates in one, tile n-1 leaves from the other, eight rows per K-step.
 //
 // The constant terms z_lb / z_ub ([Lx, Ly] per head, 1/D_in of the work, O(1) cancelling terms)
 // are summed in double by a small kernel.
@@ -30,9 +43,14 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int TI = 128, TJ = 128, BK = 8;
+constexpr int TI = 128, TJ = 64, BK = 8;
 constexpr int NTHREADS = 256;
-constexpr int TILE = 128 * BK;            // floats per operand tile
+constexpr int XT = TI * BK, YT = TJ * BK;        // floats per operand tile
+// one stage of LDS: offsets of the ten operand tiles
+constexpr int XL = 0, XU = XT, BP = 2 * XT, BN = 3 * XT;
+constexpr int ALP = 4 * XT, ALN = ALP + YT, AUP = ALP + 2 * YT, AUN = ALP + 3 * YT, YL = ALP + 4 * YT, YU = ALP + 5 * YT;
+constexpr int STAGE = 4 * XT + 6 * YT;
+constexpr int PIECES = 8;                        // a finished tile leaves in 8 pieces of 4 rows x 2 blocks
 
 struct DotArgs {
     const float *xlw, *xuw, *ylw, *yuw;   // [B, Lx, D, d], [B, Ly, D, d]
@@ -46,210 +64,352 @@ struct DotArgs {
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
-__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
-__device__ __forceinline__ float4 pos4(float4 v) {
-    return make_float4(fmaxf(v.x, 0.f), fmaxf(v.y, 0.f), fmaxf(v.z, 0.f), fmaxf(v.w, 0.f));
+// Buffer addressing keeps the three parts of an address apart in the instruction itself: a
+// wave-uniform descriptor (base pointer, size), a wave-uniform 32-bit offset and a per-thread
+// 32-bit offset.  With flat pointers the compiler folds the K advance into 64-bit vector adds.
+// Accesses at or beyond `bytes` from the base are dropped by the hardware (loads return zero).
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ unsigned clamp32(size_t bytes) { return (bytes >> 32) ? 0xffffffffu : (unsigned)bytes; }
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
-__device__ __forceinline__ float4 neg4(float4 v) {
-    return make_float4(fminf(v.x, 0.f), fminf(v.y, 0.f), fminf(v.z, 0.f), fminf(v.w, 0.f));
+__device__ __forceinline__ float4 ld4(__amdgpu_buffer_rsrc_t r, unsigned thread_off, unsigned uniform_off) {
+    const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, thread_off, uniform_off, 0);
+    return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
 }
+__device__ __forceinline__ void st1_nt(float v, __amdgpu_buffer_rsrc_t r, unsigned thread_off, unsigned uniform_off) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, thread_off, uniform_off, 2 /* non-temporal */);
+}
+// max(v, 0) / min(v, 0) as single instructions (fmaxf / fminf add a canonicalising v_max each)
+__device__ __forceinline__ float pos1(float v) {
+    float r;
+    asm("v_max_f32 %0, 0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+__device__ __forceinline__ float neg1(float v) {
+    float r;
+    asm("v_min_f32 %0, 0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+__device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
+__device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
 
-// position of 16-byte half `c` (0 / 1) of row `row` inside an [128 x 8] tile
+// position of 16-byte half `c` (0 / 1) of row `row` inside an [rows x 8] tile
 __device__ __forceinline__ int swz(int row, int c) { return row * BK + 4 * (c ^ ((row >> 2) & 1)); }
 
-enum { XL = 0, XU, BT, AL, AU, YL, YU, NOPS };
+// Tile numbers in mixed radix (j-tile, i-tile, m or m / 8, head), least significant first.
+struct Walk {
+    int j, i, m, t;
+};
 
 // Persistent: the grid is sized to the machine (two workgroups per CU) and every workgroup walks
 // tiles pid, pid + grid, ...  The walk is ONE software pipeline over (tile, K-step): the global
 // loads of the next step -- the first K-step of the next tile included -- are issued before the
-// MFMAs of the current step, and the accumulator stores of a finished tile are issued while
-// those loads are in flight, so neither the head nor the tail of a tile leaves the MFMA pipe idle.
+// MFMAs of the current step, and the results of the previous tile are stored piecewise between
+// them, so neither the head nor the tail of a tile leaves the MFMA pipe idle.
+//
+// xcd_map != 0 (needs dim_in % 8 == 0 and grid % 8 == 0): workgroups are dealt to the eight XCDs
+// round robin, so workgroup w only takes perturbation coordinates m = w (mod 8); the tiles of one
+// (head, m) -- which read the same x rows and y rows -- are then consecutive tiles of ONE XCD and
+// meet in its L2.
 //
 // VP = false: scores path, y is [B, Ly, D, d] (reduction axis contiguous, like x).
 // VP = true : context path (probs . value): y is the value bound object in its own natural layout
 //   [B, d, D, Ly] -- the reduction axis (key position) is the slow one and j is contiguous --
 //   and so are its concrete bounds [B, d, Ly].  The y-side tiles are then staged as [k][j]
 //   (16-byte loads along j, conflict-free) and their fragments read with four 4-byte LDS reads.
-template <bool VP>
+//
+// RAGGED = true: d % 8 == 4, half of the last K-step lies past d.  Threads past d then read their
+// K-step-0 element instead (in bounds) and discard it before it reaches LDS.
+template <bool VP, bool RAGGED>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-dot_w(const DotArgs g, const int total_tiles) {
-    __shared__ float sm[2][NOPS][TILE];
+dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
+    __shared__ float sm[2][STAGE];
 
     const int ti = (g.Lx + TI - 1) / TI, tj = (g.Ly + TJ - 1) / TJ;
     const int d = g.d;
     const int nk = (d + BK - 1) / BK;
 
     const int tid = threadIdx.x;
-    const int lane = tid % 64, wv = tid / 64;
+    const int lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wi = wv / 2, wj = wv % 2;
     const int fi = lane % 32, fh = lane / 32;
 
-    // ---- staging: one float4 per operand per thread per K-step
+    // ---- the walk: this workgroup's first tile and the stride, digit by digit
+    const int m_low = xcd_map ? (int)(blockIdx.x % 8) : 0;
+    const int m_radix = xcd_map ? g.D / 8 : g.D;
+    auto digits = [&](int n) {
+        Walk w;
+        w.j = n % tj;  n /= tj;
+        w.i = n % ti;  n /= ti;
+        w.m = n % m_radix;
+        w.t = n / m_radix;
+        return w;
+    };
+    Walk cur = digits(xcd_map ? blockIdx.x / 8 : blockIdx.x);
+    const Walk step = digits(xcd_map ? gridDim.x / 8 : gridDim.x);
+    auto advance = [&](Walk w) {
+        w.j += step.j;
+        if (w.j >= tj) { w.j -= tj; w.i += 1; }
+        w.i += step.i;
+        if (w.i >= ti) { w.i -= ti; w.m += 1; }
+        w.m += step.m;
+        if (w.m >= m_radix) { w.m -= m_radix; w.t += 1; }
+        w.t += step.t;
+        return w;
+    };
+    int tiles_left = ((int)blockIdx.x < total_tiles) ? (total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+    if (tiles_left == 0) return;
+
+    // ---- staging: per K-step every thread moves one float4 of xlw, xuw, b and two of the y side:
+    // wavefronts 0, 1 take (a_l, a_u), wavefronts 2, 3 take (ylw, yuw)
     const int srow = tid / 2, sc = tid % 2;
     const int sdst = swz(srow, sc);
-    const int vk = tid / 32, vj = (tid % 32) * 4;          // VP: this thread's (k, j..j+3) of a y-side tile
-    const int ydst = VP ? vk * TJ + vj : sdst;
-    // element offsets of this thread's source rows (32-bit: the entry point checks the sizes);
-    // xlw / xuw share one, ylw / yuw share one, a_l / a_u share one
-    unsigned ox, oy, obt, oa;
-    bool y_in = true;                                      // VP: columns past Ly are staged as zeros
-    float4 pre[NOPS];
-    auto point_at = [&](int tile) {
-        int q = tile;
-        const int j0 = (q % tj) * TJ;  q /= tj;
-        const int i0 = (q % ti) * TI;  q /= ti;
-        const int m = q % g.D, t = q / g.D;
-        const int irow = min(i0 + srow, g.Lx - 1);         // clamped rows are never stored
-        ox = ((unsigned)(t * g.Lx + irow) * g.D + m) * d + sc * 4;
-        obt = (unsigned)(t * g.Lx + irow) * d + sc * 4;
+    const bool wside = wv >= 2;
+    const int t2 = tid % 128;
+    const int yrow = t2 / 2, yc = t2 % 2;                  // scores path: (row, half) of a y-side tile
+    const int vk = t2 / 16, vj = (t2 % 16) * 4;            // context path: (k, j..j+3)
+    const int ydst = VP ? vk * TJ + vj : swz(yrow, yc);
+    // wave-uniform bases of the tile being loaded (bytes) and this thread's offsets from them
+    const float *bxl = nullptr, *bxu = nullptr, *bbt = nullptr, *by0 = nullptr, *by1 = nullptr;
+    unsigned nx = 0, nbt = 0, ny = 0;                      // bytes from those bases to the end of the tensors (< 4 GB kept)
+    unsigned vx = 0, vbt = 0, vy = 0;
+    // K-step strides in bytes: x side and scores-path y side advance along the contiguous axis (the
+    // entry point checks that one head of y spans less than 4 GB)
+    const unsigned ystride = VP ? (unsigned)BK * g.Ly * (wside ? g.D : 1) * 4u : BK * 4u;
+    // totals in elements
+    const size_t tot_x = (size_t)g.B * g.Lx * g.D * d, tot_bt = (size_t)g.B * g.Lx * d;
+    const size_t tot_y = (size_t)g.B * g.Ly * d * (wside ? g.D : 1), tot_z = (size_t)g.B * g.Lx * g.D * g.Ly;
+    // results: first element of the tile being loaded (zn) and of the tile being computed (zc)
+    size_t zn = 0, zc = 0;
+    int zn_i0 = 0, zn_j0 = 0, zc_i0 = 0, zc_j0 = 0;
+    float4 pre[5];
+
+    auto point_at = [&](const Walk &w) {
+        const int j0 = w.j * TJ, i0 = w.i * TI, t = w.t;
+        const int m = xcd_map ? w.m * 8 + m_low : w.m;
+        const size_t xrow0 = (size_t)t * g.Lx + i0;
+        const size_t x0 = (xrow0 * g.D + m) * d, bt0 = xrow0 * d;
+        bxl = g.xlw + x0;  bxu = g.xuw + x0;  nx = clamp32((tot_x - x0) * 4);
+        bbt = g.x_l + bt0;  nbt = clamp32((tot_bt - bt0) * 4);
+        const int irow = min(srow, g.Lx - 1 - i0);         // clamped rows are never stored
+        vx = ((unsigned)irow * g.D * d + sc * 4) * 4u;
+        vbt = ((unsigned)irow * d + sc * 4) * 4u;
+        size_t y0;
         if (VP) {
-            y_in = j0 + vj < g.Ly;                         // Ly % 4 == 0
-            oy = ((unsigned)(t * d + vk) * g.D + m) * g.Ly + j0 + vj;
-            oa = (unsigned)(t * d + vk) * g.Ly + j0 + vj;
+            // y[t, k, m, j] / a[t, k, j]; the j offset stays with the thread so that it can be clamped
+            y0 = wside ? ((size_t)t * d * g.D + m) * g.Ly : (size_t)t * d * g.Ly;
+            const int jc = min(j0 + vj, g.Ly - 4);         // Ly % 4 == 0; clamped columns are never stored
+            vy = ((unsigned)vk * g.Ly * (wside ? g.D : 1) + jc) * 4u;
         } else {
-            const int jrow = min(j0 + srow, g.Ly - 1);
-            oy = ((unsigned)(t * g.Ly + jrow) * g.D + m) * d + sc * 4;
-            oa = (unsigned)(t * g.Ly + jrow) * d + sc * 4;
+            const size_t yrow0 = (size_t)t * g.Ly + j0;
+            y0 = wside ? (yrow0 * g.D + m) * d : yrow0 * d;
+            const int jrow = min(yrow, g.Ly - 1 - j0);
+            vy = ((unsigned)jrow * d * (wside ? g.D : 1) + yc * 4) * 4u;
         }
+        by0 = (wside ? g.ylw : g.y_l) + y0;
+        by1 = (wside ? g.yuw : g.y_u) + y0;
+        ny = clamp32((tot_y - y0) * 4);
+        zn = (xrow0 * g.D + m) * g.Ly + j0;
+        zn_i0 = i0;
+        zn_j0 = j0;
     };
-    auto gload = [&](int kt) {
-        const int k = kt * BK;
-        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-        const bool x_ok = k + sc * 4 < d;                  // d % 4 == 0: a float4 is all in or all out
-        pre[XL] = x_ok ? ld4(g.xlw + ox + k) : zero;
-        pre[XU] = x_ok ? ld4(g.xuw + ox + k) : zero;
-        pre[BT] = x_ok ? ld4(g.x_l + obt + k) : zero;
-        if (VP) {
-            const bool y_ok = y_in && k + vk < d;
-            const unsigned ky = (unsigned)k * g.D * g.Ly, ka = (unsigned)k * g.Ly;
-            pre[AL] = y_ok ? ld4(g.y_l + oa + ka) : zero;
-            pre[AU] = y_ok ? ld4(g.y_u + oa + ka) : zero;
-            pre[YL] = y_ok ? ld4(g.ylw + oy + ky) : zero;
-            pre[YU] = y_ok ? ld4(g.yuw + oy + ky) : zero;
+    // scalar base + K advance, per-thread 32-bit offset
+    auto x_past = [&](int kt) { return RAGGED && kt * BK + sc * 4 >= d; };
+    auto y_past = [&](int kt) { return RAGGED && (VP ? kt * BK + vk >= d : kt * BK + yc * 4 >= d); };
+    auto load_step = [&](int kt) {
+        const __amdgpu_buffer_rsrc_t rxl = window(bxl, nx), rxu = window(bxu, nx), rbt = window(bbt, nbt);
+        const __amdgpu_buffer_rsrc_t ry0 = window(by0, ny), ry1 = window(by1, ny);
+        const unsigned kx = kt * (BK * 4u), ky = kt * ystride;
+        if (RAGGED) {
+            const unsigned ox = x_past(kt) ? 0u : kx, oy = y_past(kt) ? 0u : ky;
+            pre[0] = ld4(rxl, vx + ox, 0);
+            pre[1] = ld4(rxu, vx + ox, 0);
+            pre[2] = ld4(rbt, vbt + ox, 0);
+            pre[3] = ld4(ry0, vy + oy, 0);
+            pre[4] = ld4(ry1, vy + oy, 0);
         } else {
-            pre[AL] = x_ok ? ld4(g.y_l + oa + k) : zero;
-            pre[AU] = x_ok ? ld4(g.y_u + oa + k) : zero;
-            pre[YL] = x_ok ? ld4(g.ylw + oy + k) : zero;
-            pre[YU] = x_ok ? ld4(g.yuw + oy + k) : zero;
+            pre[0] = ld4(rxl, vx, kx);
+            pre[1] = ld4(rxu, vx, kx);
+            pre[2] = ld4(rbt, vbt, kx);
+            pre[3] = ld4(ry0, vy, ky);
+            pre[4] = ld4(ry1, vy, ky);
         }
     };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int o = 0; o < NOPS; ++o)
-            *reinterpret_cast<float4 *>(&sm[buf][o][(o == XL || o == XU || o == BT) ? sdst : ydst]) = pre[o];
-    };
-    // y-side fragment of block b: four K values of column j; [j][k] tile -> one 16-byte read,
-    // [k][j] tile (VP) -> four 4-byte reads, lanes along j
-    auto yfrag = [&](int buf, int o, int b) -> float4 {
-        if (VP) {
-            const float *p = &sm[buf][o][(4 * fh) * TJ + wj * 64 + b * 32 + fi];
-            return make_float4(p[0], p[TJ], p[2 * TJ], p[3 * TJ]);
+    // registers -> LDS stage `buf`; kt is the K-step the registers hold
+    auto lstore = [&](int buf, int kt) {
+        if (RAGGED) {
+            const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (x_past(kt)) pre[0] = pre[1] = pre[2] = zero;
+            if (y_past(kt)) pre[3] = pre[4] = zero;
         }
-        return *reinterpret_cast<const float4 *>(&sm[buf][o][swz(wj * 64 + b * 32 + fi, fh)]);
+        float *s = sm[buf];
+        *reinterpret_cast<float4 *>(s + XL + sdst) = pre[0];
+        *reinterpret_cast<float4 *>(s + XU + sdst) = pre[1];
+        *reinterpret_cast<float4 *>(s + BP + sdst) = pos4(pre[2]);
+        *reinterpret_cast<float4 *>(s + BN + sdst) = neg4(pre[2]);
+        if (wside) {
+            *reinterpret_cast<float4 *>(s + YL + ydst) = pre[3];
+            *reinterpret_cast<float4 *>(s + YU + ydst) = pre[4];
+        } else {
+            *reinterpret_cast<float4 *>(s + ALP + ydst) = pos4(pre[3]);
+            *reinterpret_cast<float4 *>(s + ALN + ydst) = neg4(pre[3]);
+            *reinterpret_cast<float4 *>(s + AUP + ydst) = pos4(pre[4]);
+            *reinterpret_cast<float4 *>(s + AUN + ydst) = neg4(pre[4]);
+        }
     };
 
+    // ---- fragments: x side rows wi*64 + {0, 32} + fi, y side column wj*32 + fi; this lane's four K
+    // values are half `fh` of the K-step
     int fa[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) fa[s] = swz(wi * 64 + s * 32 + fi, fh);
+    const int fy = VP ? (4 * fh) * TJ + wj * 32 + fi : swz(wj * 32 + fi, fh);
+    auto yfrag = [&](const float *s, int o) -> float4 {
+        if (VP) {
+            const float *p = s + o + fy;
+            return make_float4(p[0], p[TJ], p[2 * TJ], p[3 * TJ]);
+        }
+        return *reinterpret_cast<const float4 *>(s + o + fy);
+    };
+    auto compute = [&](int buf, floatx16 (&cl)[2], floatx16 (&cu)[2]) {
+        const float *s = sm[buf];
+        float4 xl[2], xu[2], bp[2], bn[2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            xl[a] = *reinterpret_cast<const float4 *>(s + XL + fa[a]);
+            xu[a] = *reinterpret_cast<const float4 *>(s + XU + fa[a]);
+        }
+        const float4 alp = yfrag(s, ALP), aup = yfrag(s, AUP), aln = yfrag(s, ALN), aun = yfrag(s, AUN);
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            bp[a] = *reinterpret_cast<const float4 *>(s + BP + fa[a]);
+            bn[a] = *reinterpret_cast<const float4 *>(s + BN + fa[a]);
+        }
+        const float4 yl = yfrag(s, YL), yu = yfrag(s, YU);
+#define FAITH_DOT_STEP(c)                                   \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a] = mfma(xl[a].c, alp.c, cl[a]);                \
+        cu[a] = mfma(xu[a].c, aup.c, cu[a]);                \
+    }                                                       \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a] = mfma(xu[a].c, aln.c, cl[a]);                \
+        cu[a] = mfma(xl[a].c, aun.c, cu[a]);                \
+    }                                                       \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a] = mfma(bp[a].c, yl.c, cl[a]);                 \
+        cu[a] = mfma(bp[a].c, yu.c, cu[a]);                 \
+    }                                                       \
+    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
+        cl[a] = mfma(bn[a].c, yu.c, cl[a]);                 \
+        cu[a] = mfma(bn[a].c, yl.c, cu[a]);                 \
+    }
+        FAITH_DOT_STEP(x)
+        FAITH_DOT_STEP(y)
+        FAITH_DOT_STEP(z)
+        FAITH_DOT_STEP(w)
+#undef FAITH_DOT_STEP
+    };
 
-    floatx16 cl[2][2], cu[2][2];
-    int tile = blockIdx.x;
-    if (tile >= total_tiles) return;
-    point_at(tile);
-    gload(0);
-    lstore(0);
+    // ---- results of a finished tile: z[t, i, m, j]; register r of block a is row
+    // a*32 + 8*(r/4) + 4*(lane/32) + r%4 of the wavefront tile, lanes run along j.
+    // Piece c holds registers 4*(c%4) .. +3 of block c/4.  A row is a uniform offset from the tile's
+    // first element, the lane's own offset never changes (the entry point checks that a tile spans
+    // less than 4 GB).
+    const unsigned rsb = (unsigned)g.D * g.Ly * 4u;        // one step in i, bytes
+    const unsigned lane_off = (unsigned)(wi * 64 + 4 * fh) * rsb + (wj * 32 + fi) * 4u;
+    size_t pz = 0;                                         // finished tile: its first element
+    bool pfull = false;                                    // it lies wholly inside z
+    int prows = 0;                                         // else: rows this lane may store (0: none, the state
+                                                           // before the first tile has finished)
+    auto store_piece = [&](int c, const floatx16 (&pl)[2], const floatx16 (&pu)[2]) {
+        const int a = c / 4, q4 = c % 4;
+        const unsigned nz = clamp32((tot_z - pz) * 4);
+        const __amdgpu_buffer_rsrc_t rl = window(g.zlw + pz, nz), ru = window(g.zuw + pz, nz);
+        unsigned step_b = rsb;
+        asm volatile("" : "+s"(step_b));                   // keeps 32 row offsets from being hoisted and held
+        if (pfull) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const unsigned row = (a * 32 + 8 * q4 + rr) * step_b;
+                st1_nt(pl[a][4 * q4 + rr], rl, lane_off, row);
+                st1_nt(pu[a][4 * q4 + rr], ru, lane_off, row);
+            }
+        } else {
+            int rows = prows;
+            asm volatile("" : "+v"(rows));                 // likewise 32 row predicates
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                if (a * 32 + 8 * q4 + rr < rows) {
+                    const unsigned row = (a * 32 + 8 * q4 + rr) * step_b;
+                    st1_nt(pl[a][4 * q4 + rr], rl, lane_off, row);
+                    st1_nt(pu[a][4 * q4 + rr], ru, lane_off, row);
+                }
+            }
+        }
+    };
+
+    point_at(cur);
+    load_step(0);
+    lstore(0, 0);
+    zc = zn;  zc_i0 = zn_i0;  zc_j0 = zn_j0;
     __syncthreads();
     int buf = 0;
-    for (; tile < total_tiles; tile += gridDim.x) {
+
+    // one tile into (cl, cu) while the previous one leaves from (pl, pu)
+    auto run_tile = [&](floatx16 (&cl)[2], floatx16 (&cu)[2], const floatx16 (&pl)[2], const floatx16 (&pu)[2]) {
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
-        const int next_tile = tile + gridDim.x;
-        const bool has_next = next_tile < total_tiles;
+            for (int r = 0; r < 16; ++r) cl[a][r] = cu[a][r] = 0.f;
+        const bool has_next = tiles_left > 1;
         for (int kt = 0; kt < nk; ++kt) {
             const bool last = kt + 1 == nk;
-            if (!last) {
-                gload(kt + 1);
-            } else if (has_next) {
-                point_at(next_tile);
-                gload(0);
+            // ONE load site for "next K-step" and "first K-step of the next tile": two sites would
+            // land in different registers and be reconciled by copies that wait for the loads
+            if (last && has_next) {
+                cur = advance(cur);
+                point_at(cur);
             }
-            float4 xl[2], xu[2], bp[2], bn[2];
+            if (!last || has_next) load_step(last ? 0 : kt + 1);
+            compute(buf, cl, cu);
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                xl[s] = *reinterpret_cast<const float4 *>(&sm[buf][XL][fa[s]]);
-                xu[s] = *reinterpret_cast<const float4 *>(&sm[buf][XU][fa[s]]);
-                const float4 bt = *reinterpret_cast<const float4 *>(&sm[buf][BT][fa[s]]);
-                bp[s] = pos4(bt);
-                bn[s] = neg4(bt);
-            }
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const float4 al = yfrag(buf, AL, b), au = yfrag(buf, AU, b);
-                const float4 yl = yfrag(buf, YL, b), yu = yfrag(buf, YU, b);
-                const float4 alp = pos4(al), aln = neg4(al), aup = pos4(au), aun = neg4(au);
-#define FAITH_DOT_STEP(c)                                   \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a][b] = mfma(xl[a].c, alp.c, cl[a][b]);          \
-        cu[a][b] = mfma(xu[a].c, aup.c, cu[a][b]);          \
-    }                                                       \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a][b] = mfma(xu[a].c, aln.c, cl[a][b]);          \
-        cu[a][b] = mfma(xl[a].c, aun.c, cu[a][b]);          \
-    }                                                       \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a][b] = mfma(bp[a].c, yl.c, cl[a][b]);           \
-        cu[a][b] = mfma(bp[a].c, yu.c, cu[a][b]);           \
-    }                                                       \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a][b] = mfma(bn[a].c, yu.c, cl[a][b]);           \
-        cu[a][b] = mfma(bn[a].c, yl.c, cu[a][b]);           \
-    }
-                FAITH_DOT_STEP(x)
-                FAITH_DOT_STEP(y)
-                FAITH_DOT_STEP(z)
-                FAITH_DOT_STEP(w)
-#undef FAITH_DOT_STEP
-            }
+            for (int c = 0; c < PIECES; ++c)
+                if (kt == c) store_piece(c, pl, pu);
             if (!last) {
-                lstore(buf ^ 1);
+                lstore(buf ^ 1, kt + 1);
                 __syncthreads();
                 buf ^= 1;
             }
         }
-        {
-            // ---- z[t, i, m, j]; register r of a block is row 8*(r/4) + 4*(lane/32) + r%4.
-            // Issued while the first K-step of the next tile is on its way.
-            int q = tile;
-            const int j0 = (q % tj) * TJ;  q /= tj;
-            const int i0 = (q % ti) * TI;  q /= ti;
-            const int m = q % g.D, t = q / g.D;
-            const unsigned rs = (unsigned)g.D * g.Ly;                     // one step in i
-            const int ib = i0 + wi * 64 + 4 * fh;
-            const unsigned ob = ((unsigned)(t * g.Lx + ib) * g.D + m) * g.Ly + j0 + wj * 64 + fi;
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                if (j0 + wj * 64 + b * 32 + fi >= g.Ly) continue;
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int di = a * 32 + 8 * (r / 4) + (r % 4);
-                        if (ib + di < g.Lx) {
-                            const unsigned o = ob + di * rs + b * 32;
-                            __builtin_nontemporal_store(cl[a][b][r], &g.zlw[o]);
-                            __builtin_nontemporal_store(cu[a][b][r], &g.zuw[o]);
-                        }
-                    }
-                }
-            }
-        }
-        if (has_next) lstore(buf ^ 1);
+        for (int c = 0; c < PIECES; ++c)
+            if (c >= nk) store_piece(c, pl, pu);
+        // this tile becomes the one that leaves
+        pz = zc;
+        pfull = zc_i0 + TI <= g.Lx && zc_j0 + TJ <= g.Ly;
+        prows = zc_j0 + wj * 32 + fi < g.Ly ? g.Lx - (zc_i0 + wi * 64 + 4 * fh) : 0;
+        zc = zn;  zc_i0 = zn_i0;  zc_j0 = zn_j0;
+        if (has_next) lstore(buf ^ 1, 0);
         __syncthreads();
         buf ^= 1;
+        tiles_left -= 1;
+    };
+
+    floatx16 al_[2], au_[2], bl_[2], bu_[2];
+    for (;;) {
+        run_tile(al_, au_, bl_, bu_);
+        if (tiles_left == 0) {
+#pragma unroll
+            for (int c = 0; c < PIECES; ++c) store_piece(c, al_, au_);
+            break;
+        }
+        run_tile(bl_, bu_, al_, au_);
+        if (tiles_left == 0) {
+#pragma unroll
+            for (int c = 0; c < PIECES; ++c) store_piece(c, bl_, bu_);
+            break;
+        }
     }
 }
 
@@ -411,14 +571,25 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
 
     const bool fast = (d % 4 == 0) && (!VP || Ly % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
                       faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
-                      faith::aligned(y_l, 16) && faith::aligned(y_u, 16) && nw < 0xffffffffLL && nx < 0xffffffffLL &&
-                      ny < 0xffffffffLL;
+                      faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
+                      (long long)TI * D * (d > Ly ? d : Ly) * 4 < 0xffffffffLL &&    // 32-bit offsets inside a tile
+                      (!VP || (long long)d * D * Ly * 4 < 0xffffffffLL);             // and along K inside a head
     if (fast) {
         const long long tiles = (long long)B * D * ((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ);
         FAITH_REQUIRE(tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: too many tiles", who);
         const long long resident = 2LL * faith::compute_units();      // 56 KB of LDS each: two per CU
-        hipLaunchKernelGGL(dot_w<VP>, dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(NTHREADS), 0, st, g,
-                           (int)tiles);
+        // the XCD-aware walk deals perturbation coordinates m over the XCDs: needs dim_in % 8 == 0 and
+        // a grid that keeps workgroup number % 8 fixed along a walk
+        long long grid = tiles < resident ? tiles : resident;
+        int xcd_map = 0;
+        if (D % 8 == 0 && grid >= 8) {
+            grid -= grid % 8;
+            xcd_map = 1;
+        }
+        if (d % BK == 0)
+            hipLaunchKernelGGL((dot_w<VP, false>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
+        else
+            hipLaunchKernelGGL((dot_w<VP, true>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
     } else {
         const long long blocks = (nw + 255) / 256;
         hipLaunchKernelGGL(dot_w_simple<VP>, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
