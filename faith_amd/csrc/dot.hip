@@ -32,8 +32,9 @@
 //   * bounds predicates exist only on the paths for ragged tiles and a ragged last K-step.
 //
 // The reduction is short (d = 64 is eight K-steps), so a tile's 64 KB of results would otherwise
-// leave in a burst during which no MFMA issues.  Each wavefront therefore holds TWO accumulator
-// sets: while tile n accumulates in one, tile n-1 leaves from the other, eight rows per K-step.
+// leave in a burst during which no MFMA issues.  Each wavefront therefore holds TWO register sets:
+// a finished tile is moved aside (32 v_mov_b64) and leaves from there, eight rows per K-step,
+// while the next tile accumulates.
 //
 // The constant terms z_lb / z_ub ([Lx, Ly] per head, 1/D_in of the work, O(1) cancelling terms)
 // are summed in double by a small kernel.
@@ -119,9 +120,12 @@ struct Walk {
 //   and so are its concrete bounds [B, d, Ly].  The y-side tiles are then staged as [k][j]
 //   (16-byte loads along j, conflict-free) and their fragments read with four 4-byte LDS reads.
 //
-// RAGGED = true: d % 8 == 4, half of the last K-step lies past d.  Threads past d then read their
-// K-step-0 element instead (in bounds) and discard it before it reaches LDS.
-template <bool VP, bool RAGGED>
+//
+// EXACT = true: d % 8 == 0, Lx % 128 == 0 and Ly % 64 == 0, so no access needs a predicate and a
+// K-step is straight-line code.  EXACT = false: when d % 8 == 4, half of the last K-step lies past
+// d; threads past d then read their K-step-0 element instead (in bounds) and discard it before it
+// reaches LDS; rows and columns of ragged tiles are stored under a per-lane predicate.
+template <bool VP, bool EXACT>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     __shared__ float sm[2][STAGE];
@@ -129,6 +133,7 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     const int ti = (g.Lx + TI - 1) / TI, tj = (g.Ly + TJ - 1) / TJ;
     const int d = g.d;
     const int nk = (d + BK - 1) / BK;
+    constexpr bool RAGGED = !EXACT;                        // the last K-step may be half empty
 
     const int tid = threadIdx.x;
     const int lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -272,7 +277,7 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         }
         return *reinterpret_cast<const float4 *>(s + o + fy);
     };
-    auto compute = [&](int buf, floatx16 (&cl)[2], floatx16 (&cu)[2]) {
+    auto compute = [&](int buf, floatx16 (&cl)[2], floatx16 (&cu)[2], auto &&after_quarter) {
         const float *s = sm[buf];
         float4 xl[2], xu[2], bp[2], bn[2];
 #pragma unroll
@@ -305,8 +310,11 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         cu[a] = mfma(bn[a].c, yl.c, cu[a]);                 \
     }
         FAITH_DOT_STEP(x)
+        after_quarter(0);
         FAITH_DOT_STEP(y)
+        after_quarter(1);
         FAITH_DOT_STEP(z)
+        after_quarter(2);
         FAITH_DOT_STEP(w)
 #undef FAITH_DOT_STEP
     };
@@ -319,18 +327,19 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     const unsigned rsb = (unsigned)g.D * g.Ly * 4u;        // one step in i, bytes
     const unsigned lane_off = (unsigned)(wi * 64 + 4 * fh) * rsb + (wj * 32 + fi) * 4u;
     size_t pz = 0;                                         // finished tile: its first element
-    bool pfull = false;                                    // it lies wholly inside z
-    int prows = 0;                                         // else: rows this lane may store (0: none, the state
-                                                           // before the first tile has finished)
-    auto store_piece = [&](int c, const floatx16 (&pl)[2], const floatx16 (&pu)[2]) {
+    unsigned pbytes = 0;                                   // bytes from there to the end of z; 0 before the first
+                                                           // tile has finished: the hardware drops those stores
+    int prows = 0;                                         // !EXACT: rows this lane may store (0: none)
+    // rows r0 .. r1-1 of piece c
+    auto store_piece = [&](int c, const floatx16 (&pl)[2], const floatx16 (&pu)[2], int r0 = 0, int r1 = 4) {
         const int a = c / 4, q4 = c % 4;
-        const unsigned nz = clamp32((tot_z - pz) * 4);
-        const __amdgpu_buffer_rsrc_t rl = window(g.zlw + pz, nz), ru = window(g.zuw + pz, nz);
+        const __amdgpu_buffer_rsrc_t rl = window(g.zlw + pz, pbytes), ru = window(g.zuw + pz, pbytes);
         unsigned step_b = rsb;
         asm volatile("" : "+s"(step_b));                   // keeps 32 row offsets from being hoisted and held
-        if (pfull) {
+        if (EXACT) {
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
+                if (rr < r0 || rr >= r1) continue;
                 const unsigned row = (a * 32 + 8 * q4 + rr) * step_b;
                 st1_nt(pl[a][4 * q4 + rr], rl, lane_off, row);
                 st1_nt(pu[a][4 * q4 + rr], ru, lane_off, row);
@@ -340,7 +349,7 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
             asm volatile("" : "+v"(rows));                 // likewise 32 row predicates
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
-                if (a * 32 + 8 * q4 + rr < rows) {
+                if (rr >= r0 && rr < r1 && a * 32 + 8 * q4 + rr < rows) {
                     const unsigned row = (a * 32 + 8 * q4 + rr) * step_b;
                     st1_nt(pl[a][4 * q4 + rr], rl, lane_off, row);
                     st1_nt(pu[a][4 * q4 + rr], ru, lane_off, row);
@@ -356,61 +365,77 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     __syncthreads();
     int buf = 0;
 
-    // one tile into (cl, cu) while the previous one leaves from (pl, pu)
-    auto run_tile = [&](floatx16 (&cl)[2], floatx16 (&cu)[2], const floatx16 (&pl)[2], const floatx16 (&pu)[2]) {
+    // One K-step that is not the last of its tile: fetch the next step, multiply this one, let one piece
+    // of the previous tile go (`piece` is a constant after unrolling; with_piece = false: none),
+    // stage the fetched step.  Straight-line when EXACT, so that loads, stores and scalar work can sit
+    // between the MFMAs; the staging must stay behind them (it waits for the fetch).
+    floatx16 cl[2], cu[2], ol[2], ou[2];                   // accumulating tile; finished tile on its way out
+    auto inner_step = [&](int kt, bool with_piece, int piece) {
+        load_step(kt + 1);
+        __builtin_amdgcn_sched_barrier(0);                 // the fetch goes first
+        compute(buf, cl, cu, [&](int quarter) {
+            // the piece leaves in two halves, after the second and the third quarter of the MFMAs
+            // (behind the last MFMA it costs 2 % more); the fences also keep the compiler from moving
+            // the staging below up into the MFMAs, where it would wait for the fetch
+            __builtin_amdgcn_sched_barrier(0);
+            if (with_piece && quarter == 1) store_piece(piece, ol, ou, 0, 2);
+            if (with_piece && quarter == 2) store_piece(piece, ol, ou, 2, 4);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        lstore(buf ^ 1, kt + 1);
+        __syncthreads();
+        buf ^= 1;
+    };
+
+    for (; tiles_left > 0; --tiles_left) {
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) cl[a][r] = cu[a][r] = 0.f;
         const bool has_next = tiles_left > 1;
-        for (int kt = 0; kt < nk; ++kt) {
-            const bool last = kt + 1 == nk;
-            // ONE load site for "next K-step" and "first K-step of the next tile": two sites would
-            // land in different registers and be reconciled by copies that wait for the loads
-            if (last && has_next) {
-                cur = advance(cur);
-                point_at(cur);
-            }
-            if (!last || has_next) load_step(last ? 0 : kt + 1);
-            compute(buf, cl, cu);
+        const int inner = nk - 1;
+        // pieces 0 .. 6 leave during the first seven K-steps when the tile has that many before its
+        // last one (d >= 64); shorter reductions are dominated by their stores anyway
+        const bool trickle = inner >= PIECES - 1;
+        int kt = 0;
+        if (trickle) {
 #pragma unroll
-            for (int c = 0; c < PIECES; ++c)
-                if (kt == c) store_piece(c, pl, pu);
-            if (!last) {
-                lstore(buf ^ 1, kt + 1);
-                __syncthreads();
-                buf ^= 1;
-            }
+            for (int c = 0; c < PIECES - 1; ++c) inner_step(c, true, c);
+            kt = PIECES - 1;
         }
+        for (; kt < inner; ++kt) inner_step(kt, false, 0);
+        // last K-step: the fetch is the first step of the next tile
+        if (has_next) {
+            cur = advance(cur);
+            point_at(cur);
+            load_step(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        compute(buf, cl, cu, [](int) {});
+        if (trickle) {
+            store_piece(PIECES - 1, ol, ou);
+        } else {
 #pragma unroll
-        for (int c = 0; c < PIECES; ++c)
-            if (c >= nk) store_piece(c, pl, pu);
+            for (int c = 0; c < PIECES; ++c) store_piece(c, ol, ou);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         // this tile becomes the one that leaves
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            ol[a] = cl[a];
+            ou[a] = cu[a];
+        }
         pz = zc;
-        pfull = zc_i0 + TI <= g.Lx && zc_j0 + TJ <= g.Ly;
+        pbytes = clamp32((tot_z - zc) * 4);
         prows = zc_j0 + wj * 32 + fi < g.Ly ? g.Lx - (zc_i0 + wi * 64 + 4 * fh) : 0;
         zc = zn;  zc_i0 = zn_i0;  zc_j0 = zn_j0;
         if (has_next) lstore(buf ^ 1, 0);
         __syncthreads();
         buf ^= 1;
-        tiles_left -= 1;
-    };
-
-    floatx16 al_[2], au_[2], bl_[2], bu_[2];
-    for (;;) {
-        run_tile(al_, au_, bl_, bu_);
-        if (tiles_left == 0) {
-#pragma unroll
-            for (int c = 0; c < PIECES; ++c) store_piece(c, al_, au_);
-            break;
-        }
-        run_tile(bl_, bu_, al_, au_);
-        if (tiles_left == 0) {
-#pragma unroll
-            for (int c = 0; c < PIECES; ++c) store_piece(c, bl_, bu_);
-            break;
-        }
     }
+#pragma unroll
+    for (int c = 0; c < PIECES; ++c) store_piece(c, ol, ou);
 }
 
 // Any-shape coefficient kernel (d not a multiple of 4, unaligned pointers): one thread per
@@ -586,10 +611,10 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
             grid -= grid % 8;
             xcd_map = 1;
         }
-        if (d % BK == 0)
-            hipLaunchKernelGGL((dot_w<VP, false>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
-        else
+        if (d % BK == 0 && Lx % TI == 0 && Ly % TJ == 0)
             hipLaunchKernelGGL((dot_w<VP, true>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
+        else
+            hipLaunchKernelGGL((dot_w<VP, false>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
     } else {
         const long long blocks = (nw + 255) / 256;
         hipLaunchKernelGGL(dot_w_simple<VP>, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
