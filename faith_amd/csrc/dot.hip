@@ -471,38 +471,46 @@ __global__ void __launch_bounds__(256) dot_w_simple(const DotArgs g) {
     }
 }
 
-// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns a 16 x 16 tile of
-// (i, j) of one head, stages the seven [16 x d-chunk] operand rows in LDS and sums in double.
-constexpr int BT_T = 16, BT_K = 64;
+// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns an 8 x 8 tile of
+// (i, j) of one head; four groups of 64 threads each take a quarter of every 64-wide chunk of the
+// reduction, the seven [8 x chunk] operand rows are staged in LDS, sums are kept in double and the
+// four partial sums meet in LDS at the end.
+constexpr int BT_T = 8, BT_K = 64, BT_S = 4;
 template <bool VP>
 __global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
     __shared__ float sx[3][BT_T][BT_K + 1];     // b (= l_x), xlb, xub
     __shared__ float sy[4][BT_T][BT_K + 1];     // a_l, a_u, ylb, yub
+    __shared__ double red[2][BT_S][BT_T * BT_T];
     const int ti = (g.Lx + BT_T - 1) / BT_T, tj = (g.Ly + BT_T - 1) / BT_T;
     int pid = blockIdx.x;
     const int j0 = (pid % tj) * BT_T;  pid /= tj;
     const int i0 = (pid % ti) * BT_T;  pid /= ti;
     const int t = pid;
-    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;     // output (i0 + ty, j0 + tx)
+    const int ks = threadIdx.x / 64, o = threadIdx.x % 64;
+    const int tx = o % BT_T, ty = o / BT_T;                     // output (i0 + ty, j0 + tx)
     double sl = 0.0, su = 0.0;
     for (int k0 = 0; k0 < g.d; k0 += BT_K) {
         for (int e = threadIdx.x; e < BT_T * BT_K; e += 256) {
+            // x rows are contiguous along k; so are y rows on the scores path, while on the context path
+            // y is contiguous along j
             const int r = e / BT_K, k = e % BT_K;
-            const bool kin = k0 + k < g.d;
-            const bool xin = kin && i0 + r < g.Lx, yin = kin && j0 + r < g.Ly;
+            const bool xin = k0 + k < g.d && i0 + r < g.Lx;
             const size_t xo = (size_t)(t * g.Lx + i0 + r) * g.d + k0 + k;
-            const size_t yo = VP ? (size_t)(t * g.d + k0 + k) * g.Ly + j0 + r : (size_t)(t * g.Ly + j0 + r) * g.d + k0 + k;
             sx[0][r][k] = xin ? g.x_l[xo] : 0.f;
             sx[1][r][k] = xin ? g.xlb[xo] : 0.f;
             sx[2][r][k] = xin ? g.xub[xo] : 0.f;
-            sy[0][r][k] = yin ? g.y_l[yo] : 0.f;
-            sy[1][r][k] = yin ? g.y_u[yo] : 0.f;
-            sy[2][r][k] = yin ? g.ylb[yo] : 0.f;
-            sy[3][r][k] = yin ? g.yub[yo] : 0.f;
+            const int ry = VP ? e % BT_T : r, ky = VP ? e / BT_T : k;
+            const bool yin = k0 + ky < g.d && j0 + ry < g.Ly;
+            const size_t yo = VP ? (size_t)(t * g.d + k0 + ky) * g.Ly + j0 + ry : (size_t)(t * g.Ly + j0 + ry) * g.d + k0 + ky;
+            sy[0][ry][ky] = yin ? g.y_l[yo] : 0.f;
+            sy[1][ry][ky] = yin ? g.y_u[yo] : 0.f;
+            sy[2][ry][ky] = yin ? g.ylb[yo] : 0.f;
+            sy[3][ry][ky] = yin ? g.yub[yo] : 0.f;
         }
         __syncthreads();
-#pragma unroll 8
-        for (int k = 0; k < BT_K; ++k) {
+#pragma unroll 4
+        for (int kk = 0; kk < BT_K / BT_S; ++kk) {
+            const int k = ks * (BT_K / BT_S) + kk;
             const double bt = sx[0][ty][k], xlb = sx[1][ty][k], xub = sx[2][ty][k];
             const double al = sy[0][tx][k], au = sy[1][tx][k], ylb = sy[2][tx][k], yub = sy[3][tx][k];
             const double bp = bt > 0 ? bt : 0, bn = bt < 0 ? bt : 0;
@@ -511,11 +519,16 @@ __global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
         }
         __syncthreads();
     }
-    const int i = i0 + ty, j = j0 + tx;
-    if (i < g.Lx && j < g.Ly) {
-        const size_t o = ((size_t)t * g.Lx + i) * g.Ly + j;
-        g.zlb[o] = (float)sl;
-        g.zub[o] = (float)su;
+    red[0][ks][o] = sl;
+    red[1][ks][o] = su;
+    __syncthreads();
+    if (ks == 0) {
+        const int i = i0 + ty, j = j0 + tx;
+        if (i < g.Lx && j < g.Ly) {
+            const size_t z = ((size_t)t * g.Lx + i) * g.Ly + j;
+            g.zlb[z] = (float)(red[0][0][o] + red[0][1][o] + red[0][2][o] + red[0][3][o]);
+            g.zub[z] = (float)(red[1][0][o] + red[1][1][o] + red[1][2][o] + red[1][3][o]);
+        }
     }
 }
 
