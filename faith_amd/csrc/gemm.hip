@@ -7,19 +7,25 @@
 // A_l, A_u are the bound rows ([rows*D_in, H] for lw/uw, [rows, H] for lb/ub, both K-contiguous),
 // W is [N, H] as nn.Linear stores it, so both operands stream along K.
 //
-// The MFMA kernel can take the constant-term rows as trailing M-blocks of the same grid (as the
-// reference's CUTLASS path does: tvm_kernels/cuda_kernel/mma/mma_kernel.h:251-259), but the entry
-// point sends them to the exact-accumulation kernel below instead: they are 1/D_in of the work
-// and the only outputs whose O(1) terms cancel.
+// The reference's CUTLASS path takes the constant-term rows as trailing M-blocks of the same grid
+// (tvm_kernels/cuda_kernel/mma/mma_kernel.h:251-259); here they go to the exact-accumulation
+// kernel below instead: they are 1/D_in of the work and the only outputs whose O(1) terms cancel.
 //
 // Tiling (gfx950): workgroup = 4 wavefronts, macro-tile BM x BN = 128 x 128, K-step 16,
 // wavefront tile 64 x 64 = 2 x 2 v_mfma_f32_32x32x2_f32 blocks for EACH of C_l and C_u
 // (128 accumulator registers).  Every fragment set (A_l, A_u, W+, W-) feeds four MFMAs, so one
-// 16-byte LDS read per operand block covers four K-pairs: 6 LDS reads per 64 MFMAs.  W+ / W-
-// are formed with v_max / v_min after the LDS read; W itself is staged once, unsplit.
-// LDS rows are padded to K-step + 4 floats so that the 16-byte reads of 8 neighbouring lanes
-// fall in distinct banks.  Global -> register -> LDS staging is double-buffered: the loads of
-// K-step t+1 are in flight while step t is multiplied; one barrier per K-step.
+// 16-byte LDS read per operand block covers four K-pairs: 8 LDS reads per 64 MFMAs.
+//
+// On this part every vector-ALU instruction a wavefront issues takes its slot from the MFMA pipe,
+// so the K-loop issues almost none: W is split by sign ONCE, by the thread that stages it (W+ and
+// W- are separate LDS tiles); global addresses are buffer addresses (a wave-uniform descriptor and
+// K offset, one per-thread offset per row that never changes), and the K-step is straight-line:
+// fetch of step t+1, half the MFMAs of step t, staging of step t+1, the other half, one barrier.
+//
+// LDS: a K-step of an operand is two [128 x 8] halves; rows are 8 floats with the two 16-byte
+// pieces swapped on every other group of four rows, which makes the 16-byte stores and the
+// 16-byte fragment reads bank-conflict free without padding.  4 operands x 8 KB x 2 stages = 64 KB,
+// two workgroups per CU.
 //
 // blockIdx -> tile mapping is XCD-aware: workgroups are dealt round-robin to the 8 XCDs, so
 // the N-tiles that share an M-block (and with it A_l / A_u rows) are given ids 8 apart and
@@ -29,11 +35,14 @@
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128, BN = 128, BK = 16;
-constexpr int LDK = BK + 4;          // padded LDS row
 constexpr int NTHREADS = 256;
 constexpr int XCDS = 8;
+constexpr int HALF = 128 * 8;            // floats in one [128 x 8] half of an operand's K-step
+constexpr int OPER = 2 * HALF;           // one operand, one K-step
+constexpr int S_AL = 0, S_AU = OPER, S_WP = 2 * OPER, S_WN = 3 * OPER, STAGE = 4 * OPER;
 
 struct GemmArgs {
     const float *Al, *Au;   // [Mw, K] coefficient rows (lower, upper)
@@ -48,71 +57,102 @@ struct GemmArgs {
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
+// max(v, 0) / min(v, 0) as single instructions (fmaxf / fminf add a canonicalising v_max each)
+__device__ __forceinline__ float pos1(float v) {
+    float r;
+    asm("v_max_f32 %0, 0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+__device__ __forceinline__ float neg1(float v) {
+    float r;
+    asm("v_min_f32 %0, 0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+__device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
+__device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
 
-__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+// Accesses at or beyond `bytes` from the base are dropped by the hardware (loads return zero).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void *base, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0,
+                                             (int)((bytes >> 32) ? 0xffffffffu : (unsigned)bytes), 0x00020000);
+}
+__device__ __forceinline__ float4 ld4(__amdgpu_buffer_rsrc_t r, unsigned thread_off, unsigned uniform_off) {
+    const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, thread_off, uniform_off, 0);
+    return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
 
+// position of 16-byte piece `c` (0 / 1) of row `row` inside a [128 x 8] half
+__device__ __forceinline__ int swz(int row, int c) { return row * 8 + 4 * (c ^ ((row >> 2) & 1)); }
+
+// EXACT = true: K % 16 == 0.  Otherwise (K % 4 == 0) the last K-step is partly past K: threads past
+// it read their K-step-0 piece instead (in bounds) and discard it before it reaches LDS.
+template <bool EXACT>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 signsplit_gemm(const GemmArgs g) {
-    __shared__ float sAl[2][BM * LDK];
-    __shared__ float sAu[2][BM * LDK];
-    __shared__ float sW[2][BN * LDK];
+    __shared__ float sm[2][STAGE];
 
     // ---- tile of this workgroup
     const int tiles_n = (g.N + BN - 1) / BN;
-    const int mblk_w = (g.Mw + BM - 1) / BM;
-    const int mblk_b = (g.Mb + BM - 1) / BM;
+    const int mblks = (g.Mw + BM - 1) / BM;
     const int pid = blockIdx.x;
     const int xcd = pid % XCDS, local = pid / XCDS;
     const int m_blk = (local / tiles_n) * XCDS + xcd;
     const int n_blk = local % tiles_n;
-    if (m_blk >= mblk_w + mblk_b) return;
-    const bool brows = m_blk >= mblk_w;
-    const float *__restrict__ Al = brows ? g.Bl : g.Al;
-    const float *__restrict__ Au = brows ? g.Bu : g.Au;
-    float *__restrict__ Cl = brows ? g.Dl : g.Cl;
-    float *__restrict__ Cu = brows ? g.Du : g.Cu;
-    const int M = brows ? g.Mb : g.Mw;
-    const int m0 = (brows ? m_blk - mblk_w : m_blk) * BM;
-    const int n0 = n_blk * BN;
+    if (m_blk >= mblks) return;
+    const int M = g.Mw;
+    const int m0 = m_blk * BM, n0 = n_blk * BN;
     const int K = g.K;
 
     const int tid = threadIdx.x;
-    const int lane = tid % 64, wv = tid / 64;
+    const int lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wv / 2, wn = wv % 2;            // 2 x 2 wavefronts, 64 x 64 each
 
-    // ---- staging: a tile is 128 rows x 16 floats = 512 float4, two per thread per operand
-    const int kq = tid % 4;                        // which float4 of the 16-float row
-    const int r0 = tid / 4;                        // rows r0 and r0 + 64
-    size_t offA[2], offW[2];
+    // ---- staging: an operand's K-step is 128 rows x 16 floats = 512 float4, two per thread:
+    // piece kq of rows r0 and r0 + 64.  Offsets are relative to the first row of the tile (the entry
+    // point checks that 128 rows span less than 4 GB); rows past the end re-read the last row, their
+    // products are never stored.
+    const int kq = tid % 4, r0 = tid / 4;
+    const __amdgpu_buffer_rsrc_t wal = window(g.Al + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
+    const __amdgpu_buffer_rsrc_t wau = window(g.Au + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
+    const __amdgpu_buffer_rsrc_t ww = window(g.W + (size_t)n0 * K, ((size_t)(g.N - n0) * K) * 4);
+    unsigned va[2], vw[2];
+    int dst[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int ra = min(m0 + r0 + 64 * i, M - 1);       // rows past the end re-read the last row;
-        const int rw = min(n0 + r0 + 64 * i, g.N - 1);     // their products are never stored
-        offA[i] = (size_t)ra * K + kq * 4;
-        offW[i] = (size_t)rw * K + kq * 4;
+        const int ra = min(r0 + 64 * i, M - 1 - m0);
+        const int rw = min(r0 + 64 * i, g.N - 1 - n0);
+        va[i] = ((unsigned)ra * K + kq * 4) * 4u;
+        vw[i] = ((unsigned)rw * K + kq * 4) * 4u;
+        dst[i] = (kq / 2) * HALF + swz(r0 + 64 * i, kq % 2);
     }
+    const int nk = (K + BK - 1) / BK;
     float4 pal[2], pau[2], pw[2];
+    auto past = [&](int kt) { return !EXACT && kt * BK + kq * 4 >= K; };
     auto gload = [&](int kt) {
-        const int k = kt * BK;
-        const bool in = k + kq * 4 < K;            // K % 4 == 0: a float4 is all in or all out
+        const unsigned k = kt * (BK * 4u);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            if (in) {
-                pal[i] = ld4(Al + offA[i] + k);
-                pau[i] = ld4(Au + offA[i] + k);
-                pw[i] = ld4(g.W + offW[i] + k);
+            if (EXACT) {
+                pal[i] = ld4(wal, va[i], k);
+                pau[i] = ld4(wau, va[i], k);
+                pw[i] = ld4(ww, vw[i], k);
             } else {
-                pal[i] = pau[i] = pw[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                const unsigned kk = past(kt) ? 0u : k;
+                pal[i] = ld4(wal, va[i] + kk, 0);
+                pau[i] = ld4(wau, va[i] + kk, 0);
+                pw[i] = ld4(ww, vw[i] + kk, 0);
             }
         }
     };
-    auto lstore = [&](int buf) {
+    auto lstore = [&](int buf, int kt) {
+        float *s = sm[buf];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int o = (r0 + 64 * i) * LDK + kq * 4;
-            *reinterpret_cast<float4 *>(&sAl[buf][o]) = pal[i];
-            *reinterpret_cast<float4 *>(&sAu[buf][o]) = pau[i];
-            *reinterpret_cast<float4 *>(&sW[buf][o]) = pw[i];
+            if (past(kt)) pal[i] = pau[i] = pw[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4 *>(s + S_AL + dst[i]) = pal[i];
+            *reinterpret_cast<float4 *>(s + S_AU + dst[i]) = pau[i];
+            *reinterpret_cast<float4 *>(s + S_WP + dst[i]) = pos4(pw[i]);
+            *reinterpret_cast<float4 *>(s + S_WN + dst[i]) = neg4(pw[i]);
         }
     };
 
@@ -124,28 +164,26 @@ signsplit_gemm(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
 
-    // fragment addresses: lane (i = lane % 32, h = lane / 32) reads k = 8*ks + 4*h .. +3 of row i
+    // fragments: lane (fi = lane % 32, fh = lane / 32) reads k = 8*ks + 4*fh .. +3 of row fi
     const int fi = lane % 32, fh = lane / 32;
-    const int fa = (wm * 64 + fi) * LDK + fh * 4;
-    const int fw = (wn * 64 + fi) * LDK + fh * 4;
-
-    const int nk = (K + BK - 1) / BK;
-    gload(0);
-    lstore(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) gload(kt + 1);
+    int fa[2], fw[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        fa[s] = swz(wm * 64 + s * 32 + fi, fh);
+        fw[s] = swz(wn * 64 + s * 32 + fi, fh);
+    }
+    auto compute = [&](int buf, auto &&halfway) {
+        const float *s = sm[buf];
 #pragma unroll
         for (int ks = 0; ks < BK / 8; ++ks) {
+            if (ks == 1) halfway();
             float4 al[2], au[2], wp[2], wq[2];
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                al[s] = *reinterpret_cast<const float4 *>(&sAl[buf][fa + s * 32 * LDK + ks * 8]);
-                au[s] = *reinterpret_cast<const float4 *>(&sAu[buf][fa + s * 32 * LDK + ks * 8]);
-                const float4 w = *reinterpret_cast<const float4 *>(&sW[buf][fw + s * 32 * LDK + ks * 8]);
-                wp[s] = make_float4(fmaxf(w.x, 0.f), fmaxf(w.y, 0.f), fmaxf(w.z, 0.f), fmaxf(w.w, 0.f));
-                wq[s] = make_float4(fminf(w.x, 0.f), fminf(w.y, 0.f), fminf(w.z, 0.f), fminf(w.w, 0.f));
+            for (int t = 0; t < 2; ++t) {
+                al[t] = *reinterpret_cast<const float4 *>(s + S_AL + ks * HALF + fa[t]);
+                au[t] = *reinterpret_cast<const float4 *>(s + S_AU + ks * HALF + fa[t]);
+                wp[t] = *reinterpret_cast<const float4 *>(s + S_WP + ks * HALF + fw[t]);
+                wq[t] = *reinterpret_cast<const float4 *>(s + S_WN + ks * HALF + fw[t]);
             }
 #define FAITH_STEP(c)                                                           \
     _Pragma("unroll") for (int a = 0; a < 2; ++a) _Pragma("unroll") for (int b = 0; b < 2; ++b) { \
@@ -162,16 +200,32 @@ signsplit_gemm(const GemmArgs g) {
             FAITH_STEP(w)
 #undef FAITH_STEP
         }
-        if (kt + 1 < nk) lstore(buf ^ 1);
+    };
+
+    gload(0);
+    lstore(0, 0);
+    __syncthreads();
+    int buf = 0;
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+        gload(kt + 1);
+        __builtin_amdgcn_sched_barrier(0);         // the fetch goes first: it has the whole step to arrive
+        compute(buf, [&]() {
+            // staging between the two halves of the MFMAs costs less of them than staging behind the
+            // last one (measured: 0.7 %); the fetch has had half a step (64 MFMAs) to arrive
+            __builtin_amdgcn_sched_barrier(0);
+            lstore(buf ^ 1, kt + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        });
         __syncthreads();
+        buf ^= 1;
     }
+    compute(buf, []() {});
 
     // ---- epilogue: register r of a 32x32 block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
         const int col = n0 + wn * 64 + b * 32 + fi;
         if (col >= g.N) continue;
-        const float add = (brows && g.bias) ? g.bias[col] : 0.f;
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
 #pragma unroll
@@ -179,8 +233,8 @@ signsplit_gemm(const GemmArgs g) {
                 const int row = m0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (row < M) {
                     const size_t o = (size_t)row * g.N + col;
-                    __builtin_nontemporal_store(cl[a][b][r] + add, &Cl[o]);
-                    __builtin_nontemporal_store(cu[a][b][r] + add, &Cu[o]);
+                    __builtin_nontemporal_store(cl[a][b][r], &g.Cl[o]);
+                    __builtin_nontemporal_store(cu[a][b][r], &g.Cu[o]);
                 }
             }
         }
@@ -252,7 +306,7 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
     GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
-                      faith::aligned(x_lb, 16) && faith::aligned(x_ub, 16) && faith::aligned(W, 16);
+                      faith::aligned(W, 16) && (long long)BM * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
         GemmArgs gw = g;
@@ -260,7 +314,10 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
         const long long mblks = (mw + BM - 1) / BM;
         const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + BN - 1) / BN);
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
-        hipLaunchKernelGGL(signsplit_gemm, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
+        if (dim_out % BK == 0)
+            hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
+        else
+            hipLaunchKernelGGL(signsplit_gemm<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
         GemmArgs gb = g;
         gb.Mw = 0;
         const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);

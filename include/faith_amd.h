@@ -50,7 +50,7 @@ int faith_version(void);
  * Process-wide, not thread-safe; results never depend on it, only speed.
  */
 #define FAITH_TUNE_ACT_VARIANT   0   /* tile shape of the natural-layout relaxation kernels */
-#define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split MFMA contraction       */
+#define FAITH_TUNE_GEMM_VARIANT  1   /* reserved (the MFMA contraction has one variant)     */
 #define FAITH_TUNE_COUNT         4
 int faith_tune_set(int knob, int value);
 
