@@ -182,19 +182,35 @@ conv_signsplit(const ConvArgs g) {
 
 // ------------------------------------------------------------------ 3x3, stride 1 fast path
 // Same tiling with every extent a compile-time constant (patch 6 x 34, weight rows of 36 + 1),
-// plus a register prefetch across chunks: the global loads of chunk c+1 are issued before the
-// MFMAs of chunk c and land in LDS after them, so their latency is covered by 288 MFMAs per
-// wavefront instead of being exposed at the head of every chunk.  Needs C_in % 4 == 0 and a
-// 16-byte aligned weight pointer (float4 weight loads).
+// LDS double-buffered and a register prefetch across chunks: the global loads of chunk c+1 are
+// issued before the MFMAs of chunk c, land in the other LDS buffer halfway through them, and ONE
+// barrier per chunk (288 MFMAs per wavefront) publishes them.  Global addresses are buffer
+// addresses: the per-thread offsets are fixed for the whole reduction, the chunk advances the
+// wave-uniform base, and a patch element that lies in the padding carries an offset past the end of
+// the buffer, which the hardware answers with zero -- no predicate, no select.
+// Needs C_in % 4 == 0 and a 16-byte aligned weight pointer (float4 weight loads).
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void *base, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0,
+                                             (int)((bytes >> 32) ? 0xffffffffu : (unsigned)bytes), 0x00020000);
+}
+// max(v, 0) / min(v, 0) as single instructions (fmaxf / fminf add a canonicalising v_max each).
+// As a median of three, which the compiler knows to be a vector-ALU write: inline assembly would
+// hide that from its hazard recognizer, and the MFMA that reads the result next would not get the
+// wait states it needs.
+__device__ __forceinline__ float pos1(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, __builtin_inff()); }
+__device__ __forceinline__ float neg1(float v) { return __builtin_amdgcn_fmed3f(v, -__builtin_inff(), 0.f); }
+
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 conv_signsplit_k3s1(const ConvArgs g) {
     constexpr int K = 3, KK = 9, PROW = TR - 1 + K, PCOL = TC - 1 + K, PP = PROW * PCOL;   // 6, 34, 204
     constexpr int WS = CC * KK + 1;                      // 37
     constexpr int NP = (CC * PP + NTHREADS - 1) / NTHREADS;          // patch elements per thread and bound: 4
     constexpr int NW4 = (TCO * CC * KK / 4 + NTHREADS - 1) / NTHREADS;   // weight float4 per thread: 5
-    __shared__ float sXl[CC * PP];
-    __shared__ float sXu[CC * PP];
-    __shared__ float sW[TCO * WS];
+    constexpr unsigned NOWHERE = 0xfffffff0u;            // a buffer offset the hardware answers with zero
+    __shared__ float sXl[2][CC * PP];
+    __shared__ float sXu[2][CC * PP];
+    __shared__ float sW[2][TCO * WS];
 
     const int tcol = (g.Wo + TC - 1) / TC, trow = (g.Ho + TR - 1) / TR, tco = (g.Co + TCO - 1) / TCO;
     int pid = blockIdx.x;
@@ -210,58 +226,67 @@ conv_signsplit_k3s1(const ConvArgs g) {
 
     const int ih0 = oh0 - g.P, iw0 = ow0 - g.P;
     const int img = g.H * g.W;
-    const float *xl_n = g.xl + (size_t)n * g.Ci * img;
-    const float *xu_n = g.xu + (size_t)n * g.Ci * img;
+    // one image of x (the entry point checks that it spans less than 4 GB) and the weight rows of this
+    // channel block
+    const size_t image = (size_t)g.Ci * img;
+    const float *xl_n = g.xl + n * image, *xu_n = g.xu + n * image;
+    const float *w_blk = g.w + (size_t)co0 * g.Ci * KK;
+    const size_t w_bytes = (size_t)(g.Co - co0) * g.Ci * KK * 4;
 
-    // ---- staging plan, fixed for the whole reduction
-    int poff[NP];                                        // offset inside a 4-channel slab, -1 = zero
+    // ---- staging plan, fixed for the whole reduction: byte offsets inside a 4-channel slab
+    unsigned poff[NP];
 #pragma unroll
     for (int u = 0; u < NP; ++u) {
         const int e = tid + u * NTHREADS;
         const int ci = e / PP, r2 = e % PP, pr = r2 / PCOL, pc = r2 % PCOL;
         const int ih = ih0 + pr, iw = iw0 + pc;
         const bool ok = e < CC * PP && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
-        poff[u] = ok ? ci * img + ih * g.W + iw : -1;
+        poff[u] = ok ? (unsigned)(ci * img + ih * g.W + iw) * 4u : NOWHERE;
     }
-    int wsrc[NW4], wdst[NW4];
+    unsigned wsrc[NW4];
+    int wdst[NW4];
 #pragma unroll
     for (int u = 0; u < NW4; ++u) {
         const int e = tid + u * NTHREADS;
         const int co = e / 9, f = e % 9;
         const bool ok = e < TCO * 9;
-        wsrc[u] = ok ? min(co0 + co, g.Co - 1) * g.Ci * KK + f * 4 : -1;     // rows past C_out are never stored
-        wdst[u] = co * WS + f * 4;
+        // rows past C_out re-read the last row; they are never stored
+        wsrc[u] = ok ? (unsigned)(min(co, g.Co - 1 - co0) * g.Ci * KK + f * 4) * 4u : NOWHERE;
+        wdst[u] = ok ? co * WS + f * 4 : -1;
     }
     float pxl[NP], pxu[NP];
     float4 pw[NW4];
     auto prefetch = [&](int c0) {
-        const float *xl = xl_n + (size_t)c0 * img, *xu = xu_n + (size_t)c0 * img;
-        const float *w = g.w + c0 * KK;
+        const __amdgpu_buffer_rsrc_t rl = window(xl_n, image * 4), ru = window(xu_n, image * 4);
+        const __amdgpu_buffer_rsrc_t rw = window(w_blk, w_bytes);
+        const unsigned cx = (unsigned)c0 * img * 4u, cw = (unsigned)c0 * KK * 4u;
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
-            pxl[u] = poff[u] >= 0 ? xl[poff[u]] : 0.f;
-            pxu[u] = poff[u] >= 0 ? xu[poff[u]] : 0.f;
+            pxl[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, poff[u], cx, 0));
+            pxu[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ru, poff[u], cx, 0));
         }
 #pragma unroll
-        for (int u = 0; u < NW4; ++u)
-            pw[u] = wsrc[u] >= 0 ? *reinterpret_cast<const float4 *>(w + wsrc[u]) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int u = 0; u < NW4; ++u) {
+            const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rw, wsrc[u], cw, 0);
+            pw[u] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+        }
     };
-    auto commit = [&]() {
+    auto commit = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
             const int e = tid + u * NTHREADS;
             if (e < CC * PP) {
-                sXl[e] = pxl[u];
-                sXu[e] = pxu[u];
+                sXl[buf][e] = pxl[u];
+                sXu[buf][e] = pxu[u];
             }
         }
 #pragma unroll
         for (int u = 0; u < NW4; ++u) {
-            if (wsrc[u] >= 0) {
-                sW[wdst[u] + 0] = pw[u].x;
-                sW[wdst[u] + 1] = pw[u].y;
-                sW[wdst[u] + 2] = pw[u].z;
-                sW[wdst[u] + 3] = pw[u].w;
+            if (wdst[u] >= 0) {
+                sW[buf][wdst[u] + 0] = pw[u].x;
+                sW[buf][wdst[u] + 1] = pw[u].y;
+                sW[buf][wdst[u] + 2] = pw[u].z;
+                sW[buf][wdst[u] + 3] = pw[u].w;
             }
         }
     };
@@ -280,47 +305,58 @@ conv_signsplit_k3s1(const ConvArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
 
-    prefetch(0);
-    for (int c0 = 0; c0 < g.Ci; c0 += CC) {
-        commit();
-        __syncthreads();
-        if (c0 + CC < g.Ci) prefetch(c0 + CC);
+    // the MFMAs of one channel pair (cp) of the chunk in LDS buffer `buf`
+    auto multiply = [&](int buf, int cp) {
 #pragma unroll
-        for (int cp = 0; cp < CC / 2; ++cp) {
+        for (int tap = 0; tap < KK; ++tap) {
+            const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
+            const int wo = cp * KK + tap;
+            float wp[2], wq[2], xl[2], xu[2];
 #pragma unroll
-            for (int tap = 0; tap < KK; ++tap) {
-                const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
-                const int wo = cp * KK + tap;
-                float wp[2], wq[2], xl[2], xu[2];
+            for (int a = 0; a < 2; ++a) {
+                const float w = sW[buf][woff[a] + wo];
+                wp[a] = pos1(w);
+                wq[a] = neg1(w);
+            }
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    const float w = sW[woff[a] + wo];
-                    wp[a] = fmaxf(w, 0.f);
-                    wq[a] = fminf(w, 0.f);
-                }
+            for (int b = 0; b < 2; ++b) {
+                xl[b] = sXl[buf][xoff[b] + xo];
+                xu[b] = sXu[buf][xoff[b] + xo];
+            }
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
 #pragma unroll
                 for (int b = 0; b < 2; ++b) {
-                    xl[b] = sXl[xoff[b] + xo];
-                    xu[b] = sXu[xoff[b] + xo];
+                    cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
+                    cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
                 }
 #pragma unroll
-                for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < 2; ++a)
 #pragma unroll
-                    for (int b = 0; b < 2; ++b) {
-                        cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
-                        cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
-                    }
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int b = 0; b < 2; ++b) {
-                        cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
-                        cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
-                    }
-            }
+                for (int b = 0; b < 2; ++b) {
+                    cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
+                    cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                }
         }
+    };
+
+    prefetch(0);
+    commit(0);
+    __syncthreads();
+    int buf = 0;
+    for (int c0 = 0; c0 + CC < g.Ci; c0 += CC) {
+        prefetch(c0 + CC);
+        __builtin_amdgcn_sched_barrier(0);         // the fetch goes first
+        multiply(buf, 0);
+        __builtin_amdgcn_sched_barrier(0);         // staging between the two halves of the MFMAs
+        commit(buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(buf, 1);
         __syncthreads();
+        buf ^= 1;
     }
+    multiply(buf, 0);
+    multiply(buf, 1);
 
     const int ow = ow0 + fi;
     if (ow >= g.Wo) return;
@@ -429,7 +465,8 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
     const long long grid = (long long)dim_in * ((COUT + TCO - 1) / TCO) * ((Ho + TR - 1) / TR) * ((Wo + TC - 1) / TC);
     FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_convolution_verification: grid too large");
     const bool k3s1 = K == 3 && Stride == 1 && CIN % 4 == 0 && faith::aligned(W, 16) &&
-                      (long long)CIN * Height * Width < 0x7fffffffLL && (long long)COUT * CIN * 9 < 0x7fffffffLL;
+                      (long long)CIN * Height * Width * 4 < 0xfffffff0LL &&      // 32-bit byte offsets inside an image
+                      (long long)128 * CIN * 9 * 4 + (long long)CIN * 9 * 4 < 0xfffffff0LL;   // and inside a block of weight rows
     if (k3s1)
         hipLaunchKernelGGL(conv_signsplit_k3s1, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
     else
