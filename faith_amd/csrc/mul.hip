@@ -168,6 +168,127 @@ __global__ void __launch_bounds__(NTHREADS) mul_natural(const MulArgs a) {
     }
 }
 
+// The common shape, straight-line: D_in <= RG * RPT (all four coefficient tensors of the tile stay
+// in registers), D_in a multiple of RG, H a multiple of the tile width, 16-byte aligned.  Row
+// existence is then a scalar branch and there are neither column predicates nor a second pass.
+template <int Q, int TPR, int NTHREADS, int RPT>
+__global__ void __launch_bounds__(NTHREADS) mul_resident(const MulArgs a) {
+    constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
+    static_assert(TH <= WAVE, "one lane per neuron in wavefront 0");
+    extern __shared__ float smem[];
+    float *part = smem;                          // [words][NW][4][TH]: x.lw, x.uw, y.lw, y.uw partial norms
+    float *coef = part + a.words * NW * 4 * TH;  // [3][TH]: a_l, a_u, b
+
+    const int tiles = a.H / TH;
+    const int r = blockIdx.x / tiles, col0 = (blockIdx.x % tiles) * TH;
+    const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
+    const int c = tid % TPR, rg = tid / TPR;
+    const size_t base = ((size_t)r * a.D + rg) * a.H + col0 + c * VEC;
+    const size_t row_step = (size_t)RG * a.H;
+    const float *__restrict__ src[4] = {a.xlw + base, a.xuw + base, a.ylw + base, a.yuw + base};
+
+    Vec<VEC> d[4][RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (i * RG < a.D)
+                d[t][i].load(src[t] + i * row_step);
+            else
+                d[t][i].zero();
+        }
+    }
+    const int blk = a.D / a.words;
+    for (int w = 0; w < a.words; ++w) {
+        const int lo_row = w * blk, hi_row = lo_row + blk;
+        float pn[4][VEC];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) pn[t][v] = 0.f;
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            const int row = i * RG + rg;
+            if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v));
+            }
+        }
+#pragma unroll
+        for (int m = TPR; m < WAVE; m <<= 1)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) pn[t][v] = ncomb<Q>(pn[t][v], __shfl_xor(pn[t][v], m, WAVE));
+        if (lane < TPR) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) part[((w * NW + wv) * 4 + t) * TH + c * VEC + v] = pn[t][v];
+        }
+    }
+    __syncthreads();
+
+    // one lane per neuron: both concretizations (Bounds.py:611-612), planes, constant terms
+    if (wv == 0 && lane < TH) {
+        const size_t bi = (size_t)r * a.H + col0 + lane;
+        const float xlb = a.xlb[bi], xub = a.xub[bi], ylb = a.ylb[bi], yub = a.yub[bi];
+        float lx = xlb, ly = ylb, uy = yub;
+        for (int w = 0; w < a.words; ++w) {
+            float n[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int g = 0; g < NW; ++g)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) n[t] = ncomb<Q>(n[t], part[((w * NW + g) * 4 + t) * TH + lane]);
+            lx += (-a.eps) * nfin<Q>(n[0]);
+            ly += (-a.eps) * nfin<Q>(n[2]);
+            uy += a.eps * nfin<Q>(n[3]);
+        }
+        const float al = ly, au = uy, bt = lx;
+        coef[lane] = al;
+        coef[TH + lane] = au;
+        coef[2 * TH + lane] = bt;
+        // Bounds.py:631-646: ((b_src - 0) * k + gamma) then + ((b_src - 0) * k + 0)
+        const float gl = -al * bt, gu = -au * bt;
+        a.zlb[bi] = ((al > 0.f ? xlb : xub) * al + gl) + (bt > 0.f ? ylb : yub) * bt;
+        a.zub[bi] = ((au > 0.f ? xub : xlb) * au + gu) + (bt > 0.f ? yub : ylb) * bt;
+    }
+    __syncthreads();
+
+    float al[VEC], au[VEC], bt[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        al[v] = coef[c * VEC + v];
+        au[v] = coef[TH + c * VEC + v];
+        bt[v] = coef[2 * TH + c * VEC + v];
+    }
+    float *__restrict__ q_lw = a.zlw + base, *__restrict__ q_uw = a.zuw + base;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        if (i * RG < a.D) {
+            Vec<VEC> ol, ou;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                const float xl = d[0][i].get(v), xu = d[1][i].get(v), yl = d[2][i].get(v), yu = d[3][i].get(v);
+                ol.set(v, (al[v] > 0.f ? xl : xu) * al[v] + (bt[v] > 0.f ? yl : yu) * bt[v]);
+                ou.set(v, (au[v] > 0.f ? xu : xl) * au[v] + (bt[v] > 0.f ? yu : yl) * bt[v]);
+            }
+            ol.store(q_lw + i * row_step);
+            ou.store(q_uw + i * row_step);
+        }
+    }
+}
+
+template <int Q, int TPR, int NTHREADS, int RPT>
+void launch_mul_resident(const MulArgs &a, hipStream_t st) {
+    constexpr int TH = TPR * 4;
+    const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 4 * TH + 3 * TH) * sizeof(float);
+    hipLaunchKernelGGL((mul_resident<Q, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS), smem,
+                       st, a);
+}
+
 template <int Q, int VEC, int TPR, int NTHREADS, int RPT>
 void launch_mul(const MulArgs &a, hipStream_t st) {
     constexpr int TH = TPR * VEC;
@@ -182,6 +303,12 @@ void dispatch_mul(const MulArgs &a, hipStream_t st) {
     const bool vec4 = a.H % 4 == 0 && faith::aligned(a.xlw, 16) && faith::aligned(a.xuw, 16) &&
                       faith::aligned(a.ylw, 16) && faith::aligned(a.yuw, 16) && faith::aligned(a.zlw, 16) &&
                       faith::aligned(a.zuw, 16);
+    const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
+    if (vec4 && a.H % 32 == 0 && a.D % 64 == 0 && a.D <= 256 && tv != 9) {
+        // 32-neuron tiles, 512 threads holding 4 rows of each of the four tensors (64 values per thread)
+        launch_mul_resident<Q, 8, 512, 4>(a, st);
+        return;
+    }
     if (!vec4)
         launch_mul<Q, 1, 64, 256, 8>(a, st);      // 64 neurons x 32 rows per pass
     else if (a.D <= 128)
