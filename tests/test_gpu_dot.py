@@ -90,6 +90,34 @@ def test_dot_config3_reduced():
     check(as_bounds(c["x"]), as_bounds(c["y"]), c["p"], c["eps"], c["words"], "config3/4")
 
 
+@pytest.mark.parametrize("shape", [
+    # B, Lx, Ly, D, d: shapes the straight-line contraction kernel takes (d % 8 == 0, Lx % 128 == 0, Ly % 64 == 0)
+    (1, 128, 128, 8, 64),      # results of a tile leave during the next tile's first seven K-steps
+    (1, 128, 64, 4, 128),      # sixteen K-steps: unrolled seven, then the rolled loop
+    (1, 128, 64, 8, 32),       # four K-steps: too few for piecewise stores
+    (2, 128, 128, 160, 16),    # 640 tiles on 512 workgroups: a workgroup walks from one tile to the next
+    (1, 256, 128, 12, 64),     # two i-tiles; dim_in not a multiple of 8 (plain tile numbering)
+])
+def test_dot_exact_shapes_against_float64(shape):
+    """The whole result against the float64 planes (the CPU oracle's broadcast would be too large here)."""
+    from faith_amd import ops
+    B, Lx, Ly, D, d = shape
+    g = torch.Generator().manual_seed(35)
+    x = rand_bounds(g, B, Lx, D, d, ordered=False, sw=0.3, sb=1.0)
+    y = rand_bounds(g, B, Ly, D, d, ordered=False, sw=0.3, sb=1.0)
+    print(f"[case] dot exact x={tuple(x.lw.shape)} y={tuple(y.lw.shape)}", flush=True)
+    zlw, zlb, zuw, zub, (xl, xu, yl, yu) = ops.dot_product_qk(dev(x), dev(y), 2.0, 0.05, 1, return_intervals=True)
+    torch.cuda.synchronize()
+    exl, exu = O.concretize(x, 2.0, 0.05, 1)
+    eyl, eyu = O.concretize(y, 2.0, 0.05, 1)
+    assert close(xl, exl) and close(xu, exu) and close(yl, eyl) and close(yu, eyu)
+    ref, mag = dot64(x, y, 2.0, 0.05, 1)
+    tol = lambda r, m: 1e-6 + 1e-5 * r.abs() + 8 * 2.0 ** -24 * m
+    for name, got in (("lw", zlw), ("lb", zlb), ("uw", zuw), ("ub", zub)):
+        err = (got.cpu().double() - ref[name]).abs()
+        assert bool((err <= tol(ref[name], mag[name])).all()), f"{name}: max err {float(err.max()):.3g}"
+
+
 def test_dot_config3_full_size_properties():
     """Full configuration 3: soundness of the propagated planes on sampled perturbations
     (any x, y inside their bounds => x.y^T inside z's bounds), plus one head against float64."""
@@ -156,6 +184,18 @@ def test_context_shapes(shape, p):
     probs = rand_bounds(g, B, L, D, L, ordered=False, sw=0.2, sb=0.5)
     value = rand_bounds(g, B, L, D, dv, ordered=False, sw=0.3, sb=1.0)
     check_v(probs, value, p, 0.1, 1, "sweep")
+
+
+@pytest.mark.parametrize("shape", [
+    # B, queries, keys, D, value width: shapes the straight-line kernel takes on the context path
+    (1, 128, 128, 8, 64), (2, 128, 64, 16, 128), (1, 128, 32, 160, 64),
+])
+def test_context_exact_shapes(shape):
+    B, Lq, Lk, D, dv = shape
+    g = torch.Generator().manual_seed(36)
+    probs = rand_bounds(g, B, Lq, D, Lk, ordered=False, sw=0.2, sb=0.5)
+    value = rand_bounds(g, B, Lk, D, dv, ordered=False, sw=0.3, sb=1.0)
+    check_v(probs, value, 2.0, 0.05, 1, "exact")
 
 
 def test_context_rectangular_and_two_words():
