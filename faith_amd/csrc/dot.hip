@@ -438,6 +438,147 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     for (int c = 0; c < PIECES; ++c) store_piece(c, ol, ou);
 }
 
+// Short sequences (Lx, Ly <= 64, d <= 80): the 128 x 64 tile above would be mostly padding, so here
+// a WAVEFRONT owns one 32 x 32 block of z for one perturbation coordinate m (one MFMA block for
+// z_lw, one for z_uw).  The four wavefronts of a workgroup share the (head, i-block, j-block): the
+// operands that do not depend on m (b+, b-, a_l+-, a_u+-, split by sign) are staged in LDS once for
+// the whole reduction, and every wavefront walks its own `mpw` coordinates, loading its x and y
+// fragments straight from global memory in MFMA layout (rows of 32 bytes per lane and K-step: poor
+// coalescing, but these problems are a few megabytes and latency is what counts).
+constexpr int SB = 32;                         // block edge
+template <bool VP>
+__global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mpw) {
+    extern __shared__ float sh[];              // six operands, each d/8 swizzled [32 x 8] pieces
+    const int d = g.d, nq = d / 8;
+    const int OP = SB * d;                     // floats per operand
+    float *s_bp = sh, *s_bn = sh + OP, *s_alp = sh + 2 * OP, *s_aln = sh + 3 * OP, *s_aup = sh + 4 * OP, *s_aun = sh + 5 * OP;
+
+    const int nib = (g.Lx + SB - 1) / SB, njb = (g.Ly + SB - 1) / SB;
+    const int mgroups = (g.D + 4 * mpw - 1) / (4 * mpw);
+    int pid = blockIdx.x;
+    const int mg = pid % mgroups;  pid /= mgroups;
+    const int j0 = (pid % njb) * SB;  pid /= njb;
+    const int i0 = (pid % nib) * SB;  pid /= nib;
+    const int t = pid;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wv = tid / 64;
+    const int fi = lane % 32, fh = lane / 32;
+
+    // ---- operands shared by every m: b = l_x rows i0.., a_l / a_u rows (columns of z) j0..
+    for (int e = tid; e < SB * d / 4; e += 256) {
+        const int row = e / (d / 4), c4 = e % (d / 4);
+        const int dst = (c4 / 2) * (SB * 8) + swz(row, c4 % 2);
+        const float4 bt = *reinterpret_cast<const float4 *>(g.x_l + (size_t)(t * g.Lx + min(i0 + row, g.Lx - 1)) * d + c4 * 4);
+        *reinterpret_cast<float4 *>(s_bp + dst) = pos4(bt);
+        *reinterpret_cast<float4 *>(s_bn + dst) = neg4(bt);
+        if (!VP) {
+            const size_t o = (size_t)(t * g.Ly + min(j0 + row, g.Ly - 1)) * d + c4 * 4;
+            const float4 al = *reinterpret_cast<const float4 *>(g.y_l + o), au = *reinterpret_cast<const float4 *>(g.y_u + o);
+            *reinterpret_cast<float4 *>(s_alp + dst) = pos4(al);
+            *reinterpret_cast<float4 *>(s_aln + dst) = neg4(al);
+            *reinterpret_cast<float4 *>(s_aup + dst) = pos4(au);
+            *reinterpret_cast<float4 *>(s_aun + dst) = neg4(au);
+        }
+    }
+    if (VP) {
+        // a[t, k, j]: j is the contiguous axis
+        for (int e = tid; e < SB * d; e += 256) {
+            const int j = e % SB, k = e / SB;
+            const size_t o = (size_t)(t * d + k) * g.Ly + min(j0 + j, g.Ly - 1);
+            const float al = g.y_l[o], au = g.y_u[o];
+            const int dst = (k / 8) * (SB * 8) + swz(j, (k % 8) / 4) + k % 4;
+            s_alp[dst] = pos1(al);
+            s_aln[dst] = neg1(al);
+            s_aup[dst] = pos1(au);
+            s_aun[dst] = neg1(au);
+        }
+    }
+    __syncthreads();
+
+    const int frag = swz(fi, fh);              // this lane's 16 bytes inside a [32 x 8] piece
+    const int irow = min(i0 + fi, g.Lx - 1), jcol = min(j0 + fi, g.Ly - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(wv);
+    // per-lane byte offsets from the first element of (head, m); they do not depend on m
+    const unsigned vx = ((unsigned)irow * g.D * d + fh * 4) * 4u;
+    const unsigned vy = VP ? ((unsigned)(fh * 4) * g.D * g.Ly + jcol) * 4u : ((unsigned)jcol * g.D * d + fh * 4) * 4u;
+    const unsigned ykstep = (unsigned)g.D * g.Ly * 4u;             // context path: one step in k, bytes
+    const size_t head_x = (size_t)g.Lx * g.D * d, head_y = (size_t)g.Ly * g.D * d;
+    for (int s = 0; s < mpw; ++s) {
+        const int m = (mg * 4 + wave) * mpw + s;
+        if (m >= g.D) break;
+        // windows that start at (head t, coordinate m) and end with the head
+        const size_t x0 = t * head_x + (size_t)m * d, y0 = t * head_y + (size_t)m * (VP ? g.Ly : d);
+        const __amdgpu_buffer_rsrc_t wxl = window(g.xlw + x0, clamp32((head_x - (size_t)m * d) * 4));
+        const __amdgpu_buffer_rsrc_t wxu = window(g.xuw + x0, clamp32((head_x - (size_t)m * d) * 4));
+        const __amdgpu_buffer_rsrc_t wyl = window(g.ylw + y0, clamp32((head_y - (size_t)m * (VP ? g.Ly : d)) * 4));
+        const __amdgpu_buffer_rsrc_t wyu = window(g.yuw + y0, clamp32((head_y - (size_t)m * (VP ? g.Ly : d)) * 4));
+        floatx16 cl, cu;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) cl[r] = cu[r] = 0.f;
+        for (int q0 = 0; q0 < nq; q0 += 4) {
+            float4 xl[4], xu[4], yl[4], yu[4];
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq) {
+                if (q0 + qq < nq) {
+                    const unsigned k = (q0 + qq) * 8;
+                    xl[qq] = ld4(wxl, vx, k * 4u);
+                    xu[qq] = ld4(wxu, vx, k * 4u);
+                    if (VP) {
+                        // y[t, k, m, j]: four keys, one column per lane
+                        float yv[2][4];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            yv[0][c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wyl, vy, (k + c) * ykstep, 0));
+                            yv[1][c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wyu, vy, (k + c) * ykstep, 0));
+                        }
+                        yl[qq] = make_float4(yv[0][0], yv[0][1], yv[0][2], yv[0][3]);
+                        yu[qq] = make_float4(yv[1][0], yv[1][1], yv[1][2], yv[1][3]);
+                    } else {
+                        yl[qq] = ld4(wyl, vy, k * 4u);
+                        yu[qq] = ld4(wyu, vy, k * 4u);
+                    }
+                }
+            }
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq) {
+                if (q0 + qq < nq) {
+                    const int o = (q0 + qq) * (SB * 8) + frag;
+                    const float4 bp = *reinterpret_cast<const float4 *>(s_bp + o), bn = *reinterpret_cast<const float4 *>(s_bn + o);
+                    const float4 alp = *reinterpret_cast<const float4 *>(s_alp + o), aln = *reinterpret_cast<const float4 *>(s_aln + o);
+                    const float4 aup = *reinterpret_cast<const float4 *>(s_aup + o), aun = *reinterpret_cast<const float4 *>(s_aun + o);
+#define FAITH_DOT_SMALL(c)                          \
+    cl = mfma(xl[qq].c, alp.c, cl);                 \
+    cu = mfma(xu[qq].c, aup.c, cu);                 \
+    cl = mfma(xu[qq].c, aln.c, cl);                 \
+    cu = mfma(xl[qq].c, aun.c, cu);                 \
+    cl = mfma(bp.c, yl[qq].c, cl);                  \
+    cu = mfma(bp.c, yu[qq].c, cu);                  \
+    cl = mfma(bn.c, yu[qq].c, cl);                  \
+    cu = mfma(bn.c, yl[qq].c, cu);
+                    FAITH_DOT_SMALL(x)
+                    FAITH_DOT_SMALL(y)
+                    FAITH_DOT_SMALL(z)
+                    FAITH_DOT_SMALL(w)
+#undef FAITH_DOT_SMALL
+                }
+            }
+        }
+        // register r is row 8*(r/4) + 4*(lane/32) + r%4 of the block, lanes run along j
+        if (j0 + fi < g.Ly) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = i0 + 8 * (r / 4) + 4 * fh + (r % 4);
+                if (i < g.Lx) {
+                    const size_t o = (((size_t)t * g.Lx + i) * g.D + m) * g.Ly + j0 + fi;
+                    __builtin_nontemporal_store(cl[r], &g.zlw[o]);
+                    __builtin_nontemporal_store(cu[r], &g.zuw[o]);
+                }
+            }
+        }
+    }
+}
+
 // Any-shape coefficient kernel (d not a multiple of 4, unaligned pointers): one thread per
 // (i, m, j), products and sums in double.
 template <bool VP>
@@ -612,7 +753,17 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
                       faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
                       (long long)TI * D * (d > Ly ? d : Ly) * 4 < 0xffffffffLL &&    // 32-bit offsets inside a tile
                       (!VP || (long long)d * D * Ly * 4 < 0xffffffffLL);             // and along K inside a head
-    if (fast) {
+    if (fast && Lx <= 64 && Ly <= 64 && d % 8 == 0 && d <= 80) {
+        // short sequences: one 32 x 32 block per wavefront and perturbation coordinate; enough
+        // coordinates per wavefront that the grid is about four workgroups per CU
+        const long long blocks = (long long)B * ((Lx + SB - 1) / SB) * ((Ly + SB - 1) / SB);
+        long long mpw = (blocks * D) / (16LL * faith::compute_units());
+        mpw = mpw < 1 ? 1 : (mpw > 16 ? 16 : mpw);
+        const long long grid = blocks * ((D + 4 * mpw - 1) / (4 * mpw));
+        FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+        hipLaunchKernelGGL(dot_w_small<VP>, dim3((unsigned)grid), dim3(256), (size_t)6 * SB * d * sizeof(float), st, g,
+                           (int)mpw);
+    } else if (fast) {
         const long long tiles = (long long)B * D * ((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ);
         FAITH_REQUIRE(tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: too many tiles", who);
         const long long resident = 2LL * faith::compute_units();      // 56 KB of LDS each: two per CU

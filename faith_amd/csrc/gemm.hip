@@ -37,12 +37,9 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int BK = 16;
 constexpr int NTHREADS = 256;
 constexpr int XCDS = 8;
-constexpr int HALF = 128 * 8;            // floats in one [128 x 8] half of an operand's K-step
-constexpr int OPER = 2 * HALF;           // one operand, one K-step
-constexpr int S_AL = 0, S_AU = OPER, S_WP = 2 * OPER, S_WN = 3 * OPER, STAGE = 4 * OPER;
 
 struct GemmArgs {
     const float *Al, *Au;   // [Mw, K] coefficient rows (lower, upper)
@@ -86,10 +83,18 @@ __device__ __forceinline__ int swz(int row, int c) { return row * 8 + 4 * (c ^ (
 
 // EXACT = true: K % 16 == 0.  Otherwise (K % 4 == 0) the last K-step is partly past K: threads past
 // it read their K-step-0 piece instead (in bounds) and discard it before it reaches LDS.
-template <bool EXACT>
-__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-signsplit_gemm(const GemmArgs g) {
-    __shared__ float sm[2][STAGE];
+//
+// MB = MFMA blocks per wavefront and dimension: 2 is the 128 x 128 macro-tile described above; 1 is a
+// 64 x 64 macro-tile (wavefront tile 32 x 32, 32 accumulator registers, 32 KB of LDS) for problems
+// with too few 128 x 128 tiles to fill the machine: a wavefront then works through 32 MFMAs per
+// K-step instead of 128, a quarter of the latency, at a lower MFMA rate per byte staged.
+template <bool EXACT, int MB>
+__device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *smem) {
+    constexpr int BM = 64 * MB, BN = 64 * MB;
+    constexpr int HALF = BM * 8;             // floats in one [BM x 8] half of an operand's K-step
+    constexpr int OPER = 2 * HALF;           // one operand, one K-step
+    constexpr int S_AL = 0, S_AU = OPER, S_WP = 2 * OPER, S_WN = 3 * OPER, STAGE = 4 * OPER;
+    float(*sm)[STAGE] = reinterpret_cast<float(*)[STAGE]>(smem);
 
     // ---- tile of this workgroup
     const int tiles_n = (g.N + BN - 1) / BN;
@@ -105,20 +110,20 @@ signsplit_gemm(const GemmArgs g) {
 
     const int tid = threadIdx.x;
     const int lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
-    const int wm = wv / 2, wn = wv % 2;            // 2 x 2 wavefronts, 64 x 64 each
+    const int wm = wv / 2, wn = wv % 2;            // 2 x 2 wavefronts, (32 MB) x (32 MB) each
 
-    // ---- staging: an operand's K-step is 128 rows x 16 floats = 512 float4, two per thread:
-    // piece kq of rows r0 and r0 + 64.  Offsets are relative to the first row of the tile (the entry
-    // point checks that 128 rows span less than 4 GB); rows past the end re-read the last row, their
+    // ---- staging: an operand's K-step is BM rows x 16 floats = 256 MB float4, MB per thread:
+    // piece kq of rows r0 (and r0 + 64).  Offsets are relative to the first row of the tile (the entry
+    // point checks that a tile's rows span less than 4 GB); rows past the end re-read the last row, their
     // products are never stored.
     const int kq = tid % 4, r0 = tid / 4;
     const __amdgpu_buffer_rsrc_t wal = window(g.Al + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
     const __amdgpu_buffer_rsrc_t wau = window(g.Au + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
     const __amdgpu_buffer_rsrc_t ww = window(g.W + (size_t)n0 * K, ((size_t)(g.N - n0) * K) * 4);
-    unsigned va[2], vw[2];
-    int dst[2];
+    unsigned va[MB], vw[MB];
+    int dst[MB];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < MB; ++i) {
         const int ra = min(r0 + 64 * i, M - 1 - m0);
         const int rw = min(r0 + 64 * i, g.N - 1 - n0);
         va[i] = ((unsigned)ra * K + kq * 4) * 4u;
@@ -126,12 +131,12 @@ signsplit_gemm(const GemmArgs g) {
         dst[i] = (kq / 2) * HALF + swz(r0 + 64 * i, kq % 2);
     }
     const int nk = (K + BK - 1) / BK;
-    float4 pal[2], pau[2], pw[2];
+    float4 pal[MB], pau[MB], pw[MB];
     auto past = [&](int kt) { return !EXACT && kt * BK + kq * 4 >= K; };
     auto gload = [&](int kt) {
         const unsigned k = kt * (BK * 4u);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < MB; ++i) {
             if (EXACT) {
                 pal[i] = ld4(wal, va[i], k);
                 pau[i] = ld4(wau, va[i], k);
@@ -147,7 +152,7 @@ signsplit_gemm(const GemmArgs g) {
     auto lstore = [&](int buf, int kt) {
         float *s = sm[buf];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < MB; ++i) {
             if (past(kt)) pal[i] = pau[i] = pw[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             *reinterpret_cast<float4 *>(s + S_AL + dst[i]) = pal[i];
             *reinterpret_cast<float4 *>(s + S_AU + dst[i]) = pau[i];
@@ -156,41 +161,41 @@ signsplit_gemm(const GemmArgs g) {
         }
     };
 
-    floatx16 cl[2][2], cu[2][2];
+    floatx16 cl[MB][MB], cu[MB][MB];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < MB; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < MB; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
 
     // fragments: lane (fi = lane % 32, fh = lane / 32) reads k = 8*ks + 4*fh .. +3 of row fi
     const int fi = lane % 32, fh = lane / 32;
-    int fa[2], fw[2];
+    int fa[MB], fw[MB];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        fa[s] = swz(wm * 64 + s * 32 + fi, fh);
-        fw[s] = swz(wn * 64 + s * 32 + fi, fh);
+    for (int s = 0; s < MB; ++s) {
+        fa[s] = swz((wm * MB + s) * 32 + fi, fh);
+        fw[s] = swz((wn * MB + s) * 32 + fi, fh);
     }
     auto compute = [&](int buf, auto &&halfway) {
         const float *s = sm[buf];
 #pragma unroll
         for (int ks = 0; ks < BK / 8; ++ks) {
             if (ks == 1) halfway();
-            float4 al[2], au[2], wp[2], wq[2];
+            float4 al[MB], au[MB], wp[MB], wq[MB];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < MB; ++t) {
                 al[t] = *reinterpret_cast<const float4 *>(s + S_AL + ks * HALF + fa[t]);
                 au[t] = *reinterpret_cast<const float4 *>(s + S_AU + ks * HALF + fa[t]);
                 wp[t] = *reinterpret_cast<const float4 *>(s + S_WP + ks * HALF + fw[t]);
                 wq[t] = *reinterpret_cast<const float4 *>(s + S_WN + ks * HALF + fw[t]);
             }
 #define FAITH_STEP(c)                                                           \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) _Pragma("unroll") for (int b = 0; b < 2; ++b) { \
+    _Pragma("unroll") for (int a = 0; a < MB; ++a) _Pragma("unroll") for (int b = 0; b < MB; ++b) { \
         cl[a][b] = mfma(al[a].c, wp[b].c, cl[a][b]);                            \
         cu[a][b] = mfma(au[a].c, wp[b].c, cu[a][b]);                            \
     }                                                                           \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) _Pragma("unroll") for (int b = 0; b < 2; ++b) { \
+    _Pragma("unroll") for (int a = 0; a < MB; ++a) _Pragma("unroll") for (int b = 0; b < MB; ++b) { \
         cl[a][b] = mfma(au[a].c, wq[b].c, cl[a][b]);                            \
         cu[a][b] = mfma(al[a].c, wq[b].c, cu[a][b]);                            \
     }
@@ -223,14 +228,14 @@ signsplit_gemm(const GemmArgs g) {
 
     // ---- epilogue: register r of a 32x32 block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        const int col = n0 + wn * 64 + b * 32 + fi;
+    for (int b = 0; b < MB; ++b) {
+        const int col = n0 + (wn * MB + b) * 32 + fi;
         if (col >= g.N) continue;
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < MB; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+                const int row = m0 + (wm * MB + a) * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (row < M) {
                     const size_t o = (size_t)row * g.N + col;
                     __builtin_nontemporal_store(cl[a][b][r], &g.Cl[o]);
@@ -239,6 +244,18 @@ signsplit_gemm(const GemmArgs g) {
             }
         }
     }
+}
+
+template <bool EXACT>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+signsplit_gemm(const GemmArgs g) {
+    __shared__ float sm[2 * 4 * 2 * 128 * 8];            // two stages of four operands, 64 KB
+    signsplit_gemm_body<EXACT, 2>(g, sm);
+}
+template <bool EXACT>
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs g) {
+    __shared__ float sm[2 * 4 * 2 * 64 * 8];             // 32 KB
+    signsplit_gemm_body<EXACT, 1>(g, sm);
 }
 
 // ------------------------------------------------------------------ exact-accumulation kernel
@@ -306,18 +323,27 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
     GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
-                      faith::aligned(W, 16) && (long long)BM * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
+                      faith::aligned(W, 16) && 128LL * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
         GemmArgs gw = g;
         gw.Mb = 0;
-        const long long mblks = (mw + BM - 1) / BM;
-        const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + BN - 1) / BN);
+        // 64 x 64 macro-tiles when 128 x 128 ones would leave compute units without work
+        const long long big_tiles = ((mw + 127) / 128) * ((dim_y_out + 127) / 128);
+        // (they run within 2 % of the large tiles even at configuration 2, so the switch point is not critical)
+        const int tile = big_tiles < 2 * faith::compute_units() ? 64 : 128;
+        const long long mblks = (mw + tile - 1) / tile;
+        const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tile - 1) / tile);
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
-        if (dim_out % BK == 0)
+        const bool exact = dim_out % BK == 0;
+        if (tile == 128 && exact)
             hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
-        else
+        else if (tile == 128)
             hipLaunchKernelGGL(signsplit_gemm<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
+        else if (exact)
+            hipLaunchKernelGGL(signsplit_gemm_small<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
+        else
+            hipLaunchKernelGGL(signsplit_gemm_small<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
         GemmArgs gb = g;
         gb.Mw = 0;
         const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
