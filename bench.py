@@ -274,6 +274,53 @@ def bench_config4(args, ops, O, wl):
     return [e, e2]
 
 
+def bench_layer(args, wl):
+    """The path as its caller uses it: one encoder layer + pooler + margin classifier propagated by
+    faith_amd/forward.py (about 60 kernel launches), at a small-BERT size.  Wall clock, host included."""
+    import time
+    import torch
+    from types import SimpleNamespace
+    from faith_amd import Bounds, forward as F
+    hidden, heads, inter, length, eps, p = 256, 4, 512, 32, 0.01, 2.0
+    g = torch.Generator().manual_seed(77)
+    layer = wl.random_layer(g, hidden, heads, inter)
+    norm = SimpleNamespace(weight=1.0 + 0.1 * torch.randn(hidden, generator=g), bias=0.05 * torch.randn(hidden, generator=g))
+    pooler = SimpleNamespace(weight=torch.randn(hidden, hidden, generator=g) / hidden ** 0.5, bias=0.05 * torch.randn(hidden, generator=g))
+    clf = SimpleNamespace(weight=torch.randn(2, hidden, generator=g) / hidden ** 0.5, bias=0.05 * torch.randn(2, generator=g))
+    emb = torch.randn(1, length, hidden, generator=g)
+
+    def run(make, parts, e):
+        lay, nrm, pool, cl = parts
+        x = F.bound_input(make, e, 3, eps, 1, p, nrm, "no_var")
+        _, _, out = F.bound_layer(x, lay, "no_var", "relu")
+        return F.bound_classifier(F.bound_pooling(out, pool, make), cl, 0)
+
+    gparts = tuple(wl.to_device(x, "cuda") for x in (layer, norm, pooler, clf))
+    gmake = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    ge = emb.cuda()
+    t0 = time.time()
+    while time.time() - t0 < max(WARM_SECONDS, 0.05):
+        run(gmake, gparts, ge)
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        run(gmake, gparts, ge)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    e = {"op": f"extra: encoder layer + pooler + classifier, hidden {hidden}, {heads} heads, FFN {inter}, L={length}, "
+               f"one perturbed word, p=2 (forward.py, wall clock)",
+         "latency_us": round(statistics.median(times) * 1e3, 1), "latency_min_us": round(min(times) * 1e3, 1),
+         "bound": "host", "achieved": 0.0, "peak": 1.0, "unit": "-", "frac": 0.0, "work": 0}
+    if not args.no_cpu:
+        from tests.oracle_bounds import OracleBounds            # cpu_baseline leg only
+        omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)
+        s = cpu_time_s(lambda: run(omake, (layer, norm, pooler, clf), emb), reps=2, warmup=1)
+        e["cpu_baseline"] = {"latency_ms": round(s * 1e3, 1), "cores": torch.get_num_threads(), "kind": "port",
+                             "sample": "the same layer on the CPU oracle, median of 2"}
+    return e
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -316,6 +363,8 @@ def main():
         entries += bench_config3(args, ops, O, wl)
     if 4 in extra:
         entries += bench_config4(args, ops, O, wl)
+    if extra and not args.profile:
+        entries.append(bench_layer(args, wl))
 
     for e in entries:
         cb = e.get("cpu_baseline")

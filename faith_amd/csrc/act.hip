@@ -578,7 +578,7 @@ __global__ void __launch_bounds__(256) act_transposed(const ActArgs a) {
 // ------------------------------------------------------------------ host dispatch
 template <int MODE, int Q, int VEC, int TPR, int NTHREADS, int RPT>
 void launch_natural(const ActArgs &a, hipStream_t st) {
-    constexpr int TH = TPR * VEC, RG = NTHREADS / TPR;
+    constexpr int TH = TPR * VEC;
     const int tiles = (a.H + TH - 1) / TH;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
     hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)((a.rows + a.rows2) * tiles)),

@@ -716,7 +716,6 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
                   "%s: batch=%d rows of x=%d columns of z=%d reduction length=%d dim_in=%d must be positive", who, B,
                   Lx, Ly, d, D);
     const long long nw = (long long)B * Lx * D * Ly;
-    const long long nx = (long long)B * Lx * D * d, ny = (long long)B * Ly * D * d;
     FAITH_REQUIRE((long long)B * (Lx > Ly ? Lx : Ly) * D <= 0x7fffffffLL && (long long)B * d * D <= 0x7fffffffLL,
                   FAITH_ERR_SHAPE, "%s: batch*length*dim_in exceeds 2^31", who);
 

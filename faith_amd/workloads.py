@@ -8,6 +8,7 @@ lw, the uw gap, lb, the ub gap, and then the layer's W and bias.
 from __future__ import annotations
 
 import math
+from types import SimpleNamespace
 
 import torch
 
@@ -66,3 +67,29 @@ def make_config(cfg: int, scale: float = 1.0) -> dict:
         b = torch.randn(128, generator=g) * 0.01
         return dict(op="conv", x=x, W=W, bias=b, stride=1, padding=1, p=INF, eps=2.0 / 255)
     raise ValueError(f"no such configuration: {cfg}")
+
+
+# ------------------------------------------------------------------ a whole encoder layer
+def random_layer(g, hidden, heads, inter, scale=0.5):
+    """Random weights of one Transformer encoder layer, laid out like the reference's BERT modules
+    (the attribute names faith_amd/forward.py reads)."""
+    def lin(n_out, n_in):
+        return SimpleNamespace(weight=torch.randn(n_out, n_in, generator=g) * scale / n_in ** 0.5,
+                               bias=torch.randn(n_out, generator=g) * 0.05)
+
+    def norm(n):
+        return SimpleNamespace(weight=1.0 + 0.1 * torch.randn(n, generator=g), bias=0.05 * torch.randn(n, generator=g))
+    att_self = SimpleNamespace(query=lin(hidden, hidden), key=lin(hidden, hidden), value=lin(hidden, hidden),
+                               num_attention_heads=heads, attention_head_size=hidden // heads)
+    attention = SimpleNamespace(self=att_self, output=SimpleNamespace(dense=lin(hidden, hidden), LayerNorm=norm(hidden)))
+    return SimpleNamespace(attention=attention, intermediate=SimpleNamespace(dense=lin(inter, hidden)),
+                           output=SimpleNamespace(dense=lin(hidden, inter), LayerNorm=norm(hidden)))
+
+
+def to_device(obj, device):
+    """Deep copy of a layer description with every tensor moved to `device`."""
+    if isinstance(obj, torch.Tensor):
+        return obj.to(device)
+    if isinstance(obj, SimpleNamespace):
+        return SimpleNamespace(**{k: to_device(v, device) for k, v in vars(obj).items()})
+    return obj

@@ -58,27 +58,7 @@ for _name in ("relu", "tanh", "exp", "sqr", "sqrt", "reciprocal", "softmax"):
     setattr(OracleBounds, _name, _method)
 
 
-def random_layer(g, hidden, heads, inter, scale=0.5):
-    def lin(n_out, n_in):
-        return SimpleNamespace(weight=torch.randn(n_out, n_in, generator=g) * scale / n_in ** 0.5,
-                               bias=torch.randn(n_out, generator=g) * 0.05)
-
-    def norm(n):
-        return SimpleNamespace(weight=1.0 + 0.1 * torch.randn(n, generator=g), bias=0.05 * torch.randn(n, generator=g))
-    att_self = SimpleNamespace(query=lin(hidden, hidden), key=lin(hidden, hidden), value=lin(hidden, hidden),
-                               num_attention_heads=heads, attention_head_size=hidden // heads)
-    attention = SimpleNamespace(self=att_self, output=SimpleNamespace(dense=lin(hidden, hidden), LayerNorm=norm(hidden)))
-    return SimpleNamespace(attention=attention, intermediate=SimpleNamespace(dense=lin(inter, hidden)),
-                           output=SimpleNamespace(dense=lin(hidden, inter), LayerNorm=norm(hidden)))
-
-
-def to_device(obj, device):
-    """Deep copy of a layer description with every tensor moved to `device`."""
-    if isinstance(obj, torch.Tensor):
-        return obj.to(device)
-    if isinstance(obj, SimpleNamespace):
-        return SimpleNamespace(**{k: to_device(v, device) for k, v in vars(obj).items()})
-    return obj
+from faith_amd.workloads import random_layer, to_device  # noqa: E402,F401  (synthetic layers are shared with bench.py)
 
 
 def true_layer(x, layer, embed_norm, mode, pooler, classifier):
