@@ -40,8 +40,11 @@ WARM_SECONDS = 0.25            # minimum warm-up per measurement; --profile sets
 
 # HBM bytes per launch of the dominant relaxation kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE, scaled by the same counters on faith_copy_f32 of known size (see
-# profiles/hbm_traffic_pmc.md).  None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = 270_180_000   # tanh kernel: (2.000 * 65,906 + 132,036) KiB
+# profiles/hbm_traffic_pmc.md), per relaxation (FETCH_SIZE reads half of what was fetched on this part).
+TRAFFIC_BYTES_PER_LAUNCH = {
+    "relu": 271_810_000,   # (2.000 * 66,349 + 132,750) KiB
+    "tanh": 269_980_000,   # (2.000 * 65,887 + 131,877) KiB
+}
 
 
 def log(*a):
@@ -182,7 +185,7 @@ def bench_config1(args, ops, O, wl, steps, warmup):
                 "achieved": round(nbytes / avg_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(nbytes / avg_ms / 1e6 / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(avg_ms * 1e3, 2), "bytes_per_launch": nbytes,
-                "traffic": TRAFFIC_BYTES_PER_LAUNCH}
+                "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom[0])}
 
     cpu = None
     if not args.no_cpu:

@@ -53,6 +53,31 @@ class Bounds:
         lw, lb, uw, ub = self._c()
         return ops.concretize(lw, lb, uw, ub, self.p, self.eps, self.perturbed_words)
 
+    # ---- Bounds.py:311-317: -/+ eps * ||w||_q over the whole of dim_in (no perturbed-word blocks)
+    def concretize_l(self, lw=None):
+        lw = (self.lw if lw is None else lw).contiguous()
+        zero = torch.zeros(lw.shape[:2] + lw.shape[3:], device=lw.device)
+        return ops.concretize(lw, zero, lw, zero, self.p, self.eps, 1)[0]
+
+    def concretize_u(self, uw=None):
+        uw = (self.uw if uw is None else uw).contiguous()
+        zero = torch.zeros(uw.shape[:2] + uw.shape[3:], device=uw.device)
+        return ops.concretize(uw, zero, uw, zero, self.p, self.eps, 1)[1]
+
+    # ---- Bounds.py:328-333
+    def clone(self):
+        return self._like(self.lw.clone(), self.lb.clone(), self.uw.clone(), self.ub.clone())
+
+    # ---- Bounds.py:299-309
+    def print(self, message):
+        print(message)
+        l, u = self.concretize()
+        print("mean abs %.5f %.5f" % (l.abs().mean(), u.abs().mean()))
+        print("diff %.5f %.5f %.5f" % ((u - l).min(), (u - l).max(), (u - l).mean()))
+        print("min", l.min())
+        print("max", u.max())
+        print()
+
     # ---- Bounds.py:383-395
     def add(self, delta):
         if isinstance(delta, Bounds):

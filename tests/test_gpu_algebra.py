@@ -101,3 +101,22 @@ def test_rowsum_broadcast():
         out = ops.rowsum_broadcast(t.cuda())
         exp = t.sum(-1, keepdim=True).expand_as(t)
         assert close(out, exp, rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.gpu
+def test_concretize_halves_and_clone():
+    """Bounds.concretize_l / concretize_u (Bounds.py:311-317) and clone (:328-333)."""
+    import math
+    from faith_amd import Bounds
+    g = torch.Generator().manual_seed(91)
+    lw = torch.randn(2, 5, 24, 40, generator=g)
+    lb = torch.randn(2, 5, 40, generator=g)
+    for p in (1.0, 2.0, float("inf")):
+        q = float("inf") if p == 1 else (1.0 if math.isinf(p) else 2.0)
+        b = Bounds(None, p, 0.3, lw=lw.cuda(), lb=lb.cuda(), uw=(lw + 0.1).cuda(), ub=(lb + 0.1).cuda())
+        want_l = -0.3 * torch.linalg.vector_norm(lw.double(), ord=q, dim=-2)
+        want_u = 0.3 * torch.linalg.vector_norm((lw + 0.1).double(), ord=q, dim=-2)
+        assert torch.allclose(b.concretize_l().cpu().double(), want_l, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(b.concretize_u().cpu().double(), want_u, rtol=1e-5, atol=1e-6)
+        c = b.clone()
+        assert c.lw.data_ptr() != b.lw.data_ptr() and torch.equal(c.lw, b.lw) and torch.equal(c.ub, b.ub)
