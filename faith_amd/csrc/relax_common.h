@@ -15,7 +15,8 @@ __device__ __forceinline__ float nacc(float acc, float v) {
     // words and held for every value a thread keeps (64 more registers)
     if (Q == FAITH_Q_2) return __builtin_fmaf(v, v, acc);
     if (Q == FAITH_Q_1) return acc + fabsf(v);
-    return fmaxf(acc, fabsf(v));
+    // max(acc, |v|) as one median-of-three (fmaxf adds a canonicalising v_max per value)
+    return __builtin_amdgcn_fmed3f(acc, fabsf(v), __builtin_inff());
 }
 template <int Q>
 __device__ __forceinline__ float ncomb(float a, float b) {
