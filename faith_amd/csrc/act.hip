@@ -177,6 +177,46 @@ __device__ __forceinline__ void tanh_pure_lines(float l, float u, Line &lo, Line
     }
 }
 
+// tanh lines of the TH neurons of a tile whose concrete intervals are in s_lu ([2][TH]), entered by
+// every thread after a barrier: three wavefronts share the per-neuron work, lane = neuron.  Slopes end
+// up in s_ln[0 .. TH) and s_ln[3 TH .. 4 TH) (complete once the barrier inside has been passed), the
+// constant terms in olb / oub.
+template <int TH>
+__device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, float *s_ln,
+                                           const float *__restrict__ p_lb, const float *__restrict__ p_ub, size_t bi,
+                                           bool n_ok, int lane, int wv) {
+    // three wavefronts share the per-neuron work: 0 = lower tangent search, 1 = upper tangent
+    // search (straddling neurons), 2 = tangent / chord of one-signed neurons
+    if (wv < 3 && n_ok) {
+        const float l = s_lu[lane], u = s_lu[TH + lane];
+        const bool pure = (u < 0.f || l > 0.f);
+        if (wv == 2) {
+            if (pure) {
+                Line lo, up;
+                tanh_pure_lines(l, u, lo, up);
+                s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
+                s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
+            }
+        } else if (!pure) {
+            if (wv == 0) {
+                const Line lo = tanh_tangent_line<true>(l, u);
+                s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
+            } else {
+                const Line up = tanh_tangent_line<false>(l, u);
+                s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
+            }
+        }
+    }
+    __syncthreads();
+    if (wv == 0 && n_ok) {
+        const Line lo = {s_ln[lane], s_ln[TH + lane], s_ln[2 * TH + lane]};
+        const Line up = {s_ln[3 * TH + lane], s_ln[4 * TH + lane], s_ln[5 * TH + lane]};
+        const float lb = p_lb[bi], ub = p_ub[bi];
+        a.olb[bi] = line_bias(lo, lb, ub);
+        a.oub[bi] = line_bias(up, ub, lb);
+    }
+}
+
 // The per-neuron part of a natural-layout tile, entered by every thread after the partial norms are
 // in `part` ([words][NW][2][TH]) and a barrier: one lane per neuron (wavefront 0) finishes the
 // norms and concretizes; the slopes of the two lines end up in s_ln[0 .. TH) and s_ln[3 TH .. 4 TH),
@@ -215,38 +255,7 @@ __device__ __forceinline__ void neuron_stage(const ActArgs &a, const float *part
     if (MODE == CONCRETIZE) return;
     __syncthreads();
 
-    if (MODE == TANH) {
-        // three wavefronts share the per-neuron work: 0 = lower tangent search, 1 = upper tangent
-        // search (straddling neurons), 2 = tangent / chord of one-signed neurons
-        if (wv < 3 && n_ok) {
-            const float l = s_lu[lane], u = s_lu[TH + lane];
-            const bool pure = (u < 0.f || l > 0.f);
-            if (wv == 2) {
-                if (pure) {
-                    Line lo, up;
-                    tanh_pure_lines(l, u, lo, up);
-                    s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
-                    s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
-                }
-            } else if (!pure) {
-                if (wv == 0) {
-                    const Line lo = tanh_tangent_line<true>(l, u);
-                    s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
-                } else {
-                    const Line up = tanh_tangent_line<false>(l, u);
-                    s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
-                }
-            }
-        }
-        __syncthreads();
-        if (wv == 0 && n_ok) {
-            const Line lo = {s_ln[lane], s_ln[TH + lane], s_ln[2 * TH + lane]};
-            const Line up = {s_ln[3 * TH + lane], s_ln[4 * TH + lane], s_ln[5 * TH + lane]};
-            const float lb = p_lb[bi], ub = p_ub[bi];
-            a.olb[bi] = line_bias(lo, lb, ub);
-            a.oub[bi] = line_bias(up, ub, lb);
-        }
-    }
+    if (MODE == TANH) tanh_stage<TH>(a, s_lu, s_ln, p_lb, p_ub, bi, n_ok, lane, wv);
 }
 
 // TPR threads cover one row of the tile (TH = TPR * VEC neurons); RG = NTHREADS / TPR rows are
@@ -391,7 +400,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
 // per-neuron stage between its loads and its stores: at configuration 1 it runs within 3 % of
 // that copy, where the general kernel above needs 25 % more.
 template <int MODE, int Q, int TPR, int NTHREADS, int RPT>
-__global__ void __launch_bounds__(NTHREADS) act_resident(const ActArgs a) {
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4))) act_resident(const ActArgs a) {
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
     static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
     extern __shared__ float smem[];
@@ -593,6 +602,117 @@ void launch_resident(const ActArgs &a, hipStream_t st) {
                        smem, st, a);
 }
 
+// Transposed layout, D_in = 256 V (V = 1, 2), 16-byte aligned: a wavefront owns 8 / V neurons, one
+// 16-byte load per lane covers 256 coefficients of a neuron's contiguous row, and everything a
+// wavefront reads (64 values per thread) stays in registers between the norm and the scaling: one
+// read, one write, no LDS and no barrier.  The norms of a neuron end up in every lane of its
+// wavefront (butterfly); lane i then derives the lines of the wavefront's i-th neuron, and the slopes
+// travel back by cross-lane reads.
+template <int MODE, int Q, int V>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) act_transposed_resident(const ActArgs a) {
+    constexpr int NPW = 8 / V;
+    const int lane = threadIdx.x % WAVE, wv = threadIdx.x / WAVE;
+    const long long total = (long long)a.rows * a.H;
+    const long long n0 = ((long long)blockIdx.x * 4 + wv) * NPW;      // first neuron of this wavefront
+    const int blk = a.D / a.words;
+
+    Vec<4> dl[NPW][V], du[NPW][V];
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) {
+        const long long n = n0 + i < total ? n0 + i : total - 1;      // a clamped neuron is never stored
+        const float *pl = a.lw + (size_t)n * a.D + lane * 4, *pu = a.uw + (size_t)n * a.D + lane * 4;
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            dl[i][v].load(pl + v * 256);
+            du[i][v].load(pu + v * 256);
+        }
+    }
+    float l[NPW], u[NPW];
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) {
+        const long long n = n0 + i < total ? n0 + i : total - 1;
+        float li = a.lb[n], ui = a.ub[n];
+        for (int w = 0; w < a.words; ++w) {
+            float nl = 0.f, nu = 0.f;
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const int k0 = v * 256 + lane * 4;                    // blk % 4 == 0: a float4 lies in one word
+                if (k0 >= w * blk && k0 < (w + 1) * blk) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        nl = nacc<Q>(nl, dl[i][v].get(c));
+                        nu = nacc<Q>(nu, du[i][v].get(c));
+                    }
+                }
+            }
+            nl = Q == FAITH_Q_INF ? wave_max(nl) : wave_sum(nl);
+            nu = Q == FAITH_Q_INF ? wave_max(nu) : wave_sum(nu);
+            li += (-a.eps) * nfin<Q>(nl);
+            ui += a.eps * nfin<Q>(nu);
+        }
+        l[i] = li;
+        u[i] = ui;
+    }
+    // lane i takes the wavefront's i-th neuron
+    float myl = l[0], myu = u[0];
+#pragma unroll
+    for (int i = 1; i < NPW; ++i) {
+        if (lane == i) {
+            myl = l[i];
+            myu = u[i];
+        }
+    }
+    float klo = 0.f, kup = 0.f;
+    const long long mine = n0 + lane;
+    if (lane < NPW && mine < total) {
+        if (a.l) a.l[mine] = myl;
+        if (a.u) a.u[mine] = myu;
+        if (MODE != CONCRETIZE && MODE != TANH) {
+            float olb, oub;
+            relax_any<MODE>(myl, myu, a.lb[mine], a.ub[mine], klo, kup, olb, oub);
+            a.olb[mine] = olb;
+            a.oub[mine] = oub;
+        }
+    }
+    if (MODE == CONCRETIZE) return;
+    if (MODE == TANH) {
+        // the search for the tangent points is long: gather the workgroup's neurons in LDS and let three
+        // wavefronts do it for all of them at once, one neuron per lane
+        constexpr int NPB = 4 * NPW;
+        __shared__ float s_lu[2 * NPB], s_ln[6 * NPB];
+        if (lane < NPW) {
+            s_lu[wv * NPW + lane] = myl;
+            s_lu[NPB + wv * NPW + lane] = myu;
+        }
+        __syncthreads();
+        const long long first = (long long)blockIdx.x * NPB;
+        tanh_stage<NPB>(a, s_lu, s_ln, a.lb, a.ub, (size_t)(first + lane), lane < NPB && first + lane < total, lane, wv);
+        if (lane < NPW) {
+            klo = s_ln[wv * NPW + lane];
+            kup = s_ln[3 * NPB + wv * NPW + lane];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) {
+        const float k_lo = __shfl(klo, i, WAVE), k_up = __shfl(kup, i, WAVE);
+        if (n0 + i < total) {
+            float *ql = a.olw + (size_t)(n0 + i) * a.D + lane * 4, *qu = a.ouw + (size_t)(n0 + i) * a.D + lane * 4;
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                Vec<4> ol, ou;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float xl = dl[i][v].get(c), xu = du[i][v].get(c);
+                    ol.set(c, (k_lo > 0.f ? xl : xu) * k_lo);
+                    ou.set(c, (k_up > 0.f ? xu : xl) * k_up);
+                }
+                ol.store(ql + v * 256);
+                ou.store(qu + v * 256);
+            }
+        }
+    }
+}
+
 template <int MODE, int Q>
 void dispatch_natural(const ActArgs &a, hipStream_t st) {
     const bool vec4 = (a.H % 4 == 0) && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
@@ -648,7 +768,14 @@ void dispatch_layout(const ActArgs &a, int layout, hipStream_t st) {
         dispatch_natural<MODE, Q>(a, st);
     } else {
         const long long total = (long long)a.rows * a.H;
-        hipLaunchKernelGGL((act_transposed<MODE, Q>), dim3((unsigned)((total + 63) / 64)), dim3(256), 0, st, a);
+        const bool vec = (a.D / a.words) % 4 == 0 && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
+                         (MODE == CONCRETIZE || (faith::aligned(a.olw, 16) && faith::aligned(a.ouw, 16)));
+        if (vec && a.D == 256)
+            hipLaunchKernelGGL((act_transposed_resident<MODE, Q, 1>), dim3((unsigned)((total + 31) / 32)), dim3(256), 0, st, a);
+        else if (vec && a.D == 512)
+            hipLaunchKernelGGL((act_transposed_resident<MODE, Q, 2>), dim3((unsigned)((total + 15) / 16)), dim3(256), 0, st, a);
+        else
+            hipLaunchKernelGGL((act_transposed<MODE, Q>), dim3((unsigned)((total + 63) / 64)), dim3(256), 0, st, a);
     }
 }
 

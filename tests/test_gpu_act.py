@@ -45,7 +45,7 @@ def check(kind, x, p, eps, words, layout="natural"):
 def test_concretize(p, words, layout):
     from faith_amd import ops
     g = torch.Generator().manual_seed(5)
-    for (B, L, D, H) in [(1, 3, 64, 64), (2, 5, 96, 40), (1, 2, 600, 132), (1, 1, 6, 7)]:
+    for (B, L, D, H) in [(1, 3, 64, 64), (2, 5, 96, 40), (1, 2, 600, 132), (1, 1, 6, 7), (1, 3, 256, 41), (1, 2, 512, 21)]:
         x = rand_bounds(g, B, L, D, H, ordered=False)
         lw, lb, uw, ub = dev(*x.tensors())
         if layout == "natural":
@@ -64,7 +64,7 @@ def test_activation_small_shapes(kind, p, layout):
     g = torch.Generator().manual_seed(6)
     # register-resident, chunked (D_in > 512), ragged H (scalar path), tiny
     for (L, D, H, words) in [(4, 64, 64, 1), (3, 128, 192, 2), (2, 256, 64, 2), (2, 512, 64, 1),
-                             (1, 1100, 72, 1), (2, 48, 37, 3), (1, 2, 5, 1)]:
+                             (1, 1100, 72, 1), (2, 48, 37, 3), (1, 2, 5, 1), (3, 256, 37, 4), (1, 512, 9, 2)]:
         x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
         check(kind, x, p, 0.05, words, layout)
 
