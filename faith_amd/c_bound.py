@@ -23,7 +23,7 @@ words = 1      # perturbed_words
 
 
 def _s(t):
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return ops._stream(t)
 
 
 def _act(entry, src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw, length, dim_in, dim_out, epsilon):
