@@ -29,11 +29,14 @@ SIGNATURES = {
     "faith_tanh_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_unary_verification": [_I] + [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_multiply_verification": [_P] * 12 + [_I, _I, _I, _F, _I, _I, _P],
-    "faith_scale_add": [_P, _P, _P, _F, _P, _P, _P, _P, _P, ctypes.c_longlong, _I, _P],
-    "faith_rowsum_broadcast": [_P, _P, ctypes.c_longlong, _I, _P],
+    "faith_affine_verification": [_P] * 5 + [_F] + [_P] * 9 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
+    "faith_rowsum_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
+    "faith_layer_norm_verification": [_P] * 10 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],
     "faith_dot_product_verification_QK": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_dot_product_verification_V": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
+    "faith_attention_scores": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
+    "faith_attention_context": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_convolution_verification": [_P] * 10 + [_I] * 9 + [_P],
 }
 

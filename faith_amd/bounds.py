@@ -82,8 +82,7 @@ class Bounds:
     def add(self, delta):
         if isinstance(delta, Bounds):
             return self._like(*ops.add(self._c(), delta._c()))
-        lb, ub = ops.shift(self.lb.contiguous(), self.ub.contiguous(), delta)
-        return self._like(self.lw, lb, self.uw, ub)
+        return self._like(*ops.shift(*self._c(), delta))
 
     # ---- Bounds.py:594-664: by a float, by a per-neuron tensor, or by another bound object
     def multiply(self, W):
@@ -100,24 +99,23 @@ class Bounds:
     # ---- Bounds.py:1005-1014
     def softmax(self):
         e = self.exp()
-        total = self._like(ops.rowsum_broadcast(e.lw), ops.rowsum_broadcast(e.lb),
-                           ops.rowsum_broadcast(e.uw), ops.rowsum_broadcast(e.ub))
-        return e.divide(total)
+        return e.divide(self._like(*ops.rowsum(*e._c())))
 
     # ---- Bounds.py:1111-1131
     def layer_norm(self, normalizer, layer_norm):
         if layer_norm == "no":
             return self
+        weight, bias = normalizer.weight.detach().contiguous(), normalizer.bias.detach().contiguous()
+        if layer_norm == "no_var":
+            # mean subtraction, weight and bias in one launch
+            return self._like(*ops.layer_norm(*self._c(), weight, bias))
+        assert layer_norm == "standard"
         H = self.dim_out
+        minus_mu = self._like(*ops.layer_norm(*self._c()))
         w_avg = torch.full((H, H), 1.0 / H, device=self.device, dtype=torch.float32)
-        minus_mu = self.add(self.matmul(w_avg).multiply(-1.0))
-        if layer_norm == "standard":
-            variance = minus_mu.sqr().matmul(w_avg)
-            normalized = minus_mu.divide(variance.add(1e-12).sqrt())
-        else:
-            assert layer_norm == "no_var"
-            normalized = minus_mu
-        return normalized.multiply(normalizer.weight.detach().contiguous()).add(normalizer.bias.detach().contiguous())
+        variance = minus_mu.sqr().matmul(w_avg)
+        normalized = minus_mu.divide(variance.add(1e-12).sqrt())
+        return normalized._like(*ops.affine(normalized._c(), scale=weight, shift=bias))
 
     # ---- Bounds.py:397-413, :1177-1199
     def matmul(self, W, bias=None):
@@ -186,6 +184,16 @@ class Bounds:
     # ---- Bounds.py:843-850
     def context(self, value):
         return self.dot_product(value.t())
+
+    # ---- VerifierForward.py:208-229 + Bounds.py:833-841: scores of all heads, self = query and key
+    # both [1, L, D, heads * size]; the kernels address each head in place
+    def attention_scores(self, key, heads):
+        return self._like(*ops.attention_scores(self._c(), key._c(), heads, self.p, self.eps, self.perturbed_words))
+
+    # ---- VerifierForward.py:208-229 + Bounds.py:843-850 + VerifierForward.py:253-263: self = probabilities
+    # [heads, Lx, D, Lk], value [1, Lk, D, heads * size] -> [1, Lx, D, heads * size]
+    def attention_context(self, value):
+        return self._like(*ops.attention_context(self._c(), value._c(), self.p, self.eps, self.perturbed_words))
 
 
 class ConvBounds:

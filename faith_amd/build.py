@@ -29,6 +29,7 @@ EXTRA = {
     # the relaxations round (b - x0) * k and + y0 separately, as the PyTorch path does
     "act.hip": ["-ffp-contract=off"],
     "mul.hip": ["-ffp-contract=off"],
+    "affine.hip": ["-ffp-contract=off"],
 }
 
 

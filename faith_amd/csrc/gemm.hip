@@ -9,7 +9,9 @@
 //
 // The reference's CUTLASS path takes the constant-term rows as trailing M-blocks of the same grid
 // (tvm_kernels/cuda_kernel/mma/mma_kernel.h:251-259); here they go to the exact-accumulation
-// kernel below instead: they are 1/D_in of the work and the only outputs whose O(1) terms cancel.
+// code below instead: they are 1/D_in of the work and the only outputs whose O(1) terms cancel.
+// For small problems those tiles are the leading workgroups of the MFMA launch, for large ones a
+// launch of their own.
 //
 // Tiling (gfx950): workgroup = 4 wavefronts, macro-tile BM x BN = 128 x 128, K-step 16,
 // wavefront tile 64 x 64 = 2 x 2 v_mfma_f32_32x32x2_f32 blocks for EACH of C_l and C_u
@@ -89,7 +91,7 @@ __device__ __forceinline__ int swz(int row, int c) { return row * 8 + 4 * (c ^ (
 // with too few 128 x 128 tiles to fill the machine: a wavefront then works through 32 MFMAs per
 // K-step instead of 128, a quarter of the latency, at a lower MFMA rate per byte staged.
 template <bool EXACT, int MB>
-__device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *smem) {
+__device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *smem, const int pid) {
     constexpr int BM = 64 * MB, BN = 64 * MB;
     constexpr int HALF = BM * 8;             // floats in one [BM x 8] half of an operand's K-step
     constexpr int OPER = 2 * HALF;           // one operand, one K-step
@@ -99,7 +101,6 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
     // ---- tile of this workgroup
     const int tiles_n = (g.N + BN - 1) / BN;
     const int mblks = (g.Mw + BM - 1) / BM;
-    const int pid = blockIdx.x;
     const int xcd = pid % XCDS, local = pid / XCDS;
     const int m_blk = (local / tiles_n) * XCDS + xcd;
     const int n_blk = local % tiles_n;
@@ -246,18 +247,6 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
     }
 }
 
-template <bool EXACT>
-__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-signsplit_gemm(const GemmArgs g) {
-    __shared__ float sm[2 * 4 * 2 * 128 * 8];            // two stages of four operands, 64 KB
-    signsplit_gemm_body<EXACT, 2>(g, sm);
-}
-template <bool EXACT>
-__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs g) {
-    __shared__ float sm[2 * 4 * 2 * 64 * 8];             // 32 KB
-    signsplit_gemm_body<EXACT, 1>(g, sm);
-}
-
 // ------------------------------------------------------------------ exact-accumulation kernel
 // 16 x 16 outputs per workgroup, scalar loads, products and sums in double (an fp32 x fp32
 // product is exact in double), one rounding at the end.  Two uses:
@@ -265,11 +254,13 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs 
 //    which is where the order of an fp32 summation shows; accumulated in double they carry no
 //    summation error at all;
 //  * any shape the MFMA kernel does not take (K not a multiple of 4, unaligned pointers).
-__global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
-    __shared__ float sl[16][17], su[16][17], sw[16][17];
+// One 16 x 16 tile: M-block m_blk counts through the coefficient rows first, then the constant rows.
+// smem: 3 * 16 * 17 floats.
+__device__ __forceinline__ void simple_tile(const GemmArgs &g, const int m_blk, const int n_blk, float *smem) {
+    float(*sl)[17] = reinterpret_cast<float(*)[17]>(smem);
+    float(*su)[17] = reinterpret_cast<float(*)[17]>(smem + 16 * 17);
+    float(*sw)[17] = reinterpret_cast<float(*)[17]>(smem + 2 * 16 * 17);
     const int mblk_w = (g.Mw + 15) / 16;
-    const int tiles_n = (g.N + 15) / 16;
-    const int m_blk = blockIdx.x / tiles_n, n_blk = blockIdx.x % tiles_n;
     const bool brows = m_blk >= mblk_w;
     const float *Al = brows ? g.Bl : g.Al, *Au = brows ? g.Bu : g.Au;
     float *Cl = brows ? g.Dl : g.Cl, *Cu = brows ? g.Du : g.Cu;
@@ -304,6 +295,33 @@ __global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
     }
 }
 
+__global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
+    __shared__ float sm[3 * 16 * 17];
+    const int tiles_n = (g.N + 15) / 16;
+    simple_tile(g, blockIdx.x / tiles_n, blockIdx.x % tiles_n, sm);
+}
+
+template <bool EXACT>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+signsplit_gemm(const GemmArgs g) {
+    __shared__ float sm[2 * 4 * 2 * 128 * 8];            // two stages of four operands, 64 KB
+    signsplit_gemm_body<EXACT, 2>(g, sm, blockIdx.x);
+}
+// Small problems: the first `b_tiles` workgroups take the 16 x 16 tiles of the constant-term rows
+// (exact accumulation; each is a long chain of short steps, so they start first and run beside the
+// MFMA tiles instead of in a launch of their own), the others a 64 x 64 MFMA tile each.
+template <bool EXACT>
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs g, const int b_tiles) {
+    __shared__ float sm[2 * 4 * 2 * 64 * 8];             // 32 KB
+    if ((int)blockIdx.x < b_tiles) {
+        const int tiles_n = (g.N + 15) / 16;
+        const int m_blk = blockIdx.x / tiles_n;
+        if (m_blk < (g.Mb + 15) / 16) simple_tile(g, (g.Mw + 15) / 16 + m_blk, blockIdx.x % tiles_n, sm);
+        return;
+    }
+    signsplit_gemm_body<EXACT, 1>(g, sm, blockIdx.x - b_tiles);
+}
+
 }  // namespace
 
 extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
@@ -326,8 +344,6 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
                       faith::aligned(W, 16) && 128LL * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
-        GemmArgs gw = g;
-        gw.Mb = 0;
         // 64 x 64 macro-tiles when 128 x 128 ones would leave compute units without work
         const long long big_tiles = ((mw + 127) / 128) * ((dim_y_out + 127) / 128);
         // (they run within 2 % of the large tiles even at configuration 2, so the switch point is not critical)
@@ -336,18 +352,27 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
         const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tile - 1) / tile);
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
         const bool exact = dim_out % BK == 0;
-        if (tile == 128 && exact)
-            hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
-        else if (tile == 128)
-            hipLaunchKernelGGL(signsplit_gemm<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
-        else if (exact)
-            hipLaunchKernelGGL(signsplit_gemm_small<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
-        else
-            hipLaunchKernelGGL(signsplit_gemm_small<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
-        GemmArgs gb = g;
-        gb.Mw = 0;
         const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
-        hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+        if (tile == 64) {
+            // constant-term tiles in front, rounded up to a multiple of 8 so that the MFMA tiles keep
+            // their XCD (workgroup number mod 8)
+            const long long b_tiles = (gridb + XCDS - 1) / XCDS * XCDS;
+            FAITH_REQUIRE(grid + b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
+            if (exact)
+                hipLaunchKernelGGL(signsplit_gemm_small<true>, dim3((unsigned)(grid + b_tiles)), dim3(NTHREADS), 0, st, g,
+                                   (int)b_tiles);
+            else
+                hipLaunchKernelGGL(signsplit_gemm_small<false>, dim3((unsigned)(grid + b_tiles)), dim3(NTHREADS), 0, st, g,
+                                   (int)b_tiles);
+        } else {
+            if (exact)
+                hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
+            else
+                hipLaunchKernelGGL(signsplit_gemm<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
+            GemmArgs gb = g;
+            gb.Mw = 0;
+            hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+        }
     } else {
         const long long grid = ((mw + 15) / 16 + (rows + 15) / 16) * ((dim_y_out + 15) / 16);
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");

@@ -317,57 +317,6 @@ void dispatch_mul(const MulArgs &a, hipStream_t st) {
         launch_mul<Q, 4, 8, 256, 8>(a, st);       // D_in <= 256 in registers (128 values per thread), passes beyond
 }
 
-// ------------------------------------------------------------------ plain elementwise kernels
-// out = a * s+ + a' * s-  per column (Bounds.multiply with a float or a tensor, Bounds.py:595-607, :653-664),
-// optionally followed by + b (Bounds.add, :383-395).  inner = elements per scale entry cycle:
-// element e uses scale[(e % H)].
-__global__ void __launch_bounds__(256) scale_add_kernel(const float *__restrict__ lo, const float *__restrict__ up,
-                                                        const float *__restrict__ scale, float scalar,
-                                                        const float *__restrict__ add_lo,
-                                                        const float *__restrict__ add_up,
-                                                        const float *__restrict__ shift, float *__restrict__ out_lo,
-                                                        float *__restrict__ out_up, size_t n, int H) {
-    const size_t stride = (size_t)gridDim.x * 256;
-    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
-        float l = lo[e], u = up[e];
-        if (scale || scalar != 1.f) {
-            const float s = scale ? scale[e % H] : scalar;
-            const float sp = s > 0.f ? s : 0.f * s;      // W * (W > 0): zero keeps the sign rule of the product
-            const float sn = s - sp;
-            const float nl = l * sp + u * sn, nu = l * sn + u * sp;
-            l = nl;
-            u = nu;
-        }
-        if (add_lo) {
-            l += add_lo[e];
-            u += add_up[e];
-        }
-        if (shift) {
-            const float t = shift[e % H];
-            l += t;
-            u += t;
-        }
-        out_lo[e] = l;
-        out_up[e] = u;
-    }
-}
-
-// dst[r, :] = sum_h src[r, h] for every h (torch.sum(dim=-1, keepdim=True).repeat, Bounds.py:1009-1012):
-// a wavefront per row, cross-lane butterfly, broadcast store.
-__global__ void __launch_bounds__(256) rowsum_broadcast_kernel(const float *__restrict__ src, float *__restrict__ dst,
-                                                               long long rows, int H) {
-    const long long r = (long long)blockIdx.x * 4 + threadIdx.x / WAVE;
-    if (r >= rows) return;
-    const int lane = threadIdx.x % WAVE;
-    const float *p = src + (size_t)r * H;
-    float s = 0.f;
-    for (int h = lane; h < H; h += WAVE) s += p[h];
-#pragma unroll
-    for (int m = WAVE / 2; m > 0; m >>= 1) s += __shfl_xor(s, m, WAVE);
-    float *q = dst + (size_t)r * H;
-    for (int h = lane; h < H; h += WAVE) q[h] = s;
-}
-
 }  // namespace
 
 extern "C" int faith_multiply_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
@@ -392,27 +341,4 @@ extern "C" int faith_multiply_verification(const float *x_lb, const float *x_ub,
     else if (q == FAITH_Q_2) dispatch_mul<FAITH_Q_2>(a, st);
     else dispatch_mul<FAITH_Q_INF>(a, st);
     return faith::check_launch("faith_multiply_verification");
-}
-
-extern "C" int faith_scale_add(const float *lo, const float *up, const float *scale, float scalar,
-                               const float *add_lo, const float *add_up, const float *shift, float *out_lo,
-                               float *out_up, long long n, int period, void *stream) {
-    FAITH_NOT_NULL(lo); FAITH_NOT_NULL(up); FAITH_NOT_NULL(out_lo); FAITH_NOT_NULL(out_up);
-    FAITH_REQUIRE(n > 0 && period > 0, FAITH_ERR_SHAPE, "faith_scale_add: n=%lld period=%d must be positive", n, period);
-    FAITH_REQUIRE((add_lo == nullptr) == (add_up == nullptr), FAITH_ERR_NULL,
-                  "faith_scale_add: add_lo and add_up must be given together");
-    const long long blocks = (n + 255) / 256;
-    hipLaunchKernelGGL(scale_add_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), lo, up, scale, scalar, add_lo, add_up, shift, out_lo, out_up,
-                       (size_t)n, period);
-    return faith::check_launch("faith_scale_add");
-}
-
-extern "C" int faith_rowsum_broadcast(const float *src, float *dst, long long rows, int dim_out, void *stream) {
-    FAITH_NOT_NULL(src); FAITH_NOT_NULL(dst);
-    FAITH_REQUIRE(rows > 0 && dim_out > 0 && (rows + 3) / 4 <= 0x7fffffffLL, FAITH_ERR_SHAPE,
-                  "faith_rowsum_broadcast: rows=%lld dim_out=%d out of range", rows, dim_out);
-    hipLaunchKernelGGL(rowsum_broadcast_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), src, dst, rows, dim_out);
-    return faith::check_launch("faith_rowsum_broadcast");
 }

@@ -74,6 +74,11 @@ def bound_attention(bounds_input, attention):
     query = bounds_input.dense(attention.self.query)
     key = bounds_input.dense(attention.self.key)
     value = bounds_input.dense(attention.self.value)
+    if hasattr(query, "attention_scores"):
+        # the HIP kernels address the heads where the dense layers leave them: no permuted copies
+        scores = query.attention_scores(key, heads).multiply(1.0 / math.sqrt(size))
+        probs = scores.softmax()
+        return scores, probs, probs.attention_context(value)
     _fold_heads(query, heads, size)
     _fold_heads(key, heads, size)
     scores = query.dot_product(key).multiply(1.0 / math.sqrt(size))

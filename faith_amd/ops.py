@@ -173,60 +173,89 @@ def multiply(x, y, p, eps, words=1, out=None):
     return zlw, zlb, zuw, zub
 
 
-def _scale_add_pair(lo, up, scale, scalar, add_lo, add_up, shift, period):
-    out_lo, out_up = torch.empty_like(lo), torch.empty_like(up)
-    with _on(lo.device):
-        _lib.call("faith_scale_add", _ptr(lo), _ptr(up), _ptr(scale), float(scalar), _ptr(add_lo), _ptr(add_up),
-                  _ptr(shift), _ptr(out_lo), _ptr(out_up), lo.numel(), int(period), _stream(lo))
-    return out_lo, out_up
+def _object(lw, lb, uw, ub, what="x"):
+    """Checks the four tensors of one bound object; returns (rows_w, rows_b, H)."""
+    _check(f"{what}.lw", lw); _check(f"{what}.uw", uw, lw.shape); _check(f"{what}.lb", lb); _check(f"{what}.ub", ub, lb.shape)
+    H = lw.shape[-1]
+    if lb.shape[-1] != H:
+        raise ValueError(f"{what}: lw {tuple(lw.shape)} and lb {tuple(lb.shape)} disagree in the last axis")
+    return lw.numel() // H, lb.numel() // H, H
+
+
+def affine(x, scale=None, other=None, shift=None):
+    """Bounds.multiply by a float or a per-neuron tensor, Bounds.add with another object and / or a
+    per-neuron tensor (which moves the constant terms only) -- any combination, one launch.
+    x, other: (lw, lb, uw, ub)."""
+    lw, lb, uw, ub = x
+    rows_w, rows_b, H = _object(lw, lb, uw, ub)
+    vec, scalar = None, 1.0
+    if isinstance(scale, torch.Tensor):
+        _check("scale", scale, (H,))
+        vec = scale
+    elif scale is not None:
+        scalar = float(scale)
+    if other is not None:
+        _check("other.lw", other[0], lw.shape); _check("other.uw", other[2], lw.shape)
+        _check("other.lb", other[1], lb.shape); _check("other.ub", other[3], lb.shape)
+        alw, alb, auw, aub = other
+    else:
+        alw = alb = auw = aub = None
+    if shift is not None:
+        if not isinstance(shift, torch.Tensor):
+            shift = torch.full((H,), float(shift), device=lb.device, dtype=torch.float32)
+        _check("shift", shift, (H,))
+    olb, oub = torch.empty_like(lb), torch.empty_like(ub)
+    if scale is None and other is None:
+        # a shift moves the constant terms only: the coefficient tensors are shared, as in the reference
+        olw, ouw, rows_w = lw, uw, 0
+    else:
+        olw, ouw = torch.empty_like(lw), torch.empty_like(uw)
+    with _on(lw.device):
+        _lib.call("faith_affine_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(vec), scalar,
+                  _ptr(alb), _ptr(aub), _ptr(alw), _ptr(auw), _ptr(shift), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
+                  rows_w, rows_b, H, _stream(lw))
+    return olw, olb, ouw, oub
 
 
 def scale(lw, lb, uw, ub, W):
     """Bounds.multiply with a float or a per-neuron tensor W [H] (sign-split elementwise scaling)."""
-    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
-    H = lw.shape[-1]
-    if isinstance(W, torch.Tensor):
-        _check("W", W, (H,))
-        vec, scalar = W, 1.0
-    else:
-        vec, scalar = None, float(W)
-    olw, ouw = _scale_add_pair(lw, uw, vec, scalar, None, None, None, H)
-    olb, oub = _scale_add_pair(lb, ub, vec, scalar, None, None, None, H)
-    return olw, olb, ouw, oub
+    return affine((lw, lb, uw, ub), scale=W)
 
 
 def add(x, y):
     """Bounds.add with a Bounds argument: elementwise sum of two objects."""
-    xlw, xlb, xuw, xub = x
-    ylw, ylb, yuw, yub = y
-    for n, t, s_ in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
-                     ("y.lw", ylw, xlw.shape), ("y.uw", yuw, xlw.shape), ("y.lb", ylb, xlb.shape),
-                     ("y.ub", yub, xlb.shape)):
-        _check(n, t, s_)
-    H = xlw.shape[-1]
-    olw, ouw = _scale_add_pair(xlw, xuw, None, 1.0, ylw, yuw, None, H)
-    olb, oub = _scale_add_pair(xlb, xub, None, 1.0, ylb, yub, None, H)
+    return affine(x, other=y)
+
+
+def shift(lw, lb, uw, ub, delta):
+    """Bounds.add with a float or a tensor [H]: moves the constant terms only."""
+    return affine((lw, lb, uw, ub), shift=delta)
+
+
+def rowsum(lw, lb, uw, ub):
+    """Sum over the last axis, written to every position of that axis, for all four tensors
+    (the sum / repeat pair of Bounds.softmax)."""
+    rows_w, rows_b, H = _object(lw, lb, uw, ub)
+    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    with _on(lw.device):
+        _lib.call("faith_rowsum_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw),
+                  _ptr(ouw), rows_w, rows_b, H, _stream(lw))
     return olw, olb, ouw, oub
 
 
-def shift(lb, ub, delta):
-    """Bounds.add with a float or a tensor [H]: moves the constant terms only."""
-    _check("lb", lb); _check("ub", ub, lb.shape)
-    H = lb.shape[-1]
-    if not isinstance(delta, torch.Tensor):
-        delta = torch.full((H,), float(delta), device=lb.device, dtype=torch.float32)
-    _check("delta", delta, (H,))
-    return _scale_add_pair(lb, ub, None, 1.0, None, None, delta, H)
-
-
-def rowsum_broadcast(t):
-    """sum over the last axis, written to every position of that axis."""
-    _check("t", t)
-    out = torch.empty_like(t)
-    H = t.shape[-1]
-    with _on(t.device):
-        _lib.call("faith_rowsum_broadcast", _ptr(t), _ptr(out), t.numel() // H, H, _stream(t))
-    return out
+def layer_norm(lw, lb, uw, ub, weight=None, bias=None):
+    """Mean subtraction along the last axis, then per-neuron weight (split by sign) and bias:
+    Bounds.layer_norm in mode "no_var"; with weight = bias = None its first step in mode "standard"."""
+    rows_w, rows_b, H = _object(lw, lb, uw, ub)
+    if weight is not None:
+        _check("weight", weight, (H,))
+    if bias is not None:
+        _check("bias", bias, (H,))
+    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    with _on(lw.device):
+        _lib.call("faith_layer_norm_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
+                  _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), rows_w, rows_b, H, _stream(lw))
+    return olw, olb, ouw, oub
 
 
 def linear(lw, lb, uw, ub, weight, bias=None, out=None):
@@ -322,6 +351,71 @@ def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
                   _stream(xlw))
     if return_intervals:
         return zlw, zlb, zuw, zub, (x_l, x_u, y_l, y_u)
+    return zlw, zlb, zuw, zub
+
+
+def attention_scores(x, y, heads, p, eps, words=1):
+    """Scores of all heads from query / key bounds as the dense layers leave them.
+
+    x, y: (lw [1, L, D, heads*size], lb [1, L, heads*size], uw, ub).  Same result as folding both with
+    transpose_for_scores (VerifierForward.py:208-229) and dot_product_qk, without the eight permuted
+    copies: returns (lw [heads, Lx, D, Ly], lb [heads, Lx, Ly], uw, ub)."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    B, Lx, D, H = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    B2, Ly, D2, H2 = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
+    if B != 1 or B2 != 1 or (D2, H2) != (D, H):
+        raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} must be [1, L, dim_in, heads*size] alike")
+    if heads <= 0 or H % heads:
+        raise ValueError(f"{heads} heads do not divide a row of {H}")
+    for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                    ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
+        _check(n, t, s)
+    dev = xlw.device
+    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
+    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
+    zlw = torch.empty(heads, Lx, D, Ly, device=dev, dtype=torch.float32)
+    zuw = torch.empty_like(zlw)
+    zlb = torch.empty(heads, Lx, Ly, device=dev, dtype=torch.float32)
+    zub = torch.empty_like(zlb)
+    with _on(dev):
+        _lib.call("faith_attention_scores", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
+                  _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
+                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), heads, Lx, Ly, H // heads, D, float(eps), q_code(p),
+                  int(words), _stream(xlw))
+    return zlw, zlb, zuw, zub
+
+
+def attention_context(x, y, p, eps, words=1):
+    """Context of all heads: probabilities x (lw [heads, Lx, D, Lk], lb [heads, Lx, Lk], uw, ub) times the
+    value bounds y as the dense layer leaves them (lw [1, Lk, D, heads*size], lb [1, Lk, heads*size], uw, ub).
+
+    Same result as transpose_for_scores on y, dot_product_v and transpose_back
+    (VerifierForward.py:208-229, :253-263) without the permuted copies: returns
+    (lw [1, Lx, D, heads*size], lb [1, Lx, heads*size], uw, ub)."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    heads, Lx, D, Lk = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    B2, Lk2, D2, H = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
+    if B2 != 1 or (Lk2, D2) != (Lk, D):
+        raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} disagree in key length or dim_in")
+    if H % heads:
+        raise ValueError(f"{heads} heads do not divide a row of {H}")
+    for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                    ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
+        _check(n, t, s)
+    dev = xlw.device
+    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
+    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
+    zlw = torch.empty(1, Lx, D, H, device=dev, dtype=torch.float32)
+    zuw = torch.empty_like(zlw)
+    zlb = torch.empty(1, Lx, H, device=dev, dtype=torch.float32)
+    zub = torch.empty_like(zlb)
+    with _on(dev):
+        _lib.call("faith_attention_context", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
+                  _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
+                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), heads, Lx, Lk, H // heads, D, float(eps), q_code(p),
+                  int(words), _stream(xlw))
     return zlw, zlb, zuw, zub
 
 

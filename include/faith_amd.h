@@ -133,21 +133,46 @@ int faith_multiply_verification(const float *x_lb, const float *x_ub, const floa
                                 int q, int words, void *stream);
 
 /*
- * out_lo[e] = lo[e] * s+ + up[e] * s- (+ add_lo[e]) (+ shift[e % period]),  out_up mirrored, with
- * s = scale[e % period] when scale is given, else `scalar`;  s+ = s * (s > 0), s- = s - s+.
- * One kernel behind Bounds.multiply with a float or a tensor (Bounds.py:595-607, :653-664) and
- * Bounds.add (:383-395); called once for (lw, uw) and once for (lb, ub).  scale, add_lo / add_up and
- * shift may be NULL; out may alias the inputs.
+ * The next three take a whole bound object -- rows_w coefficient rows (length * dim_in) and rows_b
+ * constant rows (length), each dim_out long -- and handle all four tensors in one launch.  The
+ * reference builds them from PyTorch expressions; there is no CUDA counterpart.  out may alias src.
+ *
+ * Scale, add, shift: Bounds.multiply with a float or a per-neuron tensor (Bounds.py:595-607,
+ * :653-664) and Bounds.add with an object or a tensor (:383-395), alone or combined:
+ *   out_l = src_l * s+ + src_u * s- (+ add_l) (+ shift on the constant rows only),  out_u mirrored,
+ * with s = scale[h] when scale is given, else `scalar`;  s+ = s * (s > 0), s- = s - s+.
+ * scale, shift and the added object may be NULL (the added object's four tensors together).
  */
-int faith_scale_add(const float *lo, const float *up, const float *scale, float scalar,
-                    const float *add_lo, const float *add_up, const float *shift,
-                    float *out_lo, float *out_up, long long n, int period, void *stream);
+int faith_affine_verification(const float *src_lb, const float *src_ub,
+                              const float *src_lw, const float *src_uw,
+                              const float *scale, float scalar,
+                              const float *add_lb, const float *add_ub,
+                              const float *add_lw, const float *add_uw,
+                              const float *shift,
+                              float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                              long long rows_w, long long rows_b, int dim_out, void *stream);
 
 /*
- * dst[r, :] = sum over h of src[r, h], written to every h: the sum / repeat pair of Bounds.softmax
- * (Bounds.py:1009-1012) without the intermediate.
+ * out[r, :] = sum over h of src[r, h], written to every h: the sum / repeat pair of
+ * Bounds.softmax (Bounds.py:1009-1012) without the intermediate.
  */
-int faith_rowsum_broadcast(const float *src, float *dst, long long rows, int dim_out, void *stream);
+int faith_rowsum_verification(const float *src_lb, const float *src_ub,
+                              const float *src_lw, const float *src_uw,
+                              float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                              long long rows_w, long long rows_b, int dim_out, void *stream);
+
+/*
+ * Layer normalisation without the variance (Bounds.layer_norm, Bounds.py:1111-1131, mode "no_var",
+ * and the first step of mode "standard"): subtract the row mean -- the mean of the UPPER tensor
+ * from the lower one and the reverse, as matmul(ones / H).multiply(-1.) gives it -- then scale by
+ * weight[h] split by sign and add bias[h] to the constant rows.  weight and bias may be NULL
+ * (NULL weight: mean subtraction only).
+ */
+int faith_layer_norm_verification(const float *src_lb, const float *src_ub,
+                                  const float *src_lw, const float *src_uw,
+                                  const float *weight, const float *bias,
+                                  float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                                  long long rows_w, long long rows_b, int dim_out, void *stream);
 
 /*
  * Sign-split affine propagation  y = x @ W^T (+ bias).  Replaces the (commented-out)
@@ -207,6 +232,45 @@ int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *
                                      int batch_size, int length_x, int length_k,
                                      int dim_out, int dim_in, float epsilon,
                                      int q, int words, void *stream);
+
+/*
+ * Attention scores with the heads taken where the dense layers leave them.  Replaces
+ * transpose_for_scores on query and key (VerifierForward.py:208-229: four permuted copies per
+ * object) followed by Bounds.dot_product (Bounds.py:833-841): the kernels address head t of
+ *   x_lw, x_uw [1, length_x, dim_in, heads * head_size];  x_lb, x_ub [1, length_x, heads * head_size]
+ *   y_lw, y_uw [1, length_y, dim_in, heads * head_size];  y_lb, y_ub [1, length_y, heads * head_size]
+ * in place.  x_l, x_u / y_l, y_u (out, caller's scratch) have the layout of x_lb / y_lb.  The
+ * scores come out with the heads stacked on the batch axis, as the softmax wants them:
+ *   z_lw, z_uw [heads, length_x, dim_in, length_y];  z_lb, z_ub [heads, length_x, length_y]
+ */
+int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u,
+                           const float *x_lb, const float *x_ub,
+                           const float *y_lb, const float *y_ub,
+                           const float *x_lw, const float *x_uw,
+                           const float *y_lw, const float *y_uw,
+                           float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                           int heads, int length_x, int length_y,
+                           int head_size, int dim_in, float epsilon,
+                           int q, int words, void *stream);
+
+/*
+ * Attention context with the values read, and the result written, where the dense layers want
+ * them.  Replaces transpose_for_scores on the values, Bounds.context (Bounds.py:843-850) and
+ * transpose_back (VerifierForward.py:253-263).
+ *   x_lw, x_uw [heads, length_x, dim_in, length_k];  x_lb, x_ub [heads, length_x, length_k]   (probabilities)
+ *   y_lw, y_uw [1, length_k, dim_in, heads * head_size];  y_lb, y_ub [1, length_k, heads * head_size]
+ *   x_l, x_u like x_lb;  y_l, y_u like y_lb   (out / scratch)
+ *   z_lw, z_uw [1, length_x, dim_in, heads * head_size];  z_lb, z_ub [1, length_x, heads * head_size]
+ */
+int faith_attention_context(float *x_l, float *y_l, float *x_u, float *y_u,
+                            const float *x_lb, const float *x_ub,
+                            const float *y_lb, const float *y_ub,
+                            const float *x_lw, const float *x_uw,
+                            const float *y_lw, const float *y_uw,
+                            float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                            int heads, int length_x, int length_k,
+                            int head_size, int dim_in, float epsilon,
+                            int q, int words, void *stream);
 
 /*
  * Sign-split propagation through a 2-D convolution (NCHW).  Replaces the (commented-out)

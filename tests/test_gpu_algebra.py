@@ -93,14 +93,51 @@ def test_layer_norm(mode, p):
     assert_bounds_close(got, exp, rtol=1e-4, atol=2e-5, what=f"layer_norm/{mode}")
 
 
-def test_rowsum_broadcast():
+def test_rowsum_of_a_whole_object():
     from faith_amd import ops
     g = torch.Generator().manual_seed(65)
-    for shape in [(2, 3, 7, 64), (1, 5, 100), (3, 1, 2, 5)]:
-        t = torch.randn(*shape, generator=g)
-        out = ops.rowsum_broadcast(t.cuda())
-        exp = t.sum(-1, keepdim=True).expand_as(t)
-        assert close(out, exp, rtol=1e-5, atol=2e-6)
+    # last axis: vector path, scalar path, longer than a wavefront keeps in registers (both paths)
+    for B, L, D, H in [(2, 3, 7, 64), (1, 5, 3, 100), (3, 1, 2, 5), (1, 2, 3, 1284), (1, 2, 2, 330)]:
+        x = rand_bounds(g, B, L, D, H, ordered=False)
+        out = ops.rowsum(*(t.cuda() for t in x.tensors()))
+        for a, t in zip(out, x.tensors()):
+            assert close(a, t.sum(-1, keepdim=True).expand_as(t), rtol=1e-5, atol=1e-5 * H ** 0.5)
+
+
+@pytest.mark.parametrize("H", [64, 10, 1284, 330])
+@pytest.mark.parametrize("with_affine", [True, False])
+def test_fused_mean_subtraction_against_float64(H, with_affine):
+    """faith_layer_norm_verification against the definition in float64: c_l = l - mean(u),
+    c_u = u - mean(l), then weight split by sign and bias on the constant terms."""
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(66)
+    x = rand_bounds(g, 1, 5, 6, H, ordered=False)
+    weight = torch.randn(H, generator=g) if with_affine else None
+    bias = torch.randn(H, generator=g) if with_affine else None
+    if with_affine:
+        weight[1] = 0.0
+    got = ops.layer_norm(*(t.cuda() for t in x.tensors()), None if weight is None else weight.cuda(),
+                         None if bias is None else bias.cuda())
+    lw, lb, uw, ub = (t.double() for t in x.tensors())
+
+    def centre(lo, up):
+        return lo - up.mean(-1, keepdim=True), up - lo.mean(-1, keepdim=True)
+    (clw, cuw), (clb, cub) = centre(lw, uw), centre(lb, ub)
+    if with_affine:
+        wp, wn = weight.double().clamp(min=0), weight.double().clamp(max=0)
+        clw, cuw = clw * wp + cuw * wn, clw * wn + cuw * wp
+        clb, cub = clb * wp + cub * wn + bias.double(), clb * wn + cub * wp + bias.double()
+    for a, e in zip(got, (clw, clb, cuw, cub)):
+        assert close(a, e, rtol=1e-5, atol=2e-6)
+
+
+def test_shift_shares_the_coefficients():
+    """Bounds.add with a tensor returns the same lw / uw tensors (Bounds.py:391-395 does too)."""
+    g = torch.Generator().manual_seed(67)
+    x = gpu_bounds(rand_bounds(g, 1, 3, 4, 8), 2.0, 0.1)
+    y = x.add(0.5)
+    assert y.lw.data_ptr() == x.lw.data_ptr() and y.uw.data_ptr() == x.uw.data_ptr()
+    assert torch.equal(y.lb, x.lb + 0.5) and torch.equal(y.ub, x.ub + 0.5)
 
 
 @pytest.mark.gpu

@@ -258,3 +258,74 @@ def test_c_bound_dot_shims():
     e = O.context(probs, value, 2.0, 0.05)
     assert close(zlw.transpose(2, 3), e.lw, rtol=1e-5, atol=2e-6) and close(zlb, e.lb, rtol=1e-5, atol=2e-6)
     assert close(zuw.transpose(2, 3), e.uw, rtol=1e-5, atol=2e-6) and close(zub, e.ub, rtol=1e-5, atol=2e-6)
+
+
+# ------------------------------------------------------------------ heads addressed in place
+def side_by_side(x):
+    """[heads, L, D, w] / [heads, L, w] -> the one object [1, L, D, heads*w] / [1, L, heads*w] that a
+    dense layer produces (inverse of transpose_for_scores, VerifierForward.py:208-229)."""
+    w = lambda t: t.permute(1, 2, 0, 3).reshape(1, t.shape[1], t.shape[2], -1).contiguous()
+    b = lambda t: t.permute(1, 0, 2).reshape(1, t.shape[1], -1).contiguous()
+    return O.LinearBounds(w(x.lw), b(x.lb), w(x.uw), b(x.ub))
+
+
+@pytest.mark.parametrize("shape", [
+    # heads, Lx, Ly, D, head size
+    (4, 128, 128, 16, 64),      # straight-line MFMA kernel
+    (2, 130, 70, 20, 36),       # ragged tiles, half-empty last K-step
+    (4, 32, 32, 64, 16),        # short sequences: one 32 x 32 block per wavefront
+    (3, 6, 4, 5, 10),           # head size % 4 != 0: any-shape kernel
+    (2, 3, 5, 1, 8),            # dim_in == 1: interval shortcut
+])
+@pytest.mark.parametrize("p", [2.0, INF])
+def test_attention_scores_reads_the_heads_in_place(shape, p):
+    from faith_amd import ops
+    heads, Lx, Ly, D, d = shape
+    g = torch.Generator().manual_seed(41)
+    x = rand_bounds(g, heads, Lx, D, d, ordered=False, sw=0.3, sb=1.0)
+    y = rand_bounds(g, heads, Ly, D, d, ordered=False, sw=0.3, sb=1.0)
+    words = 2 if D % 2 == 0 else 1
+    print(f"[case] attention_scores heads={heads} Lx={Lx} Ly={Ly} D={D} size={d} p={p} words={words}", flush=True)
+    got = ops.attention_scores(dev(side_by_side(x)), dev(side_by_side(y)), heads, p, 0.1, words)
+    torch.cuda.synchronize()
+    exp = O.dot_product(x, y, p, 0.1, words)
+    if D == 1:
+        for a, e in zip(got, exp.tensors()):
+            assert close(a, e)
+        return
+    ref, mag = dot64(x, y, p, 0.1, words)
+    for name, a, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
+        assert a.shape == e.shape
+        compare_contraction(name, a, e, ref[name], mag[name])
+
+
+@pytest.mark.parametrize("shape", [
+    # heads, queries, keys, D, head size
+    (4, 128, 128, 16, 64), (2, 128, 64, 8, 128),    # straight-line MFMA kernel
+    (2, 130, 72, 12, 20),       # ragged
+    (4, 32, 32, 64, 16),        # short sequences
+    (3, 6, 6, 4, 10),           # any-shape kernel
+    (2, 4, 4, 1, 8),            # interval shortcut
+])
+@pytest.mark.parametrize("p", [2.0, INF])
+def test_attention_context_reads_and_writes_the_heads_in_place(shape, p):
+    from faith_amd import ops
+    heads, Lq, Lk, D, dv = shape
+    g = torch.Generator().manual_seed(42)
+    probs = rand_bounds(g, heads, Lq, D, Lk, ordered=False, sw=0.2, sb=0.5)
+    value = rand_bounds(g, heads, Lk, D, dv, ordered=False, sw=0.3, sb=1.0)
+    print(f"[case] attention_context heads={heads} Lq={Lq} Lk={Lk} D={D} size={dv} p={p}", flush=True)
+    got = ops.attention_context(dev(probs), dev(side_by_side(value)), p, 0.1, 1)
+    torch.cuda.synchronize()
+    exp = O.context(probs, value, p, 0.1, 1)
+    exp_sbs = side_by_side(exp)
+    if D == 1:
+        for a, e in zip(got, exp_sbs.tensors()):
+            assert close(a, e)
+        return
+    ref, mag = dot64(probs, O.transpose_bounds(value), p, 0.1, 1)
+    wrap = lambda r: side_by_side(O.LinearBounds(r["lw"], r["lb"], r["uw"], r["ub"]))
+    ref_s, mag_s = wrap(ref), wrap(mag)
+    for name, a, e, r, m in zip(("lw", "lb", "uw", "ub"), got, exp_sbs.tensors(), ref_s.tensors(), mag_s.tensors()):
+        assert a.shape == e.shape
+        compare_contraction(name, a, e, r, m)
