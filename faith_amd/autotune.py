@@ -1,0 +1,354 @@
+"""Kernel-variant autotuner: heuristics propose, a cost model ranks, the GPU decides.
+
+Counterpart of the reference's autotuner (autotuner/autotuner.py:99-147: rounds of sampling, the
+first at random and the later ones ranked by a learned cost model; expert_knowledge_metafile.py:
+16-80, :96-190: a hardware "metafile" and validity heuristics such as "the block tile fits in
+shared memory" and "the warp tile fits in registers"; cost_model.py: a regressor on
+[implementation parameters + metafile]).  The reference rewrites matmul_config.h and recompiles
+for every sample; here the variants are template instantiations that are already in
+libfaith_amd.so and are selected per call through faith_tune_set, so a sample costs a few launches.
+
+What can be tuned (see the FAITH_TUNE_* knobs in include/faith_amd.h):
+
+    linear       macro-tile of the sign-split GEMM: 64x64, 128x128, 128x64, 64x128
+    dot_qk/dot_v 128x64 persistent tiles, or one 32x32 block per wavefront with 1..16 perturbation
+                 coordinates per wavefront
+    act          tile shape of the relaxation kernels (relu, tanh, exp, ...)
+    concretize   tile shape of the concretize kernel
+
+Results are kept in a TuningTable keyed by (operator, shape); `use(table)` makes the wrappers in
+faith_amd.ops apply an entry around the matching call.  Results never depend on the variant, only
+speed does.
+"""
+from __future__ import annotations
+
+import contextlib
+import json
+import random
+from dataclasses import dataclass, field
+
+import numpy as np
+
+# knob numbers of include/faith_amd.h
+TUNE_ACT_VARIANT, TUNE_GEMM_VARIANT, TUNE_DOT_VARIANT, TUNE_DOT_COORDS = 0, 1, 2, 3
+
+# Hardware description the heuristics and the cost model see (the reference's a100_metafile).
+mi355x_metafile = {
+    "COMPUTE_UNITS": 256,
+    "MAX_LDS_KB": 160,              # per compute unit
+    "MAX_NUM_REGISTER_PER_LANE": 512,   # vector + accumulator registers of one wavefront
+    "MAX_WAVES_PER_SIMD": 8,
+    "SIMDS_PER_CU": 4,
+    "XCDS": 8,
+}
+
+
+def metafile_of_device(index=0):
+    """The metafile with the compute-unit count of the GPU that is present."""
+    import torch
+    m = dict(mi355x_metafile)
+    m["COMPUTE_UNITS"] = torch.cuda.get_device_properties(index).multi_processor_count
+    return m
+
+
+@dataclass(frozen=True)
+class Candidate:
+    """One implementation choice: knob settings plus the quantities the heuristics reason about."""
+    knobs: tuple                    # ((knob, value), ...)
+    params: tuple                   # ((name, number), ...): tile sizes, LDS bytes, registers, ...
+
+    def knob_dict(self):
+        return dict(self.knobs)
+
+    def param(self, name, default=0.0):
+        return dict(self.params).get(name, default)
+
+
+def _cand(knobs, **params):
+    return Candidate(tuple(sorted(knobs.items())), tuple(sorted(params.items())))
+
+
+class Heuristics:
+    """Proposes candidates for an (operator, shape) and rejects the ones that cannot be good
+    (expert_knowledge_metafile.py:36-190 plays this role for the CUTLASS tile parameters)."""
+
+    OPERATORS = ("linear", "dot_qk", "dot_v", "act", "concretize")
+
+    def __init__(self, metafile=None):
+        self.metafile = dict(mi355x_metafile if metafile is None else metafile)
+
+    # ---- checks shared by the operators
+    def check_lds(self, lds_bytes):
+        return lds_bytes <= self.metafile["MAX_LDS_KB"] * 1024
+
+    def check_registers(self, registers_per_lane):
+        return registers_per_lane <= self.metafile["MAX_NUM_REGISTER_PER_LANE"]
+
+    def resident_workgroups(self, lds_bytes, registers_per_lane, waves_per_group=4):
+        """Workgroups one compute unit can hold at a time."""
+        by_lds = (self.metafile["MAX_LDS_KB"] * 1024) // max(lds_bytes, 1)
+        waves = min(self.metafile["MAX_WAVES_PER_SIMD"],
+                    self.metafile["MAX_NUM_REGISTER_PER_LANE"] // max(registers_per_lane, 1))
+        by_regs = waves * self.metafile["SIMDS_PER_CU"] // waves_per_group
+        return max(0, min(by_lds, by_regs))
+
+    # ---- proposals
+    def propose(self, op, shape):
+        """All candidates for the operator, valid or not."""
+        if op == "linear":
+            rows, k, n = shape
+            out = []
+            for variant, (tm, tn) in {1: (64, 64), 2: (128, 128), 3: (128, 64), 4: (64, 128)}.items():
+                lds = 2 * 2 * 16 * (tm + tn) * 4            # two stages; A_l, A_u [tm x 16] and W+, W- [tn x 16] floats
+                acc = 2 * (tm // 2) * (tn // 2) // 64 * 1   # accumulator registers per lane for C_l and C_u
+                tiles = -(-rows // tm) * -(-n // tn)
+                out.append(_cand({TUNE_GEMM_VARIANT: variant}, tile_m=tm, tile_n=tn, lds_bytes=lds,
+                                 registers=acc + 40 + 12 * (tm + tn) // 64, workgroups=tiles,
+                                 padding=(-(-rows // tm) * tm * -(-n // tn) * tn) / float(rows * n) - 1.0,
+                                 steps=-(-k // 16), mfma_per_step=(tm // 64) * (tn // 64) * 32))
+            return out
+        if op in ("dot_qk", "dot_v"):
+            batch, lx, ly, d_in, d = shape
+            out = [_cand({TUNE_DOT_VARIANT: 1}, tile_m=128, tile_n=64, lds_bytes=2 * (4 * 128 + 6 * 64) * 8 * 4,
+                         registers=232, workgroups=batch * d_in * -(-lx // 128) * -(-ly // 64),
+                         padding=(-(-lx // 128) * 128 * -(-ly // 64) * 64) / float(lx * ly) - 1.0,
+                         steps=-(-d // 8), mfma_per_step=64, coords=0)]
+            blocks = batch * -(-lx // 32) * -(-ly // 32)
+            for coords in (1, 2, 3, 4, 6, 8, 12, 16):
+                out.append(_cand({TUNE_DOT_VARIANT: 2, TUNE_DOT_COORDS: coords}, tile_m=32, tile_n=32,
+                                 lds_bytes=6 * 32 * d * 4, registers=166,
+                                 workgroups=blocks * -(-d_in // (4 * coords)),
+                                 padding=(-(-lx // 32) * 32 * -(-ly // 32) * 32) / float(lx * ly) - 1.0,
+                                 steps=-(-d // 8) * coords, mfma_per_step=32, coords=coords))
+            return out
+        if op == "act":
+            rows, d_in, h = shape
+            table = {0: (32, 32, 256), 9: (32, 256, 256), 1: (32, 256, 256), 2: (64, 256, 512), 3: (64, 256, 1024),
+                     4: (32, 256, 512), 5: (64, 256, 256)}   # neurons per tile, rows per pass, threads
+            out = []
+            for variant, (neurons, chunk, threads) in table.items():
+                held = min(d_in, chunk) * neurons * 2 // threads       # values a thread keeps between its two passes
+                out.append(_cand({TUNE_ACT_VARIANT: variant}, tile_n=neurons, chunk=chunk, threads=threads,
+                                 registers=held + 40, lds_bytes=8 * neurons * (threads // 64),
+                                 workgroups=rows * -(-h // neurons), resident=1.0 if variant == 0 else 0.0))
+            return out
+        if op == "concretize":
+            rows, d_in, h = shape
+            return [_cand({TUNE_ACT_VARIANT: v}, tile_n=n, threads=t, registers=48, lds_bytes=8 * n * (t // 64),
+                          workgroups=rows * -(-h // n))
+                    for v, (n, t) in {0: (64, 1024), 11: (64, 256), 13: (32, 256)}.items()]
+        raise ValueError(f"unknown operator {op!r}; one of {self.OPERATORS}")
+
+    def is_valid(self, op, shape, cand):
+        """Fits the machine and is not mostly padding."""
+        if not self.check_lds(cand.param("lds_bytes")) or not self.check_registers(cand.param("registers")):
+            return False
+        if op == "linear":
+            # a tile more than twice the problem in either direction is padding only
+            rows, _, n = shape
+            return cand.param("tile_m") < 2 * max(rows, 64) and cand.param("tile_n") < 2 * max(n, 64)
+        if op in ("dot_qk", "dot_v"):
+            _, lx, ly, _, d = shape
+            if cand.knob_dict().get(TUNE_DOT_VARIANT) == 2:
+                # the per-wavefront kernel keeps the six sign-split operands of the whole reduction in LDS
+                return d % 8 == 0 and d <= 80 and cand.param("padding") < 1.0
+            return True
+        if op == "act":
+            _, d_in, h = shape
+            if cand.knob_dict().get(TUNE_ACT_VARIANT) == 0:
+                return True                                  # the built-in choice is always available
+            return h % 4 == 0
+        return True
+
+    def candidates(self, op, shape):
+        return [c for c in self.propose(op, shape) if self.is_valid(op, shape, c)]
+
+    # ---- features for the cost model: implementation parameters, shape, metafile
+    FEATURES = ("tile_m", "tile_n", "lds_bytes", "registers", "workgroups", "padding", "steps", "mfma_per_step",
+                "coords", "chunk", "threads", "resident")
+
+    def features(self, op, shape, cand):
+        cus = self.metafile["COMPUTE_UNITS"]
+        resident = self.resident_workgroups(cand.param("lds_bytes"), cand.param("registers"))
+        rounds = cand.param("workgroups") / float(max(1, resident * cus))
+        own = [float(cand.param(name)) for name in self.FEATURES]
+        derived = [rounds, float(np.ceil(rounds)), float(resident)]
+        return np.array(own + derived + [float(s) for s in shape] + [float(v) for v in self.metafile.values()])
+
+
+class CostModel:
+    """Ridge regression of log-latency on standardised features (the reference trains an XGBoost
+    regressor, cost_model.py:15-21; with a handful of samples per shape a linear model ranks as well
+    and needs nothing beyond numpy)."""
+
+    def __init__(self, ridge=1e-2):
+        self.ridge = ridge
+        self.mean = self.scale = self.weights = None
+
+    def fit(self, features, latencies):
+        x = np.asarray(features, dtype=np.float64)
+        y = np.log(np.asarray(latencies, dtype=np.float64))
+        self.mean = x.mean(axis=0)
+        self.scale = x.std(axis=0)
+        self.scale[self.scale == 0] = 1.0
+        z = np.hstack([(x - self.mean) / self.scale, np.ones((x.shape[0], 1))])
+        reg = self.ridge * np.eye(z.shape[1])
+        reg[-1, -1] = 0.0
+        self.weights = np.linalg.solve(z.T @ z + reg, z.T @ y)
+        return self
+
+    def predict(self, features):
+        x = np.atleast_2d(np.asarray(features, dtype=np.float64))
+        z = np.hstack([(x - self.mean) / self.scale, np.ones((x.shape[0], 1))])
+        return np.exp(z @ self.weights)
+
+
+def measure_on_gpu(run, repeats=15, inner=4, warm_seconds=0.03):
+    """Latency of run() in microseconds: `inner` launches back to back between one pair of events on
+    the current stream, median over `repeats` such groups, after warming up by time (clocks take
+    milliseconds to rise after idle)."""
+    import time
+    import torch
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < warm_seconds:
+        run()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(repeats):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(inner):
+            run()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b) * 1e3 / inner)
+    return float(np.median(times))
+
+
+def _set_knobs(knobs, setter=None):
+    if setter is None:
+        from . import _lib
+        setter = lambda k, v: _lib.call("faith_tune_set", int(k), int(v))
+    for k, v in knobs.items():
+        setter(k, v)
+
+
+@contextlib.contextmanager
+def applied(knobs, setter=None):
+    """Sets the knobs for the duration of the block and restores the built-in choices afterwards."""
+    _set_knobs(knobs, setter)
+    try:
+        yield
+    finally:
+        _set_knobs({k: 0 for k in knobs}, setter)
+
+
+@dataclass
+class TuningResult:
+    op: str
+    shape: tuple
+    best: Candidate
+    best_us: float
+    measured: list = field(default_factory=list)       # [(Candidate, microseconds)], in the order measured
+    skipped: int = 0
+
+
+def autotune(op, shape, run, heuristics=None, rounds=3, samples=3, measure=None, setter=None, seed=0):
+    """Finds the fastest valid candidate for run() -- a callable that launches the operator once.
+
+    Round 0 measures `samples` candidates drawn at random; every later round fits the cost model to
+    what has been measured and measures the `samples` unmeasured candidates it predicts to be fastest
+    (autotuner.py:99-147).  The built-in choice (all knobs 0) is always among the measured ones, so the
+    result is never slower than not tuning.  measure(run) -> microseconds defaults to GPU events."""
+    heuristics = heuristics or Heuristics()
+    measure = measure or measure_on_gpu
+    rng = random.Random(seed)
+    pool = heuristics.candidates(op, shape)
+    if not pool:
+        raise ValueError(f"no valid candidate for {op} {shape}")
+    result = TuningResult(op, tuple(shape), None, float("inf"))
+    seen = set()
+
+    def take(cand):
+        seen.add(cand)
+        try:
+            with applied(cand.knob_dict(), setter):
+                us = measure(run)
+        except Exception:                                   # a variant that cannot run this shape
+            result.skipped += 1
+            return
+        result.measured.append((cand, us))
+        if us < result.best_us:
+            result.best, result.best_us = cand, us
+
+    try:
+        measure(run)        # discarded: the first measurement after idle runs at lower clocks
+    except Exception:
+        pass
+    builtin = Candidate((), (("builtin", 1.0),))
+    take(builtin)
+    for r in range(rounds):
+        rest = [c for c in pool if c not in seen]
+        if not rest:
+            break
+        fitted = [(c, us) for c, us in result.measured if c is not builtin]
+        if r == 0 or len(fitted) < 2:
+            chosen = rng.sample(rest, min(samples, len(rest)))
+        else:
+            model = CostModel().fit([heuristics.features(op, shape, c) for c, _ in fitted], [us for _, us in fitted])
+            ranked = sorted(rest, key=lambda c: float(model.predict(heuristics.features(op, shape, c))[0]))
+            chosen = ranked[:samples]
+        for cand in chosen:
+            take(cand)
+    return result
+
+
+class TuningTable:
+    """(operator, shape) -> knob settings; JSON on disk."""
+
+    def __init__(self):
+        self.entries = {}
+
+    @staticmethod
+    def key(op, shape):
+        return f"{op}:" + "x".join(str(int(s)) for s in shape)
+
+    def record(self, result):
+        self.entries[self.key(result.op, result.shape)] = {
+            "knobs": {str(k): int(v) for k, v in result.best.knob_dict().items()},
+            "microseconds": round(result.best_us, 2),
+            "measured": len(result.measured)}
+
+    def lookup(self, op, shape):
+        e = self.entries.get(self.key(op, shape))
+        return None if e is None else {int(k): int(v) for k, v in e["knobs"].items()}
+
+    def save(self, path):
+        with open(path, "w") as f:
+            json.dump(self.entries, f, indent=1, sort_keys=True)
+
+    @classmethod
+    def load(cls, path):
+        t = cls()
+        with open(path) as f:
+            t.entries = json.load(f)
+        return t
+
+
+_ACTIVE = None
+
+
+def use(table):
+    """Makes faith_amd.ops apply `table` (None: stop)."""
+    global _ACTIVE
+    _ACTIVE = table
+
+
+def tuned(op, shape):
+    """Context manager for the wrappers in faith_amd.ops: applies the active table's entry, if any."""
+    if _ACTIVE is None:
+        return contextlib.nullcontext()
+    knobs = _ACTIVE.lookup(op, shape)
+    if not knobs:
+        return contextlib.nullcontext()
+    return applied(knobs)

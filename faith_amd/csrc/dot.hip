@@ -801,7 +801,11 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
                       faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
                       (long long)TI * D * max_pitch * 4 < 0xffffffffLL &&            // 32-bit offsets inside a tile
                       (!VP || (long long)d * D * g.yp * 4 < 0xffffffffLL);           // and along K inside a head
-    if (fast && Lx <= 64 && Ly <= 64 && d % 8 == 0 && d <= 80) {
+    // short sequences take the per-wavefront kernel; the tuning knob can force either kernel
+    const bool small_ok = fast && d % 8 == 0 && d <= 80;
+    const int pick = faith::tune_get(FAITH_TUNE_DOT_VARIANT);
+    const bool small = small_ok && (pick == 2 || (pick != 1 && Lx <= 64 && Ly <= 64));
+    if (small) {
         // short sequences: one 32 x 32 block per wavefront and perturbation coordinate.  Coordinates
         // per wavefront: the count that needs the fewest rounds of resident workgroups (three per CU
         // by registers, fewer when the shared operands are large), a round costing its coordinates
@@ -815,6 +819,8 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
             const long long cost = ((wgs + resident - 1) / resident) * (2 * c + 1);
             if (best < 0 || cost < best) { best = cost; mpw = c; }
         }
+        const int forced = faith::tune_get(FAITH_TUNE_DOT_COORDS);
+        if (forced >= 1 && forced <= 16) mpw = forced;
         const long long grid = blocks * ((D + 4 * mpw - 1) / (4 * mpw));
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
         hipLaunchKernelGGL(dot_w_small<VP>, dim3((unsigned)grid), dim3(256), (size_t)6 * SB * d * sizeof(float), st, g,

@@ -86,16 +86,17 @@ __device__ __forceinline__ int swz(int row, int c) { return row * 8 + 4 * (c ^ (
 // EXACT = true: K % 16 == 0.  Otherwise (K % 4 == 0) the last K-step is partly past K: threads past
 // it read their K-step-0 piece instead (in bounds) and discard it before it reaches LDS.
 //
-// MB = MFMA blocks per wavefront and dimension: 2 is the 128 x 128 macro-tile described above; 1 is a
-// 64 x 64 macro-tile (wavefront tile 32 x 32, 32 accumulator registers, 32 KB of LDS) for problems
-// with too few 128 x 128 tiles to fill the machine: a wavefront then works through 32 MFMAs per
-// K-step instead of 128, a quarter of the latency, at a lower MFMA rate per byte staged.
-template <bool EXACT, int MB>
+// MBM, MBN = MFMA blocks per wavefront along M and N: 2 x 2 is the 128 x 128 macro-tile described
+// above; 1 x 1 is a 64 x 64 macro-tile (wavefront tile 32 x 32, 32 accumulator registers, 32 KB of LDS)
+// for problems with too few 128 x 128 tiles to fill the machine: a wavefront then works through 32
+// MFMAs per K-step instead of 128, a quarter of the latency, at a lower MFMA rate per byte staged.
+// 2 x 1 and 1 x 2 (128 x 64, 64 x 128: 64 MFMAs per K-step, 48 KB) lie between.
+template <bool EXACT, int MBM, int MBN>
 __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *smem, const int pid) {
-    constexpr int BM = 64 * MB, BN = 64 * MB;
-    constexpr int HALF = BM * 8;             // floats in one [BM x 8] half of an operand's K-step
-    constexpr int OPER = 2 * HALF;           // one operand, one K-step
-    constexpr int S_AL = 0, S_AU = OPER, S_WP = 2 * OPER, S_WN = 3 * OPER, STAGE = 4 * OPER;
+    constexpr int BM = 64 * MBM, BN = 64 * MBN;
+    constexpr int HALF_A = BM * 8, HALF_W = BN * 8;      // floats in one [rows x 8] half of an operand's K-step
+    constexpr int S_AL = 0, S_AU = 2 * HALF_A, S_WP = 4 * HALF_A, S_WN = 4 * HALF_A + 2 * HALF_W;
+    constexpr int STAGE = 4 * HALF_A + 4 * HALF_W;
     float(*sm)[STAGE] = reinterpret_cast<float(*)[STAGE]>(smem);
 
     // ---- tile of this workgroup
@@ -111,9 +112,9 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
 
     const int tid = threadIdx.x;
     const int lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
-    const int wm = wv / 2, wn = wv % 2;            // 2 x 2 wavefronts, (32 MB) x (32 MB) each
+    const int wm = wv / 2, wn = wv % 2;            // 2 x 2 wavefronts, (32 MBM) x (32 MBN) each
 
-    // ---- staging: an operand's K-step is BM rows x 16 floats = 256 MB float4, MB per thread:
+    // ---- staging: an operand's K-step is 64 or 128 rows x 16 floats, one float4 per thread and 64 rows:
     // piece kq of rows r0 (and r0 + 64).  Offsets are relative to the first row of the tile (the entry
     // point checks that a tile's rows span less than 4 GB); rows past the end re-read the last row, their
     // products are never stored.
@@ -121,82 +122,88 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
     const __amdgpu_buffer_rsrc_t wal = window(g.Al + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
     const __amdgpu_buffer_rsrc_t wau = window(g.Au + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
     const __amdgpu_buffer_rsrc_t ww = window(g.W + (size_t)n0 * K, ((size_t)(g.N - n0) * K) * 4);
-    unsigned va[MB], vw[MB];
-    int dst[MB];
+    unsigned va[MBM], vw[MBN];
+    int dsta[MBM], dstw[MBN];
 #pragma unroll
-    for (int i = 0; i < MB; ++i) {
+    for (int i = 0; i < MBM; ++i) {
         const int ra = min(r0 + 64 * i, M - 1 - m0);
-        const int rw = min(r0 + 64 * i, g.N - 1 - n0);
         va[i] = ((unsigned)ra * K + kq * 4) * 4u;
+        dsta[i] = (kq / 2) * HALF_A + swz(r0 + 64 * i, kq % 2);
+    }
+#pragma unroll
+    for (int i = 0; i < MBN; ++i) {
+        const int rw = min(r0 + 64 * i, g.N - 1 - n0);
         vw[i] = ((unsigned)rw * K + kq * 4) * 4u;
-        dst[i] = (kq / 2) * HALF + swz(r0 + 64 * i, kq % 2);
+        dstw[i] = (kq / 2) * HALF_W + swz(r0 + 64 * i, kq % 2);
     }
     const int nk = (K + BK - 1) / BK;
-    float4 pal[MB], pau[MB], pw[MB];
+    float4 pal[MBM], pau[MBM], pw[MBN];
     auto past = [&](int kt) { return !EXACT && kt * BK + kq * 4 >= K; };
     auto gload = [&](int kt) {
         const unsigned k = kt * (BK * 4u);
+        const unsigned kk = (!EXACT && past(kt)) ? 0u : k;     // !EXACT: the K offset travels with the thread
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-            if (EXACT) {
-                pal[i] = ld4(wal, va[i], k);
-                pau[i] = ld4(wau, va[i], k);
-                pw[i] = ld4(ww, vw[i], k);
-            } else {
-                const unsigned kk = past(kt) ? 0u : k;
-                pal[i] = ld4(wal, va[i] + kk, 0);
-                pau[i] = ld4(wau, va[i] + kk, 0);
-                pw[i] = ld4(ww, vw[i] + kk, 0);
-            }
+        for (int i = 0; i < MBM; ++i) {
+            pal[i] = EXACT ? ld4(wal, va[i], k) : ld4(wal, va[i] + kk, 0);
+            pau[i] = EXACT ? ld4(wau, va[i], k) : ld4(wau, va[i] + kk, 0);
         }
+#pragma unroll
+        for (int i = 0; i < MBN; ++i) pw[i] = EXACT ? ld4(ww, vw[i], k) : ld4(ww, vw[i] + kk, 0);
     };
     auto lstore = [&](int buf, int kt) {
         float *s = sm[buf];
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-            if (past(kt)) pal[i] = pau[i] = pw[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            *reinterpret_cast<float4 *>(s + S_AL + dst[i]) = pal[i];
-            *reinterpret_cast<float4 *>(s + S_AU + dst[i]) = pau[i];
-            *reinterpret_cast<float4 *>(s + S_WP + dst[i]) = pos4(pw[i]);
-            *reinterpret_cast<float4 *>(s + S_WN + dst[i]) = neg4(pw[i]);
+        for (int i = 0; i < MBM; ++i) {
+            if (past(kt)) pal[i] = pau[i] = zero;
+            *reinterpret_cast<float4 *>(s + S_AL + dsta[i]) = pal[i];
+            *reinterpret_cast<float4 *>(s + S_AU + dsta[i]) = pau[i];
+        }
+#pragma unroll
+        for (int i = 0; i < MBN; ++i) {
+            if (past(kt)) pw[i] = zero;
+            *reinterpret_cast<float4 *>(s + S_WP + dstw[i]) = pos4(pw[i]);
+            *reinterpret_cast<float4 *>(s + S_WN + dstw[i]) = neg4(pw[i]);
         }
     };
 
-    floatx16 cl[MB][MB], cu[MB][MB];
+    floatx16 cl[MBM][MBN], cu[MBM][MBN];
 #pragma unroll
-    for (int a = 0; a < MB; ++a)
+    for (int a = 0; a < MBM; ++a)
 #pragma unroll
-        for (int b = 0; b < MB; ++b)
+        for (int b = 0; b < MBN; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
 
     // fragments: lane (fi = lane % 32, fh = lane / 32) reads k = 8*ks + 4*fh .. +3 of row fi
     const int fi = lane % 32, fh = lane / 32;
-    int fa[MB], fw[MB];
+    int fa[MBM], fw[MBN];
 #pragma unroll
-    for (int s = 0; s < MB; ++s) {
-        fa[s] = swz((wm * MB + s) * 32 + fi, fh);
-        fw[s] = swz((wn * MB + s) * 32 + fi, fh);
-    }
+    for (int s = 0; s < MBM; ++s) fa[s] = swz((wm * MBM + s) * 32 + fi, fh);
+#pragma unroll
+    for (int s = 0; s < MBN; ++s) fw[s] = swz((wn * MBN + s) * 32 + fi, fh);
     auto compute = [&](int buf, auto &&halfway) {
         const float *s = sm[buf];
 #pragma unroll
         for (int ks = 0; ks < BK / 8; ++ks) {
             if (ks == 1) halfway();
-            float4 al[MB], au[MB], wp[MB], wq[MB];
+            float4 al[MBM], au[MBM], wp[MBN], wq[MBN];
 #pragma unroll
-            for (int t = 0; t < MB; ++t) {
-                al[t] = *reinterpret_cast<const float4 *>(s + S_AL + ks * HALF + fa[t]);
-                au[t] = *reinterpret_cast<const float4 *>(s + S_AU + ks * HALF + fa[t]);
-                wp[t] = *reinterpret_cast<const float4 *>(s + S_WP + ks * HALF + fw[t]);
-                wq[t] = *reinterpret_cast<const float4 *>(s + S_WN + ks * HALF + fw[t]);
+            for (int t = 0; t < MBM; ++t) {
+                al[t] = *reinterpret_cast<const float4 *>(s + S_AL + ks * HALF_A + fa[t]);
+                au[t] = *reinterpret_cast<const float4 *>(s + S_AU + ks * HALF_A + fa[t]);
+            }
+#pragma unroll
+            for (int t = 0; t < MBN; ++t) {
+                wp[t] = *reinterpret_cast<const float4 *>(s + S_WP + ks * HALF_W + fw[t]);
+                wq[t] = *reinterpret_cast<const float4 *>(s + S_WN + ks * HALF_W + fw[t]);
             }
 #define FAITH_STEP(c)                                                           \
-    _Pragma("unroll") for (int a = 0; a < MB; ++a) _Pragma("unroll") for (int b = 0; b < MB; ++b) { \
+    _Pragma("unroll") for (int a = 0; a < MBM; ++a) _Pragma("unroll") for (int b = 0; b < MBN; ++b) { \
         cl[a][b] = mfma(al[a].c, wp[b].c, cl[a][b]);                            \
         cu[a][b] = mfma(au[a].c, wp[b].c, cu[a][b]);                            \
     }                                                                           \
-    _Pragma("unroll") for (int a = 0; a < MB; ++a) _Pragma("unroll") for (int b = 0; b < MB; ++b) { \
+    _Pragma("unroll") for (int a = 0; a < MBM; ++a) _Pragma("unroll") for (int b = 0; b < MBN; ++b) { \
         cl[a][b] = mfma(au[a].c, wq[b].c, cl[a][b]);                            \
         cu[a][b] = mfma(al[a].c, wq[b].c, cu[a][b]);                            \
     }
@@ -229,14 +236,14 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
 
     // ---- epilogue: register r of a 32x32 block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-        const int col = n0 + (wn * MB + b) * 32 + fi;
+    for (int b = 0; b < MBN; ++b) {
+        const int col = n0 + (wn * MBN + b) * 32 + fi;
         if (col >= g.N) continue;
 #pragma unroll
-        for (int a = 0; a < MB; ++a) {
+        for (int a = 0; a < MBM; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + (wm * MB + a) * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+                const int row = m0 + (wm * MBM + a) * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (row < M) {
                     const size_t o = (size_t)row * g.N + col;
                     __builtin_nontemporal_store(cl[a][b][r], &g.Cl[o]);
@@ -295,6 +302,52 @@ __device__ __forceinline__ void simple_tile(const GemmArgs &g, const int m_blk, 
     }
 }
 
+// The same arithmetic for the constant-term rows of a SMALL problem, where a 16 x 16 tile is one long
+// chain of short dependent steps: an 8 x 8 tile per workgroup, the reduction in chunks of 64 with a
+// quarter of each chunk per group of 64 threads (four times the workgroups, a quarter of the chain),
+// the four partial sums combined in LDS.  smem: 3 * 8 * 65 floats + 2 * 4 * 64 doubles.
+__device__ __forceinline__ void sliced_tile(const GemmArgs &g, const int m_blk, const int n_blk, float *smem) {
+    constexpr int T = 8, KC = 64, S = 4;
+    float(*sl)[KC + 1] = reinterpret_cast<float(*)[KC + 1]>(smem);
+    float(*su)[KC + 1] = reinterpret_cast<float(*)[KC + 1]>(smem + T * (KC + 1));
+    float(*sw)[KC + 1] = reinterpret_cast<float(*)[KC + 1]>(smem + 2 * T * (KC + 1));
+    double(*red)[S][T * T] = reinterpret_cast<double(*)[S][T * T]>(smem + 3 * T * (KC + 1));        // 1560 floats in: 8-byte aligned
+    const int m0 = m_blk * T, n0 = n_blk * T;
+    const int ks = threadIdx.x / 64, o = threadIdx.x % 64;
+    const int tx = o % T, ty = o / T;                       // output (m0 + ty, n0 + tx)
+    double accl = 0.0, accu = 0.0;
+    for (int k0 = 0; k0 < g.K; k0 += KC) {
+        for (int e = threadIdx.x; e < T * KC; e += 256) {
+            const int r = e / KC, k = e % KC;
+            const bool kin = k0 + k < g.K;
+            const bool ain = kin && m0 + r < g.Mb, win = kin && n0 + r < g.N;
+            sl[r][k] = ain ? g.Bl[(size_t)(m0 + r) * g.K + k0 + k] : 0.f;
+            su[r][k] = ain ? g.Bu[(size_t)(m0 + r) * g.K + k0 + k] : 0.f;
+            sw[r][k] = win ? g.W[(size_t)(n0 + r) * g.K + k0 + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int kk = 0; kk < KC / S; ++kk) {
+            const int k = ks * (KC / S) + kk;
+            const float w = sw[tx][k];
+            const double wp = fmaxf(w, 0.f), wq = fminf(w, 0.f);
+            const double xl = sl[ty][k], xu = su[ty][k];
+            accl += xl * wp + xu * wq;
+            accu += xu * wp + xl * wq;
+        }
+        __syncthreads();
+    }
+    red[0][ks][o] = accl;
+    red[1][ks][o] = accu;
+    __syncthreads();
+    const int row = m0 + ty, col = n0 + tx;
+    if (ks == 0 && row < g.Mb && col < g.N) {
+        const float add = g.bias ? g.bias[col] : 0.f;
+        g.Dl[(size_t)row * g.N + col] = (float)(red[0][0][o] + red[0][1][o] + red[0][2][o] + red[0][3][o]) + add;
+        g.Du[(size_t)row * g.N + col] = (float)(red[1][0][o] + red[1][1][o] + red[1][2][o] + red[1][3][o]) + add;
+    }
+}
+
 __global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
     __shared__ float sm[3 * 16 * 17];
     const int tiles_n = (g.N + 15) / 16;
@@ -305,21 +358,21 @@ template <bool EXACT>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 signsplit_gemm(const GemmArgs g) {
     __shared__ float sm[2 * 4 * 2 * 128 * 8];            // two stages of four operands, 64 KB
-    signsplit_gemm_body<EXACT, 2>(g, sm, blockIdx.x);
+    signsplit_gemm_body<EXACT, 2, 2>(g, sm, blockIdx.x);
 }
-// Small problems: the first `b_tiles` workgroups take the 16 x 16 tiles of the constant-term rows
-// (exact accumulation; each is a long chain of short steps, so they start first and run beside the
-// MFMA tiles instead of in a launch of their own), the others a 64 x 64 MFMA tile each.
-template <bool EXACT>
+// Small problems: the first `b_tiles` workgroups take the 8 x 8 tiles of the constant-term rows
+// (exact accumulation; chains of short dependent steps, so they start first and run beside the
+// MFMA tiles instead of in a launch of their own), the others one MFMA tile of 64 MBM x 64 MBN each.
+template <bool EXACT, int MBM, int MBN>
 __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs g, const int b_tiles) {
-    __shared__ float sm[2 * 4 * 2 * 64 * 8];             // 32 KB
+    __shared__ __align__(16) float sm[2 * 4 * 64 * 8 * (MBM + MBN)];   // 32 KB (64 x 64) or 48 KB
     if ((int)blockIdx.x < b_tiles) {
-        const int tiles_n = (g.N + 15) / 16;
+        const int tiles_n = (g.N + 7) / 8;
         const int m_blk = blockIdx.x / tiles_n;
-        if (m_blk < (g.Mb + 15) / 16) simple_tile(g, (g.Mw + 15) / 16 + m_blk, blockIdx.x % tiles_n, sm);
+        if (m_blk < (g.Mb + 7) / 8) sliced_tile(g, m_blk, blockIdx.x % tiles_n, sm);
         return;
     }
-    signsplit_gemm_body<EXACT, 1>(g, sm, blockIdx.x - b_tiles);
+    signsplit_gemm_body<EXACT, MBM, MBN>(g, sm, blockIdx.x - b_tiles);
 }
 
 }  // namespace
@@ -344,27 +397,30 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
                       faith::aligned(W, 16) && 128LL * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
-        // 64 x 64 macro-tiles when 128 x 128 ones would leave compute units without work
-        const long long big_tiles = ((mw + 127) / 128) * ((dim_y_out + 127) / 128);
-        // (they run within 2 % of the large tiles even at configuration 2, so the switch point is not critical)
-        const int tile = big_tiles < 2 * faith::compute_units() ? 64 : 128;
-        const long long mblks = (mw + tile - 1) / tile;
-        const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tile - 1) / tile);
+        // macro-tile (measured on 8192 ... 131072 rows, K and N 256 ... 1024): tiny problems want the most
+        // workgroups (64 x 64); up to two 128 x 64 tiles per CU that shape is 6 - 17 % ahead of 64 x 64;
+        // beyond, 64 x 64 until there are four 128 x 128 tiles per CU (their pro- and epilogues overlap
+        // better at five workgroups per CU than at two), then 128 x 128.  The tuning knob forces a shape.
+        auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * ((dim_y_out + n - 1) / n); };
+        const long long cus = faith::compute_units();
+        int tm, tn;
+        if (tiles(64, 64) <= cus) { tm = 64; tn = 64; }
+        else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
+        else if (tiles(128, 128) < 4 * cus) { tm = 64; tn = 64; }
+        else { tm = 128; tn = 128; }
+        switch (faith::tune_get(FAITH_TUNE_GEMM_VARIANT)) {
+            case 1: tm = 64;  tn = 64;  break;
+            case 2: tm = 128; tn = 128; break;
+            case 3: tm = 128; tn = 64;  break;
+            case 4: tm = 64;  tn = 128; break;
+            default: break;
+        }
+        const long long mblks = (mw + tm - 1) / tm;
+        const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tn - 1) / tn);
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
         const bool exact = dim_out % BK == 0;
-        const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
-        if (tile == 64) {
-            // constant-term tiles in front, rounded up to a multiple of 8 so that the MFMA tiles keep
-            // their XCD (workgroup number mod 8)
-            const long long b_tiles = (gridb + XCDS - 1) / XCDS * XCDS;
-            FAITH_REQUIRE(grid + b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
-            if (exact)
-                hipLaunchKernelGGL(signsplit_gemm_small<true>, dim3((unsigned)(grid + b_tiles)), dim3(NTHREADS), 0, st, g,
-                                   (int)b_tiles);
-            else
-                hipLaunchKernelGGL(signsplit_gemm_small<false>, dim3((unsigned)(grid + b_tiles)), dim3(NTHREADS), 0, st, g,
-                                   (int)b_tiles);
-        } else {
+        if (tm == 128 && tn == 128) {
+            const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
             if (exact)
                 hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
             else
@@ -372,6 +428,20 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
             GemmArgs gb = g;
             gb.Mw = 0;
             hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+        } else {
+            // constant-term tiles in front, rounded up to a multiple of 8 so that the MFMA tiles keep
+            // their XCD (workgroup number mod 8)
+            const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
+            const long long b_tiles = (gridb + XCDS - 1) / XCDS * XCDS;
+            FAITH_REQUIRE(grid + b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
+            const dim3 gd((unsigned)(grid + b_tiles)), bd(NTHREADS);
+#define FAITH_LAUNCH_SMALL(MBM, MBN)                                                                      \
+    if (exact) hipLaunchKernelGGL((signsplit_gemm_small<true, MBM, MBN>), gd, bd, 0, st, g, (int)b_tiles); \
+    else hipLaunchKernelGGL((signsplit_gemm_small<false, MBM, MBN>), gd, bd, 0, st, g, (int)b_tiles)
+            if (tm == 64 && tn == 64) { FAITH_LAUNCH_SMALL(1, 1); }
+            else if (tm == 128) { FAITH_LAUNCH_SMALL(2, 1); }
+            else { FAITH_LAUNCH_SMALL(1, 2); }
+#undef FAITH_LAUNCH_SMALL
         }
     } else {
         const long long grid = ((mw + 15) / 16 + (rows + 15) / 16) * ((dim_y_out + 15) / 16);

@@ -10,7 +10,7 @@ import math
 
 import torch
 
-from . import _lib
+from . import _lib, autotune
 from ._lib import LAYOUT_NATURAL, LAYOUT_TRANSPOSED, Q_1, Q_2, Q_INF  # noqa: F401
 
 
@@ -61,11 +61,36 @@ class _NoGuard:
 _NO_GUARD = _NoGuard()
 
 
-def _on(device):
-    """Device guard for the launch; free when the tensor already lives on the current device."""
+class _Tuned:
+    """Device guard plus the tuning-table entry of this (operator, shape), set for the one launch."""
+
+    def __init__(self, guard, knobs):
+        self.guard, self.knobs = guard, knobs
+
+    def __enter__(self):
+        self.guard.__enter__()
+        for k, v in self.knobs.items():
+            _lib.call("faith_tune_set", k, v)
+        return self
+
+    def __exit__(self, *exc):
+        for k in self.knobs:
+            _lib.call("faith_tune_set", k, 0)
+        return self.guard.__exit__(*exc)
+
+
+def _on(device, op=None, shape=None):
+    """Device guard for the launch; free when the tensor already lives on the current device.
+    With a tuning table in use (autotune.use) the entry for (op, shape) is applied around the launch."""
     if device.index is None or device.index == torch.cuda.current_device():
-        return _NO_GUARD
-    return torch.cuda.device(device)
+        guard = _NO_GUARD
+    else:
+        guard = torch.cuda.device(device)
+    if op is not None and autotune._ACTIVE is not None:
+        knobs = autotune._ACTIVE.lookup(op, shape)
+        if knobs:
+            return _Tuned(guard, knobs)
+    return guard
 
 
 def _wb_shapes(lw, lb, layout):
@@ -87,7 +112,7 @@ def concretize(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL):
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
     l = torch.empty_like(lb)
     u = torch.empty_like(ub)
-    with _on(lw.device):
+    with _on(lw.device, "concretize", (B * L, D, H)):
         _lib.call("faith_concretize", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(l), _ptr(u),
                   B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
     return l, u
@@ -109,7 +134,7 @@ def _activation(entry, lw, lb, uw, ub, p, eps, words, layout, return_interval, o
         _check("out lb", olb, lb.shape); _check("out ub", oub, lb.shape)
     l = torch.empty_like(lb) if return_interval else None
     u = torch.empty_like(ub) if return_interval else None
-    with _on(lw.device):
+    with _on(lw.device, "act", (B * L, D, H)):
         if entry in _UNARY:
             _lib.call("faith_unary_verification", _UNARY[entry], _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb),
                       _ptr(oub), _ptr(olw), _ptr(ouw), _ptr(l), _ptr(u), B * L, D, H, float(eps), q_code(p),
@@ -277,7 +302,7 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
         olw, olb, ouw, oub = out
         _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
         _check("out lb", olb, (B, L, N)); _check("out ub", oub, (B, L, N))
-    with _on(lw.device):
+    with _on(lw.device, "linear", (B * L * D, H, weight.shape[0])):
         _lib.call("faith_matmul_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
                   _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), B, L, D, H, N, _stream(lw))
     return olw, olb, ouw, oub
@@ -307,7 +332,7 @@ def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
         zlw, zlb, zuw, zub = out
         _check("out lw", zlw, (B, Lx, D, Ly)); _check("out uw", zuw, (B, Lx, D, Ly))
         _check("out lb", zlb, (B, Lx, Ly)); _check("out ub", zub, (B, Lx, Ly))
-    with _on(dev):
+    with _on(dev, "dot_qk", (B, Lx, Ly, D, d)):
         _lib.call("faith_dot_product_verification_QK", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Ly, d, D, float(eps), q_code(p), int(words),
@@ -344,7 +369,7 @@ def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
         zlw, zlb, zuw, zub = out
         _check("out lw", zlw, (B, Lx, D, dv)); _check("out uw", zuw, (B, Lx, D, dv))
         _check("out lb", zlb, (B, Lx, dv)); _check("out ub", zub, (B, Lx, dv))
-    with _on(dev):
+    with _on(dev, "dot_v", (B, Lx, dv, D, Lk)):
         _lib.call("faith_dot_product_verification_V", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Lk, dv, D, float(eps), q_code(p), int(words),
@@ -378,7 +403,7 @@ def attention_scores(x, y, heads, p, eps, words=1):
     zuw = torch.empty_like(zlw)
     zlb = torch.empty(heads, Lx, Ly, device=dev, dtype=torch.float32)
     zub = torch.empty_like(zlb)
-    with _on(dev):
+    with _on(dev, "dot_qk", (heads, Lx, Ly, D, H // heads)):
         _lib.call("faith_attention_scores", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), heads, Lx, Ly, H // heads, D, float(eps), q_code(p),
@@ -411,7 +436,7 @@ def attention_context(x, y, p, eps, words=1):
     zuw = torch.empty_like(zlw)
     zlb = torch.empty(1, Lx, H, device=dev, dtype=torch.float32)
     zub = torch.empty_like(zlb)
-    with _on(dev):
+    with _on(dev, "dot_v", (heads, Lx, H // heads, D, Lk)):
         _lib.call("faith_attention_context", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), heads, Lx, Lk, H // heads, D, float(eps), q_code(p),

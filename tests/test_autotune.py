@@ -1,0 +1,158 @@
+"""Autotuner: heuristics, cost model, search loop and table on the CPU (the measurement is a
+stand-in); on the GPU, every GEMM / dot-product variant gives the default variant's result and a
+real tuning run never ends slower than the built-in choice."""
+import numpy as np
+import pytest
+import torch
+
+from faith_amd import autotune as A
+
+
+def test_heuristics_reject_what_cannot_fit_or_is_padding():
+    h = A.Heuristics()
+    lin = h.candidates("linear", (131072, 1024, 1024))
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in lin} == {1, 2, 3, 4}
+    # a 64-row, 64-column problem: tiles of 128 in either direction are padding
+    tiny = h.candidates("linear", (64, 64, 64))
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in tiny} == {1}
+    # the per-wavefront dot kernel needs d % 8 == 0 and d <= 80, and is pointless for long sequences
+    assert all(c.knob_dict()[A.TUNE_DOT_VARIANT] == 1 for c in h.candidates("dot_qk", (4, 128, 128, 256, 100)))
+    short = h.candidates("dot_qk", (4, 32, 32, 256, 64))
+    assert {c.knob_dict().get(A.TUNE_DOT_COORDS, 0) for c in short} == {0, 1, 2, 3, 4, 6, 8, 12, 16}
+    # a machine with a quarter of the LDS loses the large GEMM tiles
+    small_lds = dict(A.mi355x_metafile, MAX_LDS_KB=40)
+    kept = A.Heuristics(small_lds).candidates("linear", (131072, 1024, 1024))
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in kept} == {1}
+    with pytest.raises(ValueError):
+        h.propose("softmax", (1, 2, 3))
+
+
+def test_resident_workgroups_follow_lds_and_registers():
+    h = A.Heuristics()
+    assert h.resident_workgroups(64 * 1024, 196) == 2      # 128 x 128 GEMM tile: two per CU
+    assert h.resident_workgroups(32 * 1024, 88) == 5       # 64 x 64: five, by LDS and by registers
+    assert h.resident_workgroups(200 * 1024, 64) == 0
+
+
+def test_cost_model_ranks_a_planted_relation():
+    rng = np.random.default_rng(0)
+    x = rng.uniform(1, 10, size=(40, 5))
+    y = np.exp(0.3 * x[:, 0] - 0.2 * x[:, 3] + 1.0)
+    m = A.CostModel().fit(x[:30], y[:30])
+    pred = m.predict(x[30:])
+    assert np.allclose(pred, y[30:], rtol=0.05)
+    assert list(np.argsort(pred)) == list(np.argsort(y[30:]))
+    # constant columns (the metafile part of the features) must not break the fit
+    xc = np.hstack([x, np.full((40, 2), 7.0)])
+    assert np.allclose(A.CostModel().fit(xc[:30], y[:30]).predict(xc[30:]), y[30:], rtol=0.05)
+
+
+def test_search_finds_the_planted_optimum_and_restores_the_knobs():
+    h = A.Heuristics()
+    state = {}
+    calls = []
+
+    def setter(k, v):
+        state[k] = v
+        calls.append((k, v))
+
+    # stand-in measurement: latency falls with coordinates per wavefront down to 6, then rises; the
+    # persistent kernel and the built-in choice are slower
+    def measure(run):
+        if state.get(A.TUNE_DOT_VARIANT, 0) == 2:
+            return 30.0 + 2.0 * abs(state.get(A.TUNE_DOT_COORDS, 0) - 6)
+        return 80.0 if state.get(A.TUNE_DOT_VARIANT, 0) == 1 else 50.0
+
+    res = A.autotune("dot_qk", (4, 32, 32, 256, 64), run=lambda: None, heuristics=h, rounds=4, samples=2,
+                     measure=measure, setter=setter, seed=3)
+    assert res.best.knob_dict() == {A.TUNE_DOT_VARIANT: 2, A.TUNE_DOT_COORDS: 6} and res.best_us == 30.0
+    assert len(res.measured) <= 1 + 4 * 2 and res.measured[0][1] == 50.0      # built-in choice first
+    assert all(v == 0 for v in state.values())                               # everything restored
+    # exhaustive when the budget covers the space
+    full = A.autotune("linear", (8192, 256, 256), run=lambda: None, rounds=3, samples=2,
+                      measure=lambda run: 10.0 + state.get(A.TUNE_GEMM_VARIANT, 0), setter=setter)
+    assert full.best_us == 10.0 and len(full.measured) == 5
+
+
+def test_a_variant_that_raises_is_skipped():
+    state = {}
+
+    def measure(run):
+        if state.get(A.TUNE_GEMM_VARIANT) == 3:
+            raise RuntimeError("launch failed")
+        return 5.0 + state.get(A.TUNE_GEMM_VARIANT, 0)
+
+    res = A.autotune("linear", (8192, 256, 256), run=lambda: None, rounds=3, samples=4, measure=measure,
+                     setter=lambda k, v: state.__setitem__(k, v))
+    assert res.skipped == 1 and res.best_us == 5.0 and state[A.TUNE_GEMM_VARIANT] == 0
+
+
+def test_table_round_trip(tmp_path):
+    t = A.TuningTable()
+    best = A.Heuristics().candidates("linear", (8192, 256, 256))[2]
+    t.record(A.TuningResult("linear", (8192, 256, 256), best, 41.5, [(best, 41.5)]))
+    path = tmp_path / "tuned.json"
+    t.save(path)
+    back = A.TuningTable.load(path)
+    assert back.lookup("linear", (8192, 256, 256)) == best.knob_dict()
+    assert back.lookup("linear", (8192, 256, 512)) is None
+    # no table in use: the wrappers' hook is a no-op
+    A.use(None)
+    with A.tuned("linear", (8192, 256, 256)):
+        pass
+
+
+# ------------------------------------------------------------------ GPU
+def _linear_case(seed, L, D, K, N):
+    from tests.helpers import rand_bounds
+    g = torch.Generator().manual_seed(seed)
+    x = rand_bounds(g, 1, L, D, K)
+    W = torch.randn(N, K, generator=g) / K ** 0.5
+    bias = torch.randn(N, generator=g)
+    return tuple(t.cuda() for t in x.tensors()), W.cuda(), bias.cuda()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(4, 32, 64, 64), (3, 50, 36, 72), (8, 128, 256, 320), (2, 16, 20, 200)])
+def test_every_gemm_tile_gives_the_same_result(shape):
+    """The four macro-tiles differ in how the same K-ordered fp32 sums are tiled, not in their value."""
+    from faith_amd import ops
+    x, W, bias = _linear_case(71, *shape)
+    print(f"[case] gemm variants L, D, K, N = {shape}", flush=True)
+    base = ops.linear(*x, W, bias)
+    for variant in (1, 2, 3, 4):
+        with A.applied({A.TUNE_GEMM_VARIANT: variant}):
+            got = ops.linear(*x, W, bias)
+        for a, b in zip(got, base):
+            assert torch.equal(a, b), f"variant {variant}"
+
+
+@pytest.mark.gpu
+def test_dot_variants_agree_and_tuning_is_never_slower_than_the_default():
+    from faith_amd import ops
+    from tests.helpers import rand_bounds, close
+    g = torch.Generator().manual_seed(72)
+    B, L, D, d = 4, 32, 64, 32
+    x = tuple(t.cuda() for t in rand_bounds(g, B, L, D, d, ordered=False, sw=0.3).tensors())
+    y = tuple(t.cuda() for t in rand_bounds(g, B, L, D, d, ordered=False, sw=0.3).tensors())
+    base = ops.dot_product_qk(x, y, 2.0, 0.05)
+    for knobs in ({A.TUNE_DOT_VARIANT: 1}, {A.TUNE_DOT_VARIANT: 2, A.TUNE_DOT_COORDS: 1},
+                  {A.TUNE_DOT_VARIANT: 2, A.TUNE_DOT_COORDS: 5}, {A.TUNE_DOT_VARIANT: 2, A.TUNE_DOT_COORDS: 16}):
+        with A.applied(knobs):
+            got = ops.dot_product_qk(x, y, 2.0, 0.05)
+        for a, b in zip(got, base):
+            assert close(a, b, rtol=1e-5, atol=2e-6), knobs
+
+    run = lambda: ops.dot_product_qk(x, y, 2.0, 0.05)
+    res = A.autotune("dot_qk", (B, L, L, D, d), run, heuristics=A.Heuristics(A.metafile_of_device()), rounds=3, samples=3)
+    default_us = res.measured[0][1]
+    assert res.best_us <= default_us and res.skipped == 0
+    table = A.TuningTable()
+    table.record(res)
+    A.use(table)
+    try:
+        tuned = ops.dot_product_qk(x, y, 2.0, 0.05)      # goes through the table entry
+    finally:
+        A.use(None)
+    for a, b in zip(tuned, base):
+        assert close(a, b, rtol=1e-5, atol=2e-6)
