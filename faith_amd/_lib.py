@@ -35,8 +35,8 @@ SIGNATURES = {
     "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],
     "faith_dot_product_verification_QK": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_dot_product_verification_V": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
-    "faith_attention_scores": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
-    "faith_attention_context": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
+    "faith_attention_scores": [_P] * 16 + [_I] * 6 + [_F, _I, _I, _P],
+    "faith_attention_context": [_P] * 16 + [_I] * 6 + [_F, _I, _I, _P],
     "faith_convolution_verification": [_P] * 10 + [_I] * 9 + [_P],
 }
 

@@ -149,13 +149,44 @@ class Bounds:
     # check reads the concrete lower bound back from the kernel (one synchronisation).
     def sqrt(self):
         out = ops.sqrt(*self._c(), self.p, self.eps, self.perturbed_words, return_interval=True)
-        assert float(out[4].min()) > 0, "sqrt of a bound that reaches zero"
+        self._require(out[4], 0.0, True, "sqrt of a bound that reaches zero")
         return self._like(*out[:4])
 
     def reciprocal(self):
         out = ops.reciprocal(*self._c(), self.p, self.eps, self.perturbed_words, return_interval=True)
-        assert float(out[4].min()) >= 1e-12, "reciprocal of a bound that reaches zero"
+        self._require(out[4], 1e-12, False, "reciprocal of a bound that reaches zero")
         return self._like(*out[:4])
+
+    # The reference asserts these preconditions (Bounds.py:894, :1147), which costs a device
+    # synchronisation per call and fails a whole batch for one element.  Inside collect_failures the
+    # violation is recorded per batch element on the device instead and nothing waits.
+    _collector = None
+
+    @classmethod
+    def _require(cls, l, bound, strict, message):
+        c = cls._collector
+        if c is None:
+            low = float(l.min())
+            assert (low > bound) if strict else (low >= bound), message
+            return
+        per = l.reshape(c.mask.shape[0], -1).min(dim=1).values     # leading axis is batch-major
+        c.mask |= (per <= bound) if strict else (per < bound)
+
+    class collect_failures:
+        """with Bounds.collect_failures(batch, device) as f: ... ; f.mask[b] is True where a
+        precondition failed for batch element b (its results are then meaningless)."""
+
+        def __init__(self, batch, device):
+            self.mask = torch.zeros(batch, dtype=torch.bool, device=device)
+
+        def __enter__(self):
+            assert Bounds._collector is None, "collect_failures does not nest"
+            Bounds._collector = self
+            return self
+
+        def __exit__(self, *exc):
+            Bounds._collector = None
+            return False
 
     def act(self, act_name):
         if act_name == "relu":

@@ -60,16 +60,27 @@ struct DotArgs {
     float *zlw, *zuw;                     // [B, Lx, D, Ly]
     float *zlb, *zub;                     // [B, Lx, Ly]
     int B, Lx, Ly, D, d;
-    // Addressing of the three bound objects, in floats.  Coefficient (t, i, m, k) of x lies at
-    // t * xw_t + (i * D + m) * xp + k and constant term (t, i, k), like the concrete bounds, at
-    // t * xb_t + i * xp + k; likewise y and z.  Heads stacked on the batch axis: pitch = row width,
-    // head strides = one whole head.  Heads side by side in the rows of ONE object
-    // [1, L, D, heads * width] (what the dense layers produce and consume): pitch = heads * width,
-    // head strides = width.
-    int xp, yp, zp;
-    size_t xw_t, xb_t, yw_t, yb_t, zw_t, zb_t;
+    // Addressing of the three bound objects.  B counts (batch element, head) pairs t = b * heads + h.
+    // An object either stacks them on its first axis ([B, L, D, width]: `heads` = 1 below, so that
+    // b = t and h = 0) or keeps the heads of a batch element side by side in its rows
+    // ([batch, L, D, heads * width], what the dense layers produce and consume).
+    struct Obj {
+        int pitch;      // floats from one row to the next
+        int heads;      // heads side by side in a row (1: stacked)
+        int width;      // floats of one head in a row
+    } ox, oy, oz;
+    int heads;                            // heads per batch element
     int side_by_side;                     // HEADS_X | HEADS_Y | HEADS_Z: which objects keep their heads side by side
 };
+// first coefficient / first constant term of pair t of an object with `rows` positions per batch element
+__device__ __forceinline__ size_t w_base(const DotArgs::Obj &o, int t, int rows, int D) {
+    const int b = t / o.heads, h = t - b * o.heads;
+    return (size_t)b * rows * D * o.pitch + (size_t)h * o.width;
+}
+__device__ __forceinline__ size_t b_base(const DotArgs::Obj &o, int t, int rows) {
+    const int b = t / o.heads, h = t - b * o.heads;
+    return (size_t)b * rows * o.pitch + (size_t)h * o.width;
+}
 constexpr int HEADS_X = 1, HEADS_Y = 2, HEADS_Z = 4;
 
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
@@ -191,7 +202,7 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     unsigned vx = 0, vbt = 0, vy = 0;
     // K-step strides in bytes: x side and scores-path y side advance along the contiguous axis (the
     // entry point checks that one head of y spans less than 4 GB)
-    const unsigned ystride = VP ? (unsigned)BK * g.yp * (wside ? g.D : 1) * 4u : BK * 4u;
+    const unsigned ystride = VP ? (unsigned)BK * g.oy.pitch * (wside ? g.D : 1) * 4u : BK * 4u;
     // totals in elements
     const size_t tot_x = (size_t)g.B * g.Lx * g.D * d, tot_bt = (size_t)g.B * g.Lx * d;
     const size_t tot_y = (size_t)g.B * g.Ly * d * (wside ? g.D : 1), tot_z = (size_t)g.B * g.Lx * g.D * g.Ly;
@@ -203,21 +214,17 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     auto point_at = [&](const Walk &w) {
         const int j0 = w.j * TJ, i0 = w.i * TI, t = w.t;
         const int m = xcd_map ? w.m * 8 + m_low : w.m;
-        // pitches and head strides are worked out again for every tile (a handful of scalar
-        // instructions) instead of being held in 15 scalar registers across the K-loop
-        int sbs = g.side_by_side;
-        asm volatile("" : "+s"(sbs));
+        // the three objects' addressing is worked out again for every tile (a handful of scalar
+        // instructions) instead of being held in scalar registers across the K-loop
+        int sbs = g.side_by_side, heads = g.heads;
+        asm volatile("" : "+s"(sbs), "+s"(heads));
         const int y_h = VP ? g.Ly : d, y_len = VP ? d : g.Ly;
-        struct { int xp, yp, zp; size_t xw_t, xb_t, yw_t, yb_t, zw_t; } a;
-        a.xp = (sbs & HEADS_X) ? g.B * d : d;
-        a.xw_t = (sbs & HEADS_X) ? (size_t)d : (size_t)g.Lx * g.D * d;
-        a.xb_t = (sbs & HEADS_X) ? (size_t)d : (size_t)g.Lx * d;
-        a.yp = (sbs & HEADS_Y) ? g.B * y_h : y_h;
-        a.yw_t = (sbs & HEADS_Y) ? (size_t)y_h : (size_t)y_len * g.D * y_h;
-        a.yb_t = (sbs & HEADS_Y) ? (size_t)y_h : (size_t)y_len * y_h;
-        a.zp = (sbs & HEADS_Z) ? g.B * g.Ly : g.Ly;
-        a.zw_t = (sbs & HEADS_Z) ? (size_t)g.Ly : (size_t)g.Lx * g.D * g.Ly;
-        const size_t x0 = t * a.xw_t + ((size_t)i0 * g.D + m) * a.xp, bt0 = t * a.xb_t + (size_t)i0 * a.xp;
+        const DotArgs::Obj ox{(sbs & HEADS_X) ? heads * d : d, (sbs & HEADS_X) ? heads : 1, d};
+        const DotArgs::Obj oy{(sbs & HEADS_Y) ? heads * y_h : y_h, (sbs & HEADS_Y) ? heads : 1, y_h};
+        const DotArgs::Obj oz{(sbs & HEADS_Z) ? heads * g.Ly : g.Ly, (sbs & HEADS_Z) ? heads : 1, g.Ly};
+        struct { int xp, yp, zp; } a{ox.pitch, oy.pitch, oz.pitch};
+        const size_t x0 = w_base(ox, t, g.Lx, g.D) + ((size_t)i0 * g.D + m) * a.xp;
+        const size_t bt0 = b_base(ox, t, g.Lx) + (size_t)i0 * a.xp;
         bxl = g.xlw + x0;  bxu = g.xuw + x0;  nx = clamp32((tot_x - x0) * 4);
         bbt = g.x_l + bt0;  nbt = clamp32((tot_bt - bt0) * 4);
         const int irow = min(srow, g.Lx - 1 - i0);         // clamped rows are never stored
@@ -226,18 +233,18 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         size_t y0;
         if (VP) {
             // y[t, k, m, j] / a[t, k, j]; the j offset stays with the thread so that it can be clamped
-            y0 = wside ? t * a.yw_t + (size_t)m * a.yp : t * a.yb_t;
+            y0 = wside ? w_base(oy, t, y_len, g.D) + (size_t)m * a.yp : b_base(oy, t, y_len);
             const int jc = min(j0 + vj, g.Ly - 4);         // Ly % 4 == 0; clamped columns are never stored
             vy = ((unsigned)vk * a.yp * (wside ? g.D : 1) + jc) * 4u;
         } else {
-            y0 = wside ? t * a.yw_t + ((size_t)j0 * g.D + m) * a.yp : t * a.yb_t + (size_t)j0 * a.yp;
+            y0 = wside ? w_base(oy, t, y_len, g.D) + ((size_t)j0 * g.D + m) * a.yp : b_base(oy, t, y_len) + (size_t)j0 * a.yp;
             const int jrow = min(yrow, g.Ly - 1 - j0);
             vy = ((unsigned)jrow * a.yp * (wside ? g.D : 1) + yc * 4) * 4u;
         }
         by0 = (wside ? g.ylw : g.y_l) + y0;
         by1 = (wside ? g.yuw : g.y_u) + y0;
         ny = clamp32((tot_y - y0) * 4);
-        zn = t * a.zw_t + ((size_t)i0 * g.D + m) * a.zp + j0;
+        zn = w_base(oz, t, g.Lx, g.D) + ((size_t)i0 * g.D + m) * a.zp + j0;
         zn_i0 = i0;
         zn_j0 = j0;
     };
@@ -346,7 +353,7 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     // Piece c holds registers 4*(c%4) .. +3 of block c/4.  A row is a uniform offset from the tile's
     // first element, the lane's own offset never changes (the entry point checks that a tile spans
     // less than 4 GB).
-    const unsigned rsb = (unsigned)g.D * g.zp * 4u;        // one step in i, bytes
+    const unsigned rsb = (unsigned)g.D * g.oz.pitch * 4u;        // one step in i, bytes
     const unsigned lane_off = (unsigned)(wi * 64 + 4 * fh) * rsb + (wj * 32 + fi) * 4u;
     size_t pz = 0;                                         // finished tile: its first element
     unsigned pbytes = 0;                                   // bytes from there to the end of z; 0 before the first
@@ -481,7 +488,7 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
     // the same rows of different heads and their 32-byte pieces add up to whole rows
     int pid = blockIdx.x;
     int t = 0;
-    if (heads_first) { t = pid % g.B;  pid /= g.B; }
+    if (heads_first) { t = pid % g.B;  pid /= g.B; }     // (batch, head) pairs fastest
     const int mg = pid % mgroups;  pid /= mgroups;
     const int j0 = (pid % njb) * SB;  pid /= njb;
     const int i0 = (pid % nib) * SB;  pid /= nib;
@@ -491,15 +498,20 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
     const int lane = tid % 64, wv = tid / 64;
     const int fi = lane % 32, fh = lane / 32;
 
+    // first elements of this (batch element, head) in the three objects
+    const int y_len = VP ? g.d : g.Ly;
+    const size_t xb0 = b_base(g.ox, t, g.Lx), yb0 = b_base(g.oy, t, y_len);
+    const size_t xw0 = w_base(g.ox, t, g.Lx, g.D), yw0 = w_base(g.oy, t, y_len, g.D), zw0 = w_base(g.oz, t, g.Lx, g.D);
+
     // ---- operands shared by every m: b = l_x rows i0.., a_l / a_u rows (columns of z) j0..
     for (int e = tid; e < SB * d / 4; e += 256) {
         const int row = e / (d / 4), c4 = e % (d / 4);
         const int dst = (c4 / 2) * (SB * 8) + swz(row, c4 % 2);
-        const float4 bt = *reinterpret_cast<const float4 *>(g.x_l + t * g.xb_t + (size_t)min(i0 + row, g.Lx - 1) * g.xp + c4 * 4);
+        const float4 bt = *reinterpret_cast<const float4 *>(g.x_l + xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + c4 * 4);
         *reinterpret_cast<float4 *>(s_bp + dst) = pos4(bt);
         *reinterpret_cast<float4 *>(s_bn + dst) = neg4(bt);
         if (!VP) {
-            const size_t o = t * g.yb_t + (size_t)min(j0 + row, g.Ly - 1) * g.yp + c4 * 4;
+            const size_t o = yb0 + (size_t)min(j0 + row, g.Ly - 1) * g.oy.pitch + c4 * 4;
             const float4 al = *reinterpret_cast<const float4 *>(g.y_l + o), au = *reinterpret_cast<const float4 *>(g.y_u + o);
             *reinterpret_cast<float4 *>(s_alp + dst) = pos4(al);
             *reinterpret_cast<float4 *>(s_aln + dst) = neg4(al);
@@ -511,7 +523,7 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
         // a[t, k, j]: j is the contiguous axis
         for (int e = tid; e < SB * d; e += 256) {
             const int j = e % SB, k = e / SB;
-            const size_t o = t * g.yb_t + (size_t)k * g.yp + min(j0 + j, g.Ly - 1);
+            const size_t o = yb0 + (size_t)k * g.oy.pitch + min(j0 + j, g.Ly - 1);
             const float al = g.y_l[o], au = g.y_u[o];
             const int dst = (k / 8) * (SB * 8) + swz(j, (k % 8) / 4) + k % 4;
             s_alp[dst] = pos1(al);
@@ -526,15 +538,15 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
     const int irow = min(i0 + fi, g.Lx - 1), jcol = min(j0 + fi, g.Ly - 1);
     const int wave = __builtin_amdgcn_readfirstlane(wv);
     // per-lane byte offsets from the first element of (head, m); they do not depend on m
-    const unsigned vx = ((unsigned)irow * g.D * g.xp + fh * 4) * 4u;
-    const unsigned vy = VP ? ((unsigned)(fh * 4) * g.D * g.yp + jcol) * 4u : ((unsigned)jcol * g.D * g.yp + fh * 4) * 4u;
-    const unsigned ykstep = (unsigned)g.D * g.yp * 4u;             // context path: one step in k, bytes
+    const unsigned vx = ((unsigned)irow * g.D * g.ox.pitch + fh * 4) * 4u;
+    const unsigned vy = VP ? ((unsigned)(fh * 4) * g.D * g.oy.pitch + jcol) * 4u : ((unsigned)jcol * g.D * g.oy.pitch + fh * 4) * 4u;
+    const unsigned ykstep = (unsigned)g.D * g.oy.pitch * 4u;             // context path: one step in k, bytes
     const size_t tot_x = (size_t)g.B * g.Lx * g.D * d, tot_y = (size_t)g.B * g.Ly * g.D * d;
     for (int s = 0; s < mpw; ++s) {
         const int m = (mg * 4 + wave) * mpw + s;
         if (m >= g.D) break;
         // windows that start at (head t, coordinate m) and end with the tensor
-        const size_t x0 = t * g.xw_t + (size_t)m * g.xp, y0 = t * g.yw_t + (size_t)m * g.yp;
+        const size_t x0 = xw0 + (size_t)m * g.ox.pitch, y0 = yw0 + (size_t)m * g.oy.pitch;
         const __amdgpu_buffer_rsrc_t wxl = window(g.xlw + x0, clamp32((tot_x - x0) * 4));
         const __amdgpu_buffer_rsrc_t wxu = window(g.xuw + x0, clamp32((tot_x - x0) * 4));
         const __amdgpu_buffer_rsrc_t wyl = window(g.ylw + y0, clamp32((tot_y - y0) * 4));
@@ -596,7 +608,7 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
             for (int r = 0; r < 16; ++r) {
                 const int i = i0 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (i < g.Lx) {
-                    const size_t o = t * g.zw_t + ((size_t)i * g.D + m) * g.zp + j0 + fi;
+                    const size_t o = zw0 + ((size_t)i * g.D + m) * g.oz.pitch + j0 + fi;
                     __builtin_nontemporal_store(cl[r], &g.zlw[o]);
                     __builtin_nontemporal_store(cu[r], &g.zuw[o]);
                 }
@@ -615,14 +627,14 @@ __global__ void __launch_bounds__(256) dot_w_simple(const DotArgs g) {
         const int m = (idx / g.Ly) % g.D;
         const int i = (idx / ((size_t)g.Ly * g.D)) % g.Lx;
         const int t = idx / ((size_t)g.Ly * g.D * g.Lx);
-        const float *xl = g.xlw + t * g.xw_t + ((size_t)i * g.D + m) * g.xp;
-        const float *xu = g.xuw + t * g.xw_t + ((size_t)i * g.D + m) * g.xp;
+        const float *xl = g.xlw + w_base(g.ox, t, g.Lx, g.D) + ((size_t)i * g.D + m) * g.ox.pitch;
+        const float *xu = g.xuw + w_base(g.ox, t, g.Lx, g.D) + ((size_t)i * g.D + m) * g.ox.pitch;
         // y element (j, m, k): scores path [t, j, m, k]; context path [t, k, m, j]
-        const size_t ybase = t * g.yw_t + (VP ? (size_t)m * g.yp + j : ((size_t)j * g.D + m) * g.yp);
-        const size_t ystep = VP ? (size_t)g.D * g.yp : 1;
-        const size_t abase = t * g.yb_t + (VP ? (size_t)j : (size_t)j * g.yp);
-        const size_t astep = VP ? g.yp : 1;
-        const float *bt = g.x_l + t * g.xb_t + (size_t)i * g.xp;
+        const size_t ybase = w_base(g.oy, t, VP ? g.d : g.Ly, g.D) + (VP ? (size_t)m * g.oy.pitch + j : ((size_t)j * g.D + m) * g.oy.pitch);
+        const size_t ystep = VP ? (size_t)g.D * g.oy.pitch : 1;
+        const size_t abase = b_base(g.oy, t, VP ? g.d : g.Ly) + (VP ? (size_t)j : (size_t)j * g.oy.pitch);
+        const size_t astep = VP ? g.oy.pitch : 1;
+        const float *bt = g.x_l + b_base(g.ox, t, g.Lx) + (size_t)i * g.ox.pitch;
         double sl = 0.0, su = 0.0;
         for (int k = 0; k < g.d; ++k) {
             const float yl = g.ylw[ybase + k * ystep], yu = g.yuw[ybase + k * ystep];
@@ -633,7 +645,7 @@ __global__ void __launch_bounds__(256) dot_w_simple(const DotArgs g) {
             sl += xl[k] * alp + xu[k] * aln + bp * yl + bn * yu;
             su += xu[k] * aup + xl[k] * aun + bp * yu + bn * yl;
         }
-        const size_t z = t * g.zw_t + ((size_t)i * g.D + m) * g.zp + j;
+        const size_t z = w_base(g.oz, t, g.Lx, g.D) + ((size_t)i * g.D + m) * g.oz.pitch + j;
         g.zlw[z] = (float)sl;
         g.zuw[z] = (float)su;
     }
@@ -663,13 +675,13 @@ __global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
             // y is contiguous along j
             const int r = e / BT_K, k = e % BT_K;
             const bool xin = k0 + k < g.d && i0 + r < g.Lx;
-            const size_t xo = t * g.xb_t + (size_t)(i0 + r) * g.xp + k0 + k;
+            const size_t xo = b_base(g.ox, t, g.Lx) + (size_t)(i0 + r) * g.ox.pitch + k0 + k;
             sx[0][r][k] = xin ? g.x_l[xo] : 0.f;
             sx[1][r][k] = xin ? g.xlb[xo] : 0.f;
             sx[2][r][k] = xin ? g.xub[xo] : 0.f;
             const int ry = VP ? e % BT_T : r, ky = VP ? e / BT_T : k;
             const bool yin = k0 + ky < g.d && j0 + ry < g.Ly;
-            const size_t yo = t * g.yb_t + (VP ? (size_t)(k0 + ky) * g.yp + j0 + ry : (size_t)(j0 + ry) * g.yp + k0 + ky);
+            const size_t yo = b_base(g.oy, t, VP ? g.d : g.Ly) + (VP ? (size_t)(k0 + ky) * g.oy.pitch + j0 + ry : (size_t)(j0 + ry) * g.oy.pitch + k0 + ky);
             sy[0][ry][ky] = yin ? g.y_l[yo] : 0.f;
             sy[1][ry][ky] = yin ? g.y_u[yo] : 0.f;
             sy[2][ry][ky] = yin ? g.ylb[yo] : 0.f;
@@ -693,7 +705,7 @@ __global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
     if (ks == 0) {
         const int i = i0 + ty, j = j0 + tx;
         if (i < g.Lx && j < g.Ly) {
-            const size_t z = t * g.zb_t + (size_t)i * g.zp + j;
+            const size_t z = b_base(g.oz, t, g.Lx) + (size_t)i * g.oz.pitch + j;
             g.zlb[z] = (float)(red[0][0][o] + red[0][1][o] + red[0][2][o] + red[0][3][o]);
             g.zub[z] = (float)(red[1][0][o] + red[1][1][o] + red[1][2][o] + red[1][3][o]);
         }
@@ -710,8 +722,8 @@ __global__ void __launch_bounds__(256) dot_interval(const DotArgs g) {
     const int j = idx % g.Ly;
     const int i = (idx / g.Ly) % g.Lx;
     const int t = idx / ((size_t)g.Ly * g.Lx);
-    const size_t xo = t * g.xb_t + (size_t)i * g.xp;
-    const size_t yo = t * g.yb_t + (VP ? (size_t)j : (size_t)j * g.yp), ys = VP ? g.yp : 1;
+    const size_t xo = b_base(g.ox, t, g.Lx) + (size_t)i * g.ox.pitch;
+    const size_t yo = b_base(g.oy, t, VP ? g.d : g.Ly) + (VP ? (size_t)j : (size_t)j * g.oy.pitch), ys = VP ? g.oy.pitch : 1;
     float lo = 0.f, hi = 0.f;
     for (int k = 0; k < g.d; ++k) {
         const float l1 = g.xlb[xo + k], u1 = g.xub[xo + k], l2 = g.ylb[yo + k * ys], u2 = g.yub[yo + k * ys];
@@ -719,7 +731,7 @@ __global__ void __launch_bounds__(256) dot_interval(const DotArgs g) {
         lo += fminf(fminf(c1, c2), fminf(c3, c4));
         hi += fmaxf(fmaxf(c1, c2), fmaxf(c3, c4));
     }
-    const size_t zb = t * g.zb_t + (size_t)i * g.zp + j, zw = t * g.zw_t + (size_t)i * g.zp + j;   // dim_in == 1
+    const size_t zb = b_base(g.oz, t, g.Lx) + (size_t)i * g.oz.pitch + j, zw = w_base(g.oz, t, g.Lx, g.D) + (size_t)i * g.oz.pitch + j;   // dim_in == 1
     g.zlb[zb] = lo;
     g.zub[zb] = hi;
     g.zlw[zw] = 0.f;
@@ -737,7 +749,7 @@ template <bool VP>
 int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb, const float *x_ub,
               const float *y_lb, const float *y_ub, const float *x_lw, const float *x_uw, const float *y_lw,
               const float *y_uw, float *z_lb, float *z_ub, float *z_lw, float *z_uw, int B, int Lx, int Ly, int d, int D,
-              float epsilon, int q, int words, int side_by_side, void *stream) {
+              float epsilon, int q, int words, int side_by_side, int heads, void *stream) {
     FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
     FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
     FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
@@ -756,16 +768,13 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     // y is [rows of y, D, width of y] per head
     const int y_len = VP ? d : Ly, y_h = VP ? Ly : d;
     const bool x_sbs = side_by_side & HEADS_X, y_sbs = side_by_side & HEADS_Y, z_sbs = side_by_side & HEADS_Z;
-    FAITH_REQUIRE((long long)B * (d > Ly ? d : Ly) <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: heads * row width exceeds 2^31", who);
-    g.xp = x_sbs ? B * d : d;
-    g.xw_t = x_sbs ? (size_t)d : (size_t)Lx * D * d;
-    g.xb_t = x_sbs ? (size_t)d : (size_t)Lx * d;
-    g.yp = y_sbs ? B * y_h : y_h;
-    g.yw_t = y_sbs ? (size_t)y_h : (size_t)y_len * D * y_h;
-    g.yb_t = y_sbs ? (size_t)y_h : (size_t)y_len * y_h;
-    g.zp = z_sbs ? B * Ly : Ly;
-    g.zw_t = z_sbs ? (size_t)Ly : (size_t)Lx * D * Ly;
-    g.zb_t = z_sbs ? (size_t)Ly : (size_t)Lx * Ly;
+    FAITH_REQUIRE(heads >= 1 && B % heads == 0, FAITH_ERR_SHAPE, "%s: %d heads do not divide %d (batch, head) pairs", who,
+                  heads, B);
+    FAITH_REQUIRE((long long)heads * (d > Ly ? d : Ly) <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: heads * row width exceeds 2^31", who);
+    g.ox = {x_sbs ? heads * d : d, x_sbs ? heads : 1, d};
+    g.oy = {y_sbs ? heads * y_h : y_h, y_sbs ? heads : 1, y_h};
+    g.oz = {z_sbs ? heads * Ly : Ly, z_sbs ? heads : 1, Ly};
+    g.heads = heads;
     g.side_by_side = side_by_side;
     if (D == 1) {
         const long long n = (long long)B * Lx * Ly;
@@ -777,8 +786,8 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     // interface exposes it, the planes do not use it.  One launch when both objects have the same
     // [D, H] shape (always on the scores path).
     // An object with its heads side by side is concretized as the one [L, D, heads * width] object it is.
-    const int cx_rows = x_sbs ? Lx : B * Lx, cx_h = x_sbs ? B * d : d;
-    const int cy_rows = y_sbs ? y_len : B * y_len, cy_h = y_sbs ? B * y_h : y_h;
+    const int cx_rows = x_sbs ? B / heads * Lx : B * Lx, cx_h = x_sbs ? heads * d : d;
+    const int cy_rows = y_sbs ? B / heads * y_len : B * y_len, cy_h = y_sbs ? heads * y_h : y_h;
     int rc;
     if (cx_h == cy_h) {
         rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows,
@@ -795,12 +804,12 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     hipLaunchKernelGGL(dot_b<VP>, dim3((unsigned)((long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T))),
                        dim3(256), 0, st, g);
 
-    const int max_pitch = g.xp > g.yp ? (g.xp > g.zp ? g.xp : g.zp) : (g.yp > g.zp ? g.yp : g.zp);
+    const int max_pitch = g.ox.pitch > g.oy.pitch ? (g.ox.pitch > g.oz.pitch ? g.ox.pitch : g.oz.pitch) : (g.oy.pitch > g.oz.pitch ? g.oy.pitch : g.oz.pitch);
     const bool fast = (d % 4 == 0) && (!VP || Ly % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
                       faith::aligned(y_lw, 16) && faith::aligned(y_uw, 16) && faith::aligned(x_l, 16) &&
                       faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
                       (long long)TI * D * max_pitch * 4 < 0xffffffffLL &&            // 32-bit offsets inside a tile
-                      (!VP || (long long)d * D * g.yp * 4 < 0xffffffffLL);           // and along K inside a head
+                      (!VP || (long long)d * D * g.oy.pitch * 4 < 0xffffffffLL);           // and along K inside a head
     // short sequences take the per-wavefront kernel; the tuning knob can force either kernel
     const bool small_ok = fast && d % 8 == 0 && d <= 80;
     const int pick = faith::tune_get(FAITH_TUNE_DOT_VARIANT);
@@ -859,7 +868,7 @@ extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *
                                                  void *stream) {
     return dot_entry<false>("faith_dot_product_verification_QK", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
                             y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, length_y, dim_out, dim_in, epsilon,
-                            q, words, 0, stream);
+                            q, words, 0, 1, stream);
 }
 
 extern "C" int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
@@ -870,25 +879,29 @@ extern "C" int faith_dot_product_verification_V(float *x_l, float *y_l, float *x
                                                 int dim_in, float epsilon, int q, int words, void *stream) {
     return dot_entry<true>("faith_dot_product_verification_V", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
                            y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, dim_out, length_k, dim_in, epsilon,
-                           q, words, 0, stream);
+                           q, words, 0, 1, stream);
 }
 
 extern "C" int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
                                       const float *x_ub, const float *y_lb, const float *y_ub, const float *x_lw,
                                       const float *x_uw, const float *y_lw, const float *y_uw, float *z_lb, float *z_ub,
-                                      float *z_lw, float *z_uw, int heads, int length_x, int length_y, int head_size,
-                                      int dim_in, float epsilon, int q, int words, void *stream) {
+                                      float *z_lw, float *z_uw, int batch_size, int heads, int length_x, int length_y,
+                                      int head_size, int dim_in, float epsilon, int q, int words, void *stream) {
+    FAITH_REQUIRE(batch_size > 0 && heads > 0 && (long long)batch_size * heads <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "faith_attention_scores: batch=%d heads=%d out of range", batch_size, heads);
     return dot_entry<false>("faith_attention_scores", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
-                            z_lb, z_ub, z_lw, z_uw, heads, length_x, length_y, head_size, dim_in, epsilon, q, words,
-                            HEADS_X | HEADS_Y, stream);
+                            z_lb, z_ub, z_lw, z_uw, batch_size * heads, length_x, length_y, head_size, dim_in, epsilon, q,
+                            words, HEADS_X | HEADS_Y, heads, stream);
 }
 
 extern "C" int faith_attention_context(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
                                        const float *x_ub, const float *y_lb, const float *y_ub, const float *x_lw,
                                        const float *x_uw, const float *y_lw, const float *y_uw, float *z_lb, float *z_ub,
-                                       float *z_lw, float *z_uw, int heads, int length_x, int length_k, int head_size,
-                                       int dim_in, float epsilon, int q, int words, void *stream) {
+                                       float *z_lw, float *z_uw, int batch_size, int heads, int length_x, int length_k,
+                                       int head_size, int dim_in, float epsilon, int q, int words, void *stream) {
+    FAITH_REQUIRE(batch_size > 0 && heads > 0 && (long long)batch_size * heads <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "faith_attention_context: batch=%d heads=%d out of range", batch_size, heads);
     return dot_entry<true>("faith_attention_context", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
-                           z_lb, z_ub, z_lw, z_uw, heads, length_x, head_size, length_k, dim_in, epsilon, q, words,
-                           HEADS_Y | HEADS_Z, stream);
+                           z_lb, z_ub, z_lw, z_uw, batch_size * heads, length_x, head_size, length_k, dim_in, epsilon, q,
+                           words, HEADS_Y | HEADS_Z, heads, stream);
 }

@@ -4,10 +4,18 @@ operator surface only.
 Host-side mirror of the reference's per-network propagation
 (Transformer_Verification_Code/Verifiers/VerifierForward.py): `bound_input` (:127-156),
 `bound_attention` (:198-267), `bound_layer` (:158-196), `bound_pooling` (:269-287) and
-`bound_classifier` (:289-319).  Nothing here touches tensors except to fold attention heads into
-the batch axis and back (reshape / permute, as the reference does); all arithmetic happens in the
-methods of the bound object that is passed in, so the same code drives `faith_amd.Bounds` (HIP
-kernels) and any other object with those methods (the tests drive the CPU oracle with it).
+`bound_classifier` (:289-319), `verify_safety` (:93-125), and of the search for the certified radius
+of every position (Verifiers/Verifier.py:107-147).  Nothing here touches tensors except to build the
+input object and to fold attention heads into the batch axis and back where the bound object cannot
+address them in place; all arithmetic happens in the methods of the bound object that is passed in,
+so the same code drives `faith_amd.Bounds` (HIP kernels) and any other object with those methods
+(the tests drive the CPU oracle with it).
+
+The reference verifies one (position, radius) at a time.  Every operator here is independent
+across the batch axis, so `certified_radii` can also run the bisections of all positions in
+lockstep, one batch element per position (`bound_inputs`): the radius of an element is folded into
+its input coefficients (w = r * I with eps = 1 describes the same set as w = I with eps = r), so
+elements with different radii share every launch.
 
 Layers are plain objects with `.weight` / `.bias` tensors, laid out like the reference's BERT:
 
@@ -55,13 +63,15 @@ def _fold_heads(x, heads, size):
     return x
 
 
-def _unfold_heads(x):
-    """transpose_back (VerifierForward.py:253-263): [heads, L, D, size] -> [1, L, D, heads*size]."""
+def _unfold_heads(x, heads):
+    """transpose_back (VerifierForward.py:253-263): [B*heads, L, D, size] -> [B, L, D, heads*size]."""
     def w(t):
-        return t.permute(1, 2, 0, 3).reshape(1, t.shape[1], t.shape[2], -1)
+        n, L, D, size = t.shape
+        return t.reshape(n // heads, heads, L, D, size).permute(0, 2, 3, 1, 4).reshape(n // heads, L, D, -1)
 
     def b(t):
-        return t.permute(1, 0, 2).reshape(1, t.shape[1], -1)
+        n, L, size = t.shape
+        return t.reshape(n // heads, heads, L, size).permute(0, 2, 1, 3).reshape(n // heads, L, -1)
     x.lw, x.uw, x.lb, x.ub = w(x.lw), w(x.uw), b(x.lb), b(x.ub)
     x.update_shape()
     return x
@@ -85,7 +95,7 @@ def bound_attention(bounds_input, attention):
     probs = scores.softmax()
     _fold_heads(value, heads, size)
     context = probs.context(value)
-    _unfold_heads(context)
+    _unfold_heads(context, heads)
     return scores, probs, context
 
 
@@ -106,14 +116,97 @@ def bound_pooling(bounds, pooler_dense, make_bounds):
     return first.dense(pooler_dense).tanh()
 
 
-def bound_classifier(bounds, classifier, label):
-    """VerifierForward._bound_classifier: margin logit[0] - logit[1], concretized; True if provably safe."""
+def _margin(bounds, classifier):
     class Margin:
         weight = classifier.weight.clone()
         bias = classifier.bias.clone()
     Margin.weight[0, :] -= Margin.weight[1, :]
     Margin.bias[0] -= Margin.bias[1]
-    out = bounds.dense(Margin)
-    l, u = out.concretize()
+    return bounds.dense(Margin).concretize()
+
+
+def bound_classifier(bounds, classifier, label):
+    """VerifierForward._bound_classifier: margin logit[0] - logit[1], concretized; True if provably safe."""
+    l, u = _margin(bounds, classifier)
     safe = bool(l[0][0][0] > 0) if label == 0 else bool(u[0][0][0] < 0)
     return safe, l, u
+
+
+def bound_inputs(make_bounds, embeddings, indices, radii, p=2.0, norm=None, layer_norm="no_var"):
+    """Independent problems in one object: batch element b perturbs position indices[b] of the same
+    sentence within radius radii[b].  The radius goes into the coefficients and the object carries
+    eps = 1 (see the module docstring).  embeddings [1, L, dim]."""
+    length, dim = embeddings.shape[1], embeddings.shape[2]
+    n = len(indices)
+    dev = embeddings.device
+    w = torch.zeros((n, length, dim, dim), device=dev)
+    eye = torch.eye(dim, device=dev)
+    scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
+    w[torch.arange(n, device=dev), torch.as_tensor(indices, device=dev)] = scale[:, None, None] * eye
+    b = embeddings[0].unsqueeze(0).expand(n, length, dim).contiguous()
+    bounds = make_bounds(p, 1.0, w, b, w.clone(), b.clone())
+    if norm is not None:
+        bounds = bounds.layer_norm(norm, layer_norm)
+    return bounds
+
+
+def propagate(bounds, network):
+    """Embedding bounds -> bounds of the pooled output: every encoder layer, then the pooler
+    (the body of VerifierForward.verify_safety, :98-116)."""
+    for layer in network.layers:
+        _, _, bounds = bound_layer(bounds, layer, network.layer_norm, network.hidden_act)
+    return bounds
+
+
+def verify_safety(make_bounds, network, embeddings, index, eps, label, p=2.0, perturbed_words=1):
+    """VerifierForward.verify_safety (:93-125): True if the label provably survives every
+    perturbation of norm <= eps of the embedding at `index`.  A failed precondition inside the
+    propagation (reciprocal or sqrt of a bound that reaches zero) counts as not verified, as there."""
+    try:
+        x = bound_input(make_bounds, embeddings, index, eps, perturbed_words, p, network.embedding_norm,
+                        network.layer_norm)
+        x = propagate(x, network)
+        pooled = bound_pooling(x, network.pooler, make_bounds)
+        return bound_classifier(pooled, network.classifier, label)[0]
+    except AssertionError:
+        return False
+
+
+def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label, p=2.0):
+    """verify_safety for several (position, radius) pairs of one sentence in one propagation.
+    Returns a list of bools.  Needs a bound object that reports failed preconditions per batch
+    element instead of raising (`collect_failures`, as faith_amd.Bounds has)."""
+    x = bound_inputs(make_bounds, embeddings, indices, radii, p, network.embedding_norm, network.layer_norm)
+    with type(x).collect_failures(len(indices), embeddings.device) as failed:
+        x = propagate(x, network)
+        pooled = bound_pooling(x, network.pooler, make_bounds)
+        l, u = _margin(pooled, network.classifier)
+        ok = (l[:, 0, 0] > 0) if label == 0 else (u[:, 0, 0] < 0)
+        return [bool(v) for v in (ok & ~failed.mask).tolist()]
+
+
+def certified_radii(make_bounds, network, embeddings, positions, label, p=2.0, max_eps=0.1, num_iters=10,
+                    batched=False):
+    """The bisection of Verifier.verify (Verifiers/Verifier.py:131-139) for every position: l, r = 0,
+    max_eps; num_iters times { m = (l + r) / 2; verified at m ? l = m : r = m }; the answer is l.
+    batched = True runs step j of all positions as one propagation."""
+    lo = [0.0] * len(positions)
+    hi = [float(max_eps)] * len(positions)
+    if batched:
+        for _ in range(num_iters):
+            mid = [(a + b) / 2 for a, b in zip(lo, hi)]
+            safe = verify_safety_batch(make_bounds, network, embeddings, positions, mid, label, p)
+            for i, s in enumerate(safe):
+                if s:
+                    lo[i] = mid[i]
+                else:
+                    hi[i] = mid[i]
+        return lo
+    for i, pos in enumerate(positions):
+        for _ in range(num_iters):
+            m = (lo[i] + hi[i]) / 2
+            if verify_safety(make_bounds, network, embeddings, pos, m, label, p):
+                lo[i] = m
+            else:
+                hi[i] = m
+    return lo

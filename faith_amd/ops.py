@@ -382,15 +382,15 @@ def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
 def attention_scores(x, y, heads, p, eps, words=1):
     """Scores of all heads from query / key bounds as the dense layers leave them.
 
-    x, y: (lw [1, L, D, heads*size], lb [1, L, heads*size], uw, ub).  Same result as folding both with
+    x, y: (lw [B, L, D, heads*size], lb [B, L, heads*size], uw, ub).  Same result as folding both with
     transpose_for_scores (VerifierForward.py:208-229) and dot_product_qk, without the eight permuted
-    copies: returns (lw [heads, Lx, D, Ly], lb [heads, Lx, Ly], uw, ub)."""
+    copies: returns (lw [B*heads, Lx, D, Ly], lb [B*heads, Lx, Ly], uw, ub)."""
     xlw, xlb, xuw, xub = x
     ylw, ylb, yuw, yub = y
     B, Lx, D, H = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
     B2, Ly, D2, H2 = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
-    if B != 1 or B2 != 1 or (D2, H2) != (D, H):
-        raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} must be [1, L, dim_in, heads*size] alike")
+    if (B2, D2, H2) != (B, D, H):
+        raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} must be [B, L, dim_in, heads*size] alike")
     if heads <= 0 or H % heads:
         raise ValueError(f"{heads} heads do not divide a row of {H}")
     for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
@@ -399,47 +399,48 @@ def attention_scores(x, y, heads, p, eps, words=1):
     dev = xlw.device
     x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
     y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
-    zlw = torch.empty(heads, Lx, D, Ly, device=dev, dtype=torch.float32)
+    zlw = torch.empty(B * heads, Lx, D, Ly, device=dev, dtype=torch.float32)
     zuw = torch.empty_like(zlw)
-    zlb = torch.empty(heads, Lx, Ly, device=dev, dtype=torch.float32)
+    zlb = torch.empty(B * heads, Lx, Ly, device=dev, dtype=torch.float32)
     zub = torch.empty_like(zlb)
-    with _on(dev, "dot_qk", (heads, Lx, Ly, D, H // heads)):
+    with _on(dev, "dot_qk", (B * heads, Lx, Ly, D, H // heads)):
         _lib.call("faith_attention_scores", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
-                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), heads, Lx, Ly, H // heads, D, float(eps), q_code(p),
+                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, heads, Lx, Ly, H // heads, D, float(eps), q_code(p),
                   int(words), _stream(xlw))
     return zlw, zlb, zuw, zub
 
 
 def attention_context(x, y, p, eps, words=1):
-    """Context of all heads: probabilities x (lw [heads, Lx, D, Lk], lb [heads, Lx, Lk], uw, ub) times the
-    value bounds y as the dense layer leaves them (lw [1, Lk, D, heads*size], lb [1, Lk, heads*size], uw, ub).
+    """Context of all heads: probabilities x (lw [B*heads, Lx, D, Lk], lb [B*heads, Lx, Lk], uw, ub) times the
+    value bounds y as the dense layer leaves them (lw [B, Lk, D, heads*size], lb [B, Lk, heads*size], uw, ub).
 
     Same result as transpose_for_scores on y, dot_product_v and transpose_back
     (VerifierForward.py:208-229, :253-263) without the permuted copies: returns
-    (lw [1, Lx, D, heads*size], lb [1, Lx, heads*size], uw, ub)."""
+    (lw [B, Lx, D, heads*size], lb [B, Lx, heads*size], uw, ub)."""
     xlw, xlb, xuw, xub = x
     ylw, ylb, yuw, yub = y
-    heads, Lx, D, Lk = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
-    B2, Lk2, D2, H = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
-    if B2 != 1 or (Lk2, D2) != (Lk, D):
+    BH, Lx, D, Lk = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    B, Lk2, D2, H = _wb_shapes(ylw, ylb, LAYOUT_NATURAL)
+    if (Lk2, D2) != (Lk, D):
         raise ValueError(f"x {tuple(xlw.shape)} and y {tuple(ylw.shape)} disagree in key length or dim_in")
-    if H % heads:
-        raise ValueError(f"{heads} heads do not divide a row of {H}")
+    if BH % B or H % (BH // B):
+        raise ValueError(f"x has {BH} (batch, head) pairs; y has batch {B} and rows of {H}")
+    heads = BH // B
     for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
     x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
     y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
-    zlw = torch.empty(1, Lx, D, H, device=dev, dtype=torch.float32)
+    zlw = torch.empty(B, Lx, D, H, device=dev, dtype=torch.float32)
     zuw = torch.empty_like(zlw)
-    zlb = torch.empty(1, Lx, H, device=dev, dtype=torch.float32)
+    zlb = torch.empty(B, Lx, H, device=dev, dtype=torch.float32)
     zub = torch.empty_like(zlb)
-    with _on(dev, "dot_v", (heads, Lx, H // heads, D, Lk)):
+    with _on(dev, "dot_v", (BH, Lx, H // heads, D, Lk)):
         _lib.call("faith_attention_context", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
-                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), heads, Lx, Lk, H // heads, D, float(eps), q_code(p),
+                  _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, heads, Lx, Lk, H // heads, D, float(eps), q_code(p),
                   int(words), _stream(xlw))
     return zlw, zlb, zuw, zub
 

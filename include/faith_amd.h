@@ -238,12 +238,14 @@ int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *
 /*
  * Attention scores with the heads taken where the dense layers leave them.  Replaces
  * transpose_for_scores on query and key (VerifierForward.py:208-229: four permuted copies per
- * object) followed by Bounds.dot_product (Bounds.py:833-841): the kernels address head t of
- *   x_lw, x_uw [1, length_x, dim_in, heads * head_size];  x_lb, x_ub [1, length_x, heads * head_size]
- *   y_lw, y_uw [1, length_y, dim_in, heads * head_size];  y_lb, y_ub [1, length_y, heads * head_size]
+ * object) followed by Bounds.dot_product (Bounds.py:833-841): the kernels address head h of
+ *   x_lw, x_uw [batch, length_x, dim_in, heads * head_size];  x_lb, x_ub [batch, length_x, heads * head_size]
+ *   y_lw, y_uw [batch, length_y, dim_in, heads * head_size];  y_lb, y_ub [batch, length_y, heads * head_size]
  * in place.  x_l, x_u / y_l, y_u (out, caller's scratch) have the layout of x_lb / y_lb.  The
  * scores come out with the heads stacked on the batch axis, as the softmax wants them:
- *   z_lw, z_uw [heads, length_x, dim_in, length_y];  z_lb, z_ub [heads, length_x, length_y]
+ *   z_lw, z_uw [batch * heads, length_x, dim_in, length_y];  z_lb, z_ub [batch * heads, length_x, length_y]
+ * (the reference verifies one input at a time, batch = 1; batch > 1 carries independent problems,
+ * e.g. the perturbed positions of one sentence).
  */
 int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u,
                            const float *x_lb, const float *x_ub,
@@ -251,7 +253,7 @@ int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u,
                            const float *x_lw, const float *x_uw,
                            const float *y_lw, const float *y_uw,
                            float *z_lb, float *z_ub, float *z_lw, float *z_uw,
-                           int heads, int length_x, int length_y,
+                           int batch_size, int heads, int length_x, int length_y,
                            int head_size, int dim_in, float epsilon,
                            int q, int words, void *stream);
 
@@ -259,10 +261,10 @@ int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u,
  * Attention context with the values read, and the result written, where the dense layers want
  * them.  Replaces transpose_for_scores on the values, Bounds.context (Bounds.py:843-850) and
  * transpose_back (VerifierForward.py:253-263).
- *   x_lw, x_uw [heads, length_x, dim_in, length_k];  x_lb, x_ub [heads, length_x, length_k]   (probabilities)
- *   y_lw, y_uw [1, length_k, dim_in, heads * head_size];  y_lb, y_ub [1, length_k, heads * head_size]
+ *   x_lw, x_uw [batch * heads, length_x, dim_in, length_k];  x_lb, x_ub [batch * heads, length_x, length_k]   (probabilities)
+ *   y_lw, y_uw [batch, length_k, dim_in, heads * head_size];  y_lb, y_ub [batch, length_k, heads * head_size]
  *   x_l, x_u like x_lb;  y_l, y_u like y_lb   (out / scratch)
- *   z_lw, z_uw [1, length_x, dim_in, heads * head_size];  z_lb, z_ub [1, length_x, heads * head_size]
+ *   z_lw, z_uw [batch, length_x, dim_in, heads * head_size];  z_lb, z_ub [batch, length_x, heads * head_size]
  */
 int faith_attention_context(float *x_l, float *y_l, float *x_u, float *y_u,
                             const float *x_lb, const float *x_ub,
@@ -270,7 +272,7 @@ int faith_attention_context(float *x_l, float *y_l, float *x_u, float *y_u,
                             const float *x_lw, const float *x_uw,
                             const float *y_lw, const float *y_uw,
                             float *z_lb, float *z_ub, float *z_lw, float *z_uw,
-                            int heads, int length_x, int length_k,
+                            int batch_size, int heads, int length_x, int length_k,
                             int head_size, int dim_in, float epsilon,
                             int q, int words, void *stream);
 

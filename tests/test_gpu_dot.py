@@ -261,32 +261,39 @@ def test_c_bound_dot_shims():
 
 
 # ------------------------------------------------------------------ heads addressed in place
-def side_by_side(x):
-    """[heads, L, D, w] / [heads, L, w] -> the one object [1, L, D, heads*w] / [1, L, heads*w] that a
-    dense layer produces (inverse of transpose_for_scores, VerifierForward.py:208-229)."""
-    w = lambda t: t.permute(1, 2, 0, 3).reshape(1, t.shape[1], t.shape[2], -1).contiguous()
-    b = lambda t: t.permute(1, 0, 2).reshape(1, t.shape[1], -1).contiguous()
+def side_by_side(x, heads):
+    """[batch*heads, L, D, w] / [batch*heads, L, w] -> [batch, L, D, heads*w] / [batch, L, heads*w], the
+    object a dense layer produces (inverse of transpose_for_scores, VerifierForward.py:208-229)."""
+    def w(t):
+        bh, L, D, width = t.shape
+        return t.reshape(bh // heads, heads, L, D, width).permute(0, 2, 3, 1, 4).reshape(bh // heads, L, D, -1).contiguous()
+
+    def b(t):
+        bh, L, width = t.shape
+        return t.reshape(bh // heads, heads, L, width).permute(0, 2, 1, 3).reshape(bh // heads, L, -1).contiguous()
     return O.LinearBounds(w(x.lw), b(x.lb), w(x.uw), b(x.ub))
 
 
 @pytest.mark.parametrize("shape", [
-    # heads, Lx, Ly, D, head size
-    (4, 128, 128, 16, 64),      # straight-line MFMA kernel
-    (2, 130, 70, 20, 36),       # ragged tiles, half-empty last K-step
-    (4, 32, 32, 64, 16),        # short sequences: one 32 x 32 block per wavefront
-    (3, 6, 4, 5, 10),           # head size % 4 != 0: any-shape kernel
-    (2, 3, 5, 1, 8),            # dim_in == 1: interval shortcut
+    # batch, heads, Lx, Ly, D, head size
+    (1, 4, 128, 128, 16, 64),      # straight-line MFMA kernel
+    (2, 2, 128, 64, 8, 32),        # the same with two batch elements
+    (1, 2, 130, 70, 20, 36),       # ragged tiles, half-empty last K-step
+    (1, 4, 32, 32, 64, 16),        # short sequences: one 32 x 32 block per wavefront
+    (3, 2, 20, 40, 24, 24),        # short, ragged, three batch elements
+    (2, 3, 6, 4, 5, 10),           # head size % 4 != 0: any-shape kernel
+    (2, 2, 3, 5, 1, 8),            # dim_in == 1: interval shortcut
 ])
 @pytest.mark.parametrize("p", [2.0, INF])
 def test_attention_scores_reads_the_heads_in_place(shape, p):
     from faith_amd import ops
-    heads, Lx, Ly, D, d = shape
+    batch, heads, Lx, Ly, D, d = shape
     g = torch.Generator().manual_seed(41)
-    x = rand_bounds(g, heads, Lx, D, d, ordered=False, sw=0.3, sb=1.0)
-    y = rand_bounds(g, heads, Ly, D, d, ordered=False, sw=0.3, sb=1.0)
+    x = rand_bounds(g, batch * heads, Lx, D, d, ordered=False, sw=0.3, sb=1.0)
+    y = rand_bounds(g, batch * heads, Ly, D, d, ordered=False, sw=0.3, sb=1.0)
     words = 2 if D % 2 == 0 else 1
-    print(f"[case] attention_scores heads={heads} Lx={Lx} Ly={Ly} D={D} size={d} p={p} words={words}", flush=True)
-    got = ops.attention_scores(dev(side_by_side(x)), dev(side_by_side(y)), heads, p, 0.1, words)
+    print(f"[case] attention_scores batch={batch} heads={heads} Lx={Lx} Ly={Ly} D={D} size={d} p={p} words={words}", flush=True)
+    got = ops.attention_scores(dev(side_by_side(x, heads)), dev(side_by_side(y, heads)), heads, p, 0.1, words)
     torch.cuda.synchronize()
     exp = O.dot_product(x, y, p, 0.1, words)
     if D == 1:
@@ -300,31 +307,33 @@ def test_attention_scores_reads_the_heads_in_place(shape, p):
 
 
 @pytest.mark.parametrize("shape", [
-    # heads, queries, keys, D, head size
-    (4, 128, 128, 16, 64), (2, 128, 64, 8, 128),    # straight-line MFMA kernel
-    (2, 130, 72, 12, 20),       # ragged
-    (4, 32, 32, 64, 16),        # short sequences
-    (3, 6, 6, 4, 10),           # any-shape kernel
-    (2, 4, 4, 1, 8),            # interval shortcut
+    # batch, heads, queries, keys, D, head size
+    (1, 4, 128, 128, 16, 64), (1, 2, 128, 64, 8, 128),    # straight-line MFMA kernel
+    (2, 2, 128, 64, 8, 64),        # two batch elements
+    (1, 2, 130, 72, 12, 20),       # ragged
+    (1, 4, 32, 32, 64, 16),        # short sequences
+    (3, 2, 24, 16, 16, 24),        # short, three batch elements
+    (2, 3, 6, 6, 4, 10),           # any-shape kernel
+    (2, 2, 4, 4, 1, 8),            # interval shortcut
 ])
 @pytest.mark.parametrize("p", [2.0, INF])
 def test_attention_context_reads_and_writes_the_heads_in_place(shape, p):
     from faith_amd import ops
-    heads, Lq, Lk, D, dv = shape
+    batch, heads, Lq, Lk, D, dv = shape
     g = torch.Generator().manual_seed(42)
-    probs = rand_bounds(g, heads, Lq, D, Lk, ordered=False, sw=0.2, sb=0.5)
-    value = rand_bounds(g, heads, Lk, D, dv, ordered=False, sw=0.3, sb=1.0)
-    print(f"[case] attention_context heads={heads} Lq={Lq} Lk={Lk} D={D} size={dv} p={p}", flush=True)
-    got = ops.attention_context(dev(probs), dev(side_by_side(value)), p, 0.1, 1)
+    probs = rand_bounds(g, batch * heads, Lq, D, Lk, ordered=False, sw=0.2, sb=0.5)
+    value = rand_bounds(g, batch * heads, Lk, D, dv, ordered=False, sw=0.3, sb=1.0)
+    print(f"[case] attention_context batch={batch} heads={heads} Lq={Lq} Lk={Lk} D={D} size={dv} p={p}", flush=True)
+    got = ops.attention_context(dev(probs), dev(side_by_side(value, heads)), p, 0.1, 1)
     torch.cuda.synchronize()
     exp = O.context(probs, value, p, 0.1, 1)
-    exp_sbs = side_by_side(exp)
+    exp_sbs = side_by_side(exp, heads)
     if D == 1:
         for a, e in zip(got, exp_sbs.tensors()):
             assert close(a, e)
         return
     ref, mag = dot64(probs, O.transpose_bounds(value), p, 0.1, 1)
-    wrap = lambda r: side_by_side(O.LinearBounds(r["lw"], r["lb"], r["uw"], r["ub"]))
+    wrap = lambda r: side_by_side(O.LinearBounds(r["lw"], r["lb"], r["uw"], r["ub"]), heads)
     ref_s, mag_s = wrap(ref), wrap(mag)
     for name, a, e, r, m in zip(("lw", "lb", "uw", "ub"), got, exp_sbs.tensors(), ref_s.tensors(), mag_s.tensors()):
         assert a.shape == e.shape

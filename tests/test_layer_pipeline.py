@@ -97,3 +97,78 @@ def test_pipeline_on_hip_matches_the_oracle_and_is_sound(mode, p):
     gl, gu = g_out.concretize()
     check_sound(gl.cpu(), gu.cpu(), g_l.cpu(), g_u.cpu(), emb, parts, mode, p, eps, index,
                 torch.Generator().manual_seed(9))
+
+
+# ------------------------------------------------------------------ verification driver
+def network_of(parts, mode):
+    layer, embed_norm, pooler, classifier = parts
+    return SimpleNamespace(embedding_norm=embed_norm, layers=[layer], pooler=pooler, classifier=classifier,
+                           layer_norm=mode, hidden_act="relu")
+
+
+def test_certified_radius_on_the_oracle_brackets_the_verdict():
+    """Bisection of Verifier.verify: the radius it returns verifies, one step above it does not, and
+    the true network keeps its label inside the radius."""
+    layer, embed_norm, pooler, classifier, emb = build(11, "no_var")
+    net = network_of((layer, embed_norm, pooler, classifier), "no_var")
+    make = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)
+    _, margin = true_layer(emb.double(), layer, embed_norm, "no_var", pooler, classifier)
+    label = 0 if float(margin[0, 0]) > 0 else 1
+    max_eps, iters = 0.5, 6
+    (r,) = F.certified_radii(make, net, emb, [2], label, 2.0, max_eps, iters)
+    step = max_eps / 2 ** iters
+    assert 0 <= r < max_eps
+    if r > 0:
+        assert F.verify_safety(make, net, emb, 2, r, label, 2.0)
+    assert not F.verify_safety(make, net, emb, 2, r + step, label, 2.0)
+    # soundness: perturbations inside the certified radius do not flip the label
+    g = torch.Generator().manual_seed(12)
+    d = torch.randn(256, HIDDEN, generator=g, dtype=torch.float64)
+    d = d / d.norm(dim=1, keepdim=True) * r
+    x = emb.double().repeat(256, 1, 1)
+    x[:, 2] += d
+    _, m = true_layer(x, layer, embed_norm, "no_var", pooler, classifier)
+    assert bool(((m[:, 0] > 0) == (label == 0)).all())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+def test_batched_bisection_on_hip_matches_one_at_a_time_and_the_oracle(mode):
+    """All positions in lockstep (one batch element each, radius folded into the coefficients) give
+    the radii of the reference's one-at-a-time search, on the HIP path and on the oracle."""
+    from faith_amd import Bounds
+    layer, embed_norm, pooler, classifier, emb = build(11, mode)
+    parts = (layer, embed_norm, pooler, classifier)
+    _, margin = true_layer(emb.double(), layer, embed_norm, mode, pooler, classifier)
+    label = 0 if float(margin[0, 0]) > 0 else 1
+    positions, max_eps, iters = [1, 2, 3, 4], 0.5, 6
+    step = max_eps / 2 ** iters
+    omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)
+    want = F.certified_radii(omake, network_of(parts, mode), emb, positions, label, 2.0, max_eps, iters)
+
+    gnet = network_of(tuple(to_device(x, "cuda") for x in parts), mode)
+    gmake = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    one = F.certified_radii(gmake, gnet, emb.cuda(), positions, label, 2.0, max_eps, iters)
+    lock = F.certified_radii(gmake, gnet, emb.cuda(), positions, label, 2.0, max_eps, iters, batched=True)
+    print(f"[case] radii oracle {want} hip {one} hip batched {lock}", flush=True)
+    # a verdict that sits within rounding of the decision threshold may fall either way: one step
+    for a, b, c in zip(want, one, lock):
+        assert abs(a - b) <= step + 1e-12 and abs(a - c) <= step + 1e-12
+    assert sum(a == c for a, c in zip(want, lock)) >= len(positions) - 1
+
+
+@pytest.mark.gpu
+def test_failed_preconditions_are_recorded_per_batch_element():
+    """Inside collect_failures a reciprocal whose interval reaches zero marks its own batch element
+    only and nothing raises; outside it asserts, as the reference does."""
+    from faith_amd import Bounds
+    g = torch.Generator().manual_seed(13)
+    lw = 0.01 * torch.randn(3, 4, 8, 16, generator=g)
+    lb = torch.rand(3, 4, 16, generator=g) + 1.0
+    lb[1, 2, 5] = -0.5                                      # element 1 crosses zero
+    b = Bounds(None, 2.0, 0.1, lw=lw.cuda(), lb=lb.cuda(), uw=lw.cuda() + 0.001, ub=lb.cuda() + 0.1)
+    with Bounds.collect_failures(3, "cuda") as f:
+        b.reciprocal()
+        assert f.mask.tolist() == [False, True, False]
+    with pytest.raises(AssertionError):
+        b.reciprocal()
