@@ -360,7 +360,27 @@ def bench_layer(args, wl):
           "latency_us": round(per, 1), "latency_min_us": round(min(times) * 1e3 / len(positions), 1),
           "bound": "host", "achieved": 0.0, "peak": 1.0, "unit": "-", "frac": 0.0, "work": 0,
           "batch_latency_us": round(statistics.median(times) * 1e3, 1)}
-    return [e, e2]
+
+    # the same two, replayed from a HIP graph captured once (forward.CapturedVerifier)
+    out = [e, e2]
+    for batch, pos in ((1, [3]), (len(positions), positions)):
+        cap = F.CapturedVerifier(gmake, net, ge, batch, 0, p)
+        rr = [eps] * batch
+        t0 = time.time()
+        while time.time() - t0 < max(WARM_SECONDS, 0.05):
+            cap(pos, rr)
+        times = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            cap(pos, rr)
+            times.append((time.perf_counter() - t0) * 1e3)
+        out.append({"op": f"extra: the same network from a captured HIP graph, {batch} (position, radius) per replay "
+                          f"(wall clock per pair, input update and verdict readback included)",
+                    "latency_us": round(statistics.median(times) * 1e3 / batch, 1),
+                    "latency_min_us": round(min(times) * 1e3 / batch, 1), "bound": "host", "achieved": 0.0, "peak": 1.0,
+                    "unit": "-", "frac": 0.0, "work": 0})
+        del cap
+    return out
 
 
 def main():

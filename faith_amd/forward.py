@@ -176,8 +176,10 @@ def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label,
     """verify_safety for several (position, radius) pairs of one sentence in one propagation.
     Returns a list of bools.  Needs a bound object that reports failed preconditions per batch
     element instead of raising (`collect_failures`, as faith_amd.Bounds has)."""
-    x = bound_inputs(make_bounds, embeddings, indices, radii, p, network.embedding_norm, network.layer_norm)
+    x = bound_inputs(make_bounds, embeddings, indices, radii, p)
     with type(x).collect_failures(len(indices), embeddings.device) as failed:
+        if network.embedding_norm is not None:
+            x = x.layer_norm(network.embedding_norm, network.layer_norm)
         x = propagate(x, network)
         pooled = bound_pooling(x, network.pooler, make_bounds)
         l, u = _margin(pooled, network.classifier)
@@ -186,16 +188,19 @@ def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label,
 
 
 def certified_radii(make_bounds, network, embeddings, positions, label, p=2.0, max_eps=0.1, num_iters=10,
-                    batched=False):
+                    batched=False, captured=False):
     """The bisection of Verifier.verify (Verifiers/Verifier.py:131-139) for every position: l, r = 0,
     max_eps; num_iters times { m = (l + r) / 2; verified at m ? l = m : r = m }; the answer is l.
-    batched = True runs step j of all positions as one propagation."""
+    batched = True runs step j of all positions as one propagation; captured = True also replays
+    that propagation from a HIP graph captured at the first step."""
     lo = [0.0] * len(positions)
     hi = [float(max_eps)] * len(positions)
-    if batched:
+    if batched or captured:
+        step = CapturedVerifier(make_bounds, network, embeddings, len(positions), label, p) if captured else \
+            (lambda idx, r: verify_safety_batch(make_bounds, network, embeddings, idx, r, label, p))
         for _ in range(num_iters):
             mid = [(a + b) / 2 for a, b in zip(lo, hi)]
-            safe = verify_safety_batch(make_bounds, network, embeddings, positions, mid, label, p)
+            safe = step(positions, mid)
             for i, s in enumerate(safe):
                 if s:
                     lo[i] = mid[i]
@@ -210,3 +215,56 @@ def certified_radii(make_bounds, network, embeddings, positions, label, p=2.0, m
             else:
                 hi[i] = m
     return lo
+
+
+class CapturedVerifier:
+    """verify_safety_batch for one sentence with the whole propagation captured ONCE as a HIP graph.
+
+    A propagation is a fixed sequence of launches whose arguments depend on shapes only: the radius
+    lives in the input coefficients (eps = 1, see bound_inputs) and failed preconditions are recorded
+    on the device, so nothing in it waits for the host.  Replaying the graph takes the per-launch
+    host work (23 C-ABI calls and about as many tensor allocations per layer) out of every
+    (positions, radii) query after the first.  Needs a bound object with collect_failures
+    (faith_amd.Bounds).  `batch` is the number of (position, radius) pairs per replay."""
+
+    def __init__(self, make_bounds, network, embeddings, batch, label, p=2.0):
+        length, dim = embeddings.shape[1], embeddings.shape[2]
+        dev = embeddings.device
+        self.batch, self.label, self.dim = batch, label, dim
+        self.w = torch.zeros((batch, length, dim, dim), device=dev)
+        self.b = embeddings[0].unsqueeze(0).expand(batch, length, dim).contiguous()
+        self.eye = torch.eye(dim, device=dev)
+        self.rows = torch.arange(batch, device=dev)
+
+        def body():
+            x = make_bounds(p, 1.0, self.w, self.b, self.w.clone(), self.b.clone())
+            with type(x).collect_failures(batch, dev) as failed:
+                if network.embedding_norm is not None:
+                    x = x.layer_norm(network.embedding_norm, network.layer_norm)
+                pooled = bound_pooling(propagate(x, network), network.pooler, make_bounds)
+                l, u = _margin(pooled, network.classifier)
+            ok = (l[:, 0, 0] > 0) if label == 0 else (u[:, 0, 0] < 0)
+            return ok & ~failed.mask
+
+        # torch's capture protocol: run eagerly on a side stream first (library handles, caches of
+        # device properties, the allocator's pools), then capture
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                body()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.safe = body()
+
+    def __call__(self, indices, radii):
+        """Verdicts for batch element b = (position indices[b], radius radii[b]); len == batch."""
+        assert len(indices) == self.batch and len(radii) == self.batch
+        dev = self.w.device
+        self.w.zero_()
+        scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
+        self.w[self.rows, torch.as_tensor(indices, device=dev)] = scale[:, None, None] * self.eye
+        self.graph.replay()
+        return [bool(v) for v in self.safe.tolist()]

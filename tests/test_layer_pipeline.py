@@ -172,3 +172,34 @@ def test_failed_preconditions_are_recorded_per_batch_element():
         assert f.mask.tolist() == [False, True, False]
     with pytest.raises(AssertionError):
         b.reciprocal()
+
+
+@pytest.mark.gpu
+def test_captured_propagation_replays_like_the_eager_one():
+    """The propagation captured as a HIP graph: every replay -- with other radii and positions, and
+    with eager work and synchronisations in between -- gives the eager verdicts and margins."""
+    from faith_amd import Bounds
+    layer, embed_norm, pooler, classifier, emb = build(11, "standard")
+    parts = (layer, embed_norm, pooler, classifier)
+    _, margin = true_layer(emb.double(), layer, embed_norm, "standard", pooler, classifier)
+    label = 0 if float(margin[0, 0]) > 0 else 1
+    gnet = network_of(tuple(to_device(x, "cuda") for x in parts), "standard")
+    gmake = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    ge = emb.cuda()
+    cap = F.CapturedVerifier(gmake, gnet, ge, 4, label, 2.0)
+    queries = [([1, 2, 3, 4], [0.004, 0.004, 0.004, 0.004]), ([4, 3, 2, 1], [0.001, 0.02, 0.008, 0.3]),
+               ([1, 1, 1, 1], [0.0005, 0.009, 0.0078125, 1.0]), ([2, 4, 2, 4], [0.012, 0.012, 0.25, 0.004]),
+               ([1, 2, 3, 4], [0.004, 0.004, 0.004, 0.004])]
+    seen = set()
+    for idx, radii in queries:
+        print(f"[case] captured replay positions {idx} radii {radii}", flush=True)
+        got = cap(idx, radii)
+        want = F.verify_safety_batch(gmake, gnet, ge, idx, radii, label, 2.0)      # eager work between replays
+        torch.cuda.synchronize()
+        assert got == want, (idx, radii, got, want)
+        seen.update(got)
+    assert seen == {True, False}                  # the queries exercise both verdicts
+    # and the search built on it finds the same radii
+    a = F.certified_radii(gmake, gnet, ge, [1, 2, 3, 4], label, 2.0, 0.5, 6, batched=True)
+    b = F.certified_radii(gmake, gnet, ge, [1, 2, 3, 4], label, 2.0, 0.5, 6, captured=True)
+    assert a == b
