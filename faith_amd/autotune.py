@@ -256,7 +256,7 @@ class TuningResult:
 def autotune(op, shape, run, heuristics=None, rounds=3, samples=3, measure=None, setter=None, seed=0):
     """Finds the fastest valid candidate for run() -- a callable that launches the operator once.
 
-    Round 0 measures `samples` candidates drawn at random; every later round fits the cost model to
+    The first tuning round measures `samples` candidates drawn at random; every later one fits the cost model to
     what has been measured and measures the `samples` unmeasured candidates it predicts to be fastest
     (autotuner.py:99-147).  The built-in choice (all knobs 0) is always among the measured ones, so the
     result is never slower than not tuning.  measure(run) -> microseconds defaults to GPU events."""

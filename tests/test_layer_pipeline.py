@@ -203,3 +203,49 @@ def test_captured_propagation_replays_like_the_eager_one():
     a = F.certified_radii(gmake, gnet, ge, [1, 2, 3, 4], label, 2.0, 0.5, 6, batched=True)
     b = F.certified_radii(gmake, gnet, ge, [1, 2, 3, 4], label, 2.0, 0.5, 6, captured=True)
     assert a == b
+
+
+def two_layer_network(seed, mode):
+    g = torch.Generator().manual_seed(seed)
+    layers = [random_layer(g, HIDDEN, HEADS, INTER), random_layer(g, HIDDEN, HEADS, INTER)]
+    embed_norm = SimpleNamespace(weight=1.0 + 0.1 * torch.randn(HIDDEN, generator=g),
+                                 bias=0.05 * torch.randn(HIDDEN, generator=g))
+    pooler = SimpleNamespace(weight=torch.randn(HIDDEN, HIDDEN, generator=g) / HIDDEN ** 0.5,
+                             bias=0.05 * torch.randn(HIDDEN, generator=g))
+    classifier = SimpleNamespace(weight=torch.randn(2, HIDDEN, generator=g) / HIDDEN ** 0.5,
+                                 bias=0.05 * torch.randn(2, generator=g))
+    emb = torch.randn(1, LENGTH, HIDDEN, generator=g)
+    net = SimpleNamespace(embedding_norm=embed_norm, layers=layers, pooler=pooler, classifier=classifier,
+                          layer_norm=mode, hidden_act="relu")
+    return net, emb
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+def test_two_layers_with_two_perturbed_words_match_the_oracle(mode):
+    """Two encoder layers, two perturbed positions (dim_in = 2 * hidden, perturbed_words = 2): the
+    margin bounds of the HIP path against the oracle's."""
+    from faith_amd import Bounds
+    net, emb = two_layer_network(21, mode)
+    eps, index, p = 0.01, [1, 4], 2.0
+
+    def margins(make, network, e):
+        x = F.bound_input(make, e, index, eps, 2, p, network.embedding_norm, network.layer_norm)
+        pooled = F.bound_pooling(F.propagate(x, network), network.pooler, make)
+        return F.bound_classifier(pooled, network.classifier, 0)
+
+    omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub, words=2)
+    _, ol, ou = margins(omake, net, emb)
+
+    two_words = SimpleNamespace(perturbed_words=2)
+    gmake = lambda p_, e_, lw, lb, uw, ub: Bounds(two_words, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    gnet = SimpleNamespace(**{k: (to_device(v, "cuda") if k in ("embedding_norm", "pooler", "classifier") else v)
+                              for k, v in vars(net).items()})
+    gnet.layers = [to_device(l, "cuda") for l in net.layers]
+    _, gl, gu = margins(gmake, gnet, emb.cuda())
+    torch.cuda.synchronize()
+    assert bool((gl <= gu).all())
+    width = float((ou - ol).abs().max())
+    # ~50 chained operators, tanh slopes at the end: compare relative to the width of the interval
+    assert float((gl.cpu() - ol).abs().max()) <= 2e-3 * max(width, 1.0), (gl, ol)
+    assert float((gu.cpu() - ou).abs().max()) <= 2e-3 * max(width, 1.0), (gu, ou)
