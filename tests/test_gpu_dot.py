@@ -338,3 +338,29 @@ def test_attention_context_reads_and_writes_the_heads_in_place(shape, p):
     for name, a, e, r, m in zip(("lw", "lb", "uw", "ub"), got, exp_sbs.tensors(), ref_s.tensors(), mag_s.tensors()):
         assert a.shape == e.shape
         compare_contraction(name, a, e, r, m)
+
+
+def test_in_place_heads_equal_stacked_heads_bit_for_bit_at_configuration_3_size():
+    """Same kernels, same summation order, different addressing: the in-place entry points must
+    reproduce the stacked ones exactly (4 heads, L = 128, D_in = 256, d = 64; scores and context)."""
+    from faith_amd import ops
+    heads, L, D, d = 4, 128, 256, 64
+    g = torch.Generator(device="cuda").manual_seed(43)
+    mk = lambda *s: torch.randn(*s, device="cuda", generator=g)
+    def obj(scale):
+        lw, lb = mk(heads, L, D, d) * scale, mk(heads, L, d)
+        return (lw, lb, lw + 0.01 * mk(heads, L, D, d).abs(), lb + 0.1 * mk(heads, L, d).abs())
+    q, k, v = obj(0.05), obj(0.05), obj(0.05)
+    sbs_w = lambda t: t.permute(1, 2, 0, 3).reshape(1, L, D, heads * d).contiguous()
+    sbs_b = lambda t: t.permute(1, 0, 2).reshape(1, L, heads * d).contiguous()
+    sbs = lambda o: (sbs_w(o[0]), sbs_b(o[1]), sbs_w(o[2]), sbs_b(o[3]))
+    print("[case] in-place heads against stacked heads, configuration 3 size", flush=True)
+    stacked = ops.dot_product_qk(q, k, INF, 0.01, 1)
+    in_place = ops.attention_scores(sbs(q), sbs(k), heads, INF, 0.01, 1)
+    for a, b in zip(stacked, in_place):
+        assert torch.equal(a, b)
+    ctx = ops.dot_product_v(stacked, v, INF, 0.01, 1)
+    ctx_in_place = ops.attention_context(stacked, sbs(v), INF, 0.01, 1)
+    for a, b in zip(ctx, ctx_in_place):
+        want = sbs_w(a) if a.dim() == 4 else sbs_b(a)
+        assert torch.equal(want, b)
