@@ -383,6 +383,19 @@ def bench_layer(args, wl):
     return out
 
 
+def measured_mfma_clock_mhz(compute_units):
+    """Median shader clock over all workgroups while every SIMD issues fp32 MFMAs (about 2 ms)."""
+    import torch
+    from faith_amd import _lib
+    n = 2 * compute_units
+    out = torch.zeros(n, device="cuda")
+    stream = torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    for _ in range(3):                       # the first launches after idle run at lower clocks
+        _lib.call("faith_mfma_clock", out.data_ptr(), n, 2000, stream)
+    torch.cuda.synchronize()
+    return float(out.median())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -413,7 +426,11 @@ def main():
         from oracle import bounds_oracle as O     # cpu_baseline leg only
 
     prop = torch.cuda.get_device_properties(0)
-    log(f"device: {prop.name}, {prop.multi_processor_count} CUs, host threads {torch.get_num_threads()}")
+    clock_mhz = measured_mfma_clock_mhz(prop.multi_processor_count)
+    peak_here = prop.multi_processor_count * 256 * clock_mhz * 1e-6        # 256 fp32 MFMA flop / clock / CU
+    log(f"device: {prop.name}, {prop.multi_processor_count} CUs, host threads {torch.get_num_threads()}; shader clock "
+        f"under MFMA load {clock_mhz:.0f} MHz -> fp32 MFMA peak at that clock {peak_here:.1f} TFLOP/s "
+        f"(roofline fractions below use the published {MFMA_FP32_PEAK_TFLOPS} TFLOP/s)")
 
     head, entries = bench_config1(args, ops, O, wl, args.steps, args.warmup)
     extra = set() if args.only_headline else {int(c) for c in args.configs.split(",") if c.strip()}
@@ -440,7 +457,8 @@ def main():
         "config": {"workload": "config1: relu+tanh relaxation, lw/uw [1,128,256,512], words=2, eps=0.01, "
                                "p in {1,2,inf} (6 launches per step)",
                    "bytes_per_step": head["bytes_per_step"], "device": prop.name,
-                   "compute_units": prop.multi_processor_count},
+                   "compute_units": prop.multi_processor_count, "shader_clock_mhz_under_mfma_load": round(clock_mhz, 1),
+                   "fp32_mfma_peak_at_measured_clock_tflops": round(peak_here, 1)},
         "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "ops": entries,
     }
     print(json.dumps(line), flush=True)

@@ -24,6 +24,7 @@ _F = ctypes.c_float
 SIGNATURES = {
     "faith_tune_set": [_I, _I],
     "faith_copy_f32": [_P, _P, ctypes.c_longlong, _P],
+    "faith_mfma_clock": [_P, _I, _I, _P],
     "faith_concretize": [_P] * 6 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_relu_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_tanh_verification": [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],

@@ -69,6 +69,42 @@ extern "C" int faith_copy_f32(const float *src, float *dst, long long n, void *s
     return faith::check_launch("faith_copy_f32");
 }
 
+// Shader clock under matrix load: every workgroup keeps its four SIMDs issuing fp32 MFMAs for
+// `iterations` rounds of 16 and divides the shader-cycle counter by the constant 100 MHz counter.
+typedef float clk_floatx16 __attribute__((ext_vector_type(16)));
+__global__ void __launch_bounds__(256) mfma_clock_kernel(float *__restrict__ mhz, const int iterations) {
+    clk_floatx16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    const float a = 1e-3f * (float)(threadIdx.x % 7), b = 0.5f;
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = __builtin_amdgcn_s_memrealtime();
+    float keep = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) keep += acc[i][0];
+    if (threadIdx.x == 0)
+        mhz[blockIdx.x] = (r1 > r0 ? (float)((double)(c1 - c0) / (double)(r1 - r0) * 100.0) : 0.f) + (keep == 1234.5f ? 1.f : 0.f);
+}
+
+extern "C" int faith_mfma_clock(float *mhz, int workgroups, int iterations, void *stream) {
+    FAITH_NOT_NULL(mhz);
+    FAITH_REQUIRE(workgroups > 0 && workgroups <= 65536 && iterations > 0 && iterations <= 100000, FAITH_ERR_SHAPE,
+                  "faith_mfma_clock: workgroups=%d (1..65536), iterations=%d (1..100000)", workgroups, iterations);
+    hipLaunchKernelGGL(mfma_clock_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), mhz,
+                       iterations);
+    return faith::check_launch("faith_mfma_clock");
+}
+
 extern "C" const char *faith_last_error(void) { return faith::g_error; }
 
 extern "C" int faith_version(void) { return 1; }

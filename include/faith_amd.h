@@ -64,6 +64,14 @@ int faith_tune_set(int knob, int value);
 int faith_copy_f32(const float *src, float *dst, long long n, void *stream);
 
 /*
+ * Shader clock under matrix load, in MHz, one value per workgroup in mhz[0 .. workgroups-1]: every
+ * workgroup issues 16 * iterations fp32 MFMAs per wavefront on all four SIMDs and divides the
+ * shader-cycle counter by the constant 100 MHz counter.  Measurement aid with no counterpart in
+ * the reference: the clock at which the MFMA peak has to be priced on the machine at hand.
+ */
+int faith_mfma_clock(float *mhz, int workgroups, int iterations, void *stream);
+
+/*
  * Dual-norm concretization.  Replaces Bounds.concretize (Bounds.py:311-326) and the
  * CUDA `concretize` kernel (HandTunedKernels/dot_product_verification.cu:47-105).
  *   l[r,j] = lb[r,j] - eps * sum_w ||lw[r, block w, j]||_q

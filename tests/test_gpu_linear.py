@@ -128,3 +128,12 @@ def test_linear_config2_full_size_properties():
     assert torch.equal(o2[0], olw * 2) and torch.equal(o2[2], ouw * 2)
     l, u = ops.concretize(olw, olb, ouw, oub, c["p"], c["eps"], c["words"])
     assert bool((l <= u).all())
+
+
+def test_mfma_clock_measurement_is_plausible():
+    """faith_mfma_clock: every workgroup reports a shader clock between 0.5 and 3.5 GHz."""
+    from faith_amd import _lib
+    out = torch.zeros(64, device="cuda")
+    _lib.call("faith_mfma_clock", out.data_ptr(), 64, 200, torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
+    torch.cuda.synchronize()
+    assert bool(((out > 500) & (out < 3500)).all()), out
