@@ -37,6 +37,7 @@ struct ActArgs {
     const float *lb2 = nullptr, *ub2 = nullptr, *lw2 = nullptr, *uw2 = nullptr;
     float *l2 = nullptr, *u2 = nullptr;
     int rows2 = 0;
+    float qv = 0.f;     // the dual exponent when it is none of 1, 2, inf
 };
 
 // y = k * (v - x0) + y0
@@ -235,8 +236,8 @@ __device__ __forceinline__ void neuron_stage(const ActArgs &a, const float *part
                 nl = ncomb<Q>(nl, part[((w * NW + g) * 2 + 0) * TH + lane]);
                 nu = ncomb<Q>(nu, part[((w * NW + g) * 2 + 1) * TH + lane]);
             }
-            l += (-a.eps) * nfin<Q>(nl);
-            u += a.eps * nfin<Q>(nu);
+            l += (-a.eps) * nfin<Q>(nl, a.qv);
+            u += a.eps * nfin<Q>(nu, a.qv);
         }
         if (p_l) p_l[bi] = l;
         if (p_u) p_u[bi] = u;
@@ -324,8 +325,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
                 if (row >= lo_row && row < hi_row) {
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) {
-                        pl[v] = nacc<Q>(pl[v], dl[i].get(v));
-                        pu[v] = nacc<Q>(pu[v], du[i].get(v));
+                        pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
+                        pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
                     }
                 }
             }
@@ -439,8 +440,8 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4
             if (row >= lo_row && row < hi_row) {
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
-                    pl[v] = nacc<Q>(pl[v], dl[i].get(v));
-                    pu[v] = nacc<Q>(pu[v], du[i].get(v));
+                    pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
+                    pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
                 }
             }
         }
@@ -543,13 +544,13 @@ __global__ void __launch_bounds__(256) act_transposed(const ActArgs a) {
         for (int w = 0; w < a.words; ++w) {
             float nl = 0.f, nu = 0.f;
             for (int k = w * blk + lane; k < (w + 1) * blk; k += WAVE) {
-                nl = nacc<Q>(nl, pl[k]);
-                nu = nacc<Q>(nu, pu[k]);
+                nl = nacc<Q>(nl, pl[k], a.qv);
+                nu = nacc<Q>(nu, pu[k], a.qv);
             }
             nl = Q == FAITH_Q_INF ? wave_max(nl) : wave_sum(nl);
             nu = Q == FAITH_Q_INF ? wave_max(nu) : wave_sum(nu);
-            l += (-a.eps) * nfin<Q>(nl);
-            u += a.eps * nfin<Q>(nu);
+            l += (-a.eps) * nfin<Q>(nl, a.qv);
+            u += a.eps * nfin<Q>(nu, a.qv);
         }
         if (lane == 0) {
             s_l[t] = l;
@@ -640,15 +641,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) a
                 if (k0 >= w * blk && k0 < (w + 1) * blk) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        nl = nacc<Q>(nl, dl[i][v].get(c));
-                        nu = nacc<Q>(nu, du[i][v].get(c));
+                        nl = nacc<Q>(nl, dl[i][v].get(c), a.qv);
+                        nu = nacc<Q>(nu, du[i][v].get(c), a.qv);
                     }
                 }
             }
             nl = Q == FAITH_Q_INF ? wave_max(nl) : wave_sum(nl);
             nu = Q == FAITH_Q_INF ? wave_max(nu) : wave_sum(nu);
-            li += (-a.eps) * nfin<Q>(nl);
-            ui += a.eps * nfin<Q>(nu);
+            li += (-a.eps) * nfin<Q>(nl, a.qv);
+            ui += a.eps * nfin<Q>(nu, a.qv);
         }
         l[i] = li;
         u[i] = ui;
@@ -785,8 +786,10 @@ int run(const char *who, ActArgs a, int q, int layout, void *stream) {
                   "%s: rows=%d dim_in=%d dim_out=%d must all be positive", who, a.rows, a.D, a.H);
     FAITH_REQUIRE(a.words >= 1 && a.words <= 16 && a.D % a.words == 0, FAITH_ERR_SHAPE,
                   "%s: words=%d must be in 1..16 and divide dim_in=%d", who, a.words, a.D);
-    FAITH_REQUIRE(q == FAITH_Q_1 || q == FAITH_Q_2 || q == FAITH_Q_INF, FAITH_ERR_UNSUPPORTED,
-                  "%s: q=%d is not one of FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF", who, q);
+    if (!faith::dual_exponent(q, &a.qv)) {
+        faith::set_error("%s: q=%d is neither FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF nor the bits of an exponent in (1, inf)", who, q);
+        return FAITH_ERR_UNSUPPORTED;
+    }
     FAITH_REQUIRE(layout == FAITH_LAYOUT_NATURAL || layout == FAITH_LAYOUT_TRANSPOSED, FAITH_ERR_UNSUPPORTED,
                   "%s: unknown layout %d", who, layout);
     FAITH_REQUIRE((long long)a.rows * a.H * 1LL <= 0x7fffffffLL * 32, FAITH_ERR_SHAPE, "%s: problem too large", who);
@@ -794,7 +797,8 @@ int run(const char *who, ActArgs a, int q, int layout, void *stream) {
     switch (q) {
         case FAITH_Q_1: dispatch_layout<MODE, FAITH_Q_1>(a, layout, st); break;
         case FAITH_Q_2: dispatch_layout<MODE, FAITH_Q_2>(a, layout, st); break;
-        default: dispatch_layout<MODE, FAITH_Q_INF>(a, layout, st); break;
+        case FAITH_Q_INF: dispatch_layout<MODE, FAITH_Q_INF>(a, layout, st); break;
+        default: dispatch_layout<MODE, Q_GENERAL>(a, layout, st); break;
     }
     return faith::check_launch(who);
 }

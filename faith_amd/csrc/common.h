@@ -20,6 +20,10 @@ int concretize_pair(const float *lb, const float *ub, const float *lw, const flo
                     const float *lb2, const float *ub2, const float *lw2, const float *uw2, float *l2, float *u2,
                     int rows2, int dim_in, int dim_out, float eps, int q, int words, void *stream);
 
+// The `q` argument of the entry points: FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF, or the IEEE-754 bits of any
+// other dual exponent in (1, inf) (written to *qv).  False if it is neither.
+bool dual_exponent(int q, float *qv);
+
 // Compute units of the current device (queried once per device, then cached).
 int compute_units();
 

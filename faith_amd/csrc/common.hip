@@ -21,6 +21,16 @@ int check_launch(const char *what) {
     return FAITH_OK;
 }
 
+bool dual_exponent(int q, float *qv) {
+    if (q == FAITH_Q_1 || q == FAITH_Q_2 || q == FAITH_Q_INF) return true;
+    float f;
+    static_assert(sizeof(f) == sizeof(q), "q carries the bits of a float");
+    __builtin_memcpy(&f, &q, sizeof(f));
+    if (!(f > 1.0f) || f > 3.0e38f) return false;      // rejects NaN, inf, and anything <= 1
+    *qv = f;
+    return true;
+}
+
 int compute_units() {
     static int cached[64] = {0};
     int dev = 0;

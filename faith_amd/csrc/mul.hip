@@ -26,6 +26,7 @@ struct MulArgs {
     float *zlb, *zub, *zlw, *zuw;
     int rows, D, H, words;
     float eps;
+    float qv = 0.f;     // the dual exponent when it is none of 1, 2, inf
 };
 
 template <int Q, int VEC, int TPR, int NTHREADS, int RPT>
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(NTHREADS) mul_natural(const MulArgs a) {
 #pragma unroll
                     for (int t = 0; t < 4; ++t)
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v));
+                        for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v), a.qv);
                 }
             }
 #pragma unroll
@@ -121,9 +122,9 @@ __global__ void __launch_bounds__(NTHREADS) mul_natural(const MulArgs a) {
             for (int g = 0; g < NW; ++g)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) n[t] = ncomb<Q>(n[t], part[((w * NW + g) * 4 + t) * TH + lane]);
-            lx += (-a.eps) * nfin<Q>(n[0]);
-            ly += (-a.eps) * nfin<Q>(n[2]);
-            uy += a.eps * nfin<Q>(n[3]);
+            lx += (-a.eps) * nfin<Q>(n[0], a.qv);
+            ly += (-a.eps) * nfin<Q>(n[2], a.qv);
+            uy += a.eps * nfin<Q>(n[3], a.qv);
         }
         const float al = ly, au = uy, bt = lx;
         coef[lane] = al;
@@ -213,7 +214,7 @@ __global__ void __launch_bounds__(NTHREADS) mul_resident(const MulArgs a) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v));
+                    for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v), a.qv);
             }
         }
 #pragma unroll
@@ -242,9 +243,9 @@ __global__ void __launch_bounds__(NTHREADS) mul_resident(const MulArgs a) {
             for (int g = 0; g < NW; ++g)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) n[t] = ncomb<Q>(n[t], part[((w * NW + g) * 4 + t) * TH + lane]);
-            lx += (-a.eps) * nfin<Q>(n[0]);
-            ly += (-a.eps) * nfin<Q>(n[2]);
-            uy += a.eps * nfin<Q>(n[3]);
+            lx += (-a.eps) * nfin<Q>(n[0], a.qv);
+            ly += (-a.eps) * nfin<Q>(n[2], a.qv);
+            uy += a.eps * nfin<Q>(n[3], a.qv);
         }
         const float al = ly, au = uy, bt = lx;
         coef[lane] = al;
@@ -332,13 +333,19 @@ extern "C" int faith_multiply_verification(const float *x_lb, const float *x_ub,
                   "faith_multiply_verification: length=%d dim_in=%d dim_out=%d must be positive", length, dim_in, dim_out);
     FAITH_REQUIRE(words >= 1 && words <= 16 && dim_in % words == 0, FAITH_ERR_SHAPE,
                   "faith_multiply_verification: words=%d must be in 1..16 and divide dim_in=%d", words, dim_in);
-    FAITH_REQUIRE(q == FAITH_Q_1 || q == FAITH_Q_2 || q == FAITH_Q_INF, FAITH_ERR_UNSUPPORTED,
-                  "faith_multiply_verification: q=%d is not one of FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF", q);
+    float qv = 0.f;
+    if (!faith::dual_exponent(q, &qv)) {
+        faith::set_error("faith_multiply_verification: q=%d is neither FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF nor the bits of "
+                         "an exponent in (1, inf)", q);
+        return FAITH_ERR_UNSUPPORTED;
+    }
     MulArgs a{x_lb, x_ub, x_lw, x_uw, y_lb, y_ub, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, length, dim_in, dim_out, words,
               epsilon};
     hipStream_t st = static_cast<hipStream_t>(stream);
+    a.qv = qv;
     if (q == FAITH_Q_1) dispatch_mul<FAITH_Q_1>(a, st);
     else if (q == FAITH_Q_2) dispatch_mul<FAITH_Q_2>(a, st);
-    else dispatch_mul<FAITH_Q_INF>(a, st);
+    else if (q == FAITH_Q_INF) dispatch_mul<FAITH_Q_INF>(a, st);
+    else dispatch_mul<Q_GENERAL>(a, st);
     return faith::check_launch("faith_multiply_verification");
 }

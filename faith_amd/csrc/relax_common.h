@@ -9,12 +9,17 @@ constexpr int WAVE = 64;
 constexpr float TINY = 1e-12f;   // Bounds.py:27
 
 // ------------------------------------------------------------------ q-norm pieces
+// Q is FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF or Q_GENERAL (any other dual exponent q, 1 < q < inf,
+// carried at run time in `qv`): sum of |v|^q as exp2(q log2|v|) -- two quarter-rate instructions per
+// value, still far below what an HBM-bound pass has to spare -- and the 1/q power at the end.
+constexpr int Q_GENERAL = 3;
 template <int Q>
-__device__ __forceinline__ float nacc(float acc, float v) {
+__device__ __forceinline__ float nacc(float acc, float v, float qv) {
     // one fused instruction: a separate square would be hoisted out of the loop over the perturbed
     // words and held for every value a thread keeps (64 more registers)
     if (Q == FAITH_Q_2) return __builtin_fmaf(v, v, acc);
     if (Q == FAITH_Q_1) return acc + fabsf(v);
+    if (Q == Q_GENERAL) return acc + __builtin_amdgcn_exp2f(qv * __builtin_amdgcn_logf(fabsf(v)));   // |0|^q = exp2(-inf) = 0
     // max(acc, |v|) as one median-of-three (fmaxf adds a canonicalising v_max per value)
     return __builtin_amdgcn_fmed3f(acc, fabsf(v), __builtin_inff());
 }
@@ -23,7 +28,8 @@ __device__ __forceinline__ float ncomb(float a, float b) {
     return Q == FAITH_Q_INF ? fmaxf(a, b) : a + b;
 }
 template <int Q>
-__device__ __forceinline__ float nfin(float a) {
+__device__ __forceinline__ float nfin(float a, float qv) {
+    if (Q == Q_GENERAL) return a > 0.f ? exp2f(log2f(a) / qv) : 0.f;
     return Q == FAITH_Q_2 ? sqrtf(a) : a;
 }
 

@@ -7,6 +7,7 @@ plus the current HIP stream to libfaith_amd.so.  No arithmetic happens here.
 from __future__ import annotations
 
 import math
+import struct
 
 import torch
 
@@ -22,7 +23,10 @@ def q_code(p: float) -> int:
         return Q_2
     if math.isinf(p) or p >= 10:      # the reference treats p >= 10 as infinity
         return Q_1
-    raise ValueError(f"p={p}: only p in {{1, 2, inf}} has a kernel")
+    if p > 1:
+        # any other norm: the bits of the dual exponent travel in the int argument
+        return struct.unpack("i", struct.pack("f", 1.0 / (1.0 - 1.0 / p)))[0]
+    raise ValueError(f"p={p}: the perturbation norm must be >= 1")
 
 
 def _check(name, t, shape=None):

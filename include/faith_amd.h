@@ -37,6 +37,8 @@ extern "C" {
 #define FAITH_Q_1    1   /* p = inf : sum of magnitudes  */
 #define FAITH_Q_2    2   /* p = 2   : Euclidean norm     */
 #define FAITH_Q_INF  0   /* p = 1   : largest magnitude  */
+/* Any other p (the reference accepts every p, Bounds.py:277): pass the IEEE-754 bits of the dual
+ * exponent q = 1 / (1 - 1/p), 1 < q < inf, in the int (e.g. memcpy from a float). */
 
 #define FAITH_LAYOUT_NATURAL     0
 #define FAITH_LAYOUT_TRANSPOSED  1

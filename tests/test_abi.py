@@ -74,8 +74,12 @@ def test_python_wrappers_refuse_cpu_tensors():
     with pytest.raises(ValueError, match="no CPU path"):
         ops.relu(lw, lb, lw, lb, 2.0, 0.1)
     with pytest.raises(ValueError):
-        ops.q_code(3.0)
+        ops.q_code(0.5)
     assert ops.q_code(float("inf")) == ops.Q_1 and ops.q_code(1) == ops.Q_INF and ops.q_code(2) == ops.Q_2
+    assert ops.q_code(12) == ops.Q_1                       # the reference treats p >= 10 as infinity
+    # any other norm: the int carries the bits of the dual exponent (p = 3 -> q = 1.5)
+    import struct
+    assert struct.unpack("f", struct.pack("i", ops.q_code(3.0)))[0] == 1.5
 
 
 def test_workloads_are_reproducible():

@@ -8,7 +8,7 @@ from tests.parity import compare_activation
 
 pytestmark = pytest.mark.gpu
 INF = float("inf")
-PS = [1.0, 2.0, INF]
+PS = [1.0, 2.0, INF, 3.0, 1.5]     # 3.0 and 1.5: dual exponents 1.5 and 3, the general-norm kernels
 
 
 def dev(*ts):
@@ -163,7 +163,7 @@ def test_bad_arguments_are_rejected_not_launched():
         ops.relu(lw, lb, lw, lb, 2.0, 0.1, words=3)          # 3 does not divide 8
     assert e.value.code == -2
     with pytest.raises(ValueError):
-        ops.relu(lw, lb, lw, lb, 3.0, 0.1)                   # no kernel for q = 1.5
+        ops.relu(lw, lb, lw, lb, 0.5, 0.1)                   # not a norm
     with pytest.raises(ValueError):
         ops.relu(lw.cpu(), lb, lw, lb, 2.0, 0.1)             # CPU tensor: no fallback
     with pytest.raises(TypeError):

@@ -67,7 +67,7 @@ def check(x, y, p, eps, words, what=""):
     (1, 6, 4, 5, 10),           # d % 4 != 0: any-shape kernel
     (2, 3, 5, 1, 8),            # dim_in == 1: interval shortcut
 ])
-@pytest.mark.parametrize("p", [1.0, 2.0, INF])
+@pytest.mark.parametrize("p", [1.0, 2.0, INF, 3.0])
 def test_dot_shapes(shape, p):
     B, Lx, Ly, D, d = shape
     g = torch.Generator().manual_seed(31)
@@ -177,7 +177,7 @@ def check_v(probs, value, p, eps, words, what=""):
     (1, 5, 3, 8),          # key length % 4 != 0: any-shape kernel
     (2, 4, 1, 8),          # dim_in == 1: interval shortcut
 ])
-@pytest.mark.parametrize("p", [1.0, 2.0, INF])
+@pytest.mark.parametrize("p", [1.0, 2.0, INF, 3.0])
 def test_context_shapes(shape, p):
     B, L, D, dv = shape
     g = torch.Generator().manual_seed(33)

@@ -8,7 +8,7 @@ from tests.parity import compare_unary
 
 pytestmark = pytest.mark.gpu
 INF = float("inf")
-PS = [1.0, 2.0, INF]
+PS = [1.0, 2.0, INF, 3.0, 1.5]     # 3.0 and 1.5: dual exponents 1.5 and 3, the general-norm kernels
 KINDS = ["exp", "reciprocal", "sqr", "sqrt"]
 
 

@@ -16,7 +16,7 @@ from oracle import closed_form as C
 from tests.helpers import rand_bounds, f64
 
 INF = float("inf")
-PS = [1.0, 2.0, INF]
+PS = [1.0, 2.0, INF, 3.0, 1.5]     # 3.0 and 1.5: general dual exponents (1.5 and 3)
 
 
 def gen(seed):
