@@ -206,7 +206,8 @@ class Bounds:
     # ---- Bounds.py:833-841.  Scores path: self = query, other = key.  Context path: other is the
     # transposed value object (the reference tells the two apart by the shape of self.lb; here the
     # transposed object says so itself).
-    def dot_product(self, other):
+    def dot_product(self, other, debug=False, verbose=False, lower=True, upper=True):
+        # (the reference's extra arguments are accepted; both halves are always computed)
         src = getattr(other, "_transpose_of", None)
         if src is not None:
             return self._like(*ops.dot_product_v(self._c(), src._c(), self.p, self.eps, self.perturbed_words))
@@ -225,6 +226,15 @@ class Bounds:
     # [heads, Lx, D, Lk], value [1, Lk, D, heads * size] -> [1, Lx, D, heads * size]
     def attention_context(self, value):
         return self._like(*ops.attention_context(self._c(), value._c(), self.p, self.eps, self.perturbed_words))
+
+
+# The reference keeps three spellings of its hot methods -- the dispatcher (relu), the PyTorch body
+# (ori_relu) and the CUDA adapter (cuda_relu), chosen by a module-level FLAG (Bounds.py:1163-1175,
+# :833-841, :397-401).  Here there is one implementation, so the other spellings are the same method.
+for _name, _target in (("ori_relu", "relu"), ("cuda_relu", "relu"), ("ori_tanh", "tanh"), ("cuda_tanh", "tanh"),
+                       ("ori_matmul", "matmul"), ("ori_dot_product", "dot_product"),
+                       ("cuda_dot_product_QK", "dot_product"), ("cuda_dot_product_V", "dot_product")):
+    setattr(Bounds, _name, getattr(Bounds, _target))
 
 
 class ConvBounds:
