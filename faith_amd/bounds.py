@@ -32,10 +32,15 @@ class Bounds:
         self.p = p
         self.eps = eps
         self.perturbed_words = getattr(self.args, "perturbed_words", 1)
+        # interval bound propagation (args.method == "ibp", Bounds.py:274): zero coefficients, every
+        # relaxation maps the concrete interval to the interval of its image
+        self.ibp = getattr(self.args, "method", None) == "ibp"
         self.lw = lw if lw is not None else (w.clone() if clone else w)
         self.uw = uw if uw is not None else (w.clone() if clone else w)
         self.lb = lb if lb is not None else (b.clone() if clone else b)
         self.ub = ub if ub is not None else (b.clone() if clone else b)
+        if self.ibp:                                        # Bounds.py:285-288
+            self.lw, self.uw = self.lw[:, :, :self.perturbed_words, :], self.uw[:, :, :self.perturbed_words, :]
         self.device = self.lw.device
         self.update_shape()
 
@@ -47,6 +52,17 @@ class Bounds:
 
     def _c(self):
         return (self.lw.contiguous(), self.lb.contiguous(), self.uw.contiguous(), self.ub.contiguous())
+
+    def _interval(self, kind):
+        """method "ibp": the operator applied to the concrete interval; coefficients are zero
+        (the `if self.ibp` branches of Bounds.py:863-866, :896-898, :924-926, :973-975, :1030-1032, :1139-1143)."""
+        l, u = self.concretize()
+        if kind == "sqrt":
+            self._require(l, 0.0, True, "sqrt of a bound that reaches zero")
+        if kind == "reciprocal":
+            self._require(l, 1e-12, False, "reciprocal of a bound that reaches zero")
+        lb, ub = ops.interval_unary(kind, l, u)
+        return self._like(torch.zeros_like(self.lw), lb, torch.zeros_like(self.uw), ub)
 
     # ---- Bounds.py:319-326
     def concretize(self):
@@ -87,6 +103,10 @@ class Bounds:
     # ---- Bounds.py:594-664: by a float, by a per-neuron tensor, or by another bound object
     def multiply(self, W):
         if isinstance(W, Bounds):
+            if self.ibp:                                    # Bounds.py:667-676: the interval of the product
+                (xl, xu), (yl, yu) = self.concretize(), W.concretize()
+                lb, ub = ops.interval_product(xl, xu, yl, yu)
+                return self._like(torch.zeros_like(self.lw), lb, torch.zeros_like(self.uw), ub)
             return self._like(*ops.multiply(self._c(), W._c(), self.p, self.eps, self.perturbed_words))
         return self._like(*ops.scale(*self._c(), W))
 
@@ -133,26 +153,38 @@ class Bounds:
 
     # ---- Bounds.py:1163-1175
     def relu(self):
+        if self.ibp:
+            return self._interval("relu")
         return self._like(*ops.relu(*self._c(), self.p, self.eps, self.perturbed_words))
 
     def tanh(self):
+        if self.ibp:
+            return self._interval("tanh")
         return self._like(*ops.tanh(*self._c(), self.p, self.eps, self.perturbed_words))
 
     # ---- Bounds.py:970-1003, :860-890
     def exp(self):
+        if self.ibp:
+            return self._interval("exp")
         return self._like(*ops.exp(*self._c(), self.p, self.eps, self.perturbed_words))
 
     def sqr(self):
+        if self.ibp:
+            return self._interval("sqr")
         return self._like(*ops.sqr(*self._c(), self.p, self.eps, self.perturbed_words))
 
     # ---- Bounds.py:892-919, :1136-1161.  Both assert a positive interval in the reference; the
     # check reads the concrete lower bound back from the kernel (one synchronisation).
     def sqrt(self):
+        if self.ibp:
+            return self._interval("sqrt")
         out = ops.sqrt(*self._c(), self.p, self.eps, self.perturbed_words, return_interval=True)
         self._require(out[4], 0.0, True, "sqrt of a bound that reaches zero")
         return self._like(*out[:4])
 
     def reciprocal(self):
+        if self.ibp:
+            return self._interval("reciprocal")
         out = ops.reciprocal(*self._c(), self.p, self.eps, self.perturbed_words, return_interval=True)
         self._require(out[4], 1e-12, False, "reciprocal of a bound that reaches zero")
         return self._like(*out[:4])
@@ -209,6 +241,13 @@ class Bounds:
     def dot_product(self, other, debug=False, verbose=False, lower=True, upper=True):
         # (the reference's extra arguments are accepted; both halves are always computed)
         src = getattr(other, "_transpose_of", None)
+        if self.ibp and self.dim_in > 1:
+            # interval arithmetic on the constant terms (get_bounds_xy's ibp branch makes every
+            # coefficient zero, Bounds.py:667-676): the dim_in == 1 kernel on one row of the zero
+            # coefficients, its zero result repeated dim_in times
+            if src is not None:
+                return self._ibp_rows(lambda x, v: x.dot_product(v.t()), src)
+            return self._ibp_rows(lambda x, y: x.dot_product(y), other)
         if src is not None:
             return self._like(*ops.dot_product_v(self._c(), src._c(), self.p, self.eps, self.perturbed_words))
         return self._like(*ops.dot_product_qk(self._c(), other._c(), self.p, self.eps, self.perturbed_words))
@@ -220,11 +259,23 @@ class Bounds:
     # ---- VerifierForward.py:208-229 + Bounds.py:833-841: scores of all heads, self = query and key
     # both [1, L, D, heads * size]; the kernels address each head in place
     def attention_scores(self, key, heads):
+        if self.ibp and self.dim_in > 1:
+            return self._ibp_rows(lambda q, k: q.attention_scores(k, heads), key)
         return self._like(*ops.attention_scores(self._c(), key._c(), heads, self.p, self.eps, self.perturbed_words))
+
+    def _ibp_rows(self, op, other):
+        """method "ibp" with dim_in > 1: the interval kernels run on one row of the (zero) coefficients
+        and the zero result is repeated dim_in times."""
+        one = lambda b: b._like(b.lw[:, :, :1], b.lb, b.uw[:, :, :1], b.ub)
+        z = op(one(self), one(other))
+        zero = z.lw.expand(-1, -1, self.dim_in, -1).contiguous()
+        return self._like(zero, z.lb, zero.clone(), z.ub)
 
     # ---- VerifierForward.py:208-229 + Bounds.py:843-850 + VerifierForward.py:253-263: self = probabilities
     # [heads, Lx, D, Lk], value [1, Lk, D, heads * size] -> [1, Lx, D, heads * size]
     def attention_context(self, value):
+        if self.ibp and self.dim_in > 1:
+            return self._ibp_rows(lambda pr, v: pr.attention_context(v), value)
         return self._like(*ops.attention_context(self._c(), value._c(), self.p, self.eps, self.perturbed_words))
 
 

@@ -193,6 +193,47 @@ __global__ void __launch_bounds__(256) row_kernel(const Pair w, const Pair b, co
     }
 }
 
+// ------------------------------------------------------------------ interval arithmetic (method "ibp")
+// With interval bound propagation the coefficients are zero and an operator maps the concrete
+// interval [l, u] of every neuron to the interval of its image (the `if self.ibp` branches of
+// Bounds.py:863-866, :896-898, :924-926, :973-975, :1030-1032, :1139-1143).
+__global__ void __launch_bounds__(256) interval_unary_kernel(const int op, const float *__restrict__ l,
+                                                             const float *__restrict__ u, float *__restrict__ out_l,
+                                                             float *__restrict__ out_u, const size_t n) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+        const float a = l[e], b = u[e];
+        float lo, hi;
+        switch (op) {
+            case FAITH_OP_RELU: lo = fmaxf(a, 0.f); hi = fmaxf(b, 0.f); break;
+            case FAITH_OP_TANH: lo = tanhf(a); hi = tanhf(b); break;
+            case FAITH_OP_EXP: lo = expf(a); hi = expf(b); break;
+            case FAITH_OP_RECIPROCAL: lo = 1.f / b; hi = 1.f / a; break;
+            case FAITH_OP_SQRT: lo = sqrtf(a); hi = sqrtf(b); break;
+            default: {   // FAITH_OP_SQR: zero lower bound when the interval straddles zero (l <= 0 <= u)
+                const float aa = a * a, bb = b * b;
+                lo = (a > 0.f || b < 0.f) ? fminf(aa, bb) : 0.f;
+                hi = fmaxf(aa, bb);
+            }
+        }
+        out_l[e] = lo;
+        out_u[e] = hi;
+    }
+}
+
+// interval of a product: the extreme of the four corner products (Bounds.py:667-676)
+__global__ void __launch_bounds__(256) interval_product_kernel(const float *__restrict__ xl, const float *__restrict__ xu,
+                                                               const float *__restrict__ yl, const float *__restrict__ yu,
+                                                               float *__restrict__ zl, float *__restrict__ zu,
+                                                               const size_t n) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+        const float p1 = xl[e] * yl[e], p2 = xl[e] * yu[e], p3 = xu[e] * yl[e], p4 = xu[e] * yu[e];
+        zl[e] = fminf(fminf(p1, p2), fminf(p3, p4));
+        zu[e] = fmaxf(fmaxf(p1, p2), fmaxf(p3, p4));
+    }
+}
+
 bool all_aligned16(std::initializer_list<const void *> ptrs) {
     for (const void *p : ptrs)
         if (p != nullptr && !faith::aligned(p, 16)) return false;
@@ -264,4 +305,26 @@ extern "C" int faith_layer_norm_verification(const float *src_lb, const float *s
     FAITH_OBJECT_NOT_NULL();
     const Pair w{src_lw, src_uw, nullptr, nullptr, out_lw, out_uw}, b{src_lb, src_ub, nullptr, nullptr, out_lb, out_ub};
     return launch_rows<MODE_NORM>("faith_layer_norm_verification", w, b, weight, bias, rows_w, rows_b, dim_out, stream);
+}
+
+extern "C" int faith_interval_unary(int op, const float *l, const float *u, float *out_lb, float *out_ub, long long n,
+                                    void *stream) {
+    FAITH_NOT_NULL(l); FAITH_NOT_NULL(u); FAITH_NOT_NULL(out_lb); FAITH_NOT_NULL(out_ub);
+    FAITH_REQUIRE(op >= FAITH_OP_RELU && op <= FAITH_OP_SQRT, FAITH_ERR_UNSUPPORTED, "faith_interval_unary: unknown op %d", op);
+    FAITH_REQUIRE(n > 0, FAITH_ERR_SHAPE, "faith_interval_unary: n=%lld must be positive", n);
+    const long long blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(interval_unary_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), op, l, u, out_lb, out_ub, (size_t)n);
+    return faith::check_launch("faith_interval_unary");
+}
+
+extern "C" int faith_interval_product(const float *x_l, const float *x_u, const float *y_l, const float *y_u,
+                                      float *z_lb, float *z_ub, long long n, void *stream) {
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub);
+    FAITH_REQUIRE(n > 0, FAITH_ERR_SHAPE, "faith_interval_product: n=%lld must be positive", n);
+    const long long blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(interval_product_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), x_l, x_u, y_l, y_u, z_lb, z_ub, (size_t)n);
+    return faith::check_launch("faith_interval_product");
 }

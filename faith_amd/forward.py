@@ -32,19 +32,25 @@ import math
 import torch
 
 
-def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, norm=None, layer_norm="no_var"):
-    """VerifierForward._bound_input: identity coefficients at the perturbed position(s).
+def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, norm=None, layer_norm="no_var",
+                ibp=False):
+    """VerifierForward._bound_input (:127-156): identity coefficients at the perturbed position(s); with
+    ibp (interval bound propagation) zero coefficients and the constant terms widened by eps there.
 
     embeddings [1, L, dim]; index: position (int) or list of positions; make_bounds(p, eps, lw, lb,
     uw, ub) builds the bound object.  Returns bounds of the (layer-normed) embeddings."""
     length, dim = embeddings.shape[1], embeddings.shape[2]
     w = torch.zeros((length, dim * perturbed_words, dim), device=embeddings.device)
     positions = [index] if perturbed_words == 1 else list(index)
+    lb, ub = embeddings[0].unsqueeze(0).clone(), embeddings[0].unsqueeze(0).clone()
     for i, pos in enumerate(positions):
-        w[pos, dim * i:dim * (i + 1), :] = torch.eye(dim, device=embeddings.device)
+        if ibp:
+            lb[0, pos] -= eps
+            ub[0, pos] += eps
+        else:
+            w[pos, dim * i:dim * (i + 1), :] = torch.eye(dim, device=embeddings.device)
     lw = w.unsqueeze(0)
-    b = embeddings[0].unsqueeze(0)
-    bounds = make_bounds(p, eps, lw, b.clone(), lw.clone(), b.clone())
+    bounds = make_bounds(p, eps, lw, lb, lw.clone(), ub)
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
     return bounds

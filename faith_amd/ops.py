@@ -287,6 +287,28 @@ def layer_norm(lw, lb, uw, ub, weight=None, bias=None):
     return olw, olb, ouw, oub
 
 
+def interval_unary(kind, l, u):
+    """Interval bound propagation through relu / tanh / exp / reciprocal / sqr / sqrt: the interval of the
+    image of [l, u], elementwise.  Returns (lb, ub)."""
+    if kind not in _UNARY:
+        raise ValueError(f"unknown operator {kind!r}")
+    _check("l", l); _check("u", u, l.shape)
+    olb, oub = torch.empty_like(l), torch.empty_like(u)
+    with _on(l.device):
+        _lib.call("faith_interval_unary", _UNARY[kind], _ptr(l), _ptr(u), _ptr(olb), _ptr(oub), l.numel(), _stream(l))
+    return olb, oub
+
+
+def interval_product(xl, xu, yl, yu):
+    """Interval of the elementwise product of [xl, xu] and [yl, yu].  Returns (lb, ub)."""
+    _check("xl", xl); _check("xu", xu, xl.shape); _check("yl", yl, xl.shape); _check("yu", yu, xl.shape)
+    zl, zu = torch.empty_like(xl), torch.empty_like(xl)
+    with _on(xl.device):
+        _lib.call("faith_interval_product", _ptr(xl), _ptr(xu), _ptr(yl), _ptr(yu), _ptr(zl), _ptr(zu), xl.numel(),
+                  _stream(xl))
+    return zl, zu
+
+
 def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     """Sign-split propagation through y = x @ weight.T + bias.  weight: [H_out, H]."""
     B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)

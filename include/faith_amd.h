@@ -246,6 +246,19 @@ int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *
                                      int q, int words, void *stream);
 
 /*
+ * Interval bound propagation (the reference's method "ibp": the `if self.ibp` branches of
+ * Bounds.py:863-866, :896-898, :924-926, :973-975, :1030-1032, :1139-1143 and :667-676).  The
+ * coefficients are zero there, so an operator maps the concrete interval [l, u] of every neuron
+ * (from faith_concretize) to the interval of its image; n elements.
+ *   unary:   op = FAITH_OP_RELU / TANH / EXP / RECIPROCAL / SQR / SQRT
+ *   product: the extreme of the four corner products of [x_l, x_u] and [y_l, y_u]
+ */
+int faith_interval_unary(int op, const float *l, const float *u, float *out_lb, float *out_ub,
+                         long long n, void *stream);
+int faith_interval_product(const float *x_l, const float *x_u, const float *y_l, const float *y_u,
+                           float *z_lb, float *z_ub, long long n, void *stream);
+
+/*
  * Attention scores with the heads taken where the dense layers leave them.  Replaces
  * transpose_for_scores on query and key (VerifierForward.py:208-229: four permuted copies per
  * object) followed by Bounds.dot_product (Bounds.py:833-841): the kernels address head h of

@@ -486,3 +486,35 @@ def concretize_conv(x: LinearBounds, p: float, eps: float):
     lo = x.lb - eps * torch.norm(x.lw, p=q, dim=1)
     hi = x.ub + eps * torch.norm(x.uw, p=q, dim=1)
     return lo, hi
+
+
+# --------------------------------------------------------------------------
+# interval bound propagation  (method "ibp": the `if self.ibp` branches)
+# --------------------------------------------------------------------------
+def interval_unary(kind: str, l: torch.Tensor, u: torch.Tensor):
+    """Image of the concrete interval [l, u] under a monotone operator, and sqr
+    (Bounds.py:924-926 relu, :1030-1032 tanh, :973-975 exp, :1139-1143 reciprocal,
+    :896-898 sqrt, :863-866 sqr).  Coefficients are zero in this mode."""
+    if kind == "relu":
+        zero = torch.tensor(0.0)
+        return torch.max(l, zero), torch.max(u, zero)
+    if kind == "tanh":
+        return torch.tanh(l), torch.tanh(u)
+    if kind == "exp":
+        return torch.exp(l), torch.exp(u)
+    if kind == "reciprocal":
+        return 1.0 / u, 1.0 / l
+    if kind == "sqrt":
+        return torch.sqrt(l), torch.sqrt(u)
+    if kind == "sqr":
+        both = 1 - torch.gt(l, 0).to(torch.float32) - torch.lt(u, 0).to(torch.float32)
+        lb = torch.min(l * l, u * u)
+        lb = lb - both * lb                      # the lower bound is zero when the interval holds zero
+        return lb, torch.max(l * l, u * u)
+    raise ValueError(kind)
+
+
+def interval_product(xl, xu, yl, yu):
+    """Interval of x * y from the four corner products (get_bounds_xy, Bounds.py:667-676)."""
+    p1, p2, p3, p4 = xl * yl, xl * yu, xu * yl, xu * yu
+    return (torch.min(p1, torch.min(p2, torch.min(p3, p4))), torch.max(p1, torch.max(p2, torch.max(p3, p4))))
