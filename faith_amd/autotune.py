@@ -17,7 +17,7 @@ What can be tuned (see the FAITH_TUNE_* knobs in include/faith_amd.h):
     concretize   tile shape of the concretize kernel
 
 Results are kept in a TuningTable keyed by (operator, shape); `use(table)` makes the wrappers in
-faith_amd.ops apply an entry around the matching call.  Results never depend on the variant, only
+faith_amd.ops apply an entry around the matching launch.  Results never depend on the variant, only
 speed does.
 """
 from __future__ import annotations
@@ -342,13 +342,3 @@ def use(table):
     """Makes faith_amd.ops apply `table` (None: stop)."""
     global _ACTIVE
     _ACTIVE = table
-
-
-def tuned(op, shape):
-    """Context manager for the wrappers in faith_amd.ops: applies the active table's entry, if any."""
-    if _ACTIVE is None:
-        return contextlib.nullcontext()
-    knobs = _ACTIVE.lookup(op, shape)
-    if not knobs:
-        return contextlib.nullcontext()
-    return applied(knobs)

@@ -37,18 +37,7 @@ __device__ __forceinline__ float nfin(float a, float qv) {
 // Stores are non-temporal: lw' / uw' are written once and not read again by this kernel, and
 // keeping them out of the cache's way measured 11 % faster at configuration 1 (loads are left
 // temporal: marking them non-temporal measured 15 % slower).
-//
-// Addresses are buffer addresses: a wave-uniform descriptor (base pointer, size in bytes), a
-// wave-uniform 32-bit offset (the row) and one per-thread 32-bit offset (the column), so that a
-// thread holds ONE address register for all the rows it loads and stores, not a 64-bit pointer per
-// row.  Accesses at or beyond the size are dropped by the hardware (loads return zero).
 typedef float v4f __attribute__((ext_vector_type(4)));
-typedef unsigned v4u __attribute__((ext_vector_type(4)));
-typedef __amdgpu_buffer_rsrc_t Window;
-__device__ __forceinline__ Window window(const void *base, size_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0,
-                                             (int)((bytes >> 32) ? 0xffffffffu : (unsigned)bytes), 0x00020000);
-}
 template <int VEC>
 struct Vec;
 template <>
@@ -58,14 +47,6 @@ struct Vec<4> {
     __device__ __forceinline__ void store(float *p) const {
         const v4f t = {v.x, v.y, v.z, v.w};
         __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
-    }
-    __device__ __forceinline__ void load(Window w, unsigned thread_off, unsigned uniform_off) {
-        const v4u t = __builtin_amdgcn_raw_buffer_load_b128(w, thread_off, uniform_off, 0);
-        v = make_float4(__uint_as_float(t.x), __uint_as_float(t.y), __uint_as_float(t.z), __uint_as_float(t.w));
-    }
-    __device__ __forceinline__ void store(Window w, unsigned thread_off, unsigned uniform_off) const {
-        const v4u t = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
-        __builtin_amdgcn_raw_buffer_store_b128(t, w, thread_off, uniform_off, 2 /* non-temporal */);
     }
     __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
     __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
@@ -81,12 +62,6 @@ struct Vec<1> {
     float v;
     __device__ __forceinline__ void load(const float *p) { v = *p; }
     __device__ __forceinline__ void store(float *p) const { __builtin_nontemporal_store(v, p); }
-    __device__ __forceinline__ void load(Window w, unsigned thread_off, unsigned uniform_off) {
-        v = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(w, thread_off, uniform_off, 0));
-    }
-    __device__ __forceinline__ void store(Window w, unsigned thread_off, unsigned uniform_off) const {
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), w, thread_off, uniform_off, 2 /* non-temporal */);
-    }
     __device__ __forceinline__ void zero() { v = 0.f; }
     __device__ __forceinline__ float get(int) const { return v; }
     __device__ __forceinline__ void set(int, float f) { v = f; }

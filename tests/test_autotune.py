@@ -96,10 +96,9 @@ def test_table_round_trip(tmp_path):
     back = A.TuningTable.load(path)
     assert back.lookup("linear", (8192, 256, 256)) == best.knob_dict()
     assert back.lookup("linear", (8192, 256, 512)) is None
-    # no table in use: the wrappers' hook is a no-op
+    A.use(back)
+    assert A._ACTIVE is back
     A.use(None)
-    with A.tuned("linear", (8192, 256, 256)):
-        pass
 
 
 # ------------------------------------------------------------------ GPU
