@@ -721,9 +721,12 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
                       (MODE == CONCRETIZE || (faith::aligned(a.olw, 16) && faith::aligned(a.ouw, 16)));
     if (MODE == CONCRETIZE) {
         // nothing is kept, so what counts is bytes in flight: 64-neuron tiles, 16 wavefronts, 256 rows
-        // per pass measured best or equal on every shape tried (wide and narrow H alike)
+        // per pass measured best or equal on every shape tried (wide and narrow H alike) -- except
+        // where a row of neurons is 64 KB or more (image-shaped bounds: every row of a tile then lies
+        // on another page), where four-wavefront workgroups are 12 % ahead (6.2 against 5.4 TB/s at
+        // configuration 4)
         const int pick = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
-        if (vec4 && pick == 11)
+        if (vec4 && (pick == 11 || (pick == 0 && (long long)a.H * 4 >= 65536)))
             launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);
         else if (vec4 && pick == 13)
             launch_natural<MODE, Q, 4, 8, 256, 8>(a, st);

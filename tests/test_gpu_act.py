@@ -168,3 +168,17 @@ def test_bad_arguments_are_rejected_not_launched():
         ops.relu(lw.cpu(), lb, lw, lb, 2.0, 0.1)             # CPU tensor: no fallback
     with pytest.raises(TypeError):
         ops.relu(lw.double(), lb, lw, lb, 2.0, 0.1)
+
+
+@pytest.mark.parametrize("p", [2.0, INF])
+def test_concretize_of_very_long_rows(p):
+    """Rows of 64 KB and more (image-shaped bounds flattened to [1, D_in, C*H*W]) take four-wavefront
+    workgroups; D_in beyond one pass of rows, a ragged last tile, two perturbed words."""
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(7)
+    for (D, H, words) in [(12, 16384, 1), (300, 16420, 2), (64, 32768 + 8, 1)]:
+        x = rand_bounds(g, 1, 1, D, H, ordered=False)
+        lw, lb, uw, ub = dev(*x.tensors())
+        l, u = ops.concretize(lw, lb, uw, ub, p, 0.3, words)
+        el, eu = O.concretize(x, p, 0.3, words)
+        assert close(l, el) and close(u, eu), (D, H, words)
