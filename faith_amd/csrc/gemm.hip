@@ -397,17 +397,19 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
                       faith::aligned(W, 16) && 128LL * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
-        // macro-tile (measured on 8192 ... 131072 rows, K and N 256 ... 1024): tiny problems want the most
-        // workgroups (64 x 64); up to two 128 x 64 tiles per CU that shape is 6 - 17 % ahead of 64 x 64;
-        // beyond, 64 x 64 until there are four 128 x 128 tiles per CU (their pro- and epilogues overlap
-        // better at five workgroups per CU than at two), then 128 x 128.  The tuning knob forces a shape.
+        // macro-tile, from tuner runs on 1024 ... 245760 rows, K and N 64 ... 1024 (the built-in choice is
+        // within 3 % of the best of the four there): tiny problems want the most workgroups (64 x 64); up
+        // to two 128 x 64 tiles per CU that shape is up to 17 % ahead; 128 x 128 pays only for long
+        // reductions on problems of many tiles per CU (configuration 2: 1 % ahead) -- with K <= 512 the
+        // pro- and epilogues of five small co-resident workgroups overlap better than those of two large
+        // ones (2 - 6 % at 65536 ... 245760 rows).  The tuning knob forces a shape.
         auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * ((dim_y_out + n - 1) / n); };
         const long long cus = faith::compute_units();
         int tm, tn;
         if (tiles(64, 64) <= cus) { tm = 64; tn = 64; }
         else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
-        else if (tiles(128, 128) < 4 * cus) { tm = 64; tn = 64; }
-        else { tm = 128; tn = 128; }
+        else if (dim_out >= 1024 && tiles(128, 128) >= 16 * cus) { tm = 128; tn = 128; }
+        else { tm = 64; tn = 64; }
         switch (faith::tune_get(FAITH_TUNE_GEMM_VARIANT)) {
             case 1: tm = 64;  tn = 64;  break;
             case 2: tm = 128; tn = 128; break;
