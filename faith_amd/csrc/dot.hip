@@ -810,22 +810,26 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
                       faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
                       (long long)TI * D * max_pitch * 4 < 0xffffffffLL &&            // 32-bit offsets inside a tile
                       (!VP || (long long)d * D * g.oy.pitch * 4 < 0xffffffffLL);           // and along K inside a head
-    // short sequences take the per-wavefront kernel; the tuning knob can force either kernel
+    // The per-wavefront kernel runs at about 0.85 of the tiled kernel's rate on the same padded work, so it
+    // takes the problems whose 32 x 32 blocks cover at most 0.85 of what 128 x 64 tiles would (sequence
+    // lengths up to 64, and e.g. 80 ... 112: 119 against 164 us at 4 heads, L = 80).  The tuning knob can
+    // force either kernel.
     const bool small_ok = fast && d % 8 == 0 && d <= 80;
     const int pick = faith::tune_get(FAITH_TUNE_DOT_VARIANT);
-    const bool small = small_ok && (pick == 2 || (pick != 1 && Lx <= 64 && Ly <= 64));
+    const long long pad_small = (long long)((Lx + SB - 1) / SB) * ((Ly + SB - 1) / SB) * SB * SB;
+    const long long pad_tiled = (long long)((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ) * TI * TJ;
+    const bool small = small_ok && (pick == 2 || (pick != 1 && 100 * pad_small <= 85 * pad_tiled));
     if (small) {
-        // short sequences: one 32 x 32 block per wavefront and perturbation coordinate.  Coordinates
-        // per wavefront: the count that needs the fewest rounds of resident workgroups (three per CU
-        // by registers, fewer when the shared operands are large), a round costing its coordinates
-        // plus about half a coordinate for staging the shared operands
+        // one 32 x 32 block per wavefront and perturbation coordinate.  Coordinates per wavefront: the
+        // count that leaves the busiest CU the least to do -- its share of the workgroups, each costing
+        // its coordinates plus about half a coordinate for staging the shared operands (tuner sweeps:
+        // this choice is within 5 % of the best count on every shape tried)
         const long long blocks = (long long)B * ((Lx + SB - 1) / SB) * ((Ly + SB - 1) / SB);
-        const long long lds_fit = (160 * 1024) / ((long long)6 * SB * d * sizeof(float));
-        const long long resident = faith::compute_units() * (lds_fit < 3 ? lds_fit : 3);
+        const long long cus = faith::compute_units();
         long long mpw = 1, best = -1;
         for (long long c = 1; c <= 16; ++c) {
             const long long wgs = blocks * ((D + 4 * c - 1) / (4 * c));
-            const long long cost = ((wgs + resident - 1) / resident) * (2 * c + 1);
+            const long long cost = ((wgs + cus - 1) / cus) * (2 * c + 1);
             if (best < 0 || cost < best) { best = cost; mpw = c; }
         }
         const int forced = faith::tune_get(FAITH_TUNE_DOT_COORDS);
