@@ -124,7 +124,7 @@ class Heuristics:
         if op == "act":
             rows, d_in, h = shape
             table = {0: (32, 32, 256), 9: (32, 256, 256), 1: (32, 256, 256), 2: (64, 256, 512), 3: (64, 256, 1024),
-                     4: (32, 256, 512), 5: (64, 256, 256)}   # neurons per tile, rows per pass, threads
+                     4: (32, 256, 512), 5: (64, 256, 256), 6: (32, 1024, 1024)}   # neurons per tile, rows per pass, threads
             out = []
             for variant, (neurons, chunk, threads) in table.items():
                 held = min(d_in, chunk) * neurons * 2 // threads       # values a thread keeps between its two passes

@@ -753,6 +753,7 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         case 3: launch_natural<MODE, Q, 4, 16, 1024, 4>(a, st); return;   // 64 neurons, 256 rows / chunk, 16 waves
         case 4: launch_natural<MODE, Q, 4, 8, 512, 4>(a, st); return;     // 32 neurons, 256 rows / chunk, 8 waves
         case 5: launch_natural<MODE, Q, 4, 16, 256, 16>(a, st); return;   // 64 neurons, 256 rows / chunk, 4 waves
+        case 6: launch_natural<MODE, Q, 4, 8, 1024, 8>(a, st); return;    // 32 neurons, 1024 rows / chunk, 16 waves
         default: break;
     }
     // 32-neuron tiles (128-byte row segments) keep the register footprint at 64 values per
@@ -761,8 +762,12 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         launch_natural<MODE, Q, 4, 8, 256, 4>(a, st);     // D_in <= 128 in registers
     } else if (a.D <= 256) {
         launch_natural<MODE, Q, 4, 8, 256, 8>(a, st);     // D_in <= 256 in registers
-    } else {
+    } else if (a.D <= 512 || a.D > 1024) {
         launch_natural<MODE, Q, 4, 8, 512, 8>(a, st);     // D_in <= 512 in registers, chunks beyond
+    } else {
+        // D_in <= 1024 in the registers of sixteen wavefronts: one read instead of two (8 - 13 % ahead
+        // of the chunked walk at D_in = 640 ... 1024)
+        launch_natural<MODE, Q, 4, 8, 1024, 8>(a, st);
     }
 }
 

@@ -64,7 +64,8 @@ def test_activation_small_shapes(kind, p, layout):
     g = torch.Generator().manual_seed(6)
     # register-resident, chunked (D_in > 512), ragged H (scalar path), tiny
     for (L, D, H, words) in [(4, 64, 64, 1), (3, 128, 192, 2), (2, 256, 64, 2), (2, 512, 64, 1),
-                             (1, 1100, 72, 1), (2, 48, 37, 3), (1, 2, 5, 1), (3, 256, 37, 4), (1, 512, 9, 2)]:
+                             (1, 1100, 72, 1), (2, 48, 37, 3), (1, 2, 5, 1), (3, 256, 37, 4), (1, 512, 9, 2),
+                             (2, 768, 64, 2), (1, 1024, 36, 1), (1, 516, 40, 3)]:   # 512 < D_in <= 1024: sixteen-wavefront tiles
         x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
         check(kind, x, p, 0.05, words, layout)
 
