@@ -33,10 +33,10 @@ struct ActArgs {
     float *l, *u;
     int rows, D, H, words;
     float eps;
-    // optional second bound object of the same D, H (concretize only): one launch covers both
+    // optional second bound object of the same D (concretize only): one launch covers both
     const float *lb2 = nullptr, *ub2 = nullptr, *lw2 = nullptr, *uw2 = nullptr;
     float *l2 = nullptr, *u2 = nullptr;
-    int rows2 = 0;
+    int rows2 = 0, H2 = 0;
     float qv = 0.f;     // the dual exponent when it is none of 1, 2, inf
 };
 
@@ -273,9 +273,12 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     float *s_lu = part + a.words * NW * 2 * TH;   // [2][TH] concrete interval
     float *s_ln = s_lu + 2 * TH;              // [2][3][TH] lower / upper line (k, x0, y0)
 
-    const int tiles = (a.H + TH - 1) / TH;
-    const bool second = MODE == CONCRETIZE && (int)blockIdx.x >= a.rows * tiles;
-    const int bid = second ? blockIdx.x - a.rows * tiles : blockIdx.x;
+    // concretize only: a second bound object of the same dim_in (its own dim_out) in the same launch
+    const int tiles1 = (a.H + TH - 1) / TH;
+    const bool second = MODE == CONCRETIZE && (int)blockIdx.x >= a.rows * tiles1;
+    const int H = second ? a.H2 : a.H;
+    const int tiles = (H + TH - 1) / TH;
+    const int bid = second ? blockIdx.x - a.rows * tiles1 : blockIdx.x;
     const float *__restrict__ p_lw = second ? a.lw2 : a.lw, *__restrict__ p_uw = second ? a.uw2 : a.uw;
     const float *__restrict__ p_lb = second ? a.lb2 : a.lb, *__restrict__ p_ub = second ? a.ub2 : a.ub;
     float *__restrict__ p_l = second ? a.l2 : a.l, *__restrict__ p_u = second ? a.u2 : a.u;
@@ -285,8 +288,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     const int lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid % TPR, rg = tid / TPR;
     const int col = col0 + c * VEC;
-    const bool col_ok = col < a.H;
-    const size_t base = (size_t)r * a.D * a.H + col;
+    const bool col_ok = col < H;
+    const size_t base = (size_t)r * a.D * H + col;
     const int blk = a.D / a.words;
     constexpr int CHUNK = RG * RPT;
     const int nchunks = (a.D + CHUNK - 1) / CHUNK;
@@ -307,8 +310,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
         for (int i = 0; i < RPT; ++i) {
             const int row = ch * CHUNK + i * RG + rg;
             if (col_ok && row < a.D) {
-                dl[i].load(p_lw + base + (size_t)row * a.H);
-                du[i].load(p_uw + base + (size_t)row * a.H);
+                dl[i].load(p_lw + base + (size_t)row * H);
+                du[i].load(p_uw + base + (size_t)row * H);
             } else {
                 dl[i].zero();
                 du[i].zero();
@@ -358,8 +361,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     __syncthreads();
 
     const int column = col0 + lane;
-    const bool n_ok = lane < TH && column < a.H;
-    const size_t bi = (size_t)r * a.H + column;
+    const bool n_ok = lane < TH && column < H;
+    const size_t bi = (size_t)r * H + column;
     neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, p_lb, p_ub, p_l, p_u, bi, n_ok, lane, wv);
     if (MODE == CONCRETIZE) return;
 
@@ -375,7 +378,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
         for (int i = 0; i < RPT; ++i) {
             const int row = ch * CHUNK + i * RG + rg;
             if (row < a.D) {
-                const size_t off = base + (size_t)row * a.H;
+                const size_t off = base + (size_t)row * H;
                 if (nchunks > 1) {
                     dl[i].load(p_lw + off);
                     du[i].load(p_uw + off);
@@ -591,7 +594,8 @@ void launch_natural(const ActArgs &a, hipStream_t st) {
     constexpr int TH = TPR * VEC;
     const int tiles = (a.H + TH - 1) / TH;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
-    hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)((a.rows + a.rows2) * tiles)),
+    const int tiles2 = (a.H2 + TH - 1) / TH;
+    hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles + a.rows2 * tiles2)),
                        dim3(NTHREADS), smem, st, a);
 }
 
@@ -716,7 +720,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) a
 
 template <int MODE, int Q>
 void dispatch_natural(const ActArgs &a, hipStream_t st) {
-    const bool vec4 = (a.H % 4 == 0) && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
+    const bool vec4 = (a.H % 4 == 0) && (a.H2 % 4 == 0) && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
                       faith::aligned(a.lw2, 16) && faith::aligned(a.uw2, 16) &&
                       (MODE == CONCRETIZE || (faith::aligned(a.olw, 16) && faith::aligned(a.ouw, 16)));
     if (MODE == CONCRETIZE) {
@@ -813,14 +817,14 @@ int run(const char *who, ActArgs a, int q, int layout, void *stream) {
 
 }  // namespace
 
-// Concretizes two bound objects of equal dim_in / dim_out in ONE launch (the dot product needs
-// the intervals of both operands before it can start).  Natural layout.
+// Concretizes two bound objects of equal dim_in in ONE launch (the dot product needs the intervals
+// of both operands before it can start).  Natural layout.
 int faith::concretize_pair(const float *lb, const float *ub, const float *lw, const float *uw, float *l, float *u,
                            int rows, const float *lb2, const float *ub2, const float *lw2, const float *uw2,
-                           float *l2, float *u2, int rows2, int dim_in, int dim_out, float eps, int q, int words,
-                           void *stream) {
+                           float *l2, float *u2, int rows2, int dim_in, int dim_out, int dim_out2, float eps, int q,
+                           int words, void *stream) {
     ActArgs a{lb, ub, lw, uw, nullptr, nullptr, nullptr, nullptr, l, u, rows, dim_in, dim_out, words, eps};
-    a.lb2 = lb2; a.ub2 = ub2; a.lw2 = lw2; a.uw2 = uw2; a.l2 = l2; a.u2 = u2; a.rows2 = rows2;
+    a.lb2 = lb2; a.ub2 = ub2; a.lw2 = lw2; a.uw2 = uw2; a.l2 = l2; a.u2 = u2; a.rows2 = rows2; a.H2 = dim_out2;
     return run<CONCRETIZE>("faith_concretize", a, q, FAITH_LAYOUT_NATURAL, stream);
 }
 

@@ -783,22 +783,12 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     }
 
     // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the reference
-    // interface exposes it, the planes do not use it.  One launch when both objects have the same
-    // [D, H] shape (always on the scores path).
+    // interface exposes it, the planes do not use it.  One launch for both objects.
     // An object with its heads side by side is concretized as the one [L, D, heads * width] object it is.
     const int cx_rows = x_sbs ? B / heads * Lx : B * Lx, cx_h = x_sbs ? heads * d : d;
     const int cy_rows = y_sbs ? B / heads * y_len : B * y_len, cy_h = y_sbs ? heads * y_h : y_h;
-    int rc;
-    if (cx_h == cy_h) {
-        rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows,
-                                    D, cx_h, epsilon, q, words, stream);
-    } else {
-        rc = faith_concretize(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, D, cx_h, epsilon, q, words,
-                              FAITH_LAYOUT_NATURAL, stream);
-        if (rc == FAITH_OK)
-            rc = faith_concretize(y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows, D, cy_h, epsilon, q, words,
-                                  FAITH_LAYOUT_NATURAL, stream);
-    }
+    int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows, D,
+                                    cx_h, cy_h, epsilon, q, words, stream);
     if (rc != FAITH_OK) return rc;
 
     hipLaunchKernelGGL(dot_b<VP>, dim3((unsigned)((long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T))),
