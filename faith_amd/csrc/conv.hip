@@ -394,7 +394,7 @@ __global__ void __launch_bounds__(DP * DG) conv_direct(const ConvArgs g) {
     const int oh = (id / g.Wo) % g.Ho;
     const int co = (id / ((size_t)g.Wo * g.Ho)) % g.Co;
     const int n = id / ((size_t)g.Wo * g.Ho * g.Co);
-    double sl = 0.0, su = 0.0;
+    double sm = 0.0, sr = 0.0;
     for (int ci = cg; ci < g.Ci; ci += DG) {
         const float *xl = g.xl + ((size_t)n * g.Ci + ci) * g.H * g.W;
         const float *xu = g.xu + ((size_t)n * g.Ci + ci) * g.H * g.W;
@@ -405,18 +405,20 @@ __global__ void __launch_bounds__(DP * DG) conv_direct(const ConvArgs g) {
             for (int kw = 0; kw < g.K; ++kw) {
                 const int iw = ow * g.S - g.P + kw;
                 if (iw < 0 || iw >= g.W) continue;
-                const float wv = w[kh * g.K + kw];
-                const double wp = fmaxf(wv, 0.f), wq = fminf(wv, 0.f);
+                // w+ a + w- b = w m - |w| r and w+ b + w- a = w m + |w| r with m = (a + b) / 2,
+                // r = (b - a) / 2, both exact in double: two fused multiply-adds per tap instead of four
+                const double wv = w[kh * g.K + kw];
                 const double a = xl[ih * g.W + iw], b = xu[ih * g.W + iw];
-                sl += wp * a + wq * b;
-                su += wp * b + wq * a;
+                sm += wv * (0.5 * (a + b));
+                sr += fabs(wv) * (0.5 * (b - a));
             }
         }
     }
-    red[0][cg][px] = sl;
-    red[1][cg][px] = su;
+    red[0][cg][px] = sm - sr;
+    red[1][cg][px] = sm + sr;
     __syncthreads();
     if (cg == 0 && live) {
+        double sl = red[0][0][px], su = red[1][0][px];
 #pragma unroll
         for (int c = 1; c < DG; ++c) {
             sl += red[0][c][px];

@@ -274,7 +274,7 @@ __device__ __forceinline__ void simple_tile(const GemmArgs &g, const int m_blk, 
     const int M = brows ? g.Mb : g.Mw;
     const int m0 = (brows ? m_blk - mblk_w : m_blk) * 16, n0 = n_blk * 16;
     const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    double accl = 0.0, accu = 0.0;
+    double accm = 0.0, accr = 0.0;
     for (int k0 = 0; k0 < g.K; k0 += 16) {
         const int k = k0 + tx;
         const int ra = m0 + ty, rw = n0 + ty;
@@ -285,11 +285,11 @@ __device__ __forceinline__ void simple_tile(const GemmArgs &g, const int m_blk, 
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < 16; ++kk) {
-            const float w = sw[tx][kk];
-            const double wp = fmaxf(w, 0.f), wq = fminf(w, 0.f);
+            // centre / radius form (see sliced_tile): two fused multiply-adds per term instead of four
+            const double w = sw[tx][kk];
             const double xl = sl[ty][kk], xu = su[ty][kk];
-            accl += xl * wp + xu * wq;
-            accu += xu * wp + xl * wq;
+            accm += w * (0.5 * (xl + xu));
+            accr += fabs(w) * (0.5 * (xu - xl));
         }
         __syncthreads();
     }
@@ -297,8 +297,8 @@ __device__ __forceinline__ void simple_tile(const GemmArgs &g, const int m_blk, 
     if (row < M && col < g.N) {
         // the reference adds the bias to the rounded fp32 product (Bounds.py:391-395)
         const float add = (brows && g.bias) ? g.bias[col] : 0.f;
-        Cl[(size_t)row * g.N + col] = (float)accl + add;
-        Cu[(size_t)row * g.N + col] = (float)accu + add;
+        Cl[(size_t)row * g.N + col] = (float)(accm - accr) + add;
+        Cu[(size_t)row * g.N + col] = (float)(accm + accr) + add;
     }
 }
 
@@ -315,7 +315,7 @@ __device__ __forceinline__ void sliced_tile(const GemmArgs &g, const int m_blk, 
     const int m0 = m_blk * T, n0 = n_blk * T;
     const int ks = threadIdx.x / 64, o = threadIdx.x % 64;
     const int tx = o % T, ty = o / T;                       // output (m0 + ty, n0 + tx)
-    double accl = 0.0, accu = 0.0;
+    double accm = 0.0, accr = 0.0;
     for (int k0 = 0; k0 < g.K; k0 += KC) {
         for (int e = threadIdx.x; e < T * KC; e += 256) {
             const int r = e / KC, k = e % KC;
@@ -329,16 +329,17 @@ __device__ __forceinline__ void sliced_tile(const GemmArgs &g, const int m_blk, 
 #pragma unroll 4
         for (int kk = 0; kk < KC / S; ++kk) {
             const int k = ks * (KC / S) + kk;
-            const float w = sw[tx][k];
-            const double wp = fmaxf(w, 0.f), wq = fminf(w, 0.f);
+            // xl w+ + xu w- = w m - |w| r and xu w+ + xl w- = w m + |w| r with m = (xl + xu) / 2,
+            // r = (xu - xl) / 2, both exact in double: two fused multiply-adds per term instead of four
+            const double w = sw[tx][k];
             const double xl = sl[ty][k], xu = su[ty][k];
-            accl += xl * wp + xu * wq;
-            accu += xu * wp + xl * wq;
+            accm += w * (0.5 * (xl + xu));
+            accr += fabs(w) * (0.5 * (xu - xl));
         }
         __syncthreads();
     }
-    red[0][ks][o] = accl;
-    red[1][ks][o] = accu;
+    red[0][ks][o] = accm - accr;
+    red[1][ks][o] = accm + accr;
     __syncthreads();
     const int row = m0 + ty, col = n0 + tx;
     if (ks == 0 && row < g.Mb && col < g.N) {
