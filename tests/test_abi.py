@@ -90,3 +90,31 @@ def test_workloads_are_reproducible():
     assert bool((a["x"]["uw"] >= a["x"]["lw"]).all()) and bool((a["x"]["ub"] >= a["x"]["lb"]).all())
     c3 = make_config(3, scale=0.1)
     assert c3["x"]["lw"].shape == (4, 13, 256, 64)
+
+
+def test_binding_argument_types_match_the_header(lib):
+    """Every prototype in include/faith_amd.h, parameter by parameter, against the ctypes table."""
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    protos = re.findall(r"\bint\s+(faith_\w+)\s*\(([^;]*?)\)\s*;", src, flags=re.S)
+    assert len(protos) >= 15
+    kinds = {ctypes.c_void_p: "pointer", ctypes.c_int: "int", ctypes.c_float: "float", ctypes.c_longlong: "long long"}
+    for name, params in protos:
+        if name in ("faith_version",):
+            continue
+        want = []
+        for prm in [x.strip() for x in params.replace("\n", " ").split(",")]:
+            if prm in ("void", ""):
+                continue
+            if "*" in prm:
+                want.append("pointer")
+            elif prm.startswith("long long"):
+                want.append("long long")
+            elif prm.startswith("float"):
+                want.append("float")
+            elif prm.startswith("int"):
+                want.append("int")
+            else:
+                raise AssertionError(f"{name}: cannot classify parameter {prm!r}")
+        got = [kinds[t] for t in lib.SIGNATURES[name]]
+        assert got == want, f"{name}: header {want} vs binding {got}"
