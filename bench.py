@@ -129,6 +129,45 @@ def bench_config0(args, ops, O, wl):
                     {"note": "34 MFLOP: launch-latency bound (3 launches), latency is the figure of merit"})
 
 
+def bench_notebook_shapes(args, ops, O):
+    """The shapes of the reference's own timing notebooks (Benchmark/tvm_ansor_benchmark.ipynb:369-1036:
+    Bounds.relu at B=1, L=2, D_in = H in {64, 128, 256, 512} and Bounds.matmul at L=128, D_in = H = 64),
+    the only timings the reference holds (on an NVIDIA workstation GPU; not comparable, listed for scale).
+    Launch-latency bound: the figure is microseconds per call through the Python wrapper."""
+    import torch
+    out = []
+    g = torch.Generator().manual_seed(4242)
+
+    def obj(L, D, H):
+        lw = torch.randn(1, L, D, H, generator=g) * 0.1
+        lb = torch.randn(1, L, H, generator=g)
+        return {"lw": lw, "lb": lb, "uw": lw + 0.01 * torch.rand(1, L, D, H, generator=g),
+                "ub": lb + 0.1 * torch.rand(1, L, H, generator=g)}
+    for n in (64, 128, 256, 512):
+        x = obj(2, n, n)
+        xd = to_dev(x)
+        t = gpu_times_ms(lambda: ops.relu(*quad(xd), 2.0, 0.01, 1), 100, 10)
+        cpu = None
+        if not args.no_cpu:
+            xo = O.LinearBounds(*quad(x))
+            s = cpu_time_s(lambda: O.relu(xo, 2.0, 0.01, 1), reps=10, warmup=2)
+            cpu = {"latency_us": round(s * 1e6, 1)}
+        out.append(op_entry(f"extra: reference notebook shape, relu p=2 [1,2,{n},{n}]", "hbm", t, 16 * 2 * n * n + 16 * 2 * n, cpu))
+    x = obj(128, 64, 64)
+    xd = to_dev(x)
+    W = (torch.randn(64, 64, generator=g) / 8).cuda()
+    t = gpu_times_ms(lambda: ops.linear(*quad(xd), W, None), 100, 10)
+    cpu = None
+    if not args.no_cpu:
+        xo = O.LinearBounds(*quad(x))
+        Wc = W.cpu()
+        s = cpu_time_s(lambda: O.linear(xo, Wc, None), reps=10, warmup=2)
+        cpu = {"latency_us": round(s * 1e6, 1)}
+    out.append(op_entry("extra: reference notebook shape, matmul [1,128,64,64]x[64,64]", "mfma", t,
+                        4 * 2 * (128 * 64 + 128) * 64 * 64, cpu))
+    return out
+
+
 def gpu_back_to_back_ms(fn, launches, repeats=5):
     """Average duration of one launch when `launches` of them are queued back to back between one pair of
     HIP events (the event pair's own overhead, about 2 us per launch when every launch is bracketed, is
@@ -436,6 +475,8 @@ def main():
     extra = set() if args.only_headline else {int(c) for c in args.configs.split(",") if c.strip()}
     if 0 in extra:
         entries = [bench_config0(args, ops, O, wl)] + entries
+        if not args.profile:
+            entries += bench_notebook_shapes(args, ops, O)
     if 2 in extra:
         entries += bench_config2(args, ops, O, wl)
     if 3 in extra:
