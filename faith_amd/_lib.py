@@ -32,7 +32,7 @@ SIGNATURES = {
     "faith_multiply_verification": [_P] * 12 + [_I, _I, _I, _F, _I, _I, _P],
     "faith_affine_verification": [_P] * 5 + [_F] + [_P] * 9 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_rowsum_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
-    "faith_layer_norm_verification": [_P] * 10 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
+    "faith_layer_norm_verification": [_P] * 14 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_interval_unary": [_I, _P, _P, _P, _P, ctypes.c_longlong, _P],
     "faith_interval_product": [_P] * 6 + [ctypes.c_longlong, _P],
     "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],

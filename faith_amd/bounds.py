@@ -122,16 +122,20 @@ class Bounds:
         return e.divide(self._like(*ops.rowsum(*e._c())))
 
     # ---- Bounds.py:1111-1131
-    def layer_norm(self, normalizer, layer_norm):
+    def layer_norm(self, normalizer, layer_norm, residual=None):
+        """residual (beyond the reference's signature): a bound object added first, i.e.
+        `self.add(residual).layer_norm(...)` (VerifierForward.py:166, 181-189) without the pass of the sum
+        through memory; same values."""
         if layer_norm == "no":
-            return self
+            return self if residual is None else self.add(residual)
         weight, bias = normalizer.weight.detach().contiguous(), normalizer.bias.detach().contiguous()
+        other = None if residual is None else residual._c()
         if layer_norm == "no_var":
-            # mean subtraction, weight and bias in one launch
-            return self._like(*ops.layer_norm(*self._c(), weight, bias))
+            # (residual sum,) mean subtraction, weight and bias in one launch
+            return self._like(*ops.layer_norm(*self._c(), weight, bias, other))
         assert layer_norm == "standard"
         H = self.dim_out
-        minus_mu = self._like(*ops.layer_norm(*self._c()))
+        minus_mu = self._like(*ops.layer_norm(*self._c(), other=other))
         w_avg = torch.full((H, H), 1.0 / H, device=self.device, dtype=torch.float32)
         variance = minus_mu.sqr().matmul(w_avg)
         normalized = minus_mu.divide(variance.add(1e-12).sqrt())

@@ -116,9 +116,19 @@ __global__ void __launch_bounds__(256) row_kernel(const Pair w, const Pair b, co
             const float4 c = *reinterpret_cast<const float4 *>(p.up + base + (size_t)i * 4);
             l[0] = a.x; l[1 % VEC] = a.y; l[2 % VEC] = a.z; l[3 % VEC] = a.w;
             u[0] = c.x; u[1 % VEC] = c.y; u[2 % VEC] = c.z; u[3 % VEC] = c.w;
+            if (p.add_lo) {     // Bounds.add of a second object before the row operation: one fp32 add, as the separate launch rounds it
+                const float4 a2 = *reinterpret_cast<const float4 *>(p.add_lo + base + (size_t)i * 4);
+                const float4 c2 = *reinterpret_cast<const float4 *>(p.add_up + base + (size_t)i * 4);
+                l[0] += a2.x; l[1 % VEC] += a2.y; l[2 % VEC] += a2.z; l[3 % VEC] += a2.w;
+                u[0] += c2.x; u[1 % VEC] += c2.y; u[2 % VEC] += c2.z; u[3 % VEC] += c2.w;
+            }
         } else {
             l[0] = p.lo[base + i];
             u[0] = p.up[base + i];
+            if (p.add_lo) {
+                l[0] += p.add_lo[base + i];
+                u[0] += p.add_up[base + i];
+            }
         }
     };
     float sl = 0.f, su = 0.f;
@@ -245,7 +255,8 @@ int launch_rows(const char *who, const Pair &w, const Pair &b, const float *weig
                 long long rows_b, int H, void *stream) {
     FAITH_REQUIRE(rows_w >= 0 && rows_b >= 0 && rows_w + rows_b > 0 && H > 0 && (rows_w + rows_b + 3) / 4 <= 0x7fffffffLL,
                   FAITH_ERR_SHAPE, "%s: rows=%lld + %lld, dim_out=%d out of range", who, rows_w, rows_b, H);
-    const bool vec4 = H % 4 == 0 && all_aligned16({w.lo, w.up, w.out_lo, w.out_up, b.lo, b.up, b.out_lo, b.out_up});
+    const bool vec4 = H % 4 == 0 && all_aligned16({w.lo, w.up, w.add_lo, w.add_up, w.out_lo, w.out_up, b.lo, b.up, b.add_lo, b.add_up, b.out_lo,
+                                                 b.out_up});
     const dim3 grid((unsigned)((rows_w + rows_b + 3) / 4));
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (vec4)
@@ -299,11 +310,17 @@ extern "C" int faith_rowsum_verification(const float *src_lb, const float *src_u
 }
 
 extern "C" int faith_layer_norm_verification(const float *src_lb, const float *src_ub, const float *src_lw,
-                                             const float *src_uw, const float *weight, const float *bias,
-                                             float *out_lb, float *out_ub, float *out_lw, float *out_uw,
-                                             long long rows_w, long long rows_b, int dim_out, void *stream) {
+                                             const float *src_uw, const float *add_lb, const float *add_ub,
+                                             const float *add_lw, const float *add_uw, const float *weight,
+                                             const float *bias, float *out_lb, float *out_ub, float *out_lw,
+                                             float *out_uw, long long rows_w, long long rows_b, int dim_out,
+                                             void *stream) {
     FAITH_OBJECT_NOT_NULL();
-    const Pair w{src_lw, src_uw, nullptr, nullptr, out_lw, out_uw}, b{src_lb, src_ub, nullptr, nullptr, out_lb, out_ub};
+    const bool adding = add_lb || add_ub || add_lw || add_uw;
+    FAITH_REQUIRE(!adding || (add_lb && add_ub && add_lw && add_uw), FAITH_ERR_NULL,
+                  "faith_layer_norm_verification: the four tensors of the added object must be given together");
+    FAITH_ALIGNED4(add_lb); FAITH_ALIGNED4(add_ub); FAITH_ALIGNED4(add_lw); FAITH_ALIGNED4(add_uw);
+    const Pair w{src_lw, src_uw, add_lw, add_uw, out_lw, out_uw}, b{src_lb, src_ub, add_lb, add_ub, out_lb, out_ub};
     return launch_rows<MODE_NORM>("faith_layer_norm_verification", w, b, weight, bias, rows_w, rows_b, dim_out, stream);
 }
 

@@ -105,14 +105,20 @@ def bound_attention(bounds_input, attention):
     return scores, probs, context
 
 
+def _add_norm(x, residual, normalizer, layer_norm):
+    """x.add(residual).layer_norm(...); one launch where the bound object takes the residual itself."""
+    if hasattr(x, "attention_scores"):        # the HIP-backed object (the oracle's keeps the reference's signature)
+        return x.layer_norm(normalizer, layer_norm, residual=residual)
+    return x.add(residual).layer_norm(normalizer, layer_norm)
+
+
 def bound_layer(bounds_input, layer, layer_norm="no_var", hidden_act="relu"):
     """VerifierForward._bound_layer: attention block, residual + norm, feed-forward, residual + norm."""
     scores, probs, attention = bound_attention(bounds_input, layer.attention)
     attention = attention.dense(layer.attention.output.dense)
-    attention = attention.add(bounds_input).layer_norm(layer.attention.output.LayerNorm, layer_norm)
+    attention = _add_norm(attention, bounds_input, layer.attention.output.LayerNorm, layer_norm)
     intermediate = attention.dense(layer.intermediate.dense).act(hidden_act)
-    dense = intermediate.dense(layer.output.dense).add(attention)
-    output = dense.layer_norm(layer.output.LayerNorm, layer_norm)
+    output = _add_norm(intermediate.dense(layer.output.dense), attention, layer.output.LayerNorm, layer_norm)
     return scores, probs, output
 
 

@@ -272,18 +272,26 @@ def rowsum(lw, lb, uw, ub):
     return olw, olb, ouw, oub
 
 
-def layer_norm(lw, lb, uw, ub, weight=None, bias=None):
+def layer_norm(lw, lb, uw, ub, weight=None, bias=None, other=None):
     """Mean subtraction along the last axis, then per-neuron weight (split by sign) and bias:
-    Bounds.layer_norm in mode "no_var"; with weight = bias = None its first step in mode "standard"."""
+    Bounds.layer_norm in mode "no_var"; with weight = bias = None its first step in mode "standard".
+    other: (lw, lb, uw, ub) of a second object added first (the residual connection), same launch."""
     rows_w, rows_b, H = _object(lw, lb, uw, ub)
     if weight is not None:
         _check("weight", weight, (H,))
     if bias is not None:
         _check("bias", bias, (H,))
+    if other is not None:
+        _check("other.lw", other[0], lw.shape); _check("other.uw", other[2], lw.shape)
+        _check("other.lb", other[1], lb.shape); _check("other.ub", other[3], lb.shape)
+        alw, alb, auw, aub = other
+    else:
+        alw = alb = auw = aub = None
     olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
     with _on(lw.device):
-        _lib.call("faith_layer_norm_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
-                  _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), rows_w, rows_b, H, _stream(lw))
+        _lib.call("faith_layer_norm_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(alb), _ptr(aub),
+                  _ptr(alw), _ptr(auw), _ptr(weight), _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
+                  rows_w, rows_b, H, _stream(lw))
     return olw, olb, ouw, oub
 
 

@@ -147,7 +147,8 @@ int faith_multiply_verification(const float *x_lb, const float *x_ub, const floa
 /*
  * The next three take a whole bound object -- rows_w coefficient rows (length * dim_in) and rows_b
  * constant rows (length), each dim_out long -- and handle all four tensors in one launch.  The
- * reference builds them from PyTorch expressions; there is no CUDA counterpart.  out may alias src.
+ * reference builds them from PyTorch expressions; there is no CUDA counterpart.  out may alias src (or the added
+ * object).
  *
  * Scale, add, shift: Bounds.multiply with a float or a per-neuron tensor (Bounds.py:595-607,
  * :653-664) and Bounds.add with an object or a tensor (:383-395), alone or combined:
@@ -178,10 +179,15 @@ int faith_rowsum_verification(const float *src_lb, const float *src_ub,
  * and the first step of mode "standard"): subtract the row mean -- the mean of the UPPER tensor
  * from the lower one and the reverse, as matmul(ones / H).multiply(-1.) gives it -- then scale by
  * weight[h] split by sign and add bias[h] to the constant rows.  weight and bias may be NULL
- * (NULL weight: mean subtraction only).
+ * (NULL weight: mean subtraction only).  add_* (all four or none) is a second object of the same
+ * shape added to src first: the residual connection in front of every normalisation
+ * (`dense.add(x).layer_norm(...)`, VerifierForward.py:166, 181-189) without its own pass over memory;
+ * the sum is rounded to fp32 as the separate Bounds.add rounds it.
  */
 int faith_layer_norm_verification(const float *src_lb, const float *src_ub,
                                   const float *src_lw, const float *src_uw,
+                                  const float *add_lb, const float *add_ub,
+                                  const float *add_lw, const float *add_uw,
                                   const float *weight, const float *bias,
                                   float *out_lb, float *out_ub, float *out_lw, float *out_uw,
                                   long long rows_w, long long rows_b, int dim_out, void *stream);

@@ -131,6 +131,41 @@ def test_fused_mean_subtraction_against_float64(H, with_affine):
         assert close(a, e, rtol=1e-5, atol=2e-6)
 
 
+@pytest.mark.parametrize("H", [64, 10, 1284, 330])
+@pytest.mark.parametrize("mode", ["no", "no_var", "standard"])
+def test_residual_inside_layer_norm(H, mode):
+    """layer_norm(..., residual=y) is x.add(y).layer_norm(...) in one launch: same values bit for bit
+    (the sum is rounded to fp32 before the mean, as the separate launch stores it)."""
+    g = torch.Generator().manual_seed(68)
+    x = gpu_bounds(rand_bounds(g, 2, 5, 6, H, sw=0.02, sb=1.0, gap_w=0.002, gap_b=0.02), 2.0, 0.01)
+    y = gpu_bounds(rand_bounds(g, 2, 5, 6, H, sw=0.02, sb=1.0, gap_w=0.002, gap_b=0.02), 2.0, 0.01)
+
+    class Norm:
+        weight, bias = torch.randn(H, generator=g).cuda(), torch.randn(H, generator=g).cuda()
+    fused = x.layer_norm(Norm, mode, residual=y)
+    apart = x.add(y).layer_norm(Norm, mode)
+    for a, e, name in zip((fused.lw, fused.lb, fused.uw, fused.ub), (apart.lw, apart.lb, apart.uw, apart.ub),
+                          ("lw", "lb", "uw", "ub")):
+        assert torch.equal(a, e), f"{name} differs between the fused and the separate residual sum"
+
+
+def test_residual_inside_layer_norm_in_place():
+    """The row-wise entry points may write over their inputs, the added object included."""
+    from faith_amd import ops, _lib
+    g = torch.Generator().manual_seed(69)
+    x = [t.cuda() for t in rand_bounds(g, 1, 4, 3, 1284, ordered=False).tensors()]
+    y = [t.cuda() for t in rand_bounds(g, 1, 4, 3, 1284, ordered=False).tensors()]
+    exp = ops.layer_norm(*x, other=tuple(y))
+    lw, lb, uw, ub = y                 # results go where the added object was
+    _lib.call("faith_layer_norm_verification", x[1].data_ptr(), x[3].data_ptr(), x[0].data_ptr(), x[2].data_ptr(),
+              lb.data_ptr(), ub.data_ptr(), lw.data_ptr(), uw.data_ptr(), None, None,
+              lb.data_ptr(), ub.data_ptr(), lw.data_ptr(), uw.data_ptr(), lw.numel() // 1284, lb.numel() // 1284, 1284,
+              torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for a, e in zip((lw, lb, uw, ub), exp):
+        assert torch.equal(a, e)
+
+
 def test_shift_shares_the_coefficients():
     """Bounds.add with a tensor returns the same lw / uw tensors (Bounds.py:391-395 does too)."""
     g = torch.Generator().manual_seed(67)
