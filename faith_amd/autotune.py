@@ -10,7 +10,8 @@ libfaith_amd.so and are selected per call through faith_tune_set, so a sample co
 
 What can be tuned (see the FAITH_TUNE_* knobs in include/faith_amd.h):
 
-    linear       macro-tile of the sign-split GEMM: 64x64, 128x128, 128x64, 64x128
+    linear       macro-tile of the sign-split GEMM: 64x64, 128x128, 128x64, 64x128, or 32x32 with the
+                 reduction split over the workgroup's wavefronts
     dot_qk/dot_v 128x64 persistent tiles, or one 32x32 block per wavefront with 1..16 perturbation
                  coordinates per wavefront
     act          tile shape of the relaxation kernels (relu, tanh, exp, ...)
@@ -106,6 +107,11 @@ class Heuristics:
                                  registers=acc + 40 + 12 * (tm + tn) // 64, workgroups=tiles,
                                  padding=(-(-rows // tm) * tm * -(-n // tn) * tn) / float(rows * n) - 1.0,
                                  steps=-(-k // 16), mfma_per_step=(tm // 64) * (tn // 64) * 32))
+            # 32 x 32 block per workgroup, the reduction split over its four wavefronts (tiny problems)
+            out.append(_cand({TUNE_GEMM_VARIANT: 5}, tile_m=32, tile_n=32, lds_bytes=32768, registers=140,
+                             workgroups=-(-rows // 32) * -(-n // 32),
+                             padding=(-(-rows // 32) * 32 * -(-n // 32) * 32) / float(rows * n) - 1.0,
+                             steps=-(-k // 32), mfma_per_step=16))
             return out
         if op in ("dot_qk", "dot_v"):
             batch, lx, ly, d_in, d = shape
@@ -145,7 +151,9 @@ class Heuristics:
             return False
         if op == "linear":
             # a tile more than twice the problem in either direction is padding only
-            rows, _, n = shape
+            rows, k, n = shape
+            if cand.knob_dict().get(TUNE_GEMM_VARIANT) == 5:
+                return k % 32 == 0            # each wavefront takes a quarter of K in steps of 8
             return cand.param("tile_m") < 2 * max(rows, 64) and cand.param("tile_n") < 2 * max(n, 64)
         if op in ("dot_qk", "dot_v"):
             _, lx, ly, _, d = shape

@@ -736,6 +736,10 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
             launch_natural<MODE, Q, 4, 8, 256, 8>(a, st);
         else if (vec4)
             launch_natural<MODE, Q, 4, 16, 1024, 4>(a, st);
+        else if (a.H <= 8 && a.H2 <= 8)
+            // a handful of neurons (the margin of a classifier): 64-neuron tiles would walk D_in in chunks of
+            // 32 rows, one memory latency each; 8-neuron tiles take 256 rows per chunk
+            launch_natural<MODE, Q, 1, 8, 256, 8>(a, st);
         else
             launch_natural<MODE, Q, 1, 64, 256, 8>(a, st);
         return;

@@ -376,6 +376,105 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs 
     signsplit_gemm_body<EXACT, MBM, MBN>(g, sm, blockIdx.x - b_tiles);
 }
 
+
+// Tiny problems (a pooler, a classifier: fewer 64 x 64 tiles than a quarter of the CUs): a 64 x 64 tile is
+// one wavefront's chain of K / 2 * 4 MFMAs per 32 x 32 block -- 14 us at K = 256 with nine tenths of the
+// machine idle.  Here a workgroup owns ONE 32 x 32 block of C_l and C_u and its four wavefronts split the
+// reduction four ways; every wavefront loads its fragments straight from global memory in MFMA layout (lane
+// (i, h) holds k = 8 s + 4 h .. + 3 of row i: the same K pairing as the LDS fragments above), so there is
+// no staging and no barrier in the loop; the four partial blocks meet in LDS and are added in a fixed
+// order.  K % 32 == 0.  The first `b_tiles` workgroups take the constant-term rows, as above.
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs g, const int b_tiles) {
+    __shared__ __align__(16) float sm[4 * 2 * 16 * 64];          // 32 KB: [wavefront][l, u][register][lane]
+    if ((int)blockIdx.x < b_tiles) {
+        const int tiles_n = (g.N + 7) / 8;
+        const int m_blk = blockIdx.x / tiles_n;
+        if (m_blk < (g.Mb + 7) / 8) sliced_tile(g, m_blk, blockIdx.x % tiles_n, sm);
+        return;
+    }
+    constexpr int CH = 4;                                        // K-steps of 8 fetched ahead
+    const int pid = blockIdx.x - b_tiles;
+    const int tiles_n = (g.N + 31) / 32;
+    const int m0 = (pid / tiles_n) * 32, n0 = (pid % tiles_n) * 32;
+    const int lane = threadIdx.x % 64, wv = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int fi = lane % 32, fh = lane / 32;
+    const int K = g.K, kw = K / 4, ns = kw / 8;
+    // rows past the end re-read the last row; their results are never stored
+    const size_t oa = (size_t)min(m0 + fi, g.Mw - 1) * K + wv * kw + 4 * fh;
+    const size_t ow = (size_t)min(n0 + fi, g.N - 1) * K + wv * kw + 4 * fh;
+    const float4 *__restrict__ pal = reinterpret_cast<const float4 *>(g.Al + oa);
+    const float4 *__restrict__ pau = reinterpret_cast<const float4 *>(g.Au + oa);
+    const float4 *__restrict__ pw = reinterpret_cast<const float4 *>(g.W + ow);
+
+    floatx16 cl, cu;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) cl[r] = cu[r] = 0.f;
+    float4 al[CH], au[CH], w[CH], nal[CH], nau[CH], nw[CH];
+    auto fetch = [&](float4 (&a)[CH], float4 (&b)[CH], float4 (&c)[CH], int s0) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            if (s0 + i < ns) {
+                a[i] = pal[2 * (s0 + i)];
+                b[i] = pau[2 * (s0 + i)];
+                c[i] = pw[2 * (s0 + i)];
+            }
+        }
+    };
+    fetch(al, au, w, 0);
+    for (int s0 = 0; s0 < ns; s0 += CH) {
+        if (s0 + CH < ns) fetch(nal, nau, nw, s0 + CH);
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            if (s0 + i < ns) {
+                // split by sign with ordinary float code: these values feed the MFMAs directly
+                const float4 wp = make_float4(fmaxf(w[i].x, 0.f), fmaxf(w[i].y, 0.f), fmaxf(w[i].z, 0.f), fmaxf(w[i].w, 0.f));
+                const float4 wq = make_float4(fminf(w[i].x, 0.f), fminf(w[i].y, 0.f), fminf(w[i].z, 0.f), fminf(w[i].w, 0.f));
+#define FAITH_STEP(c)                       \
+    cl = mfma(al[i].c, wp.c, cl);           \
+    cu = mfma(au[i].c, wp.c, cu);           \
+    cl = mfma(au[i].c, wq.c, cl);           \
+    cu = mfma(al[i].c, wq.c, cu);
+                FAITH_STEP(x)
+                FAITH_STEP(y)
+                FAITH_STEP(z)
+                FAITH_STEP(w)
+#undef FAITH_STEP
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            al[i] = nal[i];
+            au[i] = nau[i];
+            w[i] = nw[i];
+        }
+    }
+
+    // the four partial blocks, added in the order of their K ranges; wavefront v finishes registers 4 v .. 4 v + 3
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        sm[((wv * 2 + 0) * 16 + r) * 64 + lane] = cl[r];
+        sm[((wv * 2 + 1) * 16 + r) * 64 + lane] = cu[r];
+    }
+    __syncthreads();
+    const int col = n0 + fi;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int r = 4 * wv + q;
+        float sl = sm[((0 * 2 + 0) * 16 + r) * 64 + lane], su = sm[((0 * 2 + 1) * 16 + r) * 64 + lane];
+#pragma unroll
+        for (int v = 1; v < 4; ++v) {
+            sl += sm[((v * 2 + 0) * 16 + r) * 64 + lane];
+            su += sm[((v * 2 + 1) * 16 + r) * 64 + lane];
+        }
+        // register r of a 32 x 32 block is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
+        const int row = m0 + 8 * wv + 4 * fh + q;
+        if (row < g.Mw && col < g.N) {
+            g.Cl[(size_t)row * g.N + col] = sl;
+            g.Cu[(size_t)row * g.N + col] = su;
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
@@ -411,12 +510,21 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
         else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
         else if (dim_out >= 1024 && tiles(128, 128) >= 16 * cus) { tm = 128; tn = 128; }
         else { tm = 64; tn = 64; }
-        switch (faith::tune_get(FAITH_TUNE_GEMM_VARIANT)) {
+        const int pick = faith::tune_get(FAITH_TUNE_GEMM_VARIANT);
+        switch (pick) {
             case 1: tm = 64;  tn = 64;  break;
             case 2: tm = 128; tn = 128; break;
             case 3: tm = 128; tn = 64;  break;
             case 4: tm = 64;  tn = 128; break;
             default: break;
+        }
+        // tiny problems with a reduction worth splitting: a 32 x 32 block per workgroup, K over its wavefronts
+        if (dim_out % 32 == 0 && (pick == 5 || (pick == 0 && dim_out >= 128 && 4 * tiles(64, 64) <= cus))) {
+            const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
+            const long long grid = ((mw + 31) / 32) * ((dim_y_out + 31) / 32);
+            FAITH_REQUIRE(grid + gridb <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
+            hipLaunchKernelGGL(signsplit_gemm_ksplit, dim3((unsigned)(grid + gridb)), dim3(NTHREADS), 0, st, g, (int)gridb);
+            return faith::check_launch("faith_matmul_verification");
         }
         const long long mblks = (mw + tm - 1) / tm;
         const long long grid = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tn - 1) / tn);

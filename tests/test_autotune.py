@@ -11,10 +11,12 @@ from faith_amd import autotune as A
 def test_heuristics_reject_what_cannot_fit_or_is_padding():
     h = A.Heuristics()
     lin = h.candidates("linear", (131072, 1024, 1024))
-    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in lin} == {1, 2, 3, 4}
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in lin} == {1, 2, 3, 4, 5}
     # a 64-row, 64-column problem: tiles of 128 in either direction are padding
     tiny = h.candidates("linear", (64, 64, 64))
-    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in tiny} == {1}
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in tiny} == {1, 5}
+    # the split-reduction kernel hands each wavefront a quarter of K in steps of 8
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in h.candidates("linear", (64, 72, 64))} == {1}
     # the per-wavefront dot kernel needs d % 8 == 0 and d <= 80, and is pointless for long sequences
     assert all(c.knob_dict()[A.TUNE_DOT_VARIANT] == 1 for c in h.candidates("dot_qk", (4, 128, 128, 256, 100)))
     short = h.candidates("dot_qk", (4, 32, 32, 256, 64))
@@ -22,7 +24,7 @@ def test_heuristics_reject_what_cannot_fit_or_is_padding():
     # a machine with a quarter of the LDS loses the large GEMM tiles
     small_lds = dict(A.mi355x_metafile, MAX_LDS_KB=40)
     kept = A.Heuristics(small_lds).candidates("linear", (131072, 1024, 1024))
-    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in kept} == {1}
+    assert {c.knob_dict()[A.TUNE_GEMM_VARIANT] for c in kept} == {1, 5}
     with pytest.raises(ValueError):
         h.propose("softmax", (1, 2, 3))
 
@@ -71,7 +73,7 @@ def test_search_finds_the_planted_optimum_and_restores_the_knobs():
     # exhaustive when the budget covers the space
     full = A.autotune("linear", (8192, 256, 256), run=lambda: None, rounds=3, samples=2,
                       measure=lambda run: 10.0 + state.get(A.TUNE_GEMM_VARIANT, 0), setter=setter)
-    assert full.best_us == 10.0 and len(full.measured) == 5
+    assert full.best_us == 10.0 and len(full.measured) == 6
 
 
 def test_a_variant_that_raises_is_skipped():
@@ -124,6 +126,12 @@ def test_every_gemm_tile_gives_the_same_result(shape):
             got = ops.linear(*x, W, bias)
         for a, b in zip(got, base):
             assert torch.equal(a, b), f"variant {variant}"
+    if shape[2] % 32 == 0:
+        # the split-reduction kernel adds four partial sums: same value up to fp32 summation order
+        with A.applied({A.TUNE_GEMM_VARIANT: 5}):
+            got = ops.linear(*x, W, bias)
+        for a, b in zip(got, base):
+            torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.gpu

@@ -64,6 +64,27 @@ def test_linear_shapes(shape, with_bias):
     check(x, W, bias, "sweep")
 
 
+@pytest.mark.parametrize("shape", [
+    (1, 1, 256, 256, 256),     # a pooler: first position only
+    (1, 1, 256, 256, 2),       # a classifier's margin
+    (1, 3, 85, 128, 50),       # ragged rows and columns, shortest reduction that is split
+    (2, 2, 40, 512, 96),
+    (1, 1, 64, 3072, 64),      # long reduction, many fetch rounds
+    (1, 1, 33, 160, 33),       # K / 4 = 40: five steps, the last fetch round partly empty
+])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_linear_tiny_problems_split_reduction(shape, with_bias):
+    """Problems of a few tiles with K % 32 == 0 and K >= 128 take the kernel that splits the reduction
+    over the four wavefronts of a workgroup."""
+    B, L, D, H, N = shape
+    g = torch.Generator().manual_seed(22)
+    x = rand_bounds(g, B, L, D, H, ordered=False, sw=0.5)
+    W = torch.randn(N, H, generator=g) / H ** 0.5
+    W.view(-1)[::7] = 0.0
+    bias = torch.randn(N, generator=g) if with_bias else None
+    check(x, W, bias, "tiny")
+
+
 def test_linear_config0_with_concretize():
     from faith_amd import ops
     from faith_amd.workloads import make_config
