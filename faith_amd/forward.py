@@ -42,18 +42,32 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
     length, dim = embeddings.shape[1], embeddings.shape[2]
     w = torch.zeros((length, dim * perturbed_words, dim), device=embeddings.device)
     positions = [index] if perturbed_words == 1 else list(index)
-    lb, ub = embeddings[0].unsqueeze(0).clone(), embeddings[0].unsqueeze(0).clone()
-    for i, pos in enumerate(positions):
-        if ibp:
+    if ibp:
+        lb, ub = embeddings[0].unsqueeze(0).clone(), embeddings[0].unsqueeze(0).clone()
+        for pos in positions:
             lb[0, pos] -= eps
             ub[0, pos] += eps
-        else:
-            w[pos, dim * i:dim * (i + 1), :] = torch.eye(dim, device=embeddings.device)
+    else:
+        # lower and upper start out equal and no operator writes into its inputs: one tensor serves both
+        # (the reference copies ub and uw, :131, :149)
+        lb = ub = embeddings[0].unsqueeze(0)
+        for i, pos in enumerate(positions):
+            w[pos, dim * i:dim * (i + 1), :] = _eye(dim, embeddings.device)
     lw = w.unsqueeze(0)
-    bounds = make_bounds(p, eps, lw, lb, lw.clone(), ub)
+    bounds = make_bounds(p, eps, lw, lb, lw, ub)
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
     return bounds
+
+
+_EYES = {}
+
+
+def _eye(dim, device):
+    key = (dim, str(device))
+    if key not in _EYES:
+        _EYES[key] = torch.eye(dim, device=device)
+    return _EYES[key]
 
 
 def _fold_heads(x, heads, size):
@@ -128,13 +142,31 @@ def bound_pooling(bounds, pooler_dense, make_bounds):
     return first.dense(pooler_dense).tanh()
 
 
+class _MarginLayer:
+    def __init__(self, classifier):
+        self.weight = classifier.weight.detach().clone()
+        self.bias = classifier.bias.detach().clone()
+        self.weight[0, :] -= self.weight[1, :]
+        self.bias[0] -= self.bias[1]
+        self.made_from = _stamp(classifier)
+
+
+def _stamp(layer):
+    # identifies the parameter values: the storage and torch's in-place modification counter
+    return tuple((t.data_ptr(), t._version) for t in (layer.weight, layer.bias))
+
+
 def _margin(bounds, classifier):
-    class Margin:
-        weight = classifier.weight.clone()
-        bias = classifier.bias.clone()
-    Margin.weight[0, :] -= Margin.weight[1, :]
-    Margin.bias[0] -= Margin.bias[1]
-    return bounds.dense(Margin).concretize()
+    """Row 0 of the classifier minus row 1 (VerifierForward.py:289-292 builds it by a deep copy on every call); kept on the
+    classifier object until its parameters change."""
+    cached = getattr(classifier, "_faith_margin", None)
+    if cached is None or cached.made_from != _stamp(classifier):
+        cached = _MarginLayer(classifier)
+        try:
+            classifier._faith_margin = cached
+        except AttributeError:          # an object that takes no new attributes: rebuilt per call
+            pass
+    return bounds.dense(cached).concretize()
 
 
 def bound_classifier(bounds, classifier, label):

@@ -66,6 +66,36 @@ def test_pipeline_on_the_oracle_is_sound(mode, p):
                 torch.Generator().manual_seed(8))
 
 
+def test_margin_layer_is_kept_until_the_classifier_changes():
+    g = torch.Generator().manual_seed(9)
+    classifier = SimpleNamespace(weight=torch.randn(2, HIDDEN, generator=g), bias=torch.randn(2, generator=g))
+    lw = torch.randn(1, 1, 5, HIDDEN, generator=g)
+    lb = torch.randn(1, 1, HIDDEN, generator=g)
+    x = OracleBounds(2.0, 0.1, lw, lb, lw + 0.01, lb + 0.1)
+
+    def expected():
+        w = classifier.weight.clone()
+        b = classifier.bias.clone()
+        w[0] -= w[1]
+        b[0] -= b[1]
+        return x.dense(SimpleNamespace(weight=w, bias=b)).concretize()
+    l, u = F._margin(x, classifier)
+    el, eu = expected()
+    assert torch.equal(l, el) and torch.equal(u, eu)
+    first = classifier._faith_margin
+    F._margin(x, classifier)
+    assert classifier._faith_margin is first                 # unchanged parameters: not rebuilt
+    classifier.weight[1, 3] += 0.5                           # in place: the stamp changes
+    l, u = F._margin(x, classifier)
+    el, eu = expected()
+    assert classifier._faith_margin is not first and torch.equal(l, el) and torch.equal(u, eu)
+    classifier.bias = torch.zeros(2)                         # replaced: another storage
+    l, u = F._margin(x, classifier)
+    el, eu = expected()
+    assert torch.equal(l, el) and torch.equal(u, eu)
+    assert not torch.equal(classifier.weight[0], first.weight[0])        # the classifier itself is never modified
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["no_var", "standard"])
 @pytest.mark.parametrize("p", [2.0, float("inf")])
