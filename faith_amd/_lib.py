@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfaith_amd.so")
 
 OK = 0
+ERR_NULL, ERR_SHAPE, ERR_UNSUPPORTED, ERR_ALIGN, ERR_LAUNCH = -1, -2, -3, -4, -5
 Q_1, Q_2, Q_INF = 1, 2, 0
 LAYOUT_NATURAL, LAYOUT_TRANSPOSED = 0, 1
 OP_RELU, OP_TANH, OP_EXP, OP_RECIPROCAL, OP_SQR, OP_SQRT = 1, 2, 3, 4, 5, 6
@@ -33,6 +34,8 @@ SIGNATURES = {
     "faith_affine_verification": [_P] * 5 + [_F] + [_P] * 9 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_rowsum_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_layer_norm_verification": [_P] * 14 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
+    "faith_softmax_verification": [_P] * 9 + [_I, _I, _I, _F, _I, _I, _P],
+    "faith_softmax_fits": [_I, _I],          # a predicate: returns 1 / 0, not a status (call it through lib)
     "faith_interval_unary": [_I, _P, _P, _P, _P, ctypes.c_longlong, _P],
     "faith_interval_product": [_P] * 6 + [ctypes.c_longlong, _P],
     "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],

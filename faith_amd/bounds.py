@@ -23,7 +23,7 @@ from types import SimpleNamespace
 
 import torch
 
-from . import ops
+from . import _lib, ops
 
 
 class Bounds:
@@ -118,6 +118,16 @@ class Bounds:
 
     # ---- Bounds.py:1005-1014
     def softmax(self):
+        if not self.ibp and ops.softmax_fits(self.dim_in, self.dim_out):
+            # the four operators below on a slab that stays in registers: one launch, one read, one write
+            try:
+                out = ops.softmax(*self._c(), self.p, self.eps, self.perturbed_words, return_sum_bound=True)
+            except _lib.FaithError as err:
+                if err.code != _lib.ERR_UNSUPPORTED:         # e.g. tensors that are not 16-byte aligned
+                    raise
+            else:
+                self._require(out[4], 1e-12, False, "reciprocal of a bound that reaches zero")
+                return self._like(*out[:4])
         e = self.exp()
         return e.divide(self._like(*ops.rowsum(*e._c())))
 

@@ -30,6 +30,7 @@ EXTRA = {
     "act.hip": ["-ffp-contract=off"],
     "mul.hip": ["-ffp-contract=off"],
     "affine.hip": ["-ffp-contract=off"],
+    "softmax.hip": ["-ffp-contract=off"],
 }
 
 

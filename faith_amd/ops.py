@@ -295,6 +295,28 @@ def layer_norm(lw, lb, uw, ub, weight=None, bias=None, other=None):
     return olw, olb, ouw, oub
 
 
+def softmax_fits(dim_in, dim_out):
+    """True if softmax() takes a [dim_in, dim_out] slab in one launch (16-byte aligned tensors assumed)."""
+    return bool(_lib.lib.faith_softmax_fits(int(dim_in), int(dim_out)))
+
+
+def softmax(lw, lb, uw, ub, p, eps, words=1, return_sum_bound=False):
+    """Bounds.softmax over the last axis in one launch: exp, sum, reciprocal and product on a slab that stays
+    in registers.  Returns (lw', lb', uw', ub'[, l_sum]); l_sum [B, L] is the concrete lower bound of the sum,
+    which must be >= 1e-12 for the result to mean anything (the reference asserts it).  Raises FaithError
+    (FAITH_ERR_UNSUPPORTED) when the slab does not fit: see softmax_fits."""
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    l_sum = torch.empty((B, L), device=lw.device, dtype=torch.float32) if return_sum_bound else None
+    with _on(lw.device):
+        _lib.call("faith_softmax_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub),
+                  _ptr(olw), _ptr(ouw), _ptr(l_sum), B * L, D, H, float(eps), q_code(p), int(words), _stream(lw))
+    if return_sum_bound:
+        return olw, olb, ouw, oub, l_sum
+    return olw, olb, ouw, oub
+
+
 def interval_unary(kind, l, u):
     """Interval bound propagation through relu / tanh / exp / reciprocal / sqr / sqrt: the interval of the
     image of [l, u], elementwise.  Returns (lb, ub)."""

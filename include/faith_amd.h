@@ -175,6 +175,26 @@ int faith_rowsum_verification(const float *src_lb, const float *src_ub,
                               long long rows_w, long long rows_b, int dim_out, void *stream);
 
 /*
+ * Softmax over the last axis (Bounds.softmax, Bounds.py:1005-1014: exp, sum over dim_out repeated,
+ * reciprocal, multiply -- PyTorch only in the reference) in one launch: a position's [dim_in, dim_out]
+ * slab of coefficients stays in the registers of one workgroup through all four operators, each with
+ * the arithmetic of its own entry point (faith_unary_verification, faith_rowsum_verification,
+ * faith_multiply_verification) and every intermediate rounded to fp32 as those store it.  Natural
+ * layout, shapes as faith_relu_verification.  sum_l (out, [length], may be NULL) receives the concrete
+ * lower bound of the sum, which the reference asserts to be >= 1e-12 (Bounds.py:1140).  Outputs must
+ * not alias inputs.  Returns FAITH_ERR_UNSUPPORTED when the slab does not fit (faith_softmax_fits
+ * tells beforehand: dim_out <= 256, or <= 64 when it is no multiple of 4, and dim_in up to
+ * 128 ... 8192 depending on dim_out); the caller then composes the four operators.
+ */
+int faith_softmax_verification(const float *src_lb, const float *src_ub,
+                               const float *src_lw, const float *src_uw,
+                               float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                               float *sum_l,
+                               int length, int dim_in, int dim_out, float epsilon,
+                               int q, int words, void *stream);
+int faith_softmax_fits(int dim_in, int dim_out);
+
+/*
  * Layer normalisation without the variance (Bounds.layer_norm, Bounds.py:1111-1131, mode "no_var",
  * and the first step of mode "standard"): subtract the row mean -- the mean of the UPPER tensor
  * from the lower one and the reverse, as matmul(ones / H).multiply(-1.) gives it -- then scale by

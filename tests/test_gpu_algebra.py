@@ -75,6 +75,90 @@ def test_divide_and_softmax(p):
     assert bool((lo.sum(-1) <= 1 + 1e-4).all()) and bool((hi.sum(-1) >= 1 - 1e-4).all())
 
 
+SOFTMAX_SHAPES = [
+    # B, L, D, H, words
+    (1, 5, 256, 32, 1),      # the common case: 8 threads a slab row, 256 threads, 8 rows each
+    (2, 3, 64, 32, 2),       # fewer rows than the threads hold
+    (1, 4, 100, 16, 4),      # D_in no multiple of the rows in flight
+    (1, 2, 768, 32, 1),      # 1024 threads
+    (1, 3, 48, 128, 3),      # 32 threads a row
+    (1, 2, 40, 256, 1),      # a full wavefront a row
+    (1, 3, 30, 4, 1),        # one thread a row
+    (2, 2, 33, 23, 1),       # H no multiple of 4: one column per thread
+    (1, 2, 300, 7, 2),       # the same with 1024 threads
+    (1, 2, 20, 1, 1),        # softmax of a single score
+]
+
+
+def softmax_case(g, B, L, D, H):
+    return rand_bounds(g, B, L, D, H, sw=0.05, sb=1.0, gap_w=0.005, gap_b=0.1)
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+@pytest.mark.parametrize("p", [1.0, 2.0, INF, 3.0])
+def test_softmax_in_one_launch(shape, p):
+    """faith_softmax_verification against the oracle's composition of exp, sum, reciprocal and multiply."""
+    from faith_amd import ops
+    B, L, D, H, words = shape
+    g = torch.Generator().manual_seed(70)
+    x = softmax_case(g, B, L, D, H)
+    eps = 0.05
+    print(f"[case] softmax {shape} p={p}", flush=True)
+    assert ops.softmax_fits(D, H)
+    out = ops.softmax(*dev(x), p, eps, words, return_sum_bound=True)
+    exp = O.softmax(x, p, eps, words)
+    for name, g_, e in zip(("lw", "lb", "uw", "ub"), out, exp.tensors()):
+        assert close(g_, e, rtol=5e-5, atol=4e-6), f"softmax {name}: {worst(g_, e)}"
+    e_ = O.exp(x, p, eps, words)
+    total = O.LinearBounds(e_.lw.sum(-1, keepdim=True), e_.lb.sum(-1, keepdim=True), e_.uw.sum(-1, keepdim=True),
+                           e_.ub.sum(-1, keepdim=True))
+    l_sum, _ = O.concretize(total, p, eps, words)
+    assert close(out[4], l_sum[..., 0], rtol=2e-5, atol=1e-6), f"lower bound of the sum: {worst(out[4], l_sum[..., 0])}"
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES[:8])
+def test_softmax_in_one_launch_equals_the_four_launches(shape):
+    """Same per-neuron code and the same roundings between the operators: the fused kernel and the
+    composition differ only by the order of the row sum and of the norm reductions."""
+    from faith_amd import ops
+    B, L, D, H, words = shape
+    g = torch.Generator().manual_seed(71)
+    x = dev(softmax_case(g, B, L, D, H))
+    fused = ops.softmax(*x, 2.0, 0.05, words)
+    e = ops.exp(*x, 2.0, 0.05, words)
+    s = ops.rowsum(*e)
+    r = ops.reciprocal(*s, 2.0, 0.05, words)
+    apart = ops.multiply(e, r, 2.0, 0.05, words)
+    for name, a, b in zip(("lw", "lb", "uw", "ub"), fused, apart):
+        assert close(a, b.cpu(), rtol=1e-5, atol=1e-6), f"{name}: {worst(a, b.cpu())}"
+
+
+def test_softmax_that_does_not_fit_is_composed():
+    from faith_amd import ops, _lib
+    assert not ops.softmax_fits(64, 300) and not ops.softmax_fits(64, 66) and not ops.softmax_fits(5000, 32)
+    assert ops.softmax_fits(1024, 32) and ops.softmax_fits(8192, 4) and ops.softmax_fits(128, 256)
+    g = torch.Generator().manual_seed(72)
+    x = softmax_case(g, 1, 2, 8, 300)
+    with pytest.raises(_lib.FaithError) as err:
+        ops.softmax(*dev(x), 2.0, 0.05)
+    assert err.value.code == _lib.ERR_UNSUPPORTED
+    assert_bounds_close(gpu_bounds(x, 2.0, 0.05).softmax(), O.softmax(x, 2.0, 0.05), rtol=5e-5, atol=4e-6,
+                        what="composed softmax")
+
+
+def test_softmax_precondition_is_checked():
+    """A sum whose lower bound falls below 1e-12 fails as the reference's assertion does (Bounds.py:1140).
+    The tangent of exp is taken at most 0.99 above l, which keeps the sum's lower bound positive; only scores
+    so negative that their exponentials vanish get there."""
+    g = torch.Generator().manual_seed(73)
+    x = rand_bounds(g, 1, 2, 16, 8, sw=0.05, sb=1.0, gap_w=0.005, gap_b=0.1)
+    x = O.LinearBounds(x.lw, x.lb - 40.0, x.uw, x.ub - 40.0)
+    with pytest.raises(AssertionError, match="reciprocal"):
+        gpu_bounds(x, 2.0, 0.05).softmax()
+    with pytest.raises(AssertionError):
+        O.softmax(x, 2.0, 0.05)
+
+
 @pytest.mark.parametrize("mode", ["no", "no_var", "standard"])
 @pytest.mark.parametrize("p", [2.0, INF])
 def test_layer_norm(mode, p):
