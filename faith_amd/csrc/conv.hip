@@ -358,22 +358,32 @@ conv_signsplit_k3s1(const ConvArgs g) {
     multiply(buf, 0);
     multiply(buf, 1);
 
+    // ---- epilogue: register r of a block is channel 8*(r/4) + 4*(lane/32) + r%4, pixel lane%32.
+    // Buffer stores into image n of the result (less than 2 GB with 128 channels to spare: the entry
+    // point checks): the channel and the row of a register are a wave-uniform offset, the lane's own
+    // offset (its pixel, its half of the channels) never changes, and channels past C_out fall outside
+    // the window -- no address arithmetic and no predicate on the vector ALU.
     const int ow = ow0 + fi;
     if (ow >= g.Wo) return;
+    const size_t plane = (size_t)g.Ho * g.Wo;
+    const __amdgpu_buffer_rsrc_t wyl = window(g.yl + (size_t)n * g.Co * plane, (size_t)g.Co * plane * 4);
+    const __amdgpu_buffer_rsrc_t wyu = window(g.yu + (size_t)n * g.Co * plane, (size_t)g.Co * plane * 4);
+    const unsigned plane_b = (unsigned)plane * 4u;
+    const unsigned vo = (unsigned)(4 * fh) * plane_b + (unsigned)ow * 4u;
+    const int wvu = __builtin_amdgcn_readfirstlane(wv);        // the wavefront's number as a scalar
+    const int wmu = wvu / 2, wnu = wvu % 2;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-        const int oh = oh0 + wn * 2 + b;
+        const int oh = oh0 + wnu * 2 + b;
         if (oh >= g.Ho) continue;
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
-                if (co < g.Co) {
-                    const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
-                    __builtin_nontemporal_store(cl[a][b][r], &g.yl[o]);
-                    __builtin_nontemporal_store(cu[a][b][r], &g.yu[o]);
-                }
+                const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
+                                    (unsigned)(oh * g.Wo) * 4u;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cu[a][b][r]), wyu, vo, so, 2);
             }
         }
     }
@@ -468,7 +478,8 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
     FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_convolution_verification: grid too large");
     const bool k3s1 = K == 3 && Stride == 1 && CIN % 4 == 0 && faith::aligned(W, 16) &&
                       (long long)CIN * Height * Width * 4 < 0xfffffff0LL &&      // 32-bit byte offsets inside an image
-                      (long long)128 * CIN * 9 * 4 + (long long)CIN * 9 * 4 < 0xfffffff0LL;   // and inside a block of weight rows
+                      (long long)128 * CIN * 9 * 4 + (long long)CIN * 9 * 4 < 0xfffffff0LL &&  // and inside a block of weight rows
+                      ((long long)COUT + 132) * Ho * Wo * 4 < 0x80000000LL;                   // and inside an image of the result
     if (k3s1)
         hipLaunchKernelGGL(conv_signsplit_k3s1, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
     else

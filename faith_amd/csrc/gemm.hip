@@ -239,21 +239,29 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
     }
     compute(buf, []() {});
 
-    // ---- epilogue: register r of a 32x32 block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    // ---- epilogue: register r of a 32x32 block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    // Buffer stores: the row of a register is a wave-uniform offset from the tile's first row, the lane's
+    // own offset (its column, its half of the rows) never changes -- no per-store address arithmetic on the
+    // vector ALU, which would take issue slots from the MFMAs of the co-resident workgroups.  Rows past
+    // the end of C fall outside the window and are dropped by the hardware; a lane whose column does not
+    // exist is sent outside the window.
+    // The window is the tile's own rows (less than 2 GB: the entry point checks), so the offset that sends a
+    // lane outside it cannot wrap around 32 bits when the row offset is added.
+    const size_t c_bytes = (size_t)min(M - m0, BM) * g.N * 4;
+    const __amdgpu_buffer_rsrc_t wcl = window(g.Cl + (size_t)m0 * g.N, c_bytes);
+    const __amdgpu_buffer_rsrc_t wcu = window(g.Cu + (size_t)m0 * g.N, c_bytes);
+    const unsigned row_b = (unsigned)g.N * 4u;
 #pragma unroll
     for (int b = 0; b < MBN; ++b) {
         const int col = n0 + (wn * MBN + b) * 32 + fi;
-        if (col >= g.N) continue;
+        const unsigned vo = col < g.N ? (unsigned)(4 * fh) * row_b + (unsigned)col * 4u : 0x80000000u;
 #pragma unroll
         for (int a = 0; a < MBM; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + (wm * MBM + a) * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
-                if (row < M) {
-                    const size_t o = (size_t)row * g.N + col;
-                    __builtin_nontemporal_store(cl[a][b][r], &g.Cl[o]);
-                    __builtin_nontemporal_store(cu[a][b][r], &g.Cu[o]);
-                }
+                const unsigned so = (unsigned)((wm * MBM + a) * 32 + 8 * (r / 4) + (r % 4)) * row_b;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r]), wcl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cu[a][b][r]), wcu, vo, so, 2);
             }
         }
     }
@@ -499,7 +507,8 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
     GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
-                      faith::aligned(W, 16) && 128LL * dim_out * 4 < 0xffffffffLL;   // 32-bit offsets in a tile
+                      faith::aligned(W, 16) && 128LL * dim_out * 4 < 0xffffffffLL &&  // 32-bit offsets in a tile
+                      128LL * dim_y_out * 4 < 0x80000000LL;                           // and in a tile of the result
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
         // macro-tile, from tuner runs on 1024 ... 245760 rows, K and N 64 ... 1024 (the built-in choice is
