@@ -227,6 +227,12 @@ def bench_config1(args, ops, O, wl, steps, warmup):
     t = gpu_times_ms(lambda: ops.multiply(quad(x), quad(xp), 2.0, c["eps"], c["words"], out=out), 50, 5)
     entries.append(op_entry("extra: multiply(Bounds, Bounds) p=2 [1,128,256,512] words=2", "hbm", t,
                             24 * x["lw"].numel() + 24 * x["lb"].numel()))
+    # softmax over 128 key positions of four heads (the attention scores of configuration 3's shape): the
+    # same bytes as a relaxation of configuration 1 -- one read and one write of lw / uw
+    sx = tuple(v.reshape((4, 128, 256, 128) if v.dim() == 4 else (4, 128, 128)) for v in quad(x))
+    t = gpu_times_ms(lambda: ops.softmax(*sx, 2.0, c["eps"], c["words"]), 50, 5)
+    entries.append(op_entry("extra: softmax p=2 [4,128,256,128] words=2 (exp, sum, reciprocal, product in one launch)", "hbm",
+                            t, nbytes))
     # random contents: a buffer of zeros streams about 15 % faster on this part, which flatters a yardstick
     src = torch.randn(nbytes // 8, device="cuda")
     dst = torch.empty_like(src)

@@ -135,6 +135,17 @@ def test_whole_object_rows():
     check_rows("product", full, lambda r: ops.multiply(sl(x, r), sl(y, r), 2.0, 0.01, 1), picks)
 
 
+def test_softmax_rows():
+    L, D, H = 66000, 128, 256
+    say(f"large softmax [1, {L}, {D}, {H}]")
+    x = big_object((1, L, D, H), (1, L, H), 28, gap_b=0.1)
+    full = ops.softmax(*x, 2.0, 0.01, 2, return_sum_bound=True)
+    for r in rows_to_check(L, D * H):
+        part = ops.softmax(*sl(x, r), 2.0, 0.01, 2, return_sum_bound=True)
+        for i, (f, q) in enumerate(zip(full, part)):
+            same(f[:, r:r + 1], q, f"softmax row {r} output {i}", True)
+
+
 def heads_to_check(n, head_elems):
     return rows_to_check(n, head_elems)
 
