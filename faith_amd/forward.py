@@ -206,12 +206,25 @@ def verify_safety(make_bounds, network, embeddings, index, eps, label, p=2.0, pe
     """VerifierForward.verify_safety (:93-125): True if the label provably survives every
     perturbation of norm <= eps of the embedding at `index`.  A failed precondition inside the
     propagation (reciprocal or sqrt of a bound that reaches zero) counts as not verified, as there."""
+    x = bound_input(make_bounds, embeddings, index, eps, perturbed_words, p)
+    collector = getattr(type(x), "collect_failures", None)
     try:
-        x = bound_input(make_bounds, embeddings, index, eps, perturbed_words, p, network.embedding_norm,
-                        network.layer_norm)
-        x = propagate(x, network)
-        pooled = bound_pooling(x, network.pooler, make_bounds)
-        return bound_classifier(pooled, network.classifier, label)[0]
+        if collector is None:
+            if network.embedding_norm is not None:
+                x = x.layer_norm(network.embedding_norm, network.layer_norm)
+            x = propagate(x, network)
+            pooled = bound_pooling(x, network.pooler, make_bounds)
+            return bound_classifier(pooled, network.classifier, label)[0]
+        # a bound object that can record a failed precondition on the device: nothing waits for the GPU
+        # before the verdict is read
+        with collector(1, embeddings.device) as failed:
+            if network.embedding_norm is not None:
+                x = x.layer_norm(network.embedding_norm, network.layer_norm)
+            x = propagate(x, network)
+            pooled = bound_pooling(x, network.pooler, make_bounds)
+            l, u = _margin(pooled, network.classifier)
+            ok = (l[0, 0, 0] > 0) if label == 0 else (u[0, 0, 0] < 0)
+            return bool(ok & ~failed.mask[0])
     except AssertionError:
         return False
 
