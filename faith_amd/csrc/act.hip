@@ -53,19 +53,25 @@ __device__ __forceinline__ TanhAt tanh_at(float x) {
 // Tangent point search of Bounds.py:1065-1075 (lower = true) and :1082-1092 (lower = false).
 // `anchor` is the far end of the interval (u for the lower line, l for the upper line).
 // v > 0 is decided on (tanh difference) - sech^2(d) * (distance), which has the sign of the
-// reference's quotient form because the distance (+1e-12) is positive.
+// reference's quotient form because the distance (+1e-12) is positive; the line through the point
+// found is then formed in double.
 template <bool LOWER>
 __device__ __forceinline__ Line tanh_tangent_line(float l, float u) {
     const float anchor = LOWER ? u : l;
     const double ta = tanh_at(anchor).th;
+    const float ta32 = (float)ta;
     float d = (LOWER ? l : u) / 2, a = LOWER ? l : 0.f, b = LOWER ? 0.f : u;
     for (int it = 0; it < 10; ++it) {
-        const TanhAt f = tanh_at(d);
+        // the sign test in fp32, as the reference takes it (torch.tanh / cosh on fp32 tensors): the chain of
+        // ten dependent evaluations is what a tile waits for, and in double it is four times as long
+        const float t = __expf(2.f * fminf(fmaxf(d, -20.f), 20.f));
+        const float r = 1.f / (t + 1.f);
+        const float th = (t - 1.f) * r, s2 = 4.f * t * r * r;
         bool go;
         if (LOWER)
-            go = (ta - f.th) - f.s2 * (double)((u - d) + TINY) > 0.0;
+            go = (ta32 - th) - s2 * ((u - d) + TINY) > 0.f;
         else
-            go = (f.th - ta) - f.s2 * (double)((d - l) + TINY) > 0.0;
+            go = (th - ta32) - s2 * ((d - l) + TINY) > 0.f;
         if (LOWER == go) {   // lower & v>0, or upper & v<=0: move right
             a = d;
             d = (d + b) / 2;
