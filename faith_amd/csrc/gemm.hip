@@ -523,6 +523,9 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
         if (tiles(64, 64) <= cus) { tm = 64; tn = 64; }
         else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
         else if (dim_out >= 1024 && tiles(128, 128) >= 16 * cus) { tm = 128; tn = 128; }
+        // many column tiles re-read every block of rows from L2: the large tile halves that (3 - 5 % at
+        // 768 -> 3072 and 512 -> 2048 with 12288 ... 24576 rows) once it fills the machine four times over
+        else if (dim_y_out >= 2048 && tiles(128, 128) >= 8 * cus) { tm = 128; tn = 128; }
         else { tm = 64; tn = 64; }
         const int pick = faith::tune_get(FAITH_TUNE_GEMM_VARIANT);
         switch (pick) {
