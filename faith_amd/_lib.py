@@ -33,6 +33,7 @@ SIGNATURES = {
     "faith_multiply_verification": [_P] * 12 + [_I, _I, _I, _F, _I, _I, _P],
     "faith_affine_verification": [_P] * 5 + [_F] + [_P] * 9 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_rowsum_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
+    "faith_rowmean_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_layer_norm_verification": [_P] * 14 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_softmax_verification": [_P] * 9 + [_I, _I, _I, _F, _I, _I, _P],
     "faith_softmax_fits": [_I, _I],          # a predicate: returns 1 / 0, not a status (call it through lib)

@@ -144,10 +144,9 @@ class Bounds:
             # (residual sum,) mean subtraction, weight and bias in one launch
             return self._like(*ops.layer_norm(*self._c(), weight, bias, other))
         assert layer_norm == "standard"
-        H = self.dim_out
         minus_mu = self._like(*ops.layer_norm(*self._c(), other=other))
-        w_avg = torch.full((H, H), 1.0 / H, device=self.device, dtype=torch.float32)
-        variance = minus_mu.sqr().matmul(w_avg)
+        # the variance: matmul with the H x H matrix of 1 / H (Bounds.py:1116, :1123) is a row mean
+        variance = minus_mu._like(*ops.rowmean(*minus_mu.sqr()._c()))
         normalized = minus_mu.divide(variance.add(1e-12).sqrt())
         return normalized._like(*ops.affine(normalized._c(), scale=weight, shift=bias))
 

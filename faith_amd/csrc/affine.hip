@@ -91,10 +91,11 @@ __device__ __forceinline__ float wave_sum(float s) {
 }
 
 // MODE_SUM: out[r, :] = sum_h src[r, h]                      (Bounds.softmax, Bounds.py:1009-1012)
+// MODE_MEAN: out[r, :] = (sum_h src[r, h]) / H               (matmul with the H x H matrix of 1 / H, Bounds.py:1116, :1123)
 // MODE_NORM: c = src - mean(other side), then c * weight+- (+ bias on the constant rows)
 //            (Bounds.layer_norm without the variance, Bounds.py:1111-1131: the mean is
 //             matmul(ones / H), multiply(-1.) swaps the sides, multiply(weight) splits by sign)
-constexpr int MODE_SUM = 0, MODE_NORM = 1;
+constexpr int MODE_SUM = 0, MODE_NORM = 1, MODE_MEAN = 2;
 constexpr int CACHE = 4;        // row values a lane keeps between the two passes (rows up to 64 * CACHE * VEC)
 
 template <int MODE, int VEC>
@@ -165,6 +166,9 @@ __global__ void __launch_bounds__(256) row_kernel(const Pair w, const Pair b, co
             if (MODE == MODE_SUM) {
                 ol[v] = sl;
                 ou[v] = su;
+            } else if (MODE == MODE_MEAN) {
+                ol[v] = mean_l;
+                ou[v] = mean_u;
             } else {
                 const int col = i * VEC + v;
                 const float c_lo = l[v] - mean_u, c_up = u[v] - mean_l;
@@ -198,7 +202,7 @@ __global__ void __launch_bounds__(256) row_kernel(const Pair w, const Pair b, co
     }
     for (int i = lane + CACHE * WAVE; i < n; i += WAVE) {
         float l[VEC], u[VEC];
-        if (MODE != MODE_SUM) fetch(i, l, u);
+        if (MODE == MODE_NORM) fetch(i, l, u);
         emit(i, l, u);
     }
 }
@@ -307,6 +311,14 @@ extern "C" int faith_rowsum_verification(const float *src_lb, const float *src_u
     FAITH_OBJECT_NOT_NULL();
     const Pair w{src_lw, src_uw, nullptr, nullptr, out_lw, out_uw}, b{src_lb, src_ub, nullptr, nullptr, out_lb, out_ub};
     return launch_rows<MODE_SUM>("faith_rowsum_verification", w, b, nullptr, nullptr, rows_w, rows_b, dim_out, stream);
+}
+
+extern "C" int faith_rowmean_verification(const float *src_lb, const float *src_ub, const float *src_lw,
+                                          const float *src_uw, float *out_lb, float *out_ub, float *out_lw,
+                                          float *out_uw, long long rows_w, long long rows_b, int dim_out, void *stream) {
+    FAITH_OBJECT_NOT_NULL();
+    const Pair w{src_lw, src_uw, nullptr, nullptr, out_lw, out_uw}, b{src_lb, src_ub, nullptr, nullptr, out_lb, out_ub};
+    return launch_rows<MODE_MEAN>("faith_rowmean_verification", w, b, nullptr, nullptr, rows_w, rows_b, dim_out, stream);
 }
 
 extern "C" int faith_layer_norm_verification(const float *src_lb, const float *src_ub, const float *src_lw,

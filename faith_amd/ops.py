@@ -272,6 +272,16 @@ def rowsum(lw, lb, uw, ub):
     return olw, olb, ouw, oub
 
 
+def rowmean(lw, lb, uw, ub):
+    """Mean over the last axis, written to every position of that axis: matmul with the H x H matrix of 1 / H."""
+    rows_w, rows_b, H = _object(lw, lb, uw, ub)
+    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    with _on(lw.device):
+        _lib.call("faith_rowmean_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw),
+                  _ptr(ouw), rows_w, rows_b, H, _stream(lw))
+    return olw, olb, ouw, oub
+
+
 def layer_norm(lw, lb, uw, ub, weight=None, bias=None, other=None):
     """Mean subtraction along the last axis, then per-neuron weight (split by sign) and bias:
     Bounds.layer_norm in mode "no_var"; with weight = bias = None its first step in mode "standard".

@@ -195,6 +195,16 @@ int faith_softmax_verification(const float *src_lb, const float *src_ub,
 int faith_softmax_fits(int dim_in, int dim_out);
 
 /*
+ * out[r, :] = mean over h of src[r, h], written to every h: `matmul(w_avg)` with the dim_out x dim_out
+ * matrix of 1 / dim_out that Bounds.layer_norm uses for the variance (Bounds.py:1116, :1123) -- all weights
+ * positive, so lower stays lower -- without the GEMM.
+ */
+int faith_rowmean_verification(const float *src_lb, const float *src_ub,
+                               const float *src_lw, const float *src_uw,
+                               float *out_lb, float *out_ub, float *out_lw, float *out_uw,
+                               long long rows_w, long long rows_b, int dim_out, void *stream);
+
+/*
  * Layer normalisation without the variance (Bounds.layer_norm, Bounds.py:1111-1131, mode "no_var",
  * and the first step of mode "standard"): subtract the row mean -- the mean of the UPPER tensor
  * from the lower one and the reverse, as matmul(ones / H).multiply(-1.) gives it -- then scale by

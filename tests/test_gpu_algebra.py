@@ -250,6 +250,18 @@ def test_residual_inside_layer_norm_in_place():
         assert torch.equal(a, e)
 
 
+def test_rowmean_is_the_averaging_matmul():
+    """faith_rowmean_verification against Bounds.matmul with the H x H matrix of 1 / H (Bounds.py:1116)."""
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(74)
+    for B, L, D, H in [(2, 3, 7, 64), (1, 5, 3, 100), (1, 2, 3, 1284), (3, 1, 2, 5)]:
+        x = rand_bounds(g, B, L, D, H, ordered=False)
+        got = ops.rowmean(*dev(x))
+        exp = O.linear(x, torch.full((H, H), 1.0 / H))
+        for name, a, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
+            assert close(a, e, rtol=1e-5, atol=2e-6), f"{name}: {worst(a, e)}"
+
+
 def test_shift_shares_the_coefficients():
     """Bounds.add with a tensor returns the same lw / uw tensors (Bounds.py:391-395 does too)."""
     g = torch.Generator().manual_seed(67)
