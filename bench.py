@@ -341,7 +341,7 @@ def bench_config4(args, ops, O, wl):
 
 def bench_layer(args, wl):
     """The path as its caller uses it: one encoder layer + pooler + margin classifier propagated by
-    faith_amd/forward.py (about 60 kernel launches), at a small-BERT size.  Wall clock, host included."""
+    faith_amd/forward.py (about 30 kernel launches), at a small-BERT size.  Wall clock, host included."""
     import time
     import torch
     from types import SimpleNamespace
