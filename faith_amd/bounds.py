@@ -164,6 +164,18 @@ class Bounds:
         bias = getattr(dense, "bias", None)
         return self.matmul(dense.weight.detach(), None if bias is None else bias.detach().contiguous())
 
+    def dense_group(self, layers):
+        """[self.dense(layer) for layer in layers] for up to three layers of one shape, in one launch where that
+        pays (beyond the reference's surface: its `_bound_attention` calls dense three times,
+        VerifierForward.py:202-204)."""
+        layers = list(layers)
+        shapes = {tuple(layer.weight.shape) for layer in layers}
+        if len(layers) > 3 or len(shapes) != 1:
+            return [self.dense(layer) for layer in layers]
+        weights = [layer.weight.detach().contiguous() for layer in layers]
+        biases = [None if getattr(layer, "bias", None) is None else layer.bias.detach().contiguous() for layer in layers]
+        return [self._like(*out) for out in ops.linear_group(*self._c(), weights, biases)]
+
     # ---- Bounds.py:1163-1175
     def relu(self):
         if self.ibp:

@@ -488,6 +488,44 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs
     }
 }
 
+
+// Up to three GEMMs that share their left operand (the query, key and value layers of an attention block:
+// same bound object, three weight matrices of one shape) in ONE launch of the small-tile kernel: at 8192 rows
+// a launch is a single round of tiles, and three launches pay the fill and the drain of the machine three times.
+struct GroupArgs {
+    GemmArgs g;                 // group 0, and the operand shared by all
+    const float *W[2], *bias[2];
+    float *Cl[2], *Cu[2], *Dl[2], *Du[2];   // groups 1 and 2
+    int groups;
+};
+__device__ __forceinline__ GemmArgs group_of(const GroupArgs &G, const int grp) {
+    GemmArgs h = G.g;
+    if (grp > 0) {
+        const int i = grp - 1;
+        h.W = G.W[i];  h.bias = G.bias[i];
+        h.Cl = G.Cl[i];  h.Cu = G.Cu[i];  h.Dl = G.Dl[i];  h.Du = G.Du[i];
+    }
+    return h;
+}
+// b_tiles constant-term tiles per group first (all groups), then `w_tiles` MFMA tiles per group; both are
+// multiples of 8, so a tile keeps the XCD its number within the group gives it.
+template <bool EXACT, int MBM, int MBN>
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_grouped(const GroupArgs G, const int b_tiles, const int w_tiles) {
+    __shared__ __align__(16) float sm[2 * 4 * 64 * 8 * (MBM + MBN)];
+    int pid = blockIdx.x;
+    if (pid < b_tiles * G.groups) {
+        const GemmArgs h = group_of(G, pid / b_tiles);
+        pid %= b_tiles;
+        const int tiles_n = (h.N + 7) / 8;
+        const int m_blk = pid / tiles_n;
+        if (m_blk < (h.Mb + 7) / 8) sliced_tile(h, m_blk, pid % tiles_n, sm);
+        return;
+    }
+    pid -= b_tiles * G.groups;
+    const GemmArgs h = group_of(G, pid / w_tiles);
+    signsplit_gemm_body<EXACT, MBM, MBN>(h, sm, pid % w_tiles);
+}
+
 }  // namespace
 
 extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
@@ -577,4 +615,67 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
         hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)grid), dim3(256), 0, st, g);
     }
     return faith::check_launch("faith_matmul_verification");
+}
+
+extern "C" int faith_matmul_group_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
+                                               int groups, const float *const *W, const float *const *bias,
+                                               float *const *y_lb, float *const *y_ub, float *const *y_lw,
+                                               float *const *y_uw, int batch_size, int length, int dim_in, int dim_out,
+                                               int dim_y_out, void *stream) {
+    FAITH_NOT_NULL(W); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_REQUIRE(groups >= 1 && groups <= 3, FAITH_ERR_SHAPE, "faith_matmul_group_verification: groups=%d must be 1, 2 or 3",
+                  groups);
+    const long long rows = (long long)batch_size * length;
+    const long long mw = rows * dim_in;
+    const long long cus = faith::compute_units();
+    auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * (((long long)dim_y_out + n - 1) / n) * groups; };
+    bool fast = batch_size > 0 && length > 0 && dim_in > 0 && dim_out > 0 && dim_y_out > 0 && mw <= 0x7fffffffLL &&
+                groups > 1 && dim_out % 4 == 0 && x_lb && x_ub && x_lw && x_uw && faith::aligned(x_lb, 4) && faith::aligned(x_ub, 4) &&
+                faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
+                128LL * dim_out * 4 < 0xffffffffLL && 128LL * dim_y_out * 4 < 0x80000000LL &&
+                faith::tune_get(FAITH_TUNE_GEMM_VARIANT) == 0;
+    for (int i = 0; fast && i < groups; ++i)
+        fast = W[i] && y_lb[i] && y_ub[i] && y_lw[i] && y_uw[i] && faith::aligned(W[i], 16) && faith::aligned(y_lb[i], 4) &&
+               faith::aligned(y_ub[i], 4) && faith::aligned(y_lw[i], 4) && faith::aligned(y_uw[i], 4) &&
+               (!bias || faith::aligned(bias[i], 4));
+    // one launch where the small tiles are the choice for the three problems taken together and no single
+    // one of them is a tiny problem (those have a kernel of their own); otherwise one launch each
+    int tm = 0, tn = 0;
+    if (fast) {
+        if (tiles(64, 64) <= cus) { tm = 64; tn = 64; }
+        else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
+        else if (tiles(128, 128) < 8 * cus) { tm = 64; tn = 64; }
+        if (tm == 0 || (dim_out % 32 == 0 && dim_out >= 128 && 4 * tiles(64, 64) / groups <= cus)) fast = false;
+    }
+    if (!fast) {
+        for (int i = 0; i < groups; ++i) {
+            const int rc = faith_matmul_verification(x_lb, x_ub, x_lw, x_uw, W[i], bias ? bias[i] : nullptr, y_lb[i], y_ub[i],
+                                                     y_lw[i], y_uw[i], batch_size, length, dim_in, dim_out, dim_y_out, stream);
+            if (rc != FAITH_OK) return rc;
+        }
+        return FAITH_OK;
+    }
+    GroupArgs G{};
+    G.g = GemmArgs{x_lw, x_uw, x_lb, x_ub, W[0], bias ? bias[0] : nullptr, y_lw[0], y_uw[0], y_lb[0], y_ub[0], (int)mw, (int)rows,
+                   dim_y_out, dim_out};
+    for (int i = 1; i < groups; ++i) {
+        G.W[i - 1] = W[i];  G.bias[i - 1] = bias ? bias[i] : nullptr;
+        G.Cl[i - 1] = y_lw[i];  G.Cu[i - 1] = y_uw[i];  G.Dl[i - 1] = y_lb[i];  G.Du[i - 1] = y_ub[i];
+    }
+    G.groups = groups;
+    const long long mblks = (mw + tm - 1) / tm;
+    const long long w_tiles = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tn - 1) / tn);
+    const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
+    const long long b_tiles = (gridb + XCDS - 1) / XCDS * XCDS;
+    FAITH_REQUIRE((w_tiles + b_tiles) * groups <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_group_verification: grid too large");
+    const dim3 gd((unsigned)((w_tiles + b_tiles) * groups)), bd(NTHREADS);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool exact = dim_out % BK == 0;
+#define FAITH_LAUNCH_GROUPED(MBM, MBN)                                                                                 \
+    if (exact) hipLaunchKernelGGL((signsplit_gemm_grouped<true, MBM, MBN>), gd, bd, 0, st, G, (int)b_tiles, (int)w_tiles); \
+    else hipLaunchKernelGGL((signsplit_gemm_grouped<false, MBM, MBN>), gd, bd, 0, st, G, (int)b_tiles, (int)w_tiles)
+    if (tm == 64) { FAITH_LAUNCH_GROUPED(1, 1); }
+    else { FAITH_LAUNCH_GROUPED(2, 1); }
+#undef FAITH_LAUNCH_GROUPED
+    return faith::check_launch("faith_matmul_group_verification");
 }

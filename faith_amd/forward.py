@@ -101,9 +101,12 @@ def bound_attention(bounds_input, attention):
     """VerifierForward._bound_attention: scores = Q.K^T / sqrt(d), probs = softmax, context = probs.V."""
     heads = attention.self.num_attention_heads
     size = attention.self.attention_head_size
-    query = bounds_input.dense(attention.self.query)
-    key = bounds_input.dense(attention.self.key)
-    value = bounds_input.dense(attention.self.value)
+    if hasattr(bounds_input, "dense_group"):
+        query, key, value = bounds_input.dense_group([attention.self.query, attention.self.key, attention.self.value])
+    else:
+        query = bounds_input.dense(attention.self.query)
+        key = bounds_input.dense(attention.self.key)
+        value = bounds_input.dense(attention.self.value)
     if hasattr(query, "attention_scores"):
         # the HIP kernels address the heads where the dense layers leave them: no permuted copies
         scores = query.attention_scores(key, heads).multiply(1.0 / math.sqrt(size))

@@ -374,6 +374,38 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     return olw, olb, ouw, oub
 
 
+def linear_group(lw, lb, uw, ub, weights, biases=None):
+    """Several affine layers of one shape on the same bound object (query, key, value of an attention block):
+    one launch where that pays, the same results as linear() per layer.  weights: list of [H_out, H];
+    biases: list of [H_out] or None entries, or None.  Returns a list of (lw', lb', uw', ub')."""
+    import ctypes
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    n = len(weights)
+    if not 1 <= n <= 3:
+        raise ValueError(f"{n} layers: between one and three share a launch")
+    N = weights[0].shape[0]
+    biases = list(biases) if biases is not None else [None] * n
+    for i, (W, b) in enumerate(zip(weights, biases)):
+        _check(f"weight {i}", W, (N, H))
+        if b is not None:
+            _check(f"bias {i}", b, (N,))
+    outs = [(torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32),
+             torch.empty(B, L, N, device=lw.device, dtype=torch.float32),
+             torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32),
+             torch.empty(B, L, N, device=lw.device, dtype=torch.float32)) for _ in range(n)]
+    arr = ctypes.c_void_p * n
+    ptrs = lambda ts: arr(*[_ptr(t) for t in ts])
+    a_w, a_b = ptrs(weights), ptrs(biases)
+    a_lb, a_ub = ptrs([o[1] for o in outs]), ptrs([o[3] for o in outs])
+    a_lw, a_uw = ptrs([o[0] for o in outs]), ptrs([o[2] for o in outs])
+    with _on(lw.device):
+        _lib.call("faith_matmul_group_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), n,
+                  ctypes.addressof(a_w), ctypes.addressof(a_b), ctypes.addressof(a_lb), ctypes.addressof(a_ub),
+                  ctypes.addressof(a_lw), ctypes.addressof(a_uw), B, L, D, H, N, _stream(lw))
+    return outs
+
+
 def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
     """McCormick bounds of x . y^T.  x, y: (lw, lb, uw, ub) tuples with
     lw [B, Lx|Ly, D, d]; returns (lw [B, Lx, D, Ly], lb [B, Lx, Ly], uw, ub)."""

@@ -240,6 +240,22 @@ int faith_matmul_verification(const float *x_lb, const float *x_ub,
                               void *stream);
 
 /*
+ * `groups` (1 ... 3) affine layers of one shape applied to the same bound object -- the query, key and value
+ * layers of an attention block (VerifierForward.py:202-204, three `dense` calls in the reference) -- in one
+ * launch where that pays (problems of a single round of small tiles, which would otherwise fill and drain
+ * the machine three times), as `groups` calls of faith_matmul_verification otherwise.  W, bias, y_* are arrays
+ * of `groups` pointers (host memory; bias or any of its entries may be NULL); results equal those of the
+ * separate calls bit for bit.
+ */
+int faith_matmul_group_verification(const float *x_lb, const float *x_ub,
+                                    const float *x_lw, const float *x_uw,
+                                    int groups, const float *const *W, const float *const *bias,
+                                    float *const *y_lb, float *const *y_ub,
+                                    float *const *y_lw, float *const *y_uw,
+                                    int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
+                                    void *stream);
+
+/*
  * McCormick bounds of the attention scores  z[i,j] = sum_k x[i,k] * y[j,k].  Replaces
  * call_dot_product_verification_QK (kernel.cpp:45-51, dot_product_verification.cu:458-496)
  * with the arithmetic of Bounds.ori_dot_product (Bounds.py:710-823).  Natural layout:

@@ -85,6 +85,38 @@ def test_linear_tiny_problems_split_reduction(shape, with_bias):
     check(x, W, bias, "tiny")
 
 
+@pytest.mark.parametrize("shape", [
+    (1, 32, 256, 256, 256, 3),     # attention of the small model: one round of 64 x 64 tiles, taken together
+    (1, 16, 96, 72, 200, 3),       # ragged rows and columns, K % 16 != 0
+    (2, 8, 64, 128, 64, 2),        # two layers
+    (1, 1, 64, 256, 64, 3),        # each problem tiny: separate launches of the split-reduction kernel
+    (1, 64, 512, 64, 512, 3),      # many tiles: separate launches
+    (1, 3, 17, 37, 29, 3),         # K % 4 != 0: separate launches of the any-shape kernel
+    (1, 4, 32, 64, 64, 1),
+])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_linear_group_equals_separate_launches(shape, with_bias):
+    """faith_matmul_group_verification gives what faith_matmul_verification gives per layer, bit for bit."""
+    from faith_amd import ops
+    B, L, D, K, N, n = shape
+    g = torch.Generator().manual_seed(23)
+    x = rand_bounds(g, B, L, D, K, ordered=False, sw=0.5)
+    lw, lb, uw, ub = dev(*x.tensors())
+    Ws = [(torch.randn(N, K, generator=g) / K ** 0.5).cuda() for _ in range(n)]
+    bs = [torch.randn(N, generator=g).cuda() if with_bias and i != 1 else None for i in range(n)]   # one layer without
+    print(f"[case] linear group {shape} bias={with_bias}", flush=True)
+    got = ops.linear_group(lw, lb, uw, ub, Ws, bs)
+    for i in range(n):
+        exp = ops.linear(lw, lb, uw, ub, Ws[i], bs[i])
+        for name, a, e in zip(("lw", "lb", "uw", "ub"), got[i], exp):
+            assert torch.equal(a, e), f"layer {i} {name} differs from the separate launch"
+    if n == 3 and K % 4 == 0:
+        ref = O.linear(x, Ws[2].cpu(), None if bs[2] is None else bs[2].cpu())
+        r64, mag = linear64(x, Ws[2].cpu(), None if bs[2] is None else bs[2].cpu())
+        for name, a, e in zip(("lw", "lb", "uw", "ub"), got[2], ref.tensors()):
+            compare_contraction(name, a, e, r64[name], mag[name])
+
+
 def test_linear_config0_with_concretize():
     from faith_amd import ops
     from faith_amd.workloads import make_config
