@@ -389,26 +389,32 @@ conv_signsplit_k3s1(const ConvArgs g) {
     }
 }
 
-// Direct convolution for the constant terms: 32 neighbouring outputs x 8 channel groups per
-// workgroup; a thread sums its share of the input channels in double (an fp32 x fp32 product is
-// exact there), the 8 partial sums meet in LDS, one rounding, then the bias.
-constexpr int DP = 32, DG = 8;
+// Direct convolution for the constant terms: 32 neighbouring outputs x 4 output channels x 8 groups of
+// input channels per workgroup; a thread sums its share of the input channels in double (an fp32 x fp32
+// product is exact there) for its pixel and four output channels -- the centre and the radius of an input
+// value are formed once and serve all four --, the 8 partial sums meet in LDS, one rounding, then the bias.
+constexpr int DP = 32, DG = 8, DC = 4;
 __global__ void __launch_bounds__(DP * DG) conv_direct(const ConvArgs g) {
-    __shared__ double red[2][DG][DP];
-    const size_t total = (size_t)g.N * g.Co * g.Ho * g.Wo;
+    __shared__ double red[2][DC][DG][DP];
+    const int cob = (g.Co + DC - 1) / DC;                     // blocks of output channels
+    const size_t total = (size_t)g.N * cob * g.Ho * g.Wo;
     const int px = threadIdx.x % DP, cg = threadIdx.x / DP;
     const size_t idx = (size_t)blockIdx.x * DP + px;
     const bool live = idx < total;
     const size_t id = live ? idx : total - 1;
     const int ow = id % g.Wo;
     const int oh = (id / g.Wo) % g.Ho;
-    const int co = (id / ((size_t)g.Wo * g.Ho)) % g.Co;
-    const int n = id / ((size_t)g.Wo * g.Ho * g.Co);
-    double sm = 0.0, sr = 0.0;
+    const int co0 = (int)((id / ((size_t)g.Wo * g.Ho)) % cob) * DC;
+    const int n = id / ((size_t)g.Wo * g.Ho * cob);
+    const int KK = g.K * g.K;
+    double sm[DC], sr[DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) sm[c] = sr[c] = 0.0;
     for (int ci = cg; ci < g.Ci; ci += DG) {
         const float *xl = g.xl + ((size_t)n * g.Ci + ci) * g.H * g.W;
         const float *xu = g.xu + ((size_t)n * g.Ci + ci) * g.H * g.W;
-        const float *w = g.w + ((size_t)co * g.Ci + ci) * g.K * g.K;
+        const float *w = g.w + ((size_t)co0 * g.Ci + ci) * KK;
+        const size_t w_step = (size_t)g.Ci * KK;              // one output channel further
         for (int kh = 0; kh < g.K; ++kh) {
             const int ih = oh * g.S - g.P + kh;
             if (ih < 0 || ih >= g.H) continue;
@@ -417,26 +423,37 @@ __global__ void __launch_bounds__(DP * DG) conv_direct(const ConvArgs g) {
                 if (iw < 0 || iw >= g.W) continue;
                 // w+ a + w- b = w m - |w| r and w+ b + w- a = w m + |w| r with m = (a + b) / 2,
                 // r = (b - a) / 2, both exact in double: two fused multiply-adds per tap instead of four
-                const double wv = w[kh * g.K + kw];
                 const double a = xl[ih * g.W + iw], b = xu[ih * g.W + iw];
-                sm += wv * (0.5 * (a + b));
-                sr += fabs(wv) * (0.5 * (b - a));
+                const double m = 0.5 * (a + b), r = 0.5 * (b - a);
+#pragma unroll
+                for (int c = 0; c < DC; ++c) {
+                    // channels past C_out re-read the last one; their sums are never stored
+                    const double wv = w[(size_t)min(c, g.Co - 1 - co0) * w_step + kh * g.K + kw];
+                    sm[c] += wv * m;
+                    sr[c] += fabs(wv) * r;
+                }
             }
         }
     }
-    red[0][cg][px] = sm - sr;
-    red[1][cg][px] = sm + sr;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        red[0][c][cg][px] = sm[c] - sr[c];
+        red[1][c][cg][px] = sm[c] + sr[c];
+    }
     __syncthreads();
-    if (cg == 0 && live) {
-        double sl = red[0][0][px], su = red[1][0][px];
+    // thread (cg, px) finishes output channel co0 + cg of its pixel (cg < DC)
+    if (cg < DC && live && co0 + cg < g.Co) {
+        double sl = red[0][cg][0][px], su = red[1][cg][0][px];
 #pragma unroll
         for (int c = 1; c < DG; ++c) {
-            sl += red[0][c][px];
-            su += red[1][c][px];
+            sl += red[0][cg][c][px];
+            su += red[1][cg][c][px];
         }
+        const int co = co0 + cg;
         const float add = g.bias ? g.bias[co] : 0.f;
-        g.yl[idx] = (float)sl + add;
-        g.yu[idx] = (float)su + add;
+        const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
+        g.yl[o] = (float)sl + add;
+        g.yu[o] = (float)su + add;
     }
 }
 
@@ -487,7 +504,7 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
 
     // constant terms: batch images through the exact-accumulation kernel, bias added
     ConvArgs gb{x_lb, x_ub, W, bias, y_lb, y_ub, batch_size, CIN, Height, Width, COUT, K, Stride, padding_size, Ho, Wo};
-    const long long nb = (long long)batch_size * COUT * Ho * Wo;
+    const long long nb = (long long)batch_size * ((COUT + DC - 1) / DC) * Ho * Wo;
     hipLaunchKernelGGL(conv_direct, dim3((unsigned)((nb + DP - 1) / DP)), dim3(DP * DG), 0, st, gb);
     return faith::check_launch("faith_convolution_verification");
 }
