@@ -191,7 +191,8 @@ def bound_inputs(make_bounds, embeddings, indices, radii, p=2.0, norm=None, laye
     scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
     w[torch.arange(n, device=dev), torch.as_tensor(indices, device=dev)] = scale[:, None, None] * eye
     b = embeddings[0].unsqueeze(0).expand(n, length, dim).contiguous()
-    bounds = make_bounds(p, 1.0, w, b, w.clone(), b.clone())
+    # lower and upper start out equal and no operator writes into its inputs: one tensor serves both
+    bounds = make_bounds(p, 1.0, w, b, w, b)
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
     return bounds
@@ -297,7 +298,7 @@ class CapturedVerifier:
         self.rows = torch.arange(batch, device=dev)
 
         def body():
-            x = make_bounds(p, 1.0, self.w, self.b, self.w.clone(), self.b.clone())
+            x = make_bounds(p, 1.0, self.w, self.b, self.w, self.b)
             with type(x).collect_failures(batch, dev) as failed:
                 if network.embedding_norm is not None:
                     x = x.layer_norm(network.embedding_norm, network.layer_norm)
