@@ -35,7 +35,7 @@ SIGNATURES = {
     "faith_rowsum_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_rowmean_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_layer_norm_verification": [_P] * 14 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
-    "faith_softmax_verification": [_P] * 9 + [_I, _I, _I, _F, _I, _I, _P],
+    "faith_softmax_verification": [_P] * 9 + [_F, _I, _I, _I, _F, _I, _I, _P],
     "faith_softmax_fits": [_I, _I],          # a predicate: returns 1 / 0, not a status (call it through lib)
     "faith_interval_unary": [_I, _P, _P, _P, _P, ctypes.c_longlong, _P],
     "faith_interval_product": [_P] * 6 + [ctypes.c_longlong, _P],

@@ -117,18 +117,23 @@ class Bounds:
         return self.multiply(W.reciprocal())
 
     # ---- Bounds.py:1005-1014
-    def softmax(self):
+    def softmax(self, scale=None):
+        """scale (beyond the reference's signature): `self.multiply(scale).softmax()` for a positive float --
+        the 1 / sqrt(head size) of the attention scores (VerifierForward.py:232-240) -- in the same launch."""
+        if scale is not None and not (isinstance(scale, (int, float)) and scale > 0):
+            return self.multiply(scale).softmax()
         if not self.ibp and ops.softmax_fits(self.dim_in, self.dim_out):
             # the four operators below on a slab that stays in registers: one launch, one read, one write
             try:
-                out = ops.softmax(*self._c(), self.p, self.eps, self.perturbed_words, return_sum_bound=True)
+                out = ops.softmax(*self._c(), self.p, self.eps, self.perturbed_words, return_sum_bound=True,
+                                  scale=1.0 if scale is None else scale)
             except _lib.FaithError as err:
                 if err.code != _lib.ERR_UNSUPPORTED:         # e.g. tensors that are not 16-byte aligned
                     raise
             else:
                 self._require(out[4], 1e-12, False, "reciprocal of a bound that reaches zero")
                 return self._like(*out[:4])
-        e = self.exp()
+        e = (self if scale is None else self.multiply(scale)).exp()
         return e.divide(self._like(*ops.rowsum(*e._c())))
 
     # ---- Bounds.py:1111-1131

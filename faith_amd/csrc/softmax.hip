@@ -28,6 +28,7 @@ struct SoftmaxArgs {
     float *sum_l;                   // [rows] concrete lower bound of the sum (the reciprocal's precondition), or null
     int rows, D, H, words;
     float eps, qv;
+    float scale;                    // > 0: the object is multiplied by it first (Bounds.multiply with a float)
 };
 
 template <int Q, int VEC, int NTHREADS, int RPT>
@@ -56,6 +57,11 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
         if (col_ok && i * RG + rg < a.D) {
             dl[i].load(a.lw + base + i * row_step);
             du[i].load(a.uw + base + i * row_step);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {        // one rounding, as the separate scaling stores it
+                dl[i].set(v, dl[i].get(v) * a.scale);
+                du[i].set(v, du[i].get(v) * a.scale);
+            }
         } else {
             dl[i].zero();
             du[i].zero();
@@ -144,7 +150,7 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
     __syncthreads();
     const size_t bi = (size_t)r * a.H + tid;         // thread h < H speaks for column h
     if (tid < a.H) {
-        const float xlb = a.lb[bi], xub = a.ub[bi];
+        const float xlb = a.lb[bi] * a.scale, xub = a.ub[bi] * a.scale;
         float l, u, klo, kup, elb, eub;
         interval(part, TH, tid, xlb, xub, l, u);
         relax_point<EXP>(l, u, xlb, xub, klo, kup, elb, eub);
@@ -291,8 +297,8 @@ bool dispatch(const SoftmaxArgs &a, bool vec4, hipStream_t st) {
 
 extern "C" int faith_softmax_verification(const float *src_lb, const float *src_ub, const float *src_lw,
                                           const float *src_uw, float *out_lb, float *out_ub, float *out_lw,
-                                          float *out_uw, float *sum_l, int length, int dim_in, int dim_out,
-                                          float epsilon, int q, int words, void *stream) {
+                                          float *out_uw, float *sum_l, float scale, int length, int dim_in,
+                                          int dim_out, float epsilon, int q, int words, void *stream) {
     FAITH_NOT_NULL(src_lb); FAITH_NOT_NULL(src_ub); FAITH_NOT_NULL(src_lw); FAITH_NOT_NULL(src_uw);
     FAITH_NOT_NULL(out_lb); FAITH_NOT_NULL(out_ub); FAITH_NOT_NULL(out_lw); FAITH_NOT_NULL(out_uw);
     FAITH_ALIGNED4(src_lb); FAITH_ALIGNED4(src_ub); FAITH_ALIGNED4(src_lw); FAITH_ALIGNED4(src_uw);
@@ -303,8 +309,11 @@ extern "C" int faith_softmax_verification(const float *src_lb, const float *src_
                   dim_out);
     FAITH_REQUIRE(words >= 1 && words <= 16 && dim_in % words == 0, FAITH_ERR_SHAPE,
                   "faith_softmax_verification: words=%d must be in 1..16 and divide dim_in=%d", words, dim_in);
+    FAITH_REQUIRE(scale > 0.f, FAITH_ERR_UNSUPPORTED,
+                  "faith_softmax_verification: scale=%g must be positive (a negative factor swaps lower and upper: scale "
+                  "the object with faith_affine_verification first)", (double)scale);
     SoftmaxArgs a{src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, out_uw, sum_l, length, dim_in, dim_out, words,
-                  epsilon, 0.f};
+                  epsilon, 0.f, scale};
     if (!faith::dual_exponent(q, &a.qv)) {
         faith::set_error("faith_softmax_verification: q=%d is neither FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF nor the bits of an "
                          "exponent in (1, inf)", q);

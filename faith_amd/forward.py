@@ -97,8 +97,10 @@ def _unfold_heads(x, heads):
     return x
 
 
-def bound_attention(bounds_input, attention):
-    """VerifierForward._bound_attention: scores = Q.K^T / sqrt(d), probs = softmax, context = probs.V."""
+def bound_attention(bounds_input, attention, want_scores=True):
+    """VerifierForward._bound_attention: scores = Q.K^T / sqrt(d), probs = softmax, context = probs.V.
+    want_scores = False (the layer pipeline, which uses the context only) leaves the scaled scores unmaterialised
+    where the bound object's softmax takes the factor itself; the first element returned is then None."""
     heads = attention.self.num_attention_heads
     size = attention.self.attention_head_size
     if hasattr(bounds_input, "dense_group"):
@@ -109,6 +111,9 @@ def bound_attention(bounds_input, attention):
         value = bounds_input.dense(attention.self.value)
     if hasattr(query, "attention_scores"):
         # the HIP kernels address the heads where the dense layers leave them: no permuted copies
+        if not want_scores:
+            probs = query.attention_scores(key, heads).softmax(scale=1.0 / math.sqrt(size))
+            return None, probs, probs.attention_context(value)
         scores = query.attention_scores(key, heads).multiply(1.0 / math.sqrt(size))
         probs = scores.softmax()
         return scores, probs, probs.attention_context(value)
@@ -129,9 +134,10 @@ def _add_norm(x, residual, normalizer, layer_norm):
     return x.add(residual).layer_norm(normalizer, layer_norm)
 
 
-def bound_layer(bounds_input, layer, layer_norm="no_var", hidden_act="relu"):
-    """VerifierForward._bound_layer: attention block, residual + norm, feed-forward, residual + norm."""
-    scores, probs, attention = bound_attention(bounds_input, layer.attention)
+def bound_layer(bounds_input, layer, layer_norm="no_var", hidden_act="relu", want_scores=False):
+    """VerifierForward._bound_layer: attention block, residual + norm, feed-forward, residual + norm.
+    Returns (scores, probs, output); scores is None unless asked for (see bound_attention)."""
+    scores, probs, attention = bound_attention(bounds_input, layer.attention, want_scores)
     attention = attention.dense(layer.attention.output.dense)
     attention = _add_norm(attention, bounds_input, layer.attention.output.LayerNorm, layer_norm)
     intermediate = attention.dense(layer.intermediate.dense).act(hidden_act)

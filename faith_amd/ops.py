@@ -310,10 +310,11 @@ def softmax_fits(dim_in, dim_out):
     return bool(_lib.lib.faith_softmax_fits(int(dim_in), int(dim_out)))
 
 
-def softmax(lw, lb, uw, ub, p, eps, words=1, return_sum_bound=False):
+def softmax(lw, lb, uw, ub, p, eps, words=1, return_sum_bound=False, scale=1.0):
     """Bounds.softmax over the last axis in one launch: exp, sum, reciprocal and product on a slab that stays
     in registers.  Returns (lw', lb', uw', ub'[, l_sum]); l_sum [B, L] is the concrete lower bound of the sum,
-    which must be >= 1e-12 for the result to mean anything (the reference asserts it).  Raises FaithError
+    which must be >= 1e-12 for the result to mean anything (the reference asserts it).  scale > 0 multiplies
+    the object first (Bounds.multiply with a float), in the same launch.  Raises FaithError
     (FAITH_ERR_UNSUPPORTED) when the slab does not fit: see softmax_fits."""
     B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
@@ -321,7 +322,8 @@ def softmax(lw, lb, uw, ub, p, eps, words=1, return_sum_bound=False):
     l_sum = torch.empty((B, L), device=lw.device, dtype=torch.float32) if return_sum_bound else None
     with _on(lw.device):
         _lib.call("faith_softmax_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub),
-                  _ptr(olw), _ptr(ouw), _ptr(l_sum), B * L, D, H, float(eps), q_code(p), int(words), _stream(lw))
+                  _ptr(olw), _ptr(ouw), _ptr(l_sum), float(scale), B * L, D, H, float(eps), q_code(p), int(words),
+                  _stream(lw))
     if return_sum_bound:
         return olw, olb, ouw, oub, l_sum
     return olw, olb, ouw, oub

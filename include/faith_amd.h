@@ -181,7 +181,9 @@ int faith_rowsum_verification(const float *src_lb, const float *src_ub,
  * the arithmetic of its own entry point (faith_unary_verification, faith_rowsum_verification,
  * faith_multiply_verification) and every intermediate rounded to fp32 as those store it.  Natural
  * layout, shapes as faith_relu_verification.  sum_l (out, [length], may be NULL) receives the concrete
- * lower bound of the sum, which the reference asserts to be >= 1e-12 (Bounds.py:1140).  Outputs must
+ * lower bound of the sum, which the reference asserts to be >= 1e-12 (Bounds.py:1140).  scale > 0 multiplies
+ * the object first (the 1 / sqrt(head size) of the attention scores, VerifierForward.py:232-233; 1 for none),
+ * rounded as faith_affine_verification would store it.  Outputs must
  * not alias inputs.  Returns FAITH_ERR_UNSUPPORTED when the slab does not fit (faith_softmax_fits
  * tells beforehand: dim_out <= 256, or <= 64 when it is no multiple of 4, and dim_in up to
  * 128 ... 8192 depending on dim_out); the caller then composes the four operators.
@@ -189,7 +191,7 @@ int faith_rowsum_verification(const float *src_lb, const float *src_ub,
 int faith_softmax_verification(const float *src_lb, const float *src_ub,
                                const float *src_lw, const float *src_uw,
                                float *out_lb, float *out_ub, float *out_lw, float *out_uw,
-                               float *sum_l,
+                               float *sum_l, float scale,
                                int length, int dim_in, int dim_out, float epsilon,
                                int q, int words, void *stream);
 int faith_softmax_fits(int dim_in, int dim_out);

@@ -133,6 +133,22 @@ def test_softmax_in_one_launch_equals_the_four_launches(shape):
         assert close(a, b.cpu(), rtol=1e-5, atol=1e-6), f"{name}: {worst(a, b.cpu())}"
 
 
+@pytest.mark.parametrize("shape", [(1, 5, 256, 32, 1), (2, 2, 33, 23, 1), (1, 2, 8, 300, 1)])
+def test_softmax_takes_the_scale_of_the_scores(shape):
+    """softmax(scale=s) is multiply(s).softmax(), bit for bit in the one-launch kernel (one rounding of the product
+    either way), composed when the slab does not fit."""
+    B, L, D, H, words = shape
+    g = torch.Generator().manual_seed(75)
+    x = gpu_bounds(softmax_case(g, B, L, D, H), 2.0, 0.05, words)
+    fused, apart = x.softmax(scale=0.17), x.multiply(0.17).softmax()
+    for name in ("lw", "lb", "uw", "ub"):
+        assert torch.equal(getattr(fused, name), getattr(apart, name)), name
+    neg = x.softmax(scale=-0.5)                       # a negative factor swaps the bounds: scaled separately
+    ref = x.multiply(-0.5).softmax()
+    for name in ("lw", "lb", "uw", "ub"):
+        assert torch.equal(getattr(neg, name), getattr(ref, name)), name
+
+
 def test_softmax_that_does_not_fit_is_composed():
     from faith_amd import ops, _lib
     assert not ops.softmax_fits(64, 300) and not ops.softmax_fits(64, 66) and not ops.softmax_fits(5000, 32)
