@@ -224,3 +224,45 @@ def test_convolution_slices():
         same(ouw[:, r:r + 1], puw, f"convolution slice {r} uw", False)
         same(olb, plb, "convolution lb", False)
         same(oub, pub, "convolution ub", False)
+
+
+def test_convolution_with_images_of_a_gigabyte():
+    """One image of the result takes 1.06 GB here: past what the 3 x 3 kernel's 32-bit store offsets are allowed
+    (2 GB with 132 channels to spare), so the general kernel runs.  Rows at the top, in the middle and at the
+    bottom must equal the convolution of the matching crop of the input."""
+    D, C, HW, CO = 2, 4, 1440, 128
+    say(f"large convolution images [1, {D}, {C}, {HW}, {HW}] -> {CO} channels")
+    g = torch.Generator(device="cuda").manual_seed(29)
+    lw = torch.empty((1, D, C, HW, HW), device="cuda").normal_(0, 0.05, generator=g)
+    uw = torch.empty((1, D, C, HW, HW), device="cuda").normal_(0, 0.005, generator=g).abs_().add_(lw)
+    lb = torch.empty((1, C, HW, HW), device="cuda").normal_(0, 1, generator=g)
+    ub = torch.empty((1, C, HW, HW), device="cuda").normal_(0, 0.1, generator=g).abs_().add_(lb)
+    W = torch.empty((CO, C, 3, 3), device="cuda").normal_(0, (2 / (9 * C)) ** 0.5, generator=g)
+    bias = torch.empty((CO,), device="cuda").normal_(0, 0.01, generator=g)
+    olw, olb, ouw, oub = ops.conv2d(lw, lb, uw, ub, W, bias, 1, 1)
+    assert olw.shape == (1, D, CO, HW, HW)
+    for r0 in (0, HW // 2, HW - 24):
+        # input rows r0 - 1 .. r0 + 24 (clipped to the image) give output rows r0 .. r0 + 23 exactly, once the rows
+        # next to a cut that is not the image's edge are left out
+        top, bottom = max(r0 - 1, 0), min(r0 + 25, HW)
+        crop = lambda t: t[..., top:bottom, :].contiguous()
+        plw, plb, puw, pub = ops.conv2d(crop(lw), crop(lb), crop(uw), crop(ub), W, bias, 1, 1)
+        skip = r0 - top                                 # rows of the crop's result above output row r0
+        for full, part, name in ((olw, plw, "lw"), (ouw, puw, "uw"), (olb, plb, "lb"), (oub, pub, "ub")):
+            same(full[..., r0:r0 + 24, :], part[..., skip:skip + 24, :], f"convolution rows {r0}.. {name}", False)
+
+
+def test_linear_with_four_million_outputs():
+    """A row of the result is 16.8 MB: 128 rows of it pass what the MFMA kernel's 32-bit store offsets are
+    allowed, so the any-shape kernel runs.  Column ranges must equal the layer restricted to those outputs."""
+    L, D, K, N = 1, 16, 4, 4_200_000
+    say(f"large linear outputs [1, {L}, {D}, {K}] x [{N}, {K}]")
+    x = big_object((1, L, D, K), (1, L, K), 30)
+    g = torch.Generator(device="cuda").manual_seed(31)
+    W = torch.empty((N, K), device="cuda").normal_(0, 0.5, generator=g)
+    bias = torch.empty((N,), device="cuda").normal_(0, 0.01, generator=g)
+    full = ops.linear(*x, W, bias)
+    for c0 in (0, N // 2, N - 1000):
+        part = ops.linear(*x, W[c0:c0 + 1000].contiguous(), bias[c0:c0 + 1000].contiguous())
+        for i, (f, q) in enumerate(zip(full, part)):
+            same(f[..., c0:c0 + 1000], q, f"linear columns {c0}.. output {i}", False)
