@@ -50,11 +50,11 @@ def rows_to_check(n_rows, row_elems):
     return sorted(r for r in picks if 0 <= r < n_rows)
 
 
-def same(full, part, what, exact):
+def same(full, part, what, exact, atol=1e-6):
     if exact:
         assert torch.equal(full, part), f"{what}: differs from the run on these rows alone"
     else:
-        torch.testing.assert_close(full, part, rtol=1e-5, atol=1e-6, msg=lambda m: f"{what}: {m}")
+        torch.testing.assert_close(full, part, rtol=1e-5, atol=atol, msg=lambda m: f"{what}: {m}")
 
 
 def check_rows(name, full, run_slice, picks, exact=True):
@@ -266,3 +266,27 @@ def test_linear_with_four_million_outputs():
         part = ops.linear(*x, W[c0:c0 + 1000].contiguous(), bias[c0:c0 + 1000].contiguous())
         for i, (f, q) in enumerate(zip(full, part)):
             same(f[..., c0:c0 + 1000], q, f"linear columns {c0}.. output {i}", False)
+
+
+def test_attention_in_place_past_the_tile_limit():
+    """128 positions of an object with its heads side by side would span more than 4 GB here (dim_in 2048, rows of
+    4096), past the 32-bit offsets of the MFMA kernels: the any-shape kernel runs.  Heads must equal the stacked
+    entry points on folded copies."""
+    heads, L, D, size = 16, 8, 2048, 256
+    say(f"attention in place past the tile limit [1, {L}, {D}, {heads} x {size}]")
+    q = big_object((1, L, D, heads * size), (1, L, heads * size), 32, gap_b=0.2)
+    k = big_object((1, L, D, heads * size), (1, L, heads * size), 33, gap_b=0.2)
+    v = big_object((1, L, D, heads * size), (1, L, heads * size), 34, gap_b=0.2)
+
+    def fold(t, h):
+        return t[..., h * size:(h + 1) * size].contiguous()
+    scores = ops.attention_scores(q, k, heads, 2.0, 0.01, 1)              # [heads, L, D, L]
+    context = ops.attention_context(scores, v, 2.0, 0.01, 1)              # [1, L, D, heads * size]
+    # the any-shape kernel sums in double, the MFMA kernels in fp32: the bar allows for the order of 256 cancelling terms
+    for h in (0, heads - 1):
+        part = ops.dot_product_qk(tuple(fold(t, h) for t in q), tuple(fold(t, h) for t in k), 2.0, 0.01, 1)
+        for i, (f, p_) in enumerate(zip(scores, part)):
+            same(f[h:h + 1], p_, f"scores head {h} output {i}", False, atol=1e-5)
+        ctx = ops.dot_product_v(tuple(t[h:h + 1] for t in scores), tuple(fold(t, h) for t in v), 2.0, 0.01, 1)
+        for i, (f, p_) in enumerate(zip(context, ctx)):
+            same(f[..., h * size:(h + 1) * size], p_, f"context head {h} output {i}", False, atol=1e-5)
