@@ -135,6 +135,37 @@ def test_every_gemm_tile_gives_the_same_result(shape):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(3, 256, 64), (2, 600, 128), (1, 1024, 96), (2, 96, 32)])
+def test_every_relaxation_tile_gives_the_same_result(shape):
+    """The tile shapes of the natural-layout relaxation and concretize kernels that the tuner may pick differ in
+    how the norm reduction is split over threads, not in what they compute: every one of them must meet the
+    oracle at the parity bar (they are compared through the same harness as the built-in choice)."""
+    from faith_amd import ops
+    from tests.helpers import rand_bounds, close, worst
+    from tests import test_gpu_act as T_act
+    L, D, H = shape
+    g = torch.Generator().manual_seed(76)
+    x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+    xs = tuple(t.cuda() for t in x.tensors())
+    h = A.Heuristics()
+    for op in ("relu", "tanh"):
+        base = getattr(ops, op)(*xs, 2.0, 0.05, 2, ops.LAYOUT_NATURAL, True)
+        for cand in h.candidates("act", (L, D, H)):
+            print(f"[case] {op} {shape} knobs {cand.knob_dict()}", flush=True)
+            with A.applied(cand.knob_dict()):
+                got = getattr(ops, op)(*xs, 2.0, 0.05, 2, ops.LAYOUT_NATURAL, True)
+                T_act.check(op, x, 2.0, 0.05, 2, "natural")
+            for a, b in zip(got, base):
+                assert close(a, b, rtol=1e-5, atol=1e-6), f"{op} {cand.knob_dict()}: {worst(a, b)}"
+    base = ops.concretize(*xs, 2.0, 0.05, 2)
+    for cand in h.candidates("concretize", (L, D, H)):
+        with A.applied(cand.knob_dict()):
+            got = ops.concretize(*xs, 2.0, 0.05, 2)
+        for a, b in zip(got, base):
+            assert close(a, b, rtol=1e-5, atol=1e-6), f"concretize {cand.knob_dict()}: {worst(a, b)}"
+
+
+@pytest.mark.gpu
 def test_dot_variants_agree_and_tuning_is_never_slower_than_the_default():
     from faith_amd import ops
     from tests.helpers import rand_bounds, close
