@@ -118,3 +118,30 @@ def test_binding_argument_types_match_the_header(lib):
                 raise AssertionError(f"{name}: cannot classify parameter {prm!r}")
         got = [kinds[t] for t in lib.SIGNATURES[name]]
         assert got == want, f"{name}: header {want} vs binding {got}"
+
+
+def test_header_and_library_serve_a_plain_c_caller(tmp_path, lib):
+    """The boundary is a C ABI: a C99 program that includes the header and links the library calls it
+    (version, argument validation -- nothing is launched, so no GPU is needed)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "caller.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "faith_amd.h"\n'
+        "int main(void) {\n"
+        "    float buf[16];\n"
+        "    if (faith_version() <= 0) return 1;\n"
+        "    if (faith_concretize(NULL, buf, buf, buf, buf, buf, 1, 4, 4, 0.1f, FAITH_Q_2, 1, FAITH_LAYOUT_NATURAL, NULL) != FAITH_ERR_NULL) return 2;\n"
+        "    if (strstr(faith_last_error(), \"NULL\") == NULL) return 3;\n"
+        "    if (faith_concretize(buf, buf, buf, buf, buf, buf, 0, 4, 4, 0.1f, FAITH_Q_2, 1, FAITH_LAYOUT_NATURAL, NULL) != FAITH_ERR_SHAPE) return 4;\n"
+        "    if (faith_softmax_fits(256, 32) != 1 || faith_softmax_fits(64, 300) != 0) return 5;\n"
+        '    printf("ok %d\\n", faith_version());\n'
+        "    return 0;\n}\n")
+    exe = tmp_path / "caller"
+    libdir = os.path.dirname(lib.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", f"-I{os.path.join(ROOT, 'include')}", str(src),
+                    f"-L{libdir}", "-lfaith_amd", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.startswith("ok"), (out.returncode, out.stdout, out.stderr)
