@@ -467,6 +467,73 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     for (int c = 0; c < PIECES; ++c) store_piece(c, ol, ou);
 }
 
+// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns an 8 x 8 tile of
+// (i, j) of one head; four groups of 64 threads each take a quarter of every 64-wide chunk of the
+// reduction, the seven [8 x chunk] operand rows are staged in LDS, sums are kept in double and the
+// four partial sums meet in LDS at the end.
+constexpr int BT_T = 8, BT_K = 64, BT_S = 4;
+constexpr int BT_LDS = 7 * BT_T * (BT_K + 1) + 2 * 2 * BT_S * BT_T * BT_T;      // floats of LDS a tile needs
+template <bool VP>
+__device__ __forceinline__ void dot_b_tile(const DotArgs &g, int pid, float *smem) {
+    float(*sx)[BT_T][BT_K + 1] = reinterpret_cast<float(*)[BT_T][BT_K + 1]>(smem);                             // b (= l_x), xlb, xub
+    float(*sy)[BT_T][BT_K + 1] = reinterpret_cast<float(*)[BT_T][BT_K + 1]>(smem + 3 * BT_T * (BT_K + 1));    // a_l, a_u, ylb, yub
+    double(*red)[BT_S][BT_T * BT_T] = reinterpret_cast<double(*)[BT_S][BT_T * BT_T]>(smem + 7 * BT_T * (BT_K + 1));   // 3640 floats in: 8-byte aligned
+    const int ti = (g.Lx + BT_T - 1) / BT_T, tj = (g.Ly + BT_T - 1) / BT_T;
+    const int j0 = (pid % tj) * BT_T;  pid /= tj;
+    const int i0 = (pid % ti) * BT_T;  pid /= ti;
+    const int t = pid;
+    const int ks = threadIdx.x / 64, o = threadIdx.x % 64;
+    const int tx = o % BT_T, ty = o / BT_T;                     // output (i0 + ty, j0 + tx)
+    double sl = 0.0, su = 0.0;
+    for (int k0 = 0; k0 < g.d; k0 += BT_K) {
+        for (int e = threadIdx.x; e < BT_T * BT_K; e += 256) {
+            // x rows are contiguous along k; so are y rows on the scores path, while on the context path
+            // y is contiguous along j
+            const int r = e / BT_K, k = e % BT_K;
+            const bool xin = k0 + k < g.d && i0 + r < g.Lx;
+            const size_t xo = b_base(g.ox, t, g.Lx) + (size_t)(i0 + r) * g.ox.pitch + k0 + k;
+            sx[0][r][k] = xin ? g.x_l[xo] : 0.f;
+            sx[1][r][k] = xin ? g.xlb[xo] : 0.f;
+            sx[2][r][k] = xin ? g.xub[xo] : 0.f;
+            const int ry = VP ? e % BT_T : r, ky = VP ? e / BT_T : k;
+            const bool yin = k0 + ky < g.d && j0 + ry < g.Ly;
+            const size_t yo = b_base(g.oy, t, VP ? g.d : g.Ly) + (VP ? (size_t)(k0 + ky) * g.oy.pitch + j0 + ry : (size_t)(j0 + ry) * g.oy.pitch + k0 + ky);
+            sy[0][ry][ky] = yin ? g.y_l[yo] : 0.f;
+            sy[1][ry][ky] = yin ? g.y_u[yo] : 0.f;
+            sy[2][ry][ky] = yin ? g.ylb[yo] : 0.f;
+            sy[3][ry][ky] = yin ? g.yub[yo] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int kk = 0; kk < BT_K / BT_S; ++kk) {
+            const int k = ks * (BT_K / BT_S) + kk;
+            const double bt = sx[0][ty][k], xlb = sx[1][ty][k], xub = sx[2][ty][k];
+            const double al = sy[0][tx][k], au = sy[1][tx][k], ylb = sy[2][tx][k], yub = sy[3][tx][k];
+            const double bp = bt > 0 ? bt : 0, bn = bt < 0 ? bt : 0;
+            sl += -al * bt + (al > 0 ? al * xlb : al * xub) + bp * ylb + bn * yub;
+            su += -au * bt + (au > 0 ? au * xub : au * xlb) + bp * yub + bn * ylb;
+        }
+        __syncthreads();
+    }
+    red[0][ks][o] = sl;
+    red[1][ks][o] = su;
+    __syncthreads();
+    if (ks == 0) {
+        const int i = i0 + ty, j = j0 + tx;
+        if (i < g.Lx && j < g.Ly) {
+            const size_t z = b_base(g.oz, t, g.Lx) + (size_t)i * g.oz.pitch + j;
+            g.zlb[z] = (float)(red[0][0][o] + red[0][1][o] + red[0][2][o] + red[0][3][o]);
+            g.zub[z] = (float)(red[1][0][o] + red[1][1][o] + red[1][2][o] + red[1][3][o]);
+        }
+    }
+}
+
+template <bool VP>
+__global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
+    __shared__ __align__(16) float sm[BT_LDS];
+    dot_b_tile<VP>(g, blockIdx.x, sm);
+}
+
 // Short sequences (Lx, Ly <= 64, d <= 80): the 128 x 64 tile above would be mostly padding, so here
 // a WAVEFRONT owns one 32 x 32 block of z for one perturbation coordinate m (one MFMA block for
 // z_lw, one for z_uw).  The four wavefronts of a workgroup share the (head, i-block, j-block): the
@@ -475,9 +542,16 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
 // fragments straight from global memory in MFMA layout (rows of 32 bytes per lane and K-step: poor
 // coalescing, but these problems are a few megabytes and latency is what counts).
 constexpr int SB = 32;                         // block edge
+// The workgroups from `w_tiles` on take the 8 x 8 tiles of the constant terms instead (short chains of double
+// arithmetic that run beside the MFMA blocks rather than in a launch of their own).  They come last: the
+// MFMA workgroups that share rows of x count on starting together.
 template <bool VP>
-__global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mpw, const int heads_first) {
-    extern __shared__ float sh[];              // six operands, each d/8 swizzled [32 x 8] pieces
+__global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mpw, const int heads_first, const int w_tiles) {
+    extern __shared__ __align__(16) float sh[];   // six operands, each d/8 swizzled [32 x 8] pieces (or a constant-term tile)
+    if ((int)blockIdx.x >= w_tiles) {
+        dot_b_tile<VP>(g, blockIdx.x - w_tiles, sh);
+        return;
+    }
     const int d = g.d, nq = d / 8;
     const int OP = SB * d;                     // floats per operand
     float *s_bp = sh, *s_bn = sh + OP, *s_alp = sh + 2 * OP, *s_aln = sh + 3 * OP, *s_aup = sh + 4 * OP, *s_aun = sh + 5 * OP;
@@ -651,67 +725,6 @@ __global__ void __launch_bounds__(256) dot_w_simple(const DotArgs g) {
     }
 }
 
-// Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns an 8 x 8 tile of
-// (i, j) of one head; four groups of 64 threads each take a quarter of every 64-wide chunk of the
-// reduction, the seven [8 x chunk] operand rows are staged in LDS, sums are kept in double and the
-// four partial sums meet in LDS at the end.
-constexpr int BT_T = 8, BT_K = 64, BT_S = 4;
-template <bool VP>
-__global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
-    __shared__ float sx[3][BT_T][BT_K + 1];     // b (= l_x), xlb, xub
-    __shared__ float sy[4][BT_T][BT_K + 1];     // a_l, a_u, ylb, yub
-    __shared__ double red[2][BT_S][BT_T * BT_T];
-    const int ti = (g.Lx + BT_T - 1) / BT_T, tj = (g.Ly + BT_T - 1) / BT_T;
-    int pid = blockIdx.x;
-    const int j0 = (pid % tj) * BT_T;  pid /= tj;
-    const int i0 = (pid % ti) * BT_T;  pid /= ti;
-    const int t = pid;
-    const int ks = threadIdx.x / 64, o = threadIdx.x % 64;
-    const int tx = o % BT_T, ty = o / BT_T;                     // output (i0 + ty, j0 + tx)
-    double sl = 0.0, su = 0.0;
-    for (int k0 = 0; k0 < g.d; k0 += BT_K) {
-        for (int e = threadIdx.x; e < BT_T * BT_K; e += 256) {
-            // x rows are contiguous along k; so are y rows on the scores path, while on the context path
-            // y is contiguous along j
-            const int r = e / BT_K, k = e % BT_K;
-            const bool xin = k0 + k < g.d && i0 + r < g.Lx;
-            const size_t xo = b_base(g.ox, t, g.Lx) + (size_t)(i0 + r) * g.ox.pitch + k0 + k;
-            sx[0][r][k] = xin ? g.x_l[xo] : 0.f;
-            sx[1][r][k] = xin ? g.xlb[xo] : 0.f;
-            sx[2][r][k] = xin ? g.xub[xo] : 0.f;
-            const int ry = VP ? e % BT_T : r, ky = VP ? e / BT_T : k;
-            const bool yin = k0 + ky < g.d && j0 + ry < g.Ly;
-            const size_t yo = b_base(g.oy, t, VP ? g.d : g.Ly) + (VP ? (size_t)(k0 + ky) * g.oy.pitch + j0 + ry : (size_t)(j0 + ry) * g.oy.pitch + k0 + ky);
-            sy[0][ry][ky] = yin ? g.y_l[yo] : 0.f;
-            sy[1][ry][ky] = yin ? g.y_u[yo] : 0.f;
-            sy[2][ry][ky] = yin ? g.ylb[yo] : 0.f;
-            sy[3][ry][ky] = yin ? g.yub[yo] : 0.f;
-        }
-        __syncthreads();
-#pragma unroll 4
-        for (int kk = 0; kk < BT_K / BT_S; ++kk) {
-            const int k = ks * (BT_K / BT_S) + kk;
-            const double bt = sx[0][ty][k], xlb = sx[1][ty][k], xub = sx[2][ty][k];
-            const double al = sy[0][tx][k], au = sy[1][tx][k], ylb = sy[2][tx][k], yub = sy[3][tx][k];
-            const double bp = bt > 0 ? bt : 0, bn = bt < 0 ? bt : 0;
-            sl += -al * bt + (al > 0 ? al * xlb : al * xub) + bp * ylb + bn * yub;
-            su += -au * bt + (au > 0 ? au * xub : au * xlb) + bp * yub + bn * ylb;
-        }
-        __syncthreads();
-    }
-    red[0][ks][o] = sl;
-    red[1][ks][o] = su;
-    __syncthreads();
-    if (ks == 0) {
-        const int i = i0 + ty, j = j0 + tx;
-        if (i < g.Lx && j < g.Ly) {
-            const size_t z = b_base(g.oz, t, g.Lx) + (size_t)i * g.oz.pitch + j;
-            g.zlb[z] = (float)(red[0][0][o] + red[0][1][o] + red[0][2][o] + red[0][3][o]);
-            g.zub[z] = (float)(red[1][0][o] + red[1][1][o] + red[1][2][o] + red[1][3][o]);
-        }
-    }
-}
-
 // dim_in == 1: the reference switches to plain interval arithmetic on the constant terms and
 // returns zero coefficients (Bounds.py:711-721).
 template <bool VP>
@@ -791,8 +804,9 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
                                     cx_h, cy_h, epsilon, q, words, stream);
     if (rc != FAITH_OK) return rc;
 
-    hipLaunchKernelGGL(dot_b<VP>, dim3((unsigned)((long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T))),
-                       dim3(256), 0, st, g);
+    const long long b_tiles = (long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T);
+    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    auto constant_terms = [&]() { hipLaunchKernelGGL(dot_b<VP>, dim3((unsigned)b_tiles), dim3(256), 0, st, g); };
 
     const int max_pitch = g.ox.pitch > g.oy.pitch ? (g.ox.pitch > g.oz.pitch ? g.ox.pitch : g.oz.pitch) : (g.oy.pitch > g.oz.pitch ? g.oy.pitch : g.oz.pitch);
     const bool fast = (d % 4 == 0) && (!VP || Ly % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
@@ -825,10 +839,17 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
         const int forced = faith::tune_get(FAITH_TUNE_DOT_COORDS);
         if (forced >= 1 && forced <= 16) mpw = forced;
         const long long grid = blocks * ((D + 4 * mpw - 1) / (4 * mpw));
-        FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
-        hipLaunchKernelGGL(dot_w_small<VP>, dim3((unsigned)grid), dim3(256), (size_t)6 * SB * d * sizeof(float), st, g,
-                           (int)mpw, x_sbs ? 1 : 0);
+        FAITH_REQUIRE(grid + b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+        // the constant-term tiles are the trailing workgroups of the same launch while the machine is not
+        // filled many times over (one small problem: 30.7 -> 25.1 us); behind a long queue of MFMA workgroups
+        // they would only lengthen the tail (batch of 30: 554 -> 567 us), so there they keep their own launch
+        const bool fold = blocks * ((D + 3) / 4) <= 16 * cus;      // wavefront-coordinates of work, whatever their grouping
+        if (!fold) constant_terms();
+        const size_t lds = (size_t)(6 * SB * d > BT_LDS ? 6 * SB * d : BT_LDS) * sizeof(float);
+        hipLaunchKernelGGL(dot_w_small<VP>, dim3((unsigned)(grid + (fold ? b_tiles : 0))), dim3(256), lds, st, g, (int)mpw,
+                           x_sbs ? 1 : 0, (int)grid);
     } else if (fast) {
+        constant_terms();
         const long long tiles = (long long)B * D * ((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ);
         FAITH_REQUIRE(tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: too many tiles", who);
         const long long resident = 2LL * faith::compute_units();      // 56 KB of LDS each: two per CU
@@ -845,6 +866,7 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
         else
             hipLaunchKernelGGL((dot_w<VP, false>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
     } else {
+        constant_terms();
         const long long blocks = (nw + 255) / 256;
         hipLaunchKernelGGL(dot_w_simple<VP>, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, st, g);
     }
