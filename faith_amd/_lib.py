@@ -77,8 +77,11 @@ def _load():
 lib = _load()
 
 
+_ENTRY = {name: getattr(lib, name) for name in SIGNATURES}
+
+
 def call(name, *args):
     """Invoke an entry point; raise FaithError on a non-zero status."""
-    rc = getattr(lib, name)(*args)
-    if rc != OK:
+    rc = _ENTRY[name](*args)
+    if rc:
         raise FaithError(name, rc, lib.faith_last_error().decode())

@@ -38,7 +38,7 @@ def _check(name, t, shape=None):
         raise TypeError(f"{name}: must be float32, got {t.dtype}")
     if not t.is_contiguous():
         raise ValueError(f"{name}: must be contiguous")
-    if shape is not None and tuple(t.shape) != tuple(shape):
+    if shape is not None and t.shape != shape and tuple(t.shape) != tuple(shape):      # torch.Size is a tuple
         raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
     return t
 
