@@ -545,15 +545,22 @@ constexpr int SB = 32;                         // block edge
 // The workgroups from `w_tiles` on take the 8 x 8 tiles of the constant terms instead (short chains of double
 // arithmetic that run beside the MFMA blocks rather than in a launch of their own).  They come last: the
 // MFMA workgroups that share rows of x count on starting together.
-template <bool VP>
+//
+// RAGGED (context path only): the reduction length -- the number of key positions -- is any number, as the
+// length of a sentence is.  The staged operands are zero beyond it, up to the next multiple of 8, so whatever
+// the fragments of x and y hold there (the start of the next row, or the zero that reads past the end of a
+// tensor return) does not count; the rows of x then start on any 4-byte boundary and are read 4 bytes at a time.
+template <bool VP, bool RAGGED = false>
 __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mpw, const int heads_first, const int w_tiles) {
+    static_assert(VP || !RAGGED, "a ragged reduction exists on the context path only");
     extern __shared__ __align__(16) float sh[];   // six operands, each d/8 swizzled [32 x 8] pieces (or a constant-term tile)
     if ((int)blockIdx.x >= w_tiles) {
         dot_b_tile<VP>(g, blockIdx.x - w_tiles, sh);
         return;
     }
-    const int d = g.d, nq = d / 8;
-    const int OP = SB * d;                     // floats per operand
+    const int d = g.d;
+    const int dp = RAGGED ? (d + 7) / 8 * 8 : d, nq = dp / 8;      // the reduction as the MFMAs walk it
+    const int OP = SB * dp;                    // floats per operand
     float *s_bp = sh, *s_bn = sh + OP, *s_alp = sh + 2 * OP, *s_aln = sh + 3 * OP, *s_aup = sh + 4 * OP, *s_aun = sh + 5 * OP;
 
     const int nib = (g.Lx + SB - 1) / SB, njb = (g.Ly + SB - 1) / SB;
@@ -578,7 +585,16 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
     const size_t xw0 = w_base(g.ox, t, g.Lx, g.D), yw0 = w_base(g.oy, t, y_len, g.D), zw0 = w_base(g.oz, t, g.Lx, g.D);
 
     // ---- operands shared by every m: b = l_x rows i0.., a_l / a_u rows (columns of z) j0..
-    for (int e = tid; e < SB * d / 4; e += 256) {
+    if (RAGGED) {
+        for (int e = tid; e < SB * dp; e += 256) {
+            const int row = e / dp, k = e % dp;
+            const float bt = k < d ? g.x_l[xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + k] : 0.f;
+            const int dst = (k / 8) * (SB * 8) + swz(row, (k % 8) / 4) + k % 4;
+            s_bp[dst] = pos1(bt);
+            s_bn[dst] = neg1(bt);
+        }
+    }
+    for (int e = tid; !RAGGED && e < SB * d / 4; e += 256) {
         const int row = e / (d / 4), c4 = e % (d / 4);
         const int dst = (c4 / 2) * (SB * 8) + swz(row, c4 % 2);
         const float4 bt = *reinterpret_cast<const float4 *>(g.x_l + xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + c4 * 4);
@@ -595,10 +611,10 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
     }
     if (VP) {
         // a[t, k, j]: j is the contiguous axis
-        for (int e = tid; e < SB * d; e += 256) {
+        for (int e = tid; e < SB * dp; e += 256) {
             const int j = e % SB, k = e / SB;
-            const size_t o = yb0 + (size_t)k * g.oy.pitch + min(j0 + j, g.Ly - 1);
-            const float al = g.y_l[o], au = g.y_u[o];
+            const size_t o = yb0 + (size_t)min(k, d - 1) * g.oy.pitch + min(j0 + j, g.Ly - 1);
+            const float al = k < d ? g.y_l[o] : 0.f, au = k < d ? g.y_u[o] : 0.f;
             const int dst = (k / 8) * (SB * 8) + swz(j, (k % 8) / 4) + k % 4;
             s_alp[dst] = pos1(al);
             s_aln[dst] = neg1(al);
@@ -634,8 +650,19 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
             for (int qq = 0; qq < 4; ++qq) {
                 if (q0 + qq < nq) {
                     const unsigned k = (q0 + qq) * 8;
-                    xl[qq] = ld4(wxl, vx, k * 4u);
-                    xu[qq] = ld4(wxu, vx, k * 4u);
+                    if (RAGGED) {
+                        float xv[2][4];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            xv[0][c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wxl, vx, (k + c) * 4u, 0));
+                            xv[1][c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wxu, vx, (k + c) * 4u, 0));
+                        }
+                        xl[qq] = make_float4(xv[0][0], xv[0][1], xv[0][2], xv[0][3]);
+                        xu[qq] = make_float4(xv[1][0], xv[1][1], xv[1][2], xv[1][3]);
+                    } else {
+                        xl[qq] = ld4(wxl, vx, k * 4u);
+                        xu[qq] = ld4(wxu, vx, k * 4u);
+                    }
                     if (VP) {
                         // y[t, k, m, j]: four keys, one column per lane
                         float yv[2][4];
@@ -822,7 +849,14 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     const int pick = faith::tune_get(FAITH_TUNE_DOT_VARIANT);
     const long long pad_small = (long long)((Lx + SB - 1) / SB) * ((Ly + SB - 1) / SB) * SB * SB;
     const long long pad_tiled = (long long)((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ) * TI * TJ;
-    const bool small = small_ok && (pick == 2 || (pick != 1 && 100 * pad_small <= 85 * pad_tiled));
+    // Context path with a reduction length (key positions) that is no multiple of 8 -- sentences come in every
+    // length: the per-wavefront kernel's ragged mode reads 4 bytes at a time and needs no alignment; it takes
+    // such problems whenever they are short, and all of them when the tiled kernel cannot (length % 4 != 0),
+    // where the only alternative is the any-shape kernel (L = 30: 101 us against 22 us).
+    const bool ragged_ok = VP && d % 8 != 0 && d <= 80 && (long long)TI * D * max_pitch * 4 < 0xffffffffLL &&
+                           (long long)d * D * g.oy.pitch * 4 < 0xffffffffLL;
+    const bool small = (small_ok && (pick == 2 || (pick != 1 && 100 * pad_small <= 85 * pad_tiled))) ||
+                       (ragged_ok && (pick == 2 || !fast || (pick != 1 && 100 * pad_small <= 85 * pad_tiled)));
     if (small) {
         // one 32 x 32 block per wavefront and perturbation coordinate.  Coordinates per wavefront: the
         // count that leaves the busiest CU the least to do -- its share of the workgroups, each costing
@@ -845,9 +879,17 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
         // they would only lengthen the tail (batch of 30: 554 -> 567 us), so there they keep their own launch
         const bool fold = blocks * ((D + 3) / 4) <= 16 * cus;      // wavefront-coordinates of work, whatever their grouping
         if (!fold) constant_terms();
-        const size_t lds = (size_t)(6 * SB * d > BT_LDS ? 6 * SB * d : BT_LDS) * sizeof(float);
-        hipLaunchKernelGGL(dot_w_small<VP>, dim3((unsigned)(grid + (fold ? b_tiles : 0))), dim3(256), lds, st, g, (int)mpw,
-                           x_sbs ? 1 : 0, (int)grid);
+        const int dp = (d + 7) / 8 * 8;
+        const size_t lds = (size_t)(6 * SB * dp > BT_LDS ? 6 * SB * dp : BT_LDS) * sizeof(float);
+        const dim3 gd((unsigned)(grid + (fold ? b_tiles : 0)));
+        if constexpr (VP) {
+            if (d % 8 != 0)
+                hipLaunchKernelGGL((dot_w_small<true, true>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
+            else
+                hipLaunchKernelGGL((dot_w_small<true, false>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
+        } else {
+            hipLaunchKernelGGL((dot_w_small<false, false>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
+        }
     } else if (fast) {
         constant_terms();
         const long long tiles = (long long)B * D * ((Lx + TI - 1) / TI) * ((Ly + TJ - 1) / TJ);

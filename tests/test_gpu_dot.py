@@ -198,6 +198,21 @@ def test_context_exact_shapes(shape):
     check_v(probs, value, 2.0, 0.05, 1, "exact")
 
 
+@pytest.mark.parametrize("shape", [
+    # B, queries, keys, D, value width: any number of key positions (the length of a sentence) on the per-wavefront
+    # kernel's ragged mode -- staged operands zero beyond the last key, x read 4 bytes at a time
+    (4, 30, 30, 64, 64), (2, 23, 23, 32, 64), (1, 36, 36, 16, 32), (1, 40, 77, 8, 16), (2, 33, 20, 24, 64),
+    (1, 7, 1, 8, 8), (1, 31, 31, 16, 10), (1, 130, 30, 4, 64),
+])
+@pytest.mark.parametrize("words", [1, 2])
+def test_context_any_number_of_keys(shape, words):
+    B, Lq, Lk, D, dv = shape
+    g = torch.Generator().manual_seed(37)
+    probs = rand_bounds(g, B, Lq, D, Lk, ordered=False, sw=0.2, sb=0.5)
+    value = rand_bounds(g, B, Lk, D, dv, ordered=False, sw=0.3, sb=1.0)
+    check_v(probs, value, 2.0, 0.05, words, "any number of keys")
+
+
 def test_context_rectangular_and_two_words():
     """More keys than queries, two perturbed words."""
     g = torch.Generator().manual_seed(34)
@@ -313,7 +328,9 @@ def test_attention_scores_reads_the_heads_in_place(shape, p):
     (1, 2, 130, 72, 12, 20),       # ragged
     (1, 4, 32, 32, 64, 16),        # short sequences
     (3, 2, 24, 16, 16, 24),        # short, three batch elements
-    (2, 3, 6, 6, 4, 10),           # any-shape kernel
+    (2, 3, 6, 6, 4, 10),           # six keys: ragged reduction
+    (1, 4, 30, 30, 64, 64),        # a sentence of 30 tokens
+    (2, 2, 23, 23, 16, 32),
     (2, 2, 4, 4, 1, 8),            # interval shortcut
 ])
 @pytest.mark.parametrize("p", [2.0, INF])
