@@ -652,6 +652,20 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         // where a row of neurons is 64 KB or more (image-shaped bounds: every row of a tile then lies
         // on another page), where four-wavefront workgroups are 12 % ahead (6.2 against 5.4 TB/s at
         // configuration 4)
+        if (!vec4 && a.rows2 > 0) {
+            // two objects of which at least one cannot be read 16 bytes at a time (a row of attention
+            // probabilities is as long as the sentence): a launch each, so that the other keeps its fast path
+            ActArgs first = a, second = a;
+            first.rows2 = 0;  first.H2 = 0;
+            first.lb2 = first.ub2 = first.lw2 = first.uw2 = nullptr;  first.l2 = first.u2 = nullptr;
+            second.lb = a.lb2;  second.ub = a.ub2;  second.lw = a.lw2;  second.uw = a.uw2;
+            second.l = a.l2;  second.u = a.u2;  second.rows = a.rows2;  second.H = a.H2;
+            second.rows2 = 0;  second.H2 = 0;
+            second.lb2 = second.ub2 = second.lw2 = second.uw2 = nullptr;  second.l2 = second.u2 = nullptr;
+            dispatch_natural<MODE, Q>(first, st);
+            dispatch_natural<MODE, Q>(second, st);
+            return;
+        }
         const int pick = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
         if (vec4 && (pick == 11 || (pick == 0 && (long long)a.H * 4 >= 65536)))
             launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);
@@ -663,6 +677,8 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
             // a handful of neurons (the margin of a classifier): 64-neuron tiles would walk D_in in chunks of
             // 32 rows, one memory latency each; 8-neuron tiles take 256 rows per chunk
             launch_natural<MODE, Q, 1, 8, 256, 8>(a, st);
+        else if (a.H <= 32 && a.H2 <= 32)
+            launch_natural<MODE, Q, 1, 32, 256, 8>(a, st);      // no lane without a neuron, 64 rows per chunk
         else
             launch_natural<MODE, Q, 1, 64, 256, 8>(a, st);
         return;

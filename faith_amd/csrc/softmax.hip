@@ -287,6 +287,7 @@ bool dispatch(const SoftmaxArgs &a, bool vec4, hipStream_t st) {
         else return false;
     } else {
         if ((256 / tpr) * 16 >= a.D) launch<Q, 1, 256, 16>(a, k, st);
+        else if ((1024 / tpr) * 8 >= a.D) launch<Q, 1, 1024, 8>(a, k, st);
         else if ((1024 / tpr) * 24 >= a.D) launch<Q, 1, 1024, 24>(a, k, st);
         else return false;
     }

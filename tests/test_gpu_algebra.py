@@ -85,7 +85,9 @@ SOFTMAX_SHAPES = [
     (1, 2, 40, 256, 1),      # a full wavefront a row
     (1, 3, 30, 4, 1),        # one thread a row
     (2, 2, 33, 23, 1),       # H no multiple of 4: one column per thread
-    (1, 2, 300, 7, 2),       # the same with 1024 threads
+    (1, 2, 300, 7, 2),       # the same, more rows per thread
+    (1, 3, 256, 31, 1),      # a sentence of 31 tokens at dim_in 256: 1024 threads, one column each
+    (1, 2, 300, 50, 1),      # 1024 threads, 24 rows per thread
     (1, 2, 20, 1, 1),        # softmax of a single score
 ]
 
@@ -116,7 +118,7 @@ def test_softmax_in_one_launch(shape, p):
     assert close(out[4], l_sum[..., 0], rtol=2e-5, atol=1e-6), f"lower bound of the sum: {worst(out[4], l_sum[..., 0])}"
 
 
-@pytest.mark.parametrize("shape", SOFTMAX_SHAPES[:8])
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES[:11])
 def test_softmax_in_one_launch_equals_the_four_launches(shape):
     """Same per-neuron code and the same roundings between the operators: the fused kernel and the
     composition differ only by the order of the row sum and of the norm reductions."""
