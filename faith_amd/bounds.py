@@ -169,6 +169,15 @@ class Bounds:
         bias = getattr(dense, "bias", None)
         return self.matmul(dense.weight.detach(), None if bias is None else bias.detach().contiguous())
 
+    def dense_concretize(self, dense):
+        """(self.dense(dense), its concrete interval) through one entry point -- one launch for small problems such
+        as the classifier, whose result is concretized at once (VerifierForward.py:300-314).  Returns (bounds, l, u)."""
+        bias = getattr(dense, "bias", None)
+        out = ops.linear_concretize(*self._c(), dense.weight.detach().contiguous(),
+                                    None if bias is None else bias.detach().contiguous(),
+                                    self.p, self.eps, self.perturbed_words)
+        return self._like(*out[:4]), out[4], out[5]
+
     def dense_group(self, layers):
         """[self.dense(layer) for layer in layers] for up to three layers of one shape, in one launch where that
         pays (beyond the reference's surface: its `_bound_attention` calls dense three times,

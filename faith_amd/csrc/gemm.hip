@@ -679,3 +679,219 @@ extern "C" int faith_matmul_group_verification(const float *x_lb, const float *x
 #undef FAITH_LAUNCH_GROUPED
     return faith::check_launch("faith_matmul_group_verification");
 }
+
+
+// ------------------------------------------------------------------------------------------------------------
+// Affine layer and concretization of its result in ONE launch, for problems of a single round of tiles
+// (the reference's 16-position, 64-coordinate case; the classifier at the end of the verifier, whose result
+// is concretized at once: VerifierForward.py:300-314).  There the layer and the dual norm are two launches
+// of a few microseconds each, and the second only re-reads what the first has just written.
+//
+// A workgroup owns one position (row) and 32 columns of the result: every coefficient row of that position
+// passes through it, so the dual norms over dim_in are complete inside the workgroup.  Wavefront v takes
+// the 32-row blocks v, v + 4, ... of the position's dim_in rows, each as one 32 x 32 MFMA block over the whole
+// reduction with fragments loaded straight from global memory (the K pairing of signsplit_gemm_ksplit), stores
+// the block and folds its column norms into its own slots in LDS; the constant-term row is accumulated in
+// double by all threads first (the arithmetic of sliced_tile).  dim_in % (32 words) == 0, K % 8 == 0.
+#include "relax_common.h"
+
+namespace {
+
+struct FusedArgs {
+    GemmArgs g;
+    float *l, *u;               // [Mb, N] concrete interval of the result
+    int D, words;
+    float eps, qv;
+};
+
+constexpr int FUSED_MAX_WORDS = 8;
+
+template <int Q>
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_concretize(const FusedArgs f) {
+    __shared__ float part[FUSED_MAX_WORDS * 4 * 2 * 64];          // [word][wavefront][l, u][lane]
+    __shared__ double red[2][8][32];                               // constant terms: [l, u][K slice][column]
+    const GemmArgs &g = f.g;
+    const int tiles_n = (g.N + 31) / 32;
+    const int row = blockIdx.x / tiles_n, n0 = (blockIdx.x % tiles_n) * 32;
+    const int tid = threadIdx.x, lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int K = g.K;
+
+    // ---- constant terms of (row, n0 .. n0 + 31): eight K slices per column, lanes along K
+    {
+        const int c = tid / 8, ks = tid % 8;
+        const float *__restrict__ w = g.W + (size_t)min(n0 + c, g.N - 1) * K;
+        const float *__restrict__ xl = g.Bl + (size_t)row * K, *__restrict__ xu = g.Bu + (size_t)row * K;
+        double accm = 0.0, accr = 0.0;
+        for (int k = ks; k < K; k += 8) {
+            const double wk = w[k], a = xl[k], b = xu[k];
+            accm += wk * (0.5 * (a + b));
+            accr += fabs(wk) * (0.5 * (b - a));
+        }
+        red[0][ks][c] = accm - accr;
+        red[1][ks][c] = accm + accr;
+    }
+    for (int w = 0; w < f.words; ++w) {
+        part[((w * 4 + wv) * 2 + 0) * 64 + lane] = 0.f;
+        part[((w * 4 + wv) * 2 + 1) * 64 + lane] = 0.f;
+    }
+
+    // ---- coefficient rows: 32 x 32 blocks of this position, one per wavefront at a time
+    const int fi = lane % 32, fh = lane / 32;
+    const int ns = K / 8, blk = f.D / f.words;
+    const float4 *__restrict__ pw = reinterpret_cast<const float4 *>(g.W + (size_t)min(n0 + fi, g.N - 1) * K + 4 * fh);
+    const int col = n0 + fi;
+    for (int db = wv; db < f.D / 32; db += 4) {
+        const size_t r0 = (size_t)row * f.D + db * 32;
+        const float4 *__restrict__ pal = reinterpret_cast<const float4 *>(g.Al + (r0 + fi) * K + 4 * fh);
+        const float4 *__restrict__ pau = reinterpret_cast<const float4 *>(g.Au + (r0 + fi) * K + 4 * fh);
+        floatx16 cl, cu;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) cl[r] = cu[r] = 0.f;
+        constexpr int CH = 4;                                       // K-steps of 8 fetched ahead
+        float4 al[CH], au[CH], w[CH], nal[CH], nau[CH], nw[CH];
+        auto fetch = [&](float4 (&a)[CH], float4 (&b)[CH], float4 (&c)[CH], int s0) {
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if (s0 + i < ns) {
+                    a[i] = pal[2 * (s0 + i)];
+                    b[i] = pau[2 * (s0 + i)];
+                    c[i] = pw[2 * (s0 + i)];
+                }
+            }
+        };
+        fetch(al, au, w, 0);
+        for (int s0 = 0; s0 < ns; s0 += CH) {
+            if (s0 + CH < ns) fetch(nal, nau, nw, s0 + CH);
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if (s0 + i < ns) {
+                    const float4 wp = make_float4(fmaxf(w[i].x, 0.f), fmaxf(w[i].y, 0.f), fmaxf(w[i].z, 0.f), fmaxf(w[i].w, 0.f));
+                    const float4 wq = make_float4(fminf(w[i].x, 0.f), fminf(w[i].y, 0.f), fminf(w[i].z, 0.f), fminf(w[i].w, 0.f));
+#define FAITH_STEP(c)                       \
+    cl = mfma(al[i].c, wp.c, cl);           \
+    cu = mfma(au[i].c, wp.c, cu);           \
+    cl = mfma(au[i].c, wq.c, cl);           \
+    cu = mfma(al[i].c, wq.c, cu);
+                    FAITH_STEP(x)
+                    FAITH_STEP(y)
+                    FAITH_STEP(z)
+                    FAITH_STEP(w)
+#undef FAITH_STEP
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                al[i] = nal[i];
+                au[i] = nau[i];
+                w[i] = nw[i];
+            }
+        }
+        // register r of the block is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
+        float pl = 0.f, pu = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            pl = nacc<Q>(pl, cl[r], f.qv);
+            pu = nacc<Q>(pu, cu[r], f.qv);
+            if (col < g.N) {
+                const size_t o = (r0 + 8 * (r / 4) + 4 * fh + r % 4) * g.N + col;
+                g.Cl[o] = cl[r];
+                g.Cu[o] = cu[r];
+            }
+        }
+        pl = ncomb<Q>(pl, __shfl_xor(pl, 32, 64));
+        pu = ncomb<Q>(pu, __shfl_xor(pu, 32, 64));
+        const int w_id = (db * 32) / blk;                           // a block lies inside one perturbed word
+        float *slot = part + ((w_id * 4 + wv) * 2) * 64 + lane;
+        slot[0] = ncomb<Q>(slot[0], pl);
+        slot[64] = ncomb<Q>(slot[64], pu);
+    }
+    __syncthreads();
+
+    // ---- constant terms out, and the interval: l = lb' - eps * sum over words of the norm (Bounds.py:311-326)
+    if (tid < 32 && n0 + tid < g.N) {
+        double sl = red[0][0][tid], su = red[1][0][tid];
+#pragma unroll
+        for (int s = 1; s < 8; ++s) {
+            sl += red[0][s][tid];
+            su += red[1][s][tid];
+        }
+        const float add = g.bias ? g.bias[n0 + tid] : 0.f;         // added to the rounded product (Bounds.py:391-395)
+        const float lb = (float)sl + add, ub = (float)su + add;
+        const size_t o = (size_t)row * g.N + n0 + tid;
+        g.Dl[o] = lb;
+        g.Du[o] = ub;
+        float l = lb, u = ub;
+        for (int w = 0; w < f.words; ++w) {
+            float nl = 0.f, nu = 0.f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                nl = ncomb<Q>(nl, part[((w * 4 + v) * 2 + 0) * 64 + tid]);
+                nu = ncomb<Q>(nu, part[((w * 4 + v) * 2 + 1) * 64 + tid]);
+            }
+            l = __fadd_rn(l, __fmul_rn(-f.eps, nfin<Q>(nl, f.qv)));
+            u = __fadd_rn(u, __fmul_rn(f.eps, nfin<Q>(nu, f.qv)));
+        }
+        f.l[o] = l;
+        f.u[o] = u;
+    }
+}
+
+}  // namespace
+
+extern "C" int faith_matmul_concretize_verification(const float *x_lb, const float *x_ub, const float *x_lw,
+                                                    const float *x_uw, const float *W, const float *bias, float *y_lb,
+                                                    float *y_ub, float *y_lw, float *y_uw, float *l, float *u,
+                                                    int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
+                                                    float epsilon, int q, int words, void *stream) {
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(W);
+    FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_NOT_NULL(l); FAITH_NOT_NULL(u);
+    FAITH_ALIGNED4(x_lb); FAITH_ALIGNED4(x_ub); FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(W);
+    FAITH_ALIGNED4(bias); FAITH_ALIGNED4(y_lb); FAITH_ALIGNED4(y_ub); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_ALIGNED4(l); FAITH_ALIGNED4(u);
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && dim_in > 0 && dim_out > 0 && dim_y_out > 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_concretize_verification: batch=%d length=%d dim_in=%d dim_out=%d dim_y_out=%d must be "
+                  "positive", batch_size, length, dim_in, dim_out, dim_y_out);
+    FAITH_REQUIRE(words >= 1 && words <= 16 && dim_in % words == 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_concretize_verification: words=%d must be in 1..16 and divide dim_in=%d", words, dim_in);
+    FusedArgs f{};
+    if (!faith::dual_exponent(q, &f.qv)) {
+        faith::set_error("faith_matmul_concretize_verification: q=%d is neither FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF nor "
+                         "the bits of an exponent in (1, inf)", q);
+        return FAITH_ERR_UNSUPPORTED;
+    }
+    const long long rows = (long long)batch_size * length;
+    const long long mw = rows * dim_in;
+    const long long cus = faith::compute_units();
+    const long long tiles64 = ((mw + 63) / 64) * ((dim_y_out + 63) / 64);
+    const long long grid = rows * ((dim_y_out + 31) / 32);
+    const int pick = faith::tune_get(FAITH_TUNE_GEMM_VARIANT);
+    const bool fits = dim_out % 8 == 0 && dim_in % (32 * words) == 0 && words <= FUSED_MAX_WORDS &&
+                      faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) && faith::aligned(W, 16) &&
+                      mw <= 0x7fffffffLL && grid <= 0x7fffffffLL;
+    // one round of the smallest MFMA tiles at most: beyond that the tiled kernels' reuse of W and of the rows
+    // is worth more than the launch saved; and a wavefront's chain of 32 x 32 blocks (each as long as the reduction)
+    // no longer than the launch it saves: measured 17 against 19.5 us per call up to 128, 26 against 24 us at 256
+    // and 44 against 24 us for the 256 -> 2 classifier (512), whose few positions leave the tiled kernel more
+    // workgroups than this one has
+    const long long chain = (long long)((dim_in + 127) / 128) * dim_out;
+    if (fits && (pick == 6 || (pick == 0 && tiles64 <= cus && chain <= 128))) {
+        f.g = GemmArgs{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
+        f.l = l; f.u = u; f.D = dim_in; f.words = words; f.eps = epsilon;
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        const dim3 gd((unsigned)grid), bd(NTHREADS);
+        switch (q) {
+            case FAITH_Q_1: hipLaunchKernelGGL(signsplit_gemm_concretize<FAITH_Q_1>, gd, bd, 0, st, f); break;
+            case FAITH_Q_2: hipLaunchKernelGGL(signsplit_gemm_concretize<FAITH_Q_2>, gd, bd, 0, st, f); break;
+            case FAITH_Q_INF: hipLaunchKernelGGL(signsplit_gemm_concretize<FAITH_Q_INF>, gd, bd, 0, st, f); break;
+            default: hipLaunchKernelGGL(signsplit_gemm_concretize<Q_GENERAL>, gd, bd, 0, st, f); break;
+        }
+        return faith::check_launch("faith_matmul_concretize_verification");
+    }
+    const int rc = faith_matmul_verification(x_lb, x_ub, x_lw, x_uw, W, bias, y_lb, y_ub, y_lw, y_uw, batch_size, length,
+                                             dim_in, dim_out, dim_y_out, stream);
+    if (rc != FAITH_OK) return rc;
+    FAITH_REQUIRE(rows <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_concretize_verification: batch*length exceeds 2^31");
+    return faith_concretize(y_lb, y_ub, y_lw, y_uw, l, u, (int)rows, dim_in, dim_y_out, epsilon, q, words,
+                            FAITH_LAYOUT_NATURAL, stream);
+}

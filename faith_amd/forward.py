@@ -175,6 +175,10 @@ def _margin(bounds, classifier):
             classifier._faith_margin = cached
         except AttributeError:          # an object that takes no new attributes: rebuilt per call
             pass
+    fused = getattr(bounds, "dense_concretize", None)
+    if fused is not None:
+        _, l, u = fused(cached)
+        return l, u
     return bounds.dense(cached).concretize()
 
 

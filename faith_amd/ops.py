@@ -376,6 +376,30 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     return olw, olb, ouw, oub
 
 
+def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1):
+    """linear() and concretize() of its result through one entry point (one launch for small problems).
+    Returns (lw', lb', uw', ub', l, u)."""
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    _check("weight", weight)
+    if weight.dim() != 2 or weight.shape[1] != H:
+        raise ValueError(f"weight must be [H_out, {H}], got {tuple(weight.shape)}")
+    N = weight.shape[0]
+    if bias is not None:
+        _check("bias", bias, (N,))
+    olw = torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32)
+    ouw = torch.empty_like(olw)
+    olb = torch.empty(B, L, N, device=lw.device, dtype=torch.float32)
+    oub = torch.empty_like(olb)
+    l = torch.empty_like(olb)
+    u = torch.empty_like(olb)
+    with _on(lw.device, "linear", (B * L * D, H, N)):
+        _lib.call("faith_matmul_concretize_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight),
+                  _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), _ptr(l), _ptr(u), B, L, D, H, N,
+                  float(eps), q_code(p), int(words), _stream(lw))
+    return olw, olb, ouw, oub, l, u
+
+
 def linear_group(lw, lb, uw, ub, weights, biases=None):
     """Several affine layers of one shape on the same bound object (query, key, value of an attention block):
     one launch where that pays, the same results as linear() per layer.  weights: list of [H_out, H];

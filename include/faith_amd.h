@@ -52,7 +52,7 @@ int faith_version(void);
  * Process-wide, not thread-safe; results never depend on it, only speed.
  */
 #define FAITH_TUNE_ACT_VARIANT   0   /* tile shape of the natural-layout relaxation kernels */
-#define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split GEMM: 1 = 64x64, 2 = 128x128, 3 = 128x64, 4 = 64x128, 5 = 32x32 with K split over the wavefronts (dim_out % 32 == 0) */
+#define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split GEMM: 1 = 64x64, 2 = 128x128, 3 = 128x64, 4 = 64x128, 5 = 32x32 with K split over the wavefronts (dim_out % 32 == 0); 6 = faith_matmul_concretize_verification takes its one-launch kernel whenever the shape allows */
 #define FAITH_TUNE_DOT_VARIANT   2   /* dot product: 1 = 128x64 persistent tiles, 2 = one 32x32 block per wavefront (short sequences only) */
 #define FAITH_TUNE_DOT_COORDS    3   /* dot product, 32x32 kernel: perturbation coordinates per wavefront, 1..16 */
 #define FAITH_TUNE_COUNT         4
@@ -240,6 +240,25 @@ int faith_matmul_verification(const float *x_lb, const float *x_ub,
                               float *y_lb, float *y_ub, float *y_lw, float *y_uw,
                               int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
                               void *stream);
+
+/*
+ * Affine layer followed by the concretization of its result: y = x @ W^T (+ bias), then
+ * [l, u] of y.  Replaces Bounds.dense(...).concretize() (Bounds.py:1016-1025, :311-326) as the
+ * classifier at the end of the verifier uses it (VerifierForward.py:300-314); the reference has
+ * no fused counterpart (its tvm kernels keep matmul and concretize apart:
+ * tvm_kernels/cuda_kernel/matmul.cu, concretize.cu).  ONE launch for problems of a single round
+ * of tiles and a short reduction per position (ceil(dim_in / 128) * dim_out <= 128) with
+ * dim_out % 8 == 0, dim_in % (32 words) == 0, words <= 8 and 16-byte aligned x_lw, x_uw, W;
+ * otherwise faith_matmul_verification followed by faith_concretize on the same stream.  Arguments as faith_matmul_verification, plus l, u [batch*length, dim_y_out] and
+ * epsilon, q, words as faith_concretize.
+ */
+int faith_matmul_concretize_verification(const float *x_lb, const float *x_ub,
+                                         const float *x_lw, const float *x_uw,
+                                         const float *W, const float *bias,
+                                         float *y_lb, float *y_ub, float *y_lw, float *y_uw,
+                                         float *l, float *u,
+                                         int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
+                                         float epsilon, int q, int words, void *stream);
 
 /*
  * `groups` (1 ... 3) affine layers of one shape applied to the same bound object -- the query, key and value

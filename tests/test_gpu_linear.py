@@ -190,3 +190,90 @@ def test_mfma_clock_measurement_is_plausible():
     _lib.call("faith_mfma_clock", out.data_ptr(), 64, 200, torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
     torch.cuda.synchronize()
     assert bool(((out > 500) & (out < 3500)).all()), out
+
+
+# ---- affine layer + concretization through one entry point (one launch for small problems)
+def run_fused(x, W, bias, p, eps, words, force=None):
+    """force: None = built-in choice, 6 = the one-launch kernel wherever the shape allows, 1 = never."""
+    from faith_amd import ops, _lib
+    lw, lb, uw, ub, W, bias = dev(*x.tensors(), W, bias)
+    if force is not None:
+        _lib.call("faith_tune_set", 1, force)
+    try:
+        out = ops.linear_concretize(lw, lb, uw, ub, W, bias, p, eps, words)
+        torch.cuda.synchronize()
+    finally:
+        if force is not None:
+            _lib.call("faith_tune_set", 1, 0)
+    return out
+
+
+@pytest.mark.parametrize("shape", [
+    (1, 16, 64, 64, 64, 1),      # benchmark configuration 0
+    (1, 1, 256, 256, 2, 1),      # the margin classifier: two columns
+    (1, 3, 128, 72, 40, 2),      # two perturbed words, columns ragged against the 32-column block
+    (2, 5, 32, 8, 33, 1),        # one block per position, shortest reduction
+    (1, 2, 512, 200, 100, 4),    # more blocks than wavefronts, four words
+    (1, 4, 96, 64, 64, 3),       # blocks per word not a multiple of the wavefronts
+    (1, 40, 256, 128, 96, 1),    # several rounds of workgroups (forced)
+])
+@pytest.mark.parametrize("p", [1.0, 2.0, INF, 3.0])
+def test_linear_concretize_one_launch(shape, p):
+    B, L, D, H, N, words = shape
+    print(f"[case] linear_concretize forced one-launch shape={shape} p={p}", flush=True)
+    g = torch.Generator().manual_seed(77)
+    x = rand_bounds(g, B, L, D, H, ordered=False, sw=0.5)
+    W = torch.randn(N, H, generator=g) / H ** 0.5
+    bias = 0.01 * torch.randn(N, generator=g)
+    eps = 0.02
+    got = run_fused(x, W, bias, p, eps, words, force=6)
+    exp = O.linear(x, W, bias)
+    ref, mag = linear64(x, W, bias)
+    for name, a, e in zip(("lw", "lb", "uw", "ub"), got[:4], exp.tensors()):
+        compare_contraction(name, a, e, ref[name], mag[name])
+    # the interval is checked on the GPU's own propagated bounds (summation orders of the contraction differ)
+    el, eu = O.concretize(O.LinearBounds(*(t.cpu() for t in got[:4])), p, eps, words)
+    assert close(got[4], el) and close(got[5], eu), (worst(got[4].cpu(), el), worst(got[5].cpu(), eu))
+    # and it equals the two separate entry points within the bar
+    sep = run_fused(x, W, bias, p, eps, words, force=1)
+    for a, b in zip(got, sep):
+        assert close(a, b.cpu()), worst(a.cpu(), b.cpu())
+
+
+@pytest.mark.parametrize("shape,words", [
+    ((1, 3, 17, 37, 29), 1),      # nothing divisible: the separate kernels
+    ((1, 4, 48, 64, 64), 1),      # dim_in not a multiple of 32
+    ((1, 64, 128, 256, 512), 2),  # more than one round of tiles: the tiled kernel and the concretize kernel
+    ((1, 2, 64, 64, 64), 16),     # more words than the one-launch kernel keeps slots for
+])
+def test_linear_concretize_general_shapes(shape, words):
+    B, L, D, H, N = shape
+    print(f"[case] linear_concretize built-in choice shape={shape} words={words}", flush=True)
+    g = torch.Generator().manual_seed(78)
+    x = rand_bounds(g, B, L, D, H, ordered=False, sw=0.5)
+    W = torch.randn(N, H, generator=g) / H ** 0.5
+    got = run_fused(x, W, None, 2.0, 0.05, words)
+    from faith_amd import ops
+    lw, lb, uw, ub, Wd = dev(*x.tensors(), W)
+    lin = ops.linear(lw, lb, uw, ub, Wd, None)
+    l, u = ops.concretize(*lin, 2.0, 0.05, words)
+    for a, b in zip(got, (*lin, l, u)):
+        assert torch.equal(a, b)
+
+
+def test_linear_concretize_config0_against_oracle():
+    from faith_amd.workloads import make_config
+    c = make_config(0)
+    x = as_bounds(c["x"])
+    got = run_fused(x, c["W"], c["bias"], c["p"], c["eps"], c["words"])
+    el, eu = O.concretize(O.linear(x, c["W"], c["bias"]), c["p"], c["eps"], c["words"])
+    assert close(got[4], el) and close(got[5], eu)
+    assert bool((got[4] <= got[5]).all())
+
+
+def test_linear_concretize_rejects_bad_words():
+    from faith_amd import _lib
+    g = torch.Generator().manual_seed(3)
+    x = rand_bounds(g, 1, 2, 6, 8, ordered=False)
+    with pytest.raises(_lib.FaithError):
+        run_fused(x, torch.randn(4, 8, generator=g), None, 2.0, 0.1, 4)     # 4 does not divide dim_in = 6
