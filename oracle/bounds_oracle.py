@@ -22,9 +22,12 @@ Parity status of each function (what pins it, see tests/test_oracle_*.py):
   relu         pinned: independent fp64 per-neuron closed form
                (oracle/closed_form.py), branch invariants, sampled soundness.
   tanh         pinned: independent fp64 scalar loop, odd symmetry, sampled
-               soundness.  The bisection update order is pinned by text only
-               (Bounds.py:1063-1097 cannot be imported: the module needs tvm
-               and nvcc at import time).
+               soundness, and tangency: the lines touch the curve at the
+               point the bisection returns, to the resolution of ten halvings
+               (pins the sign test and the bracket update order).  The exact
+               number of steps is pinned by text only (Bounds.py:1063-1097
+               cannot be imported: the module needs tvm and nvcc at import
+               time).
   exp, reciprocal, sqr, sqrt
                pinned: independent fp64 per-neuron closed forms, sampled soundness
                (lower line <= f <= upper line on [l, u]).

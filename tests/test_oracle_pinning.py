@@ -228,6 +228,27 @@ def test_tanh_lines_bound_the_function():
         assert (ku * (xs - xu) + yu >= np.tanh(xs) - slack).all()
 
 
+def test_tanh_bisection_lands_on_the_tangent_point():
+    """Where the true tangent point lies inside the bracket the ten bisection steps (Bounds.py:1063-1097) must end
+    next to it: the lower line through (u, tanh u) touches the curve on [l, 0], the upper line through (l, tanh l)
+    touches it on [0, u] (gap ~ curvature x (bracket / 2^11)^2), and each stays on its side of the curve.  A
+    bisection that moves the wrong end of its bracket ends at l, 0 or u instead: the line then cuts through the
+    curve or stands off it by far more."""
+    for lo, hi in [(-4.0, 4.0), (-2.0, 3.0), (-3.0, 1.5), (-1.0, 1.2)]:
+        (kl, xl, yl), (ku, xu, yu) = C.tanh_lines(lo, hi)
+        xs = np.linspace(lo, hi, 20001)
+        gap_l = np.tanh(xs) - (kl * (xs - xl) + yl)
+        gap_u = (ku * (xs - xu) + yu) - np.tanh(xs)
+        # the brackets are [lo, 0] and [0, hi]: 2^-11 of their length after ten steps
+        for gap, side, bracket in ((gap_l, xs <= 0, -lo), (gap_u, xs >= 0, hi)):
+            assert gap.min() > -1e-4
+            assert gap[side].min() < 4 * (bracket / 2048) ** 2 + 1e-6, (lo, hi, gap[side].min())
+        # the line's anchor is the tangent point itself: slope = derivative there, to first order in the bracket
+        assert abs(kl - (1 - np.tanh(xl) ** 2)) < 4 * (-lo / 2048) + 1e-6
+        assert abs(ku - (1 - np.tanh(xu) ** 2)) < 4 * (hi / 2048) + 1e-6
+        assert lo < xl < 0 < xu < hi
+
+
 # ---------------------------------------------------------------- dot product
 @pytest.mark.parametrize("p", PS)
 @pytest.mark.parametrize("words", [1, 2])
