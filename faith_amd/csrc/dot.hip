@@ -816,20 +816,25 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     g.oz = {z_sbs ? heads * Ly : Ly, z_sbs ? heads : 1, Ly};
     g.heads = heads;
     g.side_by_side = side_by_side;
+    FAITH_REQUIRE(words >= 1 && (D == 1 || D % words == 0), FAITH_ERR_SHAPE, "%s: words=%d must divide dim_in=%d", who, words, D);
+    // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the reference
+    // interface exposes it, the planes do not use it.  One launch for both objects.
+    // An object with its heads side by side is concretized as the one [L, D, heads * width] object it is.
+    // (With dim_in == 1 the interval shortcut below does not read them; they are still the documented
+    // outputs of the entry point, so they are written there too.)
+    const int cx_rows = x_sbs ? B / heads * Lx : B * Lx, cx_h = x_sbs ? heads * d : d;
+    const int cy_rows = y_sbs ? B / heads * y_len : B * y_len, cy_h = y_sbs ? heads * y_h : y_h;
+    // dim_in == 1 with several words: the reference's blocks are then empty (dim_in // words == 0,
+    // Bounds.py:319-326) and its intervals are the constant terms themselves -- a radius of zero here
+    const bool empty_blocks = D == 1 && words > 1;
+    int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows, D,
+                                    cx_h, cy_h, empty_blocks ? 0.f : epsilon, q, empty_blocks ? 1 : words, stream);
+    if (rc != FAITH_OK) return rc;
     if (D == 1) {
         const long long n = (long long)B * Lx * Ly;
         hipLaunchKernelGGL(dot_interval<VP>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, g);
         return faith::check_launch(who);
     }
-
-    // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the reference
-    // interface exposes it, the planes do not use it.  One launch for both objects.
-    // An object with its heads side by side is concretized as the one [L, D, heads * width] object it is.
-    const int cx_rows = x_sbs ? B / heads * Lx : B * Lx, cx_h = x_sbs ? heads * d : d;
-    const int cy_rows = y_sbs ? B / heads * y_len : B * y_len, cy_h = y_sbs ? heads * y_h : y_h;
-    int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows, D,
-                                    cx_h, cy_h, epsilon, q, words, stream);
-    if (rc != FAITH_OK) return rc;
 
     const long long b_tiles = (long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T);
     FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);

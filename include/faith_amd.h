@@ -285,7 +285,9 @@ int faith_matmul_group_verification(const float *x_lb, const float *x_ub,
  *   x_l, x_u   [batch, length_x, dim_out]  (out: concrete interval of x; caller's scratch)
  *   y_l, y_u   [batch, length_y, dim_out]  (out: concrete interval of y)
  *   z_lw, z_uw [batch, length_x, dim_in, length_y];  z_lb, z_ub [batch, length_x, length_y]
- * The reference entry has one `length`; here x and y may differ in length.
+ * The reference entry has one `length`; here x and y may differ in length.  With dim_in == 1 the
+ * result is the interval product of the constant terms (Bounds.py:711-721); x_l .. y_u are written
+ * all the same.  words must divide dim_in.
  */
 int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u,
                                       const float *x_lb, const float *x_ub,

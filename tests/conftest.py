@@ -20,3 +20,37 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def _ledger():
+    from tests import parity
+    return parity.LEDGER
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """Keeps the parity concessions of the run (tests/parity.py) where the run's output is kept."""
+    import json
+    led = _ledger()
+    if not led["comparisons"]:
+        return
+    out = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "parity_ledger.json"), "w") as f:
+            json.dump(led, f, indent=1)
+    except OSError:
+        pass
+
+
+def pytest_terminal_summary(terminalreporter):
+    led = _ledger()
+    if not led["comparisons"]:
+        return
+    kinds = {}
+    for c in led["concessions"]:
+        kinds[c["kind"]] = kinds.get(c["kind"], 0) + 1
+    terminalreporter.write_line(
+        f"parity ledger: {led['comparisons']} harness comparisons, {led['plain']} on the plain bar "
+        f"(rtol 1e-5 / atol 1e-6), concessions: {kinds if kinds else 'none'}")
+    for c in led["concessions"]:
+        terminalreporter.write_line(f"  {c}")

@@ -26,12 +26,30 @@ tolerance:
 """
 from __future__ import annotations
 
+import os
+
 import numpy as np
 import torch
 
 from oracle import closed_form as C
 
 RTOL, ATOL = 1e-5, 1e-6
+
+# Every comparison that did not pass on the plain bar alone is entered here -- which test, which
+# tensor, which concession, how large -- and every comparison is counted.  tests/conftest.py prints
+# the totals at the end of the session and writes them to gpurun_out/parity_ledger.json, so a run
+# shows how many tensors or neurons leaned on a concession even when it prints nothing else.
+LEDGER = {"comparisons": 0, "plain": 0, "concessions": []}
+
+
+def _note(kind, name, **detail):
+    test = os.environ.get("PYTEST_CURRENT_TEST", "").split(" (")[0]
+    LEDGER["concessions"].append(dict(test=test, kind=kind, tensor=name, **detail))
+
+
+def _count(plain):
+    LEDGER["comparisons"] += 1
+    LEDGER["plain"] += int(plain)
 
 
 def _bad(got, exp, rtol=RTOL, atol=ATOL):
@@ -68,10 +86,13 @@ def compare_activation(kind, x, got, exp, l_gpu, u_gpu, l_ref, u_ref,
             f"neuron {(b, r, j)} with [l,u]=[{lo},{hi}] is off the bar and not a boundary case"
         e = C.lines_applied(*lines(lo, hi), x.lw[b, r, :, j].double().numpy(), float(x.lb[b, r, j]),
                             x.uw[b, r, :, j].double().numpy(), float(x.ub[b, r, j]))
-        np.testing.assert_allclose(glw[b, r, :, j].double().numpy(), e[0], rtol=1e-4, atol=1e-5)
-        np.testing.assert_allclose(float(glb[b, r, j]), e[1], rtol=1e-4, atol=1e-5)
-        np.testing.assert_allclose(guw[b, r, :, j].double().numpy(), e[2], rtol=1e-4, atol=1e-5)
-        np.testing.assert_allclose(float(gub[b, r, j]), e[3], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(glw[b, r, :, j].double().numpy(), e[0], rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(float(glb[b, r, j]), e[1], rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(guw[b, r, :, j].double().numpy(), e[2], rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(float(gub[b, r, j]), e[3], rtol=RTOL, atol=ATOL)
+    _count(not idx)
+    if idx:
+        _note("boundary-neuron", kind, neurons=len(idx), of=total)
     return {"neurons": total, "explained_boundary_cases": len(idx)}
 
 
@@ -104,6 +125,9 @@ def compare_unary(kind, x, got, exp, l_gpu, u_gpu, l_ref, u_ref, max_inherited_f
         np.testing.assert_allclose(guw[b, r, :, j].double().numpy(), e[2], rtol=1e-5, atol=1e-6)
         assert abs(float(glb[b, r, j]) - e[1]) <= 1e-6 + 1e-5 * (abs(e[1]) + big), (kind, b, r, j)
         assert abs(float(gub[b, r, j]) - e[3]) <= 1e-6 + 1e-5 * (abs(e[3]) + big), (kind, b, r, j)
+    _count(not idx)
+    if idx:
+        _note("inherited-from-interval", kind, neurons=len(idx), of=total)
     return {"neurons": total, "inherited_from_interval": len(idx)}
 
 
@@ -113,9 +137,25 @@ def compare_unary(kind, x, got, exp, l_gpu, u_gpu, l_ref, u_ref, max_inherited_f
 KAPPA = 8.0
 U32 = 2.0 ** -24
 
+# The two declared reasons a contraction tensor may lean on the accumulation-aware bar.
+# Both require that the fp32 oracle itself is further than atol from the float64 value of the
+# same fp32 inputs on that tensor (asserted): there the bar is finer than fp32 resolves, and
+# two correct fp32 summations cannot be held to it against each other.
+B_IN_DOUBLE = ("constant terms are accumulated in double here and rounded once; the fp32 oracle's own "
+               "distance from float64 exceeds atol, the GPU's does not exceed the oracle's")
+UNIT_SCALE = ("test operands of unit scale (not a benchmark configuration): 4*d (or K) products of size ~1 "
+              "cancel to ~0; one MFMA K-chain here, four blocked GEMMs and three adds in the oracle")
+CONSTANT_TERMS = {"lb": B_IN_DOUBLE, "ub": B_IN_DOUBLE}
+UNIT_SCALE_ALL = {"lw": UNIT_SCALE, "uw": UNIT_SCALE, "lb": B_IN_DOUBLE, "ub": B_IN_DOUBLE}
 
-def compare_contraction(name, got, oracle32, ref64, abs_terms):
+
+def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None):
     """Parity of one output tensor of a contraction.
+
+    `allow`: None (the default) means this tensor must meet the plain bar and the fallback below
+    is a failure; a caller that expects a tensor on the fallback passes the reason -- a string, or
+    a dict from tensor name to reason (a name that is missing has none) -- and the case is
+    entered in LEDGER.
 
     First the plain bar against the fp32 CPU oracle (rtol 1e-5, atol 1e-6).  Two fp32
     summations of the same K products in different orders (MKL blocks on the CPU, MFMA K-pairs
@@ -132,9 +172,12 @@ def compare_contraction(name, got, oracle32, ref64, abs_terms):
     expected; more would point at the kernel, not at fp32).
     Returns "plain" or "accumulation-aware".
     """
+    if isinstance(allow, dict):
+        allow = allow.get(name)
     got = got.detach().cpu().double()
     o32 = oracle32.detach().cpu().double()
     if not bool(_bad(got, o32).any()):
+        _count(True)
         return "plain"
     ref64 = ref64.detach().cpu().double()
     tol = ATOL + RTOL * ref64.abs() + KAPPA * U32 * abs_terms.detach().cpu().double()
@@ -143,7 +186,15 @@ def compare_contraction(name, got, oracle32, ref64, abs_terms):
     print(f"   [{name}] plain bar missed by {int(_bad(got, o32).sum())} of {got.numel()} elements; "
           f"vs float64: gpu max err {float(err.max()):.3g}, cpu-oracle max err {float(oerr.max()):.3g}, "
           f"max err/allowance {float((err / tol).max()):.3f}", flush=True)
+    assert allow is not None, (f"{name}: misses rtol {RTOL} / atol {ATOL} against the oracle and no concession is "
+                               f"declared for it (worst error vs float64 {float(err.max()):.3g}, oracle's {float(oerr.max()):.3g})")
+    assert float(oerr.max()) > ATOL, f"{name}: the oracle is within atol of float64 here, so the GPU must meet the plain bar"
+    if allow is B_IN_DOUBLE:
+        assert float(err.max()) <= float(oerr.max()), f"{name}: accumulated in double, yet further from float64 than the oracle"
     assert bool((err <= tol).all()), f"{name}: outside the accumulation-aware bar"
     assert float(err.max()) <= 8.0 * float(oerr.max()) + ATOL, \
         f"{name}: the CPU oracle is much closer to float64 than the GPU ({float(oerr.max()):.3g} vs {float(err.max()):.3g})"
+    _count(False)
+    _note("accumulation-aware", name, reason=allow, missed=int(_bad(got, o32).sum()), of=got.numel(),
+          gpu_err_vs_f64=float(err.max()), oracle_err_vs_f64=float(oerr.max()))
     return "accumulation-aware"

@@ -5,7 +5,7 @@ import torch.nn.functional as F
 
 from oracle import bounds_oracle as O
 from tests.helpers import close
-from tests.parity import compare_contraction
+from tests.parity import compare_contraction, CONSTANT_TERMS
 
 pytestmark = pytest.mark.gpu
 INF = float("inf")
@@ -42,7 +42,7 @@ def check(x, W, bias, stride, pad, what=""):
     ref, mag = conv64(x, W, bias, stride, pad)
     for name, g_, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
         assert g_.shape == e.shape
-        compare_contraction(name, g_, e, ref[name], mag[name])
+        compare_contraction(name, g_, e, ref[name], mag[name], CONSTANT_TERMS)
     return got
 
 

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from tests.helpers import rand_bounds
+from tests.parity import UNIT_SCALE_ALL
 from tests import test_gpu_act as T_act
 from tests import test_gpu_dot as T_dot
 from tests import test_gpu_linear as T_lin
@@ -64,9 +65,9 @@ def test_random_dot_shapes(seed):
     if rng.random() < 0.5:
         x = rand_bounds(g, B, Lx, D, d, ordered=False, sw=0.3, sb=1.0)
         y = rand_bounds(g, B, Ly, D, d, ordered=False, sw=0.3, sb=1.0)
-        T_dot.check(x, y, p, 0.1, words, f"random {seed}")
+        T_dot.check(x, y, p, 0.1, words, f"random {seed}", UNIT_SCALE_ALL)
     else:
         dv = pick(rng, dims(rng, 4, 80, 4), rng.randrange(1, 40))
         probs = rand_bounds(g, B, Lx, D, Ly, ordered=False, sw=0.2, sb=0.5)
         value = rand_bounds(g, B, Ly, D, dv, ordered=False, sw=0.3, sb=1.0)
-        T_dot.check_v(probs, value, p, 0.1, words, f"random {seed}")
+        T_dot.check_v(probs, value, p, 0.1, words, f"random {seed}", UNIT_SCALE_ALL)
