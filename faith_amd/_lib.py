@@ -43,6 +43,7 @@ SIGNATURES = {
     "faith_matmul_concretize_verification": [_P] * 12 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_matmul_group_verification": [_P] * 4 + [_I] + [_P] * 6 + [_I] * 5 + [_P],
     "faith_dot_product_verification_QK": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
+    "faith_dot_product_verification_QK_static": [_P] * 12 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_dot_product_verification_V": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_attention_scores": [_P] * 16 + [_I] * 6 + [_F, _I, _I, _P],
     "faith_attention_context": [_P] * 16 + [_I] * 6 + [_F, _I, _I, _P],
@@ -68,6 +69,8 @@ def _load():
     lib.faith_last_error.argtypes = []
     lib.faith_version.restype = _I
     lib.faith_version.argtypes = []
+    lib.faith_static_scratch_bytes.restype = ctypes.c_longlong
+    lib.faith_static_scratch_bytes.argtypes = []
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
         fn.restype = _I

@@ -38,6 +38,8 @@
 //
 // The constant terms z_lb / z_ub ([Lx, Ly] per head, 1/D_in of the work, O(1) cancelling terms)
 // are summed in double by a small kernel.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -943,6 +945,69 @@ extern "C" int faith_dot_product_verification_V(float *x_l, float *y_l, float *x
     return dot_entry<true>("faith_dot_product_verification_V", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
                            y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, dim_out, length_k, dim_in, epsilon,
                            q, words, 0, 1, stream);
+}
+
+// ------------------------------------------------------------------------------------------
+// An entry point that allocates nothing and takes no scratch from its caller.
+//
+// faith_dot_product_verification_QK needs four scratch arrays from its caller (the concrete intervals
+// x_l, x_u, y_l, y_u).  The variant below keeps them in a file-scope device array instead, for callers
+// that cannot allocate: code under HIP graph capture, tight serving loops.  Each GPU holds its own copy
+// of the array (4 MiB) at its own address until the process ends; the address is looked up once per
+// device, with that device current, and only that address -- never the array's name, which is a
+// host-side stand-in -- is handed to kernels.  Nothing in it has to start at zero: every call overwrites
+// the part it reads.  Calls that overlap on one GPU share the array and race.
+// ------------------------------------------------------------------------------------------
+constexpr size_t STATIC_SCRATCH_FLOATS = (size_t)1 << 20;
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+static float *scratch_ptr[MAX_DEVICES];
+static std::mutex scratch_mutex;
+
+// Device address of this GPU's copy of `scratch` (looked up on the first call per device).
+static int scratch_address(const char *who, float **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    FAITH_REQUIRE(e == hipSuccess && dev >= 0 && dev < MAX_DEVICES, FAITH_ERR_LAUNCH, "%s: hipGetDevice: %s (device %d)", who,
+                  hipGetErrorString(e), dev);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        float *p = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+        FAITH_REQUIRE(e == hipSuccess && p != nullptr, FAITH_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", who,
+                      hipGetErrorString(e));
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return FAITH_OK;
+}
+
+extern "C" long long faith_static_scratch_bytes(void) { return (long long)(STATIC_SCRATCH_FLOATS * sizeof(float)); }
+
+extern "C" int faith_dot_product_verification_QK_static(const float *x_lb, const float *x_ub, const float *y_lb,
+                                                        const float *y_ub, const float *x_lw, const float *x_uw,
+                                                        const float *y_lw, const float *y_uw, float *z_lb, float *z_ub,
+                                                        float *z_lw, float *z_uw, int batch_size, int length_x,
+                                                        int length_y, int dim_out, int dim_in, float epsilon, int q,
+                                                        int words, void *stream) {
+    const char *who = "faith_dot_product_verification_QK_static";
+    FAITH_REQUIRE(batch_size > 0 && length_x > 0 && length_y > 0 && dim_out > 0 && dim_in > 0, FAITH_ERR_SHAPE,
+                  "%s: batch=%d length_x=%d length_y=%d dim_out=%d dim_in=%d must be positive", who, batch_size, length_x,
+                  length_y, dim_out, dim_in);
+    // four segments (x_l, x_u, y_l, y_u), each rounded up to 64 floats so that every one starts 256-byte aligned
+    auto seg = [](long long n) { return (n + 63) / 64 * 64; };
+    const long long nx = seg((long long)batch_size * length_x * dim_out), ny = seg((long long)batch_size * length_y * dim_out);
+    FAITH_REQUIRE(2 * nx + 2 * ny <= (long long)STATIC_SCRATCH_FLOATS, FAITH_ERR_UNSUPPORTED,
+                  "%s: the concrete intervals need %lld floats of scratch (2 * batch * (length_x + length_y) * dim_out, "
+                  "segments rounded to 64), the static array holds %lld; use faith_dot_product_verification_QK with "
+                  "caller-owned scratch for this size", who, 2 * nx + 2 * ny, (long long)STATIC_SCRATCH_FLOATS);
+    float *base = nullptr;
+    const int rc = scratch_address(who, &base);
+    if (rc != FAITH_OK) return rc;
+    float *x_l = base, *x_u = base + nx, *y_l = base + 2 * nx, *y_u = base + 2 * nx + ny;
+    return dot_entry<false>(who, x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw,
+                            batch_size, length_x, length_y, dim_out, dim_in, epsilon, q, words, 0, 1, stream);
 }
 
 extern "C" int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,

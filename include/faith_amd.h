@@ -300,6 +300,26 @@ int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float 
                                       int q, int words, void *stream);
 
 /*
+ * faith_dot_product_verification_QK for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments
+ * and results, minus the four scratch arrays x_l, x_u, y_l, y_u: the concrete intervals live in a
+ * device array inside the library, faith_static_scratch_bytes() = 4 MiB per GPU, held until the process
+ * ends.  The call allocates and frees nothing.  Limit: 2 * batch * (length_x + length_y) * dim_out floats
+ * (each of the four segments rounded up to 64 floats) must fit the array, else FAITH_ERR_UNSUPPORTED
+ * (configuration-size attention, 4 heads x 128 x 64, needs 0.5 MiB).  Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU (two streams, two threads) race.
+ */
+long long faith_static_scratch_bytes(void);
+int faith_dot_product_verification_QK_static(const float *x_lb, const float *x_ub,
+                                             const float *y_lb, const float *y_ub,
+                                             const float *x_lw, const float *x_uw,
+                                             const float *y_lw, const float *y_uw,
+                                             float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                                             int batch_size, int length_x, int length_y,
+                                             int dim_out, int dim_in, float epsilon,
+                                             int q, int words, void *stream);
+
+/*
  * McCormick bounds of the attention context  z[i,j] = sum_k x[i,k] * y[k,j]  (probabilities times
  * values).  Replaces call_dot_product_verification_V (kernel.cpp:53-60,
  * dot_product_verification.cu:498-535) with the arithmetic of Bounds.context -> ori_dot_product

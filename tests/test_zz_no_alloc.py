@@ -1,0 +1,60 @@
+"""The allocation-free dot product (faith_dot_product_verification_QK_static, scratch in a device array
+inside the library) against faith_dot_product_verification_QK with caller-owned scratch, both through
+the C ABI: same kernels, same inputs, so the results must be identical bit for bit.  Two calls in a
+row, the second smaller, so that what the first left in the shared array cannot leak into the second.
+Collected last: a failure here must not hide the other tests under `pytest -x`."""
+import ctypes
+
+import pytest
+import torch
+
+from tests.helpers import rand_bounds
+
+pytestmark = pytest.mark.gpu
+INF = float("inf")
+
+
+def _call_both(B, Lx, Ly, D, d, p, words, seed):
+    from faith_amd import _lib, ops
+    g = torch.Generator().manual_seed(seed)
+    x = [t.cuda().contiguous() for t in rand_bounds(g, B, Lx, D, d, sw=0.2, sb=1.0).tensors()]
+    y = [t.cuda().contiguous() for t in rand_bounds(g, B, Ly, D, d, sw=0.2, sb=1.0).tensors()]
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    new = lambda *s: torch.full(s, float("nan"), device="cuda")
+    outs = []
+    for static in (False, True):
+        zlb, zub, zlw, zuw = new(B, Lx, Ly), new(B, Lx, Ly), new(B, Lx, D, Ly), new(B, Lx, D, Ly)
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        tail = (B, Lx, Ly, d, D, 0.05, ops.q_code(p), words, stream)
+        if static:
+            before = torch.cuda.memory_allocated()
+            _lib.call("faith_dot_product_verification_QK_static", P(xlb), P(xub), P(ylb), P(yub), P(xlw), P(xuw), P(ylw),
+                      P(yuw), P(zlb), P(zub), P(zlw), P(zuw), *tail)
+            assert torch.cuda.memory_allocated() == before
+        else:
+            xl, xu, yl, yu = new(B, Lx, d), new(B, Lx, d), new(B, Ly, d), new(B, Ly, d)
+            _lib.call("faith_dot_product_verification_QK", P(xl), P(yl), P(xu), P(yu), P(xlb), P(xub), P(ylb), P(yub),
+                      P(xlw), P(xuw), P(ylw), P(yuw), P(zlb), P(zub), P(zlw), P(zuw), *tail)
+        torch.cuda.synchronize()
+        outs.append((zlw, zlb, zuw, zub))
+    return outs
+
+
+def test_static_scratch_dot_product_equals_the_caller_scratch_entry_twice_in_a_row():
+    # first call: configuration-3-like (tiled kernel); second: smaller and ragged (short-sequence kernel), other norm
+    for case in ((4, 128, 128, 32, 64, INF, 1, 11), (2, 24, 17, 8, 32, 2.0, 2, 12), (1, 5, 3, 1, 16, 2.0, 1, 13)):
+        print(f"[case] static-scratch dot product B,Lx,Ly,D,d,p,words,seed={case}", flush=True)
+        ref, got = _call_both(*case)
+        for name, a, b in zip(("lw", "lb", "uw", "ub"), got, ref):
+            assert not torch.isnan(a).any(), f"{name}: not fully written"
+            assert torch.equal(a, b), f"{name} differs from the caller-scratch entry point at {case}"
+
+
+def test_static_scratch_dot_product_rejects_what_does_not_fit():
+    from faith_amd import _lib
+    z = torch.zeros(8, device="cuda")
+    P = ctypes.c_void_p(z.data_ptr())
+    with pytest.raises(_lib.FaithError, match="scratch"):
+        _lib.call("faith_dot_product_verification_QK_static", *([P] * 12), 16, 512, 512, 64, 8, 0.1, 1, 1, None)
