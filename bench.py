@@ -38,13 +38,34 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 INF = float("inf")
 WARM_SECONDS = 0.25            # minimum warm-up per measurement; --profile sets it to 0
 
-# HBM bytes per launch of the dominant relaxation kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE, scaled by the same counters on faith_copy_f32 of known size (see
-# profiles/hbm_traffic_pmc.md), per relaxation (FETCH_SIZE reads half of what was fetched on this part).
-TRAFFIC_BYTES_PER_LAUNCH = {
-    "relu": 271_810_000,   # (2.000 * 66,349 + 132,750) KiB
-    "tanh": 269_980_000,   # (2.000 * 65,887 + 131,877) KiB
-}
+COLD_SETS = 5                  # disjoint operand sets cycled by the cold measurement (1.35 GB between reuses)
+
+
+def traffic_from_profile():
+    """HBM bytes per launch of the relaxation kernels as the hardware counters saw them: the lines
+    `traffic_bytes_per_launch <relu|tanh> <warm|cold> <bytes>` of profiles/hbm_traffic_pmc.md (rocprofv3
+    --pmc FETCH_SIZE / WRITE_SIZE of this program, scaled by the same counters on faith_copy_f32 of known
+    size).  Empty if the summary is missing."""
+    import re
+    out = {}
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic_pmc.md")) as f:
+            for m in re.finditer(r"^traffic_bytes_per_launch\s+(\w+)\s+(warm|cold)\s+(\d+)", f.read(), flags=re.M):
+                out[(m.group(1), m.group(2))] = int(m.group(3))
+    except OSError:
+        pass
+    return out
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def log(*a):
@@ -242,11 +263,69 @@ def bench_config1(args, ops, O, wl, steps, warmup):
 
     dom = max(per_kernel, key=lambda k: statistics.mean(per_kernel[k]))
     avg_ms = statistics.mean(gpu_back_to_back_ms(lambda: one(*dom), 20))
+    traffic = traffic_from_profile()
     roofline = {"bound": "hbm", "kernel": f"act_resident<{dom[0]}, p={dom[1]:g}>",
                 "achieved": round(nbytes / avg_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(nbytes / avg_ms / 1e6 / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(avg_ms * 1e3, 2), "bytes_per_launch": nbytes,
-                "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom[0])}
+                "traffic": traffic.get((dom[0], "warm")),
+                "note": "the configuration as specified: one operand set (269 MB) reused by every launch, against 256 MB "
+                        "of Infinity Cache; roofline_cold cycles disjoint sets"}
+
+    # Cold: the same launches over COLD_SETS disjoint operand and result sets, so that 1.35 GB pass
+    # through the memory system before any byte is touched again and nothing is served from the 256 MB
+    # Infinity Cache.  Same kernel, same bytes per launch.
+    sets = [(x, out)] + [({k: v.clone() for k, v in x.items()}, tuple(torch.empty_like(t) for t in out))
+                         for _ in range(COLD_SETS - 1)]
+    turn = [0]
+
+    def one_cold(kind, p):
+        xs, os_ = sets[turn[0] % COLD_SETS]
+        turn[0] += 1
+        getattr(ops, kind)(*quad(xs), p, c["eps"], c["words"], out=os_)
+
+    cold_entries = {}
+    streaming = {}
+    for kind in ("relu", "tanh"):
+        for _ in range(2 * COLD_SETS):
+            one_cold(kind, dom[1])
+        cold_ms = statistics.mean(gpu_back_to_back_ms(lambda: one_cold(kind, dom[1]), 4 * COLD_SETS))
+        cold_entries[kind] = cold_ms
+        entries.append(op_entry(f"config1 {kind} p={dom[1]:g} COLD: {COLD_SETS} disjoint operand sets in turn "
+                                f"({COLD_SETS * nbytes / 1e9:.2f} GB between reuses), average of back-to-back launches",
+                                "hbm", [cold_ms], nbytes))
+        # the thread shape the library takes by itself for objects that cannot be cache resident (more than
+        # 320 MB of traffic), forced here through the tuning knob: what a cold stream of this shape can reach
+        _lib.call("faith_tune_set", 0, 7)
+        try:
+            for _ in range(2 * COLD_SETS):
+                one_cold(kind, dom[1])
+            streaming[kind] = statistics.mean(gpu_back_to_back_ms(lambda: one_cold(kind, dom[1]), 4 * COLD_SETS))
+        finally:
+            _lib.call("faith_tune_set", 0, 0)
+        entries.append(op_entry(f"config1 {kind} p={dom[1]:g} COLD, thread shape for HBM streams forced (tuning knob)",
+                                "hbm", [streaming[kind]], nbytes))
+    srcs = [torch.randn(nbytes // 8, device="cuda") for _ in range(COLD_SETS)]
+    dsts = [torch.empty_like(t) for t in srcs]
+
+    def copy_cold():
+        i = turn[0] % COLD_SETS
+        turn[0] += 1
+        _lib.call("faith_copy_f32", srcs[i].data_ptr(), dsts[i].data_ptr(), srcs[i].numel(), st)
+    for _ in range(2 * COLD_SETS):
+        copy_cold()
+    copy_cold_ms = statistics.mean(gpu_back_to_back_ms(copy_cold, 4 * COLD_SETS))
+    entries.append(op_entry(f"plain copy of the same byte count COLD ({COLD_SETS} disjoint buffer pairs in turn; yardstick)",
+                            "hbm", [copy_cold_ms], nbytes))
+    del srcs, dsts
+    cold_ms = cold_entries[dom[0]]
+    roofline_cold = {"bound": "hbm", "kernel": roofline["kernel"], "achieved": round(nbytes / cold_ms / 1e6, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / cold_ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "avg_launch_us": round(cold_ms * 1e3, 2), "bytes_per_launch": nbytes,
+                     "traffic": traffic.get((dom[0], "cold")), "operand_sets": COLD_SETS,
+                     "plain_copy_cold_frac": round(nbytes / copy_cold_ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "frac_with_streaming_thread_shape": round(nbytes / streaming[dom[0]] / 1e6 / HBM_PEAK_GBS, 4)}
+    del sets
 
     cpu = None
     if not args.no_cpu:
@@ -258,12 +337,40 @@ def bench_config1(args, ops, O, wl, steps, warmup):
         getattr(O, "relu")(xo, 2.0, c["eps"], c["words"])      # warm the allocator
         s = cpu_time_s(cpu_step, reps=2)
         cpu = {"value": round(len(calls) * nbytes / s / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
-               "kind": "port", "sec_per_step": round(s, 3),
+               "cpu_model": cpu_model(), "kind": "port", "sec_per_step": round(s, 3),
                "sample": "2 full steps (6 calls each) on the identical tensors, median"}
     head = {"value": round(len(calls) * nbytes / ms_per_step / 1e6, 1), "ms_per_step": round(ms_per_step, 4),
-            "roofline": roofline, "cpu_baseline": cpu,
+            "roofline": roofline, "roofline_cold": roofline_cold, "cpu_baseline": cpu,
             "bytes_per_step": len(calls) * nbytes}
     return head, entries
+
+
+def run_cold_only(ops, wl):
+    """For counter runs (rocprofv3 --pmc ...): nothing but cold launches of the configuration-1 relaxations
+    (p = inf) and of the plain copy, each over COLD_SETS disjoint operand sets in turn, so that the per-kernel
+    averages of the counters are those of launches that find nothing in the Infinity Cache."""
+    import torch
+    from faith_amd import _lib
+    c = wl.make_config(1)
+    x = to_dev(c["x"])
+    sets = [({k: v.clone() for k, v in x.items()}, tuple(torch.empty_like(t) for t in quad(x))) for _ in range(COLD_SETS)]
+    srcs = [torch.randn(x["lw"].numel() * 2, device="cuda") for _ in range(COLD_SETS)]
+    dsts = [torch.empty_like(t) for t in srcs]
+    st = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    n = 0
+    for rnd in range(4):
+        for i in range(COLD_SETS):
+            xs, os_ = sets[i]
+            ops.relu(*quad(xs), INF, c["eps"], c["words"], out=os_)
+        for i in range(COLD_SETS):
+            xs, os_ = sets[i]
+            ops.tanh(*quad(xs), INF, c["eps"], c["words"], out=os_)
+        for i in range(COLD_SETS):
+            _lib.call("faith_copy_f32", srcs[i].data_ptr(), dsts[i].data_ptr(), srcs[i].numel(), st)
+        n += 3 * COLD_SETS
+    torch.cuda.synchronize()
+    print(json.dumps({"cold_only": True, "launches": n, "operand_sets": COLD_SETS}), flush=True)
 
 
 def bench_config2(args, ops, O, wl):
@@ -274,8 +381,9 @@ def bench_config2(args, ops, O, wl):
     out = (torch.empty(1, L, D, N, device="cuda"), torch.empty(1, L, N, device="cuda"),
            torch.empty(1, L, D, N, device="cuda"), torch.empty(1, L, N, device="cuda"))
     flop = 4 * 2 * (L * D + L) * H * N
-    t = gpu_times_ms(lambda: ops.linear(*quad(x), W, b, out=out), 10, 2)
-    tc = gpu_times_ms(lambda: ops.concretize(*out, c["p"], c["eps"], 1), 10, 2)
+    n = 10 if args.profile else 100
+    t = gpu_times_ms(lambda: ops.linear(*quad(x), W, b, out=out), n, 2)
+    tc = gpu_times_ms(lambda: ops.concretize(*out, c["p"], c["eps"], 1), n, 2)
     cpu = None
     if not args.no_cpu:
         # bounded sample: L = 32 of 256 rows (1/8 of the work), same D_in, H, N
@@ -325,8 +433,9 @@ def bench_config4(args, ops, O, wl):
     out = (torch.empty(1, D, Co, Hh, Hh, device="cuda"), torch.empty(1, Co, Hh, Hh, device="cuda"),
            torch.empty(1, D, Co, Hh, Hh, device="cuda"), torch.empty(1, Co, Hh, Hh, device="cuda"))
     flop = 4 * 2 * (D + 1) * Co * Hh * Hh * Ci * 9
-    t = gpu_times_ms(lambda: ops.conv2d(*quad(x), W, b, 1, 1, out=out), 10, 2)
-    tc = gpu_times_ms(lambda: ops.concretize_conv(*out, c["p"], c["eps"]), 10, 2)
+    n = 10 if args.profile else 100
+    t = gpu_times_ms(lambda: ops.conv2d(*quad(x), W, b, 1, 1, out=out), n, 2)
+    tc = gpu_times_ms(lambda: ops.concretize_conv(*out, c["p"], c["eps"]), n, 2)
     cpu = None
     if not args.no_cpu:
         xs = O.LinearBounds(c["x"]["lw"][:, :32], c["x"]["lb"], c["x"]["uw"][:, :32], c["x"]["ub"])
@@ -448,6 +557,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only-headline", action="store_true", help="skip configurations 0, 2, 3, 4")
     ap.add_argument("--configs", default="0,2,3,4", help="extra configurations to report under 'ops'")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="for counter runs: only cold launches of the configuration-1 relaxations and of the plain copy")
     ap.add_argument("--profile", action="store_true",
                     help="for runs under rocprofv3: warm up by count only, so the trace stays small")
     args = ap.parse_args()
@@ -469,10 +580,14 @@ def main():
     if not args.no_cpu:
         from oracle import bounds_oracle as O     # cpu_baseline leg only
 
+    if args.cold_only:
+        run_cold_only(ops, wl)
+        return
+
     prop = torch.cuda.get_device_properties(0)
     clock_mhz = measured_mfma_clock_mhz(prop.multi_processor_count)
     peak_here = prop.multi_processor_count * 256 * clock_mhz * 1e-6        # 256 fp32 MFMA flop / clock / CU
-    log(f"device: {prop.name}, {prop.multi_processor_count} CUs, host threads {torch.get_num_threads()}; shader clock "
+    log(f"device: {prop.name}, {prop.multi_processor_count} CUs, host: {cpu_model()}, {torch.get_num_threads()} threads; shader clock "
         f"under MFMA load {clock_mhz:.0f} MHz -> fp32 MFMA peak at that clock {peak_here:.1f} TFLOP/s "
         f"(roofline fractions below use the published {MFMA_FP32_PEAK_TFLOPS} TFLOP/s)")
 
@@ -505,7 +620,8 @@ def main():
                    "bytes_per_step": head["bytes_per_step"], "device": prop.name,
                    "compute_units": prop.multi_processor_count, "shader_clock_mhz_under_mfma_load": round(clock_mhz, 1),
                    "fp32_mfma_peak_at_measured_clock_tflops": round(peak_here, 1)},
-        "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "ops": entries,
+        "roofline": head["roofline"], "roofline_cold": head["roofline_cold"], "cpu_baseline": head["cpu_baseline"],
+        "ops": entries,
     }
     print(json.dumps(line), flush=True)
 

@@ -326,8 +326,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
 // column predicates and no second pass, and the kernel is a slab copy with the reduction and the
 // per-neuron stage between its loads and its stores: at configuration 1 it runs within 3 % of
 // that copy, where the general kernel above needs 25 % more.
-template <int MODE, int Q, int TPR, int NTHREADS, int RPT>
-__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4))) act_resident(const ActArgs a) {
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE))) act_resident(const ActArgs a) {
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
     static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
     extern __shared__ float smem[];
@@ -518,15 +518,17 @@ void launch_natural(const ActArgs &a, hipStream_t st) {
     const int tiles = (a.H + TH - 1) / TH;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
     const int tiles2 = (a.H2 + TH - 1) / TH;
+    faith::reserve_lds(act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>, smem);      // many perturbed words: beyond 64 KB
     hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles + a.rows2 * tiles2)),
                        dim3(NTHREADS), smem, st, a);
 }
 
-template <int MODE, int Q, int TPR, int NTHREADS, int RPT>
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4>
 void launch_resident(const ActArgs &a, hipStream_t st) {
     constexpr int TH = TPR * 4;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
-    hipLaunchKernelGGL((act_resident<MODE, Q, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS),
+    faith::reserve_lds(act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE>, smem);
+    hipLaunchKernelGGL((act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS),
                        smem, st, a);
 }
 
@@ -690,7 +692,16 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
     // straight-line kernel for the common shape: 32-neuron tiles, 32 rows in flight, up to 8 rows a thread
     const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
     if (tv != 9 && a.rows2 == 0 && a.H % 32 == 0 && a.D % 32 == 0 && a.D <= 256) {
+        // Two thread shapes for the 256-row tile.  Four wavefronts holding eight rows each are 5 % ahead
+        // while the operands can sit in the 256 MB memory-side cache (40.2 against 42.8 us at
+        // [128, 256, 512], every launch on the same 269 MB); sixteen wavefronts holding two rows each are
+        // 12 % ahead when every byte comes from and goes to HBM (55 against 62 us on the same shape with
+        // five operand sets in turn).  An object whose traffic exceeds the cache by more than a quarter
+        // cannot be resident, so it takes the second shape; knob values 7 / 8 force one or the other.
+        const long long traffic = 16LL * a.rows * a.D * a.H;
+        const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 5LL * (256LL << 20) / 4);
         if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(a, st);
+        else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8>(a, st);
         else launch_resident<MODE, Q, 8, 256, 8>(a, st);
         return;
     }

@@ -30,6 +30,17 @@ int compute_units();
 // Tuning knobs (faith_tune_set); 0 = built-in choice.
 int tune_get(int knob);
 
+// A launch that asks for more than 64 KB of dynamic LDS has to raise the kernel's limit first (160 KB per
+// workgroup on this part).  False if the request cannot be met; a launch that follows a false return fails
+// and is reported by check_launch.
+template <typename Kernel>
+inline bool reserve_lds(Kernel kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) return true;
+    if (bytes > 160 * 1024) return false;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               static_cast<int>(bytes)) == hipSuccess;
+}
+
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 inline int ceil_div(long long a, long long b) { return static_cast<int>((a + b - 1) / b); }

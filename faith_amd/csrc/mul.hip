@@ -286,6 +286,7 @@ template <int Q, int TPR, int NTHREADS, int RPT>
 void launch_mul_resident(const MulArgs &a, hipStream_t st) {
     constexpr int TH = TPR * 4;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 4 * TH + 3 * TH) * sizeof(float);
+    faith::reserve_lds(mul_resident<Q, TPR, NTHREADS, RPT>, smem);
     hipLaunchKernelGGL((mul_resident<Q, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS), smem,
                        st, a);
 }
@@ -295,6 +296,7 @@ void launch_mul(const MulArgs &a, hipStream_t st) {
     constexpr int TH = TPR * VEC;
     const int tiles = (a.H + TH - 1) / TH;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 4 * TH + 3 * TH) * sizeof(float);
+    faith::reserve_lds(mul_natural<Q, VEC, TPR, NTHREADS, RPT>, smem);
     hipLaunchKernelGGL((mul_natural<Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles)), dim3(NTHREADS), smem,
                        st, a);
 }

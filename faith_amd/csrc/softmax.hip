@@ -267,10 +267,14 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
 }
 
 template <int Q, int VEC, int NTHREADS, int RPT>
-void launch(const SoftmaxArgs &a, int tpr_log2, hipStream_t st) {
+bool launch(const SoftmaxArgs &a, int tpr_log2, hipStream_t st) {
     const int TH = (1 << tpr_log2) * VEC, NW = NTHREADS / WAVE;
     const size_t smem = ((size_t)a.words * NW * 2 * TH + 5 * TH + (size_t)a.words * NW * 2 + 2) * sizeof(float);
+    // wide slabs with several perturbed words go beyond 64 KB (H = 256, two words: 71 KB); beyond the
+    // 160 KB a workgroup can have the caller composes the four operators
+    if (!faith::reserve_lds(softmax_kernel<Q, VEC, NTHREADS, RPT>, smem)) return false;
     hipLaunchKernelGGL((softmax_kernel<Q, VEC, NTHREADS, RPT>), dim3((unsigned)a.rows), dim3(NTHREADS), smem, st, a, tpr_log2);
+    return true;
 }
 
 // The smallest workgroup whose threads hold the slab: RG * RPT >= D_in with RG = NTHREADS / TPR.
@@ -282,16 +286,14 @@ bool dispatch(const SoftmaxArgs &a, bool vec4, hipStream_t st) {
     if ((1 << k) > WAVE) return false;               // a slab row wider than a wavefront covers
     const int tpr = 1 << k;
     if (vec4) {
-        if ((256 / tpr) * 8 >= a.D) launch<Q, 4, 256, 8>(a, k, st);
-        else if ((1024 / tpr) * 8 >= a.D) launch<Q, 4, 1024, 8>(a, k, st);
-        else return false;
-    } else {
-        if ((256 / tpr) * 16 >= a.D) launch<Q, 1, 256, 16>(a, k, st);
-        else if ((1024 / tpr) * 8 >= a.D) launch<Q, 1, 1024, 8>(a, k, st);
-        else if ((1024 / tpr) * 24 >= a.D) launch<Q, 1, 1024, 24>(a, k, st);
-        else return false;
+        if ((256 / tpr) * 8 >= a.D) return launch<Q, 4, 256, 8>(a, k, st);
+        if ((1024 / tpr) * 8 >= a.D) return launch<Q, 4, 1024, 8>(a, k, st);
+        return false;
     }
-    return true;
+    if ((256 / tpr) * 16 >= a.D) return launch<Q, 1, 256, 16>(a, k, st);
+    if ((1024 / tpr) * 8 >= a.D) return launch<Q, 1, 1024, 8>(a, k, st);
+    if ((1024 / tpr) * 24 >= a.D) return launch<Q, 1, 1024, 24>(a, k, st);
+    return false;
 }
 
 }  // namespace
@@ -331,8 +333,8 @@ extern "C" int faith_softmax_verification(const float *src_lb, const float *src_
         default: ok = dispatch<Q_GENERAL>(a, vec4, st); break;
     }
     if (!ok) {
-        faith::set_error("faith_softmax_verification: a [dim_in=%d, dim_out=%d] slab does not fit the registers of one "
-                         "workgroup (see faith_softmax_fits); compose exp, row sum, reciprocal and multiply instead",
+        faith::set_error("faith_softmax_verification: a [dim_in=%d, dim_out=%d] slab does not fit the registers (see "
+                         "faith_softmax_fits) or, with many perturbed words, the 160 KB of LDS of one workgroup; compose exp, row sum, reciprocal and multiply instead",
                          dim_in, dim_out);
         return FAITH_ERR_UNSUPPORTED;
     }

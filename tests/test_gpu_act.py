@@ -70,6 +70,43 @@ def test_activation_small_shapes(kind, p, layout):
         check(kind, x, p, 0.05, words, layout)
 
 
+@pytest.mark.parametrize("kind", ["concretize", "relu", "tanh"])
+@pytest.mark.parametrize("words", [8, 16])
+def test_many_perturbed_words_need_more_than_64_kb_of_lds(kind, words):
+    """The partial norms of every word and wavefront sit in LDS: with 8 or 16 words the sixteen-wavefront
+    tiles ask for 67 ... 133 KB, beyond the 64 KB a launch gets without asking."""
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(9)
+    for (L, D, H) in [(2, 64, 64), (2, 1024, 64), (1, 256, 96), (1, 2048, 40)]:
+        x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+        if kind == "concretize":
+            l, u = ops.concretize(*dev(*x.tensors()), 2.0, 0.05, words)
+            el, eu = O.concretize(x, 2.0, 0.05, words)
+            assert close(l, el) and close(u, eu), (L, D, H, words)
+        else:
+            check(kind, x, 2.0, 0.05, words)
+
+
+@pytest.mark.parametrize("kind", ["relu", "tanh"])
+@pytest.mark.parametrize("p", PS)
+def test_thread_shape_for_hbm_streams_gives_the_same_values(kind, p):
+    """Objects too large for the memory-side cache take sixteen wavefronts of two rows instead of four of
+    eight (tuning knob 7 forces that shape on a small object): same tile, same reduction tree per column
+    group, checked against the oracle and against the default shape."""
+    from faith_amd import _lib, ops
+    g = torch.Generator().manual_seed(10)
+    x = rand_bounds(g, 1, 3, 256, 96, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+    ref = getattr(ops, kind)(*dev(*x.tensors()), p, 0.05, 2)
+    _lib.call("faith_tune_set", 0, 7)
+    try:
+        check(kind, x, p, 0.05, 2)
+        got = getattr(ops, kind)(*dev(*x.tensors()), p, 0.05, 2)
+    finally:
+        _lib.call("faith_tune_set", 0, 0)
+    for a, b in zip(got, ref):
+        assert close(a, b.cpu())
+
+
 @pytest.mark.parametrize("kind", ["relu", "tanh"])
 def test_activation_reference_test_distribution(kind):
     """Inputs drawn as the reference's own op test draws them

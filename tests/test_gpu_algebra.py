@@ -89,6 +89,8 @@ SOFTMAX_SHAPES = [
     (1, 3, 256, 31, 1),      # a sentence of 31 tokens at dim_in 256: 1024 threads, one column each
     (1, 2, 300, 50, 1),      # 1024 threads, 24 rows per thread
     (1, 2, 20, 1, 1),        # softmax of a single score
+    (1, 2, 64, 256, 2),      # sixteen wavefronts, a full wavefront a row, two words: 71 KB of LDS
+    (1, 2, 32, 256, 4),      # the same with four words: 137 KB
 ]
 
 

@@ -84,7 +84,17 @@ def test_relaxation_rows(op, p, layout, shape):
     fn = getattr(ops, op)
     full = fn(*x, p, 0.01, 2, lay, True)
     picks = rows_to_check(L, A * B)
-    check_rows(f"{op} {layout}", full, lambda r: fn(*sl(x, r), p, 0.01, 2, lay, True), picks)
+    # an object of this size streams from HBM and takes the register-resident kernel's sixteen-wavefront
+    # thread shape; a single row would take the four-wavefront one (another reduction tree), so the slices
+    # are held to the shape of the whole (tuning knob 7) and the comparison stays bit for bit
+    from faith_amd import _lib
+    resident = layout == "natural" and A <= 256
+    if resident:
+        _lib.call("faith_tune_set", 0, 7)
+    try:
+        check_rows(f"{op} {layout}", full, lambda r: fn(*sl(x, r), p, 0.01, 2, lay, True), picks)
+    finally:
+        _lib.call("faith_tune_set", 0, 0)
     conc = ops.concretize(*x, p, 0.01, 2, lay)
     check_rows(f"concretize {layout}", conc, lambda r: ops.concretize(*sl(x, r), p, 0.01, 2, lay), picks)
     same(conc[0], full[4], "interval of the relaxation against concretize (l)", False)
