@@ -52,40 +52,35 @@ def c_tanh_verification(src_lb, src_ub, src_lw, src_uw, out_lb, out_ub, out_lw, 
          length, dim_in, dim_out, epsilon)
 
 
+def _dot(entry, x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw,
+         batch_size, length_x, length_y, dim_out, dim_in, epsilon):
+    for n, t in (("x_l", x_l), ("y_l", y_l), ("x_u", x_u), ("y_u", y_u), ("x_lb", x_lb), ("x_ub", x_ub), ("y_lb", y_lb),
+                 ("y_ub", y_ub), ("x_lw", x_lw), ("x_uw", x_uw), ("y_lw", y_lw), ("y_uw", y_uw), ("z_lb", z_lb),
+                 ("z_ub", z_ub), ("z_lw", z_lw), ("z_uw", z_uw)):
+        ops._check(n, t)
+    with torch.cuda.device(x_lw.device):
+        _lib.call(entry, x_l.data_ptr(), y_l.data_ptr(), x_u.data_ptr(), y_u.data_ptr(), x_lb.data_ptr(), x_ub.data_ptr(),
+                  y_lb.data_ptr(), y_ub.data_ptr(), x_lw.data_ptr(), x_uw.data_ptr(), y_lw.data_ptr(), y_uw.data_ptr(),
+                  z_lb.data_ptr(), z_ub.data_ptr(), z_lw.data_ptr(), z_uw.data_ptr(), batch_size, length_x, length_y,
+                  dim_out, dim_in, float(epsilon), ops.q_code(p), int(words), _lib.LAYOUT_TRANSPOSED, _s(x_lw))
+
+
 def c_dot_product_verification_QK(x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
                                   z_lb, z_ub, z_lw, z_uw, batch_size, length, dim_out, dim_in, epsilon):
-    """kernel.cpp:133-186.  x_lw .. y_uw are [B, L, dim_out, dim_in]; z_lw, z_uw are [B, L, L, dim_in].
-
-    The contraction kernel works on the natural layout, so this compatibility entry
-    re-lays the transposed operands out with torch copies before and after the call;
-    callers that keep the natural layout (faith_amd.Bounds) pay none of that.
-    """
-    nat = [t.transpose(2, 3).contiguous() for t in (x_lw, x_uw, y_lw, y_uw)]
-    zlw, zlb, zuw, zub, (xl, xu, yl, yu) = ops.dot_product_qk(
-        (nat[0], x_lb.contiguous(), nat[1], x_ub.contiguous()),
-        (nat[2], y_lb.contiguous(), nat[3], y_ub.contiguous()),
-        p, epsilon, words, return_intervals=True)
-    z_lw.copy_(zlw.transpose(2, 3)); z_uw.copy_(zuw.transpose(2, 3))
-    z_lb.copy_(zlb); z_ub.copy_(zub)
-    x_l.copy_(xl); x_u.copy_(xu); y_l.copy_(yl); y_u.copy_(yu)
+    """kernel.cpp:133-186.  x_lw .. y_uw are [B, L, dim_out, dim_in]; z_lw, z_uw are [B, L, L, dim_in]: the
+    library takes these tensors as they are (FAITH_LAYOUT_TRANSPOSED), nothing is copied.  x and y may differ
+    in length (the lengths are read off the tensors; `length` is the reference's single argument)."""
+    _dot("faith_dot_product_verification_QK", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
+         z_lb, z_ub, z_lw, z_uw, batch_size, x_lw.shape[1], y_lw.shape[1], dim_out, dim_in, epsilon)
 
 
 def c_dot_product_verification_V(x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
                                  z_lb, z_ub, z_lw, z_uw, batch_size, length, dim_out, dim_in, epsilon):
     """kernel.cpp:188-241; adapter Bounds.py:1306-1343.  x_* is the probability object with lw transposed
     to [B, L, L, dim_in]; y_* is the TRANSPOSED value object (lb [B, dim_out, L], lw [B, dim_out, L, dim_in]);
-    z_lw, z_uw are [B, L, dim_out, dim_in].  The kernel reads values in their natural layout, so this
-    compatibility entry re-lays the operands out with torch copies, as the QK entry does."""
-    xn = [t.transpose(2, 3).contiguous() for t in (x_lw, x_uw)]                    # [B, L, dim_in, L]
-    yn = [t.permute(0, 2, 3, 1).contiguous() for t in (y_lw, y_uw)]                # [B, L, dim_in, dim_out]
-    ylb, yub = y_lb.transpose(1, 2).contiguous(), y_ub.transpose(1, 2).contiguous()  # [B, L, dim_out]
-    zlw, zlb, zuw, zub, (xl, xu, yl, yu) = ops.dot_product_v(
-        (xn[0], x_lb.contiguous(), xn[1], x_ub.contiguous()), (yn[0], ylb, yn[1], yub),
-        p, epsilon, words, return_intervals=True)
-    z_lw.copy_(zlw.transpose(2, 3)); z_uw.copy_(zuw.transpose(2, 3))
-    z_lb.copy_(zlb); z_ub.copy_(zub)
-    x_l.copy_(xl); x_u.copy_(xu)
-    y_l.copy_(yl.transpose(1, 2)); y_u.copy_(yu.transpose(1, 2))
+    z_lw, z_uw are [B, L, dim_out, dim_in].  Taken as they are (FAITH_LAYOUT_TRANSPOSED), nothing is copied."""
+    _dot("faith_dot_product_verification_V", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
+         z_lb, z_ub, z_lw, z_uw, batch_size, x_lw.shape[1], x_lw.shape[2], dim_out, dim_in, epsilon)
 
 
 def c_matmul_verification(x_lb, x_ub, x_lw, x_uw, W, y_lb, y_ub, y_lw, y_uw,

@@ -104,17 +104,11 @@ __device__ __forceinline__ float4 ld4(__amdgpu_buffer_rsrc_t r, unsigned thread_
 __device__ __forceinline__ void st1_nt(float v, __amdgpu_buffer_rsrc_t r, unsigned thread_off, unsigned uniform_off) {
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, thread_off, uniform_off, 2 /* non-temporal */);
 }
-// max(v, 0) / min(v, 0) as single instructions (fmaxf / fminf add a canonicalising v_max each)
-__device__ __forceinline__ float pos1(float v) {
-    float r;
-    asm("v_max_f32 %0, 0, %1" : "=v"(r) : "v"(v));
-    return r;
-}
-__device__ __forceinline__ float neg1(float v) {
-    float r;
-    asm("v_min_f32 %0, 0, %1" : "=v"(r) : "v"(v));
-    return r;
-}
+// max(v, 0) / min(v, 0) as one instruction each, as a median of three with +-infinity: fmaxf / fminf come with a
+// canonicalising v_max each, and the compiler sees this form (no inline assembly whose result an MFMA or an LDS
+// store could consume before the hazard recognizer knows it was written)
+__device__ __forceinline__ float pos1(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, __builtin_inff()); }
+__device__ __forceinline__ float neg1(float v) { return __builtin_amdgcn_fmed3f(v, -__builtin_inff(), 0.f); }
 __device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
 __device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
 
@@ -922,6 +916,182 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     return faith::check_launch(who);
 }
 
+// ------------------------------------------------------------------------------------------
+// Transposed layout: what the reference's adapters hand to its kernels (Bounds.py:1279-1290, :1319-1329;
+// kernel.cpp:133-241).  Coefficients are [B, L, K, D_in] with the perturbation coordinate m contiguous,
+// K the reduction axis (head size for the scores; key positions for the context, where y is the value
+// object already transposed to [B, width, keys, D_in]), and the result is z [B, Lx, Ly, D_in]:
+//     z[i, j, m] = sum_k  x[i, k, m] a[j, k] + b[i, k] y[j, k, m]        (a, b split by sign as above).
+// A fixed-m slice of an operand is a 4-byte gather here, so the MFMA tiling of the natural layout (rows i,
+// columns j, one m per tile) would read 4 bytes per 128-byte line.  Lanes run along m instead: every load and
+// store of a wavefront is one contiguous 256-byte run, the coefficients a[j, k], b[i, k] are wave-uniform
+// (scalar loads), and each lane keeps an RI x RJ block of (i, j) pairs for its m in registers -- 8 RI RJ
+// fused multiply-adds per 2 (RI + RJ) loads.  Vector ALU, not MFMA: this is the compatibility layout;
+// callers that keep the natural layout take the MFMA kernels above.
+// ------------------------------------------------------------------------------------------
+struct DotTArgs {
+    const float *xlw, *xuw, *ylw, *yuw;   // [B, Lx, K, D], [B, Ly, K, D]
+    const float *x_l, *y_l, *y_u;         // [B, Lx, K], [B, Ly, K]
+    float *zlw, *zuw;                     // [B, Lx, Ly, D]
+    int B, Lx, Ly, K, D;
+    int mw;                               // wavefronts of a workgroup along m (1, 2 or 4); the others along j
+    int n_i, n_j, n_m;                    // blocks along i, j, m
+};
+
+template <int RI, int RJ>
+__global__ void __launch_bounds__(256) dot_w_transposed(const DotTArgs g) {
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);     // wave-uniform by construction
+    const int wm = wave % g.mw, wj = wave / g.mw, jw = 4 / g.mw;
+    int blk = blockIdx.x;
+    const int mb = blk % g.n_m;  blk /= g.n_m;
+    const int jb = blk % g.n_j;  blk /= g.n_j;
+    const int ib = blk % g.n_i;
+    const int t = blk / g.n_i;
+    const int m = (mb * g.mw + wm) * 64 + lane;
+    const int i0 = ib * RI, j0 = (jb * jw + wj) * RJ;
+    if (j0 >= g.Ly) return;                                  // a wavefront without columns (no barrier below)
+    const bool m_ok = m < g.D;
+    const int mc = m_ok ? m : g.D - 1;                       // out-of-range lanes read a valid address, store nothing
+
+    // Buffer addressing: one window per tensor and (batch, head) pair, a wave-uniform byte offset per row
+    // (scalar registers, advanced by one k per step) and the lane's own offset m.  Rows past the end repeat
+    // the last one; their results are not stored.  The coefficients a[j, k], b[i, k] are scalar loads.
+    const size_t xh = (size_t)g.Lx * g.K * g.D, yh = (size_t)g.Ly * g.K * g.D;      // floats of one head
+    const __amdgpu_buffer_rsrc_t wxl = window(g.xlw + t * xh, clamp32(xh * 4)), wxu = window(g.xuw + t * xh, clamp32(xh * 4));
+    const __amdgpu_buffer_rsrc_t wyl = window(g.ylw + t * yh, clamp32(yh * 4)), wyu = window(g.yuw + t * yh, clamp32(yh * 4));
+    // the concrete intervals were written by an earlier launch and do not change during this one: read through
+    // the constant address space, a wave-uniform address there is a scalar load
+    typedef const float __attribute__((address_space(4))) *uniform_ptr;
+    const uniform_ptr cb = (uniform_ptr)(g.x_l + (size_t)t * g.Lx * g.K);
+    const uniform_ptr cal = (uniform_ptr)(g.y_l + (size_t)t * g.Ly * g.K), cau = (uniform_ptr)(g.y_u + (size_t)t * g.Ly * g.K);
+    const unsigned vm = (unsigned)mc * 4u, kstep = (unsigned)g.D * 4u;
+    unsigned xo[RI], yo[RJ], bo[RI], ao[RJ];
+#pragma unroll
+    for (int a = 0; a < RI; ++a) {
+        const unsigned i = i0 + a < g.Lx ? i0 + a : g.Lx - 1;
+        xo[a] = i * (unsigned)g.K * kstep;
+        bo[a] = i * (unsigned)g.K;
+    }
+#pragma unroll
+    for (int c = 0; c < RJ; ++c) {
+        const unsigned j = j0 + c < g.Ly ? j0 + c : g.Ly - 1;
+        yo[c] = j * (unsigned)g.K * kstep;
+        ao[c] = j * (unsigned)g.K;
+    }
+    float zl[RI][RJ], zu[RI][RJ];
+#pragma unroll
+    for (int a = 0; a < RI; ++a)
+#pragma unroll
+        for (int c = 0; c < RJ; ++c) zl[a][c] = zu[a][c] = 0.f;
+
+#pragma unroll 1
+    for (int k = 0; k < g.K; ++k) {
+        float xl[RI], xu[RI], yl[RJ], yu[RJ], bp[RI], bn[RI], alp[RJ], aln[RJ], aup[RJ], aun[RJ];
+#pragma unroll
+        for (int a = 0; a < RI; ++a) {
+            xl[a] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wxl, vm, xo[a], 0));
+            xu[a] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wxu, vm, xo[a], 0));
+            const float b = cb[bo[a] + k];
+            bp[a] = pos1(b);
+            bn[a] = neg1(b);
+            xo[a] += kstep;
+        }
+#pragma unroll
+        for (int c = 0; c < RJ; ++c) {
+            yl[c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wyl, vm, yo[c], 0));
+            yu[c] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wyu, vm, yo[c], 0));
+            const float al = cal[ao[c] + k], au = cau[ao[c] + k];
+            alp[c] = pos1(al);  aln[c] = neg1(al);
+            aup[c] = pos1(au);  aun[c] = neg1(au);
+            yo[c] += kstep;
+        }
+#pragma unroll
+        for (int a = 0; a < RI; ++a)
+#pragma unroll
+            for (int c = 0; c < RJ; ++c) {
+                float l = zl[a][c], u = zu[a][c];
+                l = __builtin_fmaf(xl[a], alp[c], l);  u = __builtin_fmaf(xu[a], aup[c], u);
+                l = __builtin_fmaf(xu[a], aln[c], l);  u = __builtin_fmaf(xl[a], aun[c], u);
+                l = __builtin_fmaf(bp[a], yl[c], l);   u = __builtin_fmaf(bp[a], yu[c], u);
+                l = __builtin_fmaf(bn[a], yu[c], l);   u = __builtin_fmaf(bn[a], yl[c], u);
+                zl[a][c] = l;  zu[a][c] = u;
+            }
+    }
+    if (!m_ok) return;
+#pragma unroll
+    for (int a = 0; a < RI; ++a) {
+        if (i0 + a >= g.Lx) break;
+#pragma unroll
+        for (int c = 0; c < RJ; ++c) {
+            if (j0 + c >= g.Ly) break;
+            const size_t z = (((size_t)t * g.Lx + i0 + a) * g.Ly + j0 + c) * g.D + m;
+            __builtin_nontemporal_store(zl[a][c], g.zlw + z);
+            __builtin_nontemporal_store(zu[a][c], g.zuw + z);
+        }
+    }
+}
+
+// Both entry points in the transposed layout: `K` is the reduction length (head size for the scores, key
+// positions for the context), `Ly` the number of result columns (key positions / width of the values).
+int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
+                         const float *x_ub, const float *y_lb, const float *y_ub, const float *x_lw, const float *x_uw,
+                         const float *y_lw, const float *y_uw, float *z_lb, float *z_ub, float *z_lw, float *z_uw, int B,
+                         int Lx, int Ly, int K, int D, float epsilon, int q, int words, void *stream) {
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
+    FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
+    FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_ALIGNED4(z_lw); FAITH_ALIGNED4(z_uw); FAITH_ALIGNED4(z_lb); FAITH_ALIGNED4(z_ub);
+    FAITH_REQUIRE(B > 0 && Lx > 0 && Ly > 0 && K > 0 && D > 0, FAITH_ERR_SHAPE,
+                  "%s: batch=%d rows of x=%d columns of z=%d reduction length=%d dim_in=%d must be positive", who, B, Lx,
+                  Ly, K, D);
+    FAITH_REQUIRE((long long)B * (Lx > Ly ? Lx : Ly) * K <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "%s: batch * length * reduction length exceeds 2^31", who);
+    FAITH_REQUIRE(words >= 1 && (D == 1 || D % words == 0), FAITH_ERR_SHAPE, "%s: words=%d must divide dim_in=%d", who, words, D);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    // concrete intervals of both objects: [B * L, K] neurons whose D_in coefficients are contiguous
+    const bool empty_blocks = D == 1 && words > 1;      // Bounds.py:319-326 with dim_in // words == 0: the constant terms
+    const float eps = empty_blocks ? 0.f : epsilon;
+    const int w = empty_blocks ? 1 : words;
+    int rc = faith_concretize(x_lb, x_ub, x_lw, x_uw, x_l, x_u, B * Lx, D, K, eps, q, w, FAITH_LAYOUT_TRANSPOSED, stream);
+    if (rc != FAITH_OK) return rc;
+    rc = faith_concretize(y_lb, y_ub, y_lw, y_uw, y_l, y_u, B * Ly, D, K, eps, q, w, FAITH_LAYOUT_TRANSPOSED, stream);
+    if (rc != FAITH_OK) return rc;
+
+    // constant terms and the dim_in == 1 shortcut do not involve the coefficient layout: the kernels of the
+    // natural layout serve (scores form: rows of x and of y, reduction over their last axis)
+    DotArgs g{x_lw, x_uw, y_lw, y_uw, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, z_lw, z_uw, z_lb, z_ub, B, Lx, Ly, D, K};
+    g.ox = {K, 1, K};
+    g.oy = {K, 1, K};
+    g.oz = {Ly, 1, Ly};
+    g.heads = 1;
+    g.side_by_side = 0;
+    if (D == 1) {
+        const long long n = (long long)B * Lx * Ly;      // z_lw [B, Lx, Ly, 1] and [B, Lx, 1, Ly] coincide
+        hipLaunchKernelGGL(dot_interval<false>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, g);
+        return faith::check_launch(who);
+    }
+    const long long b_tiles = (long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T);
+    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    hipLaunchKernelGGL(dot_b<false>, dim3((unsigned)b_tiles), dim3(256), 0, st, g);
+
+    FAITH_REQUIRE((long long)(Lx > Ly ? Lx : Ly) * K * D * 4 < 0xffffffffLL, FAITH_ERR_UNSUPPORTED,
+                  "%s: the coefficients of one batch element exceed 4 GB in the transposed layout (32-bit offsets)", who);
+    constexpr int RI = 4, RJ = 8;
+    DotTArgs a{x_lw, x_uw, y_lw, y_uw, x_l, y_l, y_u, z_lw, z_uw, B, Lx, Ly, K, D};
+    a.mw = D > 128 ? 4 : D > 64 ? 2 : 1;
+    a.n_i = (Lx + RI - 1) / RI;
+    a.n_j = (Ly + RJ * (4 / a.mw) - 1) / (RJ * (4 / a.mw));
+    a.n_m = (D + 64 * a.mw - 1) / (64 * a.mw);
+    const long long grid = (long long)B * a.n_i * a.n_j * a.n_m;
+    FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    hipLaunchKernelGGL((dot_w_transposed<RI, RJ>), dim3((unsigned)grid), dim3(256), 0, st, a);
+    return faith::check_launch(who);
+}
+
 }  // namespace
 
 extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
@@ -930,7 +1100,12 @@ extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *
                                                  const float *y_uw, float *z_lb, float *z_ub, float *z_lw,
                                                  float *z_uw, int batch_size, int length_x, int length_y,
                                                  int dim_out, int dim_in, float epsilon, int q, int words,
-                                                 void *stream) {
+                                                 int layout, void *stream) {
+    if (layout == FAITH_LAYOUT_TRANSPOSED)
+        return dot_entry_transposed("faith_dot_product_verification_QK", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw,
+                                    x_uw, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, length_y, dim_out,
+                                    dim_in, epsilon, q, words, stream);
+    FAITH_REQUIRE(layout == FAITH_LAYOUT_NATURAL, FAITH_ERR_UNSUPPORTED, "faith_dot_product_verification_QK: unknown layout %d", layout);
     return dot_entry<false>("faith_dot_product_verification_QK", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
                             y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, length_y, dim_out, dim_in, epsilon,
                             q, words, 0, 1, stream);
@@ -941,7 +1116,12 @@ extern "C" int faith_dot_product_verification_V(float *x_l, float *y_l, float *x
                                                 const float *x_lw, const float *x_uw, const float *y_lw,
                                                 const float *y_uw, float *z_lb, float *z_ub, float *z_lw,
                                                 float *z_uw, int batch_size, int length_x, int length_k, int dim_out,
-                                                int dim_in, float epsilon, int q, int words, void *stream) {
+                                                int dim_in, float epsilon, int q, int words, int layout, void *stream) {
+    if (layout == FAITH_LAYOUT_TRANSPOSED)      // y is the value object transposed: [batch, dim_out, length_k, dim_in]
+        return dot_entry_transposed("faith_dot_product_verification_V", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw,
+                                    x_uw, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, dim_out, length_k,
+                                    dim_in, epsilon, q, words, stream);
+    FAITH_REQUIRE(layout == FAITH_LAYOUT_NATURAL, FAITH_ERR_UNSUPPORTED, "faith_dot_product_verification_V: unknown layout %d", layout);
     return dot_entry<true>("faith_dot_product_verification_V", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw,
                            y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size, length_x, dim_out, length_k, dim_in, epsilon,
                            q, words, 0, 1, stream);
@@ -990,7 +1170,7 @@ extern "C" int faith_dot_product_verification_QK_static(const float *x_lb, const
                                                         const float *y_lw, const float *y_uw, float *z_lb, float *z_ub,
                                                         float *z_lw, float *z_uw, int batch_size, int length_x,
                                                         int length_y, int dim_out, int dim_in, float epsilon, int q,
-                                                        int words, void *stream) {
+                                                        int words, int layout, void *stream) {
     const char *who = "faith_dot_product_verification_QK_static";
     FAITH_REQUIRE(batch_size > 0 && length_x > 0 && length_y > 0 && dim_out > 0 && dim_in > 0, FAITH_ERR_SHAPE,
                   "%s: batch=%d length_x=%d length_y=%d dim_out=%d dim_in=%d must be positive", who, batch_size, length_x,
@@ -1006,6 +1186,10 @@ extern "C" int faith_dot_product_verification_QK_static(const float *x_lb, const
     const int rc = scratch_address(who, &base);
     if (rc != FAITH_OK) return rc;
     float *x_l = base, *x_u = base + nx, *y_l = base + 2 * nx, *y_u = base + 2 * nx + ny;
+    if (layout == FAITH_LAYOUT_TRANSPOSED)
+        return dot_entry_transposed(who, x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw, z_lb, z_ub, z_lw,
+                                    z_uw, batch_size, length_x, length_y, dim_out, dim_in, epsilon, q, words, stream);
+    FAITH_REQUIRE(layout == FAITH_LAYOUT_NATURAL, FAITH_ERR_UNSUPPORTED, "%s: unknown layout %d", who, layout);
     return dot_entry<false>(who, x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw,
                             batch_size, length_x, length_y, dim_out, dim_in, epsilon, q, words, 0, 1, stream);
 }

@@ -29,7 +29,17 @@ def q_code(p: float) -> int:
     raise ValueError(f"p={p}: the perturbation norm must be >= 1")
 
 
+_F32 = torch.float32
+
+
 def _check(name, t, shape=None):
+    # one expression for the tensor that is fine (a small launch is bound by its host side); the
+    # detailed tests below only run to name what is wrong
+    try:
+        if t.is_cuda and t.dtype is _F32 and t.is_contiguous() and (shape is None or t.shape == shape):
+            return t
+    except AttributeError:
+        pass
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name}: expected a tensor, got {type(t).__name__}")
     if not t.is_cuda:
@@ -38,7 +48,7 @@ def _check(name, t, shape=None):
         raise TypeError(f"{name}: must be float32, got {t.dtype}")
     if not t.is_contiguous():
         raise ValueError(f"{name}: must be contiguous")
-    if shape is not None and t.shape != shape and tuple(t.shape) != tuple(shape):      # torch.Size is a tuple
+    if shape is not None and tuple(t.shape) != tuple(shape):
         raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
     return t
 
@@ -376,9 +386,11 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     return olw, olb, ouw, oub
 
 
-def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1):
+def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1, out=None):
     """linear() and concretize() of its result through one entry point (one launch for small problems).
-    Returns (lw', lb', uw', ub', l, u)."""
+    Returns (lw', lb', uw', ub', l, u).  `out`: the six result tensors, owned by the caller as in the
+    reference's interface (Bounds.py:1270-1277); a small layer is bound by its host side, and six
+    allocations are a third of it."""
     B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
     _check("weight", weight)
@@ -387,12 +399,18 @@ def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1):
     N = weight.shape[0]
     if bias is not None:
         _check("bias", bias, (N,))
-    olw = torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32)
-    ouw = torch.empty_like(olw)
-    olb = torch.empty(B, L, N, device=lw.device, dtype=torch.float32)
-    oub = torch.empty_like(olb)
-    l = torch.empty_like(olb)
-    u = torch.empty_like(olb)
+    if out is None:
+        olw = torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32)
+        ouw = torch.empty_like(olw)
+        olb = torch.empty(B, L, N, device=lw.device, dtype=torch.float32)
+        oub = torch.empty_like(olb)
+        l = torch.empty_like(olb)
+        u = torch.empty_like(olb)
+    else:
+        olw, olb, ouw, oub, l, u = out
+        _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
+        for name, t in (("out lb", olb), ("out ub", oub), ("out l", l), ("out u", u)):
+            _check(name, t, (B, L, N))
     with _on(lw.device, "linear", (B * L * D, H, N)):
         _lib.call("faith_matmul_concretize_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight),
                   _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), _ptr(l), _ptr(u), B, L, D, H, N,
@@ -460,7 +478,7 @@ def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
         _lib.call("faith_dot_product_verification_QK", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Ly, d, D, float(eps), q_code(p), int(words),
-                  _stream(xlw))
+                  LAYOUT_NATURAL, _stream(xlw))
     if return_intervals:
         return zlw, zlb, zuw, zub, (x_l, x_u, y_l, y_u)
     return zlw, zlb, zuw, zub
@@ -497,7 +515,7 @@ def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
         _lib.call("faith_dot_product_verification_V", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
                   _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, Lx, Lk, dv, D, float(eps), q_code(p), int(words),
-                  _stream(xlw))
+                  LAYOUT_NATURAL, _stream(xlw))
     if return_intervals:
         return zlw, zlb, zuw, zub, (x_l, x_u, y_l, y_u)
     return zlw, zlb, zuw, zub

@@ -279,12 +279,19 @@ int faith_matmul_group_verification(const float *x_lb, const float *x_ub,
 /*
  * McCormick bounds of the attention scores  z[i,j] = sum_k x[i,k] * y[j,k].  Replaces
  * call_dot_product_verification_QK (kernel.cpp:45-51, dot_product_verification.cu:458-496)
- * with the arithmetic of Bounds.ori_dot_product (Bounds.py:710-823).  Natural layout:
- *   x_lw, x_uw [batch, length_x, dim_in, dim_out];  x_lb, x_ub [batch, length_x, dim_out]
- *   y_lw, y_uw [batch, length_y, dim_in, dim_out];  y_lb, y_ub [batch, length_y, dim_out]
+ * with the arithmetic of Bounds.ori_dot_product (Bounds.py:710-823).
+ * layout = FAITH_LAYOUT_NATURAL:
+ *   x_lw, x_uw [batch, length_x, dim_in, dim_out];  y_lw, y_uw [batch, length_y, dim_in, dim_out]
+ *   z_lw, z_uw [batch, length_x, dim_in, length_y]
+ * layout = FAITH_LAYOUT_TRANSPOSED -- what the reference's adapter passes (Bounds.py:1279-1290,
+ * kernel.cpp:133-186):
+ *   x_lw, x_uw [batch, length_x, dim_out, dim_in];  y_lw, y_uw [batch, length_y, dim_out, dim_in]
+ *   z_lw, z_uw [batch, length_x, length_y, dim_in]
+ * Either way:
+ *   x_lb, x_ub [batch, length_x, dim_out];  y_lb, y_ub [batch, length_y, dim_out]
  *   x_l, x_u   [batch, length_x, dim_out]  (out: concrete interval of x; caller's scratch)
  *   y_l, y_u   [batch, length_y, dim_out]  (out: concrete interval of y)
- *   z_lw, z_uw [batch, length_x, dim_in, length_y];  z_lb, z_ub [batch, length_x, length_y]
+ *   z_lb, z_ub [batch, length_x, length_y]
  * The reference entry has one `length`; here x and y may differ in length.  With dim_in == 1 the
  * result is the interval product of the constant terms (Bounds.py:711-721); x_l .. y_u are written
  * all the same.  words must divide dim_in.
@@ -297,7 +304,7 @@ int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float 
                                       float *z_lb, float *z_ub, float *z_lw, float *z_uw,
                                       int batch_size, int length_x, int length_y,
                                       int dim_out, int dim_in, float epsilon,
-                                      int q, int words, void *stream);
+                                      int q, int words, int layout, void *stream);
 
 /*
  * faith_dot_product_verification_QK for callers that cannot allocate (code under HIP graph capture,
@@ -317,18 +324,25 @@ int faith_dot_product_verification_QK_static(const float *x_lb, const float *x_u
                                              float *z_lb, float *z_ub, float *z_lw, float *z_uw,
                                              int batch_size, int length_x, int length_y,
                                              int dim_out, int dim_in, float epsilon,
-                                             int q, int words, void *stream);
+                                             int q, int words, int layout, void *stream);
 
 /*
  * McCormick bounds of the attention context  z[i,j] = sum_k x[i,k] * y[k,j]  (probabilities times
  * values).  Replaces call_dot_product_verification_V (kernel.cpp:53-60,
  * dot_product_verification.cu:498-535) with the arithmetic of Bounds.context -> ori_dot_product
- * (Bounds.py:843-850, :710-823).  The value bounds are taken in their own natural layout: the
- * transposed views that Bounds.t() builds (Bounds.py:335-346) are never materialised.
+ * (Bounds.py:843-850, :710-823).
+ * layout = FAITH_LAYOUT_NATURAL: the value bounds are taken in their own natural layout; the transposed
+ * views that Bounds.t() builds (Bounds.py:335-346) are never materialised.
  *   x_lw, x_uw [batch, length_x, dim_in, length_k];  x_lb, x_ub [batch, length_x, length_k]
  *   y_lw, y_uw [batch, length_k, dim_in, dim_out];   y_lb, y_ub [batch, length_k, dim_out]
  *   x_l, x_u   [batch, length_x, length_k];  y_l, y_u [batch, length_k, dim_out]   (out / scratch)
  *   z_lw, z_uw [batch, length_x, dim_in, dim_out];   z_lb, z_ub [batch, length_x, dim_out]
+ * layout = FAITH_LAYOUT_TRANSPOSED -- what the reference's adapter passes (Bounds.py:1306-1329,
+ * kernel.cpp:188-241): y is the value object after Bounds.t(), and every coefficient array has dim_in last.
+ *   x_lw, x_uw [batch, length_x, length_k, dim_in];  x_lb, x_ub [batch, length_x, length_k]
+ *   y_lw, y_uw [batch, dim_out, length_k, dim_in];   y_lb, y_ub [batch, dim_out, length_k]
+ *   x_l, x_u   [batch, length_x, length_k];  y_l, y_u [batch, dim_out, length_k]   (out / scratch)
+ *   z_lw, z_uw [batch, length_x, dim_out, dim_in];   z_lb, z_ub [batch, length_x, dim_out]
  */
 int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *y_u,
                                      const float *x_lb, const float *x_ub,
@@ -338,7 +352,7 @@ int faith_dot_product_verification_V(float *x_l, float *y_l, float *x_u, float *
                                      float *z_lb, float *z_ub, float *z_lw, float *z_uw,
                                      int batch_size, int length_x, int length_k,
                                      int dim_out, int dim_in, float epsilon,
-                                     int q, int words, void *stream);
+                                     int q, int words, int layout, void *stream);
 
 /*
  * Interval bound propagation (the reference's method "ibp": the `if self.ibp` branches of

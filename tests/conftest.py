@@ -46,11 +46,13 @@ def pytest_terminal_summary(terminalreporter):
     led = _ledger()
     if not led["comparisons"]:
         return
-    kinds = {}
+    kinds, per_test = {}, {}
     for c in led["concessions"]:
         kinds[c["kind"]] = kinds.get(c["kind"], 0) + 1
+        fn = c["test"].split("[")[0]
+        per_test[(fn, c["kind"], c["tensor"])] = per_test.get((fn, c["kind"], c["tensor"]), 0) + 1
     terminalreporter.write_line(
         f"parity ledger: {led['comparisons']} harness comparisons, {led['plain']} on the plain bar "
-        f"(rtol 1e-5 / atol 1e-6), concessions: {kinds if kinds else 'none'}")
-    for c in led["concessions"]:
-        terminalreporter.write_line(f"  {c}")
+        f"(rtol 1e-5 / atol 1e-6), concessions: {kinds if kinds else 'none'} (each one in gpurun_out/parity_ledger.json)")
+    for (fn, kind, tensor), n in sorted(per_test.items()):
+        terminalreporter.write_line(f"  {n:4d} x {kind:<24s} {tensor:<6s} {fn}")

@@ -60,17 +60,21 @@ def test_null_and_shape_errors_are_status_codes(lib):
     assert L.faith_matmul_verification(q, p, p, p, p, None, p, p, p, p, 1, 1, 4, 4, 4, None) == -4
     assert L.faith_matmul_verification(p, p, p, p, p, None, p, p, p, p, 1, 0, 4, 4, 4, None) == -2
     assert L.faith_dot_product_verification_QK(p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, p,
-                                               1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, None) == -2
+                                               1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, 0, None) == -2
+    assert L.faith_dot_product_verification_QK(p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, p,
+                                               1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, 1, None) == -2      # transposed layout
+    assert L.faith_dot_product_verification_V(p, p, p, p, p, p, p, p, p, p, p, p, p, p, p, p,
+                                              1, 4, 4, 4, 4, 0.1, lib.Q_1, 1, 5, None) == -3       # unknown layout
     # kernel larger than the padded image
     assert L.faith_convolution_verification(p, p, p, p, p, None, p, p, p, p, 1, 2, 2, 1, 1, 5, 1, 0, 1, None) == -2
     assert L.faith_tune_set(99, 1) == -3
     # the allocation-free dot product refuses what its 4 MiB array cannot hold, before touching the GPU
     assert L.faith_static_scratch_bytes() == 4 << 20
     assert L.faith_dot_product_verification_QK_static(p, p, p, p, p, p, p, p, p, p, p, p,
-                                                      16, 512, 512, 64, 8, 0.1, lib.Q_1, 1, None) == -3
+                                                      16, 512, 512, 64, 8, 0.1, lib.Q_1, 1, 0, None) == -3
     assert b"scratch" in L.faith_last_error()
     assert L.faith_dot_product_verification_QK_static(p, p, p, p, p, p, p, p, p, p, p, p,
-                                                      1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, None) == -2
+                                                      1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, 0, None) == -2
 
 
 def test_python_wrappers_refuse_cpu_tensors():

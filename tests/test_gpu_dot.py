@@ -277,6 +277,104 @@ def test_c_bound_dot_shims():
     assert close(zuw.transpose(2, 3), e.uw, rtol=1e-5, atol=2e-6) and close(zub, e.ub, rtol=1e-5, atol=2e-6)
 
 
+@pytest.mark.parametrize("p", [2.0, INF, 1.0, 3.0])
+@pytest.mark.parametrize("shape", [
+    # B, Lx, Ly, D, d (scores) / B, Lx, Lk, D, dv (context); words
+    (2, 8, 8, 16, 12, 1),         # D_in below a wavefront: the four wavefronts of a workgroup along the columns
+    (1, 5, 9, 100, 20, 2),        # two wavefronts along m, ragged rows, columns and lanes
+    (4, 32, 32, 256, 64, 1),      # configuration-3 operands at a quarter of the length: four wavefronts along m
+    (1, 3, 70, 300, 7, 3),        # D_in beyond one workgroup's 256 lanes, more columns than a workgroup takes
+    (2, 6, 4, 1, 10, 1),          # dim_in == 1: the interval shortcut
+])
+def test_dot_products_in_the_reference_layout_through_the_c_abi(shape, p):
+    """faith_dot_product_verification_QK / _V with FAITH_LAYOUT_TRANSPOSED, called as a C binder would call them
+    (raw pointers through the C ABI): operands [B, L, dim_out, dim_in], z_lw [B, Lx, Ly, dim_in], exactly the
+    tensors the reference's adapters build (Bounds.py:1279-1290, 1319-1329); against the oracle."""
+    import ctypes
+    from faith_amd import _lib, ops
+    B, Lx, L2, D, d, words = shape
+    g = torch.Generator().manual_seed(37)
+    eps = 0.05
+    P = lambda t_: ctypes.c_void_p(t_.data_ptr())
+    T = lambda t_: t_.cuda().transpose(2, 3).contiguous()
+    nan = lambda *s_: torch.full(s_, float("nan"), device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call(entry, x, y, Ly, K, y_shape):
+        x_l, x_u = nan(B, Lx, K), nan(B, Lx, K)
+        y_l, y_u = nan(*y_shape), nan(*y_shape)
+        zlb, zub, zlw, zuw = nan(B, Lx, Ly), nan(B, Lx, Ly), nan(B, Lx, Ly, D), nan(B, Lx, Ly, D)
+        ops_ = [x.lb.cuda().contiguous(), x.ub.cuda().contiguous(), y.lb.cuda().contiguous(), y.ub.cuda().contiguous(),
+                T(x.lw), T(x.uw), T(y.lw), T(y.uw)]
+        dims = (B, Lx, Ly, K, D) if entry.endswith("QK") else (B, Lx, K, Ly, D)
+        _lib.call(entry, P(x_l), P(y_l), P(x_u), P(y_u), *(P(t_) for t_ in ops_), P(zlb), P(zub), P(zlw), P(zuw),
+                  *dims, eps, ops.q_code(p), words, _lib.LAYOUT_TRANSPOSED, stream)
+        torch.cuda.synchronize()
+        return (zlw.transpose(2, 3), zlb, zuw.transpose(2, 3), zub), (x_l, x_u, y_l, y_u)
+
+    # scores: x [B, Lx, D, d], y [B, L2, D, d]
+    x, y = rand_bounds(g, B, Lx, D, d, sw=0.2), rand_bounds(g, B, L2, D, d, sw=0.2)
+    print(f"[case] transposed-layout QK {shape} p={p}", flush=True)
+    got, (x_l, x_u, y_l, y_u) = call("faith_dot_product_verification_QK", x, y, L2, d, (B, L2, d))
+    exp = O.dot_product(x, y, p, eps, words)
+    exl, exu = O.concretize(x, p, eps, words)
+    eyl, eyu = O.concretize(y, p, eps, words)
+    assert close(x_l, exl) and close(x_u, exu) and close(y_l, eyl) and close(y_u, eyu)
+    if D == 1:
+        for a, e in zip(got, exp.tensors()):
+            assert close(a, e)
+    else:
+        ref, mag = dot64(x, y, p, eps, words)
+        for name, a, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
+            assert a.shape == e.shape
+            compare_contraction(name, a, e, ref[name], mag[name], UNIT_SCALE_ALL)
+
+    # context: probabilities [B, Lx, D, Lk = L2], values [B, Lk, D, dv = d]; y is handed over as value.t()
+    probs, value = rand_bounds(g, B, Lx, D, L2, sw=0.2, sb=0.5), rand_bounds(g, B, L2, D, d, sw=0.2)
+    vt = O.transpose_bounds(value)                         # lw [B, dv, D, Lk], lb [B, dv, Lk]
+    print(f"[case] transposed-layout V {shape} p={p}", flush=True)
+    got, (x_l, x_u, y_l, y_u) = call("faith_dot_product_verification_V", probs, vt, d, L2, (B, d, L2))
+    exp = O.context(probs, value, p, eps, words)
+    epl, epu = O.concretize(probs, p, eps, words)
+    evl, evu = O.concretize(vt, p, eps, words)
+    assert close(x_l, epl) and close(x_u, epu) and close(y_l, evl) and close(y_u, evu)
+    if D == 1:
+        for a, e in zip(got, exp.tensors()):
+            assert close(a, e)
+    else:
+        ref, mag = dot64(probs, vt, p, eps, words)
+        for name, a, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
+            assert a.shape == e.shape
+            compare_contraction(name, a, e, ref[name], mag[name], UNIT_SCALE_ALL)
+
+
+def test_reference_layout_dot_product_at_configuration_3_size_equals_the_natural_layout():
+    """Full-size configuration 3 through the transposed entry: every element within the parity bar of the MFMA
+    path of the natural layout (same inputs re-laid out; two fp32 summation orders of 256 terms)."""
+    from faith_amd import c_bound, ops
+    from faith_amd.workloads import make_config
+    c = make_config(3)
+    x, y = dev(as_bounds(c["x"])), dev(as_bounds(c["y"]))
+    B, L, D, d = x[0].shape
+    nat = ops.dot_product_qk(x, y, c["p"], c["eps"], 1)
+    T = lambda t_: t_.transpose(2, 3).contiguous()
+    z = lambda *s_: torch.empty(*s_, device="cuda")
+    scratch = [z(B, L, d) for _ in range(4)]
+    zlb, zub, zlw, zuw = z(B, L, L), z(B, L, L), z(B, L, L, D), z(B, L, L, D)
+    c_bound.p, c_bound.words = c["p"], 1
+    try:
+        c_bound.c_dot_product_verification_QK(*scratch, x[1], x[3], y[1], y[3], T(x[0]), T(x[2]), T(y[0]), T(y[2]),
+                                              zlb, zub, zlw, zuw, B, L, d, D, c["eps"])
+    finally:
+        c_bound.p = 2.0
+    # the same constant-term kernel, fed by intervals from two concretize kernels (another reduction order: last
+    # bits of l, u differ) whose differences 64 O(1) terms per element carry into the sums
+    torch.testing.assert_close(zlb, nat[1], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(zub, nat[3], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(zlw.transpose(2, 3), nat[0], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(zuw.transpose(2, 3), nat[2], rtol=1e-5, atol=1e-6)
+
+
 # ------------------------------------------------------------------ heads addressed in place
 def side_by_side(x, heads):
     """[batch*heads, L, D, w] / [batch*heads, L, w] -> [batch, L, D, heads*w] / [batch, L, heads*w], the

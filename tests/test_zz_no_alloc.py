@@ -27,7 +27,7 @@ def _call_both(B, Lx, Ly, D, d, p, words, seed):
         zlb, zub, zlw, zuw = new(B, Lx, Ly), new(B, Lx, Ly), new(B, Lx, D, Ly), new(B, Lx, D, Ly)
         P = lambda t: ctypes.c_void_p(t.data_ptr())
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        tail = (B, Lx, Ly, d, D, 0.05, ops.q_code(p), words, stream)
+        tail = (B, Lx, Ly, d, D, 0.05, ops.q_code(p), words, _lib.LAYOUT_NATURAL, stream)
         if static:
             before = torch.cuda.memory_allocated()
             _lib.call("faith_dot_product_verification_QK_static", P(xlb), P(xub), P(ylb), P(yub), P(xlw), P(xuw), P(ylw),
@@ -57,4 +57,4 @@ def test_static_scratch_dot_product_rejects_what_does_not_fit():
     z = torch.zeros(8, device="cuda")
     P = ctypes.c_void_p(z.data_ptr())
     with pytest.raises(_lib.FaithError, match="scratch"):
-        _lib.call("faith_dot_product_verification_QK_static", *([P] * 12), 16, 512, 512, 64, 8, 0.1, 1, 1, None)
+        _lib.call("faith_dot_product_verification_QK_static", *([P] * 12), 16, 512, 512, 64, 8, 0.1, 1, 1, 0, None)
