@@ -27,6 +27,8 @@
 //
 // The constant-term path (batch images, 1/D_in of the work, O(1) cancelling terms) runs in a
 // direct kernel that accumulates in double and adds the bias.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -389,6 +391,308 @@ conv_signsplit_k3s1(const ConvArgs g) {
     }
 }
 
+// ------------------------------------------------------------------ other common layers, same scheme
+// The straight-line, double-buffered kernel above with its extents as template parameters: kernel size K,
+// stride S, input channels per reduction chunk CCH (a 1 x 1 layer has one tap per channel, so it takes 16
+// channels a chunk to give a barrier 128 MFMAs; 3 x 3 and 5 x 5 take 4), and whether a row of the weight
+// slab can be fetched 16 bytes at a time (WVEC: C_in % 4 == 0, aligned) or needs 4-byte loads (the first
+// layer of an image classifier has C_in = 3).  Channels past C_in need no predicate on either operand: the
+// input window ends with the image's last channel, so such a patch element reads as zero, and a zero patch
+// makes whatever finite weight the slab holds at that position irrelevant.
+//
+// The tile is a parameter too.  An MFMA block is 32 channels x 32 pixels; the 32 pixels are TCB columns x 32 / TCB
+// rows of the image (TCB = 32: one row; 16: two rows of a 16-wide image, which a 32-column tile would fill by
+// half), and the workgroup's four wavefronts are WM x 4 / WM over (halves of 64 channels) x (pairs of pixel
+// blocks): WM = 2 is 128 channels x 4 blocks, WM = 1 is 64 channels x 8 blocks for layers of up to 64 channels.
+template <int K, int S, int CCH, bool WVEC, int TCB, int WM>
+struct FastTile {
+    static constexpr int RPB = 32 / TCB;                 // image rows of one pixel block
+    static constexpr int NPB = 2 * (4 / WM);             // pixel blocks of a workgroup
+    static constexpr int ROWS = NPB * RPB, CHANNELS = 64 * WM;
+    static constexpr int KK = K * K, PROW = (ROWS - 1) * S + K, PCOL = (TCB - 1) * S + K, PP = PROW * PCOL;
+    static constexpr int WS = (CCH * KK) | 1;
+    static constexpr size_t LDS = ((size_t)4 * CCH * PP + (size_t)2 * CHANNELS * WS) * sizeof(float);
+};
+
+template <int K, int S, int CCH, bool WVEC, int TCB, int WM>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+conv_signsplit_fast(const ConvArgs g) {
+    using T = FastTile<K, S, CCH, WVEC, TCB, WM>;
+    constexpr int TCO = T::CHANNELS, TR = T::ROWS, TC = TCB, RPB = T::RPB;      // shadow the file-scope tile
+    constexpr int KK = K * K, PROW = T::PROW, PCOL = T::PCOL, PP = T::PP;
+    constexpr int WROW = CCH * KK;                       // floats of one weight row in a chunk
+    constexpr int WS = WROW | 1;                         // padded to an odd length: conflict-free column reads
+    constexpr int NP = (CCH * PP + NTHREADS - 1) / NTHREADS;             // patch elements per thread and bound
+    constexpr int WPT = WVEC ? 4 : 1;                                    // floats per weight load
+    constexpr int NWL = (TCO * WROW / WPT + NTHREADS - 1) / NTHREADS;    // weight loads per thread
+    constexpr unsigned NOWHERE = 0xfffffff0u;            // a buffer offset the hardware answers with zero
+    static_assert(CCH % 4 == 0 && WROW % 4 == 0, "a chunk is split into two halves of channel pairs");
+    extern __shared__ float smem[];
+    float *sXl = smem;                                   // [2][CCH * PP]
+    float *sXu = sXl + 2 * CCH * PP;
+    float *sW = sXu + 2 * CCH * PP;                      // [2][TCO * WS]
+
+    const int tcol = (g.Wo + TC - 1) / TC, trow = (g.Ho + TR - 1) / TR, tco = (g.Co + TCO - 1) / TCO;
+    int pid = blockIdx.x;
+    const int ow0 = (pid % tcol) * TC;  pid /= tcol;
+    const int oh0 = (pid % trow) * TR;  pid /= trow;
+    const int co0 = (pid % tco) * TCO;  pid /= tco;
+    const int n = pid;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % 64, wv = tid / 64;
+    const int wm = wv / (4 / WM), wn = wv % (4 / WM);
+    const int fi = lane % 32, fh = lane / 32;
+    const int fr = fi / TCB, fc = fi % TCB;              // the lane's pixel inside a block: row, column
+
+    const int ih0 = oh0 * S - g.P, iw0 = ow0 * S - g.P;
+    const int img = g.H * g.W;
+    const size_t image = (size_t)g.Ci * img;
+    const float *xl_n = g.xl + n * image, *xu_n = g.xu + n * image;
+    const float *w_blk = g.w + (size_t)co0 * g.Ci * KK;
+    const size_t w_bytes = (size_t)(g.Co - co0) * g.Ci * KK * 4;
+
+    // ---- staging plan, fixed for the whole reduction: byte offsets inside a chunk of channels
+    unsigned poff[NP];
+#pragma unroll
+    for (int u = 0; u < NP; ++u) {
+        const int e = tid + u * NTHREADS;
+        const int ci = e / PP, r2 = e % PP, pr = r2 / PCOL, pc = r2 % PCOL;
+        const int ih = ih0 + pr, iw = iw0 + pc;
+        const bool ok = e < CCH * PP && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+        poff[u] = ok ? (unsigned)(ci * img + ih * g.W + iw) * 4u : NOWHERE;
+    }
+    // weight load u of a thread: element e = tid + u * NTHREADS of the slab, row e / (WROW / WPT); its source and
+    // destination are a few integer operations on compile-time divisors, recomputed where they are used so
+    // that they do not occupy 2 NWL registers across the MFMAs (rows past C_out re-read the last row; they are
+    // never stored)
+    const int last_row = g.Co - 1 - co0;
+    // (the empty asm makes the thread number opaque inside a chunk: otherwise the compiler hoists all 2 NWL values
+    // out of the reduction loop again)
+    auto wsrc = [&](int u, int tid_) -> unsigned {
+        const int e = tid_ + u * NTHREADS;
+        const int co = e / (WROW / WPT), f = e % (WROW / WPT);
+        return e < TCO * (WROW / WPT) ? (unsigned)(min(co, last_row) * g.Ci * KK + f * WPT) * 4u : NOWHERE;
+    };
+    auto wdst = [&](int u, int tid_) -> int {
+        const int e = tid_ + u * NTHREADS;
+        return e < TCO * (WROW / WPT) ? (e / (WROW / WPT)) * WS + (e % (WROW / WPT)) * WPT : -1;
+    };
+    // A large weight slab (5 x 5: 50 floats per thread and chunk) is fetched in two parts so that its registers
+    // fit beside the 128 accumulators: part 1 with the patch, before the first half of the MFMAs, part 2 after
+    // the first part has gone to LDS, before the second half.
+    constexpr bool TWO_PARTS = NWL * WPT > 32;
+    constexpr int NW1 = TWO_PARTS ? (NWL + 1) / 2 : NWL, NW2 = NWL - NW1, NWR = NW1 > NW2 ? NW1 : NW2;
+    float pxl[NP], pxu[NP];
+    float pw[NWR][WPT];
+    auto fetch_patch = [&](int c0) {
+        const __amdgpu_buffer_rsrc_t rl = window(xl_n, image * 4), ru = window(xu_n, image * 4);
+        const unsigned cx = (unsigned)c0 * img * 4u;
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            pxl[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, poff[u], cx, 0));
+            pxu[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ru, poff[u], cx, 0));
+        }
+    };
+    auto fetch_weights = [&](int c0, auto first, auto count) {
+        const __amdgpu_buffer_rsrc_t rw = window(w_blk, w_bytes);
+        const unsigned cw = (unsigned)c0 * KK * 4u;
+        int tid_ = tid;
+        asm volatile("" : "+v"(tid_));
+#pragma unroll
+        for (int u = 0; u < decltype(count)::value; ++u) {
+            if constexpr (WVEC) {
+                const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rw, wsrc(u + decltype(first)::value, tid_), cw, 0);
+                pw[u][0] = __uint_as_float(v.x);
+                pw[u][1] = __uint_as_float(v.y);
+                pw[u][2] = __uint_as_float(v.z);
+                pw[u][3] = __uint_as_float(v.w);
+            } else {
+                pw[u][0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rw, wsrc(u + decltype(first)::value, tid_), cw, 0));
+            }
+        }
+    };
+    auto commit_patch = [&](int buf) {
+        float *dl = sXl + buf * CCH * PP, *du = sXu + buf * CCH * PP;
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            const int e = tid + u * NTHREADS;
+            if (e < CCH * PP) {
+                dl[e] = pxl[u];
+                du[e] = pxu[u];
+            }
+        }
+    };
+    auto commit_weights = [&](int buf, auto first, auto count) {
+        float *dw = sW + buf * TCO * WS;
+        int tid_ = tid;
+        asm volatile("" : "+v"(tid_));
+#pragma unroll
+        for (int u = 0; u < decltype(count)::value; ++u) {
+            const int d = wdst(u + decltype(first)::value, tid_);
+            if (d >= 0) {
+#pragma unroll
+                for (int q = 0; q < WPT; ++q) dw[d + q] = pw[u][q];
+            }
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, NW1>;
+    using I2 = std::integral_constant<int, NW2>;
+
+    int xoff[2], woff[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) xoff[b] = fh * (CCH / 2) * PP + (((wn * 2 + b) * RPB + fr) * S) * PCOL + fc * S;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) woff[a] = (wm * 64 + a * 32 + fi) * WS + fh * (CCH / 2) * KK;
+
+    floatx16 cl[2][2], cu[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
+
+    // the MFMAs of channel pairs [cp0, cp1) of the chunk in LDS buffer `buf`
+    auto multiply = [&](int buf, int cp0, int cp1) {
+        const float *bl = sXl + buf * CCH * PP, *bu = sXu + buf * CCH * PP, *bw = sW + buf * TCO * WS;
+#pragma unroll
+        for (int cp = cp0; cp < cp1; ++cp) {
+#pragma unroll
+            for (int tap = 0; tap < KK; ++tap) {
+                const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
+                const int wo = cp * KK + tap;
+                float wp[2], wq[2], xl[2], xu[2];
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const float w = bw[woff[a] + wo];
+                    wp[a] = pos1(w);
+                    wq[a] = neg1(w);
+                }
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    xl[b] = bl[xoff[b] + xo];
+                    xu[b] = bu[xoff[b] + xo];
+                }
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
+                        cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
+                    }
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
+                        cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                    }
+            }
+        }
+    };
+
+    fetch_patch(0);
+    fetch_weights(0, I0{}, I1{});
+    commit_patch(0);
+    commit_weights(0, I0{}, I1{});
+    if constexpr (TWO_PARTS) {
+        fetch_weights(0, I1{}, I2{});
+        commit_weights(0, I1{}, I2{});
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int c0 = 0; c0 + CCH < g.Ci; c0 += CCH) {
+        fetch_patch(c0 + CCH);
+        fetch_weights(c0 + CCH, I0{}, I1{});
+        __builtin_amdgcn_sched_barrier(0);         // the fetch goes first
+        multiply(buf, 0, CCH / 4);
+        __builtin_amdgcn_sched_barrier(0);         // staging between the two halves of the MFMAs
+        commit_patch(buf ^ 1);
+        commit_weights(buf ^ 1, I0{}, I1{});
+        if constexpr (TWO_PARTS) fetch_weights(c0 + CCH, I1{}, I2{});
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(buf, CCH / 4, CCH / 2);
+        if constexpr (TWO_PARTS) {
+            __builtin_amdgcn_sched_barrier(0);
+            commit_weights(buf ^ 1, I1{}, I2{});
+        }
+        __syncthreads();
+        buf ^= 1;
+    }
+    multiply(buf, 0, CCH / 2);
+
+    // ---- epilogue: as in the 3 x 3 stride-1 kernel (buffer stores into image n of the result); a lane whose
+    // pixel lies outside the image carries an offset outside the window
+    const size_t plane = (size_t)g.Ho * g.Wo;
+    const __amdgpu_buffer_rsrc_t wyl = window(g.yl + (size_t)n * g.Co * plane, (size_t)g.Co * plane * 4);
+    const __amdgpu_buffer_rsrc_t wyu = window(g.yu + (size_t)n * g.Co * plane, (size_t)g.Co * plane * 4);
+    const unsigned plane_b = (unsigned)plane * 4u;
+    const int wvu = __builtin_amdgcn_readfirstlane(wv);
+    const int wmu = wvu / (4 / WM), wnu = wvu % (4 / WM);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int row0 = oh0 + (wnu * 2 + b) * RPB;                  // first image row of this pixel block
+        if (row0 >= g.Ho) continue;
+        const bool inside = ow0 + fc < g.Wo && row0 + fr < g.Ho;
+        const unsigned vo = inside ? (unsigned)(4 * fh) * plane_b + (unsigned)(fr * g.Wo + ow0 + fc) * 4u : 0x80000000u;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
+                                    (unsigned)(row0 * g.Wo) * 4u;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cu[a][b][r]), wyu, vo, so, 2);
+            }
+        }
+    }
+}
+
+template <int K, int S, int CCH, bool WVEC, int TCB, int WM>
+bool launch_tile(const ConvArgs &g, hipStream_t st) {
+    using T = FastTile<K, S, CCH, WVEC, TCB, WM>;
+    static_assert(T::LDS <= 160 * 1024, "the two LDS stages of this instantiation do not fit a workgroup");
+    const long long grid = (long long)g.N * ((g.Co + T::CHANNELS - 1) / T::CHANNELS) * ((g.Ho + T::ROWS - 1) / T::ROWS) *
+                           ((g.Wo + TCB - 1) / TCB);
+    if (grid > 0x7fffffffLL) return false;
+    if (!faith::reserve_lds(conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>, T::LDS)) return false;
+    hipLaunchKernelGGL((conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>), dim3((unsigned)grid), dim3(NTHREADS), T::LDS, st, g);
+    return true;
+}
+
+// Tile for this layer: 16-column pixel blocks when the last (or only) 32-column tile of a row would be at most
+// half full, 64-channel workgroups when the last (or only) 128-channel tile would be.
+template <int K, int S, int CCH, bool WVEC>
+bool launch_fast(const ConvArgs &g, hipStream_t st) {
+    const bool narrow = (g.Wo - 1) % 32 < 16, few = (g.Co - 1) % 128 < 64;
+    if (narrow && few) return launch_tile<K, S, CCH, WVEC, 16, 1>(g, st);
+    if (narrow) return launch_tile<K, S, CCH, WVEC, 16, 2>(g, st);
+    if (few) return launch_tile<K, S, CCH, WVEC, 32, 1>(g, st);
+    return launch_tile<K, S, CCH, WVEC, 32, 2>(g, st);
+}
+
+// The straight-line instantiation for this layer, if there is one: 3 x 3 at stride 1 or 2, 1 x 1, 5 x 5.
+bool dispatch_fast(const ConvArgs &g, bool wvec, hipStream_t st) {
+    const int key = g.K * 10 + g.S;
+    if (wvec) {
+        switch (key) {
+            case 31: return launch_fast<3, 1, 4, true>(g, st);      // layers that fill 128 x (4 x 32) tiles take the kernel above
+            case 32: return launch_fast<3, 2, 4, true>(g, st);
+            case 11: return launch_fast<1, 1, 16, true>(g, st);
+            case 51: return launch_fast<5, 1, 4, true>(g, st);
+            default: return false;
+        }
+    }
+    switch (key) {
+        case 31: return launch_fast<3, 1, 4, false>(g, st);
+        case 32: return launch_fast<3, 2, 4, false>(g, st);
+        case 11: return launch_fast<1, 1, 16, false>(g, st);
+        default: return false;
+    }
+}
+
 // Direct convolution for the constant terms: 32 neighbouring outputs x 4 output channels x 8 groups of
 // input channels per workgroup; a thread sums its share of the input channels in double (an fp32 x fp32
 // product is exact there) for its pixel and four output channels -- the centre and the radius of an input
@@ -497,9 +801,17 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
                       (long long)CIN * Height * Width * 4 < 0xfffffff0LL &&      // 32-bit byte offsets inside an image
                       (long long)128 * CIN * 9 * 4 + (long long)CIN * 9 * 4 < 0xfffffff0LL &&  // and inside a block of weight rows
                       ((long long)COUT + 132) * Ho * Wo * 4 < 0x80000000LL;                   // and inside an image of the result
-    if (k3s1)
+    // the limits of 32-bit byte offsets, for any kernel size: inside an image of x, inside a block of 128 weight
+    // rows plus one chunk, inside an image of the result
+    const bool offsets_fit = (long long)CIN * Height * Width * 4 < 0xfffffff0LL &&
+                             (long long)129 * CIN * K * K * 4 + 64LL * K * K * 4 < 0xfffffff0LL &&
+                             ((long long)COUT + 132) * Ho * Wo * 4 < 0x80000000LL;
+    const bool wvec = CIN % 4 == 0 && faith::aligned(W, 16);
+    const int forced = faith::tune_get(FAITH_TUNE_CONV_VARIANT);      // 1: the general kernel, whatever the layer
+    const bool full_tiles = (Wo - 1) % 32 >= 16 && (COUT - 1) % 128 >= 64;     // else a smaller tile wastes less
+    if (k3s1 && full_tiles && forced != 1)
         hipLaunchKernelGGL(conv_signsplit_k3s1, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
-    else
+    else if (!(forced != 1 && offsets_fit && dispatch_fast(gw, wvec, st)))
         hipLaunchKernelGGL(conv_signsplit, dim3((unsigned)grid), dim3(NTHREADS), smem, st, gw);
 
     // constant terms: batch images through the exact-accumulation kernel, bias added

@@ -55,6 +55,25 @@ def check(x, W, bias, stride, pad, what=""):
     (1, 5, 4, 9, 9, 1, 1, 0),          # 1x1
     (2, 2, 3, 12, 12, 5, 2, 2),        # 5x5 stride 2
     (1, 1, 1, 3, 3, 3, 1, 1),          # degenerate
+    # the straight-line kernels of the common layers, each with and without 16-byte weight rows, ragged tiles included
+    (2, 8, 130, 17, 40, 3, 2, 1),      # 3x3 stride 2, C_in % 4 == 0, two channel tiles
+    (2, 12, 20, 9, 33, 3, 2, 0),       # 3x3 stride 2, three chunks, no padding
+    (2, 3, 16, 32, 32, 3, 2, 1),       # 3x3 stride 2, C_in = 3 (4-byte weight loads)
+    (3, 3, 64, 32, 32, 3, 1, 1),       # the first layer of an image classifier: 3x3 stride 1, C_in = 3
+    (2, 6, 40, 11, 35, 3, 1, 1),       # 3x3 stride 1, C_in = 6: a chunk and a half
+    (2, 32, 64, 8, 40, 1, 1, 0),       # 1x1, two chunks of 16 channels
+    (2, 20, 130, 9, 9, 1, 1, 0),       # 1x1, C_in no multiple of the chunk (zero patch beyond the last channel)
+    (2, 5, 7, 6, 6, 1, 1, 1),          # 1x1 with padding, C_in = 5
+    (2, 8, 24, 14, 36, 5, 1, 2),       # 5x5 stride 1, two chunks (the weight slab goes to LDS in two parts)
+    (1, 16, 130, 12, 12, 5, 1, 0),     # 5x5, four chunks, two channel tiles
+    # tile variants: 16-column pixel blocks (two image rows a block), 64-channel workgroups, and both
+    (2, 8, 128, 33, 33, 3, 2, 1),      # Wo = 17: 16 + 1 columns, full channel tile
+    (2, 8, 40, 30, 64, 3, 1, 1),       # 64-channel workgroups (8 pixel blocks), 32-column blocks
+    (2, 4, 64, 9, 16, 3, 1, 1),        # both: 64 channels, 16 columns, ragged rows
+    (2, 16, 200, 16, 16, 1, 1, 0),     # 1x1: 128 + 72 channels -> 64-channel workgroups? no: (200-1)%128 = 71 -> full tiles; 16 columns
+    (2, 16, 24, 7, 12, 1, 1, 0),       # 1x1: both small
+    (1, 8, 32, 10, 10, 5, 1, 2),       # 5x5: both small
+    (3, 3, 32, 16, 16, 3, 1, 1),       # C_in = 3, both small
 ])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_conv_shapes(case, with_bias):
@@ -65,6 +84,30 @@ def test_conv_shapes(case, with_bias):
     W.view(-1)[::5] = 0.0
     bias = torch.randn(Co, generator=g) if with_bias else None
     check(x, W, bias, s, p, "sweep")
+
+
+@pytest.mark.parametrize("case", [(3, 8, 40, 17, 40, 3, 2, 1), (2, 32, 64, 8, 40, 1, 1, 0), (2, 8, 24, 14, 36, 5, 1, 2),
+                                  (3, 3, 64, 32, 32, 3, 1, 1)])
+def test_straight_line_conv_kernels_equal_the_general_kernel(case):
+    """Same reduction order (channel chunks, channel pairs, taps) in both kernels of a layer: bit for bit where
+    the chunk is the same (4 channels); the 1x1 kernel takes 16 channels a chunk and is held to the parity bar."""
+    from faith_amd import _lib, ops
+    D, Ci, Co, Hh, Ww, K, s_, p = case
+    g = torch.Generator().manual_seed(43)
+    x = make(g, D, Ci, Hh, Ww, ordered=False)
+    W = (torch.randn(Co, Ci, K, K, generator=g) * (2.0 / (Ci * K * K)) ** 0.5).cuda()
+    args = [t.cuda() for t in x.tensors()]
+    fast = ops.conv2d(*args, W, None, s_, p)
+    _lib.call("faith_tune_set", 4, 1)
+    try:
+        general = ops.conv2d(*args, W, None, s_, p)
+    finally:
+        _lib.call("faith_tune_set", 4, 0)
+    for a, b in zip(fast, general):
+        if K == 1:
+            assert close(a, b.cpu())
+        else:
+            assert torch.equal(a, b)
 
 
 def test_conv_config4_reduced():
