@@ -33,6 +33,7 @@
 // the N-tiles that share an M-block (and with it A_l / A_u rows) are given ids 8 apart and
 // meet in the same L2.
 #include "common.h"
+#include "relax_common.h"
 
 namespace {
 
@@ -85,21 +86,18 @@ __device__ __forceinline__ int swz(int row, int c) { return row * 8 + 4 * (c ^ (
 // for problems with too few 128 x 128 tiles to fill the machine: a wavefront then works through 32
 // MFMAs per K-step instead of 128, a quarter of the latency, at a lower MFMA rate per byte staged.
 // 2 x 1 and 1 x 2 (128 x 64, 64 x 128: 64 MFMAs per K-step, 48 KB) lie between.
-template <bool EXACT, int MBM, int MBN>
-__device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *smem, const int pid) {
+// NQ >= 0 (a dual-norm selector): the tile's contribution to the column norms of C_l and C_u -- over its BM rows,
+// which the caller guarantees to exist and to belong to one position -- is folded into pl / pu, one running
+// value per lane and column block; NQ = -1: no norms.
+template <bool EXACT, int MBM, int MBN, int NQ = -1>
+__device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *smem, const int m_blk, const int n_blk,
+                                                    float *pl = nullptr, float *pu = nullptr, float qv = 0.f) {
     constexpr int BM = 64 * MBM, BN = 64 * MBN;
     constexpr int HALF_A = BM * 8, HALF_W = BN * 8;      // floats in one [rows x 8] half of an operand's K-step
     constexpr int S_AL = 0, S_AU = 2 * HALF_A, S_WP = 4 * HALF_A, S_WN = 4 * HALF_A + 2 * HALF_W;
     constexpr int STAGE = 4 * HALF_A + 4 * HALF_W;
     float(*sm)[STAGE] = reinterpret_cast<float(*)[STAGE]>(smem);
 
-    // ---- tile of this workgroup
-    const int tiles_n = (g.N + BN - 1) / BN;
-    const int mblks = (g.Mw + BM - 1) / BM;
-    const int xcd = pid % XCDS, local = pid / XCDS;
-    const int m_blk = (local / tiles_n) * XCDS + xcd;
-    const int n_blk = local % tiles_n;
-    if (m_blk >= mblks) return;
     const int M = g.Mw;
     const int m0 = m_blk * BM, n0 = n_blk * BN;
     const int K = g.K;
@@ -259,6 +257,33 @@ __device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *sm
             }
         }
     }
+    if constexpr (NQ >= 0) {
+        // the lane's 16 MBM rows of each of its columns, in register order (a fixed order: the result does not
+        // depend on scheduling)
+#pragma unroll
+        for (int b = 0; b < MBN; ++b)
+#pragma unroll
+            for (int a = 0; a < MBM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    pl[b] = nacc<NQ>(pl[b], cl[a][b][r], qv);
+                    pu[b] = nacc<NQ>(pu[b], cu[a][b][r], qv);
+                }
+    }
+}
+
+// One tile per workgroup: workgroups are dealt round-robin to the XCDs, so the N-tiles that share an M-block
+// get ids 8 apart and meet in one L2.
+template <bool EXACT, int MBM, int MBN>
+__device__ __forceinline__ void signsplit_gemm_body(const GemmArgs &g, float *smem, const int pid) {
+    constexpr int BM = 64 * MBM, BN = 64 * MBN;
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int mblks = (g.Mw + BM - 1) / BM;
+    const int xcd = pid % XCDS, local = pid / XCDS;
+    const int m_blk = (local / tiles_n) * XCDS + xcd;
+    const int n_blk = local % tiles_n;
+    if (m_blk >= mblks) return;
+    signsplit_gemm_tile<EXACT, MBM, MBN>(g, smem, m_blk, n_blk);
 }
 
 // ------------------------------------------------------------------ exact-accumulation kernel
@@ -522,6 +547,31 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_grouped(const GroupAr
 
 }  // namespace
 
+// Macro-tile of the MFMA kernel for a problem of mw coefficient rows, from tuner runs on 1024 ... 245760 rows, K and
+// N 64 ... 1024 (the built-in choice is within 3 % of the best of the four there).  The tuning knob forces a shape.
+static void choose_tile(long long mw, int dim_out, int dim_y_out, int *tm, int *tn) {
+    auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * ((dim_y_out + n - 1) / n); };
+    const long long cus = faith::compute_units();
+    // tiny problems want the most workgroups (64 x 64); up to two 128 x 64 tiles per CU that shape is up to 17 %
+    // ahead; 128 x 128 pays only for long reductions on problems of many tiles per CU (configuration 2: 1 % ahead)
+    // -- with K <= 512 the pro- and epilogues of five small co-resident workgroups overlap better than those of two
+    // large ones (2 - 6 % at 65536 ... 245760 rows)
+    if (tiles(64, 64) <= cus) { *tm = 64; *tn = 64; }
+    else if (tiles(128, 64) <= 2 * cus) { *tm = 128; *tn = 64; }
+    else if (dim_out >= 1024 && tiles(128, 128) >= 16 * cus) { *tm = 128; *tn = 128; }
+    // many column tiles re-read every block of rows from L2: the large tile halves that (3 - 5 % at
+    // 768 -> 3072 and 512 -> 2048 with 12288 ... 24576 rows) once it fills the machine four times over
+    else if (dim_y_out >= 2048 && tiles(128, 128) >= 8 * cus) { *tm = 128; *tn = 128; }
+    else { *tm = 64; *tn = 64; }
+    switch (faith::tune_get(FAITH_TUNE_GEMM_VARIANT)) {
+        case 1: *tm = 64;  *tn = 64;  break;
+        case 2: *tm = 128; *tn = 128; break;
+        case 3: *tm = 128; *tn = 64;  break;
+        case 4: *tm = 64;  *tn = 128; break;
+        default: break;
+    }
+}
+
 extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
                                          const float *W, const float *bias, float *y_lb, float *y_ub, float *y_lw,
                                          float *y_uw, int batch_size, int length, int dim_in, int dim_out,
@@ -543,30 +593,11 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
                       128LL * dim_y_out * 4 < 0x80000000LL;                           // and in a tile of the result
     if (fast) {
         // coefficient rows on MFMA, constant-term rows on the exact-accumulation kernel
-        // macro-tile, from tuner runs on 1024 ... 245760 rows, K and N 64 ... 1024 (the built-in choice is
-        // within 3 % of the best of the four there): tiny problems want the most workgroups (64 x 64); up
-        // to two 128 x 64 tiles per CU that shape is up to 17 % ahead; 128 x 128 pays only for long
-        // reductions on problems of many tiles per CU (configuration 2: 1 % ahead) -- with K <= 512 the
-        // pro- and epilogues of five small co-resident workgroups overlap better than those of two large
-        // ones (2 - 6 % at 65536 ... 245760 rows).  The tuning knob forces a shape.
         auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * ((dim_y_out + n - 1) / n); };
         const long long cus = faith::compute_units();
         int tm, tn;
-        if (tiles(64, 64) <= cus) { tm = 64; tn = 64; }
-        else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
-        else if (dim_out >= 1024 && tiles(128, 128) >= 16 * cus) { tm = 128; tn = 128; }
-        // many column tiles re-read every block of rows from L2: the large tile halves that (3 - 5 % at
-        // 768 -> 3072 and 512 -> 2048 with 12288 ... 24576 rows) once it fills the machine four times over
-        else if (dim_y_out >= 2048 && tiles(128, 128) >= 8 * cus) { tm = 128; tn = 128; }
-        else { tm = 64; tn = 64; }
+        choose_tile(mw, dim_out, dim_y_out, &tm, &tn);
         const int pick = faith::tune_get(FAITH_TUNE_GEMM_VARIANT);
-        switch (pick) {
-            case 1: tm = 64;  tn = 64;  break;
-            case 2: tm = 128; tn = 128; break;
-            case 3: tm = 128; tn = 64;  break;
-            case 4: tm = 64;  tn = 128; break;
-            default: break;
-        }
         // tiny problems with a reduction worth splitting: a 32 x 32 block per workgroup, K over its wavefronts
         if (dim_out % 32 == 0 && (pick == 5 || (pick == 0 && dim_out >= 128 && 4 * tiles(64, 64) <= cus))) {
             const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
@@ -687,8 +718,6 @@ extern "C" int faith_matmul_group_verification(const float *x_lb, const float *x
 // reduction with fragments loaded straight from global memory (the K pairing of signsplit_gemm_ksplit), stores
 // the block and folds its column norms into its own slots in LDS; the constant-term row is accumulated in
 // double by all threads first (the arithmetic of sliced_tile).  dim_in % (32 words) == 0, K % 8 == 0.
-#include "relax_common.h"
-
 namespace {
 
 struct FusedArgs {
@@ -697,6 +726,76 @@ struct FusedArgs {
     int D, words;
     float eps, qv;
 };
+
+// Layer and dual norm of LARGE problems.  The separate concretize re-reads the 2 * rows * dim_in * N floats the
+// layer has just written (1.07 GB, 176 us after configuration 2).  Instead a workgroup here takes the dim_in / BM
+// tiles of ONE position and one block of columns in turn, so that the column norms of C_l and C_u over all dim_in
+// rows are complete inside the workgroup: each tile's epilogue folds its accumulators into one running value per
+// lane and column block (128 more vector-ALU instructions per 64 x 64 wavefront tile), the lane halves and the two
+// wavefronts that share a column meet in LDS at the end, and the workgroup writes l and u itself -- from the
+// constant terms, which the exact-accumulation kernel has produced in the launch before.  No scratch, a fixed
+// order of additions.  One perturbed word, dim_in % BM == 0, K % 16 == 0.
+struct NormArgs {
+    float *l, *u;      // [Mb, N]
+    int D;
+    float eps, qv;
+};
+
+template <int Q, int MBM, int MBN>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+signsplit_gemm_norms(const GemmArgs g, const NormArgs n) {
+    constexpr int BM = 64 * MBM, BN = 64 * MBN;
+    __shared__ __align__(16) float sm[2 * 4 * 64 * 8 * (MBM + MBN)];
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int xcd = blockIdx.x % XCDS, local = blockIdx.x / XCDS;
+    const int pos = (local / tiles_n) * XCDS + xcd;          // the column blocks of a position meet in one L2
+    const int n_blk = local % tiles_n;
+    if (pos >= g.Mb) return;
+    const int per = n.D / BM;
+    float pl[MBN], pu[MBN];
+#pragma unroll
+    for (int b = 0; b < MBN; ++b) pl[b] = pu[b] = 0.f;
+    for (int t = 0; t < per; ++t) {
+        signsplit_gemm_tile<true, MBM, MBN, Q>(g, sm, pos * per + t, n_blk, pl, pu, n.qv);
+        __syncthreads();          // the next tile's first stage overwrites LDS that a slower wavefront may still read
+    }
+    const int tid = threadIdx.x, lane = tid % 64, wv = tid / 64;
+    const int wm = wv / 2, wn = wv % 2, fi = lane % 32, fh = lane / 32;
+#pragma unroll
+    for (int b = 0; b < MBN; ++b) {
+        pl[b] = ncomb<Q>(pl[b], __shfl_xor(pl[b], 32, 64));
+        pu[b] = ncomb<Q>(pu[b], __shfl_xor(pu[b], 32, 64));
+        if (fh == 0) {
+            const int col = (wn * MBN + b) * 32 + fi;
+            sm[(0 * 2 + wm) * BN + col] = pl[b];
+            sm[(1 * 2 + wm) * BN + col] = pu[b];
+        }
+    }
+    __syncthreads();
+    if (tid < BN) {
+        const int col = n_blk * BN + tid;
+        if (col < g.N) {
+            const float nl = ncomb<Q>(sm[(0 * 2 + 0) * BN + tid], sm[(0 * 2 + 1) * BN + tid]);
+            const float nu = ncomb<Q>(sm[(1 * 2 + 0) * BN + tid], sm[(1 * 2 + 1) * BN + tid]);
+            const size_t o = (size_t)pos * g.N + col;
+            // l = lb + (-eps * norm), two roundings as Bounds.concretize has them (Bounds.py:313, 324)
+            n.l[o] = __fadd_rn(g.Dl[o], __fmul_rn(-n.eps, nfin<Q>(nl, n.qv)));
+            n.u[o] = __fadd_rn(g.Du[o], __fmul_rn(n.eps, nfin<Q>(nu, n.qv)));
+        }
+    }
+}
+
+template <int MBM, int MBN>
+void launch_norms(const GemmArgs &g, const NormArgs &n, int q, hipStream_t st) {
+    const long long tiles_n = (g.N + 64 * MBN - 1) / (64 * MBN);
+    const dim3 gd((unsigned)(((long long)(g.Mb + XCDS - 1) / XCDS) * XCDS * tiles_n)), bd(NTHREADS);
+    switch (q) {
+        case FAITH_Q_1: hipLaunchKernelGGL((signsplit_gemm_norms<FAITH_Q_1, MBM, MBN>), gd, bd, 0, st, g, n); break;
+        case FAITH_Q_2: hipLaunchKernelGGL((signsplit_gemm_norms<FAITH_Q_2, MBM, MBN>), gd, bd, 0, st, g, n); break;
+        case FAITH_Q_INF: hipLaunchKernelGGL((signsplit_gemm_norms<FAITH_Q_INF, MBM, MBN>), gd, bd, 0, st, g, n); break;
+        default: hipLaunchKernelGGL((signsplit_gemm_norms<Q_GENERAL, MBM, MBN>), gd, bd, 0, st, g, n); break;
+    }
+}
 
 constexpr int FUSED_MAX_WORDS = 8;
 
@@ -881,6 +980,32 @@ extern "C" int faith_matmul_concretize_verification(const float *x_lb, const flo
             default: hipLaunchKernelGGL(signsplit_gemm_concretize<Q_GENERAL>, gd, bd, 0, st, f); break;
         }
         return faith::check_launch("faith_matmul_concretize_verification");
+    }
+    // large problems: the tiled kernel, one position's tiles per workgroup, column norms in its epilogue
+    {
+        int tm = 0, tn = 0;
+        choose_tile(mw, dim_out, dim_y_out, &tm, &tn);
+        if (tm == 64) tn = 64;                    // 64 x 128 has no instantiation with norms
+        // knob value 7 keeps layer and concretize apart (for measuring one against the other)
+        const bool tiled = pick != 7 && words == 1 && tiles64 > cus && dim_out % BK == 0 && dim_in % tm == 0 &&
+                           faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) && faith::aligned(W, 16) &&
+                           128LL * dim_out * 4 < 0xffffffffLL && 128LL * dim_y_out * 4 < 0x80000000LL &&   // 32-bit offsets in a tile
+                           mw <= 0x7fffffffLL && (rows + XCDS) * ((dim_y_out + tn - 1) / tn) <= 0x7fffffffLL;
+        if (tiled) {
+            hipStream_t st = static_cast<hipStream_t>(stream);
+            GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
+            // the constant terms first: the coefficient kernel reads them when it writes l and u
+            GemmArgs gb = g;
+            gb.Mw = 0;
+            const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
+            FAITH_REQUIRE(gridb <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_concretize_verification: grid too large");
+            hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+            const NormArgs na{l, u, dim_in, epsilon, f.qv};
+            if (tm == 128 && tn == 128) launch_norms<2, 2>(g, na, q, st);
+            else if (tm == 128) launch_norms<2, 1>(g, na, q, st);
+            else launch_norms<1, 1>(g, na, q, st);
+            return faith::check_launch("faith_matmul_concretize_verification");
+        }
     }
     const int rc = faith_matmul_verification(x_lb, x_ub, x_lw, x_uw, W, bias, y_lb, y_ub, y_lw, y_uw, batch_size, length,
                                              dim_in, dim_out, dim_y_out, stream);

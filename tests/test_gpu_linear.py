@@ -4,7 +4,7 @@ import torch
 
 from oracle import bounds_oracle as O
 from tests.helpers import rand_bounds, as_bounds, close, worst
-from tests.parity import compare_contraction
+from tests.parity import compare_contraction, UNIT_SCALE_ALL
 
 pytestmark = pytest.mark.gpu
 INF = float("inf")
@@ -259,6 +259,47 @@ def test_linear_concretize_general_shapes(shape, words):
     l, u = ops.concretize(*lin, 2.0, 0.05, words)
     for a, b in zip(got, (*lin, l, u)):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("p", [2.0, float("inf"), 1.0, 3.0])
+@pytest.mark.parametrize("shape,force", [
+    ((1, 16, 256, 256, 512), None),    # 128 x 64 tiles (built-in choice), two tiles per position
+    ((1, 128, 64, 128, 576), None),    # 64 x 64 tiles, one tile per position, ragged last column block
+    ((2, 9, 384, 64, 200), 2),         # 128 x 128 tiles forced: three tiles per position, positions over two batch elements
+    ((1, 24, 128, 1024, 1024), 2),     # configuration 2's reduction and width, 24 positions
+])
+def test_linear_concretize_tiled_kernel_with_norms_in_its_epilogue(shape, force, p):
+    """Large problems: the tiled MFMA kernel walks the tiles of one position and finishes l, u itself.  Against the
+    oracle's linear (the harness for contractions) and the oracle's concretize of the GPU's own coefficients; the
+    coefficients must equal the plain layer bit for bit (same tiles, same reduction order)."""
+    from faith_amd import ops, _lib
+    B, L, D, H, N = shape
+    print(f"[case] linear_concretize tiled with norms shape={shape} force={force} p={p}", flush=True)
+    g = torch.Generator().manual_seed(79)
+    x = rand_bounds(g, B, L, D, H, ordered=False, sw=0.5)
+    W = torch.randn(N, H, generator=g) / H ** 0.5
+    bias = 0.01 * torch.randn(N, generator=g)
+    eps = 0.02
+    got = run_fused(x, W, bias, p, eps, 1, force=force)
+    exp = O.linear(x, W, bias)
+    ref, mag = linear64(x, W, bias)
+    for name, a, e in zip(("lw", "lb", "uw", "ub"), got[:4], exp.tensors()):
+        compare_contraction(name, a, e, ref[name], mag[name], UNIT_SCALE_ALL)
+    el, eu = O.concretize(O.LinearBounds(*(t.cpu() for t in got[:4])), p, eps, 1)
+    assert close(got[4], el) and close(got[5], eu), (worst(got[4].cpu(), el), worst(got[5].cpu(), eu))
+    assert bool((got[4] <= got[5]).all())
+    lw, lb, uw, ub, Wd, bd = dev(*x.tensors(), W, bias)
+    if force is not None:
+        _lib.call("faith_tune_set", 1, force)
+    try:
+        lin = ops.linear(lw, lb, uw, ub, Wd, bd)
+    finally:
+        _lib.call("faith_tune_set", 1, 0)
+    for a, b in zip(got[:4], lin):
+        assert torch.equal(a, b)
+    # knob 7 keeps the two launches apart: the same values within the bar (another order of the norm's additions)
+    sep = run_fused(x, W, bias, p, eps, 1, force=7)
+    assert close(got[4], sep[4].cpu()) and close(got[5], sep[5].cpu())
 
 
 def test_linear_concretize_config0_against_oracle():
