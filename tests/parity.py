@@ -149,8 +149,17 @@ CONSTANT_TERMS = {"lb": B_IN_DOUBLE, "ub": B_IN_DOUBLE}
 UNIT_SCALE_ALL = {"lw": UNIT_SCALE, "uw": UNIT_SCALE, "lb": B_IN_DOUBLE, "ub": B_IN_DOUBLE}
 
 
-def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None):
+def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None, ref64_own=None):
     """Parity of one output tensor of a contraction.
+
+    `ref64_own` (dot products): the float64 value of the same formula evaluated from the concrete
+    intervals the GPU itself computed and used.  Those intervals are compared with the oracle's at the
+    plain bar before this is called; their admissible last-bit differences enter every product, and where
+    the products cancel the result inherits them at a size atol does not cover.  An element that misses
+    the plain bar against the oracle but meets it against `ref64_own` is the correct function of its own
+    intervals: it is accepted, counted and entered in LEDGER as "inherited-from-interval" (needs `allow`
+    like any concession); only the elements that remain go on to the accumulation-aware bar, which is then
+    taken against `ref64_own` too.
 
     `allow`: None (the default) means this tensor must meet the plain bar and the fallback below
     is a failure; a caller that expects a tensor on the fallback passes the reason -- a string, or
@@ -179,18 +188,28 @@ def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None):
     if not bool(_bad(got, o32).any()):
         _count(True)
         return "plain"
+    missed = _bad(got, o32)
     ref64 = ref64.detach().cpu().double()
+    oerr = (o32 - ref64).abs()                       # the oracle against the float64 value of ITS intervals
+    if ref64_own is not None:
+        ref64 = ref64_own.detach().cpu().double()    # the GPU against the float64 value of ITS intervals
+        explained = missed & ~_bad(got, ref64)
+        if bool(explained.any()):
+            assert allow is not None, f"{name}: {int(explained.sum())} elements inherit interval differences and no concession is declared"
+            _note("inherited-from-interval", name, elements=int(explained.sum()), of=got.numel())
+        missed = missed & ~explained
+        if not bool(missed.any()):
+            _count(False)
+            return "inherited-from-interval"
     tol = ATOL + RTOL * ref64.abs() + KAPPA * U32 * abs_terms.detach().cpu().double()
     err = (got - ref64).abs()
-    oerr = (o32 - ref64).abs()
-    print(f"   [{name}] plain bar missed by {int(_bad(got, o32).sum())} of {got.numel()} elements; "
+    print(f"   [{name}] plain bar missed by {int(missed.sum())} of {got.numel()} elements; "
           f"vs float64: gpu max err {float(err.max()):.3g}, cpu-oracle max err {float(oerr.max()):.3g}, "
           f"max err/allowance {float((err / tol).max()):.3f}", flush=True)
     assert allow is not None, (f"{name}: misses rtol {RTOL} / atol {ATOL} against the oracle and no concession is "
                                f"declared for it (worst error vs float64 {float(err.max()):.3g}, oracle's {float(oerr.max()):.3g})")
     # the concession is only for elements where atol is finer than an fp32 sum of these terms can promise:
     # the forward-error allowance of the element's own terms, KAPPA * u * sum_k |a_k w_k|, must reach atol
-    missed = _bad(got, o32)
     allowance = KAPPA * U32 * abs_terms.detach().cpu().double()
     assert bool((allowance[missed] >= ATOL).all()), \
         f"{name}: misses the plain bar on elements whose terms are small enough for an fp32 sum to meet atol"

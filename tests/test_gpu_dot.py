@@ -14,11 +14,14 @@ def dev(x):
     return tuple(t.cuda().contiguous() for t in x.tensors())
 
 
-def dot64(x, y, p, eps, words):
-    """float64 value of the planes built from the oracle's fp32 concrete intervals, and the
-    per-output sum of |terms|."""
-    lx, _ = O.concretize(x, p, eps, words)
-    ly, uy = O.concretize(y, p, eps, words)
+def dot64(x, y, p, eps, words, intervals=None):
+    """float64 value of the planes built from fp32 concrete intervals -- the oracle's, or the (l_x, l_y, u_y)
+    handed in (the ones the GPU computed and used) -- and the per-output sum of |terms|."""
+    if intervals is None:
+        lx, _ = O.concretize(x, p, eps, words)
+        ly, uy = O.concretize(y, p, eps, words)
+    else:
+        lx, ly, uy = (t.detach().cpu() for t in intervals)
     lx, ly, uy = lx.double(), ly.double(), uy.double()
     X = {k: v.double() for k, v in zip(("lw", "lb", "uw", "ub"), x.tensors())}
     Y = {k: v.double() for k, v in zip(("lw", "lb", "uw", "ub"), y.tensors())}
@@ -55,8 +58,9 @@ def check(x, y, p, eps, words, what="", allow=None):
             assert close(g, e)
         return
     ref, mag = dot64(x, y, p, eps, words)
+    own, _ = dot64(x, y, p, eps, words, intervals=(xl, yl, yu))
     for name, g, e in zip(("lw", "lb", "uw", "ub"), (zlw, zlb, zuw, zub), exp.tensors()):
-        compare_contraction(name, g, e, ref[name], mag[name], allow)
+        compare_contraction(name, g, e, ref[name], mag[name], allow, ref64_own=own[name])
     return zlw, zlb, zuw, zub
 
 
@@ -165,9 +169,10 @@ def check_v(probs, value, p, eps, words, what="", allow=None):
             assert close(g, e)
         return
     ref, mag = dot64(probs, O.transpose_bounds(value), p, eps, words)
+    own, _ = dot64(probs, O.transpose_bounds(value), p, eps, words, intervals=(xl, yl.transpose(1, 2), yu.transpose(1, 2)))
     for name, g, e in zip(("lw", "lb", "uw", "ub"), (zlw, zlb, zuw, zub), exp.tensors()):
         assert g.shape == e.shape
-        compare_contraction(name, g, e, ref[name], mag[name], allow)
+        compare_contraction(name, g, e, ref[name], mag[name], allow, ref64_own=own[name])
 
 
 @pytest.mark.parametrize("shape", [

@@ -50,18 +50,22 @@ def test_reference_sweep_matmul(length):
             T_lin.check(x, W, None, f"reference sweep L={length}", allow=UNIT_SCALE_ALL)
 
 
-def _dot_case(x, y, run, oracle, what):
-    """Plain bar first; the float64 value of the same inputs is only worked out for a tensor that misses it."""
+def _dot_case(x, y, run, oracle, what, context=False):
+    """Plain bar first; the float64 values of the same inputs (from the oracle's intervals and from the GPU's own)
+    are only worked out for a case with a tensor that misses it."""
     print(f"[case] {what}", flush=True)
-    got = run()
+    *got, (x_l, _x_u, y_l, y_u) = run()
     torch.cuda.synchronize()
     exp = oracle()
     bad = [n for n, a, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()) if not close(a, e)]
     if not bad:
         return
+    if context:
+        y_l, y_u = y_l.transpose(1, 2), y_u.transpose(1, 2)          # intervals of the values as of value.t()
     ref, mag = T_dot.dot64(x, y, 2.0, 0.5, 1)
+    own, _ = T_dot.dot64(x, y, 2.0, 0.5, 1, intervals=(x_l, y_l, y_u))
     for name, a, e in zip(("lw", "lb", "uw", "ub"), got, exp.tensors()):
-        compare_contraction(name, a, e, ref[name], mag[name], UNIT_SCALE_ALL)
+        compare_contraction(name, a, e, ref[name], mag[name], UNIT_SCALE_ALL, ref64_own=own[name])
 
 
 @pytest.mark.parametrize("length", LENGTHS)
@@ -74,7 +78,7 @@ def test_reference_sweep_dot_product_qk(batch, length):
             if 16.0 * batch * length * length * dim_in * dim_out > COST_CAP:
                 continue
             x, y = draw(g, batch, length, dim_in, dim_out), draw(g, batch, length, dim_in, dim_out)
-            _dot_case(x, y, lambda: ops.dot_product_qk(T_dot.dev(x), T_dot.dev(y), 2.0, 0.5, 1),
+            _dot_case(x, y, lambda: ops.dot_product_qk(T_dot.dev(x), T_dot.dev(y), 2.0, 0.5, 1, return_intervals=True),
                       lambda: O.dot_product(x, y, 2.0, 0.5, 1), f"sweep QK B={batch} L={length} D={dim_in} d={dim_out}")
 
 
@@ -90,6 +94,6 @@ def test_reference_sweep_dot_product_v(batch, length):
             probs = draw(g, batch, length, dim_in, length)
             value = draw(g, batch, length, dim_in, dim_out)
             _dot_case(probs, O.transpose_bounds(value),
-                      lambda: ops.dot_product_v(T_dot.dev(probs), T_dot.dev(value), 2.0, 0.5, 1),
+                      lambda: ops.dot_product_v(T_dot.dev(probs), T_dot.dev(value), 2.0, 0.5, 1, return_intervals=True),
                       lambda: O.context(probs, value, 2.0, 0.5, 1),
-                      f"sweep V B={batch} L={length} D={dim_in} d={dim_out}")
+                      f"sweep V B={batch} L={length} D={dim_in} d={dim_out}", context=True)
