@@ -456,7 +456,21 @@ def bench_config3(args, ops, O, wl):
     flopv = B * (8 * 2 * L * D * L * d + 8 * 2 * L * L * d)
     tv = gpu_times_ms(lambda: ops.dot_product_v(probs, quad(y), c["p"], c["eps"], 1, out=outv), 50, 5)
     ev = op_entry("extra: context (probs.value) 4 heads [4,128,256,128].[4,128,256,64]", "mfma", tv, flopv)
-    return [e, ev]
+    # the same scores through the reference's own calling convention: operands [B, L, dim_out, dim_in], result
+    # [B, Lx, Ly, dim_in] (vector ALU with lanes along dim_in, no re-layout); the roofline is still the MFMA peak
+    from faith_amd import c_bound
+    T = lambda t_: t_.transpose(2, 3).contiguous()
+    xt, yt = (T(x["lw"]), T(x["uw"])), (T(y["lw"]), T(y["uw"]))
+    scr = [torch.empty(B, L, d, device="cuda") for _ in range(4)]
+    zt = (torch.empty(B, L, L, device="cuda"), torch.empty(B, L, L, device="cuda"),
+          torch.empty(B, L, L, D, device="cuda"), torch.empty(B, L, L, D, device="cuda"))
+    c_bound.p, c_bound.words = c["p"], 1
+    tt = gpu_times_ms(lambda: c_bound.c_dot_product_verification_QK(*scr, x["lb"], x["ub"], y["lb"], y["ub"], xt[0], xt[1],
+                                                                    yt[0], yt[1], *zt, B, L, d, D, c["eps"]), 50, 5)
+    c_bound.p = 2.0
+    et = op_entry("extra: config3 scores in the reference's transposed layout (c_bound.c_dot_product_verification_QK)",
+                  "mfma", tt, flop)
+    return [e, ev, et]
 
 
 def bench_config4(args, ops, O, wl):
@@ -478,7 +492,26 @@ def bench_config4(args, ops, O, wl):
                "sample": "D_in=32 of 256, median of 3"}
     e = op_entry("config4 conv3x3 64->128 [1,256,64,32,32]", "mfma", t, flop, cpu)
     e2 = op_entry("config4 concretize(p=inf) of the result", "hbm", tc, 8 * D * Co * Hh * Hh + 16 * Co * Hh * Hh)
-    return [e, e2]
+    out_entries = [e, e2]
+    # the other layer shapes of a CNN verifier, same D_in = 256 and 32 x 32 input (not among the five configurations):
+    # each takes a straight-line instantiation of the implicit-GEMM kernel with the tile that fits its result
+    del out
+    g = torch.Generator().manual_seed(1404)
+    for (ci, co, k, s_, p_, what) in ((64, 128, 3, 2, 1, "3x3 stride 2 64->128"), (64, 128, 1, 1, 0, "1x1 64->128"),
+                                      (32, 64, 5, 1, 2, "5x5 32->64"), (3, 64, 3, 1, 1, "3x3 3->64 (first layer)")):
+        lw = (torch.randn(1, D, ci, Hh, Hh, generator=g) * 0.05).cuda()
+        uw = lw + 0.005
+        lb = torch.randn(1, ci, Hh, Hh, generator=g).cuda()
+        ub = lb + 0.1
+        Wk = (torch.randn(co, ci, k, k, generator=g) * (2.0 / (ci * k * k)) ** 0.5).cuda()
+        ho = (Hh + 2 * p_ - k) // s_ + 1
+        o_ = ops.conv2d(lw, lb, uw, ub, Wk, None, s_, p_)
+        tk = gpu_times_ms(lambda: ops.conv2d(lw, lb, uw, ub, Wk, None, s_, p_, out=o_), 10 if args.profile else 50, 2)
+        fl = 4 * 2 * (D + 1) * co * ho * ho * ci * k * k
+        out_entries.append(op_entry(f"extra: conv {what} [1,256,{ci},32,32]", "mfma", tk, fl, None,
+                                    {"result_write_GBs": round(2 * D * co * ho * ho * 4 / statistics.median(tk) / 1e6, 1)}))
+        del lw, uw, o_
+    return out_entries
 
 
 def bench_layer(args, wl):
