@@ -326,7 +326,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
 // column predicates and no second pass, and the kernel is a slab copy with the reduction and the
 // per-neuron stage between its loads and its stores: at configuration 1 it runs within 3 % of
 // that copy, where the general kernel above needs 25 % more.
-template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4>
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE))) act_resident(const ActArgs a) {
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
     static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
@@ -347,8 +347,13 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
         if (i * RG < a.D) {
-            dl[i].load(p_lw + i * row_step);
-            du[i].load(p_uw + i * row_step);
+            if (NTL) {
+                dl[i].load_nt(p_lw + i * row_step);
+                du[i].load_nt(p_uw + i * row_step);
+            } else {
+                dl[i].load(p_lw + i * row_step);
+                du[i].load(p_uw + i * row_step);
+            }
         } else {
             dl[i].zero();
             du[i].zero();
@@ -523,12 +528,12 @@ void launch_natural(const ActArgs &a, hipStream_t st) {
                        dim3(NTHREADS), smem, st, a);
 }
 
-template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4>
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false>
 void launch_resident(const ActArgs &a, hipStream_t st) {
     constexpr int TH = TPR * 4;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
-    faith::reserve_lds(act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE>, smem);
-    hipLaunchKernelGGL((act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS),
+    faith::reserve_lds(act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE, NTL>, smem);
+    hipLaunchKernelGGL((act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE, NTL>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS),
                        smem, st, a);
 }
 
@@ -696,12 +701,13 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         // while the operands can sit in the 256 MB memory-side cache (40.2 against 42.8 us at
         // [128, 256, 512], every launch on the same 269 MB); sixteen wavefronts holding two rows each are
         // 12 % ahead when every byte comes from and goes to HBM (55 against 62 us on the same shape with
-        // five operand sets in turn).  An object whose traffic exceeds the cache by more than a quarter
-        // cannot be resident, so it takes the second shape; knob values 7 / 8 force one or the other.
+        // five operand sets in turn), and 3 % more with non-temporal loads (54 us; those cost 25 % when the
+        // operands are cached).  An object whose traffic exceeds the cache by more than a quarter cannot be
+        // resident, so it takes the second shape; knob values 7 / 8 force one or the other.
         const long long traffic = 16LL * a.rows * a.D * a.H;
         const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 5LL * (256LL << 20) / 4);
         if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(a, st);
-        else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8>(a, st);
+        else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(a, st);
         else launch_resident<MODE, Q, 8, 256, 8>(a, st);
         return;
     }

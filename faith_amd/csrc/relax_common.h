@@ -47,6 +47,10 @@ template <>
 struct Vec<4> {
     float4 v;
     __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
+    __device__ __forceinline__ void load_nt(const float *p) {
+        const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+        v = make_float4(t[0], t[1], t[2], t[3]);
+    }
     __device__ __forceinline__ void store(float *p) const {
         const v4f t = {v.x, v.y, v.z, v.w};
         __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));

@@ -27,9 +27,17 @@ Layers are plain objects with `.weight` / `.bias` tensors, laid out like the ref
 """
 from __future__ import annotations
 
+import contextlib
 import math
 
 import torch
+
+
+def _scope(buffers):
+    """`buffers`: None, or persistent result buffers for the operator calls of one propagation -- any object
+    whose scope() is a context manager (faith_amd.ops.Workspace): the caller owns results and scratch across
+    calls, as the reference's adapters do (Bounds.py:1270-1277), and a repeated propagation allocates none."""
+    return buffers.scope() if buffers is not None else contextlib.nullcontext()
 
 
 def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, norm=None, layer_norm="no_var",
@@ -216,10 +224,15 @@ def propagate(bounds, network):
     return bounds
 
 
-def verify_safety(make_bounds, network, embeddings, index, eps, label, p=2.0, perturbed_words=1):
+def verify_safety(make_bounds, network, embeddings, index, eps, label, p=2.0, perturbed_words=1, buffers=None):
     """VerifierForward.verify_safety (:93-125): True if the label provably survives every
     perturbation of norm <= eps of the embedding at `index`.  A failed precondition inside the
     propagation (reciprocal or sqrt of a bound that reaches zero) counts as not verified, as there."""
+    with _scope(buffers):
+        return _verify_safety(make_bounds, network, embeddings, index, eps, label, p, perturbed_words)
+
+
+def _verify_safety(make_bounds, network, embeddings, index, eps, label, p, perturbed_words):
     x = bound_input(make_bounds, embeddings, index, eps, perturbed_words, p)
     collector = getattr(type(x), "collect_failures", None)
     try:
@@ -243,12 +256,12 @@ def verify_safety(make_bounds, network, embeddings, index, eps, label, p=2.0, pe
         return False
 
 
-def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label, p=2.0):
+def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label, p=2.0, buffers=None):
     """verify_safety for several (position, radius) pairs of one sentence in one propagation.
     Returns a list of bools.  Needs a bound object that reports failed preconditions per batch
     element instead of raising (`collect_failures`, as faith_amd.Bounds has)."""
     x = bound_inputs(make_bounds, embeddings, indices, radii, p)
-    with type(x).collect_failures(len(indices), embeddings.device) as failed:
+    with _scope(buffers), type(x).collect_failures(len(indices), embeddings.device) as failed:
         if network.embedding_norm is not None:
             x = x.layer_norm(network.embedding_norm, network.layer_norm)
         x = propagate(x, network)
@@ -259,16 +272,17 @@ def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label,
 
 
 def certified_radii(make_bounds, network, embeddings, positions, label, p=2.0, max_eps=0.1, num_iters=10,
-                    batched=False, captured=False):
+                    batched=False, captured=False, buffers=None):
     """The bisection of Verifier.verify (Verifiers/Verifier.py:131-139) for every position: l, r = 0,
     max_eps; num_iters times { m = (l + r) / 2; verified at m ? l = m : r = m }; the answer is l.
     batched = True runs step j of all positions as one propagation; captured = True also replays
-    that propagation from a HIP graph captured at the first step."""
+    that propagation from a HIP graph captured at the first step.  buffers: persistent result buffers shared
+    by all steps (see _scope); every step overwrites what the one before produced."""
     lo = [0.0] * len(positions)
     hi = [float(max_eps)] * len(positions)
     if batched or captured:
         step = CapturedVerifier(make_bounds, network, embeddings, len(positions), label, p) if captured else \
-            (lambda idx, r: verify_safety_batch(make_bounds, network, embeddings, idx, r, label, p))
+            (lambda idx, r: verify_safety_batch(make_bounds, network, embeddings, idx, r, label, p, buffers))
         for _ in range(num_iters):
             mid = [(a + b) / 2 for a, b in zip(lo, hi)]
             safe = step(positions, mid)
@@ -281,7 +295,7 @@ def certified_radii(make_bounds, network, embeddings, positions, label, p=2.0, m
     for i, pos in enumerate(positions):
         for _ in range(num_iters):
             m = (lo[i] + hi[i]) / 2
-            if verify_safety(make_bounds, network, embeddings, pos, m, label, p):
+            if verify_safety(make_bounds, network, embeddings, pos, m, label, p, buffers=buffers):
                 lo[i] = m
             else:
                 hi[i] = m

@@ -64,6 +64,83 @@ def _stream(t):
     return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if idx is None else idx)
 
 
+# ------------------------------------------------------------------------------------------
+# Result buffers.  By default every call allocates its results (torch's caching allocator).  The reference
+# has the caller own all results and scratch (Bounds.py:1270-1277); a caller that runs the same sequence of
+# operators again and again -- one propagation per bisection step, per position, per sentence -- can do the
+# same here with a Workspace: inside `with ops.workspace(ws):` the i-th result buffer requested during the
+# pass is the i-th buffer the workspace holds (allocated on the first pass, reused when shape and device
+# match), so a repeated pass allocates nothing.  What a pass returned is overwritten by the next one.
+# ------------------------------------------------------------------------------------------
+class Workspace:
+    """Persistent result and scratch buffers of one repeated sequence of operator calls."""
+
+    def __init__(self):
+        self.buffers = []
+        self.cursor = 0
+        self.allocations = 0
+
+    def reset(self):
+        self.cursor = 0
+
+    def take(self, shape, device):
+        i = self.cursor
+        self.cursor += 1
+        if i < len(self.buffers):
+            t = self.buffers[i]
+            if t.shape == shape and t.device == device:
+                return t
+        t = torch.empty(shape, device=device, dtype=torch.float32)
+        self.allocations += 1
+        if i < len(self.buffers):
+            self.buffers[i] = t
+        else:
+            self.buffers.append(t)
+        return t
+
+    def bytes(self):
+        return sum(t.numel() * 4 for t in self.buffers)
+
+    def scope(self):
+        """Context manager: the operator calls inside take their buffers from this workspace, from its start."""
+        return workspace(self)
+
+
+_WORKSPACE = None
+
+
+class workspace:
+    """Context manager: result buffers of the calls inside come from `ws`, in call order, from its start."""
+
+    def __init__(self, ws):
+        self.ws = ws
+
+    def __enter__(self):
+        global _WORKSPACE
+        self.previous = _WORKSPACE
+        if self.ws is not None:
+            self.ws.reset()
+        _WORKSPACE = self.ws
+        return self.ws
+
+    def __exit__(self, *exc):
+        global _WORKSPACE
+        _WORKSPACE = self.previous
+        return False
+
+
+def _empty(*shape, device):
+    if _WORKSPACE is not None:
+        return _WORKSPACE.take(torch.Size(shape), device)
+    return torch.empty(shape, device=device, dtype=torch.float32)
+
+
+def _empty_like(t):
+    if _WORKSPACE is not None:
+        return _WORKSPACE.take(t.shape, t.device)
+    return torch.empty_like(t)
+
+
 class _NoGuard:
     def __enter__(self):
         return self
@@ -124,8 +201,8 @@ def concretize(lw, lb, uw, ub, p, eps, words=1, layout=LAYOUT_NATURAL):
     """Concrete interval [l, u] of every neuron.  Shapes as Bounds.concretize."""
     B, L, D, H = _wb_shapes(lw, lb, layout)
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
-    l = torch.empty_like(lb)
-    u = torch.empty_like(ub)
+    l = _empty_like(lb)
+    u = _empty_like(ub)
     with _on(lw.device, "concretize", (B * L, D, H)):
         _lib.call("faith_concretize", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(l), _ptr(u),
                   B * L, D, H, float(eps), q_code(p), int(words), layout, _stream(lw))
@@ -140,14 +217,14 @@ def _activation(entry, lw, lb, uw, ub, p, eps, words, layout, return_interval, o
     B, L, D, H = _wb_shapes(lw, lb, layout)
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
     if out is None:
-        olw, olb, ouw, oub = (torch.empty_like(lw), torch.empty_like(lb),
-                              torch.empty_like(uw), torch.empty_like(ub))
+        olw, olb, ouw, oub = (_empty_like(lw), _empty_like(lb),
+                              _empty_like(uw), _empty_like(ub))
     else:
         olw, olb, ouw, oub = out
         _check("out lw", olw, lw.shape); _check("out uw", ouw, lw.shape)
         _check("out lb", olb, lb.shape); _check("out ub", oub, lb.shape)
-    l = torch.empty_like(lb) if return_interval else None
-    u = torch.empty_like(ub) if return_interval else None
+    l = _empty_like(lb) if return_interval else None
+    u = _empty_like(ub) if return_interval else None
     with _on(lw.device, "act", (B * L, D, H)):
         if entry in _UNARY:
             _lib.call("faith_unary_verification", _UNARY[entry], _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb),
@@ -201,7 +278,7 @@ def multiply(x, y, p, eps, words=1, out=None):
                      ("y.ub", yub, xlb.shape)):
         _check(n, t, s_)
     if out is None:
-        out = (torch.empty_like(xlw), torch.empty_like(xlb), torch.empty_like(xlw), torch.empty_like(xlb))
+        out = (_empty_like(xlw), _empty_like(xlb), _empty_like(xlw), _empty_like(xlb))
     zlw, zlb, zuw, zub = out
     _check("out lw", zlw, xlw.shape); _check("out uw", zuw, xlw.shape)
     _check("out lb", zlb, xlb.shape); _check("out ub", zub, xlb.shape)
@@ -243,12 +320,12 @@ def affine(x, scale=None, other=None, shift=None):
         if not isinstance(shift, torch.Tensor):
             shift = torch.full((H,), float(shift), device=lb.device, dtype=torch.float32)
         _check("shift", shift, (H,))
-    olb, oub = torch.empty_like(lb), torch.empty_like(ub)
+    olb, oub = _empty_like(lb), _empty_like(ub)
     if scale is None and other is None:
         # a shift moves the constant terms only: the coefficient tensors are shared, as in the reference
         olw, ouw, rows_w = lw, uw, 0
     else:
-        olw, ouw = torch.empty_like(lw), torch.empty_like(uw)
+        olw, ouw = _empty_like(lw), _empty_like(uw)
     with _on(lw.device):
         _lib.call("faith_affine_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(vec), scalar,
                   _ptr(alb), _ptr(aub), _ptr(alw), _ptr(auw), _ptr(shift), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
@@ -275,7 +352,7 @@ def rowsum(lw, lb, uw, ub):
     """Sum over the last axis, written to every position of that axis, for all four tensors
     (the sum / repeat pair of Bounds.softmax)."""
     rows_w, rows_b, H = _object(lw, lb, uw, ub)
-    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    olw, olb, ouw, oub = _empty_like(lw), _empty_like(lb), _empty_like(uw), _empty_like(ub)
     with _on(lw.device):
         _lib.call("faith_rowsum_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw),
                   _ptr(ouw), rows_w, rows_b, H, _stream(lw))
@@ -285,7 +362,7 @@ def rowsum(lw, lb, uw, ub):
 def rowmean(lw, lb, uw, ub):
     """Mean over the last axis, written to every position of that axis: matmul with the H x H matrix of 1 / H."""
     rows_w, rows_b, H = _object(lw, lb, uw, ub)
-    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    olw, olb, ouw, oub = _empty_like(lw), _empty_like(lb), _empty_like(uw), _empty_like(ub)
     with _on(lw.device):
         _lib.call("faith_rowmean_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub), _ptr(olw),
                   _ptr(ouw), rows_w, rows_b, H, _stream(lw))
@@ -307,7 +384,7 @@ def layer_norm(lw, lb, uw, ub, weight=None, bias=None, other=None):
         alw, alb, auw, aub = other
     else:
         alw = alb = auw = aub = None
-    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
+    olw, olb, ouw, oub = _empty_like(lw), _empty_like(lb), _empty_like(uw), _empty_like(ub)
     with _on(lw.device):
         _lib.call("faith_layer_norm_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(alb), _ptr(aub),
                   _ptr(alw), _ptr(auw), _ptr(weight), _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
@@ -328,8 +405,8 @@ def softmax(lw, lb, uw, ub, p, eps, words=1, return_sum_bound=False, scale=1.0):
     (FAITH_ERR_UNSUPPORTED) when the slab does not fit: see softmax_fits."""
     B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
     _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
-    olw, olb, ouw, oub = torch.empty_like(lw), torch.empty_like(lb), torch.empty_like(uw), torch.empty_like(ub)
-    l_sum = torch.empty((B, L), device=lw.device, dtype=torch.float32) if return_sum_bound else None
+    olw, olb, ouw, oub = _empty_like(lw), _empty_like(lb), _empty_like(uw), _empty_like(ub)
+    l_sum = _empty(B, L, device=lw.device) if return_sum_bound else None
     with _on(lw.device):
         _lib.call("faith_softmax_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(olb), _ptr(oub),
                   _ptr(olw), _ptr(ouw), _ptr(l_sum), float(scale), B * L, D, H, float(eps), q_code(p), int(words),
@@ -345,7 +422,7 @@ def interval_unary(kind, l, u):
     if kind not in _UNARY:
         raise ValueError(f"unknown operator {kind!r}")
     _check("l", l); _check("u", u, l.shape)
-    olb, oub = torch.empty_like(l), torch.empty_like(u)
+    olb, oub = _empty_like(l), _empty_like(u)
     with _on(l.device):
         _lib.call("faith_interval_unary", _UNARY[kind], _ptr(l), _ptr(u), _ptr(olb), _ptr(oub), l.numel(), _stream(l))
     return olb, oub
@@ -354,7 +431,7 @@ def interval_unary(kind, l, u):
 def interval_product(xl, xu, yl, yu):
     """Interval of the elementwise product of [xl, xu] and [yl, yu].  Returns (lb, ub)."""
     _check("xl", xl); _check("xu", xu, xl.shape); _check("yl", yl, xl.shape); _check("yu", yu, xl.shape)
-    zl, zu = torch.empty_like(xl), torch.empty_like(xl)
+    zl, zu = _empty_like(xl), _empty_like(xl)
     with _on(xl.device):
         _lib.call("faith_interval_product", _ptr(xl), _ptr(xu), _ptr(yl), _ptr(yu), _ptr(zl), _ptr(zu), xl.numel(),
                   _stream(xl))
@@ -372,10 +449,10 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     if bias is not None:
         _check("bias", bias, (N,))
     if out is None:
-        olw = torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32)
-        ouw = torch.empty_like(olw)
-        olb = torch.empty(B, L, N, device=lw.device, dtype=torch.float32)
-        oub = torch.empty_like(olb)
+        olw = _empty(B, L, D, N, device=lw.device)
+        ouw = _empty_like(olw)
+        olb = _empty(B, L, N, device=lw.device)
+        oub = _empty_like(olb)
     else:
         olw, olb, ouw, oub = out
         _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
@@ -400,12 +477,12 @@ def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1, out=None):
     if bias is not None:
         _check("bias", bias, (N,))
     if out is None:
-        olw = torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32)
-        ouw = torch.empty_like(olw)
-        olb = torch.empty(B, L, N, device=lw.device, dtype=torch.float32)
-        oub = torch.empty_like(olb)
-        l = torch.empty_like(olb)
-        u = torch.empty_like(olb)
+        olw = _empty(B, L, D, N, device=lw.device)
+        ouw = _empty_like(olw)
+        olb = _empty(B, L, N, device=lw.device)
+        oub = _empty_like(olb)
+        l = _empty_like(olb)
+        u = _empty_like(olb)
     else:
         olw, olb, ouw, oub, l, u = out
         _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
@@ -434,10 +511,10 @@ def linear_group(lw, lb, uw, ub, weights, biases=None):
         _check(f"weight {i}", W, (N, H))
         if b is not None:
             _check(f"bias {i}", b, (N,))
-    outs = [(torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32),
-             torch.empty(B, L, N, device=lw.device, dtype=torch.float32),
-             torch.empty(B, L, D, N, device=lw.device, dtype=torch.float32),
-             torch.empty(B, L, N, device=lw.device, dtype=torch.float32)) for _ in range(n)]
+    outs = [(_empty(B, L, D, N, device=lw.device),
+             _empty(B, L, N, device=lw.device),
+             _empty(B, L, D, N, device=lw.device),
+             _empty(B, L, N, device=lw.device)) for _ in range(n)]
     arr = ctypes.c_void_p * n
     ptrs = lambda ts: arr(*[_ptr(t) for t in ts])
     a_w, a_b = ptrs(weights), ptrs(biases)
@@ -463,13 +540,13 @@ def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
-    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
+    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    y_l = _empty_like(ylb); y_u = _empty_like(ylb)
     if out is None:
-        zlw = torch.empty(B, Lx, D, Ly, device=dev, dtype=torch.float32)
-        zuw = torch.empty_like(zlw)
-        zlb = torch.empty(B, Lx, Ly, device=dev, dtype=torch.float32)
-        zub = torch.empty_like(zlb)
+        zlw = _empty(B, Lx, D, Ly, device=dev)
+        zuw = _empty_like(zlw)
+        zlb = _empty(B, Lx, Ly, device=dev)
+        zub = _empty_like(zlb)
     else:
         zlw, zlb, zuw, zub = out
         _check("out lw", zlw, (B, Lx, D, Ly)); _check("out uw", zuw, (B, Lx, D, Ly))
@@ -500,13 +577,13 @@ def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
-    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
+    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    y_l = _empty_like(ylb); y_u = _empty_like(ylb)
     if out is None:
-        zlw = torch.empty(B, Lx, D, dv, device=dev, dtype=torch.float32)
-        zuw = torch.empty_like(zlw)
-        zlb = torch.empty(B, Lx, dv, device=dev, dtype=torch.float32)
-        zub = torch.empty_like(zlb)
+        zlw = _empty(B, Lx, D, dv, device=dev)
+        zuw = _empty_like(zlw)
+        zlb = _empty(B, Lx, dv, device=dev)
+        zub = _empty_like(zlb)
     else:
         zlw, zlb, zuw, zub = out
         _check("out lw", zlw, (B, Lx, D, dv)); _check("out uw", zuw, (B, Lx, D, dv))
@@ -539,12 +616,12 @@ def attention_scores(x, y, heads, p, eps, words=1):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
-    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
-    zlw = torch.empty(B * heads, Lx, D, Ly, device=dev, dtype=torch.float32)
-    zuw = torch.empty_like(zlw)
-    zlb = torch.empty(B * heads, Lx, Ly, device=dev, dtype=torch.float32)
-    zub = torch.empty_like(zlb)
+    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    y_l = _empty_like(ylb); y_u = _empty_like(ylb)
+    zlw = _empty(B * heads, Lx, D, Ly, device=dev)
+    zuw = _empty_like(zlw)
+    zlb = _empty(B * heads, Lx, Ly, device=dev)
+    zub = _empty_like(zlb)
     with _on(dev, "dot_qk", (B * heads, Lx, Ly, D, H // heads)):
         _lib.call("faith_attention_scores", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
@@ -573,12 +650,12 @@ def attention_context(x, y, p, eps, words=1):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = torch.empty_like(xlb); x_u = torch.empty_like(xlb)
-    y_l = torch.empty_like(ylb); y_u = torch.empty_like(ylb)
-    zlw = torch.empty(B, Lx, D, H, device=dev, dtype=torch.float32)
-    zuw = torch.empty_like(zlw)
-    zlb = torch.empty(B, Lx, H, device=dev, dtype=torch.float32)
-    zub = torch.empty_like(zlb)
+    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    y_l = _empty_like(ylb); y_u = _empty_like(ylb)
+    zlw = _empty(B, Lx, D, H, device=dev)
+    zuw = _empty_like(zlw)
+    zlb = _empty(B, Lx, H, device=dev)
+    zub = _empty_like(zlb)
     with _on(dev, "dot_v", (BH, Lx, H // heads, D, Lk)):
         _lib.call("faith_attention_context", _ptr(x_l), _ptr(y_l), _ptr(x_u), _ptr(y_u),
                   _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
@@ -605,10 +682,10 @@ def conv2d(lw, lb, uw, ub, weight, bias=None, stride=1, padding=0, out=None):
     if Ho <= 0 or Wo <= 0:
         raise ValueError("convolution output would be empty")
     if out is None:
-        olw = torch.empty(1, D, Co, Ho, Wo, device=lw.device, dtype=torch.float32)
-        ouw = torch.empty_like(olw)
-        olb = torch.empty(1, Co, Ho, Wo, device=lw.device, dtype=torch.float32)
-        oub = torch.empty_like(olb)
+        olw = _empty(1, D, Co, Ho, Wo, device=lw.device)
+        ouw = _empty_like(olw)
+        olb = _empty(1, Co, Ho, Wo, device=lw.device)
+        oub = _empty_like(olb)
     else:
         olw, olb, ouw, oub = out
         _check("out lw", olw, (1, D, Co, Ho, Wo)); _check("out uw", ouw, (1, D, Co, Ho, Wo))

@@ -188,6 +188,34 @@ def test_batched_bisection_on_hip_matches_one_at_a_time_and_the_oracle(mode):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("batched", [False, True])
+def test_persistent_buffers_give_the_same_radii_and_stop_allocating(batched):
+    """The caller owns results and scratch across propagations (ops.Workspace, as the reference's adapters own
+    theirs, Bounds.py:1270-1277): the same radii as with per-call allocation, and after the first propagation
+    the operator calls allocate no buffer."""
+    from faith_amd import Bounds, ops
+    layer, embed_norm, pooler, classifier, emb = build(11, "no_var")
+    parts = (layer, embed_norm, pooler, classifier)
+    _, margin = true_layer(emb.double(), layer, embed_norm, "no_var", pooler, classifier)
+    label = 0 if float(margin[0, 0]) > 0 else 1
+    positions, max_eps, iters = [1, 2, 3], 0.5, 5
+    gnet = network_of(tuple(to_device(x, "cuda") for x in parts), "no_var")
+    gmake = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    want = F.certified_radii(gmake, gnet, emb.cuda(), positions, label, 2.0, max_eps, iters, batched=batched)
+    ws = ops.Workspace()
+    if batched:
+        F.verify_safety_batch(gmake, gnet, emb.cuda(), positions, [0.01] * 3, label, 2.0, buffers=ws)
+    else:
+        F.verify_safety(gmake, gnet, emb.cuda(), 1, 0.01, label, 2.0, buffers=ws)
+    first = ws.allocations
+    assert first > 20 and ws.bytes() > 0
+    got = F.certified_radii(gmake, gnet, emb.cuda(), positions, label, 2.0, max_eps, iters, batched=batched, buffers=ws)
+    assert got == want
+    assert ws.allocations == first, "a repeated propagation allocated result buffers"
+    assert ops._WORKSPACE is None
+
+
+@pytest.mark.gpu
 def test_failed_preconditions_are_recorded_per_batch_element():
     """Inside collect_failures a reciprocal whose interval reaches zero marks its own batch element
     only and nothing raises; outside it asserts, as the reference does."""
