@@ -196,12 +196,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void *base, size_
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0,
                                              (int)((bytes >> 32) ? 0xffffffffu : (unsigned)bytes), 0x00020000);
 }
-// max(v, 0) / min(v, 0) as single instructions (fmaxf / fminf add a canonicalising v_max each).
-// As a median of three, which the compiler knows to be a vector-ALU write: inline assembly would
-// hide that from its hazard recognizer, and the MFMA that reads the result next would not get the
-// wait states it needs.
-__device__ __forceinline__ float pos1(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, __builtin_inff()); }
-__device__ __forceinline__ float neg1(float v) { return __builtin_amdgcn_fmed3f(v, -__builtin_inff(), 0.f); }
+// max(v, 0) / min(v, 0), one instruction each: this file is compiled with -fno-honor-nans, without which fmaxf /
+// fminf (and a median of three) come with a canonicalising v_max per value.  Plain builtins: the compiler sees the
+// write, so an MFMA or an LDS store that consumes the result gets the wait states it needs.  (A NaN weight or
+// interval, which the reference would carry through, is not preserved by the split.)
+__device__ __forceinline__ float pos1(float v) { return __builtin_fmaxf(v, 0.f); }
+__device__ __forceinline__ float neg1(float v) { return __builtin_fminf(v, 0.f); }
 
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 conv_signsplit_k3s1(const ConvArgs g) {

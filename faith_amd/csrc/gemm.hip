@@ -57,11 +57,12 @@ struct GemmArgs {
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
-// max(v, 0) / min(v, 0) as one instruction each, as a median of three with +-infinity: fmaxf / fminf come with a
-// canonicalising v_max each, and the compiler sees this form (no inline assembly whose result an MFMA or an LDS
-// store could consume before the hazard recognizer knows it was written)
-__device__ __forceinline__ float pos1(float v) { return __builtin_amdgcn_fmed3f(v, 0.f, __builtin_inff()); }
-__device__ __forceinline__ float neg1(float v) { return __builtin_amdgcn_fmed3f(v, -__builtin_inff(), 0.f); }
+// max(v, 0) / min(v, 0), one instruction each: this file is compiled with -fno-honor-nans, without which fmaxf /
+// fminf (and a median of three) come with a canonicalising v_max per value.  Plain builtins: the compiler sees the
+// write, so an MFMA or an LDS store that consumes the result gets the wait states it needs.  (A NaN weight or
+// interval, which the reference would carry through, is not preserved by the split.)
+__device__ __forceinline__ float pos1(float v) { return __builtin_fmaxf(v, 0.f); }
+__device__ __forceinline__ float neg1(float v) { return __builtin_fminf(v, 0.f); }
 __device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
 __device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
 
