@@ -218,6 +218,9 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     const int nchunks = (a.D + CHUNK - 1) / CHUNK;
 
     Vec<VEC> dl[RPT], du[RPT];
+    // concretize only: an upper interval nobody asked for (the first operand of a dot product: its planes
+    // take x from below on both sides) -- the upper coefficients then stay where they are
+    const bool want_u = MODE != CONCRETIZE || p_u != nullptr;
 
     if (nchunks > 1 && lane < TPR) {
         for (int w = 0; w < a.words; ++w)
@@ -234,7 +237,8 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
             const int row = ch * CHUNK + i * RG + rg;
             if (col_ok && row < a.D) {
                 dl[i].load(p_lw + base + (size_t)row * H);
-                du[i].load(p_uw + base + (size_t)row * H);
+                if (want_u) du[i].load(p_uw + base + (size_t)row * H);
+                else du[i].zero();
             } else {
                 dl[i].zero();
                 du[i].zero();
@@ -674,7 +678,12 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
             return;
         }
         const int pick = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
-        if (vec4 && (pick == 11 || (pick == 0 && (long long)a.H * 4 >= 65536)))
+        // ... and where the objects are large (64 MB and more: the operands of a configuration-size dot product),
+        // where many small workgroups that start and finish at different times keep the memory system busier
+        // than two rounds of sixteen-wavefront ones: 23.8 against 25.4 us at 134 MB, 23.2 against 25.7 us at
+        // [512, 256, 128]
+        const long long bytes = 8LL * a.D * ((long long)a.rows * a.H + (long long)a.rows2 * a.H2);
+        if (vec4 && (pick == 11 || (pick == 0 && ((long long)a.H * 4 >= 65536 || bytes >= (64LL << 20)))))
             launch_natural<MODE, Q, 4, 16, 256, 8>(a, st);
         else if (vec4 && pick == 13)
             launch_natural<MODE, Q, 4, 8, 256, 8>(a, st);
@@ -782,10 +791,10 @@ int run(const char *who, ActArgs a, int q, int layout, void *stream) {
 int faith::concretize_pair(const float *lb, const float *ub, const float *lw, const float *uw, float *l, float *u,
                            int rows, const float *lb2, const float *ub2, const float *lw2, const float *uw2,
                            float *l2, float *u2, int rows2, int dim_in, int dim_out, int dim_out2, float eps, int q,
-                           int words, void *stream) {
+                           int words, void *stream, int layout) {
     ActArgs a{lb, ub, lw, uw, nullptr, nullptr, nullptr, nullptr, l, u, rows, dim_in, dim_out, words, eps};
     a.lb2 = lb2; a.ub2 = ub2; a.lw2 = lw2; a.uw2 = uw2; a.l2 = l2; a.u2 = u2; a.rows2 = rows2; a.H2 = dim_out2;
-    return run<CONCRETIZE>("faith_concretize", a, q, FAITH_LAYOUT_NATURAL, stream);
+    return run<CONCRETIZE>("faith_concretize", a, q, layout, stream);
 }
 
 extern "C" int faith_concretize(const float *lb, const float *ub, const float *lw, const float *uw, float *l,

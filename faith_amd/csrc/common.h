@@ -15,10 +15,13 @@ void set_error(const char *fmt, ...);
 // Returns FAITH_OK or records the HIP error text and returns FAITH_ERR_LAUNCH.
 int check_launch(const char *what);
 
-// One-launch concretization of two bound objects of one dim_in (defined with the relaxation kernels).
+// One-launch concretization of two bound objects of one dim_in (defined with the relaxation kernels); rows2 == 0:
+// of one.  `u` may be NULL (the upper interval of the first object is not wanted): its upper coefficients are
+// then not read in the natural layout.
 int concretize_pair(const float *lb, const float *ub, const float *lw, const float *uw, float *l, float *u, int rows,
                     const float *lb2, const float *ub2, const float *lw2, const float *uw2, float *l2, float *u2,
-                    int rows2, int dim_in, int dim_out, int dim_out2, float eps, int q, int words, void *stream);
+                    int rows2, int dim_in, int dim_out, int dim_out2, float eps, int q, int words, void *stream,
+                    int layout = FAITH_LAYOUT_NATURAL);
 
 // The `q` argument of the entry points: FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF, or the IEEE-754 bits of any
 // other dual exponent in (1, inf) (written to *qv).  False if it is neither.

@@ -787,7 +787,7 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
               const float *y_lb, const float *y_ub, const float *x_lw, const float *x_uw, const float *y_lw,
               const float *y_uw, float *z_lb, float *z_ub, float *z_lw, float *z_uw, int B, int Lx, int Ly, int d, int D,
               float epsilon, int q, int words, int side_by_side, int heads, void *stream) {
-    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(y_u);      // x_u may be NULL: not wanted
     FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
     FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
     FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
@@ -1039,7 +1039,7 @@ int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, fl
                          const float *x_ub, const float *y_lb, const float *y_ub, const float *x_lw, const float *x_uw,
                          const float *y_lw, const float *y_uw, float *z_lb, float *z_ub, float *z_lw, float *z_uw, int B,
                          int Lx, int Ly, int K, int D, float epsilon, int q, int words, void *stream) {
-    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(x_u); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(y_u);      // x_u may be NULL: not wanted
     FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
     FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
     FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
@@ -1057,7 +1057,8 @@ int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, fl
     const bool empty_blocks = D == 1 && words > 1;      // Bounds.py:319-326 with dim_in // words == 0: the constant terms
     const float eps = empty_blocks ? 0.f : epsilon;
     const int w = empty_blocks ? 1 : words;
-    int rc = faith_concretize(x_lb, x_ub, x_lw, x_uw, x_l, x_u, B * Lx, D, K, eps, q, w, FAITH_LAYOUT_TRANSPOSED, stream);
+    int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, B * Lx, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                    nullptr, 0, D, K, 0, eps, q, w, stream, FAITH_LAYOUT_TRANSPOSED);
     if (rc != FAITH_OK) return rc;
     rc = faith_concretize(y_lb, y_ub, y_lw, y_uw, y_l, y_u, B * Ly, D, K, eps, q, w, FAITH_LAYOUT_TRANSPOSED, stream);
     if (rc != FAITH_OK) return rc;
@@ -1176,17 +1177,18 @@ extern "C" int faith_dot_product_verification_QK_static(const float *x_lb, const
     FAITH_REQUIRE(batch_size > 0 && length_x > 0 && length_y > 0 && dim_out > 0 && dim_in > 0, FAITH_ERR_SHAPE,
                   "%s: batch=%d length_x=%d length_y=%d dim_out=%d dim_in=%d must be positive", who, batch_size, length_x,
                   length_y, dim_out, dim_in);
-    // four segments (x_l, x_u, y_l, y_u), each rounded up to 64 floats so that every one starts 256-byte aligned
+    // three segments (x_l, y_l, y_u: the upper interval of x is not asked for), each rounded up to 64 floats so
+    // that every one starts 256-byte aligned
     auto seg = [](long long n) { return (n + 63) / 64 * 64; };
     const long long nx = seg((long long)batch_size * length_x * dim_out), ny = seg((long long)batch_size * length_y * dim_out);
-    FAITH_REQUIRE(2 * nx + 2 * ny <= (long long)STATIC_SCRATCH_FLOATS, FAITH_ERR_UNSUPPORTED,
-                  "%s: the concrete intervals need %lld floats of scratch (2 * batch * (length_x + length_y) * dim_out, "
+    FAITH_REQUIRE(nx + 2 * ny <= (long long)STATIC_SCRATCH_FLOATS, FAITH_ERR_UNSUPPORTED,
+                  "%s: the concrete intervals need %lld floats of scratch (batch * (length_x + 2 * length_y) * dim_out, "
                   "segments rounded to 64), the static array holds %lld; use faith_dot_product_verification_QK with "
-                  "caller-owned scratch for this size", who, 2 * nx + 2 * ny, (long long)STATIC_SCRATCH_FLOATS);
+                  "caller-owned scratch for this size", who, nx + 2 * ny, (long long)STATIC_SCRATCH_FLOATS);
     float *base = nullptr;
     const int rc = scratch_address(who, &base);
     if (rc != FAITH_OK) return rc;
-    float *x_l = base, *x_u = base + nx, *y_l = base + 2 * nx, *y_u = base + 2 * nx + ny;
+    float *x_l = base, *x_u = nullptr, *y_l = base + nx, *y_u = base + nx + ny;
     if (layout == FAITH_LAYOUT_TRANSPOSED)
         return dot_entry_transposed(who, x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw, z_lb, z_ub, z_lw,
                                     z_uw, batch_size, length_x, length_y, dim_out, dim_in, epsilon, q, words, stream);

@@ -540,7 +540,7 @@ def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    x_l = _empty_like(xlb); x_u = _empty_like(xlb) if return_intervals else None     # nothing reads x_u
     y_l = _empty_like(ylb); y_u = _empty_like(ylb)
     if out is None:
         zlw = _empty(B, Lx, D, Ly, device=dev)
@@ -577,7 +577,7 @@ def dot_product_v(x, y, p, eps, words=1, return_intervals=False, out=None):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    x_l = _empty_like(xlb); x_u = _empty_like(xlb) if return_intervals else None     # nothing reads x_u
     y_l = _empty_like(ylb); y_u = _empty_like(ylb)
     if out is None:
         zlw = _empty(B, Lx, D, dv, device=dev)
@@ -616,7 +616,7 @@ def attention_scores(x, y, heads, p, eps, words=1):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    x_l = _empty_like(xlb); x_u = None                                               # nothing reads x_u
     y_l = _empty_like(ylb); y_u = _empty_like(ylb)
     zlw = _empty(B * heads, Lx, D, Ly, device=dev)
     zuw = _empty_like(zlw)
@@ -650,7 +650,7 @@ def attention_context(x, y, p, eps, words=1):
                     ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape)):
         _check(n, t, s)
     dev = xlw.device
-    x_l = _empty_like(xlb); x_u = _empty_like(xlb)
+    x_l = _empty_like(xlb); x_u = None                                               # nothing reads x_u
     y_l = _empty_like(ylb); y_u = _empty_like(ylb)
     zlw = _empty(B, Lx, D, H, device=dev)
     zuw = _empty_like(zlw)

@@ -292,6 +292,10 @@ int faith_matmul_group_verification(const float *x_lb, const float *x_ub,
  *   x_lb, x_ub [batch, length_x, dim_out];  y_lb, y_ub [batch, length_y, dim_out]
  *   x_l, x_u   [batch, length_x, dim_out]  (out: concrete interval of x; caller's scratch)
  *   y_l, y_u   [batch, length_y, dim_out]  (out: concrete interval of y)
+ * x_u may be NULL (here and in the three entry points below that take it): the planes take x from below on
+ * both sides (Bounds.py:761-762), so nothing reads the upper interval of x -- the reference's adapter passes
+ * it as scratch and drops it (Bounds.py:1274-1296); without it the upper coefficients of x are not read for
+ * the concretization (natural layout), a quarter of that step's traffic.
  *   z_lb, z_ub [batch, length_x, length_y]
  * The reference entry has one `length`; here x and y may differ in length.  With dim_in == 1 the
  * result is the interval product of the constant terms (Bounds.py:711-721); x_l .. y_u are written
@@ -310,11 +314,12 @@ int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float 
 /*
  * faith_dot_product_verification_QK for callers that cannot allocate (code under HIP graph capture,
  * tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments
- * and results, minus the four scratch arrays x_l, x_u, y_l, y_u: the concrete intervals live in a
- * device array inside the library, faith_static_scratch_bytes() = 4 MiB per GPU, held until the process
- * ends.  The call allocates and frees nothing.  Limit: 2 * batch * (length_x + length_y) * dim_out floats
- * (each of the four segments rounded up to 64 floats) must fit the array, else FAITH_ERR_UNSUPPORTED
- * (configuration-size attention, 4 heads x 128 x 64, needs 0.5 MiB).  Every call on a GPU shares that
+ * and results, minus the four scratch arrays x_l, x_u, y_l, y_u: the concrete intervals (x_l, y_l, y_u;
+ * the unused x_u is not computed) live in a device array inside the library, faith_static_scratch_bytes()
+ * = 4 MiB per GPU, held until the process ends.  The call allocates and frees nothing.  Limit:
+ * batch * (length_x + 2 * length_y) * dim_out floats (each of the three segments rounded up to 64 floats)
+ * must fit the array, else FAITH_ERR_UNSUPPORTED (configuration-size attention, 4 heads x 128 x 64, needs
+ * 0.4 MiB).  Every call on a GPU shares that
  * GPU's array: calls that overlap on one GPU (two streams, two threads) race.
  */
 long long faith_static_scratch_bytes(void);

@@ -353,6 +353,44 @@ def test_dot_products_in_the_reference_layout_through_the_c_abi(shape, p):
             compare_contraction(name, a, e, ref[name], mag[name], UNIT_SCALE_ALL)
 
 
+@pytest.mark.parametrize("layout", ["natural", "transposed"])
+@pytest.mark.parametrize("shape", [(2, 40, 24, 96, 32, 2), (4, 128, 128, 64, 64, 1), (1, 6, 4, 1, 10, 1)])
+def test_dot_product_without_the_upper_interval_of_x(shape, layout):
+    """x_u = NULL through the C ABI: nothing reads the upper interval of x (the planes take x from below on both
+    sides, Bounds.py:761-762; the reference's adapter drops the array, Bounds.py:1274-1296), so the entry points
+    accept its absence.  Everything else -- z and the three other intervals -- is bit for bit what the call with
+    x_u gives."""
+    import ctypes
+    from faith_amd import _lib, ops
+    B, Lx, Ly, D, d, words = shape
+    g = torch.Generator().manual_seed(41)
+    x, y = rand_bounds(g, B, Lx, D, d, sw=0.2), rand_bounds(g, B, Ly, D, d, sw=0.2)
+    P = lambda t_: None if t_ is None else ctypes.c_void_p(t_.data_ptr())
+    lay = (lambda t_: t_.cuda().contiguous()) if layout == "natural" else (lambda t_: t_.cuda().transpose(2, 3).contiguous())
+    code = _lib.LAYOUT_NATURAL if layout == "natural" else _lib.LAYOUT_TRANSPOSED
+    nan = lambda *s_: torch.full(s_, float("nan"), device="cuda")
+    operands = [x.lb.cuda().contiguous(), x.ub.cuda().contiguous(), y.lb.cuda().contiguous(), y.ub.cuda().contiguous(),
+                lay(x.lw), lay(x.uw), lay(y.lw), lay(y.uw)]
+    zshape = (B, Lx, D, Ly) if layout == "natural" else (B, Lx, Ly, D)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call(with_xu):
+        x_l, x_u, y_l, y_u = nan(B, Lx, d), (nan(B, Lx, d) if with_xu else None), nan(B, Ly, d), nan(B, Ly, d)
+        z = [nan(B, Lx, Ly), nan(B, Lx, Ly), nan(*zshape), nan(*zshape)]
+        print(f"[case] dot product {layout} {shape} x_u={'given' if with_xu else 'NULL'}", flush=True)
+        _lib.call("faith_dot_product_verification_QK", P(x_l), P(y_l), P(x_u), P(y_u), *(P(t_) for t_ in operands),
+                  *(P(t_) for t_ in z), B, Lx, Ly, d, D, 0.05, ops.q_code(2.0), words, code, stream)
+        torch.cuda.synchronize()
+        return z + [x_l, y_l, y_u], x_u
+
+    full, x_u = call(True)
+    bare, _ = call(False)
+    assert not torch.isnan(x_u).any()
+    for name, a, b in zip(("z_lb", "z_ub", "z_lw", "z_uw", "x_l", "y_l", "y_u"), full, bare):
+        assert not torch.isnan(b).any(), name
+        assert torch.equal(a, b), f"{name} differs without x_u"
+
+
 def test_reference_layout_dot_product_at_configuration_3_size_equals_the_natural_layout():
     """Full-size configuration 3 through the transposed entry: every element within the parity bar of the MFMA
     path of the natural layout (same inputs re-laid out; two fp32 summation orders of 256 terms)."""
