@@ -9,32 +9,39 @@
 // is one [Lx x Ly] tile with a reduction over d:
 //   z_lw[i,m,j] = sum_k  xlw[i,m,k] a_l+[j,k] + xuw[i,m,k] a_l-[j,k] + b+[i,k] ylw[j,m,k] + b-[i,k] yuw[j,m,k]
 //   z_uw[i,m,j] = sum_k  xuw[i,m,k] a_u+[j,k] + xlw[i,m,k] a_u-[j,k] + b+[i,k] yuw[j,m,k] + b-[i,k] ylw[j,m,k]
-// i.e. eight MFMA products per K-pair into two accumulators.  Rows (i) come from x and b, columns
-// (j) from a and y, so the accumulator tile is already laid out as z[i, m, j..]: lanes run along j
-// and every store is a 128-byte run.  Neither the [Lx, D, d, Ly] broadcast the PyTorch code
-// materialises nor the transposed add of its y-terms exists here.
+// i.e. eight products per K-pair as written.  The four y terms share their multiplier b (the planes take
+// b = l_x on both sides), and b+ + b- = b, b+ - b- = |b|, so
+//     sum_k b+ ylw + b- yuw = P + Q,     sum_k b+ yuw + b- ylw = P - Q,
+//     P = sum_k (b/2) (ylw + yuw),       Q = sum_k (|b|/2) (ylw - yuw):
+// two products where there were four -- SIX MFMA products per K-pair into four accumulators (the x terms
+// of z_lw and of z_uw, P, Q), combined when a tile is done: a quarter of the MFMA time gone.  The halving
+// is exact; ylw + yuw and ylw - yuw are rounded once each, by the thread that stages them.  Rows (i) come
+// from x and b, columns (j) from a and y, so the accumulator tile is already laid out as z[i, m, j..]:
+// lanes run along j and every store is a 128-byte run.  Neither the [Lx, D, d, Ly] broadcast the PyTorch
+// code materialises nor the transposed add of its y-terms exists here.
 //
 // Tiling: workgroup = 4 wavefronts on a 128 x 64 (i x j) tile of one (head, m); wavefront tile
-// 64 x 32 (two v_mfma_f32_32x32x2_f32 blocks along i, for each of z_lw and z_uw).  K-step 8:
-// operand tiles xlw, xuw, b+, b- [128 x 8] and a_l+, a_l-, a_u+, a_u-, ylw, yuw [64 x 8] = 28 KB,
-// double buffered, two workgroups per CU.  Rows are 8 floats with the two 16-byte halves swapped
+// 64 x 32 (two v_mfma_f32_32x32x2_f32 blocks along i, for each of the four accumulators).  K-step 8:
+// operand tiles xlw, xuw, b/2, |b|/2 [128 x 8] and a_l+, a_l-, a_u+, a_u-, ylw + yuw, ylw - yuw [64 x 8]
+// = 28 KB, double buffered, two workgroups per CU.  Rows are 8 floats with the two 16-byte halves swapped
 // on every other group of four rows, which makes both the 16-byte stores and the 16-byte fragment
 // reads bank-conflict free without padding.
 //
 // On this part every vector-ALU instruction a wavefront issues takes its slot from the MFMA pipe
 // (measured: 48 v_max / v_min per 64 MFMAs cost 5 % of the MFMA rate, more when interleaved), so
 // the K-loop is written to issue almost none:
-//   * a / b are split by sign ONCE, by the thread that stages them, not by every wavefront that
-//     reads them;
+//   * a is split by sign, b halved and the y pair summed ONCE, by the thread that stages them, not by
+//     every wavefront that reads them;
 //   * global addresses are a wave-uniform 64-bit base (scalar ALU) plus a per-thread 32-bit offset
 //     that only changes from tile to tile; the K-step advances the scalar base;
 //   * tiles are numbered in mixed radix and walked with scalar adds and carries (no division);
 //   * bounds predicates exist only on the paths for ragged tiles and a ragged last K-step.
 //
-// The reduction is short (d = 64 is eight K-steps), so a tile's 64 KB of results would otherwise
-// leave in a burst during which no MFMA issues.  Each wavefront therefore holds TWO register sets:
-// a finished tile is moved aside (32 v_mov_b64) and leaves from there, eight rows per K-step,
-// while the next tile accumulates.
+// The four accumulators fill the registers two wavefronts per SIMD leave (128 of 256), so a finished
+// tile is combined and stored in one run of 64 stores before the next one starts; the CU's other workgroup,
+// which is somewhere else in its own tile, has the MFMA pipe meanwhile.  (With eight products and two
+// accumulators a second register set let a finished tile leave piecewise under the next one's MFMAs:
+// 164 us on configuration 3, against 144 us this way.)
 //
 // The constant terms z_lb / z_ub ([Lx, Ly] per head, 1/D_in of the work, O(1) cancelling terms)
 // are summed in double by a small kernel.
@@ -50,10 +57,9 @@ constexpr int TI = 128, TJ = 64, BK = 8;
 constexpr int NTHREADS = 256;
 constexpr int XT = TI * BK, YT = TJ * BK;        // floats per operand tile
 // one stage of LDS: offsets of the ten operand tiles
-constexpr int XL = 0, XU = XT, BP = 2 * XT, BN = 3 * XT;
-constexpr int ALP = 4 * XT, ALN = ALP + YT, AUP = ALP + 2 * YT, AUN = ALP + 3 * YT, YL = ALP + 4 * YT, YU = ALP + 5 * YT;
+constexpr int XL = 0, XU = XT, BH = 2 * XT, BA = 3 * XT;
+constexpr int ALP = 4 * XT, ALN = ALP + YT, AUP = ALP + 2 * YT, AUN = ALP + 3 * YT, YS = ALP + 4 * YT, YD = ALP + 5 * YT;
 constexpr int STAGE = 4 * XT + 6 * YT;
-constexpr int PIECES = 8;                        // a finished tile leaves in 8 pieces of 4 rows x 2 blocks
 
 struct DotArgs {
     const float *xlw, *xuw, *ylw, *yuw;   // [B, Lx, D, d], [B, Ly, D, d]
@@ -112,6 +118,12 @@ __device__ __forceinline__ float pos1(float v) { return __builtin_fmaxf(v, 0.f);
 __device__ __forceinline__ float neg1(float v) { return __builtin_fminf(v, 0.f); }
 __device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
 __device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
+__device__ __forceinline__ float4 half4(float4 v) { return make_float4(0.5f * v.x, 0.5f * v.y, 0.5f * v.z, 0.5f * v.w); }
+__device__ __forceinline__ float4 half_abs4(float4 v) {
+    return make_float4(0.5f * __builtin_fabsf(v.x), 0.5f * __builtin_fabsf(v.y), 0.5f * __builtin_fabsf(v.z), 0.5f * __builtin_fabsf(v.w));
+}
+__device__ __forceinline__ float4 add4(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+__device__ __forceinline__ float4 sub4(float4 a, float4 b) { return make_float4(a.x - b.x, a.y - b.y, a.z - b.z, a.w - b.w); }
 
 // position of 16-byte half `c` (0 / 1) of row `row` inside an [rows x 8] tile
 __device__ __forceinline__ int swz(int row, int c) { return row * BK + 4 * (c ^ ((row >> 2) & 1)); }
@@ -124,8 +136,7 @@ struct Walk {
 // Persistent: the grid is sized to the machine (two workgroups per CU) and every workgroup walks
 // tiles pid, pid + grid, ...  The walk is ONE software pipeline over (tile, K-step): the global
 // loads of the next step -- the first K-step of the next tile included -- are issued before the
-// MFMAs of the current step, and the results of the previous tile are stored piecewise between
-// them, so neither the head nor the tail of a tile leaves the MFMA pipe idle.
+// MFMAs of the current step, so the head of a tile does not leave the MFMA pipe idle.
 //
 // xcd_map != 0 (needs dim_in % 8 == 0 and grid % 8 == 0): workgroups are dealt to the eight XCDs
 // round robin, so workgroup w only takes perturbation coordinates m = w (mod 8); the tiles of one
@@ -277,11 +288,11 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         float *s = sm[buf];
         *reinterpret_cast<float4 *>(s + XL + sdst) = pre[0];
         *reinterpret_cast<float4 *>(s + XU + sdst) = pre[1];
-        *reinterpret_cast<float4 *>(s + BP + sdst) = pos4(pre[2]);
-        *reinterpret_cast<float4 *>(s + BN + sdst) = neg4(pre[2]);
+        *reinterpret_cast<float4 *>(s + BH + sdst) = half4(pre[2]);
+        *reinterpret_cast<float4 *>(s + BA + sdst) = half_abs4(pre[2]);
         if (wside) {
-            *reinterpret_cast<float4 *>(s + YL + ydst) = pre[3];
-            *reinterpret_cast<float4 *>(s + YU + ydst) = pre[4];
+            *reinterpret_cast<float4 *>(s + YS + ydst) = add4(pre[3], pre[4]);
+            *reinterpret_cast<float4 *>(s + YD + ydst) = sub4(pre[3], pre[4]);
         } else {
             *reinterpret_cast<float4 *>(s + ALP + ydst) = pos4(pre[3]);
             *reinterpret_cast<float4 *>(s + ALN + ydst) = neg4(pre[3]);
@@ -303,9 +314,10 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         }
         return *reinterpret_cast<const float4 *>(s + o + fy);
     };
-    auto compute = [&](int buf, floatx16 (&cl)[2], floatx16 (&cu)[2], auto &&after_quarter) {
+    floatx16 cl[2], cu[2], cp[2], cq[2];                   // the x terms of z_lw and z_uw; P and Q of the y terms
+    auto compute = [&](int buf) {
         const float *s = sm[buf];
-        float4 xl[2], xu[2], bp[2], bn[2];
+        float4 xl[2], xu[2], bh[2], ba[2];
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
             xl[a] = *reinterpret_cast<const float4 *>(s + XL + fa[a]);
@@ -314,10 +326,10 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         const float4 alp = yfrag(s, ALP), aup = yfrag(s, AUP), aln = yfrag(s, ALN), aun = yfrag(s, AUN);
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
-            bp[a] = *reinterpret_cast<const float4 *>(s + BP + fa[a]);
-            bn[a] = *reinterpret_cast<const float4 *>(s + BN + fa[a]);
+            bh[a] = *reinterpret_cast<const float4 *>(s + BH + fa[a]);
+            ba[a] = *reinterpret_cast<const float4 *>(s + BA + fa[a]);
         }
-        const float4 yl = yfrag(s, YL), yu = yfrag(s, YU);
+        const float4 ys = yfrag(s, YS), yd = yfrag(s, YD);
 #define FAITH_DOT_STEP(c)                                   \
     _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
         cl[a] = mfma(xl[a].c, alp.c, cl[a]);                \
@@ -328,60 +340,42 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         cu[a] = mfma(xl[a].c, aun.c, cu[a]);                \
     }                                                       \
     _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a] = mfma(bp[a].c, yl.c, cl[a]);                 \
-        cu[a] = mfma(bp[a].c, yu.c, cu[a]);                 \
-    }                                                       \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a] = mfma(bn[a].c, yu.c, cl[a]);                 \
-        cu[a] = mfma(bn[a].c, yl.c, cu[a]);                 \
+        cp[a] = mfma(bh[a].c, ys.c, cp[a]);                 \
+        cq[a] = mfma(ba[a].c, yd.c, cq[a]);                 \
     }
         FAITH_DOT_STEP(x)
-        after_quarter(0);
         FAITH_DOT_STEP(y)
-        after_quarter(1);
         FAITH_DOT_STEP(z)
-        after_quarter(2);
         FAITH_DOT_STEP(w)
 #undef FAITH_DOT_STEP
     };
 
     // ---- results of a finished tile: z[t, i, m, j]; register r of block a is row
-    // a*32 + 8*(r/4) + 4*(lane/32) + r%4 of the wavefront tile, lanes run along j.
-    // Piece c holds registers 4*(c%4) .. +3 of block c/4.  A row is a uniform offset from the tile's
-    // first element, the lane's own offset never changes (the entry point checks that a tile spans
-    // less than 4 GB).
+    // a*32 + 8*(r/4) + 4*(lane/32) + r%4 of the wavefront tile, lanes run along j.  A row is a uniform offset
+    // from the tile's first element, the lane's own offset never changes (the entry point checks that a tile
+    // spans less than 4 GB).  z_lw = X_l + (P + Q), z_uw = X_u + (P - Q).  The 64 stores leave in one run: the
+    // wavefront's next MFMA waits for them to issue; the CU's other workgroup, which is somewhere else in
+    // its own tile, has the MFMA pipe meanwhile.
     const unsigned rsb = (unsigned)g.D * g.oz.pitch * 4u;        // one step in i, bytes
     const unsigned lane_off = (unsigned)(wi * 64 + 4 * fh) * rsb + (wj * 32 + fi) * 4u;
-    size_t pz = 0;                                         // finished tile: its first element
-    unsigned pbytes = 0;                                   // bytes from there to the end of z; 0 before the first
-                                                           // tile has finished: the hardware drops those stores
-    int prows = 0;                                         // !EXACT: rows this lane may store (0: none)
-    // rows r0 .. r1-1 of piece c
-    auto store_piece = [&](int c, const floatx16 (&pl)[2], const floatx16 (&pu)[2], int r0 = 0, int r1 = 4) {
-        const int a = c / 4, q4 = c % 4;
-        const __amdgpu_buffer_rsrc_t rl = window(g.zlw + pz, pbytes), ru = window(g.zuw + pz, pbytes);
+    auto store_tile = [&]() {
+        const unsigned zbytes = clamp32((tot_z - zc) * 4);
+        const __amdgpu_buffer_rsrc_t rl = window(g.zlw + zc, zbytes), ru = window(g.zuw + zc, zbytes);
+        // !EXACT: rows this lane may store (0: none)
+        const int rows = zc_j0 + wj * 32 + fi < g.Ly ? g.Lx - (zc_i0 + wi * 64 + 4 * fh) : 0;
         unsigned step_b = rsb;
         asm volatile("" : "+s"(step_b));                   // keeps 32 row offsets from being hoisted and held
-        if (EXACT) {
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-                if (rr < r0 || rr >= r1) continue;
-                const unsigned row = (a * 32 + 8 * q4 + rr) * step_b;
-                st1_nt(pl[a][4 * q4 + rr], rl, lane_off, row);
-                st1_nt(pu[a][4 * q4 + rr], ru, lane_off, row);
-            }
-        } else {
-            int rows = prows;
-            asm volatile("" : "+v"(rows));                 // likewise 32 row predicates
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-                if (rr >= r0 && rr < r1 && a * 32 + 8 * q4 + rr < rows) {
-                    const unsigned row = (a * 32 + 8 * q4 + rr) * step_b;
-                    st1_nt(pl[a][4 * q4 + rr], rl, lane_off, row);
-                    st1_nt(pu[a][4 * q4 + rr], ru, lane_off, row);
+            for (int r = 0; r < 16; ++r) {
+                const int row_in_tile = a * 32 + 8 * (r / 4) + r % 4;
+                if (EXACT || row_in_tile < rows) {
+                    const float p = cp[a][r], q = cq[a][r];
+                    st1_nt(cl[a][r] + (p + q), rl, lane_off, row_in_tile * step_b);
+                    st1_nt(cu[a][r] + (p - q), ru, lane_off, row_in_tile * step_b);
                 }
             }
-        }
     };
 
     point_at(cur);
@@ -391,23 +385,13 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
     __syncthreads();
     int buf = 0;
 
-    // One K-step that is not the last of its tile: fetch the next step, multiply this one, let one piece
-    // of the previous tile go (`piece` is a constant after unrolling; with_piece = false: none),
-    // stage the fetched step.  Straight-line when EXACT, so that loads, stores and scalar work can sit
-    // between the MFMAs; the staging must stay behind them (it waits for the fetch).
-    floatx16 cl[2], cu[2], ol[2], ou[2];                   // accumulating tile; finished tile on its way out
-    auto inner_step = [&](int kt, bool with_piece, int piece) {
+    // One K-step that is not the last of its tile: fetch the next step, multiply this one, stage the fetched
+    // step.  Straight-line when EXACT, so that loads and scalar work can sit between the MFMAs; the staging must
+    // stay behind them (it waits for the fetch).
+    auto inner_step = [&](int kt) {
         load_step(kt + 1);
         __builtin_amdgcn_sched_barrier(0);                 // the fetch goes first
-        compute(buf, cl, cu, [&](int quarter) {
-            // the piece leaves in two halves, after the second and the third quarter of the MFMAs
-            // (behind the last MFMA it costs 2 % more); the fences also keep the compiler from moving
-            // the staging below up into the MFMAs, where it would wait for the fetch
-            __builtin_amdgcn_sched_barrier(0);
-            if (with_piece && quarter == 1) store_piece(piece, ol, ou, 0, 2);
-            if (with_piece && quarter == 2) store_piece(piece, ol, ou, 2, 4);
-            __builtin_amdgcn_sched_barrier(0);
-        });
+        compute(buf);
         __builtin_amdgcn_sched_barrier(0);
         lstore(buf ^ 1, kt + 1);
         __syncthreads();
@@ -418,19 +402,9 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) cl[a][r] = cu[a][r] = 0.f;
+            for (int r = 0; r < 16; ++r) cl[a][r] = cu[a][r] = cp[a][r] = cq[a][r] = 0.f;
         const bool has_next = tiles_left > 1;
-        const int inner = nk - 1;
-        // pieces 0 .. 6 leave during the first seven K-steps when the tile has that many before its
-        // last one (d >= 64); shorter reductions are dominated by their stores anyway
-        const bool trickle = inner >= PIECES - 1;
-        int kt = 0;
-        if (trickle) {
-#pragma unroll
-            for (int c = 0; c < PIECES - 1; ++c) inner_step(c, true, c);
-            kt = PIECES - 1;
-        }
-        for (; kt < inner; ++kt) inner_step(kt, false, 0);
+        for (int kt = 0; kt < nk - 1; ++kt) inner_step(kt);
         // last K-step: the fetch is the first step of the next tile
         if (has_next) {
             cur = advance(cur);
@@ -438,30 +412,14 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
             load_step(0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        compute(buf, cl, cu, [](int) {});
-        if (trickle) {
-            store_piece(PIECES - 1, ol, ou);
-        } else {
-#pragma unroll
-            for (int c = 0; c < PIECES; ++c) store_piece(c, ol, ou);
-        }
+        compute(buf);
         __builtin_amdgcn_sched_barrier(0);
-        // this tile becomes the one that leaves
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-            ol[a] = cl[a];
-            ou[a] = cu[a];
-        }
-        pz = zc;
-        pbytes = clamp32((tot_z - zc) * 4);
-        prows = zc_j0 + wj * 32 + fi < g.Ly ? g.Lx - (zc_i0 + wi * 64 + 4 * fh) : 0;
+        store_tile();
         zc = zn;  zc_i0 = zn_i0;  zc_j0 = zn_j0;
         if (has_next) lstore(buf ^ 1, 0);
         __syncthreads();
         buf ^= 1;
     }
-#pragma unroll
-    for (int c = 0; c < PIECES; ++c) store_piece(c, ol, ou);
 }
 
 // Constant terms (Bounds.py:761-762 gamma, :804-807, :815-818): a workgroup owns an 8 x 8 tile of
