@@ -115,16 +115,30 @@ def quad(d):
 # ------------------------------------------------------------------------------------------
 # per-configuration measurements
 # ------------------------------------------------------------------------------------------
-def op_entry(name, kind, times_ms, work, cpu=None, extra=None):
-    """kind 'hbm': work in bytes -> GB/s; kind 'mfma': work in flop -> TFLOP/s."""
+# Products the kernels multiply out of those the reference's formulas write.  The sign-split pair
+# C_l = A_l W+ + A_u W-, C_u = A_u W+ + A_l W- is computed as centre -+ radius (two products, not four); of the
+# dot product's eight products per term the four y terms, which share their multiplier, become two.  The roofline
+# fraction counts the products that are multiplied (what the MFMA pipe does); the rate in the reference's own
+# formulation is reported beside it for comparison with numbers quoted that way.
+EXECUTED = {"linear": 2 / 4, "conv": 2 / 4, "dot": 6 / 8, "dot_transposed": 1.0}
+
+
+def op_entry(name, kind, times_ms, work, cpu=None, extra=None, form=None):
+    """kind 'hbm': work in bytes -> GB/s; kind 'mfma': work in flop of the reference's formulation -> TFLOP/s of
+    the products that are executed (form: a key of EXECUTED)."""
     med = statistics.median(times_ms)
+    reference_work = work
     if kind == "hbm":
         ach, peak, unit = work / med / 1e6, HBM_PEAK_GBS, "GB/s"
     else:
+        work = int(work * EXECUTED[form])
         ach, peak, unit = work / med / 1e9, MFMA_FP32_PEAK_TFLOPS, "TFLOP/s"
     e = {"op": name, "latency_us": round(med * 1e3, 2), "latency_min_us": round(min(times_ms) * 1e3, 2),
          "bound": kind, "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
          "work": work}
+    if kind == "mfma" and EXECUTED[form] != 1.0:
+        e["reference_formulation"] = {"flop": reference_work, "tflops": round(reference_work / med / 1e9, 2),
+                                      "products_executed_of_written": EXECUTED[form]}
     if cpu is not None:
         e["cpu_baseline"] = cpu
     if extra:
@@ -170,7 +184,7 @@ def bench_config0(args, ops, O, wl):
         xo = O.LinearBounds(*quad(c["x"]))
         s_ = cpu_time_s(lambda: O.concretize(O.linear(xo, c["W"], c["bias"]), c["p"], c["eps"]), reps=20, warmup=3)
         cpu = {"latency_us": round(s_ * 1e6, 1), "value": round(flop / s_ / 1e12, 4), "unit": "TFLOP/s"}
-    return op_entry("config0 linear+concretize(p=inf) [1,16,64,64]x[64,64]", "mfma", t, flop, cpu,
+    return op_entry("config0 linear+concretize(p=inf) [1,16,64,64]x[64,64]", "mfma", t, flop, cpu, form="linear", extra=
                     {"note": "34 MFLOP: launch-latency bound (layer and dual norm in one launch), latency is the figure of merit; "
                              "latency_us is one call through the Python wrapper into caller-owned results",
                      "kernel_us_back_to_back_from_a_graph": kernel_us,
@@ -212,7 +226,7 @@ def bench_notebook_shapes(args, ops, O):
         s = cpu_time_s(lambda: O.linear(xo, Wc, None), reps=10, warmup=2)
         cpu = {"latency_us": round(s * 1e6, 1)}
     out.append(op_entry("extra: reference notebook shape, matmul [1,128,64,64]x[64,64]", "mfma", t,
-                        4 * 2 * (128 * 64 + 128) * 64 * 64, cpu))
+                        4 * 2 * (128 * 64 + 128) * 64 * 64, cpu, form="linear"))
     return out
 
 
@@ -419,14 +433,14 @@ def bench_config2(args, ops, O, wl):
         s = cpu_time_s(lambda: O.linear(xs, c["W"], c["bias"]), reps=3, warmup=1)
         cpu = {"value": round(flop / 8 / s / 1e12, 4), "unit": "TFLOP/s", "sample": "L=32 of 256 rows, median of 3",
                "sec_full_size_est": round(s * 8, 2)}
-    e = op_entry("config2 linear [1,256,512,1024]x[1024,1024]", "mfma", t, flop, cpu)
+    e = op_entry("config2 linear [1,256,512,1024]x[1024,1024]", "mfma", t, flop, cpu, form="linear")
     e2 = op_entry("config2 concretize(p=2) of the result", "hbm", tc, 8 * L * D * N + 16 * L * N)
     # layer and dual norm through one entry point: the tiled kernel folds the column norms into its epilogue and
     # writes l, u itself, the result is not read again
     lu = (torch.empty(1, L, N, device="cuda"), torch.empty(1, L, N, device="cuda"))
     tf = gpu_times_ms(lambda: ops.linear_concretize(*quad(x), W, b, c["p"], c["eps"], 1, out=(*out, *lu)), n, 2)
     e3 = op_entry("config2 linear + concretize(p=2) in one call (column norms in the GEMM epilogue)", "mfma", tf, flop,
-                  None, {"separately_us": round((statistics.median(t) + statistics.median(tc)) * 1e3, 1)})
+                  None, form="linear", extra={"separately_us": round((statistics.median(t) + statistics.median(tc)) * 1e3, 1)})
     return [e, e2, e3]
 
 
@@ -446,7 +460,7 @@ def bench_config3(args, ops, O, wl):
         cpu = {"value": round(flop / s / 1e12, 4), "unit": "TFLOP/s", "sample": "full size, median of 3",
                "latency_ms": round(s * 1e3, 1)}
     e = op_entry("config3 dot_product QK 4 heads [4,128,256,64] (concretize + planes + contraction)",
-                 "mfma", t, flop, cpu)
+                 "mfma", t, flop, cpu, form="dot")
     # the second half of attention on the same shapes (not one of the five configurations): context =
     # probabilities [4,128,256,128] . values [4,128,256,64]; the scores bounds just computed serve as
     # the probability operand
@@ -455,7 +469,7 @@ def bench_config3(args, ops, O, wl):
             torch.empty(B, L, D, d, device="cuda"), torch.empty(B, L, d, device="cuda"))
     flopv = B * (8 * 2 * L * D * L * d + 8 * 2 * L * L * d)
     tv = gpu_times_ms(lambda: ops.dot_product_v(probs, quad(y), c["p"], c["eps"], 1, out=outv), 50, 5)
-    ev = op_entry("extra: context (probs.value) 4 heads [4,128,256,128].[4,128,256,64]", "mfma", tv, flopv)
+    ev = op_entry("extra: context (probs.value) 4 heads [4,128,256,128].[4,128,256,64]", "mfma", tv, flopv, form="dot")
     # the same scores through the reference's own calling convention: operands [B, L, dim_out, dim_in], result
     # [B, Lx, Ly, dim_in] (vector ALU with lanes along dim_in, no re-layout); the roofline is still the MFMA peak
     from faith_amd import c_bound
@@ -469,7 +483,7 @@ def bench_config3(args, ops, O, wl):
                                                                     yt[0], yt[1], *zt, B, L, d, D, c["eps"]), 50, 5)
     c_bound.p = 2.0
     et = op_entry("extra: config3 scores in the reference's transposed layout (c_bound.c_dot_product_verification_QK)",
-                  "mfma", tt, flop)
+                  "mfma", tt, flop, form="dot_transposed")
     return [e, ev, et]
 
 
@@ -490,7 +504,7 @@ def bench_config4(args, ops, O, wl):
         s = cpu_time_s(lambda: O.conv2d(xs, c["W"], c["bias"], 1, 1), reps=3, warmup=1)
         cpu = {"value": round(4 * 2 * 33 * Co * Hh * Hh * Ci * 9 / s / 1e12, 4), "unit": "TFLOP/s",
                "sample": "D_in=32 of 256, median of 3"}
-    e = op_entry("config4 conv3x3 64->128 [1,256,64,32,32]", "mfma", t, flop, cpu)
+    e = op_entry("config4 conv3x3 64->128 [1,256,64,32,32]", "mfma", t, flop, cpu, form="conv")
     e2 = op_entry("config4 concretize(p=inf) of the result", "hbm", tc, 8 * D * Co * Hh * Hh + 16 * Co * Hh * Hh)
     out_entries = [e, e2]
     # the other layer shapes of a CNN verifier, same D_in = 256 and 32 x 32 input (not among the five configurations):
@@ -508,7 +522,7 @@ def bench_config4(args, ops, O, wl):
         o_ = ops.conv2d(lw, lb, uw, ub, Wk, None, s_, p_)
         tk = gpu_times_ms(lambda: ops.conv2d(lw, lb, uw, ub, Wk, None, s_, p_, out=o_), 10 if args.profile else 50, 2)
         fl = 4 * 2 * (D + 1) * co * ho * ho * ci * k * k
-        out_entries.append(op_entry(f"extra: conv {what} [1,256,{ci},32,32]", "mfma", tk, fl, None,
+        out_entries.append(op_entry(f"extra: conv {what} [1,256,{ci},32,32]", "mfma", tk, fl, None, form="conv", extra=
                                     {"result_write_GBs": round(2 * D * co * ho * ho * 4 / statistics.median(tk) / 1e6, 1)}))
         del lw, uw, o_
     return out_entries
@@ -675,8 +689,11 @@ def main():
 
     for e in entries:
         cb = e.get("cpu_baseline")
+        rf = e.get("reference_formulation")
         log(f"{e['op']:<90s} {e['latency_us']:>10.1f} us  {e['achieved']:>9.1f} {e['unit']:<8s} "
-            f"{100 * e['frac']:5.1f}% of {e['peak']:g}" + (f"   cpu: {cb}" if cb else ""))
+            f"{100 * e['frac']:5.1f}% of {e['peak']:g}"
+            + (f"   ({rf['tflops']:.1f} TFLOP/s in the reference's formulation)" if rf else "")
+            + (f"   cpu: {cb}" if cb else ""))
 
     line = {
         "metric": METRIC, "value": head["value"], "unit": "GB/s", "n_gpus": 1,

@@ -31,11 +31,9 @@ EXTRA = {
     "mul.hip": ["-ffp-contract=off"],
     "affine.hip": ["-ffp-contract=off"],
     "softmax.hip": ["-ffp-contract=off"],
-    # the contraction kernels split weights and intervals by sign with fmaxf / fminf: one instruction each
-    # only when the compiler need not quiet signalling NaNs first
-    "gemm.hip": ["-fno-honor-nans"],
+    # the dot product splits the intervals by sign with fmaxf / fminf: one instruction each only when the
+    # compiler need not quiet signalling NaNs first
     "dot.hip": ["-fno-honor-nans"],
-    "conv.hip": ["-fno-honor-nans"],
 }
 
 

@@ -9,15 +9,20 @@
 // the last K-tile, ignores the tile origin in its padding test and never stores; the arithmetic
 // above is what it sets out to compute.)
 //
+// Computed in centre / radius form (W+ + W- = W, W+ - W- = |W|):
+//     y_l = M - R,   y_u = M + R,   M = conv((x_l + x_u) / 2, W),   R = conv((x_u - x_l) / 2, |W|)
+// -- two products per tap where the formula above has four.  Centre and radius of an input pair are formed
+// once, by the thread that stages the patch (an out-of-image position is 0 in both); |W| by the wavefront that
+// reads the weight.
+//
 // Implicit GEMM:  C[co, p] = sum_k W[co, k] * X[k, p],  k = (ci, kh, kw),  p = output pixel.
-// MFMA rows are output channels (W is the sign-split operand), MFMA columns are pixels (x_l / x_u
-// is the paired operand), so lanes run along ow and every store is a contiguous run of a
+// MFMA rows are output channels (W and |W|), MFMA columns are pixels (centre and radius of x), so lanes run along ow and every store is a contiguous run of a
 // channel plane -- NCHW needs no transposition.
 //
 // Workgroup = 4 wavefronts on 128 channels x (4 output rows x 32 output columns) of one image;
 // wavefront tile 64 channels x 2 rows.  The reduction walks C_in in chunks of 4 channels.  Per
 // chunk the LDS holds
-//   * the input patch of both bounds: [2][4][(4-1)*stride + K][(32-1)*stride + K], out-of-image
+//   * the input patch, centres and radii: [2][4][(4-1)*stride + K][(32-1)*stride + K], out-of-image
 //     positions stored as exact zeros (so padding contributes +0 to both products), each input
 //     element fetched from global memory once and reused by up to K*K taps;
 //   * the weight slab [128][4*K*K] (row padded to an odd length: conflict-free column reads).
@@ -106,8 +111,9 @@ conv_signsplit(const ConvArgs g) {
             for (int pc = lane; pc < pcol; pc += 64) {
                 const int iw = iw0 + pc;
                 const bool ok = row_ok && iw >= 0 && iw < g.W;
-                sXl[rr * pcol + pc] = ok ? xl_n[rbase + iw] : 0.f;
-                sXu[rr * pcol + pc] = ok ? xu_n[rbase + iw] : 0.f;
+                const float vl = ok ? xl_n[rbase + iw] : 0.f, vu = ok ? xu_n[rbase + iw] : 0.f;
+                sXl[rr * pcol + pc] = 0.5f * (vl + vu);      // centre
+                sXu[rr * pcol + pc] = 0.5f * (vu - vl);      // radius
             }
         }
         // ---- stage the weight slab: CC*KK contiguous floats per output channel
@@ -128,12 +134,11 @@ conv_signsplit(const ConvArgs g) {
                 for (int kw = 0; kw < g.K; ++kw, ++tap) {
                     const int xo = cp * PP + kh * pcol + kw;
                     const int wo = cp * KK + tap;
-                    float wp[2], wq[2], xl[2], xu[2];
+                    float wp[2], wq[2], xl[2], xu[2];        // w, |w|; centre and radius of x
 #pragma unroll
                     for (int a = 0; a < 2; ++a) {
-                        const float w = sW[woff[a] + wo];
-                        wp[a] = fmaxf(w, 0.f);
-                        wq[a] = fminf(w, 0.f);
+                        wp[a] = sW[woff[a] + wo];
+                        wq[a] = __builtin_fabsf(wp[a]);
                     }
 #pragma unroll
                     for (int b = 0; b < 2; ++b) {
@@ -145,14 +150,7 @@ conv_signsplit(const ConvArgs g) {
 #pragma unroll
                         for (int b = 0; b < 2; ++b) {
                             cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
-                            cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
-                        }
-#pragma unroll
-                    for (int a = 0; a < 2; ++a)
-#pragma unroll
-                        for (int b = 0; b < 2; ++b) {
-                            cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
-                            cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                            cu[a][b] = mfma(wq[a], xu[b], cu[a][b]);
                         }
                 }
             }
@@ -174,8 +172,8 @@ conv_signsplit(const ConvArgs g) {
                 const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (co < g.Co) {
                     const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
-                    __builtin_nontemporal_store(cl[a][b][r], &g.yl[o]);
-                    __builtin_nontemporal_store(cu[a][b][r], &g.yu[o]);
+                    __builtin_nontemporal_store(cl[a][b][r] - cu[a][b][r], &g.yl[o]);      // centre - radius
+                    __builtin_nontemporal_store(cl[a][b][r] + cu[a][b][r], &g.yu[o]);
                 }
             }
         }
@@ -196,13 +194,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void *base, size_
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0,
                                              (int)((bytes >> 32) ? 0xffffffffu : (unsigned)bytes), 0x00020000);
 }
-// max(v, 0) / min(v, 0), one instruction each: this file is compiled with -fno-honor-nans, without which fmaxf /
-// fminf (and a median of three) come with a canonicalising v_max per value.  Plain builtins: the compiler sees the
-// write, so an MFMA or an LDS store that consumes the result gets the wait states it needs.  (A NaN weight or
-// interval, which the reference would carry through, is not preserved by the split.)
-__device__ __forceinline__ float pos1(float v) { return __builtin_fmaxf(v, 0.f); }
-__device__ __forceinline__ float neg1(float v) { return __builtin_fminf(v, 0.f); }
-
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 conv_signsplit_k3s1(const ConvArgs g) {
     constexpr int K = 3, KK = 9, PROW = TR - 1 + K, PCOL = TC - 1 + K, PP = PROW * PCOL;   // 6, 34, 204
@@ -278,8 +269,8 @@ conv_signsplit_k3s1(const ConvArgs g) {
         for (int u = 0; u < NP; ++u) {
             const int e = tid + u * NTHREADS;
             if (e < CC * PP) {
-                sXl[buf][e] = pxl[u];
-                sXu[buf][e] = pxu[u];
+                sXl[buf][e] = 0.5f * (pxl[u] + pxu[u]);      // centre
+                sXu[buf][e] = 0.5f * (pxu[u] - pxl[u]);      // radius
             }
         }
 #pragma unroll
@@ -313,12 +304,11 @@ conv_signsplit_k3s1(const ConvArgs g) {
         for (int tap = 0; tap < KK; ++tap) {
             const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
             const int wo = cp * KK + tap;
-            float wp[2], wq[2], xl[2], xu[2];
+            float wp[2], wq[2], xl[2], xu[2];                // w, |w|; centre and radius of x
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
-                const float w = sW[buf][woff[a] + wo];
-                wp[a] = pos1(w);
-                wq[a] = neg1(w);
+                wp[a] = sW[buf][woff[a] + wo];
+                wq[a] = __builtin_fabsf(wp[a]);
             }
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
@@ -330,14 +320,7 @@ conv_signsplit_k3s1(const ConvArgs g) {
 #pragma unroll
                 for (int b = 0; b < 2; ++b) {
                     cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
-                    cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
-                }
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int b = 0; b < 2; ++b) {
-                    cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
-                    cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                    cu[a][b] = mfma(wq[a], xu[b], cu[a][b]);
                 }
         }
     };
@@ -384,8 +367,9 @@ conv_signsplit_k3s1(const ConvArgs g) {
             for (int r = 0; r < 16; ++r) {
                 const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
                                     (unsigned)(oh * g.Wo) * 4u;
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cu[a][b][r]), wyu, vo, so, 2);
+                // y_l = centre - radius, y_u = centre + radius
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] - cu[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] + cu[a][b][r]), wyu, vo, so, 2);
             }
         }
     }
@@ -518,8 +502,8 @@ conv_signsplit_fast(const ConvArgs g) {
         for (int u = 0; u < NP; ++u) {
             const int e = tid + u * NTHREADS;
             if (e < CCH * PP) {
-                dl[e] = pxl[u];
-                du[e] = pxu[u];
+                dl[e] = 0.5f * (pxl[u] + pxu[u]);            // centre
+                du[e] = 0.5f * (pxu[u] - pxl[u]);            // radius
             }
         }
     };
@@ -563,12 +547,11 @@ conv_signsplit_fast(const ConvArgs g) {
             for (int tap = 0; tap < KK; ++tap) {
                 const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
                 const int wo = cp * KK + tap;
-                float wp[2], wq[2], xl[2], xu[2];
+                float wp[2], wq[2], xl[2], xu[2];            // w, |w|; centre and radius of x
 #pragma unroll
                 for (int a = 0; a < 2; ++a) {
-                    const float w = bw[woff[a] + wo];
-                    wp[a] = pos1(w);
-                    wq[a] = neg1(w);
+                    wp[a] = bw[woff[a] + wo];
+                    wq[a] = __builtin_fabsf(wp[a]);
                 }
 #pragma unroll
                 for (int b = 0; b < 2; ++b) {
@@ -580,14 +563,7 @@ conv_signsplit_fast(const ConvArgs g) {
 #pragma unroll
                     for (int b = 0; b < 2; ++b) {
                         cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
-                        cu[a][b] = mfma(wp[a], xu[b], cu[a][b]);
-                    }
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int b = 0; b < 2; ++b) {
-                        cl[a][b] = mfma(wq[a], xu[b], cl[a][b]);
-                        cu[a][b] = mfma(wq[a], xl[b], cu[a][b]);
+                        cu[a][b] = mfma(wq[a], xu[b], cu[a][b]);
                     }
             }
         }
@@ -643,8 +619,9 @@ conv_signsplit_fast(const ConvArgs g) {
             for (int r = 0; r < 16; ++r) {
                 const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
                                     (unsigned)(row0 * g.Wo) * 4u;
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cu[a][b][r]), wyu, vo, so, 2);
+                // y_l = centre - radius, y_u = centre + radius
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] - cu[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] + cu[a][b][r]), wyu, vo, so, 2);
             }
         }
     }

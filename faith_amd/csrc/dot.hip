@@ -492,7 +492,7 @@ __global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
 // Short sequences (Lx, Ly <= 64, d <= 80): the 128 x 64 tile above would be mostly padding, so here
 // a WAVEFRONT owns one 32 x 32 block of z for one perturbation coordinate m (one MFMA block for
 // z_lw, one for z_uw).  The four wavefronts of a workgroup share the (head, i-block, j-block): the
-// operands that do not depend on m (b+, b-, a_l+-, a_u+-, split by sign) are staged in LDS once for
+// operands that do not depend on m (b / 2, |b| / 2, a_l+-, a_u+- split by sign) are staged in LDS once for
 // the whole reduction, and every wavefront walks its own `mpw` coordinates, loading its x and y
 // fragments straight from global memory in MFMA layout (rows of 32 bytes per lane and K-step: poor
 // coalescing, but these problems are a few megabytes and latency is what counts).
@@ -545,16 +545,16 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
             const int row = e / dp, k = e % dp;
             const float bt = k < d ? g.x_l[xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + k] : 0.f;
             const int dst = (k / 8) * (SB * 8) + swz(row, (k % 8) / 4) + k % 4;
-            s_bp[dst] = pos1(bt);
-            s_bn[dst] = neg1(bt);
+            s_bp[dst] = 0.5f * bt;                     // b / 2 and |b| / 2: see the top of the file
+            s_bn[dst] = 0.5f * __builtin_fabsf(bt);
         }
     }
     for (int e = tid; !RAGGED && e < SB * d / 4; e += 256) {
         const int row = e / (d / 4), c4 = e % (d / 4);
         const int dst = (c4 / 2) * (SB * 8) + swz(row, c4 % 2);
         const float4 bt = *reinterpret_cast<const float4 *>(g.x_l + xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + c4 * 4);
-        *reinterpret_cast<float4 *>(s_bp + dst) = pos4(bt);
-        *reinterpret_cast<float4 *>(s_bn + dst) = neg4(bt);
+        *reinterpret_cast<float4 *>(s_bp + dst) = half4(bt);         // b / 2 and |b| / 2: see the top of the file
+        *reinterpret_cast<float4 *>(s_bn + dst) = half_abs4(bt);
         if (!VP) {
             const size_t o = yb0 + (size_t)min(j0 + row, g.Ly - 1) * g.oy.pitch + c4 * 4;
             const float4 al = *reinterpret_cast<const float4 *>(g.y_l + o), au = *reinterpret_cast<const float4 *>(g.y_u + o);
@@ -596,9 +596,9 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
         const __amdgpu_buffer_rsrc_t wxu = window(g.xuw + x0, clamp32((tot_x - x0) * 4));
         const __amdgpu_buffer_rsrc_t wyl = window(g.ylw + y0, clamp32((tot_y - y0) * 4));
         const __amdgpu_buffer_rsrc_t wyu = window(g.yuw + y0, clamp32((tot_y - y0) * 4));
-        floatx16 cl, cu;
+        floatx16 cl, cu, cp, cq;                   // x terms of z_lw and z_uw; P and Q of the y terms
 #pragma unroll
-        for (int r = 0; r < 16; ++r) cl[r] = cu[r] = 0.f;
+        for (int r = 0; r < 16; ++r) cl[r] = cu[r] = cp[r] = cq[r] = 0.f;
         for (int q0 = 0; q0 < nq; q0 += 4) {
             float4 xl[4], xu[4], yl[4], yu[4];
 #pragma unroll
@@ -638,18 +638,17 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
             for (int qq = 0; qq < 4; ++qq) {
                 if (q0 + qq < nq) {
                     const int o = (q0 + qq) * (SB * 8) + frag;
-                    const float4 bp = *reinterpret_cast<const float4 *>(s_bp + o), bn = *reinterpret_cast<const float4 *>(s_bn + o);
+                    const float4 bh = *reinterpret_cast<const float4 *>(s_bp + o), ba = *reinterpret_cast<const float4 *>(s_bn + o);
                     const float4 alp = *reinterpret_cast<const float4 *>(s_alp + o), aln = *reinterpret_cast<const float4 *>(s_aln + o);
                     const float4 aup = *reinterpret_cast<const float4 *>(s_aup + o), aun = *reinterpret_cast<const float4 *>(s_aun + o);
+                    const float4 ys = add4(yl[qq], yu[qq]), yd = sub4(yl[qq], yu[qq]);
 #define FAITH_DOT_SMALL(c)                          \
     cl = mfma(xl[qq].c, alp.c, cl);                 \
     cu = mfma(xu[qq].c, aup.c, cu);                 \
+    cp = mfma(bh.c, ys.c, cp);                      \
     cl = mfma(xu[qq].c, aln.c, cl);                 \
     cu = mfma(xl[qq].c, aun.c, cu);                 \
-    cl = mfma(bp.c, yl[qq].c, cl);                  \
-    cu = mfma(bp.c, yu[qq].c, cu);                  \
-    cl = mfma(bn.c, yu[qq].c, cl);                  \
-    cu = mfma(bn.c, yl[qq].c, cu);
+    cq = mfma(ba.c, yd.c, cq);
                     FAITH_DOT_SMALL(x)
                     FAITH_DOT_SMALL(y)
                     FAITH_DOT_SMALL(z)
@@ -665,8 +664,8 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
                 const int i = i0 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (i < g.Lx) {
                     const size_t o = zw0 + ((size_t)i * g.D + m) * g.oz.pitch + j0 + fi;
-                    __builtin_nontemporal_store(cl[r], &g.zlw[o]);
-                    __builtin_nontemporal_store(cu[r], &g.zuw[o]);
+                    __builtin_nontemporal_store(cl[r] + (cp[r] + cq[r]), &g.zlw[o]);
+                    __builtin_nontemporal_store(cu[r] + (cp[r] - cq[r]), &g.zuw[o]);
                 }
             }
         }

@@ -7,6 +7,14 @@
 // A_l, A_u are the bound rows ([rows*D_in, H] for lw/uw, [rows, H] for lb/ub, both K-contiguous),
 // W is [N, H] as nn.Linear stores it, so both operands stream along K.
 //
+// Computed in centre / radius form: W+ + W- = W and W+ - W- = |W|, so
+//     C_l = M - R,   C_u = M + R,   M = ((A_l + A_u) / 2) @ W,   R = ((A_u - A_l) / 2) @ |W|
+// -- TWO products per term where the formula above has four, i.e. half the MFMA time for the same
+// four results.  The halving is exact; centre and radius of a coefficient pair are rounded once each, by
+// the thread that stages them; what that adds to the rounding of the four-product form (each bound then
+// carries the rounding of both operands' terms: measured 1.3 - 1.9 x its error against float64, 0.1 of
+// the parity bar on the configurations) is bounded by the parity tests together with the order of summation.
+//
 // The reference's CUTLASS path takes the constant-term rows as trailing M-blocks of the same grid
 // (tvm_kernels/cuda_kernel/mma/mma_kernel.h:251-259); here they go to the exact-accumulation
 // code below instead: they are 1/D_in of the work and the only outputs whose O(1) terms cancel.
@@ -14,19 +22,20 @@
 // launch of their own.
 //
 // Tiling (gfx950): workgroup = 4 wavefronts, macro-tile BM x BN = 128 x 128, K-step 16,
-// wavefront tile 64 x 64 = 2 x 2 v_mfma_f32_32x32x2_f32 blocks for EACH of C_l and C_u
-// (128 accumulator registers).  Every fragment set (A_l, A_u, W+, W-) feeds four MFMAs, so one
-// 16-byte LDS read per operand block covers four K-pairs: 8 LDS reads per 64 MFMAs.
+// wavefront tile 64 x 64 = 2 x 2 v_mfma_f32_32x32x2_f32 blocks for EACH of M and R
+// (128 accumulator registers).  One 16-byte LDS read per operand block covers four K-pairs: 8 LDS
+// reads per 32 MFMAs.
 //
 // On this part every vector-ALU instruction a wavefront issues takes its slot from the MFMA pipe,
-// so the K-loop issues almost none: W is split by sign ONCE, by the thread that stages it (W+ and
-// W- are separate LDS tiles); global addresses are buffer addresses (a wave-uniform descriptor and
+// so the K-loop issues almost none: centres, radii and |W| are formed ONCE, by the thread that stages
+// them (separate LDS tiles); global addresses are buffer addresses (a wave-uniform descriptor and
 // K offset, one per-thread offset per row that never changes), and the K-step is straight-line:
 // fetch of step t+1, half the MFMAs of step t, staging of step t+1, the other half, one barrier.
 //
 // LDS: a K-step of an operand is two [128 x 8] halves; rows are 8 floats with the two 16-byte
 // pieces swapped on every other group of four rows, which makes the 16-byte stores and the
-// 16-byte fragment reads bank-conflict free without padding.  4 operands x 8 KB x 2 stages = 64 KB,
+// 16-byte fragment reads bank-conflict free without padding.  4 operands (centre, radius, W, |W|) x 8 KB
+// x 2 stages = 64 KB,
 // two workgroups per CU.
 //
 // blockIdx -> tile mapping is XCD-aware: workgroups are dealt round-robin to the 8 XCDs, so
@@ -57,14 +66,16 @@ struct GemmArgs {
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
-// max(v, 0) / min(v, 0), one instruction each: this file is compiled with -fno-honor-nans, without which fmaxf /
-// fminf (and a median of three) come with a canonicalising v_max per value.  Plain builtins: the compiler sees the
-// write, so an MFMA or an LDS store that consumes the result gets the wait states it needs.  (A NaN weight or
-// interval, which the reference would carry through, is not preserved by the split.)
-__device__ __forceinline__ float pos1(float v) { return __builtin_fmaxf(v, 0.f); }
-__device__ __forceinline__ float neg1(float v) { return __builtin_fminf(v, 0.f); }
-__device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
-__device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
+// centre (l + u) / 2 and radius (u - l) / 2 of a pair of coefficients; |w|
+__device__ __forceinline__ float4 mid4(float4 l, float4 u) {
+    return make_float4(0.5f * (l.x + u.x), 0.5f * (l.y + u.y), 0.5f * (l.z + u.z), 0.5f * (l.w + u.w));
+}
+__device__ __forceinline__ float4 rad4(float4 l, float4 u) {
+    return make_float4(0.5f * (u.x - l.x), 0.5f * (u.y - l.y), 0.5f * (u.z - l.z), 0.5f * (u.w - l.w));
+}
+__device__ __forceinline__ float4 abs4(float4 v) {
+    return make_float4(__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w));
+}
 
 // Accesses at or beyond `bytes` from the base are dropped by the hardware (loads return zero).
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void *base, size_t bytes) {
@@ -95,7 +106,7 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
                                                     float *pl = nullptr, float *pu = nullptr, float qv = 0.f) {
     constexpr int BM = 64 * MBM, BN = 64 * MBN;
     constexpr int HALF_A = BM * 8, HALF_W = BN * 8;      // floats in one [rows x 8] half of an operand's K-step
-    constexpr int S_AL = 0, S_AU = 2 * HALF_A, S_WP = 4 * HALF_A, S_WN = 4 * HALF_A + 2 * HALF_W;
+    constexpr int S_AM = 0, S_AR = 2 * HALF_A, S_W = 4 * HALF_A, S_WA = 4 * HALF_A + 2 * HALF_W;
     constexpr int STAGE = 4 * HALF_A + 4 * HALF_W;
     float(*sm)[STAGE] = reinterpret_cast<float(*)[STAGE]>(smem);
 
@@ -149,17 +160,19 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
 #pragma unroll
         for (int i = 0; i < MBM; ++i) {
             if (past(kt)) pal[i] = pau[i] = zero;
-            *reinterpret_cast<float4 *>(s + S_AL + dsta[i]) = pal[i];
-            *reinterpret_cast<float4 *>(s + S_AU + dsta[i]) = pau[i];
+            *reinterpret_cast<float4 *>(s + S_AM + dsta[i]) = mid4(pal[i], pau[i]);
+            *reinterpret_cast<float4 *>(s + S_AR + dsta[i]) = rad4(pal[i], pau[i]);
         }
 #pragma unroll
         for (int i = 0; i < MBN; ++i) {
             if (past(kt)) pw[i] = zero;
-            *reinterpret_cast<float4 *>(s + S_WP + dstw[i]) = pos4(pw[i]);
-            *reinterpret_cast<float4 *>(s + S_WN + dstw[i]) = neg4(pw[i]);
+            *reinterpret_cast<float4 *>(s + S_W + dstw[i]) = pw[i];
+            *reinterpret_cast<float4 *>(s + S_WA + dstw[i]) = abs4(pw[i]);
         }
     };
 
+    // cl accumulates the centre term (A_l + A_u)/2 . W and cu the radius term (A_u - A_l)/2 . |W|; they become
+    // C_l and C_u when the reduction is done
     floatx16 cl[MBM][MBN], cu[MBM][MBN];
 #pragma unroll
     for (int a = 0; a < MBM; ++a)
@@ -180,25 +193,21 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
 #pragma unroll
         for (int ks = 0; ks < BK / 8; ++ks) {
             if (ks == 1) halfway();
-            float4 al[MBM], au[MBM], wp[MBN], wq[MBN];
+            float4 am[MBM], ar[MBM], wp[MBN], wq[MBN];
 #pragma unroll
             for (int t = 0; t < MBM; ++t) {
-                al[t] = *reinterpret_cast<const float4 *>(s + S_AL + ks * HALF_A + fa[t]);
-                au[t] = *reinterpret_cast<const float4 *>(s + S_AU + ks * HALF_A + fa[t]);
+                am[t] = *reinterpret_cast<const float4 *>(s + S_AM + ks * HALF_A + fa[t]);
+                ar[t] = *reinterpret_cast<const float4 *>(s + S_AR + ks * HALF_A + fa[t]);
             }
 #pragma unroll
             for (int t = 0; t < MBN; ++t) {
-                wp[t] = *reinterpret_cast<const float4 *>(s + S_WP + ks * HALF_W + fw[t]);
-                wq[t] = *reinterpret_cast<const float4 *>(s + S_WN + ks * HALF_W + fw[t]);
+                wp[t] = *reinterpret_cast<const float4 *>(s + S_W + ks * HALF_W + fw[t]);
+                wq[t] = *reinterpret_cast<const float4 *>(s + S_WA + ks * HALF_W + fw[t]);
             }
 #define FAITH_STEP(c)                                                           \
     _Pragma("unroll") for (int a = 0; a < MBM; ++a) _Pragma("unroll") for (int b = 0; b < MBN; ++b) { \
-        cl[a][b] = mfma(al[a].c, wp[b].c, cl[a][b]);                            \
-        cu[a][b] = mfma(au[a].c, wp[b].c, cu[a][b]);                            \
-    }                                                                           \
-    _Pragma("unroll") for (int a = 0; a < MBM; ++a) _Pragma("unroll") for (int b = 0; b < MBN; ++b) { \
-        cl[a][b] = mfma(au[a].c, wq[b].c, cl[a][b]);                            \
-        cu[a][b] = mfma(al[a].c, wq[b].c, cu[a][b]);                            \
+        cl[a][b] = mfma(am[a].c, wp[b].c, cl[a][b]);                            \
+        cu[a][b] = mfma(ar[a].c, wq[b].c, cu[a][b]);                            \
     }
             // 128 x 128 only: a wavefront inside its run of 64 MFMAs goes before its neighbour's staging and
             // address arithmetic (configuration 2: 1.5 % faster; the small tiles, whose runs are 16 or 32
@@ -240,6 +249,17 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
     // exist is sent outside the window.
     // The window is the tile's own rows (less than 2 GB: the entry point checks), so the offset that sends a
     // lane outside it cannot wrap around 32 bits when the row offset is added.
+    // C_l = centre - radius, C_u = centre + radius
+#pragma unroll
+    for (int a = 0; a < MBM; ++a)
+#pragma unroll
+        for (int b = 0; b < MBN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float c = cl[a][b][r], rd = cu[a][b][r];
+                cl[a][b][r] = c - rd;
+                cu[a][b][r] = c + rd;
+            }
     const size_t c_bytes = (size_t)min(M - m0, BM) * g.N * 4;
     const __amdgpu_buffer_rsrc_t wcl = window(g.Cl + (size_t)m0 * g.N, c_bytes);
     const __amdgpu_buffer_rsrc_t wcu = window(g.Cu + (size_t)m0 * g.N, c_bytes);
@@ -459,14 +479,11 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
             if (s0 + i < ns) {
-                // split by sign with ordinary float code: these values feed the MFMAs directly
-                const float4 wp = make_float4(fmaxf(w[i].x, 0.f), fmaxf(w[i].y, 0.f), fmaxf(w[i].z, 0.f), fmaxf(w[i].w, 0.f));
-                const float4 wq = make_float4(fminf(w[i].x, 0.f), fminf(w[i].y, 0.f), fminf(w[i].z, 0.f), fminf(w[i].w, 0.f));
+                // centre / radius form, with ordinary float code: these values feed the MFMAs directly
+                const float4 am = mid4(al[i], au[i]), ar = rad4(al[i], au[i]), wa = abs4(w[i]);
 #define FAITH_STEP(c)                       \
-    cl = mfma(al[i].c, wp.c, cl);           \
-    cu = mfma(au[i].c, wp.c, cu);           \
-    cl = mfma(au[i].c, wq.c, cl);           \
-    cu = mfma(al[i].c, wq.c, cu);
+    cl = mfma(am.c, w[i].c, cl);            \
+    cu = mfma(ar.c, wa.c, cu);
                 FAITH_STEP(x)
                 FAITH_STEP(y)
                 FAITH_STEP(z)
@@ -499,11 +516,12 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs
             sl += sm[((v * 2 + 0) * 16 + r) * 64 + lane];
             su += sm[((v * 2 + 1) * 16 + r) * 64 + lane];
         }
-        // register r of a 32 x 32 block is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
+        // register r of a 32 x 32 block is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32;
+        // sl is the centre term, su the radius term
         const int row = m0 + 8 * wv + 4 * fh + q;
         if (row < g.Mw && col < g.N) {
-            g.Cl[(size_t)row * g.N + col] = sl;
-            g.Cu[(size_t)row * g.N + col] = su;
+            g.Cl[(size_t)row * g.N + col] = sl - su;
+            g.Cu[(size_t)row * g.N + col] = sl + su;
         }
     }
 }
@@ -859,13 +877,10 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_concretize(const Fuse
 #pragma unroll
             for (int i = 0; i < CH; ++i) {
                 if (s0 + i < ns) {
-                    const float4 wp = make_float4(fmaxf(w[i].x, 0.f), fmaxf(w[i].y, 0.f), fmaxf(w[i].z, 0.f), fmaxf(w[i].w, 0.f));
-                    const float4 wq = make_float4(fminf(w[i].x, 0.f), fminf(w[i].y, 0.f), fminf(w[i].z, 0.f), fminf(w[i].w, 0.f));
+                    const float4 am = mid4(al[i], au[i]), ar = rad4(al[i], au[i]), wa = abs4(w[i]);
 #define FAITH_STEP(c)                       \
-    cl = mfma(al[i].c, wp.c, cl);           \
-    cu = mfma(au[i].c, wp.c, cu);           \
-    cl = mfma(au[i].c, wq.c, cl);           \
-    cu = mfma(al[i].c, wq.c, cu);
+    cl = mfma(am.c, w[i].c, cl);            \
+    cu = mfma(ar.c, wa.c, cu);
                     FAITH_STEP(x)
                     FAITH_STEP(y)
                     FAITH_STEP(z)
@@ -884,6 +899,9 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_concretize(const Fuse
         float pl = 0.f, pu = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
+            const float c = cl[r], rd = cu[r];                      // centre and radius terms
+            cl[r] = c - rd;
+            cu[r] = c + rd;
             pl = nacc<Q>(pl, cl[r], f.qv);
             pu = nacc<Q>(pu, cu[r], f.qv);
             if (col < g.N) {
