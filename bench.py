@@ -43,13 +43,13 @@ COLD_SETS = 5                  # disjoint operand sets cycled by the cold measur
 
 def traffic_from_profile():
     """HBM bytes per launch of the relaxation kernels as the hardware counters saw them: the lines
-    `traffic_bytes_per_launch <relu|tanh> <warm|cold> <bytes>` of profiles/hbm_traffic_pmc.md (rocprofv3
+    `traffic_bytes_per_launch <relu|tanh> <warm|cold> <bytes>` of profiles/hbm_traffic_relaxations.txt (rocprofv3
     --pmc FETCH_SIZE / WRITE_SIZE of this program, scaled by the same counters on faith_copy_f32 of known
     size).  Empty if the summary is missing."""
     import re
     out = {}
     try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic_pmc.md")) as f:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic_relaxations.txt")) as f:
             for m in re.finditer(r"^traffic_bytes_per_launch\s+(\w+)\s+(warm|cold)\s+(\d+)", f.read(), flags=re.M):
                 out[(m.group(1), m.group(2))] = int(m.group(3))
     except OSError:
