@@ -27,13 +27,17 @@ def _ledger():
     return parity.LEDGER
 
 
+# the folder for what a test run leaves behind (not under version control)
+LEDGER_DIR = os.environ.get("FAITH_TEST_OUTPUT", "gpurun_out")
+
+
 def pytest_sessionfinish(session, exitstatus):
     """Keeps the parity concessions of the run (tests/parity.py) where the run's output is kept."""
     import json
     led = _ledger()
     if not led["comparisons"]:
         return
-    out = os.path.join(ROOT, "gpurun_out")
+    out = os.path.join(ROOT, LEDGER_DIR)
     try:
         os.makedirs(out, exist_ok=True)
         with open(os.path.join(out, "parity_ledger.json"), "w") as f:
@@ -53,6 +57,6 @@ def pytest_terminal_summary(terminalreporter):
         per_test[(fn, c["kind"], c["tensor"])] = per_test.get((fn, c["kind"], c["tensor"]), 0) + 1
     terminalreporter.write_line(
         f"parity ledger: {led['comparisons']} harness comparisons, {led['plain']} on the plain bar "
-        f"(rtol 1e-5 / atol 1e-6), concessions: {kinds if kinds else 'none'} (each one in gpurun_out/parity_ledger.json)")
+        f"(rtol 1e-5 / atol 1e-6), concessions: {kinds if kinds else 'none'} (each one in {LEDGER_DIR}/parity_ledger.json)")
     for (fn, kind, tensor), n in sorted(per_test.items()):
         terminalreporter.write_line(f"  {n:4d} x {kind:<24s} {tensor:<6s} {fn}")

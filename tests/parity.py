@@ -37,7 +37,7 @@ RTOL, ATOL = 1e-5, 1e-6
 
 # Every comparison that did not pass on the plain bar alone is entered here -- which test, which
 # tensor, which concession, how large -- and every comparison is counted.  tests/conftest.py prints
-# the totals at the end of the session and writes them to gpurun_out/parity_ledger.json, so a run
+# the totals at the end of the session and writes them to parity_ledger.json in the run's output folder, so a run
 # shows how many tensors or neurons leaned on a concession even when it prints nothing else.
 LEDGER = {"comparisons": 0, "plain": 0, "concessions": []}
 
