@@ -712,10 +712,12 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         // 12 % ahead when every byte comes from and goes to HBM (55 against 62 us on the same shape with
         // five operand sets in turn), and 3 % more with non-temporal loads (54 us; those cost 25 % when the
         // operands are cached).  An object whose traffic exceeds the cache by more than a quarter cannot be
-        // resident, so it takes the second shape; knob values 7 / 8 force one or the other.
+        // resident, so it takes the second shape; knob values 7 / 8 force one or the other, 12 the second
+        // without the non-temporal loads (the middle: relu 42.4 us warm / 55.1 us cold, tanh 45.8 / 58.0).
         const long long traffic = 16LL * a.rows * a.D * a.H;
         const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 5LL * (256LL << 20) / 4);
         if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(a, st);
+        else if (tv == 12) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(a, st);
         else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(a, st);
         else launch_resident<MODE, Q, 8, 256, 8>(a, st);
         return;
