@@ -135,6 +135,9 @@ def test_conv_config4_full_size_properties():
     sub = slice(100, 104)
     lw2, _, uw2, _ = ops.conv2d(x["lw"][:, sub].contiguous(), x["lb"], x["uw"][:, sub].contiguous(), x["ub"], W, bias, 1, 1)
     assert torch.equal(lw2, lw[:, sub]) and torch.equal(uw2, uw[:, sub])
+    # ordered inputs (uw >= lw here) give ordered results exactly: uw' = M + R, lw' = M - R with R a sum of
+    # non-negative products
+    assert bool((uw >= lw).all()) and bool((ub >= lb).all())
     l, u = ops.concretize_conv(lw, lb, uw, ub, c["p"], c["eps"])
     assert bool((l <= u).all())
     g = torch.Generator().manual_seed(4)

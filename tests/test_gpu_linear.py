@@ -157,7 +157,9 @@ def test_linear_closed_forms_on_gpu():
     assert torch.equal(lw, uw) and torch.equal(lb, ub)
     lw, lb, uw, ub = run_linear(x, W, None)
     assert close(uw.cpu() - lw.cpu(), (x.uw - x.lw) @ W.abs().t(), rtol=1e-4, atol=1e-5)
-    assert bool((uw >= lw - 1e-6).all())
+    # ordered coefficients stay ordered EXACTLY: the kernels form uw' = M + R and lw' = M - R with a radius term
+    # R that is a sum of non-negative products
+    assert bool((uw >= lw).all())
 
 
 def test_linear_config2_full_size_properties():
@@ -168,7 +170,7 @@ def test_linear_config2_full_size_properties():
     c = make_config(2)
     lw, lb, uw, ub, W, bias = dev(*(c["x"][k] for k in ("lw", "lb", "uw", "ub")), c["W"], c["bias"])
     olw, olb, ouw, oub = ops.linear(lw, lb, uw, ub, W, bias)
-    assert bool((ouw >= olw - 1e-6).all()) and bool((oub >= olb).all())
+    assert bool((ouw >= olw).all()) and bool((oub >= olb).all())
     # sampled rows against float64
     Wp, Wn = W.double().clamp(min=0).t(), W.double().clamp(max=0).t()
     idx = torch.randint(0, 256 * 512, (64,), generator=torch.Generator().manual_seed(1)).cuda()
