@@ -11,9 +11,9 @@
 //
 // Computed in centre / radius form (W+ + W- = W, W+ - W- = |W|):
 //     y_l = M - R,   y_u = M + R,   M = conv((x_l + x_u) / 2, W),   R = conv((x_u - x_l) / 2, |W|)
-// -- two products per tap where the formula above has four.  Centre and radius of an input pair are formed
-// once, by the thread that stages the patch (an out-of-image position is 0 in both); |W| by the wavefront that
-// reads the weight.
+// -- two products per tap where the formula above has four.  Sum and difference of an input pair are formed
+// once, by the thread that stages the patch (an out-of-image position is 0 in both), the halving is left to the
+// epilogue (exact either way); |W| by the wavefront that reads the weight.
 //
 // Implicit GEMM:  C[co, p] = sum_k W[co, k] * X[k, p],  k = (ci, kh, kw),  p = output pixel.
 // MFMA rows are output channels (W and |W|), MFMA columns are pixels (centre and radius of x), so lanes run along ow and every store is a contiguous run of a
@@ -112,8 +112,8 @@ conv_signsplit(const ConvArgs g) {
                 const int iw = iw0 + pc;
                 const bool ok = row_ok && iw >= 0 && iw < g.W;
                 const float vl = ok ? xl_n[rbase + iw] : 0.f, vu = ok ? xu_n[rbase + iw] : 0.f;
-                sXl[rr * pcol + pc] = 0.5f * (vl + vu);      // centre
-                sXu[rr * pcol + pc] = 0.5f * (vu - vl);      // radius
+                sXl[rr * pcol + pc] = vl + vu;               // twice the centre
+                sXu[rr * pcol + pc] = vu - vl;               // twice the radius
             }
         }
         // ---- stage the weight slab: CC*KK contiguous floats per output channel
@@ -172,8 +172,8 @@ conv_signsplit(const ConvArgs g) {
                 const int co = co0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (co < g.Co) {
                     const size_t o = (((size_t)n * g.Co + co) * g.Ho + oh) * g.Wo + ow;
-                    __builtin_nontemporal_store(cl[a][b][r] - cu[a][b][r], &g.yl[o]);      // centre - radius
-                    __builtin_nontemporal_store(cl[a][b][r] + cu[a][b][r], &g.yu[o]);
+                    __builtin_nontemporal_store(0.5f * (cl[a][b][r] - cu[a][b][r]), &g.yl[o]);      // centre - radius
+                    __builtin_nontemporal_store(0.5f * (cl[a][b][r] + cu[a][b][r]), &g.yu[o]);
                 }
             }
         }
@@ -269,8 +269,8 @@ conv_signsplit_k3s1(const ConvArgs g) {
         for (int u = 0; u < NP; ++u) {
             const int e = tid + u * NTHREADS;
             if (e < CC * PP) {
-                sXl[buf][e] = 0.5f * (pxl[u] + pxu[u]);      // centre
-                sXu[buf][e] = 0.5f * (pxu[u] - pxl[u]);      // radius
+                sXl[buf][e] = pxl[u] + pxu[u];               // twice the centre
+                sXu[buf][e] = pxu[u] - pxl[u];               // twice the radius
             }
         }
 #pragma unroll
@@ -367,9 +367,9 @@ conv_signsplit_k3s1(const ConvArgs g) {
             for (int r = 0; r < 16; ++r) {
                 const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
                                     (unsigned)(oh * g.Wo) * 4u;
-                // y_l = centre - radius, y_u = centre + radius
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] - cu[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] + cu[a][b][r]), wyu, vo, so, 2);
+                // y_l = centre - radius, y_u = centre + radius (the accumulators hold twice each)
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(0.5f * (cl[a][b][r] - cu[a][b][r])), wyl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(0.5f * (cl[a][b][r] + cu[a][b][r])), wyu, vo, so, 2);
             }
         }
     }
@@ -502,8 +502,8 @@ conv_signsplit_fast(const ConvArgs g) {
         for (int u = 0; u < NP; ++u) {
             const int e = tid + u * NTHREADS;
             if (e < CCH * PP) {
-                dl[e] = 0.5f * (pxl[u] + pxu[u]);            // centre
-                du[e] = 0.5f * (pxu[u] - pxl[u]);            // radius
+                dl[e] = pxl[u] + pxu[u];                     // twice the centre
+                du[e] = pxu[u] - pxl[u];                     // twice the radius
             }
         }
     };
@@ -619,9 +619,9 @@ conv_signsplit_fast(const ConvArgs g) {
             for (int r = 0; r < 16; ++r) {
                 const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
                                     (unsigned)(row0 * g.Wo) * 4u;
-                // y_l = centre - radius, y_u = centre + radius
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] - cu[a][b][r]), wyl, vo, so, 2 /* non-temporal */);
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[a][b][r] + cu[a][b][r]), wyu, vo, so, 2);
+                // y_l = centre - radius, y_u = centre + radius (the accumulators hold twice each)
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(0.5f * (cl[a][b][r] - cu[a][b][r])), wyl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(0.5f * (cl[a][b][r] + cu[a][b][r])), wyu, vo, so, 2);
             }
         }
     }

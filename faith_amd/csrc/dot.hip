@@ -12,7 +12,8 @@
 // i.e. eight products per K-pair as written.  The four y terms share their multiplier b (the planes take
 // b = l_x on both sides), and b+ + b- = b, b+ - b- = |b|, so
 //     sum_k b+ ylw + b- yuw = P + Q,     sum_k b+ yuw + b- ylw = P - Q,
-//     P = sum_k (b/2) (ylw + yuw),       Q = sum_k (|b|/2) (ylw - yuw):
+//     P = sum_k (b/2) (ylw + yuw),       Q = sum_k (|b|/2) (ylw - yuw)
+// (accumulated as 2 P and 2 Q from b and |b| and halved once per result: exact either way):
 // two products where there were four -- SIX MFMA products per K-pair into four accumulators (the x terms
 // of z_lw and of z_uw, P, Q), combined when a tile is done: a quarter of the MFMA time gone.  The halving
 // is exact; ylw + yuw and ylw - yuw are rounded once each, by the thread that stages them.  Rows (i) come
@@ -22,7 +23,7 @@
 //
 // Tiling: workgroup = 4 wavefronts on a 128 x 64 (i x j) tile of one (head, m); wavefront tile
 // 64 x 32 (two v_mfma_f32_32x32x2_f32 blocks along i, for each of the four accumulators).  K-step 8:
-// operand tiles xlw, xuw, b/2, |b|/2 [128 x 8] and a_l+, a_l-, a_u+, a_u-, ylw + yuw, ylw - yuw [64 x 8]
+// operand tiles xlw, xuw, b, |b| [128 x 8] and a_l+, a_l-, a_u+, a_u-, ylw + yuw, ylw - yuw [64 x 8]
 // = 28 KB, double buffered, two workgroups per CU.  Rows are 8 floats with the two 16-byte halves swapped
 // on every other group of four rows, which makes both the 16-byte stores and the 16-byte fragment
 // reads bank-conflict free without padding.
@@ -118,9 +119,8 @@ __device__ __forceinline__ float pos1(float v) { return __builtin_fmaxf(v, 0.f);
 __device__ __forceinline__ float neg1(float v) { return __builtin_fminf(v, 0.f); }
 __device__ __forceinline__ float4 pos4(float4 v) { return make_float4(pos1(v.x), pos1(v.y), pos1(v.z), pos1(v.w)); }
 __device__ __forceinline__ float4 neg4(float4 v) { return make_float4(neg1(v.x), neg1(v.y), neg1(v.z), neg1(v.w)); }
-__device__ __forceinline__ float4 half4(float4 v) { return make_float4(0.5f * v.x, 0.5f * v.y, 0.5f * v.z, 0.5f * v.w); }
-__device__ __forceinline__ float4 half_abs4(float4 v) {
-    return make_float4(0.5f * __builtin_fabsf(v.x), 0.5f * __builtin_fabsf(v.y), 0.5f * __builtin_fabsf(v.z), 0.5f * __builtin_fabsf(v.w));
+__device__ __forceinline__ float4 abs4(float4 v) {
+    return make_float4(__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w));
 }
 __device__ __forceinline__ float4 add4(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
 __device__ __forceinline__ float4 sub4(float4 a, float4 b) { return make_float4(a.x - b.x, a.y - b.y, a.z - b.z, a.w - b.w); }
@@ -288,8 +288,8 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
         float *s = sm[buf];
         *reinterpret_cast<float4 *>(s + XL + sdst) = pre[0];
         *reinterpret_cast<float4 *>(s + XU + sdst) = pre[1];
-        *reinterpret_cast<float4 *>(s + BH + sdst) = half4(pre[2]);
-        *reinterpret_cast<float4 *>(s + BA + sdst) = half_abs4(pre[2]);
+        *reinterpret_cast<float4 *>(s + BH + sdst) = pre[2];                 // b and |b|: P and Q come out doubled
+        *reinterpret_cast<float4 *>(s + BA + sdst) = abs4(pre[2]);          // and are halved once per result
         if (wside) {
             *reinterpret_cast<float4 *>(s + YS + ydst) = add4(pre[3], pre[4]);
             *reinterpret_cast<float4 *>(s + YD + ydst) = sub4(pre[3], pre[4]);
@@ -372,8 +372,8 @@ dot_w(const DotArgs g, const int total_tiles, const int xcd_map) {
                 const int row_in_tile = a * 32 + 8 * (r / 4) + r % 4;
                 if (EXACT || row_in_tile < rows) {
                     const float p = cp[a][r], q = cq[a][r];
-                    st1_nt(cl[a][r] + (p + q), rl, lane_off, row_in_tile * step_b);
-                    st1_nt(cu[a][r] + (p - q), ru, lane_off, row_in_tile * step_b);
+                    st1_nt(cl[a][r] + 0.5f * (p + q), rl, lane_off, row_in_tile * step_b);
+                    st1_nt(cu[a][r] + 0.5f * (p - q), ru, lane_off, row_in_tile * step_b);
                 }
             }
     };
@@ -492,7 +492,7 @@ __global__ void __launch_bounds__(256) dot_b(const DotArgs g) {
 // Short sequences (Lx, Ly <= 64, d <= 80): the 128 x 64 tile above would be mostly padding, so here
 // a WAVEFRONT owns one 32 x 32 block of z for one perturbation coordinate m (one MFMA block for
 // z_lw, one for z_uw).  The four wavefronts of a workgroup share the (head, i-block, j-block): the
-// operands that do not depend on m (b / 2, |b| / 2, a_l+-, a_u+- split by sign) are staged in LDS once for
+// operands that do not depend on m (b, |b|, a_l+-, a_u+- split by sign) are staged in LDS once for
 // the whole reduction, and every wavefront walks its own `mpw` coordinates, loading its x and y
 // fragments straight from global memory in MFMA layout (rows of 32 bytes per lane and K-step: poor
 // coalescing, but these problems are a few megabytes and latency is what counts).
@@ -545,16 +545,16 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
             const int row = e / dp, k = e % dp;
             const float bt = k < d ? g.x_l[xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + k] : 0.f;
             const int dst = (k / 8) * (SB * 8) + swz(row, (k % 8) / 4) + k % 4;
-            s_bp[dst] = 0.5f * bt;                     // b / 2 and |b| / 2: see the top of the file
-            s_bn[dst] = 0.5f * __builtin_fabsf(bt);
+            s_bp[dst] = bt;                            // b and |b|: see the top of the file
+            s_bn[dst] = __builtin_fabsf(bt);
         }
     }
     for (int e = tid; !RAGGED && e < SB * d / 4; e += 256) {
         const int row = e / (d / 4), c4 = e % (d / 4);
         const int dst = (c4 / 2) * (SB * 8) + swz(row, c4 % 2);
         const float4 bt = *reinterpret_cast<const float4 *>(g.x_l + xb0 + (size_t)min(i0 + row, g.Lx - 1) * g.ox.pitch + c4 * 4);
-        *reinterpret_cast<float4 *>(s_bp + dst) = half4(bt);         // b / 2 and |b| / 2: see the top of the file
-        *reinterpret_cast<float4 *>(s_bn + dst) = half_abs4(bt);
+        *reinterpret_cast<float4 *>(s_bp + dst) = bt;                // b and |b|: see the top of the file
+        *reinterpret_cast<float4 *>(s_bn + dst) = abs4(bt);
         if (!VP) {
             const size_t o = yb0 + (size_t)min(j0 + row, g.Ly - 1) * g.oy.pitch + c4 * 4;
             const float4 al = *reinterpret_cast<const float4 *>(g.y_l + o), au = *reinterpret_cast<const float4 *>(g.y_u + o);
@@ -664,8 +664,8 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
                 const int i = i0 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (i < g.Lx) {
                     const size_t o = zw0 + ((size_t)i * g.D + m) * g.oz.pitch + j0 + fi;
-                    __builtin_nontemporal_store(cl[r] + (cp[r] + cq[r]), &g.zlw[o]);
-                    __builtin_nontemporal_store(cu[r] + (cp[r] - cq[r]), &g.zuw[o]);
+                    __builtin_nontemporal_store(cl[r] + 0.5f * (cp[r] + cq[r]), &g.zlw[o]);
+                    __builtin_nontemporal_store(cu[r] + 0.5f * (cp[r] - cq[r]), &g.zuw[o]);
                 }
             }
         }

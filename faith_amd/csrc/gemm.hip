@@ -10,8 +10,9 @@
 // Computed in centre / radius form: W+ + W- = W and W+ - W- = |W|, so
 //     C_l = M - R,   C_u = M + R,   M = ((A_l + A_u) / 2) @ W,   R = ((A_u - A_l) / 2) @ |W|
 // -- TWO products per term where the formula above has four, i.e. half the MFMA time for the same
-// four results.  The halving is exact; centre and radius of a coefficient pair are rounded once each, by
-// the thread that stages them; what that adds to the rounding of the four-product form (each bound then
+// four results.  (The kernels accumulate 2 M and 2 R from A_l + A_u and A_u - A_l and halve once per result:
+// one vector instruction per staged element less, the same bits.)  The halving is exact; sum and difference
+// of a coefficient pair are rounded once each, by the thread that stages them; what that adds to the rounding of the four-product form (each bound then
 // carries the rounding of both operands' terms: measured 1.3 - 1.9 x its error against float64, 0.1 of
 // the parity bar on the configurations) is bounded by the parity tests together with the order of summation.
 //
@@ -66,12 +67,13 @@ struct GemmArgs {
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
-// centre (l + u) / 2 and radius (u - l) / 2 of a pair of coefficients; |w|
+// twice the centre, l + u, and twice the radius, u - l, of a pair of coefficients (the halving is left to the
+// epilogue, where it is done once per result instead of once per operand element: it is exact either way); |w|
 __device__ __forceinline__ float4 mid4(float4 l, float4 u) {
-    return make_float4(0.5f * (l.x + u.x), 0.5f * (l.y + u.y), 0.5f * (l.z + u.z), 0.5f * (l.w + u.w));
+    return make_float4(l.x + u.x, l.y + u.y, l.z + u.z, l.w + u.w);
 }
 __device__ __forceinline__ float4 rad4(float4 l, float4 u) {
-    return make_float4(0.5f * (u.x - l.x), 0.5f * (u.y - l.y), 0.5f * (u.z - l.z), 0.5f * (u.w - l.w));
+    return make_float4(u.x - l.x, u.y - l.y, u.z - l.z, u.w - l.w);
 }
 __device__ __forceinline__ float4 abs4(float4 v) {
     return make_float4(__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w));
@@ -171,7 +173,7 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
         }
     };
 
-    // cl accumulates the centre term (A_l + A_u)/2 . W and cu the radius term (A_u - A_l)/2 . |W|; they become
+    // cl accumulates twice the centre term, (A_l + A_u) . W, and cu twice the radius term, (A_u - A_l) . |W|; they become
     // C_l and C_u when the reduction is done
     floatx16 cl[MBM][MBN], cu[MBM][MBN];
 #pragma unroll
@@ -256,9 +258,9 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
         for (int b = 0; b < MBN; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float c = cl[a][b][r], rd = cu[a][b][r];
-                cl[a][b][r] = c - rd;
-                cu[a][b][r] = c + rd;
+                const float c = cl[a][b][r], rd = cu[a][b][r];      // 2 M and 2 R
+                cl[a][b][r] = 0.5f * (c - rd);
+                cu[a][b][r] = 0.5f * (c + rd);
             }
     const size_t c_bytes = (size_t)min(M - m0, BM) * g.N * 4;
     const __amdgpu_buffer_rsrc_t wcl = window(g.Cl + (size_t)m0 * g.N, c_bytes);
@@ -520,8 +522,8 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs
         // sl is the centre term, su the radius term
         const int row = m0 + 8 * wv + 4 * fh + q;
         if (row < g.Mw && col < g.N) {
-            g.Cl[(size_t)row * g.N + col] = sl - su;
-            g.Cu[(size_t)row * g.N + col] = sl + su;
+            g.Cl[(size_t)row * g.N + col] = 0.5f * (sl - su);
+            g.Cu[(size_t)row * g.N + col] = 0.5f * (sl + su);
         }
     }
 }
@@ -899,9 +901,9 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_concretize(const Fuse
         float pl = 0.f, pu = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float c = cl[r], rd = cu[r];                      // centre and radius terms
-            cl[r] = c - rd;
-            cu[r] = c + rd;
+            const float c = cl[r], rd = cu[r];                      // twice the centre and radius terms
+            cl[r] = 0.5f * (c - rd);
+            cu[r] = 0.5f * (c + rd);
             pl = nacc<Q>(pl, cl[r], f.qv);
             pu = nacc<Q>(pu, cu[r], f.qv);
             if (col < g.N) {
