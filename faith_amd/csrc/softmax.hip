@@ -31,8 +31,59 @@ struct SoftmaxArgs {
     float scale;                    // > 0: the object is multiplied by it first (Bounds.multiply with a float)
 };
 
+// Buffer addressing: the hardware compares thread offset + uniform offset against the window's size; accesses at
+// or beyond it return zero (loads) or are dropped (stores).
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t slab_window(const float *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)bytes, 0x00020000);
+}
+// the value another lane of the same row of 16 lanes holds; CTRL is the permutation (a DPP control word)
+template <int CTRL>
+__device__ __forceinline__ float lane_permute(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+// One butterfly step at distance m for 2 N values through the LDS crossbar, the 2 N exchanges in flight together.
+// (The swap instructions v_permlane16_swap / v_permlane32_swap do distances 16 and 32 on the vector ALU, but with
+// the copies and wait states they need they measured slower here: 63.7 against 61.8 us on a [256 x 128] slab.)
+template <int Q, int N>
+__device__ __forceinline__ void combine_across(float (&a)[N], float (&b)[N], int m) {
+    float ta[N], tb[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        ta[i] = __shfl_xor(a[i], m, WAVE);
+        tb[i] = __shfl_xor(b[i], m, WAVE);
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        a[i] = ncomb<Q>(a[i], ta[i]);
+        b[i] = ncomb<Q>(b[i], tb[i]);
+    }
+}
+template <int VEC>
+__device__ __forceinline__ Vec<VEC> slab_load(__amdgpu_buffer_rsrc_t w, unsigned thread_off, unsigned uniform_off) {
+    Vec<VEC> d;
+    if constexpr (VEC == 4) {
+        const uintx4 t = __builtin_amdgcn_raw_buffer_load_b128(w, thread_off, uniform_off, 0);
+        d.v = make_float4(__uint_as_float(t.x), __uint_as_float(t.y), __uint_as_float(t.z), __uint_as_float(t.w));
+    } else {
+        d.v = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(w, thread_off, uniform_off, 0));
+    }
+    return d;
+}
+template <int VEC>
+__device__ __forceinline__ void slab_store(const Vec<VEC> &d, __amdgpu_buffer_rsrc_t w, unsigned thread_off, unsigned uniform_off) {
+    if constexpr (VEC == 4) {
+        const uintx4 t = {__float_as_uint(d.v.x), __float_as_uint(d.v.y), __float_as_uint(d.v.z), __float_as_uint(d.v.w)};
+        __builtin_amdgcn_raw_buffer_store_b128(t, w, thread_off, uniform_off, 2 /* non-temporal */);
+    } else {
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(d.v), w, thread_off, uniform_off, 2);
+    }
+}
+
+// Four wavefronts per SIMD (128 registers): two workgroups of 512 threads or four of 256 on a CU, so that one's
+// arithmetic runs beside another's loads and stores.  (A general exponent keeps the registers it needs.)
 template <int Q, int VEC, int NTHREADS, int RPT>
-__global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, const int tpr_log2) {
+__global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) ? 1 : 4) softmax_kernel(const SoftmaxArgs a, const int tpr_log2) {
     constexpr int NW = NTHREADS / WAVE;
     extern __shared__ float smem[];
     const int TPR = 1 << tpr_log2, TH = TPR * VEC, RG = NTHREADS >> tpr_log2;
@@ -46,53 +97,85 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
     const int c = tid & (TPR - 1), rg = tid >> tpr_log2;
     const int col0 = c * VEC;
     const bool col_ok = col0 < a.H;                  // VEC == 4: H % 4 == 0, so the four columns stand or fall together
-    const size_t base = ((size_t)r * a.D + rg) * a.H + col0;
-    const size_t row_step = (size_t)RG * a.H;
     const int blk = a.D / a.words;
 
+    // the column's constant terms first: they are needed right after the first barrier and would otherwise
+    // be fetched then, behind the whole machine's slab loads
+    const size_t bi = (size_t)r * a.H + tid;         // thread h < H speaks for column h
+    float xlb = 0.f, xub = 0.f;
+    if (tid < a.H) {
+        xlb = a.lb[bi];
+        xub = a.ub[bi];
+    }
+
     // ---- x: the slab into registers
+    // Buffer addressing over the row's own slab: a thread whose column does not exist is sent outside the window
+    // and slab rows past D_in fall outside it, where loads return zero and stores are dropped -- no branch and
+    // no wait between the loads, all 2 RPT of a thread are in flight together.
+    const unsigned slab_bytes = (unsigned)a.D * a.H * 4u;
+    const size_t slab0 = (size_t)r * a.D * a.H;
+    const unsigned voff = col_ok ? ((unsigned)rg * a.H + col0) * 4u : 0x80000000u;
+    const unsigned step_bytes = (unsigned)RG * a.H * 4u;
     Vec<VEC> dl[RPT], du[RPT];
+    {
+        const __amdgpu_buffer_rsrc_t wl = slab_window(a.lw + slab0, slab_bytes), wu = slab_window(a.uw + slab0, slab_bytes);
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-        if (col_ok && i * RG + rg < a.D) {
-            dl[i].load(a.lw + base + i * row_step);
-            du[i].load(a.uw + base + i * row_step);
+        for (int i = 0; i < RPT; ++i) {
+            dl[i] = slab_load<VEC>(wl, voff, i * step_bytes);
+            du[i] = slab_load<VEC>(wu, voff, i * step_bytes);
+        }
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {        // one rounding, as the separate scaling stores it
                 dl[i].set(v, dl[i].get(v) * a.scale);
                 du[i].set(v, du[i].get(v) * a.scale);
             }
-        } else {
-            dl[i].zero();
-            du[i].zero();
         }
     }
 
     // column norms of what dl / du hold -> part; the caller synchronises
+    // A perturbed word owns `blk` consecutive rows.  When blk is a multiple of RG, the rows i * RG + rg of step i
+    // belong to one word for every thread: the membership test is then a scalar one per step instead of one per
+    // value (the usual case; rows past D_in hold zeros and add nothing to any norm).
+    const bool whole_steps = blk % RG == 0;
+    const int steps_per_word = blk / RG;
     auto column_norms = [&]() {
         for (int w = 0; w < a.words; ++w) {
             const int lo_row = w * blk, hi_row = lo_row + blk;
             float pl[VEC], pu[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
+            if (whole_steps) {
+                const int lo_i = w * steps_per_word, hi_i = lo_i + steps_per_word;
 #pragma unroll
-            for (int i = 0; i < RPT; ++i) {
-                const int row = i * RG + rg;
-                if (row >= lo_row && row < hi_row) {
+                for (int i = 0; i < RPT; ++i) {
+                    if (i >= lo_i && i < hi_i) {
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) {
-                        pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
-                        pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
+                        for (int v = 0; v < VEC; ++v) {
+                            pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
+                            pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RPT; ++i) {
+                    const int row = i * RG + rg;
+                    if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) {
+                            // opaque copies: |x| or x^2 of every value would otherwise be formed once, outside the
+                            // loop over the words, and held (64 more registers)
+                            float xl = dl[i].get(v), xu = du[i].get(v);
+                            asm volatile("" : "+v"(xl), "+v"(xu));
+                            pl[v] = nacc<Q>(pl[v], xl, a.qv);
+                            pu[v] = nacc<Q>(pu[v], xu, a.qv);
+                        }
                     }
                 }
             }
-            for (int m = TPR; m < WAVE; m <<= 1) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                    pl[v] = ncomb<Q>(pl[v], __shfl_xor(pl[v], m, WAVE));
-                    pu[v] = ncomb<Q>(pu[v], __shfl_xor(pu[v], m, WAVE));
-                }
-            }
+            for (int m = TPR; m < WAVE; m <<= 1) combine_across<Q>(pl, pu, m);
             if (lane < TPR) {
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
@@ -108,25 +191,22 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
     auto neuron_norms = [&]() {
         for (int w = 0; w < a.words; ++w) {
             const int lo_row = w * blk, hi_row = lo_row + blk;
-            float pl = 0.f, pu = 0.f;
+            float pl[1] = {0.f}, pu[1] = {0.f};
             if (c == 0) {
 #pragma unroll
                 for (int i = 0; i < RPT; ++i) {
                     const int row = i * RG + rg;
                     if (row >= lo_row && row < hi_row) {
-                        pl = nacc<Q>(pl, sl[i], a.qv);
-                        pu = nacc<Q>(pu, su[i], a.qv);
+                        pl[0] = nacc<Q>(pl[0], sl[i], a.qv);
+                        pu[0] = nacc<Q>(pu[0], su[i], a.qv);
                     }
                 }
             }
-#pragma unroll
-            for (int m = 1; m < WAVE; m <<= 1) {
-                pl = ncomb<Q>(pl, __shfl_xor(pl, m, WAVE));
-                pu = ncomb<Q>(pu, __shfl_xor(pu, m, WAVE));
-            }
+            // the lanes that hold something are TPR apart: the butterfly starts there
+            for (int m = TPR; m < WAVE; m <<= 1) combine_across<Q>(pl, pu, m);
             if (lane == 0) {
-                spart[(w * NW + wv) * 2 + 0] = pl;
-                spart[(w * NW + wv) * 2 + 1] = pu;
+                spart[(w * NW + wv) * 2 + 0] = pl[0];
+                spart[(w * NW + wv) * 2 + 1] = pu[0];
             }
         }
     };
@@ -135,10 +215,40 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
         l = lb;
         u = ub;
         for (int w = 0; w < a.words; ++w) {
+            // the wavefronts' partial norms are fetched eight at a time before the first is used: one LDS latency
+            // per eight wavefronts instead of one per wavefront (combined in the order of the wavefronts all the same)
+            constexpr int CH = NW < 8 ? NW : 8;
             float nl = 0.f, nu = 0.f;
-            for (int g = 0; g < NW; ++g) {
-                nl = ncomb<Q>(nl, p[((w * NW + g) * 2 + 0) * stride + offset]);
-                nu = ncomb<Q>(nu, p[((w * NW + g) * 2 + 1) * stride + offset]);
+#pragma unroll
+            for (int g0 = 0; g0 < NW; g0 += CH) {
+                float vl[CH], vu[CH];
+#pragma unroll
+                for (int g = 0; g < CH; ++g) {
+                    vl[g] = p[((w * NW + g0 + g) * 2 + 0) * stride + offset];
+                    vu[g] = p[((w * NW + g0 + g) * 2 + 1) * stride + offset];
+                }
+#pragma unroll
+                for (int g = 0; g < CH; ++g) {
+                    nl = ncomb<Q>(nl, vl[g]);
+                    nu = ncomb<Q>(nu, vu[g]);
+                }
+            }
+            l += (-a.eps) * nfin<Q>(nl, a.qv);
+            u += a.eps * nfin<Q>(nu, a.qv);
+        }
+    };
+
+    // the same for a one-neuron object from spart, every thread for itself: lane g takes wavefront g's partial norm
+    // and a butterfly over NW lanes combines them (2 log2 NW exchanges per word instead of 2 NW reads and sums)
+    auto neuron_interval = [&](float lb, float ub, float &l, float &u) {
+        l = lb;
+        u = ub;
+        for (int w = 0; w < a.words; ++w) {
+            float nl = spart[(w * NW + lane % NW) * 2 + 0], nu = spart[(w * NW + lane % NW) * 2 + 1];
+#pragma unroll
+            for (int m = 1; m < NW; m <<= 1) {
+                nl = ncomb<Q>(nl, __shfl_xor(nl, m, WAVE));
+                nu = ncomb<Q>(nu, __shfl_xor(nu, m, WAVE));
             }
             l += (-a.eps) * nfin<Q>(nl, a.qv);
             u += a.eps * nfin<Q>(nu, a.qv);
@@ -148,9 +258,9 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
     // ---- e = exp(x): Bounds.py:970-1003
     column_norms();
     __syncthreads();
-    const size_t bi = (size_t)r * a.H + tid;         // thread h < H speaks for column h
     if (tid < a.H) {
-        const float xlb = a.lb[bi] * a.scale, xub = a.ub[bi] * a.scale;
+        xlb *= a.scale;
+        xub *= a.scale;
         float l, u, klo, kup, elb, eub;
         interval(part, TH, tid, xlb, xub, l, u);
         relax_point<EXP>(l, u, xlb, xub, klo, kup, elb, eub);
@@ -187,13 +297,26 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
             tl += dl[i].get(v);
             tu += du[i].get(v);
         }
-        for (int m = 1; m < TPR; m <<= 1) {
-            tl += __shfl_xor(tl, m, WAVE);
-            tu += __shfl_xor(tu, m, WAVE);
-        }
         sl[i] = tl;
         su[i] = tu;
     }
+    // The butterfly over the threads of a slab row, all RPT rows per step.  Distances 1 to 8 are lane permutations
+    // inside a row of 16 lanes, which the vector ALU does on its own operand (no trip through the LDS crossbar):
+    // 1 and 2 as permutations of four lanes; after them the four lanes of a group hold one value, so mirroring
+    // eight lanes fetches what lane ^ 4 holds, and after that mirroring sixteen fetches what lane ^ 8 holds.
+    // Longer distances go through the crossbar, 2 RPT exchanges in flight at a time.
+    auto butterfly_step = [&](auto exchange) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            sl[i] += exchange(sl[i]);
+            su[i] += exchange(su[i]);
+        }
+    };
+    if (TPR > 1) butterfly_step([](float x) { return lane_permute<0xB1>(x); });      // lanes 1 0 3 2
+    if (TPR > 2) butterfly_step([](float x) { return lane_permute<0x4E>(x); });      // lanes 2 3 0 1
+    if (TPR > 4) butterfly_step([](float x) { return lane_permute<0x141>(x); });     // eight lanes mirrored
+    if (TPR > 8) butterfly_step([](float x) { return lane_permute<0x140>(x); });     // sixteen lanes mirrored
+    for (int m = 16; m < TPR; m <<= 1) combine_across<FAITH_Q_1>(sl, su, m);      // Q_1: a sum
     if (wv == 0) {
         float tl = 0.f, tu = 0.f;
         for (int h = lane; h < a.H; h += WAVE) {
@@ -218,7 +341,7 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
     {
         const float slb = scal[0], sub = scal[1];
         float l, u, klo, kup;
-        interval(spart, 1, 0, slb, sub, l, u);
+        neuron_interval(slb, sub, l, u);
         if (tid == 0 && a.sum_l) a.sum_l[r] = l;
         relax_point<RECIP>(l, u, slb, sub, klo, kup, rlb, rub);
 #pragma unroll
@@ -235,7 +358,7 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
     neuron_norms();
     __syncthreads();
     float al, au;
-    interval(spart, 1, 0, rlb, rub, al, au);
+    neuron_interval(rlb, rub, al, au);
     if (tid < a.H) {
         const float elb = col[2 * TH + tid], eub = col[3 * TH + tid];
         float bt, unused;
@@ -246,13 +369,27 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
         a.oub[bi] = ((au > 0.f ? eub : elb) * au + gu) + (bt > 0.f ? rub : rlb) * bt;
     }
     __syncthreads();
-    if (!col_ok) return;
     float bt[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) bt[v] = col[4 * TH + col0 + v];
+    const __amdgpu_buffer_rsrc_t wol = slab_window(a.olw + slab0, slab_bytes), wou = slab_window(a.ouw + slab0, slab_bytes);
+    // a_l and a_u are one neuron's bounds, the same for the whole workgroup: both positive (a reciprocal of a
+    // positive sum) is the case that runs without the selects on their sign
+    if (al > 0.f && au > 0.f) {
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-        if (i * RG + rg < a.D) {
+        for (int i = 0; i < RPT; ++i) {
+            Vec<VEC> ol, ou;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                ol.set(v, dl[i].get(v) * al + (bt[v] > 0.f ? sl[i] : su[i]) * bt[v]);
+                ou.set(v, du[i].get(v) * au + (bt[v] > 0.f ? su[i] : sl[i]) * bt[v]);
+            }
+            slab_store<VEC>(ol, wol, voff, i * step_bytes);
+            slab_store<VEC>(ou, wou, voff, i * step_bytes);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
             Vec<VEC> ol, ou;
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
@@ -260,8 +397,8 @@ __global__ void __launch_bounds__(NTHREADS) softmax_kernel(const SoftmaxArgs a, 
                 ol.set(v, (al > 0.f ? el : eu) * al + (bt[v] > 0.f ? sl[i] : su[i]) * bt[v]);
                 ou.set(v, (au > 0.f ? eu : el) * au + (bt[v] > 0.f ? su[i] : sl[i]) * bt[v]);
             }
-            ol.store(a.olw + base + i * row_step);
-            ou.store(a.ouw + base + i * row_step);
+            slab_store<VEC>(ol, wol, voff, i * step_bytes);
+            slab_store<VEC>(ou, wou, voff, i * step_bytes);
         }
     }
 }
@@ -287,6 +424,7 @@ bool dispatch(const SoftmaxArgs &a, bool vec4, hipStream_t st) {
     const int tpr = 1 << k;
     if (vec4) {
         if ((256 / tpr) * 8 >= a.D) return launch<Q, 4, 256, 8>(a, k, st);
+        if ((512 / tpr) * 8 >= a.D) return launch<Q, 4, 512, 8>(a, k, st);
         if ((1024 / tpr) * 8 >= a.D) return launch<Q, 4, 1024, 8>(a, k, st);
         return false;
     }
