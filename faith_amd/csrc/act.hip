@@ -106,8 +106,7 @@ __device__ __forceinline__ void tanh_pure_lines(float l, float u, Line &lo, Line
 // up in s_ln[0 .. TH) and s_ln[3 TH .. 4 TH) (complete once the barrier inside has been passed), the
 // constant terms in olb / oub.
 template <int TH>
-__device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, float *s_ln,
-                                           const float *__restrict__ p_lb, const float *__restrict__ p_ub, size_t bi,
+__device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, float *s_ln, float lb, float ub, size_t bi,
                                            bool n_ok, int lane, int wv) {
     // three wavefronts share the per-neuron work: 0 = lower tangent search, 1 = upper tangent
     // search (straddling neurons), 2 = tangent / chord of one-signed neurons
@@ -135,7 +134,6 @@ __device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, 
     if (wv == 0 && n_ok) {
         const Line lo = {s_ln[lane], s_ln[TH + lane], s_ln[2 * TH + lane]};
         const Line up = {s_ln[3 * TH + lane], s_ln[4 * TH + lane], s_ln[5 * TH + lane]};
-        const float lb = p_lb[bi], ub = p_ub[bi];
         a.olb[bi] = line_bias(lo, lb, ub);
         a.oub[bi] = line_bias(up, ub, lb);
     }
@@ -145,13 +143,15 @@ __device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, 
 // in `part` ([words][NW][2][TH]) and a barrier: one lane per neuron (wavefront 0) finishes the
 // norms and concretizes; the slopes of the two lines end up in s_ln[0 .. TH) and s_ln[3 TH .. 4 TH),
 // the constant terms in olb / oub.  Ends with a barrier (except for CONCRETIZE).
+// lb0 / ub0: the neuron's constant terms (lanes of wavefront 0 with n_ok), which the caller fetches before it
+// loads its coefficients: fetched here they would be one more memory latency between the loads and the stores of
+// every tile.
 template <int MODE, int Q, int NW, int TH>
-__device__ __forceinline__ void neuron_stage(const ActArgs &a, const float *part, float *s_lu, float *s_ln,
-                                             const float *__restrict__ p_lb, const float *__restrict__ p_ub,
-                                             float *__restrict__ p_l, float *__restrict__ p_u, size_t bi, bool n_ok,
-                                             int lane, int wv) {
+__device__ __forceinline__ void neuron_stage(const ActArgs &a, const float *part, float *s_lu, float *s_ln, float lb0,
+                                             float ub0, float *__restrict__ p_l, float *__restrict__ p_u, size_t bi,
+                                             bool n_ok, int lane, int wv) {
     if (wv == 0 && n_ok) {
-        float l = p_lb[bi], u = p_ub[bi];
+        float l = lb0, u = ub0;
         for (int w = 0; w < a.words; ++w) {
             float nl = 0.f, nu = 0.f;
 #pragma unroll
@@ -166,7 +166,7 @@ __device__ __forceinline__ void neuron_stage(const ActArgs &a, const float *part
         if (p_u) p_u[bi] = u;
         if (MODE != TANH && MODE != CONCRETIZE) {
             float klo, kup, olb, oub;
-            relax_point<MODE>(l, u, p_lb[bi], p_ub[bi], klo, kup, olb, oub);
+            relax_point<MODE>(l, u, lb0, ub0, klo, kup, olb, oub);
             s_ln[lane] = klo;
             s_ln[3 * TH + lane] = kup;
             a.olb[bi] = olb;
@@ -179,7 +179,7 @@ __device__ __forceinline__ void neuron_stage(const ActArgs &a, const float *part
     if (MODE == CONCRETIZE) return;
     __syncthreads();
 
-    if (MODE == TANH) tanh_stage<TH>(a, s_lu, s_ln, p_lb, p_ub, bi, n_ok, lane, wv);
+    if (MODE == TANH) tanh_stage<TH>(a, s_lu, s_ln, lb0, ub0, bi, n_ok, lane, wv);
 }
 
 // TPR threads cover one row of the tile (TH = TPR * VEC neurons); RG = NTHREADS / TPR rows are
@@ -216,6 +216,15 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     const int blk = a.D / a.words;
     constexpr int CHUNK = RG * RPT;
     const int nchunks = (a.D + CHUNK - 1) / CHUNK;
+
+    const int column = col0 + lane;
+    const bool n_ok = lane < TH && column < H;
+    const size_t bi = (size_t)r * H + column;
+    float lb0 = 0.f, ub0 = 0.f;
+    if (wv == 0 && n_ok) {
+        lb0 = p_lb[bi];
+        ub0 = p_ub[bi];
+    }
 
     Vec<VEC> dl[RPT], du[RPT];
     // concretize only: an upper interval nobody asked for (the first operand of a dot product: its planes
@@ -287,10 +296,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     }
     __syncthreads();
 
-    const int column = col0 + lane;
-    const bool n_ok = lane < TH && column < H;
-    const size_t bi = (size_t)r * H + column;
-    neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, p_lb, p_ub, p_l, p_u, bi, n_ok, lane, wv);
+    neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, lb0, ub0, p_l, p_u, bi, n_ok, lane, wv);
     if (MODE == CONCRETIZE) return;
 
     if (!col_ok) return;
@@ -346,6 +352,12 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
     const size_t base = ((size_t)r * a.D + rg) * a.H + col0 + c * VEC;
     const size_t row_step = (size_t)RG * a.H;
     const float *__restrict__ p_lw = a.lw + base, *__restrict__ p_uw = a.uw + base;
+    const size_t bi = (size_t)r * a.H + col0 + lane;
+    float lb0 = 0.f, ub0 = 0.f;
+    if (wv == 0 && lane < TH) {
+        lb0 = a.lb[bi];
+        ub0 = a.ub[bi];
+    }
 
     Vec<VEC> dl[RPT], du[RPT];
 #pragma unroll
@@ -398,8 +410,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
     }
     __syncthreads();
 
-    const size_t bi = (size_t)r * a.H + col0 + lane;
-    neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, a.lb, a.ub, a.l, a.u, bi, lane < TH, lane, wv);
+    neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, lb0, ub0, a.l, a.u, bi, lane < TH, lane, wv);
     if (MODE == CONCRETIZE) return;
 
     float klo[VEC], kup[VEC];
@@ -422,6 +433,131 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
             ol.store(q_lw + i * row_step);
             ou.store(q_uw + i * row_step);
         }
+    }
+}
+
+// The same tile on a persistent workgroup: the grid is sized to the machine, a workgroup walks tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ... and holds TWO tiles in registers -- the loads of the next tile are issued
+// before the norms, the per-neuron stage and the stores of the current one.  The first round of one-tile workgroups
+// all load, then all compute, then all store, and memory sits idle at every change of phase (it shows when nothing
+// is cached: the phases are then memory latencies apart); here reads and writes are in flight together from the
+// second tile on, as in a copy.  Arithmetic per tile is that of act_resident, bit for bit.
+// The tile's LDS (partial norms, intervals, lines) is reused from tile to tile: whoever writes `part` for the next
+// tile has read its slopes of this one, and the per-neuron stage writes lines only after the barrier that follows
+// those writes.
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE))) act_pipelined(const ActArgs a, const int n_tiles) {
+    static_assert(MODE != CONCRETIZE, "a read-only pass has no phases to overlap");
+    constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
+    static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
+    extern __shared__ float smem[];
+    float *part = smem;                           // [words][NW][2][TH] per-wavefront partial norms
+    float *s_lu = part + a.words * NW * 2 * TH;   // [2][TH] concrete interval
+    float *s_ln = s_lu + 2 * TH;                  // [2][3][TH] lower / upper line (k, x0, y0)
+
+    const int tiles = a.H / TH;
+    const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
+    const int c = tid % TPR, rg = tid / TPR;
+    const size_t row_step = (size_t)RG * a.H;
+    const int blk = a.D / a.words;
+
+    struct Tile {
+        Vec<VEC> dl[RPT], du[RPT];
+        float lb0, ub0;
+    };
+    auto base_of = [&](int t) { return ((size_t)(t / tiles) * a.D + rg) * a.H + (t % tiles) * TH + c * VEC; };
+    auto bias_of = [&](int t) { return (size_t)(t / tiles) * a.H + (t % tiles) * TH + lane; };
+    auto fetch = [&](int t, Tile &x) __attribute__((always_inline)) {
+        x.lb0 = x.ub0 = 0.f;
+        if (wv == 0 && lane < TH) {
+            x.lb0 = a.lb[bias_of(t)];
+            x.ub0 = a.ub[bias_of(t)];
+        }
+        const float *__restrict__ p_lw = a.lw + base_of(t), *__restrict__ p_uw = a.uw + base_of(t);
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            if (i * RG < a.D) {
+                x.dl[i].load(p_lw + i * row_step);
+                x.du[i].load(p_uw + i * row_step);
+            } else {
+                x.dl[i].zero();
+                x.du[i].zero();
+            }
+        }
+    };
+    auto finish = [&](int t, Tile &x) __attribute__((always_inline)) {
+        for (int w = 0; w < a.words; ++w) {
+            const int lo_row = w * blk, hi_row = lo_row + blk;
+            float pl[VEC], pu[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                const int row = i * RG + rg;
+                if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        pl[v] = nacc<Q>(pl[v], x.dl[i].get(v), a.qv);
+                        pu[v] = nacc<Q>(pu[v], x.du[i].get(v), a.qv);
+                    }
+                }
+            }
+#pragma unroll
+            for (int m = TPR; m < WAVE; m <<= 1) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    pl[v] = ncomb<Q>(pl[v], __shfl_xor(pl[v], m, WAVE));
+                    pu[v] = ncomb<Q>(pu[v], __shfl_xor(pu[v], m, WAVE));
+                }
+            }
+            if (lane < TPR) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    part[((w * NW + wv) * 2 + 0) * TH + c * VEC + v] = pl[v];
+                    part[((w * NW + wv) * 2 + 1) * TH + c * VEC + v] = pu[v];
+                }
+            }
+        }
+        __syncthreads();
+        neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, x.lb0, x.ub0, a.l, a.u, bias_of(t), lane < TH, lane, wv);
+        float klo[VEC], kup[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            klo[v] = s_ln[c * VEC + v];
+            kup[v] = s_ln[3 * TH + c * VEC + v];
+        }
+        float *__restrict__ q_lw = a.olw + base_of(t), *__restrict__ q_uw = a.ouw + base_of(t);
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            if (i * RG < a.D) {
+                Vec<VEC> ol, ou;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    const float xl = x.dl[i].get(v), xu = x.du[i].get(v);
+                    ol.set(v, (klo[v] > 0.f ? xl : xu) * klo[v]);
+                    ou.set(v, (kup[v] > 0.f ? xu : xl) * kup[v]);
+                }
+                ol.store(q_lw + i * row_step);
+                ou.store(q_uw + i * row_step);
+            }
+        }
+    };
+
+    Tile A, B;
+    int t = blockIdx.x;
+    if (t >= n_tiles) return;
+    fetch(t, A);
+    while (true) {
+        int tn = t + gridDim.x;
+        if (tn < n_tiles) fetch(tn, B);
+        finish(t, A);
+        if (tn >= n_tiles) break;
+        t = tn;
+        tn = t + gridDim.x;
+        if (tn < n_tiles) fetch(tn, A);
+        finish(t, B);
+        if (tn >= n_tiles) break;
+        t = tn;
     }
 }
 
@@ -541,6 +677,18 @@ void launch_resident(const ActArgs &a, hipStream_t st) {
                        smem, st, a);
 }
 
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE>
+void launch_pipelined(const ActArgs &a, hipStream_t st) {
+    constexpr int TH = TPR * 4;
+    const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
+    faith::reserve_lds(act_pipelined<MODE, Q, TPR, NTHREADS, RPT, WPE>, smem);
+    const int n_tiles = a.rows * (a.H / TH);
+    // as many workgroups as are resident at once (WPE wavefronts per SIMD), no more than there are tiles
+    const int resident = faith::compute_units() * (4 * WPE / (NTHREADS / WAVE));
+    hipLaunchKernelGGL((act_pipelined<MODE, Q, TPR, NTHREADS, RPT, WPE>), dim3((unsigned)std::min(n_tiles, resident)), dim3(NTHREADS),
+                       smem, st, a, n_tiles);
+}
+
 // Transposed layout, D_in = 256 V (V = 1, 2), 16-byte aligned: a wavefront owns 8 / V neurons, one
 // 16-byte load per lane covers 256 coefficients of a neuron's contiguous row, and everything a
 // wavefront reads (64 values per thread) stays in registers between the norm and the scaling: one
@@ -625,7 +773,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) a
         }
         __syncthreads();
         const long long first = (long long)blockIdx.x * NPB;
-        tanh_stage<NPB>(a, s_lu, s_ln, a.lb, a.ub, (size_t)(first + lane), lane < NPB && first + lane < total, lane, wv);
+        const bool mine = lane < NPB && first + lane < total;
+        const float lb0 = (wv == 0 && mine) ? a.lb[first + lane] : 0.f, ub0 = (wv == 0 && mine) ? a.ub[first + lane] : 0.f;
+        tanh_stage<NPB>(a, s_lu, s_ln, lb0, ub0, (size_t)(first + lane), mine, lane, wv);
         if (lane < NPW) {
             klo = s_ln[wv * NPW + lane];
             kup = s_ln[3 * NPB + wv * NPW + lane];
@@ -706,16 +856,28 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
     // straight-line kernel for the common shape: 32-neuron tiles, 32 rows in flight, up to 8 rows a thread
     const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
     if (tv != 9 && a.rows2 == 0 && a.H % 32 == 0 && a.D % 32 == 0 && a.D <= 256) {
-        // Two thread shapes for the 256-row tile.  Four wavefronts holding eight rows each are 5 % ahead
-        // while the operands can sit in the 256 MB memory-side cache (40.2 against 42.8 us at
-        // [128, 256, 512], every launch on the same 269 MB); sixteen wavefronts holding two rows each are
-        // 12 % ahead when every byte comes from and goes to HBM (55 against 62 us on the same shape with
-        // five operand sets in turn), and 3 % more with non-temporal loads (54 us; those cost 25 % when the
-        // operands are cached).  An object whose traffic exceeds the cache by more than a quarter cannot be
-        // resident, so it takes the second shape; knob values 7 / 8 force one or the other, 12 the second
-        // without the non-temporal loads (the middle: relu 42.4 us warm / 55.1 us cold, tanh 45.8 / 58.0).
+        // Thread shapes for the 256-row tile, on [128, 256, 512] (269 MB per launch) with every launch on the same
+        // operands (they can sit in the 256 MB memory-side cache: "warm") and with five operand sets in turn
+        // (every byte from and to HBM: "cold"), relu / tanh in us:
+        //   one tile per workgroup, 4 wavefronts x 8 rows            warm 41.5 / 40.3   cold 61 - 65 / 61 - 65
+        //   one tile per workgroup, 16 wavefronts x 2 rows           warm 44.5 / 49.6   cold 54 - 56 / 57 - 58
+        //   the same with non-temporal loads                         warm 54.7 / 56.9   cold 55.3 / 57.9
+        //   persistent, two tiles in registers, 4 wavefronts x 8     warm 41.8 / 43.8   cold 55 - 57 / 58 - 60
+        // The persistent kernel is the one that is good at both, except for tanh, whose long per-neuron stage
+        // wants more workgroups on a CU than its registers allow: tanh keeps the first shape while its operands can
+        // be cached and takes the third when they cannot (traffic more than a quarter beyond the cache).
+        // Knob values 8 / 12 / 7 force the three one-tile shapes, 15 the persistent one.
         const long long traffic = 16LL * a.rows * a.D * a.H;
         const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 5LL * (256LL << 20) / 4);
+        bool pipelined = false;
+        if constexpr (MODE != CONCRETIZE) {
+            // (with fewer than two tiles per resident workgroup there is nothing to overlap: one tile each then)
+            const long long n_tiles = (long long)a.rows * (a.H / 32);
+            pipelined = a.D > 128 && (tv == 15 || (MODE != TANH && tv != 7 && tv != 8 && tv != 12 &&
+                                                   n_tiles >= 4LL * faith::compute_units()));
+            if (pipelined) launch_pipelined<MODE, Q, 8, 256, 8, 2>(a, st);
+        }
+        if (pipelined) return;
         if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(a, st);
         else if (tv == 12) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(a, st);
         else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(a, st);

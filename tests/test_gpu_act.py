@@ -107,6 +107,46 @@ def test_thread_shape_for_hbm_streams_gives_the_same_values(kind, p):
         assert close(a, b.cpu())
 
 
+@pytest.mark.parametrize("kind,p", [("relu", 2.0), ("relu", INF), ("exp", 1.0), ("sqr", 2.0), ("tanh", 2.0)])
+@pytest.mark.parametrize("rows", [40, 43])
+def test_persistent_two_tile_kernel_gives_the_one_tile_kernels_bits(kind, p, rows):
+    """An object with at least four 32-neuron tiles per CU runs every relaxation but tanh on persistent workgroups that
+    hold the next tile while they finish the current one (tuning knob 15 forces that kernel, 8 the one-tile kernel):
+    the arithmetic per tile is the same, so the results are, bit for bit -- also when the tiles do not divide
+    evenly among the workgroups (43 rows) -- and three rows of them are checked against the oracle."""
+    from faith_amd import _lib, ops
+    g = torch.Generator(device="cuda").manual_seed(12)
+    shape = (1, rows, 256, 1024)
+    lw = torch.empty(shape, device="cuda").normal_(0, 0.05, generator=g)
+    uw = torch.empty(shape, device="cuda").normal_(0, 0.005, generator=g).abs_().add_(lw)
+    lb = torch.empty((1, rows, 1024), device="cuda").normal_(0, 1, generator=g)
+    ub = torch.empty((1, rows, 1024), device="cuda").normal_(0, 0.5, generator=g).abs_().add_(lb)
+    if kind in ("sqr",):
+        lb, ub = lb.abs() + 1.0, ub.abs() + 2.5
+        lb, ub = torch.minimum(lb, ub), torch.maximum(lb, ub)
+    print(f"[case] persistent kernel {kind} p={p} rows={rows}", flush=True)
+    fn = getattr(ops, kind)
+    by_default = fn(lw, lb, uw, ub, p, 0.01, 2, return_interval=True)
+    results = {}
+    for knob in (8, 15):
+        _lib.call("faith_tune_set", 0, knob)
+        try:
+            results[knob] = fn(lw, lb, uw, ub, p, 0.01, 2, return_interval=True)
+        finally:
+            _lib.call("faith_tune_set", 0, 0)
+    torch.cuda.synchronize()
+    for name, d, one, two in zip(("lw", "lb", "uw", "ub", "l", "u"), by_default, results[8], results[15]):
+        assert torch.equal(one, two), f"{kind} {name}: the persistent kernel differs from the one-tile kernel"
+        assert torch.equal(d, one), f"{kind} {name}: the default differs from the one-tile kernel"
+    for r in (0, rows // 2, rows - 1):
+        x = O.LinearBounds(*(t[:, r:r + 1].cpu() for t in (lw, lb, uw, ub)))
+        exp = getattr(O, kind)(x, p, 0.01, 2)
+        l_ref, u_ref = O.concretize(x, p, 0.01, 2)
+        got = tuple(t[:, r:r + 1].cpu() for t in by_default)
+        rep = compare_activation(kind, x, got[:4], exp.tensors(), got[4], got[5], l_ref, u_ref)
+        print("   ", rep, flush=True)
+
+
 @pytest.mark.parametrize("kind", ["relu", "tanh"])
 def test_activation_reference_test_distribution(kind):
     """Inputs drawn as the reference's own op test draws them
