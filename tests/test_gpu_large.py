@@ -71,7 +71,8 @@ def sl(x, r):
 
 @pytest.mark.parametrize("op,p,layout,shape", [
     ("relu", 2.0, "natural", (2100, 1024, 1024)),       # D_in = 1024: rows in the registers of sixteen wavefronts
-    ("tanh", INF, "natural", (8200, 256, 1024)),        # register-resident kernel
+    ("tanh", INF, "natural", (8200, 256, 1024)),        # register-resident kernel, one tile per workgroup
+    ("relu", 2.0, "natural", (8200, 256, 1024)),        # register-resident kernel, persistent workgroups
     ("relu", 1.0, "natural", (300, 2048, 3600)),        # chunked walk (D_in > 1024), two reads
     ("tanh", 2.0, "transposed", (2100, 4096, 256)),     # transposed, resident (D_in = 256)
     ("relu", INF, "transposed", (2100, 1000, 1040)),    # transposed, general kernel
@@ -84,13 +85,14 @@ def test_relaxation_rows(op, p, layout, shape):
     fn = getattr(ops, op)
     full = fn(*x, p, 0.01, 2, lay, True)
     picks = rows_to_check(L, A * B)
-    # an object of this size streams from HBM and takes the register-resident kernel's sixteen-wavefront
-    # thread shape; a single row would take the four-wavefront one (another reduction tree), so the slices
-    # are held to the shape of the whole (tuning knob 7) and the comparison stays bit for bit
+    # an object of this size streams from HBM: tanh then takes the register-resident kernel's sixteen-wavefront
+    # thread shape, where a single row would take the four-wavefront one (another reduction tree), so the slices
+    # are held to the shape of the whole (tuning knob 7) and the comparison stays bit for bit; relu runs on
+    # persistent workgroups with the arithmetic of the four-wavefront shape (knob 8 for the slices)
     from faith_amd import _lib
     resident = layout == "natural" and A <= 256
     if resident:
-        _lib.call("faith_tune_set", 0, 7)
+        _lib.call("faith_tune_set", 0, 7 if op == "tanh" else 8)
     try:
         check_rows(f"{op} {layout}", full, lambda r: fn(*sl(x, r), p, 0.01, 2, lay, True), picks)
     finally:
