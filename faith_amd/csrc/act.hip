@@ -583,17 +583,33 @@ __device__ __forceinline__ void relax_any(float l, float u, float lb, float ub, 
 }
 
 // ------------------------------------------------------------------ transposed layout
+// Butterfly over the 64 lanes, every lane ends with the total.  Distances 1 to 8 are lane permutations inside a
+// row of 16 lanes, done by the vector ALU on its own operand (DPP) instead of a trip through the LDS crossbar: 1 and
+// 2 as permutations of four lanes; after them the four lanes of a group hold one value, so mirroring eight lanes
+// fetches what lane ^ 4 holds, and after that mirroring sixteen fetches what lane ^ 8 holds.  16 and 32 go through
+// the crossbar.
+template <int CTRL>
+__device__ __forceinline__ float lane_permute(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
+    v += lane_permute<0xB1>(v);       // lanes 1 0 3 2
+    v += lane_permute<0x4E>(v);       // lanes 2 3 0 1
+    v += lane_permute<0x141>(v);      // eight lanes mirrored
+    v += lane_permute<0x140>(v);      // sixteen lanes mirrored
+    v += __shfl_xor(v, 16, WAVE);
+    v += __shfl_xor(v, 32, WAVE);
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int m = WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
+    v = fmaxf(v, lane_permute<0xB1>(v));
+    v = fmaxf(v, lane_permute<0x4E>(v));
+    v = fmaxf(v, lane_permute<0x141>(v));
+    v = fmaxf(v, lane_permute<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+    v = fmaxf(v, __shfl_xor(v, 32, WAVE));
     return v;
 }
-
 // 256 threads, 64 neurons per workgroup: each wavefront reduces 16 neurons (lanes along D_in,
 // cross-lane butterfly), wavefront 0 then derives the 64 pairs of lines (one neuron per lane),
 // and each wavefront scales its 16 neurons (second read comes from L2).
