@@ -270,14 +270,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
                 }
             }
             // lanes of one wavefront that share a column: butterfly over the row groups
-#pragma unroll
-            for (int m = TPR; m < WAVE; m <<= 1) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                    pl[v] = ncomb<Q>(pl[v], __shfl_xor(pl[v], m, WAVE));
-                    pu[v] = ncomb<Q>(pu[v], __shfl_xor(pu[v], m, WAVE));
-                }
-            }
+            combine_from<Q, TPR>(pl, pu);
             if (lane < TPR) {
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
@@ -392,14 +385,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
                 }
             }
         }
-#pragma unroll
-        for (int m = TPR; m < WAVE; m <<= 1) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-                pl[v] = ncomb<Q>(pl[v], __shfl_xor(pl[v], m, WAVE));
-                pu[v] = ncomb<Q>(pu[v], __shfl_xor(pu[v], m, WAVE));
-            }
-        }
+        combine_from<Q, TPR>(pl, pu);
         if (lane < TPR) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
@@ -502,14 +488,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
                     }
                 }
             }
-#pragma unroll
-            for (int m = TPR; m < WAVE; m <<= 1) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                    pl[v] = ncomb<Q>(pl[v], __shfl_xor(pl[v], m, WAVE));
-                    pu[v] = ncomb<Q>(pu[v], __shfl_xor(pu[v], m, WAVE));
-                }
-            }
+            combine_from<Q, TPR>(pl, pu);
             if (lane < TPR) {
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
@@ -588,10 +567,6 @@ __device__ __forceinline__ void relax_any(float l, float u, float lb, float ub, 
 // 2 as permutations of four lanes; after them the four lanes of a group hold one value, so mirroring eight lanes
 // fetches what lane ^ 4 holds, and after that mirroring sixteen fetches what lane ^ 8 holds.  16 and 32 go through
 // the crossbar.
-template <int CTRL>
-__device__ __forceinline__ float lane_permute(float x) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
-}
 __device__ __forceinline__ float wave_sum(float v) {
     v += lane_permute<0xB1>(v);       // lanes 1 0 3 2
     v += lane_permute<0x4E>(v);       // lanes 2 3 0 1

@@ -36,6 +36,37 @@ __device__ __forceinline__ float nfin(float a, float qv) {
     return Q == FAITH_Q_2 ? sqrtf(a) : a;
 }
 
+// ------------------------------------------------------------------ cross-lane exchange
+// The value another lane of the same row of 16 lanes holds; CTRL is the permutation (a DPP control word).  The
+// vector ALU applies it to its own operand: no trip through the LDS crossbar, which every ds_bpermute of a CU shares.
+template <int CTRL>
+__device__ __forceinline__ float lane_permute(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+// What lane ^ M holds.  M = 1, 2 (permutations of four lanes) and 8 (a row of 16 rotated by 8) are lane
+// permutations; 4, 16 and 32 go through the crossbar.
+template <int M>
+__device__ __forceinline__ float lane_xor(float x) {
+    if constexpr (M == 1) return lane_permute<0xB1>(x);
+    else if constexpr (M == 2) return lane_permute<0x4E>(x);
+    else if constexpr (M == 8) return lane_permute<0x128>(x);
+    else return __shfl_xor(x, M, WAVE);
+}
+// Butterfly over the lanes that are M, 2 M, ... 32 apart (the lanes of a wavefront that hold the same columns when
+// FIRST threads cover a row), for 2 N partial norms.
+template <int Q, int FIRST, int N>
+__device__ __forceinline__ void combine_from(float (&a)[N], float (&b)[N]) {
+#define FAITH_STEP(M)                                          \
+    if constexpr (FIRST <= M) {                                \
+        _Pragma("unroll") for (int i = 0; i < N; ++i) {        \
+            a[i] = ncomb<Q>(a[i], lane_xor<M>(a[i]));          \
+            b[i] = ncomb<Q>(b[i], lane_xor<M>(b[i]));          \
+        }                                                      \
+    }
+    FAITH_STEP(1) FAITH_STEP(2) FAITH_STEP(4) FAITH_STEP(8) FAITH_STEP(16) FAITH_STEP(32)
+#undef FAITH_STEP
+}
+
 // ------------------------------------------------------------------ vector access
 // Stores are non-temporal: lw' / uw' are written once and not read again by this kernel, and
 // keeping them out of the cache's way measured 11 % faster at configuration 1 (loads are left

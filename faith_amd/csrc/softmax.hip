@@ -37,11 +37,6 @@ typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t slab_window(const float *base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)bytes, 0x00020000);
 }
-// the value another lane of the same row of 16 lanes holds; CTRL is the permutation (a DPP control word)
-template <int CTRL>
-__device__ __forceinline__ float lane_permute(float x) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
-}
 // One butterfly step at distance m for 2 N values through the LDS crossbar, the 2 N exchanges in flight together.
 // (The swap instructions v_permlane16_swap / v_permlane32_swap do distances 16 and 32 on the vector ALU, but with
 // the copies and wait states they need they measured slower here: 63.7 against 61.8 us on a [256 x 128] slab.)
