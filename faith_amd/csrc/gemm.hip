@@ -574,12 +574,13 @@ static void choose_tile(long long mw, int dim_out, int dim_y_out, int *tm, int *
     auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * ((dim_y_out + n - 1) / n); };
     const long long cus = faith::compute_units();
     // tiny problems want the most workgroups (64 x 64); up to two 128 x 64 tiles per CU that shape is up to 17 %
-    // ahead; 128 x 128 pays only for long reductions on problems of many tiles per CU (configuration 2: 1 % ahead)
-    // -- with K <= 512 the pro- and epilogues of five small co-resident workgroups overlap better than those of two
-    // large ones (2 - 6 % at 65536 ... 245760 rows)
+    // ahead; 128 x 128 (the most MFMAs per staged operand) pays once there are a dozen of its tiles per CU, whatever
+    // the reduction length: 2 - 5 % at 131072 ... 245760 rows with K and N of 256 ... 768 (the batched propagation of
+    // a sentence's positions), level at 8 tiles per CU, behind below that, where the pro- and epilogues of five
+    // small co-resident workgroups overlap better than those of two large ones
     if (tiles(64, 64) <= cus) { *tm = 64; *tn = 64; }
     else if (tiles(128, 64) <= 2 * cus) { *tm = 128; *tn = 64; }
-    else if (dim_out >= 1024 && tiles(128, 128) >= 16 * cus) { *tm = 128; *tn = 128; }
+    else if (tiles(128, 128) >= 12 * cus) { *tm = 128; *tn = 128; }
     // many column tiles re-read every block of rows from L2: the large tile halves that (3 - 5 % at
     // 768 -> 3072 and 512 -> 2048 with 12288 ... 24576 rows) once it fills the machine four times over
     else if (dim_y_out >= 2048 && tiles(128, 128) >= 8 * cus) { *tm = 128; *tn = 128; }
