@@ -14,38 +14,47 @@ names the reference lines it follows.  Tensor convention (Bounds.py:293-297):
 A neuron (b, l, j) is bounded by  lw[b,l,:,j] . delta + lb[b,l,j]  from below
 and  uw[b,l,:,j] . delta + ub[b,l,j]  from above, for ||delta||_p <= eps.
 
-Parity status of each function (what pins it, see tests/test_oracle_*.py):
-  concretize   pinned: numpy.linalg.norm, one-hot and zero special cases,
+Parity status of each function (what pins it; tests/test_oracle_*.py, tests/test_reference_vectors.py,
+tests/test_bounds_reference_vectors.py):
+  Every function below except conv is pinned BY EXECUTION OF THE REFERENCE: tests/golden/
+  bounds_reference_vectors.npz holds what the reference's own Bounds class returns
+  (Verifiers/Bounds.py run once in the build container by tests/golden/make_bounds_golden.py,
+  without its six top-level statements that need tvm and nvcc and with nothing in their place)
+  for tanh, relu, exp, sqr, sqrt, reciprocal, multiply, divide, softmax, layer_norm (both
+  modes), concretize, dot_product, context, matmul, scalar multiply and add, at p in {1, 2, inf}
+  with one and two perturbed words, on inputs with every branch and crafted edge neurons
+  (l = 0, u = 0, |u| = |l|, a point, a tiny and a wide interval); tests/golden/
+  reference_vectors.npz holds the same for relu, matmul, concretize and dot_product from the
+  pure-torch files of HandTunedKernels/python_reference_code.  This module reproduces all of
+  them at rtol 1e-5 / atol 1e-6, and mutations of the free choices (nine bisection steps,
+  another tangent point for exp, [|u| >= |l|], beta_u = u_x) miss them.  In addition:
+  concretize   numpy.linalg.norm, one-hot and zero special cases,
                block-sum identity for perturbed_words > 1.
-  linear       pinned: brute-force triple loop, W>=0 / lw==uw closed forms,
+  linear       brute-force triple loop, W>=0 / lw==uw closed forms,
                (uw'-lw') == (uw-lw)@|W| identity.
-  relu         pinned: independent fp64 per-neuron closed form
+  relu         independent fp64 per-neuron closed form
                (oracle/closed_form.py), branch invariants, sampled soundness.
-  tanh         pinned: independent fp64 scalar loop, odd symmetry, sampled
+  tanh         independent fp64 scalar loop, odd symmetry, sampled
                soundness, and tangency: the lines touch the curve at the
-               point the bisection returns, to the resolution of ten halvings
-               (pins the sign test and the bracket update order).  The exact
-               number of steps is pinned by text only (Bounds.py:1063-1097
-               cannot be imported: the module needs tvm and nvcc at import
-               time).
+               point the bisection returns, to the resolution of ten halvings.
   exp, reciprocal, sqr, sqrt
-               pinned: independent fp64 per-neuron closed forms, sampled soundness
+               independent fp64 per-neuron closed forms, sampled soundness
                (lower line <= f <= upper line on [l, u]).
   scale, add   one-line tensor identities (checked against their definition).
-  multiply     pinned: the brute-force McCormick loop with a reduction of length 1.
+  multiply     the brute-force McCormick loop with a reduction of length 1.
   divide, softmax, layer_norm
-               compositions of pinned parts, in the reference's order; pinned as wholes
-               by sampled soundness (the true softmax / layer norm of any admissible
-               input lies between the propagated lines).
-  dot_product  pinned: brute-force five-deep loop on tiny shapes, einsum
+               compositions of the parts above, in the reference's order; sampled soundness
+               (the true softmax / layer norm of any admissible input lies between the
+               propagated lines).
+  dot_product  brute-force five-deep loop on tiny shapes, einsum
                restatement, sampled soundness of the McCormick planes.
-  context      the same function on transposed views; pinned by the brute-force loop
+  context      the same function on transposed views; the brute-force loop
                fed with explicitly transposed numpy arrays.
-  conv         pinned: brute-force loops, 1x1 conv == linear, F.conv2d
-               linearity.  The reference has NO Python conv bound; semantics
+  conv         NOT pinned by execution: the reference has NO Python conv bound; semantics
                come from HandTunedKernels/convolution_verification.cu:124-138
                and its launcher :219-239 (two launches: b with batch 1, w with
-               batch = D_in).
+               batch = D_in), which needs nvcc.  Pinned by brute-force loops,
+               1x1 conv == linear, F.conv2d linearity.
 """
 from __future__ import annotations
 
