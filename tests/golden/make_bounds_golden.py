@@ -61,8 +61,8 @@ def load_reference_bounds():
     return space["Bounds"]
 
 
-def args(words):
-    return types.SimpleNamespace(method="baf", perturbed_words=words, current_flag=0, kernel_type=0)
+def args(words, method="baf"):
+    return types.SimpleNamespace(method=method, perturbed_words=words, current_flag=0, kernel_type=0)
 
 
 def draw(g, L, D, H, sw=0.3, sb=1.0, gw=0.05, gb=0.4, positive=False):
@@ -165,6 +165,39 @@ def main():
     keep("scale_pos", ref(x, 2.0, 0.1, 1).multiply(1.3))
     keep("add_bounds", ref(x, 2.0, 0.1, 1).add(ref(x2, 2.0, 0.1, 1)))
     keep("add_vector", ref(x, 2.0, 0.1, 1).add(bias))
+
+    # ---- method "ibp" (interval bound propagation: the `if self.ibp` branches, Bounds.py:285-288, 863, 896, 973,
+    # 1030, 1139 and the matmul / layer_norm that serve both methods).  Its relu, get_bounds_xy (product, dot
+    # product) and whatever composes them call `.cuda()` on constants (Bounds.py:230, 676, 925) and cannot run in a
+    # container without a GPU: those stay pinned by their closed forms (max(., 0); the range of the four corners).
+    Li, Hi = 4, 24
+    ilb = torch.randn(1, Li, Hi, generator=g)
+    iub = ilb + torch.rand(1, Li, Hi, generator=g) * 0.6
+    plb = torch.randn(1, Li, Hi, generator=g).abs() + 0.5
+    pub = plb + torch.rand(1, Li, Hi, generator=g) * 0.6
+    out["ibp_in_lb"], out["ibp_in_ub"] = ilb.numpy(), iub.numpy()
+    out["ibp_pos_in_lb"], out["ibp_pos_in_ub"] = plb.numpy(), pub.numpy()
+    Wi = torch.randn(16, Hi, generator=g) / 4
+    out["ibp_W"] = Wi.numpy()
+    iw = 1 + 0.1 * torch.randn(Hi, generator=g)
+    iw[2] = -0.6
+    ib = 0.05 * torch.randn(Hi, generator=g)
+    out["ibp_norm_weight"], out["ibp_norm_bias"] = iw.numpy(), ib.numpy()
+
+    def interval_object(lb, ub):
+        zeros = torch.zeros(1, Li, 2 * Hi, Hi)             # the constructor keeps `perturbed_words` rows of it
+        return Bounds(args(2, "ibp"), 2.0, 0.1, lw=zeros, lb=lb.clone(), uw=zeros.clone(), ub=ub.clone())
+
+    def keep_interval(tag, y):
+        assert float(y.lw.abs().max()) == 0.0 and float(y.uw.abs().max()) == 0.0
+        out[f"ibp_{tag}_lb"], out[f"ibp_{tag}_ub"] = y.lb.numpy(), y.ub.numpy()
+
+    for kind in ("tanh", "exp", "sqr"):
+        keep_interval(kind, getattr(interval_object(ilb, iub), kind)())
+    for kind in ("sqrt", "reciprocal"):
+        keep_interval(kind, getattr(interval_object(plb, pub), kind)())
+    keep_interval("matmul", interval_object(ilb, iub).matmul(Wi))
+    keep_interval("layernorm_novar", interval_object(ilb, iub).layer_norm(types.SimpleNamespace(weight=iw, bias=ib), "no_var"))
 
     path = os.path.join(HERE, "bounds_reference_vectors.npz")
     np.savez_compressed(path, **out)

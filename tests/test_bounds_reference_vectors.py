@@ -175,3 +175,57 @@ def test_hip_affine_operators_match_the_reference():
     assert_matches(quad(x.multiply(1.3)), "scale_pos", "multiply(1.3)")
     assert_matches(quad(x.add(gpu_bounds("any2_in", 2.0, EPS, 1))), "add_bounds", "add(Bounds)")
     assert_matches(quad(x.add(t(G["norm_bias"]).cuda())), "add_vector", "add(vector)")
+
+
+# ------------------------------------------------------------------------------------------
+# method "ibp": the reference's interval branches, executed (its relu, product and dot product call .cuda() on
+# constants and could not be run where the vectors were written; tests/test_ibp.py pins those by their closed forms)
+# ------------------------------------------------------------------------------------------
+IBP_UNARY = {"tanh": "ibp_in", "exp": "ibp_in", "sqr": "ibp_in", "sqrt": "ibp_pos_in", "reciprocal": "ibp_pos_in"}
+
+
+def interval_object(tag):
+    lb, ub = t(G[f"{tag}_lb"]), t(G[f"{tag}_ub"])
+    zeros = torch.zeros(1, lb.shape[1], 2, lb.shape[2])
+    return O.LinearBounds(zeros, lb, zeros.clone(), ub)
+
+
+def assert_interval(lo, hi, tag, what, rtol=RTOL, atol=ATOL):
+    np.testing.assert_allclose(lo.detach().cpu().numpy(), G[f"ibp_{tag}_lb"], rtol=rtol, atol=atol, err_msg=f"{what} lower")
+    np.testing.assert_allclose(hi.detach().cpu().numpy(), G[f"ibp_{tag}_ub"], rtol=rtol, atol=atol, err_msg=f"{what} upper")
+
+
+@pytest.mark.parametrize("kind", list(IBP_UNARY))
+def test_oracle_interval_operators_match_the_reference(kind):
+    x = interval_object(IBP_UNARY[kind])
+    assert_interval(*O.interval_unary(kind, x.lb, x.ub), kind, f"ibp {kind}")
+
+
+def test_oracle_interval_affine_operators_match_the_reference():
+    x = interval_object("ibp_in")
+    y = O.linear(x, t(G["ibp_W"]), None)
+    assert_interval(y.lb, y.ub, "matmul", "ibp matmul")
+    z = O.layer_norm(x, t(G["ibp_norm_weight"]), t(G["ibp_norm_bias"]), "no_var", 2.0, 0.1, 2)
+    assert_interval(z.lb, z.ub, "layernorm_novar", "ibp layer_norm")
+
+
+@pytest.mark.gpu
+def test_hip_interval_mode_matches_the_reference():
+    from faith_amd import Bounds
+    args = SimpleNamespace(perturbed_words=2, method="ibp")
+
+    def gpu_interval(tag):
+        lb, ub = t(G[f"{tag}_lb"]).cuda(), t(G[f"{tag}_ub"]).cuda()
+        zeros = torch.zeros(1, lb.shape[1], 2 * lb.shape[2], lb.shape[2], device="cuda")
+        return Bounds(args, 2.0, 0.1, lw=zeros, lb=lb, uw=zeros.clone(), ub=ub)
+    for kind, src in IBP_UNARY.items():
+        print(f"[case] ibp {kind} against the executed reference", flush=True)
+        y = getattr(gpu_interval(src), kind)()
+        assert float(y.lw.abs().max()) == 0.0 and float(y.uw.abs().max()) == 0.0
+        assert_interval(y.lb, y.ub, kind, f"ibp {kind}")
+    x = gpu_interval("ibp_in")
+    y = x.matmul(t(G["ibp_W"]).cuda())
+    assert_interval(y.lb, y.ub, "matmul", "ibp matmul")
+    normalizer = SimpleNamespace(weight=t(G["ibp_norm_weight"]).cuda(), bias=t(G["ibp_norm_bias"]).cuda())
+    z = x.layer_norm(normalizer, "no_var")
+    assert_interval(z.lb, z.ub, "layernorm_novar", "ibp layer_norm", rtol=5e-5, atol=4e-6)
