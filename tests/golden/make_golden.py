@@ -1,10 +1,12 @@
 """Writes tests/golden/bounds_small.npz: tiny seeded inputs and their expected outputs.
 
 The reference holds no golden vectors for this path (its only op test draws random inputs at
-run time), and its Python cannot be imported here (Bounds.py needs tvm and nvcc at import).
-The expected values are therefore produced by oracle/closed_form.py -- the independent
+run time).  The expected values here are produced by oracle/closed_form.py -- the independent
 float64 per-neuron / brute-force restatement -- not by the tensorised oracle and not by the
-HIP path, so both of those can be checked against this file.
+HIP path, so both of those can be checked against this file.  These are a second reading of
+the reference, not the reference: what the reference itself returns is in reference_vectors.npz
+(make_reference_golden.py) and bounds_reference_vectors.npz (make_bounds_golden.py), written by
+executing its own code.
 
     python tests/golden/make_golden.py
 """
