@@ -159,6 +159,13 @@ def main():
         out[f"conc_{tag}_l"], out[f"conc_{tag}_u"] = lo.numpy(), hi.numpy()
         keep(f"dot_{tag}", ref(q, p, 0.2, words).dot_product(ref(k, p, 0.2, words)))
         keep(f"context_{tag}", ref(probs, p, 0.2, words).context(ref(value, p, 0.2, words)))
+    # any other perturbation norm (dual exponents 1.5 and 3, torch.norm(p=q)): the relaxations that the
+    # configurations name, and the intervals
+    for tag, p, words in (("p3_w1", 3.0, 1), ("p1.5_w2", 1.5, 2)):
+        keep(f"tanh_{tag}", ref(x, p, 0.1, words).tanh())
+        keep(f"relu_{tag}", ref(x, p, 0.1, words).relu())
+        lo, hi = ref(x, p, 0.1, words).concretize()
+        out[f"conc_{tag}_l"], out[f"conc_{tag}_u"] = lo.numpy(), hi.numpy()
     # operators without a norm in them: once
     keep("matmul", ref(x, 2.0, 0.1, 1).matmul(W))
     keep("scale_neg", ref(x, 2.0, 0.1, 1).multiply(-0.7))

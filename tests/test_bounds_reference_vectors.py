@@ -66,6 +66,33 @@ def test_oracle_unary_operators_match_the_reference(kind, tag):
     assert_matches(fn(obj(src), p, eps, words).tensors(), f"{kind}_{tag}", kind)
 
 
+GENERAL = {"p3_w1": (3.0, 1), "p1.5_w2": (1.5, 2)}      # dual exponents 1.5 and 3
+
+
+@pytest.mark.parametrize("tag", list(GENERAL))
+def test_oracle_general_norms_match_the_reference(tag):
+    p, words = GENERAL[tag]
+    x = obj("any_in")
+    assert_matches(O.tanh(x, p, EPS, words).tensors(), f"tanh_{tag}", "tanh")
+    assert_matches(O.relu(x, p, EPS, words).tensors(), f"relu_{tag}", "relu")
+    lo, hi = O.concretize(x, p, EPS, words)
+    np.testing.assert_allclose(lo.numpy(), G[f"conc_{tag}_l"], rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(hi.numpy(), G[f"conc_{tag}_u"], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", list(GENERAL))
+def test_hip_general_norms_match_the_reference(tag):
+    p, words = GENERAL[tag]
+    print(f"[case] tanh, relu, concretize {tag} against the executed reference", flush=True)
+    x = gpu_bounds("any_in", p, EPS, words)
+    assert_matches(quad(x.tanh()), f"tanh_{tag}", "tanh")
+    assert_matches(quad(x.relu()), f"relu_{tag}", "relu")
+    lo, hi = x.concretize()
+    np.testing.assert_allclose(lo.cpu().numpy(), G[f"conc_{tag}_l"], rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(hi.cpu().numpy(), G[f"conc_{tag}_u"], rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("tag", list(CASES))
 def test_oracle_products_match_the_reference(tag):
     p, words = CASES[tag]
