@@ -495,6 +495,38 @@ def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1, out=None):
     return olw, olb, ouw, oub, l, u
 
 
+class BoundCall:
+    """An entry point with its arguments converted once: calling the object launches again with the same device
+    pointers, sizes and stream -- for a caller that repeats one small launch (a bisection step on the same
+    buffers), where shape checks, twelve data_ptr() calls and the stream lookup are most of the host time.  The
+    tensors are kept alive by the object; their contents may change between calls, their addresses must not."""
+
+    __slots__ = ("name", "results", "_fn", "_args", "_keep")
+
+    def __init__(self, name, args, keep, results):
+        self.name, self.results = name, results
+        self._fn = _lib._ENTRY[name]
+        self._args = tuple(args)
+        self._keep = keep
+
+    def __call__(self):
+        rc = self._fn(*self._args)
+        if rc:
+            raise _lib.FaithError(self.name, rc, _lib.lib.faith_last_error().decode())
+        return self.results
+
+
+def bind_linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1, out=None):
+    """linear_concretize() as a BoundCall on torch's current stream: the checks run here, once; every call of the
+    returned object is one trip through the C ABI into the same six result tensors (`.results`)."""
+    results = linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words, out=out)      # checks, and a first launch
+    olw, olb, ouw, oub, l, u = results
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    args = (_ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias), _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw),
+            _ptr(l), _ptr(u), B, L, D, H, weight.shape[0], float(eps), q_code(p), int(words), _stream(lw))
+    return BoundCall("faith_matmul_concretize_verification", args, (lw, lb, uw, ub, weight, bias) + tuple(results), results)
+
+
 def linear_group(lw, lb, uw, ub, weights, biases=None):
     """Several affine layers of one shape on the same bound object (query, key, value of an attention block):
     one launch where that pays, the same results as linear() per layer.  weights: list of [H_out, H];

@@ -314,6 +314,27 @@ def test_linear_concretize_config0_against_oracle():
     assert bool((got[4] <= got[5]).all())
 
 
+def test_bound_call_repeats_the_launch_on_new_contents():
+    """ops.bind_linear_concretize converts the arguments once; every call of the object launches again into the same
+    result tensors and sees whatever the operand tensors hold by then."""
+    from faith_amd import ops
+    from faith_amd.workloads import make_config
+    c = make_config(0)
+    x = {k: v.cuda() for k, v in c["x"].items()}
+    W, bias = c["W"].cuda(), c["bias"].cuda()
+    bound = ops.bind_linear_concretize(x["lw"], x["lb"], x["uw"], x["ub"], W, bias, c["p"], c["eps"], c["words"])
+    first = [t.clone() for t in bound.results]
+    ref = ops.linear_concretize(x["lw"], x["lb"], x["uw"], x["ub"], W, bias, c["p"], c["eps"], c["words"])
+    assert all(torch.equal(a, b) for a, b in zip(first, ref))
+    x["lb"].add_(0.25)                                   # same addresses, new contents
+    x["ub"].add_(0.25)
+    again = bound()
+    assert again is bound.results
+    ref = ops.linear_concretize(x["lw"], x["lb"], x["uw"], x["ub"], W, bias, c["p"], c["eps"], c["words"])
+    assert all(torch.equal(a, b) for a, b in zip(again, ref))
+    assert not torch.equal(again[1], first[1])
+
+
 def test_linear_concretize_rejects_bad_words():
     from faith_amd import _lib
     g = torch.Generator().manual_seed(3)
