@@ -323,6 +323,62 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     }
 }
 
+// Column partial norms of a register-resident tile (thread (c, rg) holds rows i * RG + rg, i < RPT, of VEC columns)
+// -> part[words][NW][2][TH].  A perturbed word owns D_in / words consecutive rows; when that is a multiple of RG the
+// rows of step i belong to one word for every thread, and whether a step counts for a word is a scalar test per
+// step instead of a test (and a masked accumulation) per value -- for a general exponent, whose accumulation is two
+// quarter-rate instructions per value, that halves the arithmetic of a two-word tile.
+template <int Q, int VEC, int RPT, int RG, int TPR, int NW, int TH>
+__device__ __forceinline__ void resident_partials(const ActArgs &a, const Vec<VEC> (&dl)[RPT], const Vec<VEC> (&du)[RPT],
+                                                  float *part, int rg, int c, int lane, int wv) {
+    const int blk = a.D / a.words;
+    const bool whole_steps = blk % RG == 0;
+    const int steps = blk / RG;
+    for (int w = 0; w < a.words; ++w) {
+        float pl[VEC], pu[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
+        if (whole_steps) {
+            const int lo_i = w * steps, hi_i = lo_i + steps;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                if (i >= lo_i && i < hi_i) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
+                        pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
+                    }
+                }
+            }
+        } else {
+            const int lo_row = w * blk, hi_row = lo_row + blk;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                const int row = i * RG + rg;
+                if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        // opaque copies: |x| (or its logarithm) of every value would otherwise be formed once,
+                        // outside the loop over the words, and held: 64 more registers
+                        float xl = dl[i].get(v), xu = du[i].get(v);
+                        asm volatile("" : "+v"(xl), "+v"(xu));
+                        pl[v] = nacc<Q>(pl[v], xl, a.qv);
+                        pu[v] = nacc<Q>(pu[v], xu, a.qv);
+                    }
+                }
+            }
+        }
+        combine_from<Q, TPR>(pl, pu);
+        if (lane < TPR) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                part[((w * NW + wv) * 2 + 0) * TH + c * VEC + v] = pl[v];
+                part[((w * NW + wv) * 2 + 1) * TH + c * VEC + v] = pu[v];
+            }
+        }
+    }
+}
+
 // The common shape of the natural layout, straight-line: D_in <= RG * RPT (everything a thread
 // loads stays in registers), D_in a multiple of RG and H a multiple of the tile width, 16-byte
 // aligned.  Whether a row exists is then the same for every thread (a scalar branch), there are no
@@ -368,32 +424,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
             du[i].zero();
         }
     }
-    const int blk = a.D / a.words;
-    for (int w = 0; w < a.words; ++w) {
-        const int lo_row = w * blk, hi_row = lo_row + blk;
-        float pl[VEC], pu[VEC];
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
-#pragma unroll
-        for (int i = 0; i < RPT; ++i) {
-            const int row = i * RG + rg;
-            if (row >= lo_row && row < hi_row) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                    pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
-                    pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
-                }
-            }
-        }
-        combine_from<Q, TPR>(pl, pu);
-        if (lane < TPR) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-                part[((w * NW + wv) * 2 + 0) * TH + c * VEC + v] = pl[v];
-                part[((w * NW + wv) * 2 + 1) * TH + c * VEC + v] = pu[v];
-            }
-        }
-    }
+    resident_partials<Q, VEC, RPT, RG, TPR, NW, TH>(a, dl, du, part, rg, c, lane, wv);
     __syncthreads();
 
     neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, lb0, ub0, a.l, a.u, bi, lane < TH, lane, wv);
@@ -445,7 +476,6 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
     const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid % TPR, rg = tid / TPR;
     const size_t row_step = (size_t)RG * a.H;
-    const int blk = a.D / a.words;
 
     struct Tile {
         Vec<VEC> dl[RPT], du[RPT];
@@ -472,31 +502,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
         }
     };
     auto finish = [&](int t, Tile &x) __attribute__((always_inline)) {
-        for (int w = 0; w < a.words; ++w) {
-            const int lo_row = w * blk, hi_row = lo_row + blk;
-            float pl[VEC], pu[VEC];
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
-#pragma unroll
-            for (int i = 0; i < RPT; ++i) {
-                const int row = i * RG + rg;
-                if (row >= lo_row && row < hi_row) {
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) {
-                        pl[v] = nacc<Q>(pl[v], x.dl[i].get(v), a.qv);
-                        pu[v] = nacc<Q>(pu[v], x.du[i].get(v), a.qv);
-                    }
-                }
-            }
-            combine_from<Q, TPR>(pl, pu);
-            if (lane < TPR) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                    part[((w * NW + wv) * 2 + 0) * TH + c * VEC + v] = pl[v];
-                    part[((w * NW + wv) * 2 + 1) * TH + c * VEC + v] = pu[v];
-                }
-            }
-        }
+        resident_partials<Q, VEC, RPT, RG, TPR, NW, TH>(a, x.dl, x.du, part, rg, c, lane, wv);
         __syncthreads();
         neuron_stage<MODE, Q, NW, TH>(a, part, s_lu, s_ln, x.lb0, x.ub0, a.l, a.u, bias_of(t), lane < TH, lane, wv);
         float klo[VEC], kup[VEC];
@@ -872,7 +878,7 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(a, st);
         else if (tv == 12) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(a, st);
         else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(a, st);
-        else launch_resident<MODE, Q, 8, 256, 8>(a, st);
+        else launch_resident<MODE, Q, 8, 256, 8, (Q == Q_GENERAL ? 3 : 4)>(a, st);     // a general exponent needs more registers than 128
         return;
     }
     switch (tv) {
