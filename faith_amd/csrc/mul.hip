@@ -173,7 +173,7 @@ __global__ void __launch_bounds__(NTHREADS) mul_natural(const MulArgs a) {
 // in registers), D_in a multiple of RG, H a multiple of the tile width, 16-byte aligned.  Row
 // existence is then a scalar branch and there are neither column predicates nor a second pass.
 template <int Q, int TPR, int NTHREADS, int RPT>
-__global__ void __launch_bounds__(NTHREADS) mul_resident(const MulArgs a) {
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(Q == Q_GENERAL ? 2 : 4))) mul_resident(const MulArgs a) {
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
     static_assert(TH <= WAVE, "one lane per neuron in wavefront 0");
     extern __shared__ float smem[];
@@ -200,6 +200,10 @@ __global__ void __launch_bounds__(NTHREADS) mul_resident(const MulArgs a) {
         }
     }
     const int blk = a.D / a.words;
+    // a perturbed word owns blk consecutive rows: when that is a multiple of RG, whether step i counts for a word is
+    // a scalar test per step instead of one per value (a general exponent: half the quarter-rate arithmetic)
+    const bool whole_steps = blk % RG == 0;
+    const int steps = blk / RG;
     for (int w = 0; w < a.words; ++w) {
         const int lo_row = w * blk, hi_row = lo_row + blk;
         float pn[4][VEC];
@@ -207,22 +211,37 @@ __global__ void __launch_bounds__(NTHREADS) mul_resident(const MulArgs a) {
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int v = 0; v < VEC; ++v) pn[t][v] = 0.f;
+        if (whole_steps) {
+            const int lo_i = w * steps, hi_i = lo_i + steps;
 #pragma unroll
-        for (int i = 0; i < RPT; ++i) {
-            const int row = i * RG + rg;
-            if (row >= lo_row && row < hi_row) {
+            for (int i = 0; i < RPT; ++i) {
+                if (i >= lo_i && i < hi_i) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                    for (int t = 0; t < 4; ++t)
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v), a.qv);
+                        for (int v = 0; v < VEC; ++v) pn[t][v] = nacc<Q>(pn[t][v], d[t][i].get(v), a.qv);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                const int row = i * RG + rg;
+                if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) {
+                            // an opaque copy: |x| of every value would otherwise be formed once, outside the loop
+                            // over the words, and held (128 more registers)
+                            float x = d[t][i].get(v);
+                            asm volatile("" : "+v"(x));
+                            pn[t][v] = nacc<Q>(pn[t][v], x, a.qv);
+                        }
+                }
             }
         }
 #pragma unroll
-        for (int m = TPR; m < WAVE; m <<= 1)
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) pn[t][v] = ncomb<Q>(pn[t][v], __shfl_xor(pn[t][v], m, WAVE));
+        for (int t = 0; t < 4; t += 2) combine_from<Q, TPR>(pn[t], pn[t + 1]);
         if (lane < TPR) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
