@@ -308,16 +308,25 @@ def bench_config1(args, ops, O, wl, steps, warmup):
     tc = gpu_times_ms(lambda: _lib.call("faith_copy_f32", src.data_ptr(), dst.data_ptr(), src.numel(), st), 50, 5)
     entries.append(op_entry("plain copy of the same byte count (yardstick, not a bound op)", "hbm", tc, nbytes))
 
-    dom = max(per_kernel, key=lambda k: statistics.mean(per_kernel[k]))
+    # Two kernels share a step evenly: relu (every relaxation but tanh) runs on the persistent two-tile kernel, tanh
+    # on the one-tile kernel.  `roofline` is the slower of the two (its slowest norm); the other is quoted under "also".
+    slowest = {kind: max((k for k in per_kernel if k[0] == kind), key=lambda k: statistics.mean(per_kernel[k]))
+               for kind in ("relu", "tanh")}
+    dom = max(slowest.values(), key=lambda k: statistics.mean(per_kernel[k]))
+    other = slowest["tanh" if dom[0] == "relu" else "relu"]
     avg_ms = statistics.mean(gpu_back_to_back_ms(lambda: one(*dom), 20))
+    other_ms = statistics.mean(gpu_back_to_back_ms(lambda: one(*other), 20))
     traffic = traffic_from_profile()
-    # relu (every relaxation but tanh) runs on the persistent two-tile kernel, tanh on the one-tile kernel
-    kernel = "act_resident" if dom[0] == "tanh" else "act_pipelined"
+    kernel_of = {"relu": "act_pipelined", "tanh": "act_resident"}
+    kernel = kernel_of[dom[0]]
     roofline = {"bound": "hbm", "kernel": f"{kernel}<{dom[0]}, p={dom[1]:g}>",
                 "achieved": round(nbytes / avg_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(nbytes / avg_ms / 1e6 / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(avg_ms * 1e3, 2), "bytes_per_launch": nbytes,
                 "traffic": traffic.get((dom[0], "warm")),
+                "also": {"kernel": f"{kernel_of[other[0]]}<{other[0]}, p={other[1]:g}>",
+                         "achieved": round(nbytes / other_ms / 1e6, 1), "frac": round(nbytes / other_ms / 1e6 / HBM_PEAK_GBS, 4),
+                         "avg_launch_us": round(other_ms * 1e3, 2), "traffic": traffic.get((other[0], "warm"))},
                 "note": "the configuration as specified: one operand set (269 MB) reused by every launch, against 256 MB "
                         "of Infinity Cache; roofline_cold cycles disjoint sets"}
 
@@ -372,6 +381,11 @@ def bench_config1(args, ops, O, wl, steps, warmup):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / cold_ms / 1e6 / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(cold_ms * 1e3, 2), "bytes_per_launch": nbytes,
                      "traffic": traffic.get((dom[0], "cold")), "operand_sets": COLD_SETS,
+                     "also": {"kernel": f"{kernel_of[other[0]]}<{other[0]}, p={dom[1]:g}>",
+                              "achieved": round(nbytes / cold_entries[other[0]] / 1e6, 1),
+                              "frac": round(nbytes / cold_entries[other[0]] / 1e6 / HBM_PEAK_GBS, 4),
+                              "avg_launch_us": round(cold_entries[other[0]] * 1e3, 2),
+                              "traffic": traffic.get((other[0], "cold"))},
                      "plain_copy_cold_frac": round(nbytes / copy_cold_ms / 1e6 / HBM_PEAK_GBS, 4),
                      "frac_with_streaming_thread_shape": round(nbytes / streaming[dom[0]] / 1e6 / HBM_PEAK_GBS, 4)}
     del sets
