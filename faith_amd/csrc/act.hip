@@ -258,14 +258,32 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
             float pl[VEC], pu[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; ++v) pl[v] = pu[v] = 0.f;
+            if (blk % RG == 0) {
+                // a word owns a whole number of steps (RG rows each): whether step ch * RPT + i counts for it is a
+                // scalar test per step instead of one per value (see resident_partials)
+                const int lo_s = w * (blk / RG) - ch * RPT, hi_s = lo_s + blk / RG;
 #pragma unroll
-            for (int i = 0; i < RPT; ++i) {
-                const int row = ch * CHUNK + i * RG + rg;
-                if (row >= lo_row && row < hi_row) {
+                for (int i = 0; i < RPT; ++i) {
+                    if (i >= lo_s && i < hi_s) {
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) {
-                        pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
-                        pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
+                        for (int v = 0; v < VEC; ++v) {
+                            pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
+                            pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RPT; ++i) {
+                    const int row = ch * CHUNK + i * RG + rg;
+                    if (row >= lo_row && row < hi_row) {
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) {
+                            float xl = dl[i].get(v), xu = du[i].get(v);
+                            asm volatile("" : "+v"(xl), "+v"(xu));      // keeps |x| from being formed outside the word loop and held
+                            pl[v] = nacc<Q>(pl[v], xl, a.qv);
+                            pu[v] = nacc<Q>(pu[v], xu, a.qv);
+                        }
                     }
                 }
             }
