@@ -86,6 +86,31 @@ def test_conv_shapes(case, with_bias):
     check(x, W, bias, s, p, "sweep")
 
 
+@pytest.mark.parametrize("case", [
+    (140, 16, 64, 32, 32, 1, 1, 0),    # 1x1: 560 tiles of 64 channels x 8 rows
+    (300, 8, 64, 64, 32, 3, 2, 1),     # 3x3 stride 2: 600 tiles (16-column pixel blocks)
+    (150, 3, 64, 32, 32, 3, 1, 1),     # first layer, C_in = 3: 600 tiles
+])
+def test_conv_layers_with_more_tiles_than_resident_workgroups(case):
+    """The straight-line kernels run on persistent workgroups (two per CU): with more tiles than that, a workgroup
+    walks several, re-using its LDS stages from tile to tile.  Against the oracle, and against the general kernel
+    (one tile per workgroup)."""
+    from faith_amd import _lib, ops
+    D, Ci, Co, Hh, Ww, K, s_, p = case
+    g = torch.Generator().manual_seed(45)
+    x = make(g, D, Ci, Hh, Ww, ordered=False)
+    W = torch.randn(Co, Ci, K, K, generator=g) * (2.0 / (Ci * K * K)) ** 0.5
+    bias = torch.randn(Co, generator=g)
+    got = check(x, W, bias, s_, p, "many tiles")
+    _lib.call("faith_tune_set", 4, 1)
+    try:
+        general = ops.conv2d(*(t.cuda() for t in x.tensors()), W.cuda(), bias.cuda(), s_, p)
+    finally:
+        _lib.call("faith_tune_set", 4, 0)
+    for name, a_, b_ in zip(("lw", "lb", "uw", "ub"), got, general):
+        assert close(a_, b_.cpu(), rtol=1e-5, atol=1e-6), name
+
+
 @pytest.mark.parametrize("case", [(3, 8, 40, 17, 40, 3, 2, 1), (2, 32, 64, 8, 40, 1, 1, 0), (2, 8, 24, 14, 36, 5, 1, 2),
                                   (3, 3, 64, 32, 32, 3, 1, 1)])
 def test_straight_line_conv_kernels_equal_the_general_kernel(case):
