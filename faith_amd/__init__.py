@@ -7,11 +7,11 @@ built in-tree with `python -m faith_amd.build`.  There is no CPU fallback.
 """
 import importlib
 
-__all__ = ["Bounds", "ConvBounds", "ops", "c_bound", "workloads"]
+__all__ = ["Bounds", "CompactBounds", "BoundsMaker", "ConvBounds", "ops", "c_bound", "workloads"]
 
 
 def __getattr__(name):
-    if name in ("Bounds", "ConvBounds"):
+    if name in ("Bounds", "CompactBounds", "BoundsMaker", "ConvBounds"):
         return getattr(importlib.import_module(".bounds", __name__), name)
     if name in ("ops", "c_bound", "workloads", "build"):
         return importlib.import_module("." + name, __name__)

@@ -48,8 +48,19 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
     embeddings [1, L, dim]; index: position (int) or list of positions; make_bounds(p, eps, lw, lb,
     uw, ub) builds the bound object.  Returns bounds of the (layer-normed) embeddings."""
     length, dim = embeddings.shape[1], embeddings.shape[2]
-    w = torch.zeros((length, dim * perturbed_words, dim), device=embeddings.device)
     positions = [index] if perturbed_words == 1 else list(index)
+    compact = _compact_maker(make_bounds, 1, length, dim * perturbed_words, dim)
+    if compact is not None and not ibp:
+        # a maker that can hold the coefficients of the perturbed positions alone: the zero rows of
+        # every other position are never written, read or multiplied
+        dev = embeddings.device
+        w = torch.zeros((1, perturbed_words, dim * perturbed_words, dim), device=dev)
+        for i in range(perturbed_words):
+            w[0, i, dim * i:dim * (i + 1), :] = _eye(dim, dev)
+        b = embeddings[0].unsqueeze(0)
+        bounds = compact(p, eps, torch.as_tensor([positions], dtype=torch.int64, device=dev), w, b, w, b)
+        return bounds if norm is None else bounds.layer_norm(norm, layer_norm)
+    w = torch.zeros((length, dim * perturbed_words, dim), device=embeddings.device)
     if ibp:
         lb, ub = embeddings[0].unsqueeze(0).clone(), embeddings[0].unsqueeze(0).clone()
         for pos in positions:
@@ -66,6 +77,16 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
     return bounds
+
+
+def _compact_maker(make_bounds, batch, length, dim_in, dim_out):
+    """make_bounds.compact if the maker has one (faith_amd.BoundsMaker) and finds that leaving out the zero
+    coefficient rows pays for an object of this shape, else None."""
+    compact = getattr(make_bounds, "compact", None)
+    pays = getattr(make_bounds, "compact_pays", None)
+    if compact is None or (pays is not None and not pays(batch, length, dim_in, dim_out)):
+        return None
+    return compact
 
 
 _EYES = {}
@@ -204,13 +225,18 @@ def bound_inputs(make_bounds, embeddings, indices, radii, p=2.0, norm=None, laye
     length, dim = embeddings.shape[1], embeddings.shape[2]
     n = len(indices)
     dev = embeddings.device
-    w = torch.zeros((n, length, dim, dim), device=dev)
-    eye = torch.eye(dim, device=dev)
     scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
-    w[torch.arange(n, device=dev), torch.as_tensor(indices, device=dev)] = scale[:, None, None] * eye
     b = embeddings[0].unsqueeze(0).expand(n, length, dim).contiguous()
+    compact = _compact_maker(make_bounds, n, length, dim, dim)
     # lower and upper start out equal and no operator writes into its inputs: one tensor serves both
-    bounds = make_bounds(p, 1.0, w, b, w, b)
+    if compact is not None:
+        w = (scale[:, None, None] * _eye(dim, dev)).unsqueeze(1)              # [n, 1, dim, dim]
+        at = torch.as_tensor(indices, dtype=torch.int64, device=dev).reshape(n, 1)
+        bounds = compact(p, 1.0, at, w, b, w, b)
+    else:
+        w = torch.zeros((n, length, dim, dim), device=dev)
+        w[torch.arange(n, device=dev), torch.as_tensor(indices, device=dev)] = scale[:, None, None] * _eye(dim, dev)
+        bounds = make_bounds(p, 1.0, w, b, w, b)
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
     return bounds
@@ -316,13 +342,23 @@ class CapturedVerifier:
         length, dim = embeddings.shape[1], embeddings.shape[2]
         dev = embeddings.device
         self.batch, self.label, self.dim = batch, label, dim
-        self.w = torch.zeros((batch, length, dim, dim), device=dev)
         self.b = embeddings[0].unsqueeze(0).expand(batch, length, dim).contiguous()
         self.eye = torch.eye(dim, device=dev)
         self.rows = torch.arange(batch, device=dev)
+        compact = _compact_maker(make_bounds, batch, length, dim, dim)
+        if compact is not None:
+            # the graph reads the perturbed positions and the scaled identities from these two
+            self.at = torch.zeros((batch, 1), dtype=torch.int64, device=dev)
+            self.w = torch.zeros((batch, 1, dim, dim), device=dev)
+        else:
+            self.at = None
+            self.w = torch.zeros((batch, length, dim, dim), device=dev)
 
         def body():
-            x = make_bounds(p, 1.0, self.w, self.b, self.w, self.b)
+            if compact is not None:
+                x = compact(p, 1.0, self.at, self.w, self.b, self.w, self.b)
+            else:
+                x = make_bounds(p, 1.0, self.w, self.b, self.w, self.b)
             with type(x).collect_failures(batch, dev) as failed:
                 if network.embedding_norm is not None:
                     x = x.layer_norm(network.embedding_norm, network.layer_norm)
@@ -348,8 +384,12 @@ class CapturedVerifier:
         """Verdicts for batch element b = (position indices[b], radius radii[b]); len == batch."""
         assert len(indices) == self.batch and len(radii) == self.batch
         dev = self.w.device
-        self.w.zero_()
         scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
-        self.w[self.rows, torch.as_tensor(indices, device=dev)] = scale[:, None, None] * self.eye
+        if self.at is not None:
+            self.at.copy_(torch.as_tensor(indices, dtype=torch.int64, device=dev).reshape(-1, 1))
+            self.w.copy_((scale[:, None, None] * self.eye).unsqueeze(1))
+        else:
+            self.w.zero_()
+            self.w[self.rows, torch.as_tensor(indices, device=dev)] = scale[:, None, None] * self.eye
         self.graph.replay()
         return [bool(v) for v in self.safe.tolist()]

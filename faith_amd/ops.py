@@ -392,6 +392,29 @@ def layer_norm(lw, lb, uw, ub, weight=None, bias=None, other=None):
     return olw, olb, ouw, oub
 
 
+def spread_positions(t, positions, length):
+    """[B, P, ...] -> [B, length, ...]: row positions[b, i] of batch element b holds t[b, i], every other row
+    is zero.  positions: int64 [B, P] on t's device, distinct within a batch element.  A fill and an indexed copy
+    (nothing is computed); neither waits for the device, so both can be captured in a HIP graph."""
+    B, P = positions.shape
+    if t.shape[:2] != (B, P):
+        raise ValueError(f"t {tuple(t.shape)} does not start with positions' shape {(B, P)}")
+    out = zeros(B, length, *t.shape[2:], device=t.device)
+    key = (B, str(t.device))
+    if key not in _BATCH_INDEX:
+        _BATCH_INDEX[key] = torch.arange(B, device=t.device)[:, None]
+    out[_BATCH_INDEX[key], positions] = t
+    return out
+
+
+_BATCH_INDEX = {}
+
+
+def zeros(*shape, device):
+    """A result buffer (the caller's persistent one inside a workspace scope) filled with zeros."""
+    return _empty(*shape, device=device).zero_()
+
+
 def softmax_fits(dim_in, dim_out):
     """True if softmax() takes a [dim_in, dim_out] slab in one launch (16-byte aligned tensors assumed)."""
     return bool(_lib.lib.faith_softmax_fits(int(dim_in), int(dim_out)))

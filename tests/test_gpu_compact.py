@@ -1,0 +1,241 @@
+"""`CompactBounds`: the input object of a query with its zero rows left out.
+
+The input of a verification query has coefficients at the perturbed position(s) only
+(VerifierForward.py:127-156).  The compact object runs the embedding layer norm and the first dense
+layers on those rows alone; these tests hold it to the results of the ordinary object that carries the
+zeros -- bit for bit where the same kernel sees the same rows (layer norm), to the parity bar where the
+affine kernel may pick another tiling for the smaller problem -- and the whole propagation built on it
+to the verdicts and margins of the one built on the ordinary object."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from faith_amd import forward as F
+from tests.helpers import ATOL, RTOL, worst
+from tests.oracle_bounds import OracleBounds, to_device, true_layer
+from tests.parity import KAPPA, U32
+from tests.test_layer_pipeline import HIDDEN, LENGTH, build, network_of, two_layer_network
+
+pytestmark = pytest.mark.gpu
+
+
+def compact_and_dense(seed, B=3, P=2, D=10, H=24, L=5, words=1, shared=False):
+    from faith_amd import Bounds, CompactBounds
+    g = torch.Generator().manual_seed(seed)
+    positions = torch.stack([torch.randperm(L, generator=g)[:P] for _ in range(B)])
+    lw = torch.randn(B, P, D, H, generator=g)
+    uw = lw if shared else lw + 0.05 * torch.rand(B, P, D, H, generator=g)
+    lb = torch.randn(B, L, H, generator=g)
+    ub = lb if shared else lb + 0.3 * torch.rand(B, L, H, generator=g)
+    args = SimpleNamespace(perturbed_words=words)
+    dev = lambda t: t.cuda()
+    c = CompactBounds(args, 2.0, 0.1, dev(positions), dev(lw), dev(lb), dev(lw if shared else uw), dev(ub))
+    rows = torch.arange(B)[:, None]
+    dlw = torch.zeros(B, L, D, H); dlw[rows, positions] = lw
+    duw = torch.zeros(B, L, D, H); duw[rows, positions] = uw
+    d = Bounds(args, 2.0, 0.1, lw=dev(dlw), lb=dev(lb), uw=dev(duw), ub=dev(ub))
+    return c, d
+
+
+def same_bits(a, b, what):
+    for name in ("lw", "lb", "uw", "ub"):
+        x, y = getattr(a, name), getattr(b, name)
+        assert x.shape == y.shape, (what, name, x.shape, y.shape)
+        assert torch.equal(x, y), f"{what}.{name}: {int((x != y).sum())} values differ"
+
+
+def at_the_bar(a, b, what, src=None, weight=None):
+    """rtol 1e-5 / atol 1e-6.  With `src` and `weight` (an affine layer applied to the object src): two fp32
+    sums of the same K products in different orders -- the affine kernel tiles the smaller problem its own
+    way -- cannot be held to atol against each other where the products are larger than the sum, so each of
+    the two gets the forward-error allowance of an fp32 dot product, KAPPA * u * sum_k |a_k w_k|, on top."""
+    for name in ("lw", "lb", "uw", "ub"):
+        x, y = getattr(a, name), getattr(b, name)
+        assert x.shape == y.shape, (what, name, x.shape, y.shape)
+        err, of_bar = worst(x, y)
+        if of_bar <= 1.0:
+            continue
+        assert src is not None, f"{what}.{name}: max err {err:.3g}, {of_bar:.2f} of the bar"
+        lo, hi = (src.lw, src.uw) if name in ("lw", "uw") else (src.lb, src.ub)
+        terms = (lo.double().abs() + hi.double().abs()).cpu() @ weight.double().abs().cpu().T
+        tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
+        over = float(((x.double() - y.double()).abs().cpu() / tol).max())
+        assert over <= 1.0, f"{what}.{name}: max err {err:.3g}, {over:.2f} of the accumulation-aware bar"
+
+
+def layer_of(g, h_in, h_out, bias=True):
+    return SimpleNamespace(weight=(torch.randn(h_out, h_in, generator=g) / h_in ** 0.5).cuda(),
+                           bias=(0.1 * torch.randn(h_out, generator=g)).cuda() if bias else None)
+
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_dense_form_writes_the_zeros_out(shared):
+    c, d = compact_and_dense(3, shared=shared)
+    same_bits(c.dense_form(), d, "dense form")
+    assert c.dense_form() is c.dense_form()
+    # what the compact object does not define is the dense object's
+    assert c.lw.shape == d.lw.shape and c.dim_in == d.dim_in and c.batch_size == d.batch_size
+    (cl, cu), (dl, du) = c.concretize(), d.concretize()
+    assert torch.equal(cl, dl) and torch.equal(cu, du)
+    same_bits(c.relu(), d.relu(), "relu through the dense form")
+
+
+def test_layer_norm_keeps_the_form_and_the_bits():
+    from faith_amd import CompactBounds
+    g = torch.Generator().manual_seed(5)
+    c, d = compact_and_dense(4, B=4, P=1, D=12, H=40, L=7)
+    norm = SimpleNamespace(weight=(1.0 + 0.2 * torch.randn(40, generator=g)).cuda(), bias=(0.1 * torch.randn(40, generator=g)).cuda())
+    out = c.layer_norm(norm, "no_var")
+    assert isinstance(out, CompactBounds) and out._lw.shape == c._lw.shape
+    same_bits(out, d.layer_norm(norm, "no_var"), "layer norm, no_var")
+    # the variance mixes nothing across positions either, but has no compact kernel: through the dense form
+    same_bits(c.layer_norm(norm, "standard"), d.layer_norm(norm, "standard"), "layer norm, standard")
+    assert c.layer_norm(norm, "no") is c
+    # as the residual of another object's layer norm, and with a residual of its own
+    other = d.relu()
+    same_bits(other.layer_norm(norm, "no_var", residual=c), other.layer_norm(norm, "no_var", residual=d), "as residual")
+    same_bits(c.layer_norm(norm, "no_var", residual=other), d.layer_norm(norm, "no_var", residual=other), "with residual")
+
+
+@pytest.mark.parametrize("shape", [(3, 2, 10, 24, 5, 16), (2, 1, 64, 64, 9, 96), (5, 3, 33, 20, 4, 7), (1, 1, 256, 256, 32, 256)])
+def test_dense_layers_on_the_rows_that_are_not_zero(shape):
+    from faith_amd import Bounds
+    B, P, D, H, L, N = shape
+    g = torch.Generator().manual_seed(B * 100 + N)
+    c, d = compact_and_dense(6, B, P, D, H, L)
+    for bias in (True, False):
+        layer = layer_of(g, H, N, bias)
+        out = c.dense(layer)
+        assert isinstance(out, Bounds)
+        at_the_bar(out, d.dense(layer), f"dense {shape} bias={bias}", d, layer.weight)
+        at_the_bar(c.matmul(layer.weight, layer.bias), d.matmul(layer.weight, layer.bias), "matmul", d, layer.weight)
+    # positions without coefficients get exact zeros, whatever the buffer held before
+    zero_rows = torch.ones(B, L, dtype=torch.bool)
+    zero_rows[torch.arange(B)[:, None], c.positions.cpu()] = False
+    assert float(out.lw.cpu()[zero_rows].abs().max()) == 0.0 and float(out.uw.cpu()[zero_rows].abs().max()) == 0.0
+    layers = [layer_of(g, H, N), layer_of(g, H, N, False), layer_of(g, H, N)]
+    for got, want, layer in zip(c.dense_group(layers), d.dense_group(layers), layers):
+        at_the_bar(got, want, f"dense_group {shape}", d, layer.weight)
+    # layers of different shapes: one call each
+    mixed = [layer_of(g, H, N), layer_of(g, H, N + 3)]
+    for got, want, layer in zip(c.dense_group(mixed), d.dense_group(mixed), mixed):
+        at_the_bar(got, want, f"dense_group of two shapes {shape}", d, layer.weight)
+
+
+def test_compact_object_matches_the_oracle():
+    """Against the CPU oracle directly (not only against the HIP path's own dense object)."""
+    g = torch.Generator().manual_seed(8)
+    c, d = compact_and_dense(9, B=2, P=2, D=20, H=32, L=6)
+    norm = SimpleNamespace(weight=1.0 + 0.2 * torch.randn(32, generator=g), bias=0.1 * torch.randn(32, generator=g))
+    layer = SimpleNamespace(weight=torch.randn(48, 32, generator=g) / 32 ** 0.5, bias=0.1 * torch.randn(48, generator=g))
+    o = OracleBounds(2.0, 0.1, d.lw.cpu(), d.lb.cpu(), d.uw.cpu(), d.ub.cpu())
+    want = o.layer_norm(norm, "no_var").dense(layer)
+    got = c.layer_norm(to_device(norm, "cuda"), "no_var").dense(to_device(layer, "cuda"))
+    at_the_bar(got, want, "layer norm + dense against the oracle")
+
+
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+def test_propagation_from_the_compact_input_gives_the_ordinary_ones_margins(mode):
+    from faith_amd import Bounds, BoundsMaker, CompactBounds
+    layer, embed_norm, pooler, classifier, emb = build(7, mode)
+    gparts = tuple(to_device(x, "cuda") for x in (layer, embed_norm, pooler, classifier))
+    ge = emb.cuda()
+    plain = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    maker = BoundsMaker(compact_from=0)
+    assert isinstance(F.bound_input(maker, ge, 2, 0.02, 1, 2.0), CompactBounds)
+    # an object this small is written out at once unless the maker is told otherwise
+    assert isinstance(F.bound_input(BoundsMaker(), ge, 2, 0.02, 1, 2.0), Bounds)
+    assert isinstance(F.bound_inputs(BoundsMaker(compact_from=4 * 3 * LENGTH * HIDDEN * HIDDEN), ge, [1, 2, 3], [0.1] * 3), CompactBounds)
+    assert isinstance(F.bound_inputs(BoundsMaker(compact_from=4 * 3 * LENGTH * HIDDEN * HIDDEN + 1), ge, [1, 2, 3], [0.1] * 3), Bounds)
+    assert isinstance(F.bound_input(maker, ge, 2, 0.02, 1, 2.0, ibp=True), Bounds)
+
+    def run(make):
+        x = F.bound_input(make, ge, 2, 0.02, 1, 2.0, gparts[1], mode)
+        _, _, out = F.bound_layer(x, gparts[0], mode, "relu")
+        return out, F.bound_classifier(F.bound_pooling(out, gparts[2], make), gparts[3], 0)
+    out_c, (safe_c, l_c, u_c) = run(maker)
+    out_d, (safe_d, l_d, u_d) = run(plain)
+    # the same operators on the same values from the first attention scores on; before them the affine
+    # kernel rounds in its own order for the smaller problem
+    for name in ("lw", "lb", "uw", "ub"):
+        a, b = getattr(out_c, name).double(), getattr(out_d, name).double()
+        assert float((a - b).abs().max()) <= 1e-5 * max(float(b.abs().max()), 1.0), name
+    assert safe_c == safe_d
+    assert float((l_c - l_d).abs().max()) <= 1e-4 and float((u_c - u_d).abs().max()) <= 1e-4
+
+
+@pytest.mark.parametrize("mode", ["no_var", "standard"])
+def test_two_perturbed_words_from_the_compact_input(mode):
+    from faith_amd import Bounds, BoundsMaker
+    net, emb = two_layer_network(21, mode)
+    two_words = SimpleNamespace(perturbed_words=2)
+    gnet = SimpleNamespace(**{k: (to_device(v, "cuda") if k in ("embedding_norm", "pooler", "classifier") else v)
+                              for k, v in vars(net).items()})
+    gnet.layers = [to_device(x, "cuda") for x in net.layers]
+    ge = emb.cuda()
+
+    def margins(make):
+        x = F.bound_input(make, ge, [1, 4], 0.01, 2, 2.0, gnet.embedding_norm, gnet.layer_norm)
+        pooled = F.bound_pooling(F.propagate(x, gnet), gnet.pooler, make)
+        return F.bound_classifier(pooled, gnet.classifier, 0)
+    _, l_c, u_c = margins(BoundsMaker(two_words, compact_from=0))
+    _, l_d, u_d = margins(lambda p_, e_, lw, lb, uw, ub: Bounds(two_words, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub))
+    assert float((l_c - l_d).abs().max()) <= 1e-4 and float((u_c - u_d).abs().max()) <= 1e-4
+    omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub, words=2)
+    x = F.bound_input(omake, emb, [1, 4], 0.01, 2, 2.0, net.embedding_norm, net.layer_norm)
+    _, ol, ou = F.bound_classifier(F.bound_pooling(F.propagate(x, net), net.pooler, omake), net.classifier, 0)
+    assert float((l_c.cpu() - ol).abs().max()) <= 2e-3 and float((u_c.cpu() - ou).abs().max()) <= 2e-3
+
+
+def test_search_from_the_compact_input_finds_the_same_radii():
+    """One at a time, batched, with persistent buffers and from a captured graph: the radii of the search on the
+    ordinary object (a verdict within rounding of its threshold may fall either way: one step)."""
+    from faith_amd import Bounds, BoundsMaker, ops
+    layer, embed_norm, pooler, classifier, emb = build(11, "no_var")
+    parts = (layer, embed_norm, pooler, classifier)
+    _, margin = true_layer(emb.double(), layer, embed_norm, "no_var", pooler, classifier)
+    label = 0 if float(margin[0, 0]) > 0 else 1
+    gnet = network_of(tuple(to_device(x, "cuda") for x in parts), "no_var")
+    ge = emb.cuda()
+    positions, max_eps, iters = [1, 2, 3, 4], 0.5, 6
+    step = max_eps / 2 ** iters
+    plain = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    maker = BoundsMaker(compact_from=0)
+    want = F.certified_radii(plain, gnet, ge, positions, label, 2.0, max_eps, iters)
+    one = F.certified_radii(maker, gnet, ge, positions, label, 2.0, max_eps, iters)
+    lock = F.certified_radii(maker, gnet, ge, positions, label, 2.0, max_eps, iters, batched=True)
+    ws = ops.Workspace()
+    F.verify_safety_batch(maker, gnet, ge, positions, [0.01] * 4, label, 2.0, buffers=ws)
+    first = ws.allocations
+    kept = F.certified_radii(maker, gnet, ge, positions, label, 2.0, max_eps, iters, batched=True, buffers=ws)
+    assert ws.allocations == first, "a repeated propagation allocated result buffers"
+    graph = F.certified_radii(maker, gnet, ge, positions, label, 2.0, max_eps, iters, captured=True)
+    print(f"[case] radii ordinary {want} compact {one} batched {lock} buffers {kept} graph {graph}", flush=True)
+    assert lock == kept == graph
+    for a, b, c in zip(want, one, lock):
+        assert abs(a - b) <= step + 1e-12 and abs(a - c) <= step + 1e-12
+
+
+def test_captured_graph_on_the_compact_input_follows_new_positions_and_radii():
+    from faith_amd import BoundsMaker
+    layer, embed_norm, pooler, classifier, emb = build(11, "standard")
+    parts = (layer, embed_norm, pooler, classifier)
+    _, margin = true_layer(emb.double(), layer, embed_norm, "standard", pooler, classifier)
+    label = 0 if float(margin[0, 0]) > 0 else 1
+    gnet = network_of(tuple(to_device(x, "cuda") for x in parts), "standard")
+    ge = emb.cuda()
+    maker = BoundsMaker(compact_from=0)
+    cap = F.CapturedVerifier(maker, gnet, ge, 4, label, 2.0)
+    queries = [([1, 2, 3, 4], [0.004, 0.004, 0.004, 0.004]), ([4, 3, 2, 1], [0.001, 0.02, 0.008, 0.3]),
+               ([1, 1, 1, 1], [0.0005, 0.009, 0.0078125, 1.0]), ([2, 4, 2, 4], [0.012, 0.012, 0.25, 0.004]),
+               ([1, 2, 3, 4], [0.004, 0.004, 0.004, 0.004])]
+    seen = set()
+    for idx, radii in queries:
+        print(f"[case] captured replay on the compact input, positions {idx} radii {radii}", flush=True)
+        got = cap(idx, radii)
+        want = F.verify_safety_batch(maker, gnet, ge, idx, radii, label, 2.0)      # eager work between replays
+        torch.cuda.synchronize()
+        assert got == want, (idx, radii, got, want)
+        seen.update(got)
+    assert seen == {True, False}
