@@ -879,16 +879,21 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         //   the same with non-temporal loads                         warm 54.7 / 56.9   cold 55.3 / 57.9
         //   persistent, two tiles in registers, 4 wavefronts x 8     warm 41.8 / 43.8   cold 55 - 57 / 58 - 60
         // The persistent kernel is the one that is good at both, except for tanh, whose long per-neuron stage
-        // wants more workgroups on a CU than its registers allow: tanh keeps the first shape while its operands can
-        // be cached and takes the third when they cannot (traffic more than a quarter beyond the cache).
+        // wants more workgroups on a CU than its registers allow: tanh keeps the first shape.
+        // On [B, 32, 256, 512] with one operand set, where a launch moves more than the cache holds (MB: first /
+        // third / persistent shape, relu | tanh in us):
+        //    404:  60 /  78 /  62 |  61 /  79 /  65        537:  92 / 106 /  87 |  88 / 106 /  89
+        //    674: 144 / 130 / 134 | 143 / 132 / 140        808: 173 / 156 / 161 | 172 / 157 / 168
+        //   1347: 284 / 263 / 266 | 282 / 264 / 276       2013: 424 / 391 / 402 | 417 / 394 / 413
+        // so from 9/4 of the cache up (between the two sizes where the order flips) every mode takes the third.
         // Knob values 8 / 12 / 7 force the three one-tile shapes, 15 the persistent one.
         const long long traffic = 16LL * a.rows * a.D * a.H;
-        const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 5LL * (256LL << 20) / 4);
+        const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 9LL * (256LL << 20) / 4);
         bool pipelined = false;
         if constexpr (MODE != CONCRETIZE) {
             // (with fewer than two tiles per resident workgroup there is nothing to overlap: one tile each then)
             const long long n_tiles = (long long)a.rows * (a.H / 32);
-            pipelined = a.D > 128 && (tv == 15 || (MODE != TANH && tv != 7 && tv != 8 && tv != 12 &&
+            pipelined = a.D > 128 && (tv == 15 || (MODE != TANH && tv != 7 && tv != 8 && tv != 12 && !streams_from_hbm &&
                                                    n_tiles >= 4LL * faith::compute_units()));
             if (pipelined) launch_pipelined<MODE, Q, 8, 256, 8, 2>(a, st);
         }

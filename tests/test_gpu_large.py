@@ -72,27 +72,36 @@ def sl(x, r):
 @pytest.mark.parametrize("op,p,layout,shape", [
     ("relu", 2.0, "natural", (2100, 1024, 1024)),       # D_in = 1024: rows in the registers of sixteen wavefronts
     ("tanh", INF, "natural", (8200, 256, 1024)),        # register-resident kernel, one tile per workgroup
-    ("relu", 2.0, "natural", (8200, 256, 1024)),        # register-resident kernel, persistent workgroups
+    ("relu", 2.0, "natural", (8200, 256, 1024)),        # the same for another mode
+    ("relu", 2.0, "persistent", (8200, 256, 1024)),     # register-resident kernel, persistent workgroups (tuning knob 15)
     ("relu", 1.0, "natural", (300, 2048, 3600)),        # chunked walk (D_in > 1024), two reads
     ("tanh", 2.0, "transposed", (2100, 4096, 256)),     # transposed, resident (D_in = 256)
     ("relu", INF, "transposed", (2100, 1000, 1040)),    # transposed, general kernel
 ])
 def test_relaxation_rows(op, p, layout, shape):
+    from faith_amd import _lib
     L, A, B = shape
     say(f"large {op} p={p} {layout} [1, {L}, {A}, {B}]")
+    persistent = layout == "persistent"
+    if persistent:
+        layout = "natural"
     x = big_object((1, L, A, B), (1, L, A if layout == "transposed" else B), 11)
     lay = ops.LAYOUT_TRANSPOSED if layout == "transposed" else ops.LAYOUT_NATURAL
     fn = getattr(ops, op)
-    full = fn(*x, p, 0.01, 2, lay, True)
+    if persistent:
+        _lib.call("faith_tune_set", 0, 15)
+    try:
+        full = fn(*x, p, 0.01, 2, lay, True)
+    finally:
+        _lib.call("faith_tune_set", 0, 0)
     picks = rows_to_check(L, A * B)
-    # an object of this size streams from HBM: tanh then takes the register-resident kernel's sixteen-wavefront
-    # thread shape, where a single row would take the four-wavefront one (another reduction tree), so the slices
-    # are held to the shape of the whole (tuning knob 7) and the comparison stays bit for bit; relu runs on
-    # persistent workgroups with the arithmetic of the four-wavefront shape (knob 8 for the slices)
-    from faith_amd import _lib
+    # an object of this size streams from HBM and takes the register-resident kernel's sixteen-wavefront thread
+    # shape, where a single row would take the four-wavefront one (another reduction tree), so the slices are held
+    # to the shape of the whole (tuning knob 7) and the comparison stays bit for bit; the persistent workgroups
+    # have the arithmetic of the four-wavefront shape (knob 8 for the slices)
     resident = layout == "natural" and A <= 256
     if resident:
-        _lib.call("faith_tune_set", 0, 7 if op == "tanh" else 8)
+        _lib.call("faith_tune_set", 0, 8 if persistent else 7)
     try:
         check_rows(f"{op} {layout}", full, lambda r: fn(*sl(x, r), p, 0.01, 2, lay, True), picks)
     finally:

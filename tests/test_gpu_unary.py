@@ -59,6 +59,21 @@ def test_unary_unordered_coefficients(kind):
     check(kind, make_input(kind, g, 4, 64, 128, ordered=False), 2.0, 0.05, 1)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("p", [1.0, 2.0, float("inf")])
+def test_unary_thread_shape_for_hbm_streams(kind, p):
+    """Objects whose traffic is far beyond the memory-side cache take the register-resident kernel's sixteen-wavefront
+    thread shape (tuning knob 7 forces it on a small object): against the oracle like every other shape."""
+    from faith_amd import _lib
+    g = torch.Generator().manual_seed(54)
+    x = make_input(kind, g, 3, 256, 96)
+    _lib.call("faith_tune_set", 0, 7)
+    try:
+        check(kind, x, p, 0.05, 2)
+    finally:
+        _lib.call("faith_tune_set", 0, 0)
+
+
 def test_exp_above_the_cap():
     """Pre-activations beyond 12: the reference continues exp by its tangent (Bounds.py:984-989)."""
     g = torch.Generator().manual_seed(53)
