@@ -618,6 +618,17 @@ def bench_layer(args, wl):
           "latency_us": round(per, 1), "latency_min_us": round(min(times) * 1e3 / len(positions), 1),
           "bound": "host", "achieved": 0.0, "peak": 1.0, "unit": "-", "frac": 0.0, "work": 0,
           "batch_latency_us": round(statistics.median(times) * 1e3, 1)}
+    # the same step with the input object written out in full (zero coefficient rows included), as the reference builds it
+    from faith_amd import Bounds
+    plain = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
+    for _ in range(3):
+        F.verify_safety_batch(plain, net, ge, positions, radii, 0, p)
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        F.verify_safety_batch(plain, net, ge, positions, radii, 0, p)
+        times.append((time.perf_counter() - t0) * 1e3)
+    e2["batch_latency_us_with_the_zero_rows_written_out"] = round(statistics.median(times) * 1e3, 1)
 
     # the same two, replayed from a HIP graph captured once (forward.CapturedVerifier)
     out = [e, e2]
