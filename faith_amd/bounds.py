@@ -347,11 +347,12 @@ class CompactBounds:
         lw, uw     [B, P, D, H]     the coefficients at those positions      (as _lw, _uw)
         lb, ub     [B, L, H]        the constant terms at every position     (as _lb, _ub)
 
-    `layer_norm` keeps the form; `matmul` / `dense` / `dense_group` run the affine kernels on the P rows
-    that are not zero (and on the constants, as an object with one zero coefficient row per position) and
-    return ordinary `Bounds`; every other attribute or method is that of `dense_form()`, the equal
-    `Bounds` object with the zeros written out.  Beyond the reference's surface, which carries the zeros
-    through every operator."""
+    `layer_norm` and `matmul` / `dense` / `dense_group` keep the form: they run their kernels on the P rows
+    that are not zero (the affine ones also on the constants, as an object with one zero coefficient row per
+    position); `attention_scores` of two compact objects -- the first operator that mixes positions -- takes
+    the kernel that writes the dense scores from the compact rows; every other attribute or method is that of
+    `dense_form()`, the equal `Bounds` object with the zeros written out (built on first use).  Beyond the
+    reference's surface, which carries the zeros through every operator."""
 
     collect_failures = Bounds.collect_failures
 
@@ -368,6 +369,7 @@ class CompactBounds:
         self.device = lw.device
         self.perturbed_words = getattr(args, "perturbed_words", 1)
         self._dense = None
+        self._intervals = None
 
     def _compact_like(self, lw, lb, uw, ub):
         return CompactBounds(self.args, self.p, self.eps, self.positions, lw, lb, uw, ub)
@@ -381,7 +383,7 @@ class CompactBounds:
         return self._dense
 
     def __getattr__(self, name):            # whatever is not defined here
-        if name.startswith("__") or name in ("_lw", "_lb", "_uw", "_ub", "_dense"):
+        if name.startswith("__") or name in ("_lw", "_lb", "_uw", "_ub", "_dense", "_intervals"):
             raise AttributeError(name)
         return getattr(self.dense_form(), name)
 
@@ -410,9 +412,37 @@ class CompactBounds:
         else:
             coeffs = ops.linear_group(lw, no_b, uw, no_b, weights, None)
             consts = ops.linear_group(no_w, lb, no_w, ub, weights, biases)
-        spread = lambda t: ops.spread_positions(t, self.positions, self.length)
-        return [Bounds(self.args, self.p, self.eps, lw=spread(w[0]), lb=c[1], uw=spread(w[2]), ub=c[3])
-                for w, c in zip(coeffs, consts)]
+        return [self._compact_like(w[0], c[1], w[2], c[3]) for w, c in zip(coeffs, consts)]
+
+    # ---- Bounds.py:319-326 on the rows that have coefficients; the constants are the bounds of the others
+    def concrete_intervals(self):
+        """(l, u) [B, L, H], as concretize() of the dense form gives them (computed once)."""
+        if self._intervals is None:
+            lb, ub = self._lb.contiguous(), self._ub.contiguous()
+            l, u = ops.concretize(self._lw.contiguous(), ops.gather_positions(lb, self.positions),
+                                  self._uw.contiguous(), ops.gather_positions(ub, self.positions),
+                                  self.p, self.eps, self.perturbed_words)
+            self._intervals = (ops.put_positions(lb, self.positions, l), ops.put_positions(ub, self.positions, u))
+        return self._intervals
+
+    # ---- VerifierForward.py:208-229 + Bounds.py:833-841 for two objects with coefficients at the same positions
+    def attention_scores(self, key, heads):
+        B, P, D, H = self._lw.shape
+        if (isinstance(key, CompactBounds) and key.positions is self.positions and key._lw.shape == self._lw.shape
+                and key._lb.shape == self._lb.shape and H % heads == 0
+                and ops.attention_scores_compact_fits(self.length, P, H // heads, D)):
+            x = (self._lw.contiguous(), self._lb.contiguous(), self._uw.contiguous(), self._ub.contiguous())
+            y = (key._lw.contiguous(), key._lb.contiguous(), key._uw.contiguous(), key._ub.contiguous())
+            x_l, _ = self.concrete_intervals()
+            y_l, y_u = key.concrete_intervals()
+            try:
+                out = ops.attention_scores_compact(x, y, x_l, y_l, y_u, self.positions, heads)
+            except _lib.FaithError as err:
+                if err.code != _lib.ERR_UNSUPPORTED:         # e.g. tensors that are not 16-byte aligned
+                    raise
+            else:
+                return Bounds(self.args, self.p, self.eps, lw=out[0], lb=out[1], uw=out[2], ub=out[3])
+        return self.dense_form().attention_scores(_written_out(key), heads)
 
     def matmul(self, W, bias=None):
         if isinstance(W, (Bounds, CompactBounds)) or W.dim() != 2:

@@ -1051,6 +1051,125 @@ int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, fl
     return faith::check_launch(who);
 }
 
+
+// ---------------------------------------------------------------------------------------------------------
+// Scores of a query and a key whose coefficients vanish outside P positions of every batch element: the
+// input of a verification query has coefficients at the perturbed position(s) only (VerifierForward.py:127-156),
+// and layer norm and dense layers keep it that way.  In Bounds.py:761-818 the x terms of z[i, m, j] are sums over
+// x.lw[i, m, :] and the y terms over y.lw[j, m, :], so z_lw[i, :, j] is zero unless i or j is one of those positions:
+//     i in S:  z[i, m, j] += sum_k a(j, k) split by sign against x.lw / x.uw [i, m, k]     (every j)
+//     j in S:  z[i, m, j] += sum_k b(i, k) split by sign against y.lw / y.uw [j, m, k]     (every i)
+// Only the rows of S exist in memory ([batch, P, D, heads * size], heads side by side).  A workgroup writes the
+// coordinates m0 ... m0 + 127 of one (batch element, head, i): first the P column values per coordinate (four lanes
+// per dot product), then the [128 x L] block, 16 bytes per lane -- zeros, the column values where j is in S and, in the
+// HEAVY launch (one workgroup per row i in S), the full row of x terms against a(j, k) staged in LDS as [k][j].
+// The LIGHT launch covers every i and leaves the rows of S to the other.  The work is 1 / L of the dense
+// contraction: this is a vector-ALU kernel bound by writing z.
+struct CompactArgs {
+    const float *xlw, *xuw, *ylw, *yuw;    // [batch, P, D, heads * size]
+    const float *x_l, *y_l, *y_u;          // [batch, L, heads * size]
+    const long long *positions;            // [batch, P], distinct within a batch element; outside 0 ... L-1: no such row
+    float *zlw, *zuw;                      // [batch * heads, L, D, L]
+    int L, P, D, heads, size, chunks;
+};
+constexpr int CS_MC = 128;
+
+template <bool HEAVY>
+__global__ void __launch_bounds__(256) scores_compact(const CompactArgs g) {
+    extern __shared__ __align__(16) float cs[];
+    const int L = g.L, P = g.P, size = g.size, pitch = g.heads * g.size;
+    float *col_l = cs, *col_u = cs + P * CS_MC;                       // [P][CS_MC]
+    float *alp = cs + 2 * P * CS_MC, *aln = alp + size * L, *aup = aln + size * L, *aun = aup + size * L;   // [size][L] each
+    int pid = blockIdx.x;
+    const int c = pid % g.chunks;  pid /= g.chunks;
+    const int r = pid % (HEAVY ? P : L);  pid /= (HEAVY ? P : L);
+    const int t = pid, b = t / g.heads, h = t - b * g.heads;
+    const long long *pos = g.positions + (size_t)b * P;
+    int i = r, pi = -1;
+    if (HEAVY) {
+        const long long at = pos[r];
+        if (at < 0 || at >= L) return;                                // no such row (uniform over the workgroup)
+        i = (int)at;  pi = r;
+    } else {
+        for (int p = 0; p < P; ++p)
+            if (pos[p] == i) return;                                  // a row of S: the other launch writes it
+    }
+    const int m0 = c * CS_MC, tid = threadIdx.x;
+
+    // ---- column values: b(i, :) against the key's rows of S
+    const float *beta = g.x_l + ((size_t)b * L + i) * pitch + (size_t)h * size;
+    for (int e = tid; e < 4 * P * CS_MC; e += 256) {                  // 4 * CS_MC is a multiple of 256: no lane sits out
+        const int part = e % 4, ml = (e / 4) % CS_MC, p = e / (4 * CS_MC);
+        float sl = 0.f, su = 0.f;
+        if (m0 + ml < g.D) {
+            const size_t row = (((size_t)b * P + p) * g.D + m0 + ml) * pitch + (size_t)h * size;
+            for (int k = 4 * part; k < size; k += 16) {
+                const float4 bt = *reinterpret_cast<const float4 *>(beta + k);
+                const float4 yl = *reinterpret_cast<const float4 *>(g.ylw + row + k);
+                const float4 yu = *reinterpret_cast<const float4 *>(g.yuw + row + k);
+#define FAITH_TERM(F)                                                        \
+    {                                                                        \
+        const float bp = fmaxf(bt.F, 0.f), bn = fminf(bt.F, 0.f);            \
+        sl += bp * yl.F + bn * yu.F;                                         \
+        su += bp * yu.F + bn * yl.F;                                         \
+    }
+                FAITH_TERM(x) FAITH_TERM(y) FAITH_TERM(z) FAITH_TERM(w)
+#undef FAITH_TERM
+            }
+        }
+        sl += __shfl_xor(sl, 1);  su += __shfl_xor(su, 1);
+        sl += __shfl_xor(sl, 2);  su += __shfl_xor(su, 2);
+        if (part == 0) { col_l[p * CS_MC + ml] = sl;  col_u[p * CS_MC + ml] = su; }
+    }
+    if (HEAVY) {
+        // a_l, a_u of this head, split by sign, as [k][j]
+        for (int e = tid; e < size * L; e += 256) {
+            const int j = e / size, k = e % size;
+            const size_t o = ((size_t)b * L + j) * pitch + (size_t)h * size + k;
+            const float al = g.y_l[o], au = g.y_u[o];
+            alp[k * L + j] = fmaxf(al, 0.f);  aln[k * L + j] = fminf(al, 0.f);
+            aup[k * L + j] = fmaxf(au, 0.f);  aun[k * L + j] = fminf(au, 0.f);
+        }
+    }
+    __syncthreads();
+
+    // ---- the block of z: 16 bytes (four columns j of one coordinate m) per lane and step
+    const size_t z0 = (((size_t)t * L + i) * g.D + m0) * L;
+    const int rows = min(CS_MC, g.D - m0);
+    for (int e4 = tid; e4 < rows * L / 4; e4 += 256) {
+        const int ml = (e4 * 4) / L, j0 = (e4 * 4) % L;
+        float vl[4] = {0.f, 0.f, 0.f, 0.f}, vu[4] = {0.f, 0.f, 0.f, 0.f};
+        if (HEAVY) {
+            const size_t row = (((size_t)b * P + pi) * g.D + m0 + ml) * pitch + (size_t)h * size;
+            for (int k = 0; k < size; k += 4) {
+                const float4 xl4 = *reinterpret_cast<const float4 *>(g.xlw + row + k);
+                const float4 xu4 = *reinterpret_cast<const float4 *>(g.xuw + row + k);
+                const float xl[4] = {xl4.x, xl4.y, xl4.z, xl4.w}, xu[4] = {xu4.x, xu4.y, xu4.z, xu4.w};
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    const int o = (k + kk) * L + j0;
+                    const float4 a1 = *reinterpret_cast<const float4 *>(alp + o), a2 = *reinterpret_cast<const float4 *>(aln + o);
+                    const float4 a3 = *reinterpret_cast<const float4 *>(aup + o), a4 = *reinterpret_cast<const float4 *>(aun + o);
+                    vl[0] += a1.x * xl[kk] + a2.x * xu[kk];  vu[0] += a3.x * xu[kk] + a4.x * xl[kk];
+                    vl[1] += a1.y * xl[kk] + a2.y * xu[kk];  vu[1] += a3.y * xu[kk] + a4.y * xl[kk];
+                    vl[2] += a1.z * xl[kk] + a2.z * xu[kk];  vu[2] += a3.z * xu[kk] + a4.z * xl[kk];
+                    vl[3] += a1.w * xl[kk] + a2.w * xu[kk];  vu[3] += a3.w * xu[kk] + a4.w * xl[kk];
+                }
+            }
+        }
+        for (int p = 0; p < P; ++p) {
+            const long long jp = pos[p] - j0;
+            if (jp >= 0 && jp < 4) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (q == (int)jp) { vl[q] += col_l[p * CS_MC + ml];  vu[q] += col_u[p * CS_MC + ml]; }
+            }
+        }
+        *reinterpret_cast<float4 *>(g.zlw + z0 + (size_t)e4 * 4) = make_float4(vl[0], vl[1], vl[2], vl[3]);
+        *reinterpret_cast<float4 *>(g.zuw + z0 + (size_t)e4 * 4) = make_float4(vu[0], vu[1], vu[2], vu[3]);
+    }
+}
+
 }  // namespace
 
 extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
@@ -1164,6 +1283,55 @@ extern "C" int faith_attention_scores(float *x_l, float *y_l, float *x_u, float 
     return dot_entry<false>("faith_attention_scores", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
                             z_lb, z_ub, z_lw, z_uw, batch_size * heads, length_x, length_y, head_size, dim_in, epsilon, q,
                             words, HEADS_X | HEADS_Y, heads, stream);
+}
+
+extern "C" int faith_attention_scores_compact(const float *x_l, const float *y_l, const float *y_u, const float *x_lb,
+                                              const float *x_ub, const float *y_lb, const float *y_ub, const float *x_lw,
+                                              const float *x_uw, const float *y_lw, const float *y_uw,
+                                              const long long *positions, float *z_lb, float *z_ub, float *z_lw,
+                                              float *z_uw, int batch_size, int heads, int length, int n_positions,
+                                              int head_size, int dim_in, void *stream) {
+    const char *who = "faith_attention_scores_compact";
+    FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(y_u);
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
+    FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw); FAITH_NOT_NULL(positions);
+    FAITH_NOT_NULL(z_lb); FAITH_NOT_NULL(z_ub); FAITH_NOT_NULL(z_lw); FAITH_NOT_NULL(z_uw);
+    FAITH_ALIGNED4(x_lb); FAITH_ALIGNED4(x_ub); FAITH_ALIGNED4(y_lb); FAITH_ALIGNED4(y_ub); FAITH_ALIGNED4(z_lb); FAITH_ALIGNED4(z_ub);
+    FAITH_REQUIRE(batch_size > 0 && heads > 0 && length > 0 && n_positions > 0 && head_size > 0 && dim_in > 0, FAITH_ERR_SHAPE,
+                  "%s: batch=%d heads=%d length=%d positions=%d head size=%d dim_in=%d must be positive", who, batch_size,
+                  heads, length, n_positions, head_size, dim_in);
+    const long long B = (long long)batch_size * heads;
+    FAITH_REQUIRE(B <= 0x7fffffffLL && B * length * dim_in <= 0x7fffffffLL && (long long)heads * head_size <= 0x7fffffffLL &&
+                  (long long)batch_size * n_positions * dim_in <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "%s: batch*heads*length*dim_in exceeds 2^31", who);
+    // the kernel reads and writes 16 bytes at a time and keeps the key's intervals of one head in LDS; dim_in == 1 is the
+    // interval shortcut of the dense entry point (Bounds.py:711-721), which this one does not have
+    const size_t lds = ((size_t)2 * n_positions * CS_MC + (size_t)4 * head_size * length) * sizeof(float);
+    FAITH_REQUIRE(dim_in > 1 && length % 4 == 0 && head_size % 4 == 0 && lds <= 65536 && ((uintptr_t)positions & 7) == 0 &&
+                  faith::aligned(x_l, 16) && faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
+                  faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) && faith::aligned(y_lw, 16) &&
+                  faith::aligned(y_uw, 16) && faith::aligned(z_lw, 16) && faith::aligned(z_uw, 16), FAITH_ERR_UNSUPPORTED,
+                  "%s: needs dim_in > 1, length and head size multiples of 4, 16-byte aligned tensors and "
+                  "8 * positions * 128 + 16 * head size * length <= 65536 bytes of LDS", who);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    CompactArgs c{x_lw, x_uw, y_lw, y_uw, x_l, y_l, y_u, positions, z_lw, z_uw, length, n_positions, dim_in, heads, head_size,
+                  (dim_in + CS_MC - 1) / CS_MC};
+    const long long light = B * length * c.chunks, heavy = B * n_positions * c.chunks;
+    FAITH_REQUIRE(light <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    hipLaunchKernelGGL(scores_compact<true>, dim3((unsigned)heavy), dim3(256), lds, st, c);
+    hipLaunchKernelGGL(scores_compact<false>, dim3((unsigned)light), dim3(256), (size_t)2 * n_positions * CS_MC * sizeof(float), st, c);
+    // constant terms: the dense kernel (it reads constants and intervals only)
+    DotArgs g{nullptr, nullptr, nullptr, nullptr, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, nullptr, nullptr, z_lb, z_ub,
+              (int)B, length, length, dim_in, head_size};
+    g.ox = {heads * head_size, heads, head_size};
+    g.oy = {heads * head_size, heads, head_size};
+    g.oz = {length, 1, length};
+    g.heads = heads;
+    g.side_by_side = HEADS_X | HEADS_Y;
+    const long long b_tiles = B * ((length + BT_T - 1) / BT_T) * ((length + BT_T - 1) / BT_T);
+    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    hipLaunchKernelGGL(dot_b<false>, dim3((unsigned)b_tiles), dim3(256), 0, st, g);
+    return faith::check_launch(who);
 }
 
 extern "C" int faith_attention_context(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,

@@ -685,6 +685,69 @@ def attention_scores(x, y, heads, p, eps, words=1):
     return zlw, zlb, zuw, zub
 
 
+def gather_positions(t, positions):
+    """[B, L, ...] -> [B, P, ...]: row positions[b, i] of batch element b (the inverse of spread_positions on
+    those rows; data movement only, nothing waits for the device)."""
+    B, P = positions.shape
+    out = _empty(B, P, *t.shape[2:], device=t.device)
+    index = positions.reshape(B, P, *([1] * (t.dim() - 2))).expand(B, P, *t.shape[2:])
+    return torch.gather(t, 1, index, out=out)
+
+
+def put_positions(t, positions, rows):
+    """A copy of t [B, L, ...] with row positions[b, i] of batch element b replaced by rows[b, i]."""
+    B, P = positions.shape
+    out = _empty_like(t)
+    out.copy_(t)
+    key = (B, str(t.device))
+    if key not in _BATCH_INDEX:
+        _BATCH_INDEX[key] = torch.arange(B, device=t.device)[:, None]
+    out[_BATCH_INDEX[key], positions] = rows
+    return out
+
+
+def attention_scores_compact_fits(length, n_positions, head_size, dim_in):
+    """True if attention_scores_compact takes operands of this shape (16-byte aligned tensors assumed)."""
+    return (dim_in > 1 and length % 4 == 0 and head_size % 4 == 0
+            and 8 * n_positions * 128 + 16 * head_size * length <= 65536)
+
+
+def attention_scores_compact(x, y, x_l, y_l, y_u, positions, heads):
+    """attention_scores for a query and a key whose coefficients vanish outside `positions` [B, P] (int64, on the
+    device), with only those coefficient rows in memory:
+
+    x, y: (lw [B, P, D, heads*size], lb [B, L, heads*size], uw, ub); x_l, y_l, y_u [B, L, heads*size]: the
+    concrete lower bound of x and both bounds of y (concretize of the P rows, the constants elsewhere).
+    Returns what attention_scores returns for the operands with the zeros written out.  Raises FaithError
+    (FAITH_ERR_UNSUPPORTED) for shapes the kernel does not take: see attention_scores_compact_fits."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    _check("x.lw", xlw); _check("x.uw", xuw, xlw.shape); _check("y.lw", ylw, xlw.shape); _check("y.uw", yuw, xlw.shape)
+    _check("x.lb", xlb); _check("x.ub", xub, xlb.shape); _check("y.lb", ylb, xlb.shape); _check("y.ub", yub, xlb.shape)
+    _check("x_l", x_l, xlb.shape); _check("y_l", y_l, xlb.shape); _check("y_u", y_u, xlb.shape)
+    if xlw.dim() != 4 or xlb.dim() != 3:
+        raise ValueError(f"x.lw {tuple(xlw.shape)} must be [B, P, dim_in, heads*size] and x.lb {tuple(xlb.shape)} [B, L, heads*size]")
+    B, P, D, H = xlw.shape
+    L = xlb.shape[1]
+    if xlb.shape[0] != B or xlb.shape[2] != H:
+        raise ValueError(f"x.lw {tuple(xlw.shape)} and x.lb {tuple(xlb.shape)} disagree in batch or width")
+    if heads <= 0 or H % heads:
+        raise ValueError(f"{heads} heads do not divide a row of {H}")
+    if positions.dtype != torch.int64 or tuple(positions.shape) != (B, P) or positions.device != xlw.device \
+            or not positions.is_contiguous():
+        raise ValueError(f"positions must be a contiguous int64 tensor [{B}, {P}] on {xlw.device}")
+    dev = xlw.device
+    zlw = _empty(B * heads, L, D, L, device=dev)
+    zuw = _empty_like(zlw)
+    zlb = _empty(B * heads, L, L, device=dev)
+    zub = _empty_like(zlb)
+    with _on(dev):
+        _lib.call("faith_attention_scores_compact", _ptr(x_l), _ptr(y_l), _ptr(y_u), _ptr(xlb), _ptr(xub), _ptr(ylb),
+                  _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw), positions.data_ptr(), _ptr(zlb), _ptr(zub),
+                  _ptr(zlw), _ptr(zuw), B, heads, L, P, H // heads, D, _stream(xlw))
+    return zlw, zlb, zuw, zub
+
+
 def attention_context(x, y, p, eps, words=1):
     """Context of all heads: probabilities x (lw [B*heads, Lx, D, Lk], lb [B*heads, Lx, Lk], uw, ub) times the
     value bounds y as the dense layer leaves them (lw [B, Lk, D, heads*size], lb [B, Lk, heads*size], uw, ub).

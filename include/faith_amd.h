@@ -396,6 +396,33 @@ int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u,
                            int q, int words, void *stream);
 
 /*
+ * The same scores for a query and a key whose coefficients vanish outside n_positions positions of
+ * every batch element, with only those rows in memory.  The input of a verification query has
+ * coefficients at the perturbed position(s) alone (VerifierForward.py:127-156) and keeps that form
+ * through layer norm and dense layers; in Bounds.dot_product (Bounds.py:761-818) the x terms of
+ * z_lw[i, :, j] read x_lw[i] and the y terms y_lw[j], so z_lw[i, :, j] is zero unless i or j is one
+ * of those positions, and 1 / length of the dense contraction is left:
+ *   x_lw, x_uw, y_lw, y_uw [batch, n_positions, dim_in, heads * head_size]   coefficient rows of the positions
+ *   positions              [batch, n_positions] int64 on the device, distinct within a batch element
+ *                          (a value outside 0 ... length-1 means that the row is not there)
+ *   x_lb, x_ub, y_lb, y_ub [batch, length, heads * head_size]                constants of every position
+ *   x_l, y_l, y_u          [batch, length, heads * head_size]  IN: the concrete bounds (faith_concretize of the
+ *                          rows that have coefficients, the constants themselves elsewhere)
+ *   z_* as faith_attention_scores writes them, zeros included.
+ * FAITH_ERR_UNSUPPORTED unless dim_in > 1, length % 4 == 0, head_size % 4 == 0, the tensors are 16-byte aligned
+ * and 8 * n_positions * 128 + 16 * head_size * length <= 65536 (bytes of LDS): take the dense entry point then.
+ */
+int faith_attention_scores_compact(const float *x_l, const float *y_l, const float *y_u,
+                                   const float *x_lb, const float *x_ub,
+                                   const float *y_lb, const float *y_ub,
+                                   const float *x_lw, const float *x_uw,
+                                   const float *y_lw, const float *y_uw,
+                                   const long long *positions,
+                                   float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                                   int batch_size, int heads, int length, int n_positions,
+                                   int head_size, int dim_in, void *stream);
+
+/*
  * Attention context with the values read, and the result written, where the dense layers want
  * them.  Replaces transpose_for_scores on the values, Bounds.context (Bounds.py:843-850) and
  * transpose_back (VerifierForward.py:253-263).

@@ -20,21 +20,22 @@ from tests.test_layer_pipeline import HIDDEN, LENGTH, build, network_of, two_lay
 pytestmark = pytest.mark.gpu
 
 
-def compact_and_dense(seed, B=3, P=2, D=10, H=24, L=5, words=1, shared=False):
+def compact_and_dense(seed, B=3, P=2, D=10, H=24, L=5, words=1, shared=False, positions=None, p=2.0):
     from faith_amd import Bounds, CompactBounds
     g = torch.Generator().manual_seed(seed)
-    positions = torch.stack([torch.randperm(L, generator=g)[:P] for _ in range(B)])
+    at = positions
+    positions = torch.stack([torch.randperm(L, generator=g)[:P] for _ in range(B)]) if at is None else at.cpu()
     lw = torch.randn(B, P, D, H, generator=g)
     uw = lw if shared else lw + 0.05 * torch.rand(B, P, D, H, generator=g)
     lb = torch.randn(B, L, H, generator=g)
     ub = lb if shared else lb + 0.3 * torch.rand(B, L, H, generator=g)
     args = SimpleNamespace(perturbed_words=words)
     dev = lambda t: t.cuda()
-    c = CompactBounds(args, 2.0, 0.1, dev(positions), dev(lw), dev(lb), dev(lw if shared else uw), dev(ub))
+    c = CompactBounds(args, p, 0.1, dev(positions) if at is None else at, dev(lw), dev(lb), dev(lw if shared else uw), dev(ub))
     rows = torch.arange(B)[:, None]
     dlw = torch.zeros(B, L, D, H); dlw[rows, positions] = lw
     duw = torch.zeros(B, L, D, H); duw[rows, positions] = uw
-    d = Bounds(args, 2.0, 0.1, lw=dev(dlw), lb=dev(lb), uw=dev(duw), ub=dev(ub))
+    d = Bounds(args, p, 0.1, lw=dev(dlw), lb=dev(lb), uw=dev(duw), ub=dev(ub))
     return c, d
 
 
@@ -100,14 +101,14 @@ def test_layer_norm_keeps_the_form_and_the_bits():
 
 @pytest.mark.parametrize("shape", [(3, 2, 10, 24, 5, 16), (2, 1, 64, 64, 9, 96), (5, 3, 33, 20, 4, 7), (1, 1, 256, 256, 32, 256)])
 def test_dense_layers_on_the_rows_that_are_not_zero(shape):
-    from faith_amd import Bounds
+    from faith_amd import CompactBounds
     B, P, D, H, L, N = shape
     g = torch.Generator().manual_seed(B * 100 + N)
     c, d = compact_and_dense(6, B, P, D, H, L)
     for bias in (True, False):
         layer = layer_of(g, H, N, bias)
         out = c.dense(layer)
-        assert isinstance(out, Bounds)
+        assert isinstance(out, CompactBounds) and out.positions is c.positions
         at_the_bar(out, d.dense(layer), f"dense {shape} bias={bias}", d, layer.weight)
         at_the_bar(c.matmul(layer.weight, layer.bias), d.matmul(layer.weight, layer.bias), "matmul", d, layer.weight)
     # positions without coefficients get exact zeros, whatever the buffer held before
@@ -123,6 +124,91 @@ def test_dense_layers_on_the_rows_that_are_not_zero(shape):
         at_the_bar(got, want, f"dense_group of two shapes {shape}", d, layer.weight)
 
 
+def score_terms(x, y, heads):
+    """sum_k |a| |x.w| + |b| |y.w| per coefficient of the scores and the like for the constants: what two fp32
+    summations of the same products in different orders may differ by, up to KAPPA * u."""
+    (xl, xu), (yl, yu) = x.concretize(), y.concretize()
+    f = lambda t: t.double().cpu()
+    B, L, D, H = x.lw.shape
+    size = H // heads
+    heads_of = lambda t: f(t).reshape(B, L, *t.shape[2:-1], heads, size)
+    xa, ya = heads_of(x.lw.abs() + x.uw.abs()), heads_of(y.lw.abs() + y.uw.abs())          # [B, L, D, h, k]
+    a, b = heads_of(yl.abs() + yu.abs()), heads_of(xl.abs())                                 # [B, L, h, k]
+    w = torch.einsum("bjhk,bimhk->bhimj", a, xa) + torch.einsum("bihk,bjmhk->bhimj", b, ya)
+    xb, yb = heads_of(x.lb.abs() + x.ub.abs()), heads_of(y.lb.abs() + y.ub.abs())
+    c = torch.einsum("bjhk,bihk->bhij", a, xb + b) + torch.einsum("bihk,bjhk->bhij", b, yb)
+    return w.reshape(B * heads, L, D, L), c.reshape(B * heads, L, L)
+
+
+@pytest.mark.parametrize("shape", [(3, 1, 24, 2, 16, 8), (2, 2, 64, 4, 16, 12), (5, 3, 130, 3, 20, 16),
+                                   (4, 1, 256, 4, 64, 32), (1, 2, 512, 4, 64, 32)])
+@pytest.mark.parametrize("p", [2.0, float("inf"), 1.0])
+def test_scores_from_compact_operands(shape, p):
+    """Query and key with coefficients at the same few positions: the kernel that writes the dense scores from the
+    compact rows against the dense kernel on the operands with the zeros written out."""
+    from faith_amd import Bounds, ops
+    B, P, D, heads, size, L = shape
+    words = 2 if D % 2 == 0 and P == 2 else 1
+    print(f"[case] compact scores B={B} P={P} D={D} heads={heads} size={size} L={L} p={p} words={words}", flush=True)
+    assert ops.attention_scores_compact_fits(L, P, size, D)
+    cq, dq = compact_and_dense(31, B, P, D, heads * size, L, words=words, p=p)
+    ck, dk = compact_and_dense(32, B, P, D, heads * size, L, words=words, p=p, positions=cq.positions)
+    got, want = cq.attention_scores(ck, heads), dq.attention_scores(dk, heads)
+    assert isinstance(got, Bounds) and got.lw.shape == (B * heads, L, D, L)
+    tw, tb = score_terms(dq, dk, heads)
+    for name, terms in (("lw", tw), ("uw", tw), ("lb", tb), ("ub", tb)):
+        x, y = getattr(got, name), getattr(want, name)
+        tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
+        over = float(((x.double() - y.double()).abs().cpu() / tol).max())
+        assert over <= 1.0, f"scores.{name}: {over:.2f} of the accumulation-aware bar"
+    # exact zeros wherever neither the query's nor the key's position has coefficients
+    at = cq.positions.cpu()
+    has = torch.zeros(B, L, dtype=torch.bool)
+    has[torch.arange(B)[:, None], at] = True
+    neither = ~(has[:, :, None] | has[:, None, :])                                     # [B, i, j]
+    neither = neither[:, None].expand(B, heads, L, L).reshape(B * heads, L, L)
+    lw = got.lw.cpu().permute(0, 1, 3, 2)                                             # [B*heads, i, j, m]
+    assert float(lw[neither].abs().max()) == 0.0 and float(got.uw.cpu().permute(0, 1, 3, 2)[neither].abs().max()) == 0.0
+
+
+def test_scores_from_compact_operands_fall_back_to_the_dense_kernel():
+    """Shapes the compact kernel does not take (a length that is no multiple of 4, a key with other positions, an
+    ordinary key): the dense kernel on the written-out operands, same results as for ordinary objects."""
+    from faith_amd import ops
+    B, P, D, heads, size, L = 2, 1, 24, 2, 8, 6
+    assert not ops.attention_scores_compact_fits(L, P, size, D)
+    cq, dq = compact_and_dense(33, B, P, D, heads * size, L)
+    ck, dk = compact_and_dense(34, B, P, D, heads * size, L, positions=cq.positions)
+    same_bits(cq.attention_scores(ck, heads), dq.attention_scores(dk, heads), "length 6")
+    cq, dq = compact_and_dense(35, B, P, D, heads * size, 8)
+    ck, dk = compact_and_dense(36, B, P, D, heads * size, 8)                          # positions of its own
+    same_bits(cq.attention_scores(ck, heads), dq.attention_scores(dk, heads), "other positions")
+    same_bits(cq.attention_scores(dk, heads), dq.attention_scores(dk, heads), "ordinary key")
+    same_bits(dq.attention_scores(ck, heads), dq.attention_scores(dk, heads), "ordinary query")
+
+
+def test_compact_scores_entry_point_checks_its_arguments():
+    from faith_amd import _lib, ops
+    cq, _ = compact_and_dense(37, 2, 1, 24, 16, 8)
+    ck, _ = compact_and_dense(38, 2, 1, 24, 16, 8, positions=cq.positions)
+    x = (cq._lw, cq._lb, cq._uw, cq._ub)
+    y = (ck._lw, ck._lb, ck._uw, ck._ub)
+    (x_l, _), (y_l, y_u) = cq.concrete_intervals(), ck.concrete_intervals()
+    with pytest.raises(ValueError):
+        ops.attention_scores_compact(x, y, x_l, y_l, y_u, cq.positions.int(), 2)
+    with pytest.raises(ValueError):
+        ops.attention_scores_compact(x, y, x_l, y_l, y_u, cq.positions, 3)
+    with pytest.raises(_lib.FaithError) as err:                 # head size 2: not a multiple of 4
+        ops.attention_scores_compact(x, y, x_l, y_l, y_u, cq.positions, 8)
+    assert err.value.code == _lib.ERR_UNSUPPORTED
+    # a position outside the sentence: that row is not there, nothing is read or written out of bounds
+    far = cq.positions.clone()
+    far[0, 0] = 1000
+    out = ops.attention_scores_compact(x, y, x_l, y_l, y_u, far, 2)
+    torch.cuda.synchronize()
+    assert float(out[0][:2].abs().max()) == 0.0 and float(out[0][2:].abs().max()) > 0.0
+
+
 def test_compact_object_matches_the_oracle():
     """Against the CPU oracle directly (not only against the HIP path's own dense object)."""
     g = torch.Generator().manual_seed(8)
@@ -135,10 +221,20 @@ def test_compact_object_matches_the_oracle():
     at_the_bar(got, want, "layer norm + dense against the oracle")
 
 
+def sentence(emb, length):
+    """The test network's embeddings at another length (6 positions: the scores of compact operands fall back to
+    the dense kernel; a multiple of 4: they take the compact one)."""
+    if length == emb.shape[1]:
+        return emb
+    return torch.randn(1, length, emb.shape[2], generator=torch.Generator().manual_seed(length))
+
+
+@pytest.mark.parametrize("length", [LENGTH, 8])
 @pytest.mark.parametrize("mode", ["no_var", "standard"])
-def test_propagation_from_the_compact_input_gives_the_ordinary_ones_margins(mode):
+def test_propagation_from_the_compact_input_gives_the_ordinary_ones_margins(mode, length):
     from faith_amd import Bounds, BoundsMaker, CompactBounds
     layer, embed_norm, pooler, classifier, emb = build(7, mode)
+    emb = sentence(emb, length)
     gparts = tuple(to_device(x, "cuda") for x in (layer, embed_norm, pooler, classifier))
     ge = emb.cuda()
     plain = lambda p_, e_, lw, lb, uw, ub: Bounds(None, p_, e_, lw=lw, lb=lb, uw=uw, ub=ub)
@@ -146,8 +242,8 @@ def test_propagation_from_the_compact_input_gives_the_ordinary_ones_margins(mode
     assert isinstance(F.bound_input(maker, ge, 2, 0.02, 1, 2.0), CompactBounds)
     # an object this small is written out at once unless the maker is told otherwise
     assert isinstance(F.bound_input(BoundsMaker(), ge, 2, 0.02, 1, 2.0), Bounds)
-    assert isinstance(F.bound_inputs(BoundsMaker(compact_from=4 * 3 * LENGTH * HIDDEN * HIDDEN), ge, [1, 2, 3], [0.1] * 3), CompactBounds)
-    assert isinstance(F.bound_inputs(BoundsMaker(compact_from=4 * 3 * LENGTH * HIDDEN * HIDDEN + 1), ge, [1, 2, 3], [0.1] * 3), Bounds)
+    assert isinstance(F.bound_inputs(BoundsMaker(compact_from=4 * 3 * length * HIDDEN * HIDDEN), ge, [1, 2, 3], [0.1] * 3), CompactBounds)
+    assert isinstance(F.bound_inputs(BoundsMaker(compact_from=4 * 3 * length * HIDDEN * HIDDEN + 1), ge, [1, 2, 3], [0.1] * 3), Bounds)
     assert isinstance(F.bound_input(maker, ge, 2, 0.02, 1, 2.0, ibp=True), Bounds)
 
     def run(make):
@@ -163,6 +259,13 @@ def test_propagation_from_the_compact_input_gives_the_ordinary_ones_margins(mode
         assert float((a - b).abs().max()) <= 1e-5 * max(float(b.abs().max()), 1.0), name
     assert safe_c == safe_d
     assert float((l_c - l_d).abs().max()) <= 1e-4 and float((u_c - u_d).abs().max()) <= 1e-4
+    # and the oracle's
+    omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)
+    x = F.bound_input(omake, emb, 2, 0.02, 1, 2.0, embed_norm, mode)
+    _, _, o_out = F.bound_layer(x, layer, mode, "relu")
+    for name in ("lw", "lb", "uw", "ub"):
+        a, b = getattr(out_c, name).double().cpu(), getattr(o_out, name).double()
+        assert float((a - b).abs().max()) <= 2e-4 * max(float(b.abs().max()), 1.0), name
 
 
 @pytest.mark.parametrize("mode", ["no_var", "standard"])
@@ -188,11 +291,13 @@ def test_two_perturbed_words_from_the_compact_input(mode):
     assert float((l_c.cpu() - ol).abs().max()) <= 2e-3 and float((u_c.cpu() - ou).abs().max()) <= 2e-3
 
 
-def test_search_from_the_compact_input_finds_the_same_radii():
+@pytest.mark.parametrize("length", [LENGTH, 8])
+def test_search_from_the_compact_input_finds_the_same_radii(length):
     """One at a time, batched, with persistent buffers and from a captured graph: the radii of the search on the
     ordinary object (a verdict within rounding of its threshold may fall either way: one step)."""
     from faith_amd import Bounds, BoundsMaker, ops
     layer, embed_norm, pooler, classifier, emb = build(11, "no_var")
+    emb = sentence(emb, length)
     parts = (layer, embed_norm, pooler, classifier)
     _, margin = true_layer(emb.double(), layer, embed_norm, "no_var", pooler, classifier)
     label = 0 if float(margin[0, 0]) > 0 else 1
@@ -217,9 +322,11 @@ def test_search_from_the_compact_input_finds_the_same_radii():
         assert abs(a - b) <= step + 1e-12 and abs(a - c) <= step + 1e-12
 
 
-def test_captured_graph_on_the_compact_input_follows_new_positions_and_radii():
+@pytest.mark.parametrize("length", [LENGTH, 8])
+def test_captured_graph_on_the_compact_input_follows_new_positions_and_radii(length):
     from faith_amd import BoundsMaker
     layer, embed_norm, pooler, classifier, emb = build(11, "standard")
+    emb = sentence(emb, length)
     parts = (layer, embed_norm, pooler, classifier)
     _, margin = true_layer(emb.double(), layer, embed_norm, "standard", pooler, classifier)
     label = 0 if float(margin[0, 0]) > 0 else 1
@@ -238,4 +345,4 @@ def test_captured_graph_on_the_compact_input_follows_new_positions_and_radii():
         torch.cuda.synchronize()
         assert got == want, (idx, radii, got, want)
         seen.update(got)
-    assert seen == {True, False}
+    assert len(seen) == 2 or length != LENGTH                 # at the test network's own length both verdicts occur
