@@ -577,6 +577,13 @@ def bench_layer(args, wl):
     ge = emb.cuda()
     net = SimpleNamespace(embedding_norm=gparts[1], layers=[gparts[0]], pooler=gparts[2], classifier=gparts[3],
                           layer_norm="no_var", hidden_act="relu")
+    if args.layer_only:
+        # under a profiler: ten batched propagations of the sentence's 30 positions and nothing else
+        positions = list(range(1, length - 1))
+        for _ in range(10):
+            F.verify_safety_batch(gmake, net, ge, positions, [eps] * len(positions), 0, p)
+        torch.cuda.synchronize()
+        return []
     single = lambda: F.verify_safety(gmake, net, ge, 3, eps, 0, p)      # ends with the verdict on the host
     t0 = time.time()
     while time.time() - t0 < max(WARM_SECONDS, 0.05):
@@ -675,6 +682,8 @@ def main():
     ap.add_argument("--configs", default="0,2,3,4", help="extra configurations to report under 'ops'")
     ap.add_argument("--cold-only", action="store_true",
                     help="for counter runs: only cold launches of the configuration-1 relaxations and of the plain copy")
+    ap.add_argument("--layer-only", action="store_true",
+                    help="for runs under rocprofv3: ten batched propagations of the encoder layer (30 positions each), no timing")
     ap.add_argument("--profile", action="store_true",
                     help="for runs under rocprofv3: warm up by count only, so the trace stays small")
     args = ap.parse_args()
@@ -698,6 +707,9 @@ def main():
 
     if args.cold_only:
         run_cold_only(ops, wl)
+        return
+    if args.layer_only:
+        print(json.dumps({"ops": bench_layer(args, wl)}))
         return
 
     prop = torch.cuda.get_device_properties(0)
