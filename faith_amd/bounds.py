@@ -399,20 +399,27 @@ class CompactBounds:
 
     # ---- Bounds.py:397-413, :1016-1025
     def _affine(self, weights, biases):
-        """The affine kernel twice: the coefficients of the P positions that have any (with zero constants,
-        whose results are dropped), and the constants of all positions (with one zero coefficient row each)."""
-        B, P, D, H = self._lw.shape
-        dev = self._lw.device
-        no_b = ops.zeros(B, P, H, device=dev)
-        no_w = ops.zeros(B, self.length, 1, H, device=dev)
-        lw, lb, uw, ub = self._lw.contiguous(), self._lb.contiguous(), self._uw.contiguous(), self._ub.contiguous()
-        if len(weights) == 1:
-            coeffs = [ops.linear(lw, no_b, uw, no_b, weights[0], None)]
-            consts = [ops.linear(no_w, lb, no_w, ub, weights[0], biases[0])]
-        else:
-            coeffs = ops.linear_group(lw, no_b, uw, no_b, weights, None)
-            consts = ops.linear_group(no_w, lb, no_w, ub, weights, biases)
-        return [self._compact_like(w[0], c[1], w[2], c[3]) for w, c in zip(coeffs, consts)]
+        """The affine kernels on the P coefficient rows per batch element and the L constant rows: the entry points
+        that count the two separately."""
+        c = (self._lw.contiguous(), self._lb.contiguous(), self._uw.contiguous(), self._ub.contiguous())
+        return [self._compact_like(*out) for out in ops.linear_rows(*c, weights, biases)]
+
+    def matmul(self, W, bias=None):
+        if isinstance(W, (Bounds, CompactBounds)) or W.dim() != 2:
+            return self.dense_form().matmul(W, bias)
+        return self._affine([W.contiguous()], [bias])[0]
+
+    def dense(self, dense):
+        bias = getattr(dense, "bias", None)
+        return self.matmul(dense.weight.detach(), None if bias is None else bias.detach().contiguous())
+
+    def dense_group(self, layers):
+        layers = list(layers)
+        if len(layers) > 3 or len({tuple(layer.weight.shape) for layer in layers}) != 1:
+            return [self.dense(layer) for layer in layers]
+        weights = [layer.weight.detach().contiguous() for layer in layers]
+        biases = [None if getattr(layer, "bias", None) is None else layer.bias.detach().contiguous() for layer in layers]
+        return self._affine(weights, biases)
 
     # ---- Bounds.py:319-326 on the rows that have coefficients; the constants are the bounds of the others
     def concrete_intervals(self):
@@ -443,23 +450,6 @@ class CompactBounds:
             else:
                 return Bounds(self.args, self.p, self.eps, lw=out[0], lb=out[1], uw=out[2], ub=out[3])
         return self.dense_form().attention_scores(_written_out(key), heads)
-
-    def matmul(self, W, bias=None):
-        if isinstance(W, (Bounds, CompactBounds)) or W.dim() != 2:
-            return self.dense_form().matmul(W, bias)
-        return self._affine([W.contiguous()], [bias])[0]
-
-    def dense(self, dense):
-        bias = getattr(dense, "bias", None)
-        return self.matmul(dense.weight.detach(), None if bias is None else bias.detach().contiguous())
-
-    def dense_group(self, layers):
-        layers = list(layers)
-        if len(layers) > 3 or len({tuple(layer.weight.shape) for layer in layers}) != 1:
-            return [self.dense(layer) for layer in layers]
-        weights = [layer.weight.detach().contiguous() for layer in layers]
-        biases = [None if getattr(layer, "bias", None) is None else layer.bias.detach().contiguous() for layer in layers]
-        return self._affine(weights, biases)
 
 
 class BoundsMaker:

@@ -594,20 +594,19 @@ static void choose_tile(long long mw, int dim_out, int dim_y_out, int *tm, int *
     }
 }
 
-extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
-                                         const float *W, const float *bias, float *y_lb, float *y_ub, float *y_lw,
-                                         float *y_uw, int batch_size, int length, int dim_in, int dim_out,
-                                         int dim_y_out, void *stream) {
+// The layer on mw coefficient rows and `rows` constant-term rows (an ordinary bound object has mw = rows * dim_in).
+static int matmul_rows(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw, const float *W,
+                       const float *bias, float *y_lb, float *y_ub, float *y_lw, float *y_uw, long long mw, long long rows,
+                       int dim_out, int dim_y_out, void *stream) {
     FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(W);
     FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
     FAITH_ALIGNED4(x_lb); FAITH_ALIGNED4(x_ub); FAITH_ALIGNED4(x_lw); FAITH_ALIGNED4(x_uw); FAITH_ALIGNED4(W);
     FAITH_ALIGNED4(bias); FAITH_ALIGNED4(y_lb); FAITH_ALIGNED4(y_ub); FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
-    FAITH_REQUIRE(batch_size > 0 && length > 0 && dim_in > 0 && dim_out > 0 && dim_y_out > 0, FAITH_ERR_SHAPE,
-                  "faith_matmul_verification: batch=%d length=%d dim_in=%d dim_out=%d dim_y_out=%d must be positive",
-                  batch_size, length, dim_in, dim_out, dim_y_out);
-    const long long rows = (long long)batch_size * length;
-    const long long mw = rows * dim_in;
-    FAITH_REQUIRE(mw <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: batch*length*dim_in exceeds 2^31");
+    FAITH_REQUIRE(mw > 0 && rows > 0 && dim_out > 0 && dim_y_out > 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_verification: coefficient rows=%lld constant rows=%lld dim_out=%d dim_y_out=%d must be positive",
+                  mw, rows, dim_out, dim_y_out);
+    FAITH_REQUIRE(mw <= 0x7fffffffLL && rows <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "faith_matmul_verification: batch*length*dim_in exceeds 2^31");
     GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool fast = (dim_out % 4 == 0) && faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
@@ -664,19 +663,59 @@ extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, c
     return faith::check_launch("faith_matmul_verification");
 }
 
+extern "C" int faith_matmul_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
+                                         const float *W, const float *bias, float *y_lb, float *y_ub, float *y_lw,
+                                         float *y_uw, int batch_size, int length, int dim_in, int dim_out,
+                                         int dim_y_out, void *stream) {
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && dim_in > 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_verification: batch=%d length=%d dim_in=%d must be positive", batch_size, length, dim_in);
+    const long long rows = (long long)batch_size * length;
+    return matmul_rows(x_lb, x_ub, x_lw, x_uw, W, bias, y_lb, y_ub, y_lw, y_uw, rows * dim_in, rows, dim_out, dim_y_out, stream);
+}
+
+extern "C" int faith_matmul_rows_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
+                                              const float *W, const float *bias, float *y_lb, float *y_ub, float *y_lw,
+                                              float *y_uw, long long rows_w, long long rows_b, int dim_out, int dim_y_out,
+                                              void *stream) {
+    return matmul_rows(x_lb, x_ub, x_lw, x_uw, W, bias, y_lb, y_ub, y_lw, y_uw, rows_w, rows_b, dim_out, dim_y_out, stream);
+}
+
+static int matmul_group_rows(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw, int groups,
+                             const float *const *W, const float *const *bias, float *const *y_lb, float *const *y_ub,
+                             float *const *y_lw, float *const *y_uw, long long mw, long long rows, int dim_out, int dim_y_out,
+                             void *stream);
+
 extern "C" int faith_matmul_group_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
                                                int groups, const float *const *W, const float *const *bias,
                                                float *const *y_lb, float *const *y_ub, float *const *y_lw,
                                                float *const *y_uw, int batch_size, int length, int dim_in, int dim_out,
                                                int dim_y_out, void *stream) {
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && dim_in > 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_group_verification: batch=%d length=%d dim_in=%d must be positive", batch_size, length, dim_in);
+    const long long rows = (long long)batch_size * length;
+    return matmul_group_rows(x_lb, x_ub, x_lw, x_uw, groups, W, bias, y_lb, y_ub, y_lw, y_uw, rows * dim_in, rows, dim_out,
+                             dim_y_out, stream);
+}
+
+extern "C" int faith_matmul_group_rows_verification(const float *x_lb, const float *x_ub, const float *x_lw,
+                                                    const float *x_uw, int groups, const float *const *W,
+                                                    const float *const *bias, float *const *y_lb, float *const *y_ub,
+                                                    float *const *y_lw, float *const *y_uw, long long rows_w,
+                                                    long long rows_b, int dim_out, int dim_y_out, void *stream) {
+    return matmul_group_rows(x_lb, x_ub, x_lw, x_uw, groups, W, bias, y_lb, y_ub, y_lw, y_uw, rows_w, rows_b, dim_out,
+                             dim_y_out, stream);
+}
+
+static int matmul_group_rows(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw, int groups,
+                             const float *const *W, const float *const *bias, float *const *y_lb, float *const *y_ub,
+                             float *const *y_lw, float *const *y_uw, long long mw, long long rows, int dim_out, int dim_y_out,
+                             void *stream) {
     FAITH_NOT_NULL(W); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
     FAITH_REQUIRE(groups >= 1 && groups <= 3, FAITH_ERR_SHAPE, "faith_matmul_group_verification: groups=%d must be 1, 2 or 3",
                   groups);
-    const long long rows = (long long)batch_size * length;
-    const long long mw = rows * dim_in;
     const long long cus = faith::compute_units();
     auto tiles = [&](int m, int n) { return ((mw + m - 1) / m) * (((long long)dim_y_out + n - 1) / n) * groups; };
-    bool fast = batch_size > 0 && length > 0 && dim_in > 0 && dim_out > 0 && dim_y_out > 0 && mw <= 0x7fffffffLL &&
+    bool fast = mw > 0 && rows > 0 && dim_out > 0 && dim_y_out > 0 && mw <= 0x7fffffffLL && rows <= 0x7fffffffLL &&
                 groups > 1 && dim_out % 4 == 0 && x_lb && x_ub && x_lw && x_uw && faith::aligned(x_lb, 4) && faith::aligned(x_ub, 4) &&
                 faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) &&
                 128LL * dim_out * 4 < 0xffffffffLL && 128LL * dim_y_out * 4 < 0x80000000LL &&
@@ -696,8 +735,8 @@ extern "C" int faith_matmul_group_verification(const float *x_lb, const float *x
     }
     if (!fast) {
         for (int i = 0; i < groups; ++i) {
-            const int rc = faith_matmul_verification(x_lb, x_ub, x_lw, x_uw, W[i], bias ? bias[i] : nullptr, y_lb[i], y_ub[i],
-                                                     y_lw[i], y_uw[i], batch_size, length, dim_in, dim_out, dim_y_out, stream);
+            const int rc = matmul_rows(x_lb, x_ub, x_lw, x_uw, W[i], bias ? bias[i] : nullptr, y_lb[i], y_ub[i], y_lw[i], y_uw[i],
+                                       mw, rows, dim_out, dim_y_out, stream);
             if (rc != FAITH_OK) return rc;
         }
         return FAITH_OK;

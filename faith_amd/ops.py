@@ -582,6 +582,43 @@ def linear_group(lw, lb, uw, ub, weights, biases=None):
     return outs
 
 
+def linear_rows(lw, lb, uw, ub, weights, biases=None):
+    """linear() / linear_group() for an object whose coefficient rows and constant rows are counted separately:
+    lw, uw [..., H] (any leading axes) and lb, ub [..., H] (any other leading axes) -- an object that keeps the
+    coefficients of a few positions only.  weights: list of one to three [H_out, H] of one shape; biases: list
+    of [H_out] or None entries, or None.  One launch where linear_group would take one.  Returns a list of
+    (lw' [..., H_out], lb' [..., H_out], uw', ub')."""
+    import ctypes
+    rows_w, rows_b, H = _object(lw, lb, uw, ub)
+    n = len(weights)
+    if not 1 <= n <= 3:
+        raise ValueError(f"{n} layers: between one and three share a launch")
+    N = weights[0].shape[0]
+    biases = list(biases) if biases is not None else [None] * n
+    for i, (W, b) in enumerate(zip(weights, biases)):
+        _check(f"weight {i}", W, (N, H))
+        if b is not None:
+            _check(f"bias {i}", b, (N,))
+    dev = lw.device
+    outs = [(_empty(*lw.shape[:-1], N, device=dev), _empty(*lb.shape[:-1], N, device=dev),
+             _empty(*lw.shape[:-1], N, device=dev), _empty(*lb.shape[:-1], N, device=dev)) for _ in range(n)]
+    with _on(dev):
+        if n == 1:
+            o = outs[0]
+            _lib.call("faith_matmul_rows_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weights[0]),
+                      _ptr(biases[0]), _ptr(o[1]), _ptr(o[3]), _ptr(o[0]), _ptr(o[2]), rows_w, rows_b, H, N, _stream(lw))
+        else:
+            arr = ctypes.c_void_p * n
+            ptrs = lambda ts: arr(*[_ptr(t) for t in ts])
+            a_w, a_b = ptrs(weights), ptrs(biases)
+            a_lb, a_ub = ptrs([o[1] for o in outs]), ptrs([o[3] for o in outs])
+            a_lw, a_uw = ptrs([o[0] for o in outs]), ptrs([o[2] for o in outs])
+            _lib.call("faith_matmul_group_rows_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), n,
+                      ctypes.addressof(a_w), ctypes.addressof(a_b), ctypes.addressof(a_lb), ctypes.addressof(a_ub),
+                      ctypes.addressof(a_lw), ctypes.addressof(a_uw), rows_w, rows_b, H, N, _stream(lw))
+    return outs
+
+
 def dot_product_qk(x, y, p, eps, words=1, return_intervals=False, out=None):
     """McCormick bounds of x . y^T.  x, y: (lw, lb, uw, ub) tuples with
     lw [B, Lx|Ly, D, d]; returns (lw [B, Lx, D, Ly], lb [B, Lx, Ly], uw, ub)."""

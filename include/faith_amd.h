@@ -278,6 +278,27 @@ int faith_matmul_group_verification(const float *x_lb, const float *x_ub,
                                     void *stream);
 
 /*
+ * The two entry points above for an object whose coefficient rows and constant rows are counted
+ * separately (as faith_layer_norm_verification counts them): x_lw, x_uw [rows_w, dim_out] -> y_lw, y_uw
+ * [rows_w, dim_y_out]; x_lb, x_ub [rows_b, dim_out] -> y_lb, y_ub [rows_b, dim_y_out].  An ordinary
+ * object has rows_w = rows_b * dim_in; one that keeps the coefficients of a few positions only
+ * (VerifierForward.py:127-156 builds such an input: zero rows everywhere else) has fewer.
+ */
+int faith_matmul_rows_verification(const float *x_lb, const float *x_ub,
+                                   const float *x_lw, const float *x_uw,
+                                   const float *W, const float *bias,
+                                   float *y_lb, float *y_ub, float *y_lw, float *y_uw,
+                                   long long rows_w, long long rows_b, int dim_out, int dim_y_out,
+                                   void *stream);
+int faith_matmul_group_rows_verification(const float *x_lb, const float *x_ub,
+                                         const float *x_lw, const float *x_uw, int groups,
+                                         const float *const *W, const float *const *bias,
+                                         float *const *y_lb, float *const *y_ub,
+                                         float *const *y_lw, float *const *y_uw,
+                                         long long rows_w, long long rows_b, int dim_out, int dim_y_out,
+                                         void *stream);
+
+/*
  * McCormick bounds of the attention scores  z[i,j] = sum_k x[i,k] * y[j,k].  Replaces
  * call_dot_product_verification_QK (kernel.cpp:45-51, dot_product_verification.cu:458-496)
  * with the arithmetic of Bounds.ori_dot_product (Bounds.py:710-823).

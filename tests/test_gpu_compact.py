@@ -209,6 +209,24 @@ def test_compact_scores_entry_point_checks_its_arguments():
     assert float(out[0][:2].abs().max()) == 0.0 and float(out[0][2:].abs().max()) > 0.0
 
 
+@pytest.mark.parametrize("shape", [(2, 5, 12, 24, 16), (1, 32, 256, 256, 256), (3, 7, 33, 20, 7)])
+def test_row_count_entry_points_on_an_ordinary_object(shape):
+    """faith_matmul_rows_verification / _group_rows_ with rows_w = rows_b * dim_in: the ordinary entry points' bits."""
+    from faith_amd import ops
+    B, L, D, H, N = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    lw = torch.randn(B, L, D, H, generator=g).cuda(); uw = (lw + 0.05 * torch.rand(B, L, D, H, generator=g).cuda())
+    lb = torch.randn(B, L, H, generator=g).cuda(); ub = lb + 0.3 * torch.rand(B, L, H, generator=g).cuda()
+    layers = [layer_of(g, H, N), layer_of(g, H, N, False), layer_of(g, H, N)]
+    W, b = [x.weight for x in layers], [x.bias for x in layers]
+    for got, want in zip(ops.linear_rows(lw, lb, uw, ub, W[:1], b[:1]), [ops.linear(lw, lb, uw, ub, W[0], b[0])]):
+        assert all(torch.equal(x, y) for x, y in zip(got, want))
+    for got, want in zip(ops.linear_rows(lw, lb, uw, ub, W, b), ops.linear_group(lw, lb, uw, ub, W, b)):
+        assert all(torch.equal(x, y) for x, y in zip(got, want))
+    with pytest.raises(ValueError):
+        ops.linear_rows(lw, lb[..., :-1].contiguous(), uw, ub[..., :-1].contiguous(), W, b)
+
+
 def test_compact_object_matches_the_oracle():
     """Against the CPU oracle directly (not only against the HIP path's own dense object)."""
     g = torch.Generator().manual_seed(8)
