@@ -49,6 +49,7 @@ SIGNATURES = {
     "faith_dot_product_verification_V": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _I, _P],
     "faith_attention_scores": [_P] * 16 + [_I] * 6 + [_F, _I, _I, _P],
     "faith_attention_scores_compact": [_P] * 16 + [_I] * 6 + [_P],
+    "faith_attention_context_compact": [_P] * 17 + [_I] * 7 + [_F, _I, _I, _P],
     "faith_attention_context": [_P] * 16 + [_I] * 6 + [_F, _I, _I, _P],
     "faith_convolution_verification": [_P] * 10 + [_I] * 9 + [_P],
 }

@@ -323,6 +323,10 @@ class Bounds:
     def attention_context(self, value):
         if self.ibp and self.dim_in > 1:
             return self._ibp_rows(lambda pr, v: pr.attention_context(v), value)
+        if isinstance(value, CompactBounds):
+            out = value._context_of(self)
+            if out is not None:
+                return out
         return self._like(*ops.attention_context(self._c(), value._c(), self.p, self.eps, self.perturbed_words))
 
 
@@ -450,6 +454,26 @@ class CompactBounds:
             else:
                 return Bounds(self.args, self.p, self.eps, lw=out[0], lb=out[1], uw=out[2], ub=out[3])
         return self.dense_form().attention_scores(_written_out(key), heads)
+
+    # ---- VerifierForward.py:208-229 + Bounds.py:843-850 + VerifierForward.py:253-263 with this object as the value
+    def _context_of(self, probs):
+        """probs.attention_context(self) from the rows that exist, or None where the kernel does not take the shapes
+        (the caller then writes the zeros out)."""
+        B, P, D, H = self._lw.shape
+        heads = probs.lw.shape[0] // B if probs.lw.shape[0] % B == 0 else 0
+        if (self._dense is not None or heads == 0 or H % heads or probs.dim_in != D or probs.dim_out != self.length
+                or not ops.attention_context_compact_fits(self.length, H // heads, D)):
+            return None
+        y = (self._lw.contiguous(), self._lb.contiguous(), self._uw.contiguous(), self._ub.contiguous())
+        y_l, y_u = self.concrete_intervals()
+        try:
+            out = ops.attention_context_compact(probs._c(), y, y_l, y_u, self.positions, probs.p, probs.eps,
+                                                probs.perturbed_words)
+        except _lib.FaithError as err:
+            if err.code != _lib.ERR_UNSUPPORTED:
+                raise
+            return None
+        return probs._like(*out)
 
 
 class BoundsMaker:

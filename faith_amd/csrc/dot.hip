@@ -80,6 +80,11 @@ struct DotArgs {
     } ox, oy, oz;
     int heads;                            // heads per batch element
     int side_by_side;                     // HEADS_X | HEADS_Y | HEADS_Z: which objects keep their heads side by side
+    // Context path with a value object whose coefficients vanish outside yP key positions per batch element:
+    // ylw, yuw then hold those rows only, [batch, yP, D, row of y], and y_positions [batch, yP] says which they are
+    // (a value outside 0 ... d-1: no such row).  nullptr: the ordinary object.
+    const long long *y_positions;
+    int yP;
 };
 // first coefficient / first constant term of pair t of an object with `rows` positions per batch element
 __device__ __forceinline__ size_t w_base(const DotArgs::Obj &o, int t, int rows, int D) {
@@ -505,9 +510,14 @@ constexpr int SB = 32;                         // block edge
 // length of a sentence is.  The staged operands are zero beyond it, up to the next multiple of 8, so whatever
 // the fragments of x and y hold there (the start of the next row, or the zero that reads past the end of a
 // tensor return) does not count; the rows of x then start on any 4-byte boundary and are read 4 bytes at a time.
-template <bool VP, bool RAGGED = false>
+//
+// COMPACT_Y (context path only): the value object has coefficients at a few key positions only (DotArgs::y_positions).
+// Its y terms, sum_k b(i, k) y(k, m, j), then have one addend per such position: no y fragments, no P and Q
+// accumulators; the addends are formed from b in LDS and the lane's column of the compact rows when the block is stored.
+template <bool VP, bool RAGGED = false, bool COMPACT_Y = false>
 __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mpw, const int heads_first, const int w_tiles) {
     static_assert(VP || !RAGGED, "a ragged reduction exists on the context path only");
+    static_assert(VP || !COMPACT_Y, "compact value operands exist on the context path only");
     extern __shared__ __align__(16) float sh[];   // six operands, each d/8 swizzled [32 x 8] pieces (or a constant-term tile)
     if ((int)blockIdx.x >= w_tiles) {
         dot_b_tile<VP>(g, blockIdx.x - w_tiles, sh);
@@ -618,7 +628,9 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
                         xl[qq] = ld4(wxl, vx, k * 4u);
                         xu[qq] = ld4(wxu, vx, k * 4u);
                     }
-                    if (VP) {
+                    if (COMPACT_Y) {
+                        yl[qq] = yu[qq] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    } else if (VP) {
                         // y[t, k, m, j]: four keys, one column per lane
                         float yv[2][4];
 #pragma unroll
@@ -645,10 +657,10 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
 #define FAITH_DOT_SMALL(c)                          \
     cl = mfma(xl[qq].c, alp.c, cl);                 \
     cu = mfma(xu[qq].c, aup.c, cu);                 \
-    cp = mfma(bh.c, ys.c, cp);                      \
+    if (!COMPACT_Y) cp = mfma(bh.c, ys.c, cp);      \
     cl = mfma(xu[qq].c, aln.c, cl);                 \
     cu = mfma(xl[qq].c, aun.c, cu);                 \
-    cq = mfma(ba.c, yd.c, cq);
+    if (!COMPACT_Y) cq = mfma(ba.c, yd.c, cq);
                     FAITH_DOT_SMALL(x)
                     FAITH_DOT_SMALL(y)
                     FAITH_DOT_SMALL(z)
@@ -658,14 +670,39 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
             }
         }
         // register r is row 8*(r/4) + 4*(lane/32) + r%4 of the block, lanes run along j
+        if (COMPACT_Y) {
+            // cp, cq (zero so far) take the y terms as 2 (b+ y_lw + b- y_uw) and 2 (b+ y_uw + b- y_lw) in the places
+            // of P + Q and P - Q: one addend per key position that has coefficients
+            const int yb = t / g.oy.heads, yh = t - yb * g.oy.heads;
+            for (int p = 0; p < g.yP; ++p) {
+                const long long kp = g.y_positions[(size_t)yb * g.yP + p];
+                if (kp < 0 || kp >= d) continue;                        // no such row (the same for every lane)
+                const int kk = (int)kp;
+                const size_t o = (((size_t)yb * g.yP + p) * g.D + m) * g.oy.pitch + (size_t)yh * g.oy.width + jcol;
+                const float vl = g.ylw[o], vu = g.yuw[o];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = 8 * (r / 4) + 4 * fh + (r % 4);
+                    const float bt = s_bp[(kk / 8) * (SB * 8) + swz(row, (kk % 8) / 4) + kk % 4];
+                    const float bp = fmaxf(bt, 0.f), bn = fminf(bt, 0.f);
+                    cp[r] += bp * vl + bn * vu;
+                    cq[r] += bp * vu + bn * vl;
+                }
+            }
+        }
         if (j0 + fi < g.Ly) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int i = i0 + 8 * (r / 4) + 4 * fh + (r % 4);
                 if (i < g.Lx) {
                     const size_t o = zw0 + ((size_t)i * g.D + m) * g.oz.pitch + j0 + fi;
-                    __builtin_nontemporal_store(cl[r] + 0.5f * (cp[r] + cq[r]), &g.zlw[o]);
-                    __builtin_nontemporal_store(cu[r] + 0.5f * (cp[r] - cq[r]), &g.zuw[o]);
+                    if (COMPACT_Y) {
+                        __builtin_nontemporal_store(cl[r] + cp[r], &g.zlw[o]);
+                        __builtin_nontemporal_store(cu[r] + cq[r], &g.zuw[o]);
+                    } else {
+                        __builtin_nontemporal_store(cl[r] + 0.5f * (cp[r] + cq[r]), &g.zlw[o]);
+                        __builtin_nontemporal_store(cu[r] + 0.5f * (cp[r] - cq[r]), &g.zuw[o]);
+                    }
                 }
             }
         }
@@ -743,7 +780,11 @@ template <bool VP>
 int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb, const float *x_ub,
               const float *y_lb, const float *y_ub, const float *x_lw, const float *x_uw, const float *y_lw,
               const float *y_uw, float *z_lb, float *z_ub, float *z_lw, float *z_uw, int B, int Lx, int Ly, int d, int D,
-              float epsilon, int q, int words, int side_by_side, int heads, void *stream) {
+              float epsilon, int q, int words, int side_by_side, int heads, void *stream,
+              const long long *y_positions = nullptr, int y_n_positions = 0) {
+    // y_positions (context path): y_lw, y_uw hold the coefficient rows of those key positions only, and y_l, y_u are
+    // given (the caller concretized the rows that exist); only the per-wavefront kernel takes such an operand
+    const bool compact_y = y_positions != nullptr;
     FAITH_NOT_NULL(x_l); FAITH_NOT_NULL(y_l); FAITH_NOT_NULL(y_u);      // x_u may be NULL: not wanted
     FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub);
     FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
@@ -770,6 +811,11 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     g.oz = {z_sbs ? heads * Ly : Ly, z_sbs ? heads : 1, Ly};
     g.heads = heads;
     g.side_by_side = side_by_side;
+    g.y_positions = y_positions;
+    g.yP = y_n_positions;
+    FAITH_REQUIRE(!compact_y || (VP && y_n_positions > 0 && D > 1 && ((uintptr_t)y_positions & 7) == 0 &&
+                                 (long long)(B / heads) * y_n_positions * D <= 0x7fffffffLL), FAITH_ERR_UNSUPPORTED,
+                  "%s: a compact value operand needs the context path, dim_in > 1 and at least one position", who);
     FAITH_REQUIRE(words >= 1 && (D == 1 || D % words == 0), FAITH_ERR_SHAPE, "%s: words=%d must divide dim_in=%d", who, words, D);
     // concrete intervals of both operands (Bounds.py:725-726); x_u is produced because the reference
     // interface exposes it, the planes do not use it.  One launch for both objects.
@@ -781,8 +827,9 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     // dim_in == 1 with several words: the reference's blocks are then empty (dim_in // words == 0,
     // Bounds.py:319-326) and its intervals are the constant terms themselves -- a radius of zero here
     const bool empty_blocks = D == 1 && words > 1;
-    int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u, cy_rows, D,
-                                    cx_h, cy_h, empty_blocks ? 0.f : epsilon, q, empty_blocks ? 1 : words, stream);
+    int rc = faith::concretize_pair(x_lb, x_ub, x_lw, x_uw, x_l, x_u, cx_rows, y_lb, y_ub, y_lw, y_uw, y_l, y_u,
+                                    compact_y ? 0 : cy_rows, D, cx_h, cy_h, empty_blocks ? 0.f : epsilon, q,
+                                    empty_blocks ? 1 : words, stream);
     if (rc != FAITH_OK) return rc;
     if (D == 1) {
         const long long n = (long long)B * Lx * Ly;
@@ -814,8 +861,11 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
     // where the only alternative is the any-shape kernel (L = 30: 101 us against 22 us).
     const bool ragged_ok = VP && d % 8 != 0 && d <= 80 && (long long)TI * D * max_pitch * 4 < 0xffffffffLL &&
                            (long long)d * D * g.oy.pitch * 4 < 0xffffffffLL;
-    const bool small = (small_ok && (pick == 2 || (pick != 1 && 100 * pad_small <= 85 * pad_tiled))) ||
-                       (ragged_ok && (pick == 2 || !fast || (pick != 1 && 100 * pad_small <= 85 * pad_tiled)));
+    const bool small = (small_ok && (pick == 2 || compact_y || (pick != 1 && 100 * pad_small <= 85 * pad_tiled))) ||
+                       (ragged_ok && (pick == 2 || compact_y || !fast || (pick != 1 && 100 * pad_small <= 85 * pad_tiled)));
+    FAITH_REQUIRE(small || !compact_y, FAITH_ERR_UNSUPPORTED,
+                  "%s: a compact value operand needs at most 80 key positions, a head size that is a multiple of 4 and "
+                  "16-byte aligned tensors", who);
     if (small) {
         // one 32 x 32 block per wavefront and perturbation coordinate.  Coordinates per wavefront: the
         // count that leaves the busiest CU the least to do -- its share of the workgroups, each costing
@@ -842,7 +892,11 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
         const size_t lds = (size_t)(6 * SB * dp > BT_LDS ? 6 * SB * dp : BT_LDS) * sizeof(float);
         const dim3 gd((unsigned)(grid + (fold ? b_tiles : 0)));
         if constexpr (VP) {
-            if (d % 8 != 0)
+            if (compact_y && d % 8 != 0)
+                hipLaunchKernelGGL((dot_w_small<true, true, true>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
+            else if (compact_y)
+                hipLaunchKernelGGL((dot_w_small<true, false, true>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
+            else if (d % 8 != 0)
                 hipLaunchKernelGGL((dot_w_small<true, true>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
             else
                 hipLaunchKernelGGL((dot_w_small<true, false>), gd, dim3(256), lds, st, g, (int)mpw, x_sbs ? 1 : 0, (int)grid);
@@ -1283,6 +1337,22 @@ extern "C" int faith_attention_scores(float *x_l, float *y_l, float *x_u, float 
     return dot_entry<false>("faith_attention_scores", x_l, y_l, x_u, y_u, x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw,
                             z_lb, z_ub, z_lw, z_uw, batch_size * heads, length_x, length_y, head_size, dim_in, epsilon, q,
                             words, HEADS_X | HEADS_Y, heads, stream);
+}
+
+extern "C" int faith_attention_context_compact(float *x_l, float *x_u, const float *y_l, const float *y_u,
+                                               const float *x_lb, const float *x_ub, const float *y_lb,
+                                               const float *y_ub, const float *x_lw, const float *x_uw,
+                                               const float *y_lw, const float *y_uw, const long long *positions,
+                                               float *z_lb, float *z_ub, float *z_lw, float *z_uw, int batch_size,
+                                               int heads, int length_x, int length_k, int n_positions, int head_size,
+                                               int dim_in, float epsilon, int q, int words, void *stream) {
+    FAITH_REQUIRE(batch_size > 0 && heads > 0 && (long long)batch_size * heads <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "faith_attention_context_compact: batch=%d heads=%d out of range", batch_size, heads);
+    FAITH_NOT_NULL(positions);
+    return dot_entry<true>("faith_attention_context_compact", x_l, const_cast<float *>(y_l), x_u, const_cast<float *>(y_u),
+                           x_lb, x_ub, y_lb, y_ub, x_lw, x_uw, y_lw, y_uw, z_lb, z_ub, z_lw, z_uw, batch_size * heads,
+                           length_x, head_size, length_k, dim_in, epsilon, q, words, HEADS_Y | HEADS_Z, heads, stream,
+                           positions, n_positions);
 }
 
 extern "C" int faith_attention_scores_compact(const float *x_l, const float *y_l, const float *y_u, const float *x_lb,

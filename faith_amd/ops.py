@@ -819,6 +819,49 @@ def attention_context(x, y, p, eps, words=1):
     return zlw, zlb, zuw, zub
 
 
+def attention_context_compact_fits(length_k, head_size, dim_in):
+    """True if attention_context_compact takes a value operand of this shape (16-byte aligned tensors assumed)."""
+    return dim_in > 1 and length_k <= 80 and head_size % 4 == 0
+
+
+def attention_context_compact(x, y, y_l, y_u, positions, p, eps, words=1):
+    """attention_context for a value object whose coefficients vanish outside `positions` [B, P] (int64, on the
+    device), with only those coefficient rows in memory: y = (lw [B, P, D, heads*size], lb [B, Lk, heads*size], uw, ub);
+    y_l, y_u [B, Lk, heads*size] its concrete bounds; x: the probabilities as for attention_context.  Returns what
+    attention_context returns for the value object with the zeros written out.  Raises FaithError
+    (FAITH_ERR_UNSUPPORTED) for shapes the kernel does not take: see attention_context_compact_fits."""
+    xlw, xlb, xuw, xub = x
+    ylw, ylb, yuw, yub = y
+    BH, Lx, D, Lk = _wb_shapes(xlw, xlb, LAYOUT_NATURAL)
+    for n, t, s in (("x.lw", xlw, None), ("x.uw", xuw, xlw.shape), ("x.lb", xlb, None), ("x.ub", xub, xlb.shape),
+                    ("y.lw", ylw, None), ("y.uw", yuw, ylw.shape), ("y.lb", ylb, None), ("y.ub", yub, ylb.shape),
+                    ("y_l", y_l, ylb.shape), ("y_u", y_u, ylb.shape)):
+        _check(n, t, s)
+    if ylw.dim() != 4 or ylb.dim() != 3:
+        raise ValueError(f"y.lw {tuple(ylw.shape)} must be [B, P, dim_in, heads*size] and y.lb {tuple(ylb.shape)} [B, Lk, heads*size]")
+    B, P, D2, H = ylw.shape
+    if tuple(ylb.shape) != (B, Lk, H) or D2 != D:
+        raise ValueError(f"x {tuple(xlw.shape)}, y.lw {tuple(ylw.shape)} and y.lb {tuple(ylb.shape)} disagree in batch, key length, dim_in or width")
+    if BH % B or H % (BH // B):
+        raise ValueError(f"x has {BH} (batch, head) pairs; y has batch {B} and rows of {H}")
+    if positions.dtype != torch.int64 or tuple(positions.shape) != (B, P) or positions.device != xlw.device \
+            or not positions.is_contiguous():
+        raise ValueError(f"positions must be a contiguous int64 tensor [{B}, {P}] on {xlw.device}")
+    heads = BH // B
+    dev = xlw.device
+    x_l = _empty_like(xlb)                                                            # nothing reads x_u
+    zlw = _empty(B, Lx, D, H, device=dev)
+    zuw = _empty_like(zlw)
+    zlb = _empty(B, Lx, H, device=dev)
+    zub = _empty_like(zlb)
+    with _on(dev):
+        _lib.call("faith_attention_context_compact", _ptr(x_l), None, _ptr(y_l), _ptr(y_u),
+                  _ptr(xlb), _ptr(xub), _ptr(ylb), _ptr(yub), _ptr(xlw), _ptr(xuw), _ptr(ylw), _ptr(yuw),
+                  positions.data_ptr(), _ptr(zlb), _ptr(zub), _ptr(zlw), _ptr(zuw), B, heads, Lx, Lk, P, H // heads, D,
+                  float(eps), q_code(p), int(words), _stream(xlw))
+    return zlw, zlb, zuw, zub
+
+
 def conv2d(lw, lb, uw, ub, weight, bias=None, stride=1, padding=0, out=None):
     """Sign-split propagation through a 2-D convolution.
     lw, uw: [1, D_in, C_in, H, W]; lb, ub: [1, C_in, H, W]; weight: [C_out, C_in, K, K]."""

@@ -463,6 +463,27 @@ int faith_attention_context(float *x_l, float *y_l, float *x_u, float *y_u,
                             int q, int words, void *stream);
 
 /*
+ * The same context for a value object whose coefficients vanish outside n_positions key positions of
+ * every batch element (see faith_attention_scores_compact), with only those rows in memory:
+ *   y_lw, y_uw [batch, n_positions, dim_in, heads * head_size];  positions [batch, n_positions] int64;
+ *   y_lb, y_ub [batch, length_k, heads * head_size];  y_l, y_u (same shape) IN: its concrete bounds.
+ * The y terms of Bounds.py:761-818, sums over the key positions of b(i, k) against y_lw / y_uw [k], then have one
+ * addend per position that has coefficients; x (the probabilities), x_l, x_u and z are as for
+ * faith_attention_context.  FAITH_ERR_UNSUPPORTED beyond 80 key positions, for a head size that is no multiple
+ * of 4, dim_in == 1 or tensors that are not 16-byte aligned: take the dense entry point then.
+ */
+int faith_attention_context_compact(float *x_l, float *x_u, const float *y_l, const float *y_u,
+                                    const float *x_lb, const float *x_ub,
+                                    const float *y_lb, const float *y_ub,
+                                    const float *x_lw, const float *x_uw,
+                                    const float *y_lw, const float *y_uw,
+                                    const long long *positions,
+                                    float *z_lb, float *z_ub, float *z_lw, float *z_uw,
+                                    int batch_size, int heads, int length_x, int length_k,
+                                    int n_positions, int head_size, int dim_in, float epsilon,
+                                    int q, int words, void *stream);
+
+/*
  * Sign-split propagation through a 2-D convolution (NCHW).  Replaces the (commented-out)
  * call_convolution_verification (kernel.cpp:62-67, convolution_verification.cu:219-239).
  *   x_lw, x_uw [dim_in, CIN, Height, Width]   (dim_in plays the conv batch)

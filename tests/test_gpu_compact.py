@@ -171,6 +171,60 @@ def test_scores_from_compact_operands(shape, p):
     assert float(lw[neither].abs().max()) == 0.0 and float(got.uw.cpu().permute(0, 1, 3, 2)[neither].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("shape", [(3, 1, 24, 2, 16, 8), (2, 2, 64, 4, 16, 12), (5, 3, 130, 3, 20, 6),
+                                   (4, 1, 256, 4, 64, 32), (1, 2, 96, 2, 8, 30)])
+@pytest.mark.parametrize("p", [2.0, float("inf")])
+def test_context_from_a_compact_value_operand(shape, p):
+    """Probabilities times a value object with coefficients at a few key positions only: the context kernel that
+    takes the rows that exist against the same kernel on the value object with the zeros written out (key lengths
+    that are multiples of 8 and others: the two instantiations)."""
+    from faith_amd import Bounds, ops
+    B, P, D, heads, size, L = shape
+    print(f"[case] compact context B={B} P={P} D={D} heads={heads} size={size} L={L} p={p}", flush=True)
+    assert ops.attention_context_compact_fits(L, size, D)
+    cv, dv = compact_and_dense(41, B, P, D, heads * size, L, p=p)
+    g = torch.Generator().manual_seed(42)
+    lw = 0.3 * torch.randn(B * heads, L, D, L, generator=g); uw = lw + 0.02 * torch.rand(B * heads, L, D, L, generator=g)
+    lb = torch.rand(B * heads, L, L, generator=g); ub = lb + 0.1 * torch.rand(B * heads, L, L, generator=g)
+    probs = Bounds(cv.args, p, 0.1, lw=lw.cuda(), lb=lb.cuda(), uw=uw.cuda(), ub=ub.cuda())
+    got, want = probs.attention_context(cv), probs.attention_context(dv)
+    assert cv._dense is None, "the compact value operand was written out"
+    assert got.lw.shape == (B, L, D, heads * size)
+    # sum_k |a| |x.w| + |b| |y.w|: what two fp32 sums of the same products in different orders may differ by
+    f = lambda t: t.double().cpu()
+    (xl, xu), (yl, yu) = probs.concretize(), dv.concretize()
+    a = f(yl.abs() + yu.abs()).reshape(B, L, heads, size)                              # [b, k, h, c]
+    xa = f(probs.lw.abs() + probs.uw.abs()).reshape(B, heads, L, D, L)                 # [b, h, i, m, k]
+    ya = f(dv.lw.abs() + dv.uw.abs()).reshape(B, L, D, heads, size)                    # [b, k, m, h, c]
+    bt = f(xl.abs()).reshape(B, heads, L, L)                                           # [b, h, i, k]
+    tw = (torch.einsum("bkhc,bhimk->bimhc", a, xa) + torch.einsum("bhik,bkmhc->bimhc", bt, ya)).reshape(B, L, D, heads * size)
+    xb = f(probs.lb.abs() + probs.ub.abs()).reshape(B, heads, L, L)
+    yb = f(dv.lb.abs() + dv.ub.abs()).reshape(B, L, heads, size)
+    tb = (torch.einsum("bkhc,bhik->bihc", a, xb + bt) + torch.einsum("bhik,bkhc->bihc", bt, yb)).reshape(B, L, heads * size)
+    for name, terms in (("lw", tw), ("uw", tw), ("lb", tb), ("ub", tb)):
+        x, y = getattr(got, name), getattr(want, name)
+        tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
+        over = float(((x.double() - y.double()).abs().cpu() / tol).max())
+        assert over <= 1.0, f"context.{name}: {over:.2f} of the accumulation-aware bar"
+
+
+def test_context_from_a_compact_value_operand_falls_back():
+    """More than 80 key positions, or a value object that has been written out already: the dense kernel, same bits."""
+    from faith_amd import Bounds, ops
+    B, P, D, heads, size, L = 1, 1, 16, 2, 8, 88
+    assert not ops.attention_context_compact_fits(L, size, D)
+    cv, dv = compact_and_dense(43, B, P, D, heads * size, L)
+    g = torch.Generator().manual_seed(44)
+    lw = 0.3 * torch.randn(B * heads, 8, D, L, generator=g); lb = torch.rand(B * heads, 8, L, generator=g)
+    probs = Bounds(cv.args, 2.0, 0.1, lw=lw.cuda(), lb=lb.cuda(), uw=(lw + 0.01).cuda(), ub=(lb + 0.1).cuda())
+    same_bits(probs.attention_context(cv), probs.attention_context(dv), "88 key positions")
+    cv, dv = compact_and_dense(45, 2, 1, 16, heads * size, 8)
+    lw = 0.3 * torch.randn(2 * heads, 8, 16, 8, generator=g); lb = torch.rand(2 * heads, 8, 8, generator=g)
+    probs = Bounds(cv.args, 2.0, 0.1, lw=lw.cuda(), lb=lb.cuda(), uw=(lw + 0.01).cuda(), ub=(lb + 0.1).cuda())
+    cv.dense_form()
+    same_bits(probs.attention_context(cv), probs.attention_context(dv), "written out before")
+
+
 def test_scores_from_compact_operands_fall_back_to_the_dense_kernel():
     """Shapes the compact kernel does not take (a length that is no multiple of 4, a key with other positions, an
     ordinary key): the dense kernel on the written-out operands, same results as for ordinary objects."""
