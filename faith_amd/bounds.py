@@ -484,7 +484,7 @@ class BoundsMaker:
     compact_from: size in bytes of one coefficient tensor with the zeros written out from which the compact
     form is kept; a smaller object is written out at once.  A propagation that small is bound by its ~30
     launches, of which the compact form needs a few more: with hidden size 256 and 32 positions the two break
-    even near 3 queries per propagation (32 MiB is 4), and at 30 the compact form saves 26 % of the time."""
+    even near 3 queries per propagation (32 MiB is 4), and at 30 the compact form saves 31 % of the time."""
 
     def __init__(self, args=None, compact_from=32 << 20):
         self.args = args
