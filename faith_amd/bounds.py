@@ -354,7 +354,8 @@ class CompactBounds:
     `layer_norm` and `matmul` / `dense` / `dense_group` keep the form: they run their kernels on the P rows
     that are not zero (the affine ones also on the constants, as an object with one zero coefficient row per
     position); `attention_scores` of two compact objects -- the first operator that mixes positions -- takes
-    the kernel that writes the dense scores from the compact rows; every other attribute or method is that of
+    the kernel that writes the dense scores from the compact rows, and `probs.attention_context(value)` with a
+    compact value the context kernel that reads its rows; every other attribute or method is that of
     `dense_form()`, the equal `Bounds` object with the zeros written out (built on first use).  Beyond the
     reference's surface, which carries the zeros through every operator."""
 
