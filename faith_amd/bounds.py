@@ -357,7 +357,12 @@ class CompactBounds:
     the kernel that writes the dense scores from the compact rows, and `probs.attention_context(value)` with a
     compact value the context kernel that reads its rows; every other attribute or method is that of
     `dense_form()`, the equal `Bounds` object with the zeros written out (built on first use).  Beyond the
-    reference's surface, which carries the zeros through every operator."""
+    reference's surface, which carries the zeros through every operator.
+
+    `positions` lives on the device and is not inspected here (that would wait for the GPU): whoever builds it
+    must keep every entry inside 0 ... length-1 and the entries of a batch element distinct, as the input builders
+    of faith_amd.forward do on the host before they create it.  The compact kernels skip a row whose position lies
+    outside that range; `dense_form`, `concrete_intervals` and everything that goes through them index with it."""
 
     collect_failures = Bounds.collect_failures
 

@@ -117,4 +117,5 @@ extern "C" int faith_mfma_clock(float *mhz, int workgroups, int iterations, void
 
 extern "C" const char *faith_last_error(void) { return faith::g_error; }
 
-extern "C" int faith_version(void) { return 1; }
+// 2: faith_dot_product_verification_QK / _V take `int layout` in front of `stream` (version 1 did not).
+extern "C" int faith_version(void) { return 2; }

@@ -1062,6 +1062,19 @@ int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, fl
     FAITH_REQUIRE((long long)B * (Lx > Ly ? Lx : Ly) * K <= 0x7fffffffLL, FAITH_ERR_SHAPE,
                   "%s: batch * length * reduction length exceeds 2^31", who);
     FAITH_REQUIRE(words >= 1 && (D == 1 || D % words == 0), FAITH_ERR_SHAPE, "%s: words=%d must divide dim_in=%d", who, words, D);
+    // every requirement is checked before the first launch: a call that is refused has written nothing
+    const long long b_tiles = (long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T);
+    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    FAITH_REQUIRE(D == 1 || (long long)(Lx > Ly ? Lx : Ly) * K * D * 4 < 0xffffffffLL, FAITH_ERR_UNSUPPORTED,
+                  "%s: the coefficients of one batch element exceed 4 GB in the transposed layout (32-bit offsets)", who);
+    constexpr int RI = 4, RJ = 8;
+    DotTArgs a{x_lw, x_uw, y_lw, y_uw, x_l, y_l, y_u, z_lw, z_uw, B, Lx, Ly, K, D};
+    a.mw = D > 128 ? 4 : D > 64 ? 2 : 1;
+    a.n_i = (Lx + RI - 1) / RI;
+    a.n_j = (Ly + RJ * (4 / a.mw) - 1) / (RJ * (4 / a.mw));
+    a.n_m = (D + 64 * a.mw - 1) / (64 * a.mw);
+    const long long grid = (long long)B * a.n_i * a.n_j * a.n_m;
+    FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
     hipStream_t st = static_cast<hipStream_t>(stream);
 
     // concrete intervals of both objects: [B * L, K] neurons whose D_in coefficients are contiguous
@@ -1087,20 +1100,7 @@ int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, fl
         hipLaunchKernelGGL(dot_interval<false>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, g);
         return faith::check_launch(who);
     }
-    const long long b_tiles = (long long)B * ((Lx + BT_T - 1) / BT_T) * ((Ly + BT_T - 1) / BT_T);
-    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
     hipLaunchKernelGGL(dot_b<false>, dim3((unsigned)b_tiles), dim3(256), 0, st, g);
-
-    FAITH_REQUIRE((long long)(Lx > Ly ? Lx : Ly) * K * D * 4 < 0xffffffffLL, FAITH_ERR_UNSUPPORTED,
-                  "%s: the coefficients of one batch element exceed 4 GB in the transposed layout (32-bit offsets)", who);
-    constexpr int RI = 4, RJ = 8;
-    DotTArgs a{x_lw, x_uw, y_lw, y_uw, x_l, y_l, y_u, z_lw, z_uw, B, Lx, Ly, K, D};
-    a.mw = D > 128 ? 4 : D > 64 ? 2 : 1;
-    a.n_i = (Lx + RI - 1) / RI;
-    a.n_j = (Ly + RJ * (4 / a.mw) - 1) / (RJ * (4 / a.mw));
-    a.n_m = (D + 64 * a.mw - 1) / (64 * a.mw);
-    const long long grid = (long long)B * a.n_i * a.n_j * a.n_m;
-    FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
     hipLaunchKernelGGL((dot_w_transposed<RI, RJ>), dim3((unsigned)grid), dim3(256), 0, st, a);
     return faith::check_launch(who);
 }
@@ -1377,17 +1377,21 @@ extern "C" int faith_attention_scores_compact(const float *x_l, const float *y_l
     // the kernel reads and writes 16 bytes at a time and keeps the key's intervals of one head in LDS; dim_in == 1 is the
     // interval shortcut of the dense entry point (Bounds.py:711-721), which this one does not have
     const size_t lds = ((size_t)2 * n_positions * CS_MC + (size_t)4 * head_size * length) * sizeof(float);
-    FAITH_REQUIRE(dim_in > 1 && length % 4 == 0 && head_size % 4 == 0 && lds <= 65536 && ((uintptr_t)positions & 7) == 0 &&
+    FAITH_REQUIRE(dim_in > 1 && length % 4 == 0 && head_size % 4 == 0 && lds <= 160 * 1024 && ((uintptr_t)positions & 7) == 0 &&
                   faith::aligned(x_l, 16) && faith::aligned(y_l, 16) && faith::aligned(y_u, 16) &&
                   faith::aligned(x_lw, 16) && faith::aligned(x_uw, 16) && faith::aligned(y_lw, 16) &&
                   faith::aligned(y_uw, 16) && faith::aligned(z_lw, 16) && faith::aligned(z_uw, 16), FAITH_ERR_UNSUPPORTED,
                   "%s: needs dim_in > 1, length and head size multiples of 4, 16-byte aligned tensors and "
-                  "8 * positions * 128 + 16 * head size * length <= 65536 bytes of LDS", who);
+                  "8 * positions * 128 + 16 * head size * length <= 163840 bytes of LDS", who);
+    FAITH_REQUIRE(faith::reserve_lds(scores_compact<true>, lds), FAITH_ERR_UNSUPPORTED,
+                  "%s: %zu bytes of LDS per workgroup could not be reserved", who, lds);
     hipStream_t st = static_cast<hipStream_t>(stream);
     CompactArgs c{x_lw, x_uw, y_lw, y_uw, x_l, y_l, y_u, positions, z_lw, z_uw, length, n_positions, dim_in, heads, head_size,
                   (dim_in + CS_MC - 1) / CS_MC};
     const long long light = B * length * c.chunks, heavy = B * n_positions * c.chunks;
     FAITH_REQUIRE(light <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    const long long b_tiles = B * ((length + BT_T - 1) / BT_T) * ((length + BT_T - 1) / BT_T);
+    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
     hipLaunchKernelGGL(scores_compact<true>, dim3((unsigned)heavy), dim3(256), lds, st, c);
     hipLaunchKernelGGL(scores_compact<false>, dim3((unsigned)light), dim3(256), (size_t)2 * n_positions * CS_MC * sizeof(float), st, c);
     // constant terms: the dense kernel (it reads constants and intervals only)
@@ -1398,8 +1402,6 @@ extern "C" int faith_attention_scores_compact(const float *x_l, const float *y_l
     g.oz = {length, 1, length};
     g.heads = heads;
     g.side_by_side = HEADS_X | HEADS_Y;
-    const long long b_tiles = B * ((length + BT_T - 1) / BT_T) * ((length + BT_T - 1) / BT_T);
-    FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
     hipLaunchKernelGGL(dot_b<false>, dim3((unsigned)b_tiles), dim3(256), 0, st, g);
     return faith::check_launch(who);
 }

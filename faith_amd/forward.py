@@ -48,7 +48,9 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
     embeddings [1, L, dim]; index: position (int) or list of positions; make_bounds(p, eps, lw, lb,
     uw, ub) builds the bound object.  Returns bounds of the (layer-normed) embeddings."""
     length, dim = embeddings.shape[1], embeddings.shape[2]
-    positions = [index] if perturbed_words == 1 else list(index)
+    positions = _checked_positions([[index] if perturbed_words == 1 else list(index)], length)[0]
+    if len(positions) != perturbed_words:
+        raise ValueError(f"{len(positions)} positions given for {perturbed_words} perturbed words")
     compact = _compact_maker(make_bounds, 1, length, dim * perturbed_words, dim)
     if compact is not None and not ibp:
         # a maker that can hold the coefficients of the perturbed positions alone: the zero rows of
@@ -77,6 +79,26 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
     return bounds
+
+
+def _checked_positions(groups, length):
+    """Positions as the input builders take them: `groups` is one list of perturbed positions per batch element.
+    Every position must lie in 0 ... length-1 and the positions of one batch element must be distinct; they index
+    device tensors further on (an out-of-range index there is a device-side assert that ends the process, and a
+    repeated one makes the written-out object depend on the order of the writes), so they are checked here, on the
+    host, where the lists still are."""
+    out = []
+    for b, group in enumerate(groups):
+        g = [int(v) for v in group]
+        for v, raw in zip(g, group):
+            if v != raw:
+                raise ValueError(f"position {raw!r} of batch element {b} is not an integer")
+            if not 0 <= v < length:
+                raise ValueError(f"position {v} of batch element {b} lies outside 0 ... {length - 1}")
+        if len(set(g)) != len(g):
+            raise ValueError(f"the positions {g} of batch element {b} are not distinct")
+        out.append(g)
+    return out
 
 
 def _compact_maker(make_bounds, batch, length, dim_in, dim_out):
@@ -224,6 +246,9 @@ def bound_inputs(make_bounds, embeddings, indices, radii, p=2.0, norm=None, laye
     eps = 1 (see the module docstring).  embeddings [1, L, dim]."""
     length, dim = embeddings.shape[1], embeddings.shape[2]
     n = len(indices)
+    if len(radii) != n:
+        raise ValueError(f"{n} positions, {len(radii)} radii")
+    indices = [g[0] for g in _checked_positions([[i] for i in indices], length)]
     dev = embeddings.device
     scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
     b = embeddings[0].unsqueeze(0).expand(n, length, dim).contiguous()
@@ -341,7 +366,7 @@ class CapturedVerifier:
     def __init__(self, make_bounds, network, embeddings, batch, label, p=2.0):
         length, dim = embeddings.shape[1], embeddings.shape[2]
         dev = embeddings.device
-        self.batch, self.label, self.dim = batch, label, dim
+        self.batch, self.label, self.dim, self.length = batch, label, dim, length
         self.b = embeddings[0].unsqueeze(0).expand(batch, length, dim).contiguous()
         self.eye = torch.eye(dim, device=dev)
         self.rows = torch.arange(batch, device=dev)
@@ -382,7 +407,9 @@ class CapturedVerifier:
 
     def __call__(self, indices, radii):
         """Verdicts for batch element b = (position indices[b], radius radii[b]); len == batch."""
-        assert len(indices) == self.batch and len(radii) == self.batch
+        if len(indices) != self.batch or len(radii) != self.batch:
+            raise ValueError(f"this graph was captured for {self.batch} (position, radius) pairs per replay")
+        indices = [g[0] for g in _checked_positions([[i] for i in indices], self.length)]
         dev = self.w.device
         scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
         if self.at is not None:

@@ -746,7 +746,7 @@ def put_positions(t, positions, rows):
 def attention_scores_compact_fits(length, n_positions, head_size, dim_in):
     """True if attention_scores_compact takes operands of this shape (16-byte aligned tensors assumed)."""
     return (dim_in > 1 and length % 4 == 0 and head_size % 4 == 0
-            and 8 * n_positions * 128 + 16 * head_size * length <= 65536)
+            and 8 * n_positions * 128 + 16 * head_size * length <= 160 * 1024)
 
 
 def attention_scores_compact(x, y, x_l, y_l, y_u, positions, heads):

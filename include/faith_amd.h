@@ -44,6 +44,11 @@ extern "C" {
 #define FAITH_LAYOUT_TRANSPOSED  1
 
 const char *faith_last_error(void);
+/* Version of this interface; a binder compares it with the header it was built against.
+ *   1: first interface.
+ *   2: faith_dot_product_verification_QK and _V take `int layout` in front of `stream` (a caller built against
+ *      version 1 would pass its stream where the layout goes). */
+#define FAITH_ABI_VERSION 2
 int faith_version(void);
 
 /*
@@ -431,7 +436,7 @@ int faith_attention_scores(float *x_l, float *y_l, float *x_u, float *y_u,
  *                          rows that have coefficients, the constants themselves elsewhere)
  *   z_* as faith_attention_scores writes them, zeros included.
  * FAITH_ERR_UNSUPPORTED unless dim_in > 1, length % 4 == 0, head_size % 4 == 0, the tensors are 16-byte aligned
- * and 8 * n_positions * 128 + 16 * head_size * length <= 65536 (bytes of LDS): take the dense entry point then.
+ * and 8 * n_positions * 128 + 16 * head_size * length <= 163840 (bytes of LDS): take the dense entry point then.
  */
 int faith_attention_scores_compact(const float *x_l, const float *y_l, const float *y_u,
                                    const float *x_lb, const float *x_ub,

@@ -140,8 +140,28 @@ def score_terms(x, y, heads):
     return w.reshape(B * heads, L, D, L), c.reshape(B * heads, L, L)
 
 
+def context_terms(probs, dv, heads):
+    """sum_k |a| |x.w| + |b| |y.w| per coefficient of the context and the like for the constants: what two fp32 sums
+    of the same products in different orders may differ by, up to KAPPA * u."""
+    f = lambda t: t.double().cpu()
+    BH, L, D, Lk = probs.lw.shape
+    B = BH // heads
+    size = dv.lw.shape[3] // heads
+    (xl, xu), (yl, yu) = probs.concretize(), dv.concretize()
+    a = f(yl.abs() + yu.abs()).reshape(B, Lk, heads, size)                             # [b, k, h, c]
+    xa = f(probs.lw.abs() + probs.uw.abs()).reshape(B, heads, L, D, Lk)                # [b, h, i, m, k]
+    ya = f(dv.lw.abs() + dv.uw.abs()).reshape(B, Lk, D, heads, size)                   # [b, k, m, h, c]
+    bt = f(xl.abs()).reshape(B, heads, L, Lk)                                          # [b, h, i, k]
+    tw = (torch.einsum("bkhc,bhimk->bimhc", a, xa) + torch.einsum("bhik,bkmhc->bimhc", bt, ya)).reshape(B, L, D, heads * size)
+    xb = f(probs.lb.abs() + probs.ub.abs()).reshape(B, heads, L, Lk)
+    yb = f(dv.lb.abs() + dv.ub.abs()).reshape(B, Lk, heads, size)
+    tb = (torch.einsum("bkhc,bhik->bihc", a, xb + bt) + torch.einsum("bhik,bkhc->bihc", bt, yb)).reshape(B, L, heads * size)
+    return tw, tb
+
+
 @pytest.mark.parametrize("shape", [(3, 1, 24, 2, 16, 8), (2, 2, 64, 4, 16, 12), (5, 3, 130, 3, 20, 16),
-                                   (4, 1, 256, 4, 64, 32), (1, 2, 512, 4, 64, 32)])
+                                   (4, 1, 256, 4, 64, 32), (1, 2, 512, 4, 64, 32),
+                                   (1, 1, 64, 2, 64, 128)])      # the last: 129 KB of LDS (more than the default 64 KB)
 @pytest.mark.parametrize("p", [2.0, float("inf"), 1.0])
 def test_scores_from_compact_operands(shape, p):
     """Query and key with coefficients at the same few positions: the kernel that writes the dense scores from the
@@ -190,17 +210,7 @@ def test_context_from_a_compact_value_operand(shape, p):
     got, want = probs.attention_context(cv), probs.attention_context(dv)
     assert cv._dense is None, "the compact value operand was written out"
     assert got.lw.shape == (B, L, D, heads * size)
-    # sum_k |a| |x.w| + |b| |y.w|: what two fp32 sums of the same products in different orders may differ by
-    f = lambda t: t.double().cpu()
-    (xl, xu), (yl, yu) = probs.concretize(), dv.concretize()
-    a = f(yl.abs() + yu.abs()).reshape(B, L, heads, size)                              # [b, k, h, c]
-    xa = f(probs.lw.abs() + probs.uw.abs()).reshape(B, heads, L, D, L)                 # [b, h, i, m, k]
-    ya = f(dv.lw.abs() + dv.uw.abs()).reshape(B, L, D, heads, size)                    # [b, k, m, h, c]
-    bt = f(xl.abs()).reshape(B, heads, L, L)                                           # [b, h, i, k]
-    tw = (torch.einsum("bkhc,bhimk->bimhc", a, xa) + torch.einsum("bhik,bkmhc->bimhc", bt, ya)).reshape(B, L, D, heads * size)
-    xb = f(probs.lb.abs() + probs.ub.abs()).reshape(B, heads, L, L)
-    yb = f(dv.lb.abs() + dv.ub.abs()).reshape(B, L, heads, size)
-    tb = (torch.einsum("bkhc,bhik->bihc", a, xb + bt) + torch.einsum("bhik,bkhc->bihc", bt, yb)).reshape(B, L, heads * size)
+    tw, tb = context_terms(probs, dv, heads)
     for name, terms in (("lw", tw), ("uw", tw), ("lb", tb), ("ub", tb)):
         x, y = getattr(got, name), getattr(want, name)
         tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
@@ -261,6 +271,52 @@ def test_compact_scores_entry_point_checks_its_arguments():
     out = ops.attention_scores_compact(x, y, x_l, y_l, y_u, far, 2)
     torch.cuda.synchronize()
     assert float(out[0][:2].abs().max()) == 0.0 and float(out[0][2:].abs().max()) > 0.0
+
+
+def test_a_position_outside_the_sentence_means_the_row_is_not_there():
+    """Both compact entry points with two positions per batch element of which one lies outside 0 ... length-1: that
+    row is skipped (include/faith_amd.h), so the results are those of the dense entry points on operands that have
+    coefficients at the other position only.  Nothing is read or written out of bounds, the kernels run normally."""
+    from faith_amd import Bounds, ops
+    B, P, D, heads, size, L = 2, 2, 32, 2, 16, 12
+    cq, _ = compact_and_dense(51, B, P, D, heads * size, L)
+    ck, _ = compact_and_dense(52, B, P, D, heads * size, L, positions=cq.positions)
+    far = cq.positions.clone()
+    far[:, 1] = torch.tensor([L, -3], device=far.device)          # just past the end; negative
+    rows = torch.arange(B, device=far.device)
+
+    def dense_without_second_row(c):
+        lw = torch.zeros(B, L, D, heads * size, device="cuda")
+        uw = torch.zeros_like(lw)
+        lw[rows, cq.positions[:, 0]] = c._lw[:, 0]
+        uw[rows, cq.positions[:, 0]] = c._uw[:, 0]
+        return Bounds(c.args, c.p, c.eps, lw=lw, lb=c._lb, uw=uw, ub=c._ub)
+    dq, dk = dense_without_second_row(cq), dense_without_second_row(ck)
+    (x_l, _), (y_l, y_u) = dq.concretize(), dk.concretize()
+    got = ops.attention_scores_compact((cq._lw, cq._lb, cq._uw, cq._ub), (ck._lw, ck._lb, ck._uw, ck._ub),
+                                       x_l, y_l, y_u, far, heads)
+    torch.cuda.synchronize()
+    want = dq.attention_scores(dk, heads)
+    tw, tb = score_terms(dq, dk, heads)
+    for name, x, terms in zip(("lw", "lb", "uw", "ub"), got, (tw, tb, tw, tb)):
+        y = getattr(want, name)
+        tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
+        over = float(((x.double() - y.double()).abs().cpu() / tol).max())
+        assert over <= 1.0, f"scores.{name} with a position outside the sentence: {over:.2f} of the accumulation-aware bar"
+    # the context with a compact value operand: same convention
+    g = torch.Generator().manual_seed(53)
+    lw = 0.3 * torch.randn(B * heads, L, D, L, generator=g); lb = torch.rand(B * heads, L, L, generator=g)
+    probs = Bounds(cq.args, 2.0, 0.1, lw=lw.cuda(), lb=lb.cuda(), uw=(lw + 0.01).cuda(), ub=(lb + 0.1).cuda())
+    gotc = ops.attention_context_compact((probs.lw, probs.lb, probs.uw, probs.ub), (ck._lw, ck._lb, ck._uw, ck._ub),
+                                         y_l, y_u, far, 2.0, 0.1)
+    torch.cuda.synchronize()
+    wantc = probs.attention_context(dk)
+    cw, cb = context_terms(probs, dk, heads)
+    for name, x, terms in zip(("lw", "lb", "uw", "ub"), gotc, (cw, cb, cw, cb)):
+        y = getattr(wantc, name)
+        tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
+        over = float(((x.double() - y.double()).abs().cpu() / tol).max())
+        assert over <= 1.0, f"context.{name} with a position outside the sentence: {over:.2f} of the accumulation-aware bar"
 
 
 @pytest.mark.parametrize("shape", [(2, 5, 12, 24, 16), (1, 32, 256, 256, 256), (3, 7, 33, 20, 7)])
