@@ -34,6 +34,7 @@ EXTRA = {
     # the dot product splits the intervals by sign with fmaxf / fminf: one instruction each only when the
     # compiler need not quiet signalling NaNs first
     "dot.hip": ["-fno-honor-nans"],
+    "dot_tiled.hip": ["-fno-honor-nans"],
 }
 
 

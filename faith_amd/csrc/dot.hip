@@ -49,8 +49,13 @@
 #include <mutex>
 
 #include "common.h"
+#include "dot_tiled.h"
 
 namespace {
+
+// experiment: planes workspace taken from the static scratch (set by the static-scratch section below)
+float *experiment_workspace(long long floats);
+
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -916,7 +921,41 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
             grid -= grid % 8;
             xcd_map = 1;
         }
-        if (d % BK == 0 && Lx % TI == 0 && Ly % TJ == 0)
+        const bool exact = d % BK == 0 && Lx % TI == 0 && Ly % TJ == 0;
+        const long long wx = (long long)B * Lx * D * d, wy = (long long)B * Ly * D * d, wz = (long long)B * Lx * D * Ly;
+        const int knob = faith::tune_get(FAITH_TUNE_DOT_VARIANT);
+        if (exact && xcd_map && faith::dot_tiled_takes(d) && wx * 4 < 0xffffffffLL && wy * 4 < 0xffffffffLL &&
+            wz * 4 < 0xffffffffLL && faith::aligned(z_lw, 4) && (knob == 3 || knob == 4)) {
+            faith::DotTiledArgs a{};
+            a.xlw = x_lw; a.xuw = x_uw; a.ylw = y_lw; a.yuw = y_uw;
+            a.x_l = x_l; a.y_l = y_l; a.y_u = y_u;
+            a.zlw = z_lw; a.zuw = z_uw;
+            const long long nxi = (long long)B * Lx * d, nyi = (long long)B * Ly * d;
+            a.x_bytes = (unsigned)(wx * 4); a.y_bytes = (unsigned)(wy * 4); a.z_bytes = (unsigned)(wz * 4);
+            a.xi_bytes = (unsigned)(nxi * 4); a.yi_bytes = (unsigned)(nyi * 4);
+            a.Lx = Lx; a.Ly = Ly; a.D = D;
+            a.xp = g.ox.pitch; a.yp = g.oy.pitch; a.zp = g.oz.pitch;
+            // pair t = bb * heads + h of an object with `rows` positions: stacked on the first axis, or heads side by side
+            auto strides = [&](const DotArgs::Obj &o, long long rows, long long per_row, unsigned &bs, unsigned &hs) {
+                if (o.heads == 1) { hs = (unsigned)(rows * per_row * o.pitch); bs = (unsigned)(hs * (long long)heads); }
+                else { bs = (unsigned)(rows * per_row * o.pitch); hs = (unsigned)o.width; }
+            };
+            strides(g.ox, Lx, D, a.xw_bs, a.xw_hs);  strides(g.ox, Lx, 1, a.xi_bs, a.xi_hs);
+            strides(g.oy, y_len, D, a.yw_bs, a.yw_hs);  strides(g.oy, y_len, 1, a.yi_bs, a.yi_hs);
+            strides(g.oz, Lx, D, a.zw_bs, a.zw_hs);
+            a.heads = heads; a.batches = B / heads;
+            a.total_tiles = (int)tiles;
+            a.dbg = faith::tune_get(FAITH_TUNE_GEMM_VARIANT) >= 100 ? faith::tune_get(FAITH_TUNE_GEMM_VARIANT) - 100 : 0;
+            if (knob == 3) {
+                float *ws = experiment_workspace(faith::dot_planes_floats(nxi, nyi));
+                if (ws) {
+                    a.b_abs = ws; a.al_pos = ws + nxi; a.al_neg = a.al_pos + nyi; a.au_pos = a.al_neg + nyi; a.au_neg = a.au_pos + nyi;
+                    faith::dot_planes_launch(x_l, y_l, y_u, ws, ws + nxi, ws + nxi + nyi, ws + nxi + 2 * nyi, ws + nxi + 3 * nyi,
+                                             nxi, nyi, st);
+                }
+            }
+            faith::dot_tiled_launch(VP, d, a, (int)grid, st);
+        } else if (exact)
             hipLaunchKernelGGL((dot_w<VP, true>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
         else
             hipLaunchKernelGGL((dot_w<VP, false>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
@@ -1294,6 +1333,14 @@ static int scratch_address(const char *who, float **out) {
     *out = scratch_ptr[dev];
     return FAITH_OK;
 }
+
+namespace {
+float *experiment_workspace(long long floats) {
+    float *base = nullptr;
+    if (floats > (long long)STATIC_SCRATCH_FLOATS / 2 || scratch_address("experiment", &base) != FAITH_OK) return nullptr;
+    return base + STATIC_SCRATCH_FLOATS / 2;
+}
+}  // namespace
 
 extern "C" long long faith_static_scratch_bytes(void) { return (long long)(STATIC_SCRATCH_FLOATS * sizeof(float)); }
 
