@@ -53,9 +53,6 @@
 
 namespace {
 
-// experiment: planes workspace taken from the static scratch (set by the static-scratch section below)
-float *experiment_workspace(long long floats);
-
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -923,9 +920,10 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
         }
         const bool exact = d % BK == 0 && Lx % TI == 0 && Ly % TJ == 0;
         const long long wx = (long long)B * Lx * D * d, wy = (long long)B * Ly * D * d, wz = (long long)B * Lx * D * Ly;
-        const int knob = faith::tune_get(FAITH_TUNE_DOT_VARIANT);
-        if (exact && xcd_map && faith::dot_tiled_takes(d) && wx * 4 < 0xffffffffLL && wy * 4 < 0xffffffffLL &&
-            wz * 4 < 0xffffffffLL && faith::aligned(z_lw, 4) && (knob == 3 || knob == 4)) {
+        // reductions of 32, 64 or 128 with every array under 4 GB: the straight-line kernel (same tiles, same order of
+        // summation, same bits); the tuning knob 1 keeps the kernel with run-time extents
+        if (exact && xcd_map && pick != 1 && faith::dot_tiled_takes(d) && wx * 4 < 0xffffffffLL && wy * 4 < 0xffffffffLL &&
+            wz * 4 < 0xffffffffLL) {
             faith::DotTiledArgs a{};
             a.xlw = x_lw; a.xuw = x_uw; a.ylw = y_lw; a.yuw = y_uw;
             a.x_l = x_l; a.y_l = y_l; a.y_u = y_u;
@@ -945,15 +943,6 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
             strides(g.oz, Lx, D, a.zw_bs, a.zw_hs);
             a.heads = heads; a.batches = B / heads;
             a.total_tiles = (int)tiles;
-            a.dbg = faith::tune_get(FAITH_TUNE_GEMM_VARIANT) >= 100 ? faith::tune_get(FAITH_TUNE_GEMM_VARIANT) - 100 : 0;
-            if (knob == 3) {
-                float *ws = experiment_workspace(faith::dot_planes_floats(nxi, nyi));
-                if (ws) {
-                    a.b_abs = ws; a.al_pos = ws + nxi; a.al_neg = a.al_pos + nyi; a.au_pos = a.al_neg + nyi; a.au_neg = a.au_pos + nyi;
-                    faith::dot_planes_launch(x_l, y_l, y_u, ws, ws + nxi, ws + nxi + nyi, ws + nxi + 2 * nyi, ws + nxi + 3 * nyi,
-                                             nxi, nyi, st);
-                }
-            }
             faith::dot_tiled_launch(VP, d, a, (int)grid, st);
         } else if (exact)
             hipLaunchKernelGGL((dot_w<VP, true>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, g, (int)tiles, xcd_map);
@@ -1333,14 +1322,6 @@ static int scratch_address(const char *who, float **out) {
     *out = scratch_ptr[dev];
     return FAITH_OK;
 }
-
-namespace {
-float *experiment_workspace(long long floats) {
-    float *base = nullptr;
-    if (floats > (long long)STATIC_SCRATCH_FLOATS / 2 || scratch_address("experiment", &base) != FAITH_OK) return nullptr;
-    return base + STATIC_SCRATCH_FLOATS / 2;
-}
-}  // namespace
 
 extern "C" long long faith_static_scratch_bytes(void) { return (long long)(STATIC_SCRATCH_FLOATS * sizeof(float)); }
 

@@ -2,23 +2,24 @@
 //
 // Arithmetic and tiling are those of dot_w in dot.hip (Transformer_Verification_Code/Verifiers/Bounds.py:710-823:
 // six MFMA products per K-pair into four accumulators, 128 x 64 tiles of one (head, perturbation coordinate),
-// four wavefronts of 64 x 32, K-step 8, two workgroups per CU).  What differs is everything around the MFMAs,
-// which for a reduction of 32 ... 128 is a large part of a tile:
+// four wavefronts of 64 x 32, K-step 8, two workgroups per CU, the same order of summation: the results are the
+// same bits).  What differs is everything around the MFMAs, which for a reduction of 32 ... 128 is a large part
+// of a tile:
 //
 //   * The reduction length is a template argument (NK K-steps of 8) and a tile is straight-line code.  The first
 //     MFMA of each accumulator takes the constant 0 as its addend, so no register is cleared (128 moves per tile
-//     and wavefront before), and with an even NK the LDS stage of every step is known at compile time.
-//   * Operands that need no arithmetic go from global memory to LDS without passing through registers
-//     (buffer loads with the LDS bit: a wavefront moves 1 KB, lane i's 16 bytes land at base + 16 i; the swizzle
-//     of the tile is in the global address a lane asks for): x_lw, x_uw, and -- when the caller provides the
-//     planes, see below -- b, |b| and the four sign-split halves of a_l, a_u.  Only y_lw +- y_uw is formed by
-//     the staging threads (8 bytes each: four vector instructions per thread and K-step).
-//   * PLANES: b = x_l and a = y_l / y_u do not depend on the perturbation coordinate, yet every tile of a head
-//     split them by sign again while staging (up to 20 vector instructions per thread and K-step, each of which
-//     takes an issue slot from the MFMA pipe).  A small kernel does it once per call into workspace the caller
-//     lends (dot_planes_launch).
+//     and wavefront before), and with an even NK the LDS stage of every step is known at compile time, so every
+//     LDS address is an immediate.
+//   * x_lw and x_uw, which need no arithmetic, go from global memory to LDS without passing through registers
+//     (buffer loads with the LDS bit: a wavefront moves 1 KB per instruction, lane i's 16 bytes land at base + 16 i;
+//     the swizzle of the tile is in the global address a lane asks for).  The intervals are split by sign and
+//     y_lw +- y_uw formed by the staging threads as before, evenly over the four wavefronts.
 //   * Every array is addressed through ONE buffer descriptor and 32-bit offsets; a tile's offsets are a handful
-//     of scalar multiplies (250 scalar instructions per tile before).
+//     of scalar multiplies (250 scalar instructions per tile before), a K-step adds constants.
+//   * The results of a tile leave BEHIND the barrier of its last K-step: vector memory operations retire in order,
+//     so a wait for loads issued behind the stores would wait for the stores' acknowledgements too.
+//
+// Per tile and wavefront: 384 MFMAs, about 290 other vector instructions (465 before) and 200 scalar ones (490).
 #include "dot_tiled.h"
 
 namespace {
@@ -78,25 +79,19 @@ struct Offsets {
     unsigned x, b, y, a, z; // bytes from the first element of the arrays to the tile's first element
 };
 
-// vmcnt(N) lgkmcnt(0), then the barrier.  N = 0: this wavefront's global -> LDS loads have landed and its LDS
-// stores are done.  N = 63 behind the result stores of a tile: vector memory operations retire in order, the
-// loads were issued before the 64 stores, so all of them are done once at most 63 operations are outstanding.
-template <int VM>
+// This wavefront's global -> LDS loads have landed and its LDS stores are done; then the barrier.  (The compiler
+// does not wait in front of a bare s_barrier on this part, and it cannot see other wavefronts' loads.)
 __device__ __forceinline__ void wait_and_barrier() {
-    if (VM == 0)
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else
-        asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // VP = false: scores path, y is [.., Ly, D, d] (reduction axis contiguous, like x), tiles staged [row][8] with the swizzle.
 // VP = true : context path, y is the value object in its own layout [.., d, D, Ly] (reduction axis slow, j contiguous),
 //             and so are its intervals [.., d, Ly]; the y-side tiles are staged [k][64].
-template <bool VP, int NK, bool PLANES>
+template <bool VP, int NK>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 dot_tiled(const DotTiledArgs g) {
     static_assert(NK % 2 == 0, "the LDS stage of a K-step must not depend on the tile");
-    const int dbg = g.dbg;
     __shared__ float sm0[STAGE];
     __shared__ float sm1[STAGE];
 
@@ -135,7 +130,6 @@ dot_tiled(const DotTiledArgs g) {
     };
     int tiles_left = ((int)blockIdx.x < g.total_tiles) ? (g.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
     if (tiles_left == 0) return;
-
     auto point = [&](const Walk &w) {
         const unsigned i0 = w.i * TI, j0 = w.j * TJ, m = w.m * 8 + m_low;
         Offsets o;
@@ -159,15 +153,6 @@ dot_tiled(const DotTiledArgs g) {
     // 16 i of the chunk, i.e. slot i % 2 of row i / 2, which holds half (i % 2) ^ ((row >> 2) & 1) of that row
     const int xr = 32 * wv + lane / 2, xh = (lane % 2) ^ ((xr >> 2) & 1);
     const unsigned vx = ((unsigned)xr * g.D * g.xp + xh * 4) * 4u;
-    const unsigned vb = ((unsigned)xr * g.xp + xh * 4) * 4u;
-    // the planes of a: wavefronts 0, 1 move the two chunks of the positive halves, 2, 3 those of the negative ones
-    unsigned va;
-    if (VP) {
-        va = ((unsigned)(4 * (wv % 2) + lane / 16) * g.yp + (lane % 16) * 4) * 4u;
-    } else {
-        const int r = 32 * (wv % 2) + lane / 2, hf = (lane % 2) ^ ((r >> 2) & 1);
-        va = ((unsigned)r * g.yp + hf * 4) * 4u;
-    }
     // through registers: 8 bytes of y_lw and of y_uw per thread
     unsigned vy;
     int ydst;
@@ -180,7 +165,7 @@ dot_tiled(const DotTiledArgs g) {
         vy = ((unsigned)row * g.D * g.yp + q * 2) * 4u;
         ydst = swz(row, q / 2) + (q % 2) * 2;
     }
-    // without planes: 16 bytes of b per thread, and 16 bytes of a_l (wavefronts 0, 1) or a_u (2, 3)
+    // 16 bytes of b per thread, and 16 bytes of a_l (wavefronts 0, 1) or a_u (wavefronts 2, 3)
     const int srow = tid / 2, sc = tid % 2, t2 = tid % 128;
     const unsigned vbs = ((unsigned)srow * g.xp + sc * 4) * 4u;
     const int bdst = swz(srow, sc);
@@ -191,10 +176,7 @@ dot_tiled(const DotTiledArgs g) {
     const __amdgpu_buffer_rsrc_t rxl = window(g.xlw, g.x_bytes), rxu = window(g.xuw, g.x_bytes);
     const __amdgpu_buffer_rsrc_t ryl = window(g.ylw, g.y_bytes), ryu = window(g.yuw, g.y_bytes);
     const __amdgpu_buffer_rsrc_t rb = window(g.x_l, g.xi_bytes);
-    const __amdgpu_buffer_rsrc_t rba = window(PLANES ? g.b_abs : g.x_l, g.xi_bytes);
-    // PLANES: this wavefront's plane of a_l and of a_u; else the interval it splits itself
-    const __amdgpu_buffer_rsrc_t ral = window(PLANES ? (upper ? g.al_neg : g.al_pos) : (upper ? g.y_u : g.y_l), g.yi_bytes);
-    const __amdgpu_buffer_rsrc_t rau = window(PLANES ? (upper ? g.au_neg : g.au_pos) : g.y_u, g.yi_bytes);
+    const __amdgpu_buffer_rsrc_t ra = window(upper ? g.y_u : g.y_l, g.yi_bytes);      // the interval this wavefront splits
     const __amdgpu_buffer_rsrc_t rzl = window(g.zlw, g.z_bytes), rzu = window(g.zuw, g.z_bytes);
 
     float2 py0, py1;
@@ -204,15 +186,8 @@ dot_tiled(const DotTiledArgs g) {
         const unsigned kx = kt * 32u;
         to_lds(rxl, s + XL + wv * CHUNK, vx, o.x + kx);
         to_lds(rxu, s + XU + wv * CHUNK, vx, o.x + kx);
-        if (PLANES) {
-            to_lds(rb, s + BH + wv * CHUNK, vb, o.b + kx);
-            to_lds(rba, s + BA + wv * CHUNK, vb, o.b + kx);
-            to_lds(ral, s + (upper ? ALN : ALP) + (wv % 2) * CHUNK, va, o.a + kt * ak);
-            to_lds(rau, s + (upper ? AUN : AUP) + (wv % 2) * CHUNK, va, o.a + kt * ak);
-        } else {
-            pb = ld4(rb, vbs, o.b + kx);
-            pa = ld4(ral, vas, o.a + kt * ak);
-        }
+        pb = ld4(rb, vbs, o.b + kx);
+        pa = ld4(ra, vas, o.a + kt * ak);
         py0 = ld2(ryl, vy, o.y + kt * yk);
         py1 = ld2(ryu, vy, o.y + kt * yk);
     };
@@ -220,12 +195,10 @@ dot_tiled(const DotTiledArgs g) {
     auto stage = [&](float *s) {
         *reinterpret_cast<float2 *>(s + YS + ydst) = make_float2(py0.x + py1.x, py0.y + py1.y);
         *reinterpret_cast<float2 *>(s + YD + ydst) = make_float2(py0.x - py1.x, py0.y - py1.y);
-        if (!PLANES) {
-            *reinterpret_cast<float4 *>(s + BH + bdst) = pb;                  // b and |b|: P and Q come out doubled
-            *reinterpret_cast<float4 *>(s + BA + bdst) = abs4(pb);           // and are halved once per result
-            *reinterpret_cast<float4 *>(s + (upper ? AUP : ALP) + adst) = pos4(pa);
-            *reinterpret_cast<float4 *>(s + (upper ? AUN : ALN) + adst) = neg4(pa);
-        }
+        *reinterpret_cast<float4 *>(s + BH + bdst) = pb;                      // b and |b|: P and Q come out doubled
+        *reinterpret_cast<float4 *>(s + BA + bdst) = abs4(pb);               // and are halved once per result
+        *reinterpret_cast<float4 *>(s + (upper ? AUP : ALP) + adst) = pos4(pa);
+        *reinterpret_cast<float4 *>(s + (upper ? AUN : ALN) + adst) = neg4(pa);
     };
 
     // ---- fragments: x side rows wi*64 + {0, 32} + fi, y side column wj*32 + fi; this lane's four K values are
@@ -250,7 +223,7 @@ dot_tiled(const DotTiledArgs g) {
     Offsets here = point(cur);
     issue(0, here, sm0);
     stage(sm0);
-    wait_and_barrier<0>();
+    wait_and_barrier();
 
     for (; tiles_left > 0; --tiles_left) {
         const bool has_next = tiles_left > 1;
@@ -261,11 +234,11 @@ dot_tiled(const DotTiledArgs g) {
             float *sc_ = (kt & 1) ? sm1 : sm0, *sn_ = (kt & 1) ? sm0 : sm1;
             // the fetch of the next K-step -- the first one of the next tile included -- goes first
             if (kt < NK - 1) {
-                if (!(dbg & 2)) issue(kt + 1, here, sn_);
+                issue(kt + 1, here, sn_);
             } else if (has_next) {
                 cur = advance(cur);
                 next = point(cur);
-                if (!(dbg & 2)) issue(0, next, sn_);
+                issue(0, next, sn_);
             }
             __builtin_amdgcn_sched_barrier(0);
             {
@@ -323,350 +296,52 @@ dot_tiled(const DotTiledArgs g) {
             }
             __builtin_amdgcn_sched_barrier(0);
             if (kt == NK - 1) {
+                // The operands of the next tile's first step are staged and the barrier is passed BEFORE the results
+                // leave: vector memory operations retire in order, so a wait for loads that were issued behind the
+                // stores would wait for the stores' acknowledgements as well; this way the stores have a whole K-step
+                // before anything waits behind them.
+                if (has_next) stage(sn_);
+                wait_and_barrier();
                 // z_lw = X_l + (P + Q), z_uw = X_u + (P - Q); 64 stores in one run: the CU's other workgroup, which is
                 // somewhere else in its own tile, has the MFMA pipe meanwhile
                 unsigned step_b = rsb, z0 = here.z;
                 asm volatile("" : "+s"(step_b), "+s"(z0));         // keeps 32 row offsets from being hoisted and held
-                const bool all_stores = !(dbg & 1) || tiles_left == 1;
 #pragma unroll
                 for (int a = 0; a < 2; ++a)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int row_in_tile = a * 32 + 8 * (r / 4) + r % 4;
                         const float p = cp[a][r], q = cq[a][r];
-                        if (all_stores || r == 0) {
                         st1_nt(cl[a][r] + 0.5f * (p + q), rzl, lane_off, z0 + row_in_tile * step_b);
                         st1_nt(cu[a][r] + 0.5f * (p - q), rzu, lane_off, z0 + row_in_tile * step_b);
-                        }
                     }
                 here = next;
-                if (has_next) stage(sn_);
-                if (dbg & 4) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); else
-                wait_and_barrier<63>();
+                __builtin_amdgcn_sched_barrier(0);
             } else {
                 stage(sn_);
-                if (dbg & 4) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); else
-                wait_and_barrier<0>();
+                wait_and_barrier();
             }
         }
     }
 }
 
-// ------------------------------------------------------------------------------------------------------------
-// The same tile with NO workgroup barrier: every wavefront stages what its own 64 x 32 block needs in its own
-// 14 KB of LDS (rows of x and b for its 64 rows, planes of a and y_lw +- y_uw for its 32 columns).  The two
-// wavefronts that share rows of x fetch them twice (from L1 / L2), the pay-off is that no wavefront ever waits
-// for another: with one barrier per 48 MFMAs the four wavefronts of a workgroup -- each sharing its SIMD with a
-// wavefront of the CU's other workgroup -- spent a good part of every K-step waiting for the slowest of them,
-// and while they did, the MFMA pipes of three SIMDs had at most one wavefront to run.
-// One LDS stage per wavefront: the global -> LDS loads of K-step kt + 1 are issued as soon as the fragment reads
-// of step kt have returned, and land while its 48 MFMAs run.
-// ------------------------------------------------------------------------------------------------------------
-constexpr int WX = 64 * BK, WY = 32 * BK;          // floats of a wavefront's x-side / y-side operand tile
-constexpr int wXL = 0, wXU = WX, wBH = 2 * WX, wBA = 3 * WX;
-constexpr int wALP = 4 * WX, wALN = wALP + WY, wAUP = wALP + 2 * WY, wAUN = wALP + 3 * WY, wYS = wALP + 4 * WY, wYD = wALP + 5 * WY;
-constexpr int WSTAGE = 4 * WX + 6 * WY;            // 14 KB
-
-template <int VM>
-__device__ __forceinline__ void wait_loads_and_lds() {
-    if (VM == 0)
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    else
-        asm volatile("s_waitcnt vmcnt(63) lgkmcnt(0)" ::: "memory");
-}
-
-template <bool VP, int NK, bool PLANES>
-__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-dot_waves(const DotTiledArgs g) {
-    __shared__ float sm[4 * WSTAGE];
-
-    const int tid = threadIdx.x;
-    const int lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
-    const int wi = wv / 2, wj = wv % 2;
-    const int fi = lane % 32, fh = lane / 32;
-    float *const s = sm + wv * WSTAGE;                 // this wavefront's stage
-
-    const int ti = g.Lx / TI, tj = g.Ly / TJ;
-    const int m_low = (int)(blockIdx.x % 8), m_radix = g.D / 8;
-    auto digits = [&](int n) {
-        Walk w;
-        w.j = n % tj;  n /= tj;
-        w.i = n % ti;  n /= ti;
-        w.m = n % m_radix;  n /= m_radix;
-        w.h = n % g.heads;
-        w.b = n / g.heads;
-        return w;
-    };
-    Walk cur = digits((int)(blockIdx.x / 8));
-    const Walk step = digits((int)(gridDim.x / 8));
-    auto advance = [&](Walk w) {
-        w.j += step.j;
-        if (w.j >= tj) { w.j -= tj; w.i += 1; }
-        w.i += step.i;
-        if (w.i >= ti) { w.i -= ti; w.m += 1; }
-        w.m += step.m;
-        if (w.m >= m_radix) { w.m -= m_radix; w.h += 1; }
-        w.h += step.h;
-        if (w.h >= g.heads) { w.h -= g.heads; w.b += 1; }
-        w.b += step.b;
-        return w;
-    };
-    int tiles_left = ((int)blockIdx.x < g.total_tiles) ? (g.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
-    if (tiles_left == 0) return;
-
-    // offsets of this WAVEFRONT's block: rows wi * 64 ..., columns wj * 32 ...
-    auto point = [&](const Walk &w) {
-        const unsigned i0 = w.i * TI + wi * 64, j0 = w.j * TJ + wj * 32, m = w.m * 8 + m_low;
-        Offsets o;
-        o.x = (w.b * g.xw_bs + w.h * g.xw_hs + (i0 * g.D + m) * g.xp) * 4u;
-        o.b = (w.b * g.xi_bs + w.h * g.xi_hs + i0 * g.xp) * 4u;
-        if (VP) {
-            o.y = (w.b * g.yw_bs + w.h * g.yw_hs + m * g.yp + j0) * 4u;
-            o.a = (w.b * g.yi_bs + w.h * g.yi_hs + j0) * 4u;
-        } else {
-            o.y = (w.b * g.yw_bs + w.h * g.yw_hs + (j0 * g.D + m) * g.yp) * 4u;
-            o.a = (w.b * g.yi_bs + w.h * g.yi_hs + j0 * g.yp) * 4u;
-        }
-        o.z = (w.b * g.zw_bs + w.h * g.zw_hs + (i0 * g.D + m) * g.zp + j0) * 4u;
-        return o;
-    };
-    const unsigned yk = VP ? 8u * g.D * g.yp * 4u : 32u, ak = VP ? 8u * g.yp * 4u : 32u;
-    const unsigned x_half = 32u * g.D * g.xp * 4u, b_half = 32u * g.xp * 4u;      // rows 32 ... 63 of the block
-
-    // a 1 KB chunk is 32 rows of 32 bytes: lane i fills slot i % 2 of row i / 2, which holds half (i % 2) ^ ((row >> 2) & 1)
-    const int cr = lane / 2, ch = (lane % 2) ^ ((cr >> 2) & 1);
-    const unsigned vx = ((unsigned)cr * g.D * g.xp + ch * 4) * 4u;
-    const unsigned vb = ((unsigned)cr * g.xp + ch * 4) * 4u;
-    // y side, scores path: the same chunk shape over rows of y / a; context path: [8 k][32 j], lane = (k, four j)
-    const unsigned va = VP ? ((unsigned)(lane / 8) * g.yp + (lane % 8) * 4) * 4u : ((unsigned)cr * g.yp + ch * 4) * 4u;
-    const unsigned vy = VP ? ((unsigned)(lane / 8) * g.D * g.yp + (lane % 8) * 4) * 4u : ((unsigned)cr * g.D * g.yp + ch * 4) * 4u;
-    const int ydst = lane * 4;                          // both layouts: lane i's 16 bytes sit at 16 i of the tile
-
-    const __amdgpu_buffer_rsrc_t rxl = window(g.xlw, g.x_bytes), rxu = window(g.xuw, g.x_bytes);
-    const __amdgpu_buffer_rsrc_t ryl = window(g.ylw, g.y_bytes), ryu = window(g.yuw, g.y_bytes);
-    const __amdgpu_buffer_rsrc_t rb = window(g.x_l, g.xi_bytes);
-    const __amdgpu_buffer_rsrc_t rba = window(PLANES ? g.b_abs : g.x_l, g.xi_bytes);
-    const __amdgpu_buffer_rsrc_t r0 = window(PLANES ? g.al_pos : g.y_l, g.yi_bytes), r1 = window(PLANES ? g.al_neg : g.y_u, g.yi_bytes);
-    const __amdgpu_buffer_rsrc_t r2 = window(PLANES ? g.au_pos : g.y_u, g.yi_bytes), r3 = window(PLANES ? g.au_neg : g.y_u, g.yi_bytes);
-    const __amdgpu_buffer_rsrc_t rzl = window(g.zlw, g.z_bytes), rzu = window(g.zuw, g.z_bytes);
-
-    float4 py0, py1, pb0, pb1, pa0, pa1;
-    auto issue = [&](int kt, const Offsets &o) {
-        const unsigned kx = kt * 32u;
-        to_lds(rxl, s + wXL, vx, o.x + kx);
-        to_lds(rxl, s + wXL + CHUNK, vx, o.x + kx + x_half);
-        to_lds(rxu, s + wXU, vx, o.x + kx);
-        to_lds(rxu, s + wXU + CHUNK, vx, o.x + kx + x_half);
-        if (PLANES) {
-            to_lds(rb, s + wBH, vb, o.b + kx);
-            to_lds(rb, s + wBH + CHUNK, vb, o.b + kx + b_half);
-            to_lds(rba, s + wBA, vb, o.b + kx);
-            to_lds(rba, s + wBA + CHUNK, vb, o.b + kx + b_half);
-            to_lds(r0, s + wALP, va, o.a + kt * ak);
-            to_lds(r1, s + wALN, va, o.a + kt * ak);
-            to_lds(r2, s + wAUP, va, o.a + kt * ak);
-            to_lds(r3, s + wAUN, va, o.a + kt * ak);
-        } else {
-            pb0 = ld4(rb, vb, o.b + kx);
-            pb1 = ld4(rb, vb, o.b + kx + b_half);
-            pa0 = ld4(r0, va, o.a + kt * ak);
-            pa1 = ld4(r1, va, o.a + kt * ak);
-        }
-        py0 = ld4(ryl, vy, o.y + kt * yk);
-        py1 = ld4(ryu, vy, o.y + kt * yk);
-    };
-    auto stage = [&]() {
-        *reinterpret_cast<float4 *>(s + wYS + ydst) = make_float4(py0.x + py1.x, py0.y + py1.y, py0.z + py1.z, py0.w + py1.w);
-        *reinterpret_cast<float4 *>(s + wYD + ydst) = make_float4(py0.x - py1.x, py0.y - py1.y, py0.z - py1.z, py0.w - py1.w);
-        if (!PLANES) {
-            *reinterpret_cast<float4 *>(s + wBH + ydst) = pb0;
-            *reinterpret_cast<float4 *>(s + wBH + CHUNK + ydst) = pb1;
-            *reinterpret_cast<float4 *>(s + wBA + ydst) = abs4(pb0);
-            *reinterpret_cast<float4 *>(s + wBA + CHUNK + ydst) = abs4(pb1);
-            *reinterpret_cast<float4 *>(s + wALP + ydst) = pos4(pa0);
-            *reinterpret_cast<float4 *>(s + wALN + ydst) = neg4(pa0);
-            *reinterpret_cast<float4 *>(s + wAUP + ydst) = pos4(pa1);
-            *reinterpret_cast<float4 *>(s + wAUN + ydst) = neg4(pa1);
-        }
-    };
-
-    int fa[2];
-#pragma unroll
-    for (int a = 0; a < 2; ++a) fa[a] = swz(a * 32 + fi, fh);
-    const int fy = VP ? (4 * fh) * 32 + fi : swz(fi, fh);
-    auto yfrag = [&](int o) -> float4 {
-        if (VP) {
-            const float *p = s + o + fy;
-            return make_float4(p[0], p[32], p[64], p[96]);
-        }
-        return *reinterpret_cast<const float4 *>(s + o + fy);
-    };
-
-    const unsigned rsb = (unsigned)g.D * g.zp * 4u;
-    const unsigned lane_off = (unsigned)(4 * fh) * rsb + fi * 4u;
-
-    Offsets here = point(cur);
-    issue(0, here);
-    stage();
-    wait_loads_and_lds<0>();
-
-    for (; tiles_left > 0; --tiles_left) {
-        const bool has_next = tiles_left > 1;
-        floatx16 cl[2], cu[2], cp[2], cq[2];
-        Offsets next = here;
-#pragma unroll
-        for (int kt = 0; kt < NK; ++kt) {
-            float4 xl[2], xu[2], bh[2], ba[2];
-#pragma unroll
-            for (int a = 0; a < 2; ++a) {
-                xl[a] = *reinterpret_cast<const float4 *>(s + wXL + fa[a]);
-                xu[a] = *reinterpret_cast<const float4 *>(s + wXU + fa[a]);
-            }
-            const float4 alp = yfrag(wALP), aup = yfrag(wAUP), aln = yfrag(wALN), aun = yfrag(wAUN);
-#pragma unroll
-            for (int a = 0; a < 2; ++a) {
-                bh[a] = *reinterpret_cast<const float4 *>(s + wBH + fa[a]);
-                ba[a] = *reinterpret_cast<const float4 *>(s + wBA + fa[a]);
-            }
-            const float4 ys = yfrag(wYS), yd = yfrag(wYD);
-            __builtin_amdgcn_sched_barrier(0);
-            // the fragments are in registers: the stage is free for the next K-step's operands
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (kt < NK - 1) {
-                issue(kt + 1, here);
-            } else if (has_next) {
-                cur = advance(cur);
-                next = point(cur);
-                issue(0, next);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (kt == 0) {
-                const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    cl[a] = mfma(xl[a].x, alp.x, zero);
-                    cu[a] = mfma(xu[a].x, aup.x, zero);
-                }
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    cl[a] = mfma(xu[a].x, aln.x, cl[a]);
-                    cu[a] = mfma(xl[a].x, aun.x, cu[a]);
-                }
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    cp[a] = mfma(bh[a].x, ys.x, zero);
-                    cq[a] = mfma(ba[a].x, yd.x, zero);
-                }
-            }
-#define FAITH_DOT_STEP(c)                                   \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a] = mfma(xl[a].c, alp.c, cl[a]);                \
-        cu[a] = mfma(xu[a].c, aup.c, cu[a]);                \
-    }                                                       \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cl[a] = mfma(xu[a].c, aln.c, cl[a]);                \
-        cu[a] = mfma(xl[a].c, aun.c, cu[a]);                \
-    }                                                       \
-    _Pragma("unroll") for (int a = 0; a < 2; ++a) {         \
-        cp[a] = mfma(bh[a].c, ys.c, cp[a]);                 \
-        cq[a] = mfma(ba[a].c, yd.c, cq[a]);                 \
-    }
-            if (kt != 0) { FAITH_DOT_STEP(x) }
-            FAITH_DOT_STEP(y)
-            FAITH_DOT_STEP(z)
-            FAITH_DOT_STEP(w)
-#undef FAITH_DOT_STEP
-            __builtin_amdgcn_sched_barrier(0);
-            if (kt == NK - 1) {
-                unsigned step_b = rsb, z0 = here.z;
-                asm volatile("" : "+s"(step_b), "+s"(z0));
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int row_in_tile = a * 32 + 8 * (r / 4) + r % 4;
-                        const float p = cp[a][r], q = cq[a][r];
-                        st1_nt(cl[a][r] + 0.5f * (p + q), rzl, lane_off, z0 + row_in_tile * step_b);
-                        st1_nt(cu[a][r] + 0.5f * (p - q), rzu, lane_off, z0 + row_in_tile * step_b);
-                    }
-                here = next;
-                if (has_next) stage();
-                wait_loads_and_lds<63>();
-            } else {
-                stage();
-                wait_loads_and_lds<0>();
-            }
-        }
-    }
-}
-
-// |b| and the halves of a_l, a_u by sign, once per call: n4x float4 of x_l, n4y of y_l and y_u
-__global__ void __launch_bounds__(256) dot_planes(const float4 *__restrict__ x_l, const float4 *__restrict__ y_l,
-                                                  const float4 *__restrict__ y_u, float4 *__restrict__ b_abs,
-                                                  float4 *__restrict__ al_pos, float4 *__restrict__ al_neg,
-                                                  float4 *__restrict__ au_pos, float4 *__restrict__ au_neg, long long n4x,
-                                                  long long n4y) {
-    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (e < n4x) {
-        b_abs[e] = abs4(x_l[e]);
-    } else if (e < n4x + n4y) {
-        const long long f = e - n4x;
-        const float4 v = y_l[f];
-        al_pos[f] = pos4(v);
-        al_neg[f] = neg4(v);
-    } else if (e < n4x + 2 * n4y) {
-        const long long f = e - n4x - n4y;
-        const float4 v = y_u[f];
-        au_pos[f] = pos4(v);
-        au_neg[f] = neg4(v);
-    }
-}
-
-template <bool VP, int NK>
-void launch_nk(bool planes, const DotTiledArgs &a, int grid, hipStream_t st) {
-    if (faith::tune_get(FAITH_TUNE_DOT_COORDS) == 99) {     // experiment: the kernel without barriers
-        if (planes)
-            hipLaunchKernelGGL((dot_waves<VP, NK, true>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, a);
-        else
-            hipLaunchKernelGGL((dot_waves<VP, NK, false>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, a);
-        return;
-    }
-    const int solo = faith::tune_get(FAITH_TUNE_CONV_VARIANT) == 77;      // experiment: one workgroup per CU
-    const size_t pad = solo ? 40 * 1024 : 0;
-    if (solo) {
-        grid = grid / 2;
-        faith::reserve_lds(dot_tiled<VP, NK, true>, 100 * 1024);  faith::reserve_lds(dot_tiled<VP, NK, false>, 100 * 1024);
-    }
-    if (planes)
-        hipLaunchKernelGGL((dot_tiled<VP, NK, true>), dim3((unsigned)grid), dim3(NTHREADS), pad, st, a);
-    else
-        hipLaunchKernelGGL((dot_tiled<VP, NK, false>), dim3((unsigned)grid), dim3(NTHREADS), pad, st, a);
-}
 template <bool VP>
-void launch_vp(int reduction, bool planes, const DotTiledArgs &a, int grid, hipStream_t st) {
-    if (reduction == 32) launch_nk<VP, 4>(planes, a, grid, st);
-    else if (reduction == 64) launch_nk<VP, 8>(planes, a, grid, st);
-    else launch_nk<VP, 16>(planes, a, grid, st);
+void launch_vp(int reduction, const DotTiledArgs &a, int grid, hipStream_t st) {
+    if (reduction == 32)
+        hipLaunchKernelGGL((dot_tiled<VP, 4>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, a);
+    else if (reduction == 64)
+        hipLaunchKernelGGL((dot_tiled<VP, 8>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, a);
+    else
+        hipLaunchKernelGGL((dot_tiled<VP, 16>), dim3((unsigned)grid), dim3(NTHREADS), 0, st, a);
 }
 
 }  // namespace
 
 namespace faith {
 
-void dot_planes_launch(const float *x_l, const float *y_l, const float *y_u, float *b_abs, float *al_pos, float *al_neg,
-                       float *au_pos, float *au_neg, long long nx, long long ny, hipStream_t stream) {
-    const long long n4x = nx / 4, n4y = ny / 4, n = n4x + 2 * n4y;
-    hipLaunchKernelGGL(dot_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
-                       reinterpret_cast<const float4 *>(x_l), reinterpret_cast<const float4 *>(y_l),
-                       reinterpret_cast<const float4 *>(y_u), reinterpret_cast<float4 *>(b_abs),
-                       reinterpret_cast<float4 *>(al_pos), reinterpret_cast<float4 *>(al_neg),
-                       reinterpret_cast<float4 *>(au_pos), reinterpret_cast<float4 *>(au_neg), n4x, n4y);
-}
-
 void dot_tiled_launch(bool vp, int reduction, const DotTiledArgs &a, int grid, hipStream_t stream) {
-    const bool planes = a.b_abs != nullptr;
-    if (vp) launch_vp<true>(reduction, planes, a, grid, stream);
-    else launch_vp<false>(reduction, planes, a, grid, stream);
+    if (vp) launch_vp<true>(reduction, a, grid, stream);
+    else launch_vp<false>(reduction, a, grid, stream);
 }
 
 }  // namespace faith

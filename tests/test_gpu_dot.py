@@ -524,3 +524,46 @@ def test_in_place_heads_equal_stacked_heads_bit_for_bit_at_configuration_3_size(
     for a, b in zip(ctx, ctx_in_place):
         want = sbs_w(a) if a.dim() == 4 else sbs_b(a)
         assert torch.equal(want, b)
+
+
+@pytest.mark.parametrize("case", [
+    # path, (batch, heads) layout, pairs or (batch, heads), Lx, Ly or keys, D, head size / reduction
+    ("scores", "stacked", 4, 128, 128, 64, 64), ("scores", "stacked", 2, 256, 64, 24, 32), ("scores", "stacked", 1, 128, 192, 40, 128),
+    ("scores", "in place", (2, 3), 128, 128, 16, 64), ("scores", "in place", (1, 4), 256, 64, 8, 32),
+    ("context", "stacked", 4, 128, 128, 64, 64), ("context", "stacked", 3, 256, 32, 24, 64), ("context", "stacked", 2, 128, 64, 16, 128),
+    ("context", "in place", (2, 2), 128, 128, 16, 64), ("context", "in place", (1, 3), 128, 32, 8, 64),
+])
+def test_straight_line_tiles_equal_the_tiles_with_run_time_extents_bit_for_bit(case):
+    """Reductions of 32, 64 and 128 take a kernel whose reduction length is a template argument (operands of x
+    from global memory straight to LDS, no cleared accumulators, one descriptor per array); same tiles and same
+    order of summation as the kernel with run-time extents, which the tuning knob still selects: same bits."""
+    from faith_amd import _lib, ops
+    path, layout, pairs, Lx, Ly, D, red = case
+    batch, heads = pairs if layout == "in place" else (pairs, 1)
+    g = torch.Generator().manual_seed(61)
+    print(f"[case] straight-line dot tiles {case}", flush=True)
+    if path == "scores":
+        x = rand_bounds(g, batch * heads, Lx, D, red, ordered=False, sw=0.3, sb=1.0)
+        y = rand_bounds(g, batch * heads, Ly, D, red, ordered=False, sw=0.3, sb=1.0)
+        if layout == "in place":
+            run = lambda: ops.attention_scores(dev(side_by_side(x, heads)), dev(side_by_side(y, heads)), heads, 2.0, 0.1, 1)
+        else:
+            run = lambda: ops.dot_product_qk(dev(x), dev(y), 2.0, 0.1, 1)
+    else:       # probabilities [.., Lx, D, keys] times values [.., keys, D, width]: the reduction runs over the keys
+        width = Ly
+        probs = rand_bounds(g, batch * heads, Lx, D, red, ordered=False, sw=0.2, sb=0.5)
+        value = rand_bounds(g, batch * heads, red, D, width, ordered=False, sw=0.3, sb=1.0)
+        if layout == "in place":
+            run = lambda: ops.attention_context(dev(probs), dev(side_by_side(value, heads)), 2.0, 0.1, 1)
+        else:
+            run = lambda: ops.dot_product_v(dev(probs), dev(value), 2.0, 0.1, 1)
+    got = run()
+    torch.cuda.synchronize()
+    _lib.call("faith_tune_set", 2, 1)
+    try:
+        want = run()
+        torch.cuda.synchronize()
+    finally:
+        _lib.call("faith_tune_set", 2, 0)
+    for name, a, b in zip(("lw", "lb", "uw", "ub"), got, want):
+        assert torch.equal(a, b), f"{name}: {int((a != b).sum())} of {a.numel()} values differ"
