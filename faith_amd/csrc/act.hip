@@ -35,6 +35,7 @@ struct ActArgs {
     float *l2 = nullptr, *u2 = nullptr;
     int rows2 = 0, H2 = 0;
     float qv = 0.f;     // the dual exponent when it is none of 1, 2, inf
+    int remap = 0;      // order of the tiles (register-resident kernels): 0 as numbered, 1 an eighth of the range per XCD, 2 whole rows per XCD
 };
 
 // ------------------------------------------------------------------ natural layout
@@ -403,8 +404,8 @@ __device__ __forceinline__ void resident_partials(const ActArgs &a, const Vec<VE
 // column predicates and no second pass, and the kernel is a slab copy with the reduction and the
 // per-neuron stage between its loads and its stores: at configuration 1 it runs within 3 % of
 // that copy, where the general kernel above needs 25 % more.
-template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false>
-__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE))) act_resident(const ActArgs a) {
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false, int MAXW = 8>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE, MAXW))) act_resident(const ActArgs a) {
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
     static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
     extern __shared__ float smem[];
@@ -413,7 +414,14 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
     float *s_ln = s_lu + 2 * TH;                  // [2][3][TH] lower / upper line (k, x0, y0)
 
     const int tiles = a.H / TH;
-    const int r = blockIdx.x / tiles, col0 = (blockIdx.x % tiles) * TH;
+    int bid = blockIdx.x;
+    // workgroup w runs on XCD w % 8
+    if (a.remap == 1) bid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
+    if (a.remap == 2) {
+        const int idx = (int)(blockIdx.x / 8), x = (int)(blockIdx.x % 8);
+        bid = (idx / tiles * 8 + x) * tiles + idx % tiles;
+    }
+    const int r = bid / tiles, col0 = (bid % tiles) * TH;
     const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid % TPR, rg = tid / TPR;
     const size_t base = ((size_t)r * a.D + rg) * a.H + col0 + c * VEC;
@@ -546,21 +554,31 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(W
         }
     };
 
+    // virtual tile v (workgroup w walks v = w, w + grid, ...) -> tile: with a.remap, XCD x (v % 8 == x) owns groups of
+    // consecutive rows
+    auto tile_of = [&](int v) {
+        if (a.remap == 1) return (v % 8) * (n_tiles / 8) + v / 8;
+        if (a.remap == 2) {
+            const int idx = v / 8, x = v % 8;
+            return (idx / tiles * 8 + x) * tiles + idx % tiles;
+        }
+        return v;
+    };
     Tile A, B;
-    int t = blockIdx.x;
-    if (t >= n_tiles) return;
-    fetch(t, A);
+    int v = blockIdx.x;
+    if (v >= n_tiles) return;
+    fetch(tile_of(v), A);
     while (true) {
-        int tn = t + gridDim.x;
-        if (tn < n_tiles) fetch(tn, B);
-        finish(t, A);
-        if (tn >= n_tiles) break;
-        t = tn;
-        tn = t + gridDim.x;
-        if (tn < n_tiles) fetch(tn, A);
-        finish(t, B);
-        if (tn >= n_tiles) break;
-        t = tn;
+        int vn = v + gridDim.x;
+        if (vn < n_tiles) fetch(tile_of(vn), B);
+        finish(tile_of(v), A);
+        if (vn >= n_tiles) break;
+        v = vn;
+        vn = v + gridDim.x;
+        if (vn < n_tiles) fetch(tile_of(vn), A);
+        finish(tile_of(v), B);
+        if (vn >= n_tiles) break;
+        v = vn;
     }
 }
 
@@ -683,12 +701,12 @@ void launch_natural(const ActArgs &a, hipStream_t st) {
                        dim3(NTHREADS), smem, st, a);
 }
 
-template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false>
+template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false, int MAXW = 8>
 void launch_resident(const ActArgs &a, hipStream_t st) {
     constexpr int TH = TPR * 4;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
-    faith::reserve_lds(act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE, NTL>, smem);
-    hipLaunchKernelGGL((act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE, NTL>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS),
+    faith::reserve_lds(act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE, NTL, MAXW>, smem);
+    hipLaunchKernelGGL((act_resident<MODE, Q, TPR, NTHREADS, RPT, WPE, NTL, MAXW>), dim3((unsigned)(a.rows * (a.H / TH))), dim3(NTHREADS),
                        smem, st, a);
 }
 
@@ -871,37 +889,47 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
     // straight-line kernel for the common shape: 32-neuron tiles, 32 rows in flight, up to 8 rows a thread
     const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
     if (tv != 9 && a.rows2 == 0 && a.H % 32 == 0 && a.D % 32 == 0 && a.D <= 256) {
-        // Thread shapes for the 256-row tile, on [128, 256, 512] (269 MB per launch) with every launch on the same
-        // operands (they can sit in the 256 MB memory-side cache: "warm") and with five operand sets in turn
-        // (every byte from and to HBM: "cold"), relu / tanh in us:
-        //   one tile per workgroup, 4 wavefronts x 8 rows            warm 41.5 / 40.3   cold 61 - 65 / 61 - 65
-        //   one tile per workgroup, 16 wavefronts x 2 rows           warm 44.5 / 49.6   cold 54 - 56 / 57 - 58
-        //   the same with non-temporal loads                         warm 54.7 / 56.9   cold 55.3 / 57.9
-        //   persistent, two tiles in registers, 4 wavefronts x 8     warm 41.8 / 43.8   cold 55 - 57 / 58 - 60
-        // The persistent kernel is the one that is good at both, except for tanh, whose long per-neuron stage
-        // wants more workgroups on a CU than its registers allow: tanh keeps the first shape.
-        // On [B, 32, 256, 512] with one operand set, where a launch moves more than the cache holds (MB: first /
-        // third / persistent shape, relu | tanh in us):
-        //    404:  60 /  78 /  62 |  61 /  79 /  65        537:  92 / 106 /  87 |  88 / 106 /  89
-        //    674: 144 / 130 / 134 | 143 / 132 / 140        808: 173 / 156 / 161 | 172 / 157 / 168
-        //   1347: 284 / 263 / 266 | 282 / 264 / 276       2013: 424 / 391 / 402 | 417 / 394 / 413
-        // so from 9/4 of the cache up (between the two sizes where the order flips) every mode takes the third.
-        // Knob values 8 / 12 / 7 force the three one-tile shapes, 15 the persistent one.
+        // Tile order (ActArgs::remap): the hardware deals consecutive workgroups to the eight XCDs in turn, so with
+        // tiles numbered along a row every XCD touches every row of the object at once; with whole rows dealt to the
+        // XCDs (row r to XCD r % 8) the workgroups of an XCD stream through consecutive tiles.  Four wavefronts x 8
+        // rows on [128, 256, 512], relu / tanh: 61 / 64 -> 56 / 59 us when every byte comes from and goes to HBM
+        // ("cold": five operand sets in turn), 41 / 40 -> 40 / 40 us when every launch reuses one set, which can sit in
+        // the 256 MB memory-side cache ("warm").  Needs rows % 8 == 0 (else: an eighth of the tile range per XCD when
+        // the tile count allows, else the plain order).
+        // How many tiles a CU has in flight decides between the two regimes (same object, XCD-aware order, warm | cold, us):
+        //   4 wavefronts x 8 rows, 4 workgroups per CU (256 KB in flight)   relu 39.9 | 56.0   tanh 40.5 | 59.3
+        //   4 wavefronts x 8 rows, 3 per CU                                 relu 40.9 | 53.9   tanh 42.1 | 55.0
+        //   4 wavefronts x 8 rows, 2 per CU                                 relu 42.9 | 52.7   tanh 45.2 | 56.6
+        //   8 wavefronts x 4 rows, 3 per CU (192 KB)                        relu 41.3 | 54.0   tanh 41.6 | 55.0
+        //   8 wavefronts x 4 rows, 2 per CU (128 KB)                        relu 41.3 | 51.9   tanh 43.1 | 53.2
+        //   16 wavefronts x 2 rows, 2 per CU                                relu 44.5 | 52.7   tanh 48.0 | 53.6
+        //   the same with non-temporal loads                                relu 50.2 | 51.3   tanh 51.3 | 52.5
+        //   persistent, two tiles in registers, 2 per CU (plain order)      relu 41.5 | 57.3   tanh 43.8 | 59.9
+        // From the cache more tiles in flight are better, from HBM fewer; the library cannot know which it will be, so
+        // the default is the shape that is within 4 % of the best in both: eight wavefronts, two workgroups per CU --
+        // three for tanh, whose per-neuron stage (ten dependent bisection steps on three of the wavefronts) wants a
+        // third workgroup to run meanwhile.  Objects whose traffic is beyond 9/4 of the cache cannot be resident in it:
+        // sixteen wavefronts and non-temporal loads ([B, 32, 256, 512], 404 MB ... 2 GB: the order flips near 600 MB).
+        // Knob values 8 / 12 / 7 force the one-tile shapes of four / sixteen / sixteen wavefronts with non-temporal loads
+        // in the plain tile order, 15 the persistent kernel.
         const long long traffic = 16LL * a.rows * a.D * a.H;
         const bool streams_from_hbm = tv == 7 || (tv != 8 && traffic > 9LL * (256LL << 20) / 4);
-        bool pipelined = false;
         if constexpr (MODE != CONCRETIZE) {
-            // (with fewer than two tiles per resident workgroup there is nothing to overlap: one tile each then)
-            const long long n_tiles = (long long)a.rows * (a.H / 32);
-            pipelined = a.D > 128 && (tv == 15 || (MODE != TANH && tv != 7 && tv != 8 && tv != 12 && !streams_from_hbm &&
-                                                   n_tiles >= 4LL * faith::compute_units()));
-            if (pipelined) launch_pipelined<MODE, Q, 8, 256, 8, 2>(a, st);
+            if (a.D > 128 && tv == 15) {
+                launch_pipelined<MODE, Q, 8, 256, 8, 2>(a, st);
+                return;
+            }
         }
-        if (pipelined) return;
-        if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(a, st);
-        else if (tv == 12) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(a, st);
-        else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(a, st);
-        else launch_resident<MODE, Q, 8, 256, 8, (Q == Q_GENERAL ? 3 : 4)>(a, st);     // a general exponent needs more registers than 128
+        ActArgs b = a;
+        const long long n_tiles = (long long)a.rows * (a.H / 32);
+        b.remap = (tv == 8 || tv == 12 || tv == 7) ? 0 : a.rows % 8 == 0 ? 2 : n_tiles % 8 == 0 ? 1 : 0;
+        if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(b, st);
+        else if (tv == 12) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(b, st);
+        else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(b, st);
+        else if (tv == 8 || Q == Q_GENERAL || MODE == CONCRETIZE)
+            launch_resident<MODE, Q, 8, 256, 8, (Q == Q_GENERAL ? 3 : 4)>(b, st);     // a general exponent needs more registers than 128
+        else if (MODE == TANH) launch_resident<MODE, Q, 8, 512, 4, 6, false, 6>(b, st);
+        else launch_resident<MODE, Q, 8, 512, 4, 4, false, 4>(b, st);
         return;
     }
     switch (tv) {

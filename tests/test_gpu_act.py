@@ -110,10 +110,12 @@ def test_thread_shape_for_hbm_streams_gives_the_same_values(kind, p):
 @pytest.mark.parametrize("kind,p", [("relu", 2.0), ("relu", INF), ("exp", 1.0), ("sqr", 2.0), ("tanh", 2.0)])
 @pytest.mark.parametrize("rows", [40, 43])
 def test_persistent_two_tile_kernel_gives_the_one_tile_kernels_bits(kind, p, rows):
-    """An object with at least four 32-neuron tiles per CU runs every relaxation but tanh on persistent workgroups that
-    hold the next tile while they finish the current one (tuning knob 15 forces that kernel, 8 the one-tile kernel):
-    the arithmetic per tile is the same, so the results are, bit for bit -- also when the tiles do not divide
-    evenly among the workgroups (43 rows) -- and three rows of them are checked against the oracle."""
+    """The persistent kernel (workgroups that hold the next tile while they finish the current one: tuning knob 15)
+    against the one-tile kernel of four wavefronts (knob 8): the arithmetic per tile is the same, so the results are,
+    bit for bit -- also when the tiles do not divide evenly among the workgroups (43 rows).  The default shape (eight
+    wavefronts, whole rows dealt to the XCDs when the row count allows: 40 rows do, 43 do not) sums a column's partial
+    norms in another grouping: it is held to the one-tile kernel at the parity bar, a neuron whose interval end moved by
+    an ulp across a branch switch excepted (at most one in ten thousand), and three of its rows to the oracle."""
     from faith_amd import _lib, ops
     g = torch.Generator(device="cuda").manual_seed(12)
     shape = (1, rows, 256, 1024)
@@ -137,7 +139,8 @@ def test_persistent_two_tile_kernel_gives_the_one_tile_kernels_bits(kind, p, row
     torch.cuda.synchronize()
     for name, d, one, two in zip(("lw", "lb", "uw", "ub", "l", "u"), by_default, results[8], results[15]):
         assert torch.equal(one, two), f"{kind} {name}: the persistent kernel differs from the one-tile kernel"
-        assert torch.equal(d, one), f"{kind} {name}: the default differs from the one-tile kernel"
+        off = ((d.double() - one.double()).abs() > 1e-6 + 1e-5 * one.double().abs()).double().mean().item()
+        assert off <= 1e-4, f"{kind} {name}: the default shape is off the bar against the one-tile kernel on {off:.2e} of the values"
     for r in (0, rows // 2, rows - 1):
         x = O.LinearBounds(*(t[:, r:r + 1].cpu() for t in (lw, lb, uw, ub)))
         exp = getattr(O, kind)(x, p, 0.01, 2)
