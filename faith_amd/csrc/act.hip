@@ -202,7 +202,13 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     const bool second = MODE == CONCRETIZE && (int)blockIdx.x >= a.rows * tiles1;
     const int H = second ? a.H2 : a.H;
     const int tiles = (H + TH - 1) / TH;
-    const int bid = second ? blockIdx.x - a.rows * tiles1 : blockIdx.x;
+    int bid = second ? blockIdx.x - a.rows * tiles1 : blockIdx.x;
+    if (a.remap == 2) {
+        // whole rows of an object dealt to the XCDs (workgroup w runs on XCD w % 8; the launcher has checked that
+        // both objects start on a multiple of 8 and have a multiple of 8 rows)
+        const int idx = bid / 8, x = bid % 8;
+        bid = (idx / tiles * 8 + x) * tiles + idx % tiles;
+    }
     const float *__restrict__ p_lw = second ? a.lw2 : a.lw, *__restrict__ p_uw = second ? a.uw2 : a.uw;
     const float *__restrict__ p_lb = second ? a.lb2 : a.lb, *__restrict__ p_ub = second ? a.ub2 : a.ub;
     float *__restrict__ p_l = second ? a.l2 : a.l, *__restrict__ p_u = second ? a.u2 : a.u;
@@ -691,11 +697,15 @@ __global__ void __launch_bounds__(256) act_transposed(const ActArgs a) {
 
 // ------------------------------------------------------------------ host dispatch
 template <int MODE, int Q, int VEC, int TPR, int NTHREADS, int RPT>
-void launch_natural(const ActArgs &a, hipStream_t st) {
+void launch_natural(const ActArgs &a0, hipStream_t st) {
     constexpr int TH = TPR * VEC;
+    ActArgs a = a0;
     const int tiles = (a.H + TH - 1) / TH;
     const size_t smem = ((size_t)a.words * (NTHREADS / WAVE) * 2 * TH + 8 * TH) * sizeof(float);
     const int tiles2 = (a.H2 + TH - 1) / TH;
+    // the XCD-aware tile order of the register-resident kernels (dispatch_natural), where the row counts allow it
+    const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
+    a.remap = (tv == 0 && a.rows % 8 == 0 && tiles > 1 && (a.rows2 == 0 || (a.rows2 % 8 == 0 && ((long long)a.rows * tiles) % 8 == 0))) ? 2 : 0;
     faith::reserve_lds(act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>, smem);      // many perturbed words: beyond 64 KB
     hipLaunchKernelGGL((act_natural<MODE, Q, VEC, TPR, NTHREADS, RPT>), dim3((unsigned)(a.rows * tiles + a.rows2 * tiles2)),
                        dim3(NTHREADS), smem, st, a);

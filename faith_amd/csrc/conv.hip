@@ -52,6 +52,10 @@ struct ConvArgs {
     const float *bias;        // [Co] or nullptr
     float *yl, *yu;           // [N, Co, Ho, Wo]
     int N, Ci, H, W, Co, K, S, P, Ho, Wo;
+    // 1: whole images dealt to the XCDs (image n to XCD n % 8).  Consecutive workgroups run on the eight XCDs in turn;
+    // numbered along an image, its tiles land on different XCDs, each of which then writes every image's result in
+    // pieces; this way an XCD reads an image (halo rows and all) through one L2 and writes its planes whole.
+    int remap = 0;
 };
 
 __device__ __forceinline__ floatx16 mfma(float a, float b, floatx16 c) {
@@ -207,6 +211,10 @@ conv_signsplit_k3s1(const ConvArgs g) {
 
     const int tcol = (g.Wo + TC - 1) / TC, trow = (g.Ho + TR - 1) / TR, tco = (g.Co + TCO - 1) / TCO;
     int pid = blockIdx.x;
+    if (g.remap) {
+        const int per = tcol * trow * tco, idx = pid / 8, x = pid % 8;
+        pid = (idx / per * 8 + x) * per + idx % per;
+    }
     const int ow0 = (pid % tcol) * TC;  pid /= tcol;
     const int oh0 = (pid % trow) * TR;  pid /= trow;
     const int co0 = (pid % tco) * TCO;  pid /= tco;
@@ -425,6 +433,10 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     // first chunk before the last MFMAs of the current one as well measured no better (105 / 53.8 us).
     for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
     int pid = tile;
+    if (g.remap) {
+        const int per = tcol * trow * tco, idx = pid / 8, x = pid % 8;
+        pid = (idx / per * 8 + x) * per + idx % per;
+    }
     const int ow0 = (pid % tcol) * TC;  pid /= tcol;
     const int oh0 = (pid % trow) * TR;  pid /= trow;
     const int co0 = (pid % tco) * TCO;  pid /= tco;
@@ -645,8 +657,11 @@ bool launch_tile(const ConvArgs &g, hipStream_t st) {
     if (grid > 0x7fffffffLL) return false;
     if (!faith::reserve_lds(conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>, T::LDS)) return false;
     const long long resident = 2LL * faith::compute_units();      // two workgroups per CU at most (registers)
-    hipLaunchKernelGGL((conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>), dim3((unsigned)(grid < resident ? grid : resident)),
-                       dim3(NTHREADS), T::LDS, st, g, (int)grid);
+    const long long launched = grid < resident ? grid : resident;
+    ConvArgs h = g;
+    h.remap = (g.N % 8 == 0 && launched % 8 == 0 && faith::tune_get(FAITH_TUNE_CONV_VARIANT) != 2) ? 1 : 0;
+    hipLaunchKernelGGL((conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>), dim3((unsigned)launched), dim3(NTHREADS), T::LDS, st, h,
+                       (int)grid);
     return true;
 }
 
@@ -797,8 +812,11 @@ extern "C" int faith_convolution_verification(const float *x_lb, const float *x_
     const bool wvec = CIN % 4 == 0 && faith::aligned(W, 16);
     const int forced = faith::tune_get(FAITH_TUNE_CONV_VARIANT);      // 1: the general kernel, whatever the layer
     const bool full_tiles = (Wo - 1) % 32 >= 16 && (COUT - 1) % 128 >= 64;     // else a smaller tile wastes less
-    if (k3s1 && full_tiles && forced != 1)
+    if (k3s1 && full_tiles && forced != 1) {
+        gw.remap = (dim_in % 8 == 0 && forced != 2) ? 1 : 0;
         hipLaunchKernelGGL(conv_signsplit_k3s1, dim3((unsigned)grid), dim3(NTHREADS), 0, st, gw);
+        gw.remap = 0;
+    }
     else if (!(forced != 1 && offsets_fit && dispatch_fast(gw, wvec, st)))
         hipLaunchKernelGGL(conv_signsplit, dim3((unsigned)grid), dim3(NTHREADS), smem, st, gw);
 

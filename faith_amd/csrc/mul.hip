@@ -27,6 +27,7 @@ struct MulArgs {
     int rows, D, H, words;
     float eps;
     float qv = 0.f;     // the dual exponent when it is none of 1, 2, inf
+    int remap = 0;      // register-resident kernel: 2 = whole rows of the object dealt to the XCDs (row r to XCD r % 8)
 };
 
 template <int Q, int VEC, int TPR, int NTHREADS, int RPT>
@@ -181,7 +182,14 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(Q
     float *coef = part + a.words * NW * 4 * TH;  // [3][TH]: a_l, a_u, b
 
     const int tiles = a.H / TH;
-    const int r = blockIdx.x / tiles, col0 = (blockIdx.x % tiles) * TH;
+    // consecutive workgroups go to the eight XCDs in turn: with whole rows dealt to the XCDs the workgroups of an XCD
+    // stream through consecutive tiles instead of touching every row of the object at once
+    int bid = blockIdx.x;
+    if (a.remap == 2) {
+        const int idx = (int)(blockIdx.x / 8), x = (int)(blockIdx.x % 8);
+        bid = (idx / tiles * 8 + x) * tiles + idx % tiles;
+    }
+    const int r = bid / tiles, col0 = (bid % tiles) * TH;
     const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid % TPR, rg = tid / TPR;
     const size_t base = ((size_t)r * a.D + rg) * a.H + col0 + c * VEC;
@@ -328,7 +336,9 @@ void dispatch_mul(const MulArgs &a, hipStream_t st) {
     const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
     if (vec4 && a.H % 32 == 0 && a.D % 64 == 0 && a.D <= 256 && tv != 9) {
         // 32-neuron tiles, 512 threads holding 4 rows of each of the four tensors (64 values per thread)
-        launch_mul_resident<Q, 8, 512, 4>(a, st);
+        MulArgs b = a;
+        b.remap = (a.rows % 8 == 0 && tv != 8) ? 2 : 0;
+        launch_mul_resident<Q, 8, 512, 4>(b, st);
         return;
     }
     if (!vec4)
