@@ -36,7 +36,8 @@ METRIC = "bound-prop latency & TFLOP/s (matmul/dot/conv) or HBM GB/s (relu/tanh)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 INF = float("inf")
-WARM_SECONDS = 0.25            # minimum warm-up per measurement; --profile sets it to 0
+WARM_SECONDS = 0.25            # minimum warm-up per measurement; --profile shortens it (the trace stays small, yet the
+                               # launches that are timed, and most of those the profiler averages, run at settled clocks)
 
 COLD_SETS = 5                  # disjoint operand sets cycled by the cold measurement (1.35 GB between reuses)
 
@@ -308,8 +309,8 @@ def bench_config1(args, ops, O, wl, steps, warmup):
     tc = gpu_times_ms(lambda: _lib.call("faith_copy_f32", src.data_ptr(), dst.data_ptr(), src.numel(), st), 50, 5)
     entries.append(op_entry("plain copy of the same byte count (yardstick, not a bound op)", "hbm", tc, nbytes))
 
-    # Two kernels share a step evenly: relu (every relaxation but tanh) runs on the persistent two-tile kernel, tanh
-    # on the one-tile kernel.  `roofline` is the slower of the two (its slowest norm); the other is quoted under "also".
+    # Two instantiations of one kernel share a step evenly (relu: eight wavefronts, two workgroups per CU; tanh: three
+    # per CU).  `roofline` is the slower of the two (its slowest norm); the other is quoted under "also".
     slowest = {kind: max((k for k in per_kernel if k[0] == kind), key=lambda k: statistics.mean(per_kernel[k]))
                for kind in ("relu", "tanh")}
     dom = max(slowest.values(), key=lambda k: statistics.mean(per_kernel[k]))
@@ -317,7 +318,7 @@ def bench_config1(args, ops, O, wl, steps, warmup):
     avg_ms = statistics.mean(gpu_back_to_back_ms(lambda: one(*dom), 20))
     other_ms = statistics.mean(gpu_back_to_back_ms(lambda: one(*other), 20))
     traffic = traffic_from_profile()
-    kernel_of = {"relu": "act_pipelined", "tanh": "act_resident"}
+    kernel_of = {"relu": "act_resident", "tanh": "act_resident"}
     kernel = kernel_of[dom[0]]
     roofline = {"bound": "hbm", "kernel": f"{kernel}<{dom[0]}, p={dom[1]:g}>",
                 "achieved": round(nbytes / avg_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -352,8 +353,8 @@ def bench_config1(args, ops, O, wl, steps, warmup):
         entries.append(op_entry(f"config1 {kind} p={dom[1]:g} COLD: {COLD_SETS} disjoint operand sets in turn "
                                 f"({COLD_SETS * nbytes / 1e9:.2f} GB between reuses), average of back-to-back launches",
                                 "hbm", [cold_ms], nbytes))
-        # the one-tile kernel with sixteen wavefronts and non-temporal loads (what tanh takes by itself for objects
-        # that cannot be cache resident, more than 320 MB of traffic), forced here through the tuning knob
+        # the one-tile kernel with sixteen wavefronts and non-temporal loads (what every relaxation takes by itself for
+        # objects that cannot be cache resident, more than 576 MB of traffic), forced here through the tuning knob
         _lib.call("faith_tune_set", 0, 7)
         try:
             for _ in range(2 * COLD_SETS):
@@ -689,7 +690,7 @@ def main():
     args = ap.parse_args()
     if args.profile:
         global WARM_SECONDS
-        WARM_SECONDS = 0.0
+        WARM_SECONDS = 0.05
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every op is independent across the length axis and "
               "nothing here uses a second GPU, so --gpus must be 1", file=sys.stderr)
@@ -741,6 +742,25 @@ def main():
             f"{100 * e['frac']:5.1f}% of {e['peak']:g}"
             + (f"   ({rf['tflops']:.1f} TFLOP/s in the reference's formulation)" if rf else "")
             + (f"   cpu: {cb}" if cb else ""))
+
+    # the five configurations' dominant kernels inside `roofline` (the record that is kept whole): latency of the
+    # operator, the roofline that bounds it, the fraction reached (contractions: products executed, see EXECUTED)
+    def cfg_entry(prefix, kernel):
+        for e in entries:
+            if e["op"].startswith(prefix):
+                return {"kernel": kernel, "avg_us": e["latency_us"], "bound": e["bound"], "achieved": e["achieved"],
+                        "unit": e["unit"], "frac": e["frac"]}
+        return None
+    per_config = {
+        "0": cfg_entry("config0", "signsplit_gemm_concretize<1> (layer + dual norm, one launch; latency bound)"),
+        "1": {"kernel": head["roofline"]["kernel"], "avg_us": head["roofline"]["avg_launch_us"], "bound": "hbm",
+              "achieved": head["roofline"]["achieved"], "unit": "GB/s", "frac": head["roofline"]["frac"],
+              "cold_frac": head["roofline_cold"]["frac"]},
+        "2": cfg_entry("config2 linear [", "signsplit_gemm<true>"),
+        "3": cfg_entry("config3 dot_product", "dot_tiled<false, 8> + concretize + constant terms (whole operator)"),
+        "4": cfg_entry("config4 conv3x3", "conv_signsplit_k3s1 + constant terms (whole operator)"),
+    }
+    head["roofline"]["per_config"] = {k: v for k, v in per_config.items() if v is not None}
 
     line = {
         "metric": METRIC, "value": head["value"], "unit": "GB/s", "n_gpus": 1,

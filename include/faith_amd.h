@@ -239,6 +239,20 @@ int faith_layer_norm_verification(const float *src_lb, const float *src_ub,
  *   W          [dim_y_out, dim_out]              nn.Linear layout
  *   bias       [dim_y_out] or NULL
  *   y_lw, y_uw [batch*length, dim_in, dim_y_out];  y_lb, y_ub [batch*length, dim_y_out]
+ *
+ * Arithmetic.  The reference forms W+ = W (W > 0), W- = W - W+ and four fp32 products per term,
+ *   y_l = x_l W+ + x_u W-,   y_u = x_u W+ + x_l W-.
+ * Since W+ + W- = W and W+ - W- = |W|, the same two results are  y_l = M - R,  y_u = M + R  with
+ *   M = ((x_l + x_u) / 2) W      (centre),     R = ((x_u - x_l) / 2) |W|      (radius):
+ * two products per term, which is what the kernels multiply (the sum and the difference of a coefficient pair
+ * are rounded to fp32 once, by the thread that stages them; the halving is exact).  Consequences a binder can
+ * rely on: (1) with x_u >= x_l element-wise R is a sum of non-negative products, so y_u >= y_l holds bit for
+ * bit; (2) each result carries the rounding of BOTH operands' terms: its forward error is bounded by
+ * (K + 2) u sum_k (|x_l| + |x_u|)_k |W|_k / 2 (u = 2^-24, K the reduction length) where the four-product form has
+ * (K + 1) u sum_k |x_l|_k W+_k + |x_u|_k |W-|_k; measured against float64 on data shaped like the benchmark
+ * configurations it is 1.3 - 1.9 times the four-product form's error and under 0.15 of rtol 1e-5 / atol 1e-6;
+ * (3) the inputs must be finite (an infinite pair of opposite signs has no centre).  The constant terms
+ * y_lb, y_ub are accumulated in double and rounded once.  Results are not bit-identical to the four-product form.
  */
 int faith_matmul_verification(const float *x_lb, const float *x_ub,
                               const float *x_lw, const float *x_uw,
@@ -326,6 +340,11 @@ int faith_matmul_group_rows_verification(const float *x_lb, const float *x_ub,
  * The reference entry has one `length`; here x and y may differ in length.  With dim_in == 1 the
  * result is the interval product of the constant terms (Bounds.py:711-721); x_l .. y_u are written
  * all the same.  words must divide dim_in.
+  * Arithmetic: of the eight products per term that Bounds.ori_dot_product writes, the four y terms share their
+ * multiplier b = x_l, and b+ + b- = b, b+ - b- = |b|, so they are computed as P + Q and P - Q with
+ * P = sum (b / 2)(y_lw + y_uw), Q = sum (|b| / 2)(y_lw - y_uw): six products per term; y_lw +- y_uw are rounded to fp32
+ * once.  The constant terms z_lb, z_ub are accumulated in double.  Not bit-identical to the eight-product form; within
+ * rtol 1e-5 / atol 1e-6 of it on data shaped like the benchmark configurations.
  */
 int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u,
                                       const float *x_lb, const float *x_ub,
@@ -496,6 +515,10 @@ int faith_attention_context_compact(float *x_l, float *x_u, const float *y_l, co
  *   W          [COUT, CIN, K, K];  bias [COUT] or NULL (added to y_lb / y_ub only)
  *   y_lw, y_uw [dim_in, COUT, Ho, Wo];  y_lb, y_ub [batch_size, COUT, Ho, Wo]
  *   Ho = (Height + 2*padding_size - K) / Stride + 1, likewise Wo.
+ * Arithmetic: as faith_matmul_verification -- y_l = M - R, y_u = M + R with M = conv((x_l + x_u) / 2, W) and
+ * R = conv((x_u - x_l) / 2, |W|), two products per tap instead of the four of conv(x_l, W+) + conv(x_u, W-) and its
+ * mirror; same consequences (y_u >= y_l bit for bit for ordered inputs, the error bound with K = CIN * K * K,
+ * finite inputs); constant terms accumulated in double.
  */
 int faith_convolution_verification(const float *x_lb, const float *x_ub,
                                    const float *x_lw, const float *x_uw,

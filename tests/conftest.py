@@ -60,3 +60,19 @@ def pytest_terminal_summary(terminalreporter):
         f"(rtol 1e-5 / atol 1e-6), concessions: {kinds if kinds else 'none'} (each one in {LEDGER_DIR}/parity_ledger.json)")
     for (fn, kind, tensor), n in sorted(per_test.items()):
         terminalreporter.write_line(f"  {n:4d} x {kind:<24s} {tensor:<6s} {fn}")
+    # every contraction tensor, conceded or not: the worst distance from float64 per test, GPU and fp32 oracle, in
+    # units of the plain bar, and the worst ratio among the tensors whose GPU error is at least a quarter of the bar
+    worst = {}
+    for c in led.get("contractions", []):
+        fn = c["test"].split("[")[0]
+        w = worst.setdefault(fn, dict(n=0, gpu=0.0, oracle=0.0, ratio=0.0))
+        w["n"] += 1
+        w["gpu"] = max(w["gpu"], c["gpu_err_of_bar"])
+        w["oracle"] = max(w["oracle"], c["oracle_err_of_bar"])
+        if c["gpu_err_of_bar"] >= 0.25:
+            w["ratio"] = max(w["ratio"], c["ratio"])
+    if worst:
+        terminalreporter.write_line("contractions against float64, worst per test (units of the plain bar): tensors, GPU, fp32 "
+                                    "oracle, worst GPU / oracle ratio where the GPU error reaches a quarter of the bar")
+        for fn, w in sorted(worst.items()):
+            terminalreporter.write_line(f"  {w['n']:5d}  gpu {w['gpu']:8.3f}  oracle {w['oracle']:8.3f}  ratio {w['ratio']:6.2f}  {fn}")

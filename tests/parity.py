@@ -39,7 +39,14 @@ RTOL, ATOL = 1e-5, 1e-6
 # tensor, which concession, how large -- and every comparison is counted.  tests/conftest.py prints
 # the totals at the end of the session and writes them to parity_ledger.json in the run's output folder, so a run
 # shows how many tensors or neurons leaned on a concession even when it prints nothing else.
-LEDGER = {"comparisons": 0, "plain": 0, "concessions": []}
+LEDGER = {"comparisons": 0, "plain": 0, "concessions": [], "contractions": []}
+
+# Ceiling on (GPU error against float64) / (fp32 CPU oracle's error against float64), both in units of the plain bar,
+# for data shaped like the benchmark configurations (ordered bounds, small widths): a summation in another order
+# may be a few times further from the exact value than the oracle's blocked one, not more.  Below a quarter of the
+# bar the ratio says nothing (both are rounding noise) and is not asserted.
+CONFIG_RATIO = 3.0
+RATIO_FLOOR = 0.25
 
 
 def _note(kind, name, **detail):
@@ -149,7 +156,11 @@ CONSTANT_TERMS = {"lb": B_IN_DOUBLE, "ub": B_IN_DOUBLE}
 UNIT_SCALE_ALL = {"lw": UNIT_SCALE, "uw": UNIT_SCALE, "lb": B_IN_DOUBLE, "ub": B_IN_DOUBLE}
 
 
-def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None, ref64_own=None):
+def _of_bar(err, ref):
+    return float((err / (ATOL + RTOL * ref.abs())).max())
+
+
+def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None, ref64_own=None, ratio_ceiling=None):
     """Parity of one output tensor of a contraction.
 
     `ref64_own` (dot products): the float64 value of the same formula evaluated from the concrete
@@ -185,12 +196,23 @@ def compare_contraction(name, got, oracle32, ref64, abs_terms, allow=None, ref64
         allow = allow.get(name)
     got = got.detach().cpu().double()
     o32 = oracle32.detach().cpu().double()
+    ref64 = ref64.detach().cpu().double()
+    oerr = (o32 - ref64).abs()                       # the oracle against the float64 value of ITS intervals
+    # every tensor, conceded or not: how far the GPU and the oracle are from float64, in units of the plain bar
+    # (the GPU against the float64 value of its own intervals where the caller has it)
+    own = ref64 if ref64_own is None else ref64_own.detach().cpu().double()
+    e_gpu, e_or = _of_bar((got - own).abs(), own), _of_bar(oerr, ref64)
+    LEDGER["contractions"].append(dict(test=os.environ.get("PYTEST_CURRENT_TEST", "").split(" (")[0], tensor=name,
+                                       gpu_err_of_bar=e_gpu, oracle_err_of_bar=e_or,
+                                       ratio=e_gpu / e_or if e_or > 0 else float("inf") if e_gpu > 0 else 1.0))
+    if ratio_ceiling is not None:
+        assert e_gpu <= max(ratio_ceiling * e_or, RATIO_FLOOR), \
+            (f"{name}: the GPU is {e_gpu:.3f} of the bar from float64, the fp32 oracle {e_or:.3f}: more than "
+             f"{ratio_ceiling:g} x on data shaped like a benchmark configuration")
     if not bool(_bad(got, o32).any()):
         _count(True)
         return "plain"
     missed = _bad(got, o32)
-    ref64 = ref64.detach().cpu().double()
-    oerr = (o32 - ref64).abs()                       # the oracle against the float64 value of ITS intervals
     if ref64_own is not None:
         ref64 = ref64_own.detach().cpu().double()    # the GPU against the float64 value of ITS intervals
         explained = missed & ~_bad(got, ref64)

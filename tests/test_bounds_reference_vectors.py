@@ -174,13 +174,13 @@ def test_hip_products_softmax_and_layer_norm_match_the_reference(tag):
     print(f"[case] products, softmax, layer_norm {tag} against the executed reference", flush=True)
     x = gpu_bounds("any_in", p, EPS, words)
     assert_matches(quad(x.multiply(gpu_bounds("any2_in", p, EPS, words))), f"multiply_{tag}", "multiply")
-    # composed operators: the bar of their composition on the GPU (sums of H terms in another order)
-    assert_matches(quad(x.divide(gpu_bounds("pos_in", p, EPS, words))), f"divide_{tag}", "divide", rtol=5e-5, atol=4e-6)
-    assert_matches(quad(gpu_bounds("soft_in", p, EPS_SOFT, words).softmax()), f"softmax_{tag}", "softmax", rtol=5e-5, atol=4e-6)
+    # the composed operators too are held to the plain bar (measured: at most 0.05 of it on these vectors)
+    assert_matches(quad(x.divide(gpu_bounds("pos_in", p, EPS, words))), f"divide_{tag}", "divide")
+    assert_matches(quad(gpu_bounds("soft_in", p, EPS_SOFT, words).softmax()), f"softmax_{tag}", "softmax")
     normalizer = SimpleNamespace(weight=t(G["norm_weight"]).cuda(), bias=t(G["norm_bias"]).cuda())
     for mode, key in (("no_var", "novar"), ("standard", "standard")):
         y = gpu_bounds("norm_in", p, EPS_NORM, words).layer_norm(normalizer, mode)
-        assert_matches(quad(y), f"layernorm_{key}_{tag}", f"layer_norm {mode}", rtol=5e-5, atol=4e-6)
+        assert_matches(quad(y), f"layernorm_{key}_{tag}", f"layer_norm {mode}")
 
 
 @pytest.mark.gpu
@@ -255,4 +255,4 @@ def test_hip_interval_mode_matches_the_reference():
     assert_interval(y.lb, y.ub, "matmul", "ibp matmul")
     normalizer = SimpleNamespace(weight=t(G["ibp_norm_weight"]).cuda(), bias=t(G["ibp_norm_bias"]).cuda())
     z = x.layer_norm(normalizer, "no_var")
-    assert_interval(z.lb, z.ub, "layernorm_novar", "ibp layer_norm", rtol=5e-5, atol=4e-6)
+    assert_interval(z.lb, z.ub, "layernorm_novar", "ibp layer_norm")
