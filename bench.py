@@ -752,7 +752,7 @@ def main():
                         "unit": e["unit"], "frac": e["frac"]}
         return None
     per_config = {
-        "0": cfg_entry("config0", "signsplit_gemm_concretize<1> (layer + dual norm, one launch; latency bound)"),
+        "0": cfg_entry("config0", "signsplit_gemm_concretize_short<inf, 4> (layer + dual norm, one launch; latency bound)"),
         "1": {"kernel": head["roofline"]["kernel"], "avg_us": head["roofline"]["avg_launch_us"], "bound": "hbm",
               "achieved": head["roofline"]["achieved"], "unit": "GB/s", "frac": head["roofline"]["frac"],
               "cold_frac": head["roofline_cold"]["frac"]},

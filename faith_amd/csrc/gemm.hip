@@ -990,6 +990,152 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_concretize(const Fuse
     }
 }
 
+// The same launch for SHORT reductions (K = 16 * NS, NS = 2 / 4 / 8): a workgroup owns one position and 16
+// columns, a wavefront takes 16-row blocks of the position as 16 x 16 MFMA blocks (v_mfma_f32_16x16x4_f32: half
+// the cycles of a 32 x 32 x 2 step for a quarter of the block), and every fragment of a block -- the whole
+// reduction -- is requested before the first MFMA, so that a block costs one memory latency instead of one per
+// group of K-steps.  Lane group g = lane / 16 holds k = 4 * NS * g .. 4 * NS * (g + 1) - 1 of its row (A) or
+// column (W) as NS float4; MFMA (q, c) multiplies component c of piece q, i.e. the four k values
+// {4 NS g + 4 q + c : g = 0 .. 3}.  With dim_in = 64 all four wavefronts have a block (the 32 x 32 form leaves
+// two idle) and twice as many workgroups share the problem.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <int Q, int NS>
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_concretize_short(const FusedArgs f) {
+    constexpr int K = 16 * NS;
+    __shared__ float part[FUSED_MAX_WORDS * 4 * 2 * 16];          // [word][wavefront][l, u][column]
+    __shared__ double red[2][16][17];                              // constant terms: [l, u][K slice][column]
+    const GemmArgs &g = f.g;
+    const int tiles_n = (g.N + 15) / 16;
+    const int row = blockIdx.x / tiles_n, n0 = (blockIdx.x % tiles_n) * 16;
+    const int tid = threadIdx.x, lane = tid % 64, wv = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int fi = lane % 16, fg = lane / 16;
+    const int col = n0 + fi;
+
+    // ---- every load of the first block and of the constant terms goes out first
+    const float4 *__restrict__ pw = reinterpret_cast<const float4 *>(g.W + (size_t)min(col, g.N - 1) * K) + NS * fg;
+    float4 w[NS];
+#pragma unroll
+    for (int q = 0; q < NS; ++q) w[q] = pw[q];
+    const int blocks = f.D / 16, blk = f.D / f.words;
+    float4 al[NS], au[NS];
+    auto fetch = [&](int db) {
+        const float4 *__restrict__ pal = reinterpret_cast<const float4 *>(g.Al + ((size_t)row * f.D + db * 16 + fi) * K) + NS * fg;
+        const float4 *__restrict__ pau = reinterpret_cast<const float4 *>(g.Au + ((size_t)row * f.D + db * 16 + fi) * K) + NS * fg;
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+            al[q] = pal[q];
+            au[q] = pau[q];
+        }
+    };
+    if (wv < blocks) fetch(wv);
+
+    // ---- constant terms of (row, n0 .. n0 + 15): sixteen K slices per column, lanes along K
+    {
+        const int c = tid / 16, ks = tid % 16;
+        const float *__restrict__ wr = g.W + (size_t)min(n0 + c, g.N - 1) * K;
+        const float *__restrict__ xl = g.Bl + (size_t)row * K, *__restrict__ xu = g.Bu + (size_t)row * K;
+        double accm = 0.0, accr = 0.0;
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            const int k = ks + 16 * i;
+            const double wk = wr[k], a = xl[k], b = xu[k];
+            accm += wk * (0.5 * (a + b));
+            accr += fabs(wk) * (0.5 * (b - a));
+        }
+        red[0][ks][c] = accm - accr;
+        red[1][ks][c] = accm + accr;
+    }
+    if (lane < 32)
+        for (int wd = 0; wd < f.words; ++wd) part[((wd * 4 + wv) * 2) * 16 + lane] = 0.f;
+
+    // ---- coefficient rows: 16 x 16 blocks of this position, one per wavefront at a time
+    float4 wa[NS];
+#pragma unroll
+    for (int q = 0; q < NS; ++q) wa[q] = abs4(w[q]);
+    for (int db = wv; db < blocks; db += 4) {
+        const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+        floatx4 cl = zero, cu = zero;
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+            const float4 am = mid4(al[q], au[q]), ar = rad4(al[q], au[q]);
+#define FAITH_STEP(c)                                                           \
+    cl = __builtin_amdgcn_mfma_f32_16x16x4f32(am.c, w[q].c, cl, 0, 0, 0);       \
+    cu = __builtin_amdgcn_mfma_f32_16x16x4f32(ar.c, wa[q].c, cu, 0, 0, 0);
+            FAITH_STEP(x)
+            FAITH_STEP(y)
+            FAITH_STEP(z)
+            FAITH_STEP(w)
+#undef FAITH_STEP
+        }
+        if (db + 4 < blocks) fetch(db + 4);                       // in flight while this block is finished
+        // register r of the block is row 4 * (lane / 16) + r, column lane % 16
+        const size_t r0 = (size_t)row * f.D + db * 16 + 4 * fg;
+        float pl = 0.f, pu = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float c = cl[r], rd = cu[r];                      // twice the centre and radius terms
+            const float lo = 0.5f * (c - rd), up = 0.5f * (c + rd);
+            pl = nacc<Q>(pl, lo, f.qv);
+            pu = nacc<Q>(pu, up, f.qv);
+            if (col < g.N) {
+                g.Cl[(r0 + r) * g.N + col] = lo;
+                g.Cu[(r0 + r) * g.N + col] = up;
+            }
+        }
+        pl = ncomb<Q>(pl, __shfl_xor(pl, 16, 64));
+        pu = ncomb<Q>(pu, __shfl_xor(pu, 16, 64));
+        pl = ncomb<Q>(pl, __shfl_xor(pl, 32, 64));
+        pu = ncomb<Q>(pu, __shfl_xor(pu, 32, 64));
+        if (fg == 0) {
+            const int w_id = (db * 16) / blk;                       // a block lies inside one perturbed word
+            float *slot = part + ((w_id * 4 + wv) * 2) * 16 + fi;
+            slot[0] = ncomb<Q>(slot[0], pl);
+            slot[16] = ncomb<Q>(slot[16], pu);
+        }
+    }
+    __syncthreads();
+
+    // ---- constant terms out, and the interval: l = lb' - eps * sum over words of the norm (Bounds.py:311-326)
+    if (tid < 16 && n0 + tid < g.N) {
+        double sl = red[0][0][tid], su = red[1][0][tid];
+#pragma unroll
+        for (int s = 1; s < 16; ++s) {
+            sl += red[0][s][tid];
+            su += red[1][s][tid];
+        }
+        const float add = g.bias ? g.bias[n0 + tid] : 0.f;         // added to the rounded product (Bounds.py:391-395)
+        const float lb = (float)sl + add, ub = (float)su + add;
+        const size_t o = (size_t)row * g.N + n0 + tid;
+        g.Dl[o] = lb;
+        g.Du[o] = ub;
+        float l = lb, u = ub;
+        for (int wd = 0; wd < f.words; ++wd) {
+            float nl = 0.f, nu = 0.f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                nl = ncomb<Q>(nl, part[((wd * 4 + v) * 2 + 0) * 16 + tid]);
+                nu = ncomb<Q>(nu, part[((wd * 4 + v) * 2 + 1) * 16 + tid]);
+            }
+            l = __fadd_rn(l, __fmul_rn(-f.eps, nfin<Q>(nl, f.qv)));
+            u = __fadd_rn(u, __fmul_rn(f.eps, nfin<Q>(nu, f.qv)));
+        }
+        f.l[o] = l;
+        f.u[o] = u;
+    }
+}
+
+template <int NS>
+void launch_concretize_short(const FusedArgs &f, int q, dim3 gd, hipStream_t st) {
+    const dim3 bd(NTHREADS);
+    switch (q) {
+        case FAITH_Q_1: hipLaunchKernelGGL((signsplit_gemm_concretize_short<FAITH_Q_1, NS>), gd, bd, 0, st, f); break;
+        case FAITH_Q_2: hipLaunchKernelGGL((signsplit_gemm_concretize_short<FAITH_Q_2, NS>), gd, bd, 0, st, f); break;
+        case FAITH_Q_INF: hipLaunchKernelGGL((signsplit_gemm_concretize_short<FAITH_Q_INF, NS>), gd, bd, 0, st, f); break;
+        default: hipLaunchKernelGGL((signsplit_gemm_concretize_short<Q_GENERAL, NS>), gd, bd, 0, st, f); break;
+    }
+}
+
 }  // namespace
 
 extern "C" int faith_matmul_concretize_verification(const float *x_lb, const float *x_ub, const float *x_lw,
@@ -1029,10 +1175,20 @@ extern "C" int faith_matmul_concretize_verification(const float *x_lb, const flo
     // and 44 against 24 us for the 256 -> 2 classifier (512), whose few positions leave the tiled kernel more
     // workgroups than this one has
     const long long chain = (long long)((dim_in + 127) / 128) * dim_out;
-    if (fits && (pick == 6 || (pick == 0 && tiles64 <= cus && chain <= 128))) {
+    if (fits && (pick == 6 || pick == 8 || (pick == 0 && tiles64 <= cus && chain <= 128))) {
         f.g = GemmArgs{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
         f.l = l; f.u = u; f.D = dim_in; f.words = words; f.eps = epsilon;
         hipStream_t st = static_cast<hipStream_t>(stream);
+        // short reductions: 16 x 16 blocks, 16 columns per workgroup (knob value 8 keeps the 32 x 32 form)
+        const long long grid16 = rows * ((dim_y_out + 15) / 16);
+        if (pick != 8 && (dim_out == 32 || dim_out == 64 || dim_out == 128) && dim_in % (16 * words) == 0 &&
+            grid16 <= 0x7fffffffLL) {
+            const dim3 gd16((unsigned)grid16);
+            if (dim_out == 32) launch_concretize_short<2>(f, q, gd16, st);
+            else if (dim_out == 64) launch_concretize_short<4>(f, q, gd16, st);
+            else launch_concretize_short<8>(f, q, gd16, st);
+            return faith::check_launch("faith_matmul_concretize_verification");
+        }
         const dim3 gd((unsigned)grid), bd(NTHREADS);
         switch (q) {
             case FAITH_Q_1: hipLaunchKernelGGL(signsplit_gemm_concretize<FAITH_Q_1>, gd, bd, 0, st, f); break;

@@ -199,7 +199,8 @@ def test_mfma_clock_measurement_is_plausible():
 
 # ---- affine layer + concretization through one entry point (one launch for small problems)
 def run_fused(x, W, bias, p, eps, words, force=None):
-    """force: None = built-in choice, 6 = the one-launch kernel wherever the shape allows, 1 = never."""
+    """force: None = built-in choice, 6 = the one-launch kernel wherever the shape allows (16 x 16 blocks where
+    the reduction is 32, 64 or 128 long), 8 = the same with 32 x 32 blocks throughout, 1 = never."""
     from faith_amd import ops, _lib
     lw, lb, uw, ub, W, bias = dev(*x.tensors(), W, bias)
     if force is not None:
@@ -221,17 +222,22 @@ def run_fused(x, W, bias, p, eps, words, force=None):
     (1, 2, 512, 200, 100, 4),    # more blocks than wavefronts, four words
     (1, 4, 96, 64, 64, 3),       # blocks per word not a multiple of the wavefronts
     (1, 40, 256, 128, 96, 1),    # several rounds of workgroups (forced)
+    (2, 3, 48, 32, 20, 3),       # 16-row blocks, one per word; reduction of 32; columns ragged against 16
+    (1, 2, 144, 128, 17, 1),     # nine 16-row blocks over four wavefronts, reduction of 128
 ])
 @pytest.mark.parametrize("p", [1.0, 2.0, INF, 3.0])
-def test_linear_concretize_one_launch(shape, p):
+@pytest.mark.parametrize("form", [6, 8])
+def test_linear_concretize_one_launch(shape, p, form):
     B, L, D, H, N, words = shape
-    print(f"[case] linear_concretize forced one-launch shape={shape} p={p}", flush=True)
+    if form == 8 and H not in (32, 64, 128):
+        pytest.skip("same kernel as form 6")
+    print(f"[case] linear_concretize forced one-launch form={form} shape={shape} p={p}", flush=True)
     g = torch.Generator().manual_seed(77)
     x = rand_bounds(g, B, L, D, H, ordered=False, sw=0.5)
     W = torch.randn(N, H, generator=g) / H ** 0.5
     bias = 0.01 * torch.randn(N, generator=g)
     eps = 0.02
-    got = run_fused(x, W, bias, p, eps, words, force=6)
+    got = run_fused(x, W, bias, p, eps, words, force=form)
     exp = O.linear(x, W, bias)
     ref, mag = linear64(x, W, bias)
     for name, a, e in zip(("lw", "lb", "uw", "ub"), got[:4], exp.tensors()):
