@@ -42,6 +42,10 @@ SIGNATURES = {
     "faith_matmul_verification": [_P] * 10 + [_I] * 5 + [_P],
     "faith_matmul_concretize_verification": [_P] * 12 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_matmul_group_verification": [_P] * 4 + [_I] + [_P] * 6 + [_I] * 5 + [_P],
+    "faith_matmul_relu_fits": [ctypes.c_longlong] + [_I] * 4,           # answers 0 / 1 / 2 as well
+    "faith_matmul_relu_verification": [_P] * 10 + [_I] * 5 + [_F, _I, _I, _P],
+    "faith_matmul_layer_norm_fits": [ctypes.c_longlong] + [_I] * 4,     # answers 0 / 1 / 2 instead of a status: call it through `lib`
+    "faith_matmul_layer_norm_verification": [_P] * 11 + [_I] + [_P] * 6 + [_I] * 5 + [_P],
     "faith_matmul_rows_verification": [_P] * 10 + [ctypes.c_longlong, ctypes.c_longlong, _I, _I, _P],
     "faith_matmul_group_rows_verification": [_P] * 4 + [_I] + [_P] * 6 + [ctypes.c_longlong, ctypes.c_longlong, _I, _I, _P],
     "faith_dot_product_verification_QK": [_P] * 16 + [_I] * 5 + [_F, _I, _I, _I, _P],

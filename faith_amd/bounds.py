@@ -177,6 +177,50 @@ class Bounds:
         bias = getattr(dense, "bias", None)
         return self.matmul(dense.weight.detach(), None if bias is None else bias.detach().contiguous())
 
+    def dense_act(self, dense, act_name):
+        """`self.dense(dense).act(act_name)` (VerifierForward.py:171-179).  ReLU with a dim_in the kernel takes and
+        enough positions to fill the device: one pass over the coefficients, in which the layer's result does not
+        reach memory; otherwise the separate operators."""
+        W = dense.weight.detach().contiguous()
+        if (act_name == "relu" and not self.ibp and W.dim() == 2
+                and ops.linear_relu_fits(self.lb.shape[0] * self.lb.shape[1], self.dim_in, W.shape[1], W.shape[0],
+                                         self.perturbed_words) == 2):
+            bias = getattr(dense, "bias", None)
+            bias = None if bias is None else bias.detach().contiguous()
+            try:
+                return self._like(*ops.linear_relu(*self._c(), W, bias, self.p, self.eps, self.perturbed_words))
+            except _lib.FaithError as err:
+                if err.code != _lib.ERR_UNSUPPORTED:         # e.g. tensors that are not 16-byte aligned
+                    raise
+        return self.dense(dense).act(act_name)
+
+    def dense_layer_norm(self, dense, normalizer, layer_norm, residual=None):
+        """`self.dense(dense).add(residual).layer_norm(normalizer, layer_norm)` (VerifierForward.py:166, 181-189).
+        Mode "no_var" with a hidden size the kernel takes: one pass over the coefficients, in which neither the
+        layer's result nor the sum reaches memory (a residual that is a CompactBounds is read from the rows it
+        holds); otherwise the separate operators."""
+        W = dense.weight.detach().contiguous()
+        words = residual._lw.shape[1] if isinstance(residual, CompactBounds) else 0
+        if (layer_norm == "no_var" and not self.ibp and W.dim() == 2
+                and ops.linear_layer_norm_fits(self.lb.shape[0] * self.lb.shape[1], self.dim_in, W.shape[1], W.shape[0],
+                                               words) == 2):
+            bias = getattr(dense, "bias", None)
+            bias = None if bias is None else bias.detach().contiguous()
+            weight, shift = normalizer.weight.detach().contiguous(), normalizer.bias.detach().contiguous()
+            other = positions = None
+            if isinstance(residual, CompactBounds):
+                other = (residual._lw.contiguous(), residual._lb.contiguous(), residual._uw.contiguous(),
+                         residual._ub.contiguous())
+                positions = residual.positions
+            elif residual is not None:
+                other = residual._c()
+            try:
+                return self._like(*ops.linear_layer_norm(*self._c(), W, bias, weight, shift, other, positions))
+            except _lib.FaithError as err:
+                if err.code != _lib.ERR_UNSUPPORTED:         # e.g. tensors that are not 16-byte aligned
+                    raise
+        return self.dense(dense).layer_norm(normalizer, layer_norm, residual=residual)
+
     def dense_concretize(self, dense):
         """(self.dense(dense), its concrete interval) through one entry point -- one launch for small problems such
         as the classifier, whose result is concretized at once (VerifierForward.py:300-314).  Returns (bounds, l, u)."""
@@ -430,6 +474,12 @@ class CompactBounds:
         weights = [layer.weight.detach().contiguous() for layer in layers]
         biases = [None if getattr(layer, "bias", None) is None else layer.bias.detach().contiguous() for layer in layers]
         return self._affine(weights, biases)
+
+    def dense_layer_norm(self, dense, normalizer, layer_norm, residual=None):
+        return self.dense(dense).layer_norm(normalizer, layer_norm, residual=residual)
+
+    def dense_act(self, dense, act_name):
+        return self.dense(dense).act(act_name)
 
     # ---- Bounds.py:319-326 on the rows that have coefficients; the constants are the bounds of the others
     def concrete_intervals(self):

@@ -43,7 +43,7 @@
 // the N-tiles that share an M-block (and with it A_l / A_u rows) are given ids 8 apart and
 // meet in the same L2.
 #include "common.h"
-#include "relax_common.h"
+#include "relax_lines.h"
 
 namespace {
 
@@ -103,9 +103,35 @@ __device__ __forceinline__ int swz(int row, int c) { return row * 8 + 4 * (c ^ (
 // NQ >= 0 (a dual-norm selector): the tile's contribution to the column norms of C_l and C_u -- over its BM rows,
 // which the caller guarantees to exist and to belong to one position -- is folded into pl / pu, one running
 // value per lane and column block; NQ = -1: no norms.
-template <bool EXACT, int MBM, int MBN, int NQ = -1>
+// Epilogue of the tiles that hold whole rows of the result (the 64-row tile with all dim_y_out = 64 MBN columns):
+// a second bound object is added and the rows go through the layer normalisation without the variance
+// (Bounds.add, Bounds.layer_norm "no_var": Bounds.py:1016-1025, :1111-1131) before they are stored -- the sum
+// and the layer's own result never reach memory.
+struct RowNormArgs {
+    const float *res_l, *res_u;     // coefficients of the added object, or null
+    const long long *positions;     // null: its rows are the [Mw, N] rows of the result.  Otherwise it holds the dim_in
+    int words, length, dim_in;      // rows of `words` positions per batch element only ([batch, words, dim_in, N];
+                                    // positions [batch, words]): rows of other positions are zero
+    const float *weight;            // [N] or null
+    float *out_l, *out_u;           // [Mw, N]
+};
+
+// Epilogue of the tiles that hold every coefficient row of one position (BM = dim_in, one perturbed word): the
+// column norms over those rows are complete inside the tile, so the concrete interval of each of its neurons and
+// from it the two lines of the ReLU relaxation (Bounds.relu, Bounds.py:921-963) are known before the tile is
+// stored -- the layer's own result never reaches memory.  The constant terms of the layer (g.Dl, g.Du) have been
+// written by the launch before.
+struct ReluArgs {
+    float *out_lb, *out_ub;         // [Mb, N] constant terms behind the relaxation (may be g.Dl, g.Du themselves)
+    float eps;
+};
+
+constexpr int EPI_PLAIN = 0, EPI_ROWNORM = 1, EPI_RELU = 2;
+
+template <bool EXACT, int MBM, int MBN, int NQ = -1, int EPI = EPI_PLAIN>
 __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *smem, const int m_blk, const int n_blk,
-                                                    float *pl = nullptr, float *pu = nullptr, float qv = 0.f) {
+                                                    float *pl = nullptr, float *pu = nullptr, float qv = 0.f,
+                                                    const void *epi = nullptr) {
     constexpr int BM = 64 * MBM, BN = 64 * MBN;
     constexpr int HALF_A = BM * 8, HALF_W = BN * 8;      // floats in one [rows x 8] half of an operand's K-step
     constexpr int S_AM = 0, S_AR = 2 * HALF_A, S_W = 4 * HALF_A, S_WA = 4 * HALF_A + 2 * HALF_W;
@@ -263,6 +289,165 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
                 cu[a][b][r] = 0.5f * (c + rd);
             }
     const size_t c_bytes = (size_t)min(M - m0, BM) * g.N * 4;
+    if constexpr (EPI == EPI_RELU) {
+#pragma clang fp contract(off)          // the lines are formed with the reference's separate roundings
+        static_assert(NQ >= 0, "the dual norm of the perturbation");
+        const ReluArgs *ra = static_cast<const ReluArgs *>(epi);
+        float nl[MBN], nu[MBN];
+#pragma unroll
+        for (int b = 0; b < MBN; ++b) {
+            nl[b] = nu[b] = 0.f;
+#pragma unroll
+            for (int a = 0; a < MBM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    nl[b] = nacc<NQ>(nl[b], cl[a][b][r], qv);
+                    nu[b] = nacc<NQ>(nu[b], cu[a][b][r], qv);
+                }
+            nl[b] = ncomb<NQ>(nl[b], __shfl_xor(nl[b], 32, 64));
+            nu[b] = ncomb<NQ>(nu[b], __shfl_xor(nu[b], 32, 64));
+        }
+        // the constant terms are read before the barrier and written behind it: out_lb may be g.Dl
+        float lb0[MBN], ub0[MBN];
+#pragma unroll
+        for (int b = 0; b < MBN; ++b) {
+            const int col = n0 + (wn * MBN + b) * 32 + fi;
+            const size_t o = (size_t)m_blk * g.N + min(col, g.N - 1);
+            lb0[b] = g.Dl[o];
+            ub0[b] = g.Du[o];
+        }
+        __syncthreads();                               // every wavefront has read its last fragments: LDS is free
+        float *red = smem;                             // [wm][l, u][BN columns]
+        if (fh == 0) {
+#pragma unroll
+            for (int b = 0; b < MBN; ++b) {
+                red[(wm * 2 + 0) * BN + (wn * MBN + b) * 32 + fi] = nl[b];
+                red[(wm * 2 + 1) * BN + (wn * MBN + b) * 32 + fi] = nu[b];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < MBN; ++b) {
+            const int cb = (wn * MBN + b) * 32 + fi, col = n0 + cb;
+            const float tl = ncomb<NQ>(red[(0 * 2 + 0) * BN + cb], red[(1 * 2 + 0) * BN + cb]);
+            const float tu = ncomb<NQ>(red[(0 * 2 + 1) * BN + cb], red[(1 * 2 + 1) * BN + cb]);
+            // l = lb + (-eps * norm), two roundings as Bounds.concretize has them (Bounds.py:313, 324)
+            const float l = __fadd_rn(lb0[b], __fmul_rn(-ra->eps, nfin<NQ>(tl, qv)));
+            const float u = __fadd_rn(ub0[b], __fmul_rn(ra->eps, nfin<NQ>(tu, qv)));
+            float klo, kup, olb, oub;
+            relax_point<RELU>(l, u, lb0[b], ub0[b], klo, kup, olb, oub);
+            if (wm == 0 && fh == 0 && col < g.N) {
+                const size_t o = (size_t)m_blk * g.N + col;
+                ra->out_lb[o] = olb;
+                ra->out_ub[o] = oub;
+            }
+#pragma unroll
+            for (int a = 0; a < MBM; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    cl[a][b][r] *= klo;                 // both slopes are >= 0: each side keeps its own coefficients
+                    cu[a][b][r] *= kup;
+                }
+        }
+    }
+    if constexpr (EPI == EPI_ROWNORM) {
+        const RowNormArgs *rn = static_cast<const RowNormArgs *>(epi);
+        static_assert(MBM == 1, "whole rows: one 32-row block per wavefront");
+        const unsigned row_b = (unsigned)g.N * 4u;
+        unsigned vo[MBN];
+#pragma unroll
+        for (int b = 0; b < MBN; ++b) vo[b] = (unsigned)(4 * fh) * row_b + (unsigned)((wn * MBN + b) * 32 + fi) * 4u;
+        auto row_off = [&](int r) { return (unsigned)(wm * 32 + 8 * (r / 4) + (r % 4)) * row_b; };
+        // ---- the added object: its rows for this tile (a tile lies inside one position: dim_in % 64 == 0)
+        if (rn->res_l) {
+            long long first = m0;
+            bool there = true;
+            if (rn->positions) {
+                const int q = m0 / rn->dim_in, bb = q / rn->length, pos = q % rn->length;
+                int slot = -1;
+                for (int i = 0; i < rn->words; ++i)
+                    if (rn->positions[bb * rn->words + i] == pos) slot = i;
+                there = slot >= 0;
+                first = ((long long)bb * rn->words + slot) * rn->dim_in + m0 % rn->dim_in;
+            }
+            if (there) {
+                const __amdgpu_buffer_rsrc_t wrl = window(rn->res_l + (size_t)first * g.N, c_bytes);
+                const __amdgpu_buffer_rsrc_t wru = window(rn->res_u + (size_t)first * g.N, c_bytes);
+#pragma unroll
+                for (int b = 0; b < MBN; ++b) {
+                    float tl[16], tu[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        tl[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wrl, vo[b], row_off(r), 0));
+                        tu[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wru, vo[b], row_off(r), 0));
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        cl[0][b][r] += tl[r];          // one fp32 add, as Bounds.add rounds it
+                        cu[0][b][r] += tu[r];
+                    }
+                }
+            }
+        }
+        // ---- row sums: the lane's MBN columns, the 32 lanes of its half, the two wavefronts that share the rows
+        float sl[16], su[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            sl[r] = cl[0][0][r];
+            su[r] = cu[0][0][r];
+#pragma unroll
+            for (int b = 1; b < MBN; ++b) {
+                sl[r] += cl[0][b][r];
+                su[r] += cu[0][b][r];
+            }
+        }
+#define FAITH_STEP(MSK)                                  \
+    _Pragma("unroll") for (int r = 0; r < 16; ++r) {    \
+        sl[r] += lane_xor<MSK>(sl[r]);                  \
+        su[r] += lane_xor<MSK>(su[r]);                  \
+    }
+        FAITH_STEP(1) FAITH_STEP(2) FAITH_STEP(4) FAITH_STEP(8) FAITH_STEP(16)
+#undef FAITH_STEP
+        __syncthreads();                               // every wavefront has read its last fragments: LDS is free
+        float *red = smem;                             // [wn][l, u][64 rows of the tile]
+        if (fi == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = wm * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+                red[(wn * 2 + 0) * 64 + row] = sl[r];
+                red[(wn * 2 + 1) * 64 + row] = su[r];
+            }
+        }
+        __syncthreads();
+        const float inv = 1.f / (float)g.N;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = wm * 32 + 8 * (r / 4) + 4 * fh + (r % 4);
+            sl[r] = (red[(0 * 2 + 0) * 64 + row] + red[(1 * 2 + 0) * 64 + row]) * inv;     // mean of the lower side
+            su[r] = (red[(0 * 2 + 1) * 64 + row] + red[(1 * 2 + 1) * 64 + row]) * inv;
+        }
+        // ---- centre on the other side's mean, scale by the weight split by sign, store
+        const __amdgpu_buffer_rsrc_t wol = window(rn->out_l + (size_t)m0 * g.N, c_bytes);
+        const __amdgpu_buffer_rsrc_t wou = window(rn->out_u + (size_t)m0 * g.N, c_bytes);
+#pragma unroll
+        for (int b = 0; b < MBN; ++b) {
+            float sp = 1.f, sn = 0.f;
+            if (rn->weight) {
+                const float wgt = rn->weight[(wn * MBN + b) * 32 + fi];
+                sp = wgt > 0.f ? wgt : 0.f * wgt;
+                sn = wgt - sp;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float c_lo = cl[0][b][r] - su[r], c_up = cu[0][b][r] - sl[r];
+                const float ol = rn->weight ? c_lo * sp + c_up * sn : c_lo;
+                const float ou = rn->weight ? c_lo * sn + c_up * sp : c_up;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(ol), wol, vo[b], row_off(r), 2);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(ou), wou, vo[b], row_off(r), 2);
+            }
+        }
+        return;
+    }
     const __amdgpu_buffer_rsrc_t wcl = window(g.Cl + (size_t)m0 * g.N, c_bytes);
     const __amdgpu_buffer_rsrc_t wcu = window(g.Cu + (size_t)m0 * g.N, c_bytes);
     const unsigned row_b = (unsigned)g.N * 4u;
@@ -280,7 +465,7 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
             }
         }
     }
-    if constexpr (NQ >= 0) {
+    if constexpr (NQ >= 0 && EPI == EPI_PLAIN) {
         // the lane's 16 MBM rows of each of its columns, in register order (a fixed order: the result does not
         // depend on scheduling)
 #pragma unroll
@@ -1230,4 +1415,189 @@ extern "C" int faith_matmul_concretize_verification(const float *x_lb, const flo
     FAITH_REQUIRE(rows <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_concretize_verification: batch*length exceeds 2^31");
     return faith_concretize(y_lb, y_ub, y_lw, y_uw, l, u, (int)rows, dim_in, dim_y_out, epsilon, q, words,
                             FAITH_LAYOUT_NATURAL, stream);
+}
+
+
+// ------------------------------------------------------------------------------------------------------------
+// Affine layer, residual connection and layer normalisation without the variance in one pass over the
+// coefficients: `dense(x).add(residual).layer_norm(...)` of every encoder sub-block (VerifierForward.py:166,
+// 181-189).  Apart, the layer writes its [rows * dim_in, N] result, and the normalisation reads it, reads the
+// residual and writes again: three passes over the largest object of the propagation for two adds and a
+// multiply per element.  Here a workgroup owns 64 whole rows of the result (64 x N tile, N = 128 or 256: wavefront
+// tile 32 x N / 2, the accumulator count of the 128 x 128 tile), so the row means are complete inside it.
+// The reduction runs in the order of the plain kernel: the sum in front of the normalisation has the bits it has
+// there, and the results differ from the separate launches by the order of the row sums only.
+namespace {
+
+template <bool EXACT, int MBN>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+signsplit_gemm_rownorm(const GemmArgs g, const RowNormArgs n) {
+    extern __shared__ __align__(16) float dyn_sm[];     // two stages of (2 x 64 + 2 x 64 MBN) rows x 16 floats
+    signsplit_gemm_tile<EXACT, 1, MBN, -1, EPI_ROWNORM>(g, dyn_sm, blockIdx.x, 0, nullptr, nullptr, 0.f, &n);
+}
+
+template <bool EXACT, int MBN>
+bool launch_rownorm(const GemmArgs &g, const RowNormArgs &n, hipStream_t st) {
+    const size_t lds = 2 * 4 * 64 * 8 * (1 + MBN) * sizeof(float);
+    if (!faith::reserve_lds(signsplit_gemm_rownorm<EXACT, MBN>, lds)) return false;
+    hipLaunchKernelGGL((signsplit_gemm_rownorm<EXACT, MBN>), dim3((unsigned)((g.Mw + 63) / 64)), dim3(NTHREADS), lds, st, g, n);
+    return true;
+}
+
+}  // namespace
+
+extern "C" int faith_matmul_layer_norm_fits(long long rows, int dim_in, int dim_out, int dim_y_out, int res_words) {
+    const bool taken = rows > 0 && dim_in > 0 && dim_out > 0 && dim_out % 4 == 0 && (dim_y_out == 128 || dim_y_out == 256) &&
+                       (res_words == 0 || dim_in % 64 == 0) && 64LL * dim_out * 4 < 0xffffffffLL &&
+                       rows * dim_in <= 0x7fffffffLL;
+    if (!taken) return 0;
+    // a 64-row tile runs through the whole reduction for all columns: with fewer than two of them per compute unit
+    // the separate launches, whose layer splits the columns over more workgroups, finish first (measured at
+    // N = 128 and 256, reductions of 128 .. 512: even at 512 tiles, 15 - 40 % faster at 1024, slower below)
+    return (rows * dim_in + 63) / 64 >= 2LL * faith::compute_units() ? 2 : 1;
+}
+
+extern "C" int faith_matmul_layer_norm_verification(const float *x_lb, const float *x_ub, const float *x_lw,
+                                                    const float *x_uw, const float *W, const float *bias,
+                                                    const float *res_lb, const float *res_ub, const float *res_lw,
+                                                    const float *res_uw, const long long *res_positions, int res_words,
+                                                    const float *weight, const float *norm_bias, float *y_lb, float *y_ub,
+                                                    float *y_lw, float *y_uw, int batch_size, int length, int dim_in,
+                                                    int dim_out, int dim_y_out, void *stream) {
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(W);
+    FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_ALIGNED4(x_lb); FAITH_ALIGNED4(x_ub); FAITH_ALIGNED4(bias); FAITH_ALIGNED4(y_lb); FAITH_ALIGNED4(y_ub);
+    FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw); FAITH_ALIGNED4(res_lb); FAITH_ALIGNED4(res_ub); FAITH_ALIGNED4(res_lw);
+    FAITH_ALIGNED4(res_uw); FAITH_ALIGNED4(weight); FAITH_ALIGNED4(norm_bias);
+    FAITH_REQUIRE(faith::aligned(res_positions, 8), FAITH_ERR_ALIGN, "faith_matmul_layer_norm_verification: res_positions is not 8-byte aligned");
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && dim_in > 0 && dim_out > 0 && dim_y_out > 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_layer_norm_verification: batch=%d length=%d dim_in=%d dim_out=%d dim_y_out=%d must be "
+                  "positive", batch_size, length, dim_in, dim_out, dim_y_out);
+    const bool adding = res_lb || res_ub || res_lw || res_uw;
+    FAITH_REQUIRE(!adding || (res_lb && res_ub && res_lw && res_uw), FAITH_ERR_NULL,
+                  "faith_matmul_layer_norm_verification: the four tensors of the added object must be given together");
+    FAITH_REQUIRE(res_words >= 0 && (res_words == 0) == (res_positions == nullptr) && (res_words == 0 || adding),
+                  FAITH_ERR_SHAPE, "faith_matmul_layer_norm_verification: res_words=%d and res_positions must be given "
+                  "together, with an added object", res_words);
+    FAITH_REQUIRE(faith_matmul_layer_norm_fits((long long)batch_size * length, dim_in, dim_out, dim_y_out, res_words) &&
+                  faith::aligned(x_lw, 16) &&
+                  faith::aligned(x_uw, 16) && faith::aligned(W, 16), FAITH_ERR_UNSUPPORTED,
+                  "faith_matmul_layer_norm_verification: dim_y_out=%d must be 128 or 256, dim_out=%d a multiple of 4, "
+                  "dim_in=%d a multiple of 64 when the added object holds some positions only, batch*length*dim_in below "
+                  "2^31, and x_lw, x_uw, W 16-byte aligned", dim_y_out, dim_out, dim_in);
+    const long long rows = (long long)batch_size * length, mw = rows * dim_in;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
+    const RowNormArgs n{res_lw, res_uw, res_positions, res_words, length, dim_in, weight, y_lw, y_uw};
+    const bool exact = dim_out % BK == 0;
+    bool ok;
+    if (dim_y_out == 256) ok = exact ? launch_rownorm<true, 4>(g, n, st) : launch_rownorm<false, 4>(g, n, st);
+    else ok = exact ? launch_rownorm<true, 2>(g, n, st) : launch_rownorm<false, 2>(g, n, st);
+    FAITH_REQUIRE(ok, FAITH_ERR_UNSUPPORTED, "faith_matmul_layer_norm_verification: the device refused the LDS size");
+    // constant terms: exact accumulation, then the same normalisation on [rows, dim_y_out] in place (a row is
+    // held in registers between its read and its write)
+    GemmArgs gb = g;
+    gb.Mw = 0;
+    const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
+    FAITH_REQUIRE(gridb <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_layer_norm_verification: grid too large");
+    hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+    const int rc = faith::check_launch("faith_matmul_layer_norm_verification");
+    if (rc != FAITH_OK) return rc;
+    return faith_layer_norm_verification(y_lb, y_ub, y_lw, y_uw, res_lb, res_ub, adding ? res_lw : nullptr,
+                                         adding ? res_uw : nullptr, weight, norm_bias, y_lb, y_ub, y_lw, y_uw, 0, rows,
+                                         dim_y_out, stream);
+}
+
+
+// ------------------------------------------------------------------------------------------------------------
+// Affine layer and ReLU relaxation in one pass over the coefficients: `dense(x).relu()` of the feed-forward
+// block (VerifierForward.py:171-179 with hidden_act "relu").  Apart, the layer writes its [rows * dim_in, N]
+// result and the relaxation reads it, finds each neuron's concrete interval from the column norms over the
+// dim_in rows of its position, scales and writes again.  Here a tile holds all dim_in rows of one position
+// (dim_in = 128: the 128 x 128 tile; 256: 256 x 64, wavefront tile 128 x 32, the same accumulator count), so the
+// norms, the interval and the two slopes are known before the tile is stored.  One perturbed word.
+namespace {
+
+template <bool EXACT, int MBM, int MBN, int Q>
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+signsplit_gemm_relu(const GemmArgs g, const ReluArgs r, const float qv) {
+    extern __shared__ __align__(16) float dyn_sm[];
+    constexpr int BN = 64 * MBN;
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int xcd = blockIdx.x % XCDS, local = blockIdx.x / XCDS;
+    const int pos = (local / tiles_n) * XCDS + xcd;          // the column blocks of a position meet in one L2
+    if (pos >= g.Mb) return;
+    signsplit_gemm_tile<EXACT, MBM, MBN, Q, EPI_RELU>(g, dyn_sm, pos, local % tiles_n, nullptr, nullptr, qv, &r);
+}
+
+template <bool EXACT, int MBM, int MBN>
+const void *relu_kernel(int q) {
+    switch (q) {
+        case FAITH_Q_1: return reinterpret_cast<const void *>(signsplit_gemm_relu<EXACT, MBM, MBN, FAITH_Q_1>);
+        case FAITH_Q_2: return reinterpret_cast<const void *>(signsplit_gemm_relu<EXACT, MBM, MBN, FAITH_Q_2>);
+        case FAITH_Q_INF: return reinterpret_cast<const void *>(signsplit_gemm_relu<EXACT, MBM, MBN, FAITH_Q_INF>);
+        default: return reinterpret_cast<const void *>(signsplit_gemm_relu<EXACT, MBM, MBN, Q_GENERAL>);
+    }
+}
+
+}  // namespace
+
+extern "C" int faith_matmul_relu_fits(long long rows, int dim_in, int dim_out, int dim_y_out, int words) {
+    const bool taken = rows > 0 && rows <= 0x7fffffffLL / 256 && (dim_in == 128 || dim_in == 256) && dim_out > 0 &&
+                       dim_out % 4 == 0 && dim_y_out > 0 && words == 1 && 256LL * dim_out * 4 < 0xffffffffLL &&
+                       256LL * dim_y_out * 4 < 0x80000000LL;
+    if (!taken) return 0;
+    // one tile per position and block of columns: as the 128 x 128 tiles of the plain layer, they pay once they fill
+    // the device about twice over
+    const long long tiles = rows * ((dim_y_out + (dim_in == 128 ? 127 : 63)) / (dim_in == 128 ? 128 : 64));
+    return tiles >= 2LL * faith::compute_units() ? 2 : 1;
+}
+
+extern "C" int faith_matmul_relu_verification(const float *x_lb, const float *x_ub, const float *x_lw, const float *x_uw,
+                                              const float *W, const float *bias, float *y_lb, float *y_ub, float *y_lw,
+                                              float *y_uw, int batch_size, int length, int dim_in, int dim_out,
+                                              int dim_y_out, float epsilon, int q, int words, void *stream) {
+    FAITH_NOT_NULL(x_lb); FAITH_NOT_NULL(x_ub); FAITH_NOT_NULL(x_lw); FAITH_NOT_NULL(x_uw); FAITH_NOT_NULL(W);
+    FAITH_NOT_NULL(y_lb); FAITH_NOT_NULL(y_ub); FAITH_NOT_NULL(y_lw); FAITH_NOT_NULL(y_uw);
+    FAITH_ALIGNED4(x_lb); FAITH_ALIGNED4(x_ub); FAITH_ALIGNED4(bias); FAITH_ALIGNED4(y_lb); FAITH_ALIGNED4(y_ub);
+    FAITH_ALIGNED4(y_lw); FAITH_ALIGNED4(y_uw);
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && dim_in > 0 && dim_out > 0 && dim_y_out > 0, FAITH_ERR_SHAPE,
+                  "faith_matmul_relu_verification: batch=%d length=%d dim_in=%d dim_out=%d dim_y_out=%d must be positive",
+                  batch_size, length, dim_in, dim_out, dim_y_out);
+    float qv = 0.f;
+    if (!faith::dual_exponent(q, &qv)) {
+        faith::set_error("faith_matmul_relu_verification: q=%d is neither FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF nor the bits "
+                         "of an exponent in (1, inf)", q);
+        return FAITH_ERR_UNSUPPORTED;
+    }
+    const long long rows = (long long)batch_size * length;
+    FAITH_REQUIRE(faith_matmul_relu_fits(rows, dim_in, dim_out, dim_y_out, words) && faith::aligned(x_lw, 16) &&
+                  faith::aligned(x_uw, 16) && faith::aligned(W, 16), FAITH_ERR_UNSUPPORTED,
+                  "faith_matmul_relu_verification: dim_in=%d must be 128 or 256, words=%d one, dim_out=%d a multiple of 4, "
+                  "and x_lw, x_uw, W 16-byte aligned", dim_in, words, dim_out);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)(rows * dim_in), (int)rows, dim_y_out, dim_out};
+    const bool exact = dim_out % BK == 0, wide = dim_in == 128;      // 128 x 128 tiles, or 256 x 64
+    const void *kernel = wide ? (exact ? relu_kernel<true, 2, 2>(q) : relu_kernel<false, 2, 2>(q))
+                              : (exact ? relu_kernel<true, 4, 1>(q) : relu_kernel<false, 4, 1>(q));
+    const size_t lds = 2 * 4 * 64 * 8 * (wide ? 4 : 5) * sizeof(float);
+    const long long tiles_n = (dim_y_out + (wide ? 127 : 63)) / (wide ? 128 : 64);
+    const long long grid = ((rows + XCDS - 1) / XCDS) * XCDS * tiles_n;
+    const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
+    FAITH_REQUIRE(gridb <= 0x7fffffffLL && grid <= 0x7fffffffLL, FAITH_ERR_SHAPE,
+                  "faith_matmul_relu_verification: grid too large");
+    FAITH_REQUIRE(lds <= 64 * 1024 || hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess,
+                  FAITH_ERR_UNSUPPORTED, "faith_matmul_relu_verification: the device refused the LDS size");
+    // the constant terms of the layer first: the coefficient kernel reads them when it forms the intervals, and
+    // writes the constant terms of the relaxed object over them
+    GemmArgs gb = g;
+    gb.Mw = 0;
+    hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+    ReluArgs r{y_lb, y_ub, epsilon};
+    void *args[] = {&g, &r, &qv};
+    if (hipLaunchKernel(kernel, dim3((unsigned)grid), dim3(NTHREADS), args, lds, st) != hipSuccess) {
+        faith::set_error("faith_matmul_relu_verification: launch failed: %s", hipGetErrorString(hipGetLastError()));
+        return FAITH_ERR_LAUNCH;
+    }
+    return faith::check_launch("faith_matmul_relu_verification");
 }

@@ -1,7 +1,8 @@
 // The per-neuron lines of the relaxations (slopes and constant terms from a concrete interval), shared by
 // the relaxation kernels and the fused softmax.  fp32 operation order follows the reference line by line
-// (Transformer_Verification_Code/Verifiers/Bounds.py:348-381 add_linear, :860-1003, :1136-1161); translation
-// units that include this are built with -ffp-contract=off.
+// (Transformer_Verification_Code/Verifiers/Bounds.py:348-381 add_linear, :860-1003, :1136-1161): the functions
+// here switch the contraction of a multiply and an add into one fused operation off for their own bodies, whatever
+// the translation unit that includes them is built with.
 #pragma once
 #include "relax_common.h"
 
@@ -18,6 +19,7 @@ struct Line {
 // ------------------------------------------------------------------ the relaxations
 // Bounds.py:921-963.  Strict comparisons: l == 0 or u == 0 is a straddling neuron.
 __device__ __forceinline__ void relu_lines(float l, float u, Line &lo, Line &up) {
+#pragma clang fp contract(off)
     if (u < 0.f) {
         lo = {0.f, 0.f, 0.f};
         up = {0.f, 0.f, 0.f};
@@ -39,6 +41,7 @@ __device__ __forceinline__ double exp_capped(float x) {
 // Bounds.add_linear, constant term (Bounds.py:378, :381): a positive slope takes the same-side
 // bound, a non-positive one the opposite bound; three separate roundings.
 __device__ __forceinline__ float line_bias(const Line &ln, float same, float other) {
+#pragma clang fp contract(off)
     const float b = ln.k > 0.f ? same : other;
     return (b - ln.x0) * ln.k + ln.y0;
 }
@@ -49,6 +52,7 @@ __device__ __forceinline__ float line_bias(const Line &ln, float same, float oth
 template <int MODE>
 __device__ __forceinline__ void relax_point(float l, float u, float lb, float ub, float &klo, float &kup, float &olb,
                                             float &oub) {
+#pragma clang fp contract(off)
     if (MODE == EXP) {                       // Bounds.py:970-1003
         const float m = fminf((l + u) / 2, l + 0.99f);
         klo = (float)exp((double)fminf(m, 12.f));

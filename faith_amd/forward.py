@@ -185,14 +185,24 @@ def _add_norm(x, residual, normalizer, layer_norm):
     return x.add(residual).layer_norm(normalizer, layer_norm)
 
 
+def _dense_add_norm(x, dense, residual, normalizer, layer_norm):
+    """x.dense(dense).add(residual).layer_norm(...); one pass where the bound object has the operator for it."""
+    if hasattr(x, "dense_layer_norm"):
+        return x.dense_layer_norm(dense, normalizer, layer_norm, residual=residual)
+    return _add_norm(x.dense(dense), residual, normalizer, layer_norm)
+
+
 def bound_layer(bounds_input, layer, layer_norm="no_var", hidden_act="relu", want_scores=False):
     """VerifierForward._bound_layer: attention block, residual + norm, feed-forward, residual + norm.
     Returns (scores, probs, output); scores is None unless asked for (see bound_attention)."""
     scores, probs, attention = bound_attention(bounds_input, layer.attention, want_scores)
-    attention = attention.dense(layer.attention.output.dense)
-    attention = _add_norm(attention, bounds_input, layer.attention.output.LayerNorm, layer_norm)
-    intermediate = attention.dense(layer.intermediate.dense).act(hidden_act)
-    output = _add_norm(intermediate.dense(layer.output.dense), attention, layer.output.LayerNorm, layer_norm)
+    attention = _dense_add_norm(attention, layer.attention.output.dense, bounds_input, layer.attention.output.LayerNorm,
+                                layer_norm)
+    if hasattr(attention, "dense_act"):
+        intermediate = attention.dense_act(layer.intermediate.dense, hidden_act)
+    else:
+        intermediate = attention.dense(layer.intermediate.dense).act(hidden_act)
+    output = _dense_add_norm(intermediate, layer.output.dense, attention, layer.output.LayerNorm, layer_norm)
     return scores, probs, output
 
 

@@ -486,6 +486,84 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
     return olw, olb, ouw, oub
 
 
+def linear_relu_fits(rows, D, H, N, words=1):
+    """Whether linear_relu takes a layer [N, H] on objects of `rows` = batch * length positions with dim_in D:
+    0 no, 1 yes but the separate launches are faster, 2 yes and it is the faster choice."""
+    return int(_lib.lib.faith_matmul_relu_fits(rows, D, H, N, words))
+
+
+def linear_relu(lw, lb, uw, ub, weight, bias, p, eps, words=1):
+    """relu(linear(x)) in one pass over the coefficients (`dense(x).relu()`); returns (lw', lb', uw', ub').
+    Raises FaithError (ERR_UNSUPPORTED) for shapes linear_relu_fits refuses."""
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    _check("weight", weight)
+    if weight.dim() != 2 or weight.shape[1] != H:
+        raise ValueError(f"weight must be [H_out, {H}], got {tuple(weight.shape)}")
+    N = weight.shape[0]
+    if bias is not None:
+        _check("bias", bias, (N,))
+    olw = _empty(B, L, D, N, device=lw.device)
+    ouw = _empty_like(olw)
+    olb = _empty(B, L, N, device=lw.device)
+    oub = _empty_like(olb)
+    with _on(lw.device):
+        _lib.call("faith_matmul_relu_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
+                  _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), B, L, D, H, N, float(eps), q_code(p), int(words), _stream(lw))
+    return olw, olb, ouw, oub
+
+
+def linear_layer_norm_fits(rows, D, H, N, res_words=0):
+    """Whether linear_layer_norm takes a layer [N, H] on objects of `rows` = batch * length positions with dim_in D
+    (res_words > 0: the added object holds that many positions per batch element only): 0 no, 1 yes but the
+    separate launches are faster (too few tiles to fill the device), 2 yes and it is the faster choice."""
+    return int(_lib.lib.faith_matmul_layer_norm_fits(rows, D, H, N, res_words))
+
+
+def linear_layer_norm(lw, lb, uw, ub, weight, bias, norm_weight=None, norm_bias=None, other=None, positions=None):
+    """layer_norm(linear(x) + other) without the variance, one pass over the coefficients
+    (`dense(x).add(other).layer_norm(normalizer, "no_var")`).  other: (lw, lb, uw, ub) of the added object; with
+    `positions` (int64 [B, P] on the device) its coefficients are [B, P, D, N], the rows of those positions only.
+    Raises FaithError (ERR_UNSUPPORTED) for shapes linear_layer_norm_fits refuses."""
+    B, L, D, H = _wb_shapes(lw, lb, LAYOUT_NATURAL)
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    _check("weight", weight)
+    if weight.dim() != 2 or weight.shape[1] != H:
+        raise ValueError(f"weight must be [H_out, {H}], got {tuple(weight.shape)}")
+    N = weight.shape[0]
+    if bias is not None:
+        _check("bias", bias, (N,))
+    if norm_weight is not None:
+        _check("norm_weight", norm_weight, (N,))
+    if norm_bias is not None:
+        _check("norm_bias", norm_bias, (N,))
+    words = 0
+    if other is not None:
+        alw, alb, auw, aub = other
+        if positions is not None:
+            if positions.dtype != torch.int64 or not positions.is_cuda or not positions.is_contiguous() or \
+                    positions.dim() != 2 or positions.shape[0] != B:
+                raise ValueError(f"positions must be a contiguous int64 [{B}, P] tensor on the device")
+            words = positions.shape[1]
+            _check("other.lw", alw, (B, words, D, N)); _check("other.uw", auw, (B, words, D, N))
+        else:
+            _check("other.lw", alw, (B, L, D, N)); _check("other.uw", auw, (B, L, D, N))
+        _check("other.lb", alb, (B, L, N)); _check("other.ub", aub, (B, L, N))
+    else:
+        if positions is not None:
+            raise ValueError("positions without an added object")
+        alw = alb = auw = aub = None
+    olw = _empty(B, L, D, N, device=lw.device)
+    ouw = _empty_like(olw)
+    olb = _empty(B, L, N, device=lw.device)
+    oub = _empty_like(olb)
+    with _on(lw.device):
+        _lib.call("faith_matmul_layer_norm_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
+                  _ptr(alb), _ptr(aub), _ptr(alw), _ptr(auw), _ptr(positions), words, _ptr(norm_weight), _ptr(norm_bias),
+                  _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), B, L, D, H, N, _stream(lw))
+    return olw, olb, ouw, oub
+
+
 def linear_concretize(lw, lb, uw, ub, weight, bias, p, eps, words=1, out=None):
     """linear() and concretize() of its result through one entry point (one launch for small problems).
     Returns (lw', lb', uw', ub', l, u).  `out`: the six result tensors, owned by the caller as in the

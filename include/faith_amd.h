@@ -262,6 +262,53 @@ int faith_matmul_verification(const float *x_lb, const float *x_ub,
                               void *stream);
 
 /*
+ * Affine layer, residual connection and layer normalisation without the variance in one pass over the
+ * coefficients: y = layer_norm(x @ W^T (+ bias) + res), i.e. `dense(x).add(res).layer_norm(normalizer, "no_var")`
+ * of every encoder sub-block (VerifierForward.py:166, 181-189; Bounds.py:1016-1025, :397-413, :1111-1131).  The
+ * reference has no fused counterpart.  x_* and y_* as faith_matmul_verification; res_lb, res_ub
+ * [batch*length, dim_y_out]; res_lw, res_uw [batch*length*dim_in, dim_y_out] when res_positions is NULL (res_words 0),
+ * else [batch, res_words, dim_in, dim_y_out]: the dim_in rows of the positions res_positions[batch, res_words]
+ * (int64, as the compact attention entry points take them), every other row of the added object being zero (a position outside 0 .. length-1 names no row);
+ * all four res_* NULL: no residual.  weight, norm_bias [dim_y_out] or NULL as faith_layer_norm_verification.
+ * Shapes: dim_y_out 128 or 256, dim_out % 4 == 0, x_lw / x_uw / W 16-byte aligned, dim_in % 64 == 0 when
+ * res_positions is given; faith_matmul_layer_norm_fits (rows = batch*length) answers 0 where the shape is not taken --
+ * the entry point then returns FAITH_ERR_UNSUPPORTED with nothing written, and the caller runs
+ * faith_matmul_verification and faith_layer_norm_verification --, 1 where it is taken but those two launches are
+ * the faster choice (fewer than two 64-row tiles per compute unit), 2 where this entry point is.  The sum in front of the normalisation has the bits the separate launches
+ * give it; the results differ from theirs by the order in which a row's mean is summed.  y_* must not overlap res_*.
+ */
+int faith_matmul_layer_norm_fits(long long rows, int dim_in, int dim_out, int dim_y_out, int res_words);
+int faith_matmul_layer_norm_verification(const float *x_lb, const float *x_ub,
+                                         const float *x_lw, const float *x_uw,
+                                         const float *W, const float *bias,
+                                         const float *res_lb, const float *res_ub,
+                                         const float *res_lw, const float *res_uw,
+                                         const long long *res_positions, int res_words,
+                                         const float *weight, const float *norm_bias,
+                                         float *y_lb, float *y_ub, float *y_lw, float *y_uw,
+                                         int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
+                                         void *stream);
+
+/*
+ * Affine layer and ReLU relaxation in one pass over the coefficients: y = relu(x @ W^T (+ bias)), i.e.
+ * `dense(x).relu()` of the feed-forward block (VerifierForward.py:171-179; Bounds.py:1016-1025, :921-963).  The
+ * reference has no fused counterpart.  Arguments as faith_matmul_verification, plus epsilon, q, words as
+ * faith_relu_verification.  Shapes: dim_in 128 or 256 (a tile holds every coefficient row of a position), words 1,
+ * dim_out % 4 == 0, x_lw / x_uw / W 16-byte aligned; faith_matmul_relu_fits (rows = batch*length) answers 0 / 1 / 2
+ * as faith_matmul_layer_norm_fits does, and the entry point returns FAITH_ERR_UNSUPPORTED with nothing written
+ * where the answer is 0.  The layer's result has the bits faith_matmul_verification gives it; each neuron's
+ * interval is formed from column norms summed in the tile's order, so it may differ from faith_relu_verification's
+ * in the last bit, and the slopes with it.
+ */
+int faith_matmul_relu_fits(long long rows, int dim_in, int dim_out, int dim_y_out, int words);
+int faith_matmul_relu_verification(const float *x_lb, const float *x_ub,
+                                   const float *x_lw, const float *x_uw,
+                                   const float *W, const float *bias,
+                                   float *y_lb, float *y_ub, float *y_lw, float *y_uw,
+                                   int batch_size, int length, int dim_in, int dim_out, int dim_y_out,
+                                   float epsilon, int q, int words, void *stream);
+
+/*
  * Affine layer followed by the concretization of its result: y = x @ W^T (+ bias), then
  * [l, u] of y.  Replaces Bounds.dense(...).concretize() (Bounds.py:1016-1025, :311-326) as the
  * classifier at the end of the verifier uses it (VerifierForward.py:300-314); the reference has
