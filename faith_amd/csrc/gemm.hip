@@ -128,10 +128,12 @@ struct ReluArgs {
 
 constexpr int EPI_PLAIN = 0, EPI_ROWNORM = 1, EPI_RELU = 2;
 
-template <bool EXACT, int MBM, int MBN, int NQ = -1, int EPI = EPI_PLAIN>
+struct NoEpilogueArgs {};
+
+template <bool EXACT, int MBM, int MBN, int NQ = -1, int EPI = EPI_PLAIN, class EpiArgs = NoEpilogueArgs>
 __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *smem, const int m_blk, const int n_blk,
                                                     float *pl = nullptr, float *pu = nullptr, float qv = 0.f,
-                                                    const void *epi = nullptr) {
+                                                    const EpiArgs &epi = EpiArgs()) {
     constexpr int BM = 64 * MBM, BN = 64 * MBN;
     constexpr int HALF_A = BM * 8, HALF_W = BN * 8;      // floats in one [rows x 8] half of an operand's K-step
     constexpr int S_AM = 0, S_AR = 2 * HALF_A, S_W = 4 * HALF_A, S_WA = 4 * HALF_A + 2 * HALF_W;
@@ -292,7 +294,7 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
     if constexpr (EPI == EPI_RELU) {
 #pragma clang fp contract(off)          // the lines are formed with the reference's separate roundings
         static_assert(NQ >= 0, "the dual norm of the perturbation");
-        const ReluArgs *ra = static_cast<const ReluArgs *>(epi);
+        const ReluArgs *ra = &epi;
         float nl[MBN], nu[MBN];
 #pragma unroll
         for (int b = 0; b < MBN; ++b) {
@@ -334,8 +336,21 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
             // l = lb + (-eps * norm), two roundings as Bounds.concretize has them (Bounds.py:313, 324)
             const float l = __fadd_rn(lb0[b], __fmul_rn(-ra->eps, nfin<NQ>(tl, qv)));
             const float u = __fadd_rn(ub0[b], __fmul_rn(ra->eps, nfin<NQ>(tu, qv)));
-            float klo, kup, olb, oub;
-            relax_point<RELU>(l, u, lb0[b], ub0[b], klo, kup, olb, oub);
+            // the two lines of Bounds.relu (Bounds.py:921-963) and their constant terms as Bounds.add_linear forms
+            // them (Bounds.py:378, :381: (b - x0) * k + y0, b the same-side constant for a positive slope) --
+            // relax_point<RELU> of the relaxation kernels written out on scalars, so that nothing goes through memory
+            float klo, kup, x0up = 0.f;
+            if (u < 0.f) {
+                klo = kup = 0.f;
+            } else if (l > 0.f) {
+                klo = kup = 1.f;
+            } else {
+                kup = u / ((u - l) + TINY);
+                x0up = l;
+                klo = fabsf(u) > fabsf(l) ? 1.f : 0.f;
+            }
+            const float olb = ((klo > 0.f ? lb0[b] : ub0[b]) - 0.f) * klo + 0.f;
+            const float oub = ((kup > 0.f ? ub0[b] : lb0[b]) - x0up) * kup + 0.f;
             if (wm == 0 && fh == 0 && col < g.N) {
                 const size_t o = (size_t)m_blk * g.N + col;
                 ra->out_lb[o] = olb;
@@ -351,7 +366,7 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
         }
     }
     if constexpr (EPI == EPI_ROWNORM) {
-        const RowNormArgs *rn = static_cast<const RowNormArgs *>(epi);
+        const RowNormArgs *rn = &epi;
         static_assert(MBM == 1, "whole rows: one 32-row block per wavefront");
         const unsigned row_b = (unsigned)g.N * 4u;
         unsigned vo[MBN];
@@ -367,6 +382,7 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
                 int slot = -1;
                 for (int i = 0; i < rn->words; ++i)
                     if (rn->positions[bb * rn->words + i] == pos) slot = i;
+                slot = __builtin_amdgcn_readfirstlane(slot);     // the same in every lane: keeps the descriptors in scalar registers
                 there = slot >= 0;
                 first = ((long long)bb * rn->words + slot) * rn->dim_in + m0 % rn->dim_in;
             }
@@ -442,8 +458,9 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
                 const float c_lo = cl[0][b][r] - su[r], c_up = cu[0][b][r] - sl[r];
                 const float ol = rn->weight ? c_lo * sp + c_up * sn : c_lo;
                 const float ou = rn->weight ? c_lo * sn + c_up * sp : c_up;
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(ol), wol, vo[b], row_off(r), 2);
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(ou), wou, vo[b], row_off(r), 2);
+                const unsigned so = __builtin_amdgcn_readfirstlane(row_off(r));      // a scalar operand, stated as one
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(ol), wol, vo[b], so, 2);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(ou), wou, vo[b], so, 2);
             }
         }
         return;
@@ -593,6 +610,19 @@ __global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
     __shared__ float sm[3 * 16 * 17];
     const int tiles_n = (g.N + 15) / 16;
     simple_tile(g, blockIdx.x / tiles_n, blockIdx.x % tiles_n, sm);
+}
+
+// Launches the exact-accumulation kernel for the constant-term rows of g (its coefficient rows are left alone).
+// (The 8 x 8 tiles with the split reduction, which the small problems take inside their MFMA launch, measured
+// 40 - 170 us slower here at 960 rows x 256 .. 512 columns: four times the workgroups re-read W.)
+// False if the grid would be too large.
+static bool launch_constant_rows(const GemmArgs &g, hipStream_t st) {
+    GemmArgs gb = g;
+    gb.Mw = 0;
+    const long long gridb = ((long long)(g.Mb + 15) / 16) * ((g.N + 15) / 16);
+    if (gridb > 0x7fffffffLL) return false;
+    hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+    return true;
 }
 
 template <bool EXACT>
@@ -822,9 +852,7 @@ static int matmul_rows(const float *x_lb, const float *x_ub, const float *x_lw, 
                 hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
             else
                 hipLaunchKernelGGL(signsplit_gemm<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
-            GemmArgs gb = g;
-            gb.Mw = 0;
-            hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+            FAITH_REQUIRE(launch_constant_rows(g, st), FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
         } else {
             // constant-term tiles in front, rounded up to a multiple of 8 so that the MFMA tiles keep
             // their XCD (workgroup number mod 8)
@@ -1397,11 +1425,7 @@ extern "C" int faith_matmul_concretize_verification(const float *x_lb, const flo
             hipStream_t st = static_cast<hipStream_t>(stream);
             GemmArgs g{x_lw, x_uw, x_lb, x_ub, W, bias, y_lw, y_uw, y_lb, y_ub, (int)mw, (int)rows, dim_y_out, dim_out};
             // the constant terms first: the coefficient kernel reads them when it writes l and u
-            GemmArgs gb = g;
-            gb.Mw = 0;
-            const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
-            FAITH_REQUIRE(gridb <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_concretize_verification: grid too large");
-            hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+            FAITH_REQUIRE(launch_constant_rows(g, st), FAITH_ERR_SHAPE, "faith_matmul_concretize_verification: grid too large");
             const NormArgs na{l, u, dim_in, epsilon, f.qv};
             if (tm == 128 && tn == 128) launch_norms<2, 2>(g, na, q, st);
             else if (tm == 128) launch_norms<2, 1>(g, na, q, st);
@@ -1433,7 +1457,7 @@ template <bool EXACT, int MBN>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 signsplit_gemm_rownorm(const GemmArgs g, const RowNormArgs n) {
     extern __shared__ __align__(16) float dyn_sm[];     // two stages of (2 x 64 + 2 x 64 MBN) rows x 16 floats
-    signsplit_gemm_tile<EXACT, 1, MBN, -1, EPI_ROWNORM>(g, dyn_sm, blockIdx.x, 0, nullptr, nullptr, 0.f, &n);
+    signsplit_gemm_tile<EXACT, 1, MBN, -1, EPI_ROWNORM, RowNormArgs>(g, dyn_sm, blockIdx.x, 0, nullptr, nullptr, 0.f, n);
 }
 
 template <bool EXACT, int MBN>
@@ -1496,11 +1520,7 @@ extern "C" int faith_matmul_layer_norm_verification(const float *x_lb, const flo
     FAITH_REQUIRE(ok, FAITH_ERR_UNSUPPORTED, "faith_matmul_layer_norm_verification: the device refused the LDS size");
     // constant terms: exact accumulation, then the same normalisation on [rows, dim_y_out] in place (a row is
     // held in registers between its read and its write)
-    GemmArgs gb = g;
-    gb.Mw = 0;
-    const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
-    FAITH_REQUIRE(gridb <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_layer_norm_verification: grid too large");
-    hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+    FAITH_REQUIRE(launch_constant_rows(g, st), FAITH_ERR_SHAPE, "faith_matmul_layer_norm_verification: grid too large");
     const int rc = faith::check_launch("faith_matmul_layer_norm_verification");
     if (rc != FAITH_OK) return rc;
     return faith_layer_norm_verification(y_lb, y_ub, y_lw, y_uw, res_lb, res_ub, adding ? res_lw : nullptr,
@@ -1527,7 +1547,7 @@ signsplit_gemm_relu(const GemmArgs g, const ReluArgs r, const float qv) {
     const int xcd = blockIdx.x % XCDS, local = blockIdx.x / XCDS;
     const int pos = (local / tiles_n) * XCDS + xcd;          // the column blocks of a position meet in one L2
     if (pos >= g.Mb) return;
-    signsplit_gemm_tile<EXACT, MBM, MBN, Q, EPI_RELU>(g, dyn_sm, pos, local % tiles_n, nullptr, nullptr, qv, &r);
+    signsplit_gemm_tile<EXACT, MBM, MBN, Q, EPI_RELU, ReluArgs>(g, dyn_sm, pos, local % tiles_n, nullptr, nullptr, qv, r);
 }
 
 template <bool EXACT, int MBM, int MBN>
@@ -1590,9 +1610,7 @@ extern "C" int faith_matmul_relu_verification(const float *x_lb, const float *x_
                   FAITH_ERR_UNSUPPORTED, "faith_matmul_relu_verification: the device refused the LDS size");
     // the constant terms of the layer first: the coefficient kernel reads them when it forms the intervals, and
     // writes the constant terms of the relaxed object over them
-    GemmArgs gb = g;
-    gb.Mw = 0;
-    hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
+    launch_constant_rows(g, st);
     ReluArgs r{y_lb, y_ub, epsilon};
     void *args[] = {&g, &r, &qv};
     if (hipLaunchKernel(kernel, dim3((unsigned)grid), dim3(NTHREADS), args, lds, st) != hipSuccess) {
