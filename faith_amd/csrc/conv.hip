@@ -456,14 +456,21 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     const size_t w_bytes = (size_t)(g.Co - co0) * g.Ci * KK * 4;
 
     // ---- staging plan, fixed for the whole reduction: byte offsets inside a chunk of channels
-    unsigned poff[NP];
-#pragma unroll
-    for (int u = 0; u < NP; ++u) {
-        const int e = tid + u * NTHREADS;
+    // (a 5 x 5 layer has no registers to spare for the plan beside its weight slab, nor has a stride-2 layer with
+    // 64-channel tiles, whose patch is 18 elements per thread: they work each offset out again where it is used,
+    // a dozen integer operations per element against hundreds of MFMAs per chunk)
+    constexpr bool KEEP_PLAN = K < 5 && NP <= 12;
+    auto patch_offset = [&](int u, int tid_) -> unsigned {
+        const int e = tid_ + u * NTHREADS;
         const int ci = e / PP, r2 = e % PP, pr = r2 / PCOL, pc = r2 % PCOL;
         const int ih = ih0 + pr, iw = iw0 + pc;
         const bool ok = e < CCH * PP && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
-        poff[u] = ok ? (unsigned)(ci * img + ih * g.W + iw) * 4u : NOWHERE;
+        return ok ? (unsigned)(ci * img + ih * g.W + iw) * 4u : NOWHERE;
+    };
+    unsigned poff[KEEP_PLAN ? NP : 1];
+    if constexpr (KEEP_PLAN) {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) poff[u] = patch_offset(u, tid);
     }
     // weight load u of a thread: element e = tid + u * NTHREADS of the slab, row e / (WROW / WPT); its source and
     // destination are a few integer operations on compile-time divisors, recomputed where they are used so
@@ -491,10 +498,13 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     auto fetch_patch = [&](int c0) {
         const __amdgpu_buffer_rsrc_t rl = window(xl_n, image * 4), ru = window(xu_n, image * 4);
         const unsigned cx = (unsigned)c0 * img * 4u;
+        int tid_ = tid;
+        if constexpr (!KEEP_PLAN) asm volatile("" : "+v"(tid_));     // opaque: the offsets are not hoisted out of the loop
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
-            pxl[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, poff[u], cx, 0));
-            pxu[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ru, poff[u], cx, 0));
+            const unsigned off = KEEP_PLAN ? poff[KEEP_PLAN ? u : 0] : patch_offset(u, tid_);
+            pxl[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rl, off, cx, 0));
+            pxu[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ru, off, cx, 0));
         }
     };
     auto fetch_weights = [&](int c0, auto first, auto count) {

@@ -79,26 +79,34 @@ __device__ __forceinline__ void slab_store(const Vec<VEC> &d, __amdgpu_buffer_rs
 // arithmetic runs beside another's loads and stores.  (A general exponent keeps the registers it needs.)
 template <int Q, int VEC, int NTHREADS, int RPT>
 __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) ? 1 : 4) softmax_kernel(const SoftmaxArgs a, const int tpr_log2) {
+    // the scalar arguments as locals (read through the argument block inside the lambdas below, the block was
+    // copied to private memory in the instantiations for a general exponent)
+    const int n_words = a.words;
+    const float dual_q = a.qv;
+    const float eps_v = a.eps;
+    const int d_in = a.D;
+    const int d_out = a.H;
+    const float scale_v = a.scale;
     constexpr int NW = NTHREADS / WAVE;
     extern __shared__ float smem[];
     const int TPR = 1 << tpr_log2, TH = TPR * VEC, RG = NTHREADS >> tpr_log2;
     float *part = smem;                              // [words][NW][2][TH] column partial norms (x, then e)
-    float *col = part + a.words * NW * 2 * TH;       // [5][TH]: k_lo, k_up of exp; e.lb, e.ub; b = l_e
+    float *col = part + n_words * NW * 2 * TH;       // [5][TH]: k_lo, k_up of exp; e.lb, e.ub; b = l_e
     float *spart = col + 5 * TH;                     // [words][NW][2] partial norms of the one-neuron objects s, r
-    float *scal = spart + a.words * NW * 2;          // [2]: s.lb, s.ub
+    float *scal = spart + n_words * NW * 2;          // [2]: s.lb, s.ub
 
     const int r = blockIdx.x;
     const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
     const int c = tid & (TPR - 1), rg = tid >> tpr_log2;
     const int col0 = c * VEC;
-    const bool col_ok = col0 < a.H;                  // VEC == 4: H % 4 == 0, so the four columns stand or fall together
-    const int blk = a.D / a.words;
+    const bool col_ok = col0 < d_out;                  // VEC == 4: H % 4 == 0, so the four columns stand or fall together
+    const int blk = d_in / n_words;
 
     // the column's constant terms first: they are needed right after the first barrier and would otherwise
     // be fetched then, behind the whole machine's slab loads
-    const size_t bi = (size_t)r * a.H + tid;         // thread h < H speaks for column h
+    const size_t bi = (size_t)r * d_out + tid;         // thread h < H speaks for column h
     float xlb = 0.f, xub = 0.f;
-    if (tid < a.H) {
+    if (tid < d_out) {
         xlb = a.lb[bi];
         xub = a.ub[bi];
     }
@@ -107,10 +115,10 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
     // Buffer addressing over the row's own slab: a thread whose column does not exist is sent outside the window
     // and slab rows past D_in fall outside it, where loads return zero and stores are dropped -- no branch and
     // no wait between the loads, all 2 RPT of a thread are in flight together.
-    const unsigned slab_bytes = (unsigned)a.D * a.H * 4u;
-    const size_t slab0 = (size_t)r * a.D * a.H;
-    const unsigned voff = col_ok ? ((unsigned)rg * a.H + col0) * 4u : 0x80000000u;
-    const unsigned step_bytes = (unsigned)RG * a.H * 4u;
+    const unsigned slab_bytes = (unsigned)d_in * d_out * 4u;
+    const size_t slab0 = (size_t)r * d_in * d_out;
+    const unsigned voff = col_ok ? ((unsigned)rg * d_out + col0) * 4u : 0x80000000u;
+    const unsigned step_bytes = (unsigned)RG * d_out * 4u;
     Vec<VEC> dl[RPT], du[RPT];
     {
         const __amdgpu_buffer_rsrc_t wl = slab_window(a.lw + slab0, slab_bytes), wu = slab_window(a.uw + slab0, slab_bytes);
@@ -123,8 +131,8 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
         for (int i = 0; i < RPT; ++i) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {        // one rounding, as the separate scaling stores it
-                dl[i].set(v, dl[i].get(v) * a.scale);
-                du[i].set(v, du[i].get(v) * a.scale);
+                dl[i].set(v, dl[i].get(v) * scale_v);
+                du[i].set(v, du[i].get(v) * scale_v);
             }
         }
     }
@@ -135,8 +143,8 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
     // value (the usual case; rows past D_in hold zeros and add nothing to any norm).
     const bool whole_steps = blk % RG == 0;
     const int steps_per_word = blk / RG;
-    auto column_norms = [&]() {
-        for (int w = 0; w < a.words; ++w) {
+    auto column_norms = [&]() __attribute__((always_inline)) {
+        for (int w = 0; w < n_words; ++w) {
             const int lo_row = w * blk, hi_row = lo_row + blk;
             float pl[VEC], pu[VEC];
 #pragma unroll
@@ -148,8 +156,12 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
                     if (i >= lo_i && i < hi_i) {
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) {
-                            pl[v] = nacc<Q>(pl[v], dl[i].get(v), a.qv);
-                            pu[v] = nacc<Q>(pu[v], du[i].get(v), a.qv);
+                            float xl = dl[i].get(v), xu = du[i].get(v);
+                            // (general exponent: opaque copies as below, or log |x| of all 2 RPT VEC values is formed
+                            // outside the loop over the words and held)
+                            if (Q == Q_GENERAL) asm volatile("" : "+v"(xl), "+v"(xu));
+                            pl[v] = nacc<Q>(pl[v], xl, dual_q);
+                            pu[v] = nacc<Q>(pu[v], xu, dual_q);
                         }
                     }
                 }
@@ -164,8 +176,8 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
                             // loop over the words, and held (64 more registers)
                             float xl = dl[i].get(v), xu = du[i].get(v);
                             asm volatile("" : "+v"(xl), "+v"(xu));
-                            pl[v] = nacc<Q>(pl[v], xl, a.qv);
-                            pu[v] = nacc<Q>(pu[v], xu, a.qv);
+                            pl[v] = nacc<Q>(pl[v], xl, dual_q);
+                            pu[v] = nacc<Q>(pu[v], xu, dual_q);
                         }
                     }
                 }
@@ -183,8 +195,8 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
     // norms over D_in of a one-neuron object whose coefficients sit in sl / su (every thread of a slab row holds
     // the same values: the threads of column group 0 speak for the row) -> spart; the caller synchronises
     float sl[RPT], su[RPT];
-    auto neuron_norms = [&]() {
-        for (int w = 0; w < a.words; ++w) {
+    auto neuron_norms = [&]() __attribute__((always_inline)) {
+        for (int w = 0; w < n_words; ++w) {
             const int lo_row = w * blk, hi_row = lo_row + blk;
             float pl[1] = {0.f}, pu[1] = {0.f};
             if (c == 0) {
@@ -192,8 +204,8 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
                 for (int i = 0; i < RPT; ++i) {
                     const int row = i * RG + rg;
                     if (row >= lo_row && row < hi_row) {
-                        pl[0] = nacc<Q>(pl[0], sl[i], a.qv);
-                        pu[0] = nacc<Q>(pu[0], su[i], a.qv);
+                        pl[0] = nacc<Q>(pl[0], sl[i], dual_q);
+                        pu[0] = nacc<Q>(pu[0], su[i], dual_q);
                     }
                 }
             }
@@ -206,10 +218,10 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
         }
     };
     // [lb - eps * sum of norms, ub + eps * sum of norms] from partial norms (Bounds.py:311-326)
-    auto interval = [&](const float *p, int stride, int offset, float lb, float ub, float &l, float &u) {
+    auto interval = [&](const float *p, int stride, int offset, float lb, float ub, float &l, float &u) __attribute__((always_inline)) {
         l = lb;
         u = ub;
-        for (int w = 0; w < a.words; ++w) {
+        for (int w = 0; w < n_words; ++w) {
             // the wavefronts' partial norms are fetched eight at a time before the first is used: one LDS latency
             // per eight wavefronts instead of one per wavefront (combined in the order of the wavefronts all the same)
             constexpr int CH = NW < 8 ? NW : 8;
@@ -228,34 +240,34 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
                     nu = ncomb<Q>(nu, vu[g]);
                 }
             }
-            l += (-a.eps) * nfin<Q>(nl, a.qv);
-            u += a.eps * nfin<Q>(nu, a.qv);
+            l += (-eps_v) * nfin<Q>(nl, dual_q);
+            u += eps_v * nfin<Q>(nu, dual_q);
         }
     };
 
     // the same for a one-neuron object from spart, every thread for itself: lane g takes wavefront g's partial norm
     // and a butterfly over NW lanes combines them (2 log2 NW exchanges per word instead of 2 NW reads and sums)
-    auto neuron_interval = [&](float lb, float ub, float &l, float &u) {
+    auto neuron_interval = [&](float lb, float ub, float &l, float &u) __attribute__((always_inline)) {
         l = lb;
         u = ub;
-        for (int w = 0; w < a.words; ++w) {
+        for (int w = 0; w < n_words; ++w) {
             float nl = spart[(w * NW + lane % NW) * 2 + 0], nu = spart[(w * NW + lane % NW) * 2 + 1];
 #pragma unroll
             for (int m = 1; m < NW; m <<= 1) {
                 nl = ncomb<Q>(nl, __shfl_xor(nl, m, WAVE));
                 nu = ncomb<Q>(nu, __shfl_xor(nu, m, WAVE));
             }
-            l += (-a.eps) * nfin<Q>(nl, a.qv);
-            u += a.eps * nfin<Q>(nu, a.qv);
+            l += (-eps_v) * nfin<Q>(nl, dual_q);
+            u += eps_v * nfin<Q>(nu, dual_q);
         }
     };
 
     // ---- e = exp(x): Bounds.py:970-1003
     column_norms();
     __syncthreads();
-    if (tid < a.H) {
-        xlb *= a.scale;
-        xub *= a.scale;
+    if (tid < d_out) {
+        xlb *= scale_v;
+        xub *= scale_v;
         float l, u, klo, kup, elb, eub;
         interval(part, TH, tid, xlb, xub, l, u);
         relax_point<EXP>(l, u, xlb, xub, klo, kup, elb, eub);
@@ -300,7 +312,7 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
     // 1 and 2 as permutations of four lanes; after them the four lanes of a group hold one value, so mirroring
     // eight lanes fetches what lane ^ 4 holds, and after that mirroring sixteen fetches what lane ^ 8 holds.
     // Longer distances go through the crossbar, 2 RPT exchanges in flight at a time.
-    auto butterfly_step = [&](auto exchange) {
+    auto butterfly_step = [&](auto exchange) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < RPT; ++i) {
             sl[i] += exchange(sl[i]);
@@ -314,7 +326,7 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
     for (int m = 16; m < TPR; m <<= 1) combine_across<FAITH_Q_1>(sl, su, m);      // Q_1: a sum
     if (wv == 0) {
         float tl = 0.f, tu = 0.f;
-        for (int h = lane; h < a.H; h += WAVE) {
+        for (int h = lane; h < d_out; h += WAVE) {
             tl += col[2 * TH + h];
             tu += col[3 * TH + h];
         }
@@ -354,7 +366,7 @@ __global__ void __launch_bounds__(NTHREADS, (Q == Q_GENERAL && NTHREADS < 1024) 
     __syncthreads();
     float al, au;
     neuron_interval(rlb, rub, al, au);
-    if (tid < a.H) {
+    if (tid < d_out) {
         const float elb = col[2 * TH + tid], eub = col[3 * TH + tid];
         float bt, unused;
         interval(part, TH, tid, elb, eub, bt, unused);
