@@ -35,6 +35,7 @@ EXTRA = {
     # compiler need not quiet signalling NaNs first
     "dot.hip": ["-fno-honor-nans"],
     "dot_tiled.hip": ["-fno-honor-nans"],
+    "dot_transposed.hip": ["-fno-honor-nans"],
 }
 
 

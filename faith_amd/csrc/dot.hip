@@ -50,6 +50,7 @@
 
 #include "common.h"
 #include "dot_tiled.h"
+#include "dot_transposed.h"
 
 namespace {
 
@@ -966,8 +967,9 @@ int dot_entry(const char *who, float *x_l, float *y_l, float *x_u, float *y_u, c
 // columns j, one m per tile) would read 4 bytes per 128-byte line.  Lanes run along m instead: every load and
 // store of a wavefront is one contiguous 256-byte run, the coefficients a[j, k], b[i, k] are wave-uniform
 // (scalar loads), and each lane keeps an RI x RJ block of (i, j) pairs for its m in registers -- 8 RI RJ
-// fused multiply-adds per 2 (RI + RJ) loads.  Vector ALU, not MFMA: this is the compatibility layout;
-// callers that keep the natural layout take the MFMA kernels above.
+// fused multiply-adds per 2 (RI + RJ) loads.  Vector ALU, not MFMA: the kernel for any shape in this layout;
+// shapes of whole blocks take the two MFMA launches of dot_transposed.hip (x terms with i fixed, y terms with j
+// fixed: each alone is a matrix product whose operands need no re-layout).
 // ------------------------------------------------------------------------------------------
 struct DotTArgs {
     const float *xlw, *xuw, *ylw, *yuw;   // [B, Lx, K, D], [B, Ly, K, D]
@@ -1129,6 +1131,11 @@ int dot_entry_transposed(const char *who, float *x_l, float *y_l, float *x_u, fl
         return faith::check_launch(who);
     }
     hipLaunchKernelGGL(dot_b<false>, dim3((unsigned)b_tiles), dim3(256), 0, st, g);
+    // whole blocks everywhere: the MFMA kernels (knob value 3 keeps the vector-ALU kernel)
+    if (faith::tune_get(FAITH_TUNE_DOT_VARIANT) != 3 && faith::dot_transposed_mfma_takes(Lx, Ly, K, D)) {
+        const faith::DotTransposedArgs ta{x_lw, x_uw, y_lw, y_uw, x_l, y_l, y_u, z_lw, z_uw, B, Lx, Ly, K, D};
+        if (faith::dot_transposed_mfma_launch(ta, st)) return faith::check_launch(who);
+    }
     hipLaunchKernelGGL((dot_w_transposed<RI, RJ>), dim3((unsigned)grid), dim3(256), 0, st, a);
     return faith::check_launch(who);
 }

@@ -287,7 +287,10 @@ def test_c_bound_dot_shims():
     # B, Lx, Ly, D, d (scores) / B, Lx, Lk, D, dv (context); words
     (2, 8, 8, 16, 12, 1),         # D_in below a wavefront: the four wavefronts of a workgroup along the columns
     (1, 5, 9, 100, 20, 2),        # two wavefronts along m, ragged rows, columns and lanes
-    (4, 32, 32, 256, 64, 1),      # configuration-3 operands at a quarter of the length: four wavefronts along m
+    (4, 32, 32, 256, 64, 1),      # configuration-3 operands at a quarter of the length: whole blocks everywhere, the MFMA kernels
+    (4, 32, 32, 256, 64, -1),     # the same on the vector-ALU kernel (tuning knob): four wavefronts along m
+    (1, 128, 128, 64, 64, 1),     # MFMA kernels: four row blocks per wavefront, dim_in of two wavefronts (two stay idle)
+    (2, 64, 96, 160, 32, 2),      # MFMA kernels: 96 rows as three passes of one block, a partly filled second block of dim_in
     (1, 3, 70, 300, 7, 3),        # D_in beyond one workgroup's 256 lanes, more columns than a workgroup takes
     (2, 6, 4, 1, 10, 1),          # dim_in == 1: the interval shortcut
 ])
@@ -298,6 +301,8 @@ def test_dot_products_in_the_reference_layout_through_the_c_abi(shape, p):
     import ctypes
     from faith_amd import _lib, ops
     B, Lx, L2, D, d, words = shape
+    vector_alu = words < 0
+    words = abs(words)
     g = torch.Generator().manual_seed(37)
     eps = 0.05
     P = lambda t_: ctypes.c_void_p(t_.data_ptr())
@@ -312,9 +317,15 @@ def test_dot_products_in_the_reference_layout_through_the_c_abi(shape, p):
         ops_ = [x.lb.cuda().contiguous(), x.ub.cuda().contiguous(), y.lb.cuda().contiguous(), y.ub.cuda().contiguous(),
                 T(x.lw), T(x.uw), T(y.lw), T(y.uw)]
         dims = (B, Lx, Ly, K, D) if entry.endswith("QK") else (B, Lx, K, Ly, D)
-        _lib.call(entry, P(x_l), P(y_l), P(x_u), P(y_u), *(P(t_) for t_ in ops_), P(zlb), P(zub), P(zlw), P(zuw),
-                  *dims, eps, ops.q_code(p), words, _lib.LAYOUT_TRANSPOSED, stream)
-        torch.cuda.synchronize()
+        if vector_alu:
+            _lib.call("faith_tune_set", 2, 3)
+        try:
+            _lib.call(entry, P(x_l), P(y_l), P(x_u), P(y_u), *(P(t_) for t_ in ops_), P(zlb), P(zub), P(zlw), P(zuw),
+                      *dims, eps, ops.q_code(p), words, _lib.LAYOUT_TRANSPOSED, stream)
+            torch.cuda.synchronize()
+        finally:
+            if vector_alu:
+                _lib.call("faith_tune_set", 2, 0)
         return (zlw.transpose(2, 3), zlb, zuw.transpose(2, 3), zub), (x_l, x_u, y_l, y_u)
 
     # scores: x [B, Lx, D, d], y [B, L2, D, d]
