@@ -121,7 +121,7 @@ def quad(d):
 # dot product's eight products per term the four y terms, which share their multiplier, become two.  The roofline
 # fraction counts the products that are multiplied (what the MFMA pipe does); the rate in the reference's own
 # formulation is reported beside it for comparison with numbers quoted that way.
-EXECUTED = {"linear": 2 / 4, "conv": 2 / 4, "dot": 6 / 8, "dot_transposed": 1.0}
+EXECUTED = {"linear": 2 / 4, "conv": 2 / 4, "dot": 6 / 8}
 
 
 def op_entry(name, kind, times_ms, work, cpu=None, extra=None, form=None):
@@ -493,7 +493,7 @@ def bench_config3(args, ops, O, wl):
     tv = gpu_times_ms(lambda: ops.dot_product_v(probs, quad(y), c["p"], c["eps"], 1, out=outv), 50, 5)
     ev = op_entry("extra: context (probs.value) 4 heads [4,128,256,128].[4,128,256,64]", "mfma", tv, flopv, form="dot")
     # the same scores through the reference's own calling convention: operands [B, L, dim_out, dim_in], result
-    # [B, Lx, Ly, dim_in] (vector ALU with lanes along dim_in, no re-layout); the roofline is still the MFMA peak
+    # [B, Lx, Ly, dim_in] (MFMA with the operands straight from that layout: y terms per column j, x terms per row i)
     from faith_amd import c_bound
     T = lambda t_: t_.transpose(2, 3).contiguous()
     xt, yt = (T(x["lw"]), T(x["uw"])), (T(y["lw"]), T(y["uw"]))
@@ -504,8 +504,8 @@ def bench_config3(args, ops, O, wl):
     tt = gpu_times_ms(lambda: c_bound.c_dot_product_verification_QK(*scr, x["lb"], x["ub"], y["lb"], y["ub"], xt[0], xt[1],
                                                                     yt[0], yt[1], *zt, B, L, d, D, c["eps"]), 50, 5)
     c_bound.p = 2.0
-    et = op_entry("extra: config3 scores in the reference's transposed layout (c_bound.c_dot_product_verification_QK)",
-                  "mfma", tt, flop, form="dot_transposed")
+    et = op_entry("extra: config3 scores in the reference's transposed layout (c_bound.c_dot_product_verification_QK: "
+                  "concretize + constant terms + y-term and x-term MFMA launches)", "mfma", tt, flop, form="dot")
     return [e, ev, et]
 
 
@@ -548,6 +548,40 @@ def bench_config4(args, ops, O, wl):
                                     {"result_write_GBs": round(2 * D * co * ho * ho * 4 / statistics.median(tk) / 1e6, 1)}))
         del lw, uw, o_
     return out_entries
+
+
+def bench_sub_blocks(args, rows, hidden, inter):
+    """The encoder sub-blocks of the batched propagation as single operators, at its size (rows positions of dim_in =
+    hidden): dense + residual + layer norm and dense + ReLU in one pass over the coefficients, beside the separate
+    launches they replace.  TFLOP/s count the layer's two executed products per term."""
+    import torch
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(78)
+    n = 5 if args.profile else 20
+    out = []
+
+    def obj(width):
+        lw = (torch.randn(1, rows, hidden, width, generator=g) * 0.05).cuda()
+        lb = torch.randn(1, rows, width, generator=g).cuda()
+        return lw, lb, lw + 0.005, lb + 0.1
+    for what, K, N in (("attention output", hidden, hidden), ("feed-forward output", inter, hidden)):
+        x, r = obj(K), obj(N)
+        W, b = (torch.randn(N, K, generator=g) / K ** 0.5).cuda(), (0.05 * torch.randn(N, generator=g)).cuda()
+        w, sh = (1.0 + 0.1 * torch.randn(N, generator=g)).cuda(), (0.05 * torch.randn(N, generator=g)).cuda()
+        fused = gpu_times_ms(lambda: ops.linear_layer_norm(*x, W, b, w, sh, r), n, 2)
+        apart = gpu_times_ms(lambda: ops.layer_norm(*ops.linear(*x, W, b), w, sh, r), n, 2)
+        out.append(op_entry(f"extra: dense {K}->{N} + residual + layer norm (no_var) in one pass, {what} of the batched "
+                            f"propagation [1,{rows},{hidden},{K}]", "mfma", fused, 4 * 2 * rows * (hidden + 1) * K * N,
+                            form="linear", extra={"separate_launches_us": round(statistics.median(apart) * 1e3, 1)}))
+        del x, r
+    x = obj(hidden)
+    W, b = (torch.randn(inter, hidden, generator=g) / hidden ** 0.5).cuda(), (0.05 * torch.randn(inter, generator=g)).cuda()
+    fused = gpu_times_ms(lambda: ops.linear_relu(*x, W, b, 2.0, 0.01), n, 2)
+    apart = gpu_times_ms(lambda: ops.relu(*ops.linear(*x, W, b), 2.0, 0.01), n, 2)
+    out.append(op_entry(f"extra: dense {hidden}->{inter} + ReLU (p=2) in one pass, feed-forward input of the batched "
+                        f"propagation [1,{rows},{hidden},{hidden}]", "mfma", fused, 4 * 2 * rows * (hidden + 1) * hidden * inter,
+                        form="linear", extra={"separate_launches_us": round(statistics.median(apart) * 1e3, 1)}))
+    return out
 
 
 def bench_layer(args, wl):
@@ -640,6 +674,7 @@ def bench_layer(args, wl):
 
     # the same two, replayed from a HIP graph captured once (forward.CapturedVerifier)
     out = [e, e2]
+    out.extend(bench_sub_blocks(args, len(positions) * length, hidden, inter))
     for batch, pos in ((1, [3]), (len(positions), positions)):
         cap = F.CapturedVerifier(gmake, net, ge, batch, 0, p)
         rr = [eps] * batch

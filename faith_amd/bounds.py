@@ -167,9 +167,23 @@ class Bounds:
     def matmul(self, W, bias=None):
         if isinstance(W, (Bounds, CompactBounds)):
             raise NotImplementedError("matmul with a Bounds operand is dot_product")
-        if W.dim() != 2:
-            raise NotImplementedError("only a 2-D weight has a kernel")
         lw, lb, uw, ub = self._c()
+        if W.dim() == 3:
+            # one weight per position (Bounds.py:414-428: W [length, H_out, H], a single batch element): the layer
+            # kernel on each position's rows, which are contiguous in both objects
+            if bias is not None or lw.shape[0] != 1 or W.shape[0] != lw.shape[1] or W.shape[2] != lw.shape[3]:
+                raise ValueError(f"a per-position weight must be [length={lw.shape[1]}, H_out, {lw.shape[3]}] for one batch "
+                                 f"element and come without a bias, got {tuple(W.shape)} for lw {tuple(lw.shape)}")
+            W = W.contiguous()
+            L, N = W.shape[0], W.shape[1]
+            out = (lw.new_empty(1, L, lw.shape[2], N), lb.new_empty(1, L, N), lw.new_empty(1, L, lw.shape[2], N),
+                   lb.new_empty(1, L, N))
+            for i in range(L):
+                ops.linear(lw[:, i:i + 1], lb[:, i:i + 1], uw[:, i:i + 1], ub[:, i:i + 1], W[i], None,
+                           out=tuple(t[:, i:i + 1] for t in out))
+            return self._like(*out)
+        if W.dim() != 2:
+            raise NotImplementedError("a weight is [H_out, H] or, per position, [length, H_out, H]")
         return self._like(*ops.linear(lw, lb, uw, ub, W.contiguous(), bias))
 
     # ---- Bounds.py:1016-1025 (bias fused into the same launch)

@@ -350,3 +350,25 @@ def test_linear_concretize_rejects_bad_words():
     x = rand_bounds(g, 1, 2, 6, 8, ordered=False)
     with pytest.raises(_lib.FaithError):
         run_fused(x, torch.randn(4, 8, generator=g), None, 2.0, 0.1, 4)     # 4 does not divide dim_in = 6
+
+
+def test_per_position_weight_of_matmul_runs_the_layer_kernel_position_by_position():
+    """Bounds.matmul with a 3-D weight (Bounds.py:414-428: one [H_out, H] matrix per position, a single batch
+    element): each position against the oracle's layer with that position's matrix."""
+    from faith_amd import Bounds
+    g = torch.Generator().manual_seed(90)
+    L, D, H, N = 5, 24, 32, 20
+    x = rand_bounds(g, 1, L, D, H, ordered=False, sw=0.5)
+    W = torch.randn(L, N, H, generator=g) / H ** 0.5
+    lw, lb, uw, ub = dev(*x.tensors())
+    got = Bounds(None, 2.0, 0.01, lw=lw, lb=lb, uw=uw, ub=ub).matmul(W.cuda())
+    torch.cuda.synchronize()
+    assert got.lw.shape == (1, L, D, N) and got.lb.shape == (1, L, N)
+    for i in range(L):
+        xi = O.LinearBounds(x.lw[:, i:i + 1], x.lb[:, i:i + 1], x.uw[:, i:i + 1], x.ub[:, i:i + 1])
+        exp = O.linear(xi, W[i], None)
+        ref, mag = linear64(xi, W[i], None)
+        for name, a, e in zip(("lw", "lb", "uw", "ub"), (got.lw, got.lb, got.uw, got.ub), exp.tensors()):
+            compare_contraction(name, a[:, i:i + 1], e, ref[name], mag[name])
+    with pytest.raises(ValueError):
+        Bounds(None, 2.0, 0.01, lw=lw, lb=lb, uw=uw, ub=ub).matmul(W[:3].cuda())
