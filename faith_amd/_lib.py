@@ -32,6 +32,8 @@ SIGNATURES = {
     "faith_unary_verification": [_I] + [_P] * 10 + [_I, _I, _I, _F, _I, _I, _I, _P],
     "faith_multiply_verification": [_P] * 12 + [_I, _I, _I, _F, _I, _I, _P],
     "faith_affine_verification": [_P] * 5 + [_F] + [_P] * 9 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
+    "faith_rows_gather": [_P] * 5 + [_I] * 4 + [_P],
+    "faith_rows_put": [_P] * 7 + [_I] * 4 + [_P],
     "faith_rowsum_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_rowmean_verification": [_P] * 8 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],
     "faith_layer_norm_verification": [_P] * 14 + [ctypes.c_longlong, ctypes.c_longlong, _I, _P],

@@ -500,10 +500,10 @@ class CompactBounds:
         """(l, u) [B, L, H], as concretize() of the dense form gives them (computed once)."""
         if self._intervals is None:
             lb, ub = self._lb.contiguous(), self._ub.contiguous()
-            l, u = ops.concretize(self._lw.contiguous(), ops.gather_positions(lb, self.positions),
-                                  self._uw.contiguous(), ops.gather_positions(ub, self.positions),
+            rows_lb, rows_ub = ops.gather_positions(lb, ub, self.positions)
+            l, u = ops.concretize(self._lw.contiguous(), rows_lb, self._uw.contiguous(), rows_ub,
                                   self.p, self.eps, self.perturbed_words)
-            self._intervals = (ops.put_positions(lb, self.positions, l), ops.put_positions(ub, self.positions, u))
+            self._intervals = ops.put_positions(lb, ub, self.positions, l, u)
         return self._intervals
 
     # ---- VerifierForward.py:208-229 + Bounds.py:833-841 for two objects with coefficients at the same positions

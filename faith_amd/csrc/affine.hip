@@ -248,6 +248,47 @@ __global__ void __launch_bounds__(256) interval_product_kernel(const float *__re
     }
 }
 
+// ------------------------------------------------------------------ rows of a compact object
+// An object whose coefficients vanish outside P positions per batch element keeps [B, P, ...] rows and an
+// index positions[B, P] (VerifierForward.py:127-156 builds such an input).  Its concrete intervals are the constants
+// everywhere except at those positions: two tensors [B, L, H] are read at / rewritten at the P rows.  Data
+// movement only; a position outside 0 .. L-1 names no row (reads as zero, replaces nothing).
+__global__ void __launch_bounds__(256) rows_gather2(const float *__restrict__ a, const float *__restrict__ b,
+                                                    const long long *__restrict__ pos, float *__restrict__ oa,
+                                                    float *__restrict__ ob, const int L, const int P, const int H,
+                                                    const size_t n) {          // n = B * P * H
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+        const size_t bp = e / H;
+        const int h = (int)(e % H);
+        const long long l = pos[bp];
+        const bool there = l >= 0 && l < L;
+        const size_t src = ((bp / P) * L + (there ? l : 0)) * H + h;
+        oa[e] = there ? a[src] : 0.f;
+        ob[e] = there ? b[src] : 0.f;
+    }
+}
+
+__global__ void __launch_bounds__(256) rows_put2(const float *__restrict__ a, const float *__restrict__ b,
+                                                 const float *__restrict__ ra, const float *__restrict__ rb,
+                                                 const long long *__restrict__ pos, float *__restrict__ oa,
+                                                 float *__restrict__ ob, const int L, const int P, const int H,
+                                                 const size_t n) {             // n = B * L * H
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+        const size_t bl = e / H;
+        const int h = (int)(e % H);
+        const size_t bb = bl / L;
+        const long long l = (long long)(bl % L);
+        int slot = -1;
+        for (int p = 0; p < P; ++p)
+            if (pos[bb * P + p] == l) slot = p;
+        const size_t src = (bb * P + (slot >= 0 ? slot : 0)) * H + h;
+        oa[e] = slot >= 0 ? ra[src] : a[e];
+        ob[e] = slot >= 0 ? rb[src] : b[e];
+    }
+}
+
 bool all_aligned16(std::initializer_list<const void *> ptrs) {
     for (const void *p : ptrs)
         if (p != nullptr && !faith::aligned(p, 16)) return false;
@@ -356,4 +397,37 @@ extern "C" int faith_interval_product(const float *x_l, const float *x_u, const 
     hipLaunchKernelGGL(interval_product_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), x_l, x_u, y_l, y_u, z_lb, z_ub, (size_t)n);
     return faith::check_launch("faith_interval_product");
+}
+
+extern "C" int faith_rows_gather(const float *a, const float *b, const long long *positions, float *out_a, float *out_b,
+                                 int batch_size, int length, int n_positions, int dim_out, void *stream) {
+    FAITH_NOT_NULL(a); FAITH_NOT_NULL(b); FAITH_NOT_NULL(positions); FAITH_NOT_NULL(out_a); FAITH_NOT_NULL(out_b);
+    FAITH_ALIGNED4(a); FAITH_ALIGNED4(b); FAITH_ALIGNED4(out_a); FAITH_ALIGNED4(out_b);
+    FAITH_REQUIRE(faith::aligned(positions, 8), FAITH_ERR_ALIGN, "faith_rows_gather: positions is not 8-byte aligned");
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && n_positions > 0 && dim_out > 0, FAITH_ERR_SHAPE,
+                  "faith_rows_gather: batch=%d length=%d positions=%d dim_out=%d must be positive", batch_size, length,
+                  n_positions, dim_out);
+    const size_t n = (size_t)batch_size * n_positions * dim_out;
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(rows_gather2, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a, b, positions, out_a, out_b, length, n_positions, dim_out, n);
+    return faith::check_launch("faith_rows_gather");
+}
+
+extern "C" int faith_rows_put(const float *a, const float *b, const float *rows_a, const float *rows_b,
+                              const long long *positions, float *out_a, float *out_b, int batch_size, int length,
+                              int n_positions, int dim_out, void *stream) {
+    FAITH_NOT_NULL(a); FAITH_NOT_NULL(b); FAITH_NOT_NULL(rows_a); FAITH_NOT_NULL(rows_b); FAITH_NOT_NULL(positions);
+    FAITH_NOT_NULL(out_a); FAITH_NOT_NULL(out_b);
+    FAITH_ALIGNED4(a); FAITH_ALIGNED4(b); FAITH_ALIGNED4(rows_a); FAITH_ALIGNED4(rows_b); FAITH_ALIGNED4(out_a); FAITH_ALIGNED4(out_b);
+    FAITH_REQUIRE(faith::aligned(positions, 8), FAITH_ERR_ALIGN, "faith_rows_put: positions is not 8-byte aligned");
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && n_positions > 0 && dim_out > 0, FAITH_ERR_SHAPE,
+                  "faith_rows_put: batch=%d length=%d positions=%d dim_out=%d must be positive", batch_size, length,
+                  n_positions, dim_out);
+    const size_t n = (size_t)batch_size * length * dim_out;
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(rows_put2, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a, b, rows_a, rows_b, positions, out_a, out_b, length, n_positions,
+                       dim_out, n);
+    return faith::check_launch("faith_rows_put");
 }

@@ -800,25 +800,38 @@ def attention_scores(x, y, heads, p, eps, words=1):
     return zlw, zlb, zuw, zub
 
 
-def gather_positions(t, positions):
-    """[B, L, ...] -> [B, P, ...]: row positions[b, i] of batch element b (the inverse of spread_positions on
-    those rows; data movement only, nothing waits for the device)."""
-    B, P = positions.shape
-    out = _empty(B, P, *t.shape[2:], device=t.device)
-    index = positions.reshape(B, P, *([1] * (t.dim() - 2))).expand(B, P, *t.shape[2:])
-    return torch.gather(t, 1, index, out=out)
+def _positions_of(t, positions):
+    if t.dim() != 3:
+        raise ValueError(f"expected [B, L, H], got {tuple(t.shape)}")
+    _check("t", t)
+    B, L, H = t.shape
+    if positions.dtype != torch.int64 or positions.dim() != 2 or positions.shape[0] != B or positions.device != t.device \
+            or not positions.is_contiguous():
+        raise ValueError(f"positions must be a contiguous int64 tensor [{B}, P] on {t.device}")
+    return B, L, positions.shape[1], H
 
 
-def put_positions(t, positions, rows):
-    """A copy of t [B, L, ...] with row positions[b, i] of batch element b replaced by rows[b, i]."""
-    B, P = positions.shape
-    out = _empty_like(t)
-    out.copy_(t)
-    key = (B, str(t.device))
-    if key not in _BATCH_INDEX:
-        _BATCH_INDEX[key] = torch.arange(B, device=t.device)[:, None]
-    out[_BATCH_INDEX[key], positions] = rows
-    return out
+def gather_positions(a, b, positions):
+    """a, b [B, L, H] -> two tensors [B, P, H]: row positions[b, i] of batch element b (zero where the position lies
+    outside the sentence).  One launch for the pair; data movement only, nothing waits for the device."""
+    B, L, P, H = _positions_of(a, positions)
+    _check("b", b, a.shape)
+    oa, ob = _empty(B, P, H, device=a.device), _empty(B, P, H, device=a.device)
+    with _on(a.device):
+        _lib.call("faith_rows_gather", _ptr(a), _ptr(b), _ptr(positions), _ptr(oa), _ptr(ob), B, L, P, H, _stream(a))
+    return oa, ob
+
+
+def put_positions(a, b, positions, rows_a, rows_b):
+    """Copies of a, b [B, L, H] with row positions[b, i] of batch element b replaced by rows_a[b, i], rows_b[b, i]
+    ([B, P, H]).  One launch for the pair."""
+    B, L, P, H = _positions_of(a, positions)
+    _check("b", b, a.shape); _check("rows_a", rows_a, (B, P, H)); _check("rows_b", rows_b, (B, P, H))
+    oa, ob = _empty_like(a), _empty_like(b)
+    with _on(a.device):
+        _lib.call("faith_rows_put", _ptr(a), _ptr(b), _ptr(rows_a), _ptr(rows_b), _ptr(positions), _ptr(oa), _ptr(ob),
+                  B, L, P, H, _stream(a))
+    return oa, ob
 
 
 def attention_scores_compact_fits(length, n_positions, head_size, dim_in):

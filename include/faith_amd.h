@@ -213,6 +213,21 @@ int faith_rowmean_verification(const float *src_lb, const float *src_ub,
                                long long rows_w, long long rows_b, int dim_out, void *stream);
 
 /*
+ * Rows of an object that keeps the coefficients of n_positions positions per batch element only (the input object
+ * of VerifierForward.py:127-156 has zeros everywhere else).  No counterpart in the reference, which writes the zeros
+ * out; data movement only.  positions: int64 [batch, n_positions]; a position outside 0 .. length-1 names no row.
+ * faith_rows_gather: out_a, out_b [batch, n_positions, dim_out] = the rows a, b [batch, length, dim_out] have at the
+ * positions (zero for a position that names no row).  faith_rows_put: out_a, out_b [batch, length, dim_out] = a, b
+ * with the rows at the positions replaced by rows_a, rows_b [batch, n_positions, dim_out].  Two tensors a launch:
+ * the lower and the upper constants / intervals always travel together.  out_* must not overlap the inputs.
+ */
+int faith_rows_gather(const float *a, const float *b, const long long *positions, float *out_a, float *out_b,
+                      int batch_size, int length, int n_positions, int dim_out, void *stream);
+int faith_rows_put(const float *a, const float *b, const float *rows_a, const float *rows_b,
+                   const long long *positions, float *out_a, float *out_b,
+                   int batch_size, int length, int n_positions, int dim_out, void *stream);
+
+/*
  * Layer normalisation without the variance (Bounds.layer_norm, Bounds.py:1111-1131, mode "no_var",
  * and the first step of mode "standard"): subtract the row mean -- the mean of the UPPER tensor
  * from the lower one and the reverse, as matmul(ones / H).multiply(-1.) gives it -- then scale by

@@ -474,3 +474,27 @@ def test_captured_graph_on_the_compact_input_follows_new_positions_and_radii(len
         assert got == want, (idx, radii, got, want)
         seen.update(got)
     assert len(seen) == 2 or length != LENGTH                 # at the test network's own length both verdicts occur
+
+
+def test_rows_of_a_compact_object_are_gathered_and_put_back_by_the_library():
+    """faith_rows_gather / faith_rows_put against indexing on the CPU, a pair of tensors a launch; a position
+    outside the sentence reads as zero and replaces nothing."""
+    from faith_amd import ops
+    g = torch.Generator().manual_seed(140)
+    B, L, P, H = 3, 7, 2, 20
+    a, b = torch.randn(B, L, H, generator=g), torch.randn(B, L, H, generator=g)
+    ra, rb = torch.randn(B, P, H, generator=g), torch.randn(B, P, H, generator=g)
+    positions = torch.stack([torch.randperm(L, generator=g)[:P] for _ in range(B)])
+    positions[1, 0] = L + 2
+    ga, gb = ops.gather_positions(a.cuda(), b.cuda(), positions.cuda())
+    pa, pb = ops.put_positions(a.cuda(), b.cuda(), positions.cuda(), ra.cuda(), rb.cuda())
+    torch.cuda.synchronize()
+    ea, eb, fa, fb = torch.zeros(B, P, H), torch.zeros(B, P, H), a.clone(), b.clone()
+    for i in range(B):
+        for j in range(P):
+            l = int(positions[i, j])
+            if 0 <= l < L:
+                ea[i, j], eb[i, j] = a[i, l], b[i, l]
+                fa[i, l], fb[i, l] = ra[i, j], rb[i, j]
+    assert torch.equal(ga.cpu(), ea) and torch.equal(gb.cpu(), eb)
+    assert torch.equal(pa.cpu(), fa) and torch.equal(pb.cpu(), fb)
