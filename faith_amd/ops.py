@@ -610,8 +610,11 @@ class BoundCall:
         self._args = tuple(args)
         self._keep = keep
 
-    def __call__(self):
-        rc = self._fn(*self._args)
+    def __call__(self, stream=None):
+        """stream: a raw HIP stream handle (e.g. torch.cuda.current_stream().cuda_stream) to launch on instead of
+        the stream that was current when the call was bound -- a bound call does not follow torch's stream
+        context by itself (looking it up is part of what binding saves)."""
+        rc = self._fn(*self._args) if stream is None else self._fn(*self._args[:-1], stream)
         if rc:
             raise _lib.FaithError(self.name, rc, _lib.lib.faith_last_error().decode())
         return self.results
