@@ -606,6 +606,80 @@ __device__ __forceinline__ void sliced_tile(const GemmArgs &g, const int m_blk, 
     }
 }
 
+// The same arithmetic for MANY constant-term rows riding in front of a small problem's MFMA tiles (the query / key /
+// value layers of a batched propagation: 960 rows x 768 columns, whose 11,520 8 x 8 tiles were most of that launch):
+// a 32 x 32 tile per workgroup, 2 x 2 outputs per thread, the reduction in chunks of 32 -- a sixteenth of the
+// workgroups, each element of the operands staged once for 32 outputs instead of 8.  smem: 3 * 32 * 33 floats.
+__device__ __forceinline__ void wide_tile(const GemmArgs &g, const int m_blk, const int n_blk, float *smem) {
+    constexpr int T = 32, KC = 32;
+    float(*sl)[KC + 1] = reinterpret_cast<float(*)[KC + 1]>(smem);
+    float(*su)[KC + 1] = reinterpret_cast<float(*)[KC + 1]>(smem + T * (KC + 1));
+    float(*sw)[KC + 1] = reinterpret_cast<float(*)[KC + 1]>(smem + 2 * T * (KC + 1));
+    const int m0 = m_blk * T, n0 = n_blk * T;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;   // outputs (m0 + ty + 16 i, n0 + tx + 16 j)
+    double am[2][2] = {{0.0, 0.0}, {0.0, 0.0}}, ar[2][2] = {{0.0, 0.0}, {0.0, 0.0}};
+    for (int k0 = 0; k0 < g.K; k0 += KC) {
+#pragma unroll
+        for (int u = 0; u < T * KC / 256; ++u) {
+            const int e = threadIdx.x + u * 256;
+            const int r = e / KC, k = e % KC;
+            const bool kin = k0 + k < g.K;
+            const bool ain = kin && m0 + r < g.Mb, win = kin && n0 + r < g.N;
+            sl[r][k] = ain ? g.Bl[(size_t)(m0 + r) * g.K + k0 + k] : 0.f;
+            su[r][k] = ain ? g.Bu[(size_t)(m0 + r) * g.K + k0 + k] : 0.f;
+            sw[r][k] = win ? g.W[(size_t)(n0 + r) * g.K + k0 + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int kk = 0; kk < KC; ++kk) {
+            double m[2], r[2], w[2], wa[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const double xl = sl[ty + 16 * i][kk], xu = su[ty + 16 * i][kk];
+                m[i] = 0.5 * (xl + xu);
+                r[i] = 0.5 * (xu - xl);
+                w[i] = sw[tx + 16 * i][kk];
+                wa[i] = fabs(w[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    am[i][j] += w[j] * m[i];
+                    ar[i][j] += wa[j] * r[i];
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int row = m0 + ty + 16 * i, col = n0 + tx + 16 * j;
+            if (row < g.Mb && col < g.N) {
+                const float add = g.bias ? g.bias[col] : 0.f;
+                g.Dl[(size_t)row * g.N + col] = (float)(am[i][j] - ar[i][j]) + add;
+                g.Du[(size_t)row * g.N + col] = (float)(am[i][j] + ar[i][j]) + add;
+            }
+        }
+}
+
+// Constant-term tile `t` of a small problem: 8 x 8 tiles with the reduction split (few rows: short chains matter), or
+// 32 x 32 tiles (many rows: fewer workgroups, more reuse).  The host's count (constant_tiles) follows the same rule.
+__device__ __forceinline__ bool wide_constant_tiles(const GemmArgs &g) { return (long long)g.Mb * g.N >= (1 << 17); }
+__device__ __forceinline__ void constant_tile(const GemmArgs &g, const int t, float *smem) {
+    if (wide_constant_tiles(g)) {
+        const int tiles_n = (g.N + 31) / 32;
+        if (t / tiles_n < (g.Mb + 31) / 32) wide_tile(g, t / tiles_n, t % tiles_n, smem);
+    } else {
+        const int tiles_n = (g.N + 7) / 8;
+        if (t / tiles_n < (g.Mb + 7) / 8) sliced_tile(g, t / tiles_n, t % tiles_n, smem);
+    }
+}
+static long long constant_tiles(long long rows, long long n) {
+    return rows * n >= (1 << 17) ? ((rows + 31) / 32) * ((n + 31) / 32) : ((rows + 7) / 8) * ((n + 7) / 8);
+}
+
 __global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
     __shared__ float sm[3 * 16 * 17];
     const int tiles_n = (g.N + 15) / 16;
@@ -638,9 +712,7 @@ template <bool EXACT, int MBM, int MBN>
 __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs g, const int b_tiles) {
     __shared__ __align__(16) float sm[2 * 4 * 64 * 8 * (MBM + MBN)];   // 32 KB (64 x 64) or 48 KB
     if ((int)blockIdx.x < b_tiles) {
-        const int tiles_n = (g.N + 7) / 8;
-        const int m_blk = blockIdx.x / tiles_n;
-        if (m_blk < (g.Mb + 7) / 8) sliced_tile(g, m_blk, blockIdx.x % tiles_n, sm);
+        constant_tile(g, blockIdx.x, sm);
         return;
     }
     signsplit_gemm_body<EXACT, MBM, MBN>(g, sm, blockIdx.x - b_tiles);
@@ -770,10 +842,7 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_grouped(const GroupAr
     int pid = blockIdx.x;
     if (pid < b_tiles * G.groups) {
         const GemmArgs h = group_of(G, pid / b_tiles);
-        pid %= b_tiles;
-        const int tiles_n = (h.N + 7) / 8;
-        const int m_blk = pid / tiles_n;
-        if (m_blk < (h.Mb + 7) / 8) sliced_tile(h, m_blk, pid % tiles_n, sm);
+        constant_tile(h, pid % b_tiles, sm);
         return;
     }
     pid -= b_tiles * G.groups;
@@ -856,7 +925,7 @@ static int matmul_rows(const float *x_lb, const float *x_ub, const float *x_lw, 
         } else {
             // constant-term tiles in front, rounded up to a multiple of 8 so that the MFMA tiles keep
             // their XCD (workgroup number mod 8)
-            const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
+            const long long gridb = constant_tiles(rows, dim_y_out);
             const long long b_tiles = (gridb + XCDS - 1) / XCDS * XCDS;
             FAITH_REQUIRE(grid + b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
             const dim3 gd((unsigned)(grid + b_tiles)), bd(NTHREADS);
@@ -964,7 +1033,7 @@ static int matmul_group_rows(const float *x_lb, const float *x_ub, const float *
     G.groups = groups;
     const long long mblks = (mw + tm - 1) / tm;
     const long long w_tiles = ((mblks + XCDS - 1) / XCDS) * XCDS * ((dim_y_out + tn - 1) / tn);
-    const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
+    const long long gridb = constant_tiles(rows, dim_y_out);
     const long long b_tiles = (gridb + XCDS - 1) / XCDS * XCDS;
     FAITH_REQUIRE((w_tiles + b_tiles) * groups <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_group_verification: grid too large");
     const dim3 gd((unsigned)((w_tiles + b_tiles) * groups)), bd(NTHREADS);
