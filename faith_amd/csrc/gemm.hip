@@ -688,7 +688,9 @@ __global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
 
 // Launches the exact-accumulation kernel for the constant-term rows of g (its coefficient rows are left alone).
 // (The 8 x 8 tiles with the split reduction, which the small problems take inside their MFMA launch, measured
-// 40 - 170 us slower here at 960 rows x 256 .. 512 columns: four times the workgroups re-read W.)
+// 40 - 170 us slower here at 960 rows x 256 .. 512 columns: four times the workgroups re-read W; the 32 x 32 tiles
+// that serve many rows there 16 - 70 us slower: a quarter of the workgroups, each a four times longer chain with
+// nothing beside it.)
 // False if the grid would be too large.
 static bool launch_constant_rows(const GemmArgs &g, hipStream_t st) {
     GemmArgs gb = g;
