@@ -703,9 +703,15 @@ static bool launch_constant_rows(const GemmArgs &g, hipStream_t st) {
 
 template <bool EXACT>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-signsplit_gemm(const GemmArgs g) {
+signsplit_gemm(const GemmArgs g, const int b_tiles) {
     __shared__ float sm[2 * 4 * 2 * 128 * 8];            // two stages of four operands, 64 KB
-    signsplit_gemm_body<EXACT, 2, 2>(g, sm, blockIdx.x);
+    // the constant-term rows as leading workgroups (b_tiles of them, a multiple of 8): chains of short dependent
+    // steps that run beside the MFMA tiles instead of in a launch of their own behind them
+    if ((int)blockIdx.x < b_tiles) {
+        constant_tile(g, blockIdx.x, sm);
+        return;
+    }
+    signsplit_gemm_body<EXACT, 2, 2>(g, sm, blockIdx.x - b_tiles);
 }
 // Small problems: the first `b_tiles` workgroups take the 8 x 8 tiles of the constant-term rows
 // (exact accumulation; chains of short dependent steps, so they start first and run beside the
@@ -918,12 +924,13 @@ static int matmul_rows(const float *x_lb, const float *x_ub, const float *x_lw, 
         FAITH_REQUIRE(grid <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
         const bool exact = dim_out % BK == 0;
         if (tm == 128 && tn == 128) {
-            const long long gridb = ((rows + 15) / 16) * ((dim_y_out + 15) / 16);
+            const long long b_tiles = (constant_tiles(rows, dim_y_out) + XCDS - 1) / XCDS * XCDS;
+            FAITH_REQUIRE(grid + b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
+            const dim3 gd((unsigned)(grid + b_tiles));
             if (exact)
-                hipLaunchKernelGGL(signsplit_gemm<true>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
+                hipLaunchKernelGGL(signsplit_gemm<true>, gd, dim3(NTHREADS), 0, st, g, (int)b_tiles);
             else
-                hipLaunchKernelGGL(signsplit_gemm<false>, dim3((unsigned)grid), dim3(NTHREADS), 0, st, g);
-            FAITH_REQUIRE(launch_constant_rows(g, st), FAITH_ERR_SHAPE, "faith_matmul_verification: grid too large");
+                hipLaunchKernelGGL(signsplit_gemm<false>, gd, dim3(NTHREADS), 0, st, g, (int)b_tiles);
         } else {
             // constant-term tiles in front, rounded up to a multiple of 8 so that the MFMA tiles keep
             // their XCD (workgroup number mod 8)
@@ -1526,16 +1533,23 @@ namespace {
 
 template <bool EXACT, int MBN>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-signsplit_gemm_rownorm(const GemmArgs g, const RowNormArgs n) {
+signsplit_gemm_rownorm(const GemmArgs g, const RowNormArgs n, const int b_tiles) {
     extern __shared__ __align__(16) float dyn_sm[];     // two stages of (2 x 64 + 2 x 64 MBN) rows x 16 floats
-    signsplit_gemm_tile<EXACT, 1, MBN, -1, EPI_ROWNORM, RowNormArgs>(g, dyn_sm, blockIdx.x, 0, nullptr, nullptr, 0.f, n);
+    if ((int)blockIdx.x < b_tiles) {                    // the layer's constant-term rows, as in signsplit_gemm
+        constant_tile(g, blockIdx.x, dyn_sm);
+        return;
+    }
+    signsplit_gemm_tile<EXACT, 1, MBN, -1, EPI_ROWNORM, RowNormArgs>(g, dyn_sm, blockIdx.x - b_tiles, 0, nullptr, nullptr, 0.f, n);
 }
 
 template <bool EXACT, int MBN>
 bool launch_rownorm(const GemmArgs &g, const RowNormArgs &n, hipStream_t st) {
     const size_t lds = 2 * 4 * 64 * 8 * (1 + MBN) * sizeof(float);
     if (!faith::reserve_lds(signsplit_gemm_rownorm<EXACT, MBN>, lds)) return false;
-    hipLaunchKernelGGL((signsplit_gemm_rownorm<EXACT, MBN>), dim3((unsigned)((g.Mw + 63) / 64)), dim3(NTHREADS), lds, st, g, n);
+    const long long b_tiles = (constant_tiles(g.Mb, g.N) + XCDS - 1) / XCDS * XCDS;
+    const long long grid = (g.Mw + 63) / 64 + b_tiles;
+    if (grid > 0x7fffffffLL) return false;
+    hipLaunchKernelGGL((signsplit_gemm_rownorm<EXACT, MBN>), dim3((unsigned)grid), dim3(NTHREADS), lds, st, g, n, (int)b_tiles);
     return true;
 }
 
@@ -1588,10 +1602,9 @@ extern "C" int faith_matmul_layer_norm_verification(const float *x_lb, const flo
     bool ok;
     if (dim_y_out == 256) ok = exact ? launch_rownorm<true, 4>(g, n, st) : launch_rownorm<false, 4>(g, n, st);
     else ok = exact ? launch_rownorm<true, 2>(g, n, st) : launch_rownorm<false, 2>(g, n, st);
-    FAITH_REQUIRE(ok, FAITH_ERR_UNSUPPORTED, "faith_matmul_layer_norm_verification: the device refused the LDS size");
-    // constant terms: exact accumulation, then the same normalisation on [rows, dim_y_out] in place (a row is
-    // held in registers between its read and its write)
-    FAITH_REQUIRE(launch_constant_rows(g, st), FAITH_ERR_SHAPE, "faith_matmul_layer_norm_verification: grid too large");
+    FAITH_REQUIRE(ok, FAITH_ERR_UNSUPPORTED, "faith_matmul_layer_norm_verification: the device refused the LDS size, or the grid is too large");
+    // constant terms (exact accumulation, leading workgroups of that launch): the same normalisation on
+    // [rows, dim_y_out] in place (a row is held in registers between its read and its write)
     const int rc = faith::check_launch("faith_matmul_layer_norm_verification");
     if (rc != FAITH_OK) return rc;
     return faith_layer_norm_verification(y_lb, y_ub, y_lw, y_uw, res_lb, res_ub, adding ? res_lw : nullptr,
