@@ -306,8 +306,12 @@ class Bounds:
             low = float(l.min())
             assert (low > bound) if strict else (low >= bound), message
             return
-        per = l.reshape(c.mask.shape[0], -1).min(dim=1).values     # leading axis is batch-major
-        c.mask |= (per <= bound) if strict else (per < bound)
+        ops.flag_below(l.contiguous(), c.mask, bound, strict)           # leading axis is batch-major; one launch
+
+    @staticmethod
+    def verdict(l, u, flags, label, host=False):
+        """Safe or not per batch element (VerifierForward.py:311-314) in one launch: see ops.verdict."""
+        return ops.verdict(l.contiguous(), u.contiguous(), flags, label, host)
 
     class collect_failures:
         """with Bounds.collect_failures(batch, device) as f: ... ; f.mask[b] is True where a
@@ -423,6 +427,7 @@ class CompactBounds:
     outside that range; `dense_form`, `concrete_intervals` and everything that goes through them index with it."""
 
     collect_failures = Bounds.collect_failures
+    verdict = Bounds.verdict
 
     def __init__(self, args, p, eps, positions, lw, lb, uw, ub):
         self.args, self.p, self.eps = args, p, eps
@@ -570,6 +575,15 @@ class BoundsMaker:
 
     def compact(self, p, eps, positions, lw, lb, uw, ub):
         return CompactBounds(self.args, p, eps, positions, lw, lb, uw, ub)
+
+    # the input builders' device work, one launch each
+    @staticmethod
+    def positions_tensor(groups, device):
+        return ops.positions_tensor(groups, device)
+
+    @staticmethod
+    def input_coefficients(batch, rows, words, dim, device, positions=None, scales=None, out=None):
+        return ops.input_coefficients(batch, rows, words, dim, device, positions, scales, out=out)
 
 
 class ConvBounds:

@@ -52,18 +52,16 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
     if len(positions) != perturbed_words:
         raise ValueError(f"{len(positions)} positions given for {perturbed_words} perturbed words")
     compact = _compact_maker(make_bounds, 1, length, dim * perturbed_words, dim)
+    dev = embeddings.device
     if compact is not None and not ibp:
         # a maker that can hold the coefficients of the perturbed positions alone: the zero rows of
         # every other position are never written, read or multiplied
-        dev = embeddings.device
-        w = torch.zeros((1, perturbed_words, dim * perturbed_words, dim), device=dev)
-        for i in range(perturbed_words):
-            w[0, i, dim * i:dim * (i + 1), :] = _eye(dim, dev)
+        w = _input_coefficients(make_bounds, 1, perturbed_words, perturbed_words, dim, dev)
         b = embeddings[0].unsqueeze(0)
-        bounds = compact(p, eps, torch.as_tensor([positions], dtype=torch.int64, device=dev), w, b, w, b)
+        bounds = compact(p, eps, _positions(make_bounds, [positions], dev), w, b, w, b)
         return bounds if norm is None else bounds.layer_norm(norm, layer_norm)
-    w = torch.zeros((length, dim * perturbed_words, dim), device=embeddings.device)
     if ibp:
+        lw = torch.zeros((1, length, dim * perturbed_words, dim), device=dev)
         lb, ub = embeddings[0].unsqueeze(0).clone(), embeddings[0].unsqueeze(0).clone()
         for pos in positions:
             lb[0, pos] -= eps
@@ -72,9 +70,8 @@ def bound_input(make_bounds, embeddings, index, eps, perturbed_words=1, p=2.0, n
         # lower and upper start out equal and no operator writes into its inputs: one tensor serves both
         # (the reference copies ub and uw, :131, :149)
         lb = ub = embeddings[0].unsqueeze(0)
-        for i, pos in enumerate(positions):
-            w[pos, dim * i:dim * (i + 1), :] = _eye(dim, embeddings.device)
-    lw = w.unsqueeze(0)
+        lw = _input_coefficients(make_bounds, 1, length, perturbed_words, dim, dev,
+                                 _positions(make_bounds, [positions], dev))
     bounds = make_bounds(p, eps, lw, lb, lw, ub)
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
@@ -109,6 +106,41 @@ def _compact_maker(make_bounds, batch, length, dim_in, dim_out):
     if compact is None or (pays is not None and not pays(batch, length, dim_in, dim_out)):
         return None
     return compact
+
+
+def _positions(make_bounds, groups, device):
+    """int64 [len(groups), P] on the device; a maker may keep them across calls (`positions_tensor`)."""
+    keep = getattr(make_bounds, "positions_tensor", None)
+    if keep is not None:
+        return keep(groups, device)
+    return torch.as_tensor(groups, dtype=torch.int64, device=device).reshape(len(groups), -1)
+
+
+def _input_coefficients(make_bounds, batch, rows, words, dim, device, positions=None, scales=None, out=None):
+    """[batch, rows, dim * words, dim]: scales[b] * identity (identity without scales) in block i of the row that
+    holds perturbed word i -- row positions[b, i], or row i when positions is None (rows == words) -- and zero
+    elsewhere.  One launch when the maker brings its own builder (`input_coefficients`), tensor expressions
+    otherwise."""
+    build = getattr(make_bounds, "input_coefficients", None)
+    if build is not None:
+        return build(batch, rows, words, dim, device, positions, scales, out)
+    w = torch.zeros((batch, rows, dim * words, dim), device=device) if out is None else out.zero_()
+    eye = _eye(dim, device)
+    block = eye.expand(batch, dim, dim) if scales is None else scales[:, None, None] * eye
+    every = torch.arange(batch, device=device)
+    for i in range(words):
+        at = positions[:, i] if positions is not None else torch.full((batch,), i, device=device)
+        w[every, at, dim * i:dim * (i + 1), :] = block
+    return w
+
+
+def _verdict(bounds_type, l, u, failed, label):
+    """VerifierForward._bound_classifier (:311-314) per batch element, and not a failed precondition; a list of bools."""
+    own = getattr(bounds_type, "verdict", None)
+    if own is not None:
+        return own(l, u, failed.mask, label, host=True)
+    ok = (l[:, 0, 0] > 0) if label == 0 else (u[:, 0, 0] < 0)
+    return [bool(v) for v in (ok & ~failed.mask).tolist()]
 
 
 _EYES = {}
@@ -264,13 +296,12 @@ def bound_inputs(make_bounds, embeddings, indices, radii, p=2.0, norm=None, laye
     b = embeddings[0].unsqueeze(0).expand(n, length, dim).contiguous()
     compact = _compact_maker(make_bounds, n, length, dim, dim)
     # lower and upper start out equal and no operator writes into its inputs: one tensor serves both
+    at = _positions(make_bounds, [[i] for i in indices], dev)
     if compact is not None:
-        w = (scale[:, None, None] * _eye(dim, dev)).unsqueeze(1)              # [n, 1, dim, dim]
-        at = torch.as_tensor(indices, dtype=torch.int64, device=dev).reshape(n, 1)
+        w = _input_coefficients(make_bounds, n, 1, 1, dim, dev, scales=scale)
         bounds = compact(p, 1.0, at, w, b, w, b)
     else:
-        w = torch.zeros((n, length, dim, dim), device=dev)
-        w[torch.arange(n, device=dev), torch.as_tensor(indices, device=dev)] = scale[:, None, None] * _eye(dim, dev)
+        w = _input_coefficients(make_bounds, n, length, 1, dim, dev, at, scale)
         bounds = make_bounds(p, 1.0, w, b, w, b)
     if norm is not None:
         bounds = bounds.layer_norm(norm, layer_norm)
@@ -311,8 +342,7 @@ def _verify_safety(make_bounds, network, embeddings, index, eps, label, p, pertu
             x = propagate(x, network)
             pooled = bound_pooling(x, network.pooler, make_bounds)
             l, u = _margin(pooled, network.classifier)
-            ok = (l[0, 0, 0] > 0) if label == 0 else (u[0, 0, 0] < 0)
-            return bool(ok & ~failed.mask[0])
+            return _verdict(type(x), l, u, failed, label)[0]
     except AssertionError:
         return False
 
@@ -328,8 +358,7 @@ def verify_safety_batch(make_bounds, network, embeddings, indices, radii, label,
         x = propagate(x, network)
         pooled = bound_pooling(x, network.pooler, make_bounds)
         l, u = _margin(pooled, network.classifier)
-        ok = (l[:, 0, 0] > 0) if label == 0 else (u[:, 0, 0] < 0)
-        return [bool(v) for v in (ok & ~failed.mask).tolist()]
+        return _verdict(type(x), l, u, failed, label)
 
 
 def certified_radii(make_bounds, network, embeddings, positions, label, p=2.0, max_eps=0.1, num_iters=10,
@@ -376,10 +405,8 @@ class CapturedVerifier:
     def __init__(self, make_bounds, network, embeddings, batch, label, p=2.0):
         length, dim = embeddings.shape[1], embeddings.shape[2]
         dev = embeddings.device
-        self.batch, self.label, self.dim, self.length = batch, label, dim, length
+        self.batch, self.label, self.dim, self.length, self.make_bounds = batch, label, dim, length, make_bounds
         self.b = embeddings[0].unsqueeze(0).expand(batch, length, dim).contiguous()
-        self.eye = torch.eye(dim, device=dev)
-        self.rows = torch.arange(batch, device=dev)
         compact = _compact_maker(make_bounds, batch, length, dim, dim)
         if compact is not None:
             # the graph reads the perturbed positions and the scaled identities from these two
@@ -399,6 +426,9 @@ class CapturedVerifier:
                     x = x.layer_norm(network.embedding_norm, network.layer_norm)
                 pooled = bound_pooling(propagate(x, network), network.pooler, make_bounds)
                 l, u = _margin(pooled, network.classifier)
+            own = getattr(type(x), "verdict", None)
+            if own is not None:
+                return own(l, u, failed.mask, label)
             ok = (l[:, 0, 0] > 0) if label == 0 else (u[:, 0, 0] < 0)
             return ok & ~failed.mask
 
@@ -422,11 +452,11 @@ class CapturedVerifier:
         indices = [g[0] for g in _checked_positions([[i] for i in indices], self.length)]
         dev = self.w.device
         scale = torch.as_tensor(radii, dtype=torch.float32, device=dev)
+        at = _positions(self.make_bounds, [[i] for i in indices], dev)
         if self.at is not None:
-            self.at.copy_(torch.as_tensor(indices, dtype=torch.int64, device=dev).reshape(-1, 1))
-            self.w.copy_((scale[:, None, None] * self.eye).unsqueeze(1))
+            self.at.copy_(at)
+            _input_coefficients(self.make_bounds, self.batch, 1, 1, self.dim, dev, scales=scale, out=self.w)
         else:
-            self.w.zero_()
-            self.w[self.rows, torch.as_tensor(indices, device=dev)] = scale[:, None, None] * self.eye
+            _input_coefficients(self.make_bounds, self.batch, self.length, 1, self.dim, dev, at, scale, out=self.w)
         self.graph.replay()
         return [bool(v) for v in self.safe.tolist()]

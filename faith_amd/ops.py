@@ -837,6 +837,99 @@ def put_positions(a, b, positions, rows_a, rows_b):
     return oa, ob
 
 
+# ------------------------------------------------------------------------------------------
+# The layer driver's own device work (input coefficients, recorded preconditions, verdict): one launch each.
+# ------------------------------------------------------------------------------------------
+_POSITIONS = {}
+
+
+def positions_tensor(groups, device):
+    """int64 [len(groups), P] on the device for host-side lists of positions.  The same few tuples come back for
+    every step of a bisection and every query of a sentence, so the tensors are kept (bounded) and a repeated
+    query uploads nothing."""
+    key = (str(device), tuple(tuple(int(v) for v in g) for g in groups))
+    t = _POSITIONS.get(key)
+    if t is None:
+        if len(_POSITIONS) >= 4096:
+            _POSITIONS.clear()
+        t = torch.as_tensor(key[1], dtype=torch.int64, device=device).reshape(len(key[1]), -1)
+        _POSITIONS[key] = t
+    return t
+
+
+def input_coefficients(batch, rows, words, dim, device, positions=None, scales=None, scale=1.0, out=None):
+    """Coefficients of the input object (VerifierForward.py:127-156) [batch, rows, dim * words, dim], written whole by
+    one launch: scale * identity (scales[b] * identity with a tensor `scales` [batch]) in block i of the row that
+    holds perturbed word i -- row i when positions is None (an object that keeps those rows only: rows == words),
+    row positions[b, i] otherwise (int64 [batch, words] on the device) -- and zero elsewhere."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise ValueError(f"input_coefficients: must live on the GPU (got {device}); there is no CPU path")
+    shape = (batch, rows, dim * words, dim)
+    w = _empty(*shape, device=device) if out is None else _check("out", out, shape)
+    if positions is not None:
+        if not (positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous()
+                and tuple(positions.shape) == (batch, words)):
+            raise ValueError(f"positions: expected a contiguous int64 GPU tensor of shape {(batch, words)}")
+    elif rows != words:
+        raise ValueError(f"input_coefficients: without positions the object has one row per word ({rows} != {words})")
+    if scales is not None:
+        _check("scales", scales, (batch,))
+    with _on(w.device):
+        _lib.call("faith_input_coefficients", _ptr(w), _ptr(positions), _ptr(scales), float(scale), batch, rows, words,
+                  dim, int(positions is None), _stream(w))
+    return w
+
+
+def _flags(name, t, batch):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype in (torch.bool, torch.uint8) and t.is_contiguous()
+            and tuple(t.shape) == (batch,)):
+        raise ValueError(f"{name}: expected a contiguous bool / uint8 GPU tensor of shape ({batch},)")
+    return t
+
+
+def flag_below(l, flags, bound, strict):
+    """flags[b] |= any(l[b] fails `> bound` (strict) / `>= bound`): the preconditions of Bounds.sqrt and
+    Bounds.reciprocal (Bounds.py:892, :1147) recorded per batch element; nothing waits for the device."""
+    _check("l", l)
+    batch = flags.shape[0]
+    _flags("flags", flags, batch)
+    if l.numel() % batch:
+        raise ValueError(f"l: {l.numel()} values do not split over {batch} batch elements")
+    with _on(l.device):
+        _lib.call("faith_flag_below", _ptr(l), _ptr(flags), batch, l.numel() // batch, float(bound), int(bool(strict)),
+                  _stream(l))
+
+
+_VERDICTS = {}
+
+
+def verdict(l, u, flags, label, host=False):
+    """safe[b] = (l[b, 0, ...] > 0 if label == 0 else u[b, 0, ...] < 0) and not flags[b]
+    (VerifierForward.py:311-314 per batch element; flags may be None).  host = False: a bool tensor on the device,
+    nothing waits.  host = True: the kernel writes into pinned host memory, the stream is waited for and a list
+    of Python bools comes back -- one launch and no copy where reading a device tensor costs a copy kernel."""
+    _check("l", l)
+    _check("u", u, l.shape)
+    batch = l.shape[0]
+    if flags is not None:
+        _flags("flags", flags, batch)
+    if host:
+        key = (str(l.device), batch)
+        safe = _VERDICTS.get(key)
+        if safe is None:
+            safe = _VERDICTS[key] = torch.empty(batch, dtype=torch.bool, pin_memory=True)
+    else:
+        safe = torch.empty(batch, dtype=torch.bool, device=l.device)
+    with _on(l.device):
+        _lib.call("faith_verdict", _ptr(l), _ptr(u), _ptr(flags), _ptr(safe), batch, l.numel() // batch, int(label),
+                  _stream(l))
+        if host:
+            torch.cuda.current_stream(l.device).synchronize()
+            return safe.tolist()
+    return safe
+
+
 def attention_scores_compact_fits(length, n_positions, head_size, dim_in):
     """True if attention_scores_compact takes operands of this shape (16-byte aligned tensors assumed)."""
     return (dim_in > 1 and length % 4 == 0 and head_size % 4 == 0

@@ -228,6 +228,33 @@ int faith_rows_put(const float *a, const float *b, const float *rows_a, const fl
                    int batch_size, int length, int n_positions, int dim_out, void *stream);
 
 /*
+ * The layer driver's own device work, one launch each where the reference evaluates three or four tensor
+ * expressions; nothing here computes bounds.
+ *
+ * faith_input_coefficients: the coefficients of VerifierForward._bound_input (VerifierForward.py:127-156).
+ * w [batch, rows, dim * words, dim] is written whole: word i of batch element b owns the block
+ * [dim * i, dim * (i + 1)) x dim of one row -- row positions[b, i] (int64 [batch, words], device memory) of a
+ * dense object (rows = sentence length; a position outside 0 .. rows-1 names no row), row i of a compact one
+ * (compact != 0: rows == words, positions is not read and may be NULL) -- and that block is s * identity with
+ * s = scales[b] (device memory, [batch]) or, scales NULL, `scale`; everything else is zero.
+ *
+ * faith_flag_below: the preconditions the reference asserts on the host (Bounds.py:892 `min(l) > 0` for sqrt:
+ * strict != 0; :1147 `min(l) >= epsilon` for reciprocal: strict == 0), recorded per batch element instead:
+ * flags[b] (bytes, device memory) is set to 1 if any of the per_batch values l[b, :] fails the comparison with
+ * `bound` (a NaN fails it, as it fails the assert); flags are never cleared here.
+ *
+ * faith_verdict: VerifierForward._bound_classifier (:311-314) for every batch element:
+ * safe[b] = (label == 0 ? l[b * stride] > 0 : u[b * stride] < 0) and not flags[b] (flags may be NULL).
+ * safe: bytes, device memory or pinned host memory that the device can write.
+ */
+int faith_input_coefficients(float *w, const long long *positions, const float *scales, float scale,
+                             int batch_size, int rows, int words, int dim, int compact, void *stream);
+int faith_flag_below(const float *l, unsigned char *flags, int batch_size, long long per_batch, float bound,
+                     int strict, void *stream);
+int faith_verdict(const float *l, const float *u, const unsigned char *flags, unsigned char *safe,
+                  int batch_size, long long stride, int label, void *stream);
+
+/*
  * Layer normalisation without the variance (Bounds.layer_norm, Bounds.py:1111-1131, mode "no_var",
  * and the first step of mode "standard"): subtract the row mean -- the mean of the UPPER tensor
  * from the lower one and the reverse, as matmul(ones / H).multiply(-1.) gives it -- then scale by

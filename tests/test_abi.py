@@ -68,6 +68,12 @@ def test_null_and_shape_errors_are_status_codes(lib):
     # kernel larger than the padded image
     assert L.faith_convolution_verification(p, p, p, p, p, None, p, p, p, p, 1, 2, 2, 1, 1, 5, 1, 0, 1, None) == -2
     assert L.faith_tune_set(99, 1) == -3
+    # the driver's launches
+    assert L.faith_input_coefficients(None, p, None, 1.0, 1, 4, 1, 8, 0, None) == -1
+    assert L.faith_input_coefficients(p, None, None, 1.0, 1, 4, 1, 8, 0, None) == -1     # a dense object needs positions
+    assert L.faith_input_coefficients(p, None, None, 1.0, 1, 4, 1, 8, 1, None) == -2     # compact: one row per word
+    assert L.faith_flag_below(p, p, 0, 4, 0.0, 1, None) == -2
+    assert L.faith_verdict(p, p, None, None, 1, 1, 0, None) == -1
     # the allocation-free dot product refuses what its 4 MiB array cannot hold, before touching the GPU
     assert L.faith_static_scratch_bytes() == 4 << 20
     assert L.faith_dot_product_verification_QK_static(p, p, p, p, p, p, p, p, p, p, p, p,
