@@ -590,7 +590,7 @@ def bench_layer(args, wl):
     import time
     import torch
     from types import SimpleNamespace
-    from faith_amd import BoundsMaker, forward as F
+    from faith_amd import BoundsMaker, forward as F, ops
     hidden, heads, inter, length, eps, p = 256, 4, 512, 32, 0.01, 2.0
     g = torch.Generator().manual_seed(77)
     layer = wl.random_layer(g, hidden, heads, inter)
@@ -633,6 +633,18 @@ def bench_layer(args, wl):
                f"one perturbed word, p=2 (forward.verify_safety, wall clock)",
          "latency_us": round(statistics.median(times) * 1e3, 1), "latency_min_us": round(min(times) * 1e3, 1),
          "bound": "host", "achieved": 0.0, "peak": 1.0, "unit": "-", "frac": 0.0, "work": 0}
+    # the same query with the caller keeping every result buffer across calls (ops.Workspace): no allocation per call
+    ws = ops.Workspace()
+    kept = lambda: F.verify_safety(gmake, net, ge, 3, eps, 0, p, buffers=ws)
+    for _ in range(20):
+        kept()
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        kept()
+        times.append((time.perf_counter() - t0) * 1e3)
+    e["latency_us_with_persistent_buffers"] = round(statistics.median(times) * 1e3, 1)
+    del ws
     if not args.no_cpu:
         from tests.oracle_bounds import OracleBounds            # cpu_baseline leg only
         omake = lambda p_, e_, lw, lb, uw, ub: OracleBounds(p_, e_, lw, lb, uw, ub)

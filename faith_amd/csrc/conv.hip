@@ -396,20 +396,27 @@ conv_signsplit_k3s1(const ConvArgs g) {
 // rows of the image (TCB = 32: one row; 16: two rows of a 16-wide image, which a 32-column tile would fill by
 // half), and the workgroup's four wavefronts are WM x 4 / WM over (halves of 64 channels) x (pairs of pixel
 // blocks): WM = 2 is 128 channels x 4 blocks, WM = 1 is 64 channels x 8 blocks for layers of up to 64 channels.
-template <int K, int S, int CCH, bool WVEC, int TCB, int WM>
+// A wavefront holds MA x MB blocks (channels x pixels).  2 x 2 -- 128 accumulator registers, two wavefronts per
+// SIMD -- has the most reuse of what is read from LDS and suits long reductions.  A layer with a short reduction
+// is mostly the stream of its results; its workgroups fetch, multiply and store in phases, and with only two of them
+// on a CU the phases of the whole machine fall together (the MFMA pipe idles while everything stores).  1 x 2
+// blocks (64 accumulators) let four workgroups share a CU, whose phases then overlap.
+template <int K, int S, int CCH, bool WVEC, int TCB, int WM, int MA = 2, int MB = 2>
 struct FastTile {
     static constexpr int RPB = 32 / TCB;                 // image rows of one pixel block
-    static constexpr int NPB = 2 * (4 / WM);             // pixel blocks of a workgroup
-    static constexpr int ROWS = NPB * RPB, CHANNELS = 64 * WM;
+    static constexpr int NPB = MB * (4 / WM);            // pixel blocks of a workgroup
+    static constexpr int ROWS = NPB * RPB, CHANNELS = 32 * MA * WM;
+    static constexpr int WAVES = MA * MB == 4 ? 2 : 4;   // wavefronts per SIMD the register budget is set for
     static constexpr int KK = K * K, PROW = (ROWS - 1) * S + K, PCOL = (TCB - 1) * S + K, PP = PROW * PCOL;
     static constexpr int WS = (CCH * KK) | 1;
     static constexpr size_t LDS = ((size_t)4 * CCH * PP + (size_t)2 * CHANNELS * WS) * sizeof(float);
 };
 
-template <int K, int S, int CCH, bool WVEC, int TCB, int WM>
-__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int K, int S, int CCH, bool WVEC, int TCB, int WM, int MA = 2, int MB = 2>
+__global__ void __launch_bounds__(NTHREADS)
+    __attribute__((amdgpu_waves_per_eu(FastTile<K, S, CCH, WVEC, TCB, WM, MA, MB>::WAVES, FastTile<K, S, CCH, WVEC, TCB, WM, MA, MB>::WAVES)))
 conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
-    using T = FastTile<K, S, CCH, WVEC, TCB, WM>;
+    using T = FastTile<K, S, CCH, WVEC, TCB, WM, MA, MB>;
     constexpr int TCO = T::CHANNELS, TR = T::ROWS, TC = TCB, RPB = T::RPB;      // shadow the file-scope tile
     constexpr int KK = K * K, PROW = T::PROW, PCOL = T::PCOL, PP = T::PP;
     constexpr int WROW = CCH * KK;                       // floats of one weight row in a chunk
@@ -553,17 +560,17 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     using I1 = std::integral_constant<int, NW1>;
     using I2 = std::integral_constant<int, NW2>;
 
-    int xoff[2], woff[2];
+    int xoff[MB], woff[MA];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) xoff[b] = fh * (CCH / 2) * PP + (((wn * 2 + b) * RPB + fr) * S) * PCOL + fc * S;
+    for (int b = 0; b < MB; ++b) xoff[b] = fh * (CCH / 2) * PP + (((wn * MB + b) * RPB + fr) * S) * PCOL + fc * S;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) woff[a] = (wm * 64 + a * 32 + fi) * WS + fh * (CCH / 2) * KK;
+    for (int a = 0; a < MA; ++a) woff[a] = ((wm * MA + a) * 32 + fi) * WS + fh * (CCH / 2) * KK;
 
-    floatx16 cl[2][2], cu[2][2];
+    floatx16 cl[MA][MB], cu[MA][MB];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < MA; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < MB; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) cl[a][b][r] = cu[a][b][r] = 0.f;
 
@@ -576,21 +583,21 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
             for (int tap = 0; tap < KK; ++tap) {
                 const int xo = cp * PP + (tap / K) * PCOL + (tap % K);
                 const int wo = cp * KK + tap;
-                float wp[2], wq[2], xl[2], xu[2];            // w, |w|; centre and radius of x
+                float wp[MA], wq[MA], xl[MB], xu[MB];        // w, |w|; centre and radius of x
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
+                for (int a = 0; a < MA; ++a) {
                     wp[a] = bw[woff[a] + wo];
                     wq[a] = __builtin_fabsf(wp[a]);
                 }
 #pragma unroll
-                for (int b = 0; b < 2; ++b) {
+                for (int b = 0; b < MB; ++b) {
                     xl[b] = bl[xoff[b] + xo];
                     xu[b] = bu[xoff[b] + xo];
                 }
 #pragma unroll
-                for (int a = 0; a < 2; ++a)
+                for (int a = 0; a < MA; ++a)
 #pragma unroll
-                    for (int b = 0; b < 2; ++b) {
+                    for (int b = 0; b < MB; ++b) {
                         cl[a][b] = mfma(wp[a], xl[b], cl[a][b]);
                         cu[a][b] = mfma(wq[a], xu[b], cu[a][b]);
                     }
@@ -637,16 +644,16 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     const int wvu = __builtin_amdgcn_readfirstlane(wv);
     const int wmu = wvu / (4 / WM), wnu = wvu % (4 / WM);
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        const int row0 = oh0 + (wnu * 2 + b) * RPB;                  // first image row of this pixel block
+    for (int b = 0; b < MB; ++b) {
+        const int row0 = oh0 + (wnu * MB + b) * RPB;                 // first image row of this pixel block
         if (row0 >= g.Ho) continue;
         const bool inside = ow0 + fc < g.Wo && row0 + fr < g.Ho;
         const unsigned vo = inside ? (unsigned)(4 * fh) * plane_b + (unsigned)(fr * g.Wo + ow0 + fc) * 4u : 0x80000000u;
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < MA; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const unsigned so = (unsigned)(co0 + wmu * 64 + a * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
+                const unsigned so = (unsigned)(co0 + (wmu * MA + a) * 32 + 8 * (r / 4) + (r % 4)) * plane_b +
                                     (unsigned)(row0 * g.Wo) * 4u;
                 // y_l = centre - radius, y_u = centre + radius (the accumulators hold twice each)
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(0.5f * (cl[a][b][r] - cu[a][b][r])), wyl, vo, so, 2 /* non-temporal */);
@@ -658,20 +665,22 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     }
 }
 
-template <int K, int S, int CCH, bool WVEC, int TCB, int WM>
+template <int K, int S, int CCH, bool WVEC, int TCB, int WM, int MA = 2, int MB = 2>
 bool launch_tile(const ConvArgs &g, hipStream_t st) {
-    using T = FastTile<K, S, CCH, WVEC, TCB, WM>;
+    using T = FastTile<K, S, CCH, WVEC, TCB, WM, MA, MB>;
     static_assert(T::LDS <= 160 * 1024, "the two LDS stages of this instantiation do not fit a workgroup");
     const long long grid = (long long)g.N * ((g.Co + T::CHANNELS - 1) / T::CHANNELS) * ((g.Ho + T::ROWS - 1) / T::ROWS) *
                            ((g.Wo + TCB - 1) / TCB);
     if (grid > 0x7fffffffLL) return false;
-    if (!faith::reserve_lds(conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>, T::LDS)) return false;
-    const long long resident = 2LL * faith::compute_units();      // two workgroups per CU at most (registers)
+    if (!faith::reserve_lds(conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM, MA, MB>, T::LDS)) return false;
+    // workgroups a CU holds: one wavefront of each on every SIMD (registers), and their LDS
+    const long long by_lds = (160 * 1024) / (long long)T::LDS;
+    const long long resident = (by_lds < T::WAVES ? by_lds : T::WAVES) * faith::compute_units();
     const long long launched = grid < resident ? grid : resident;
     ConvArgs h = g;
     h.remap = (g.N % 8 == 0 && launched % 8 == 0 && faith::tune_get(FAITH_TUNE_CONV_VARIANT) != 2) ? 1 : 0;
-    hipLaunchKernelGGL((conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM>), dim3((unsigned)launched), dim3(NTHREADS), T::LDS, st, h,
-                       (int)grid);
+    hipLaunchKernelGGL((conv_signsplit_fast<K, S, CCH, WVEC, TCB, WM, MA, MB>), dim3((unsigned)launched), dim3(NTHREADS), T::LDS,
+                       st, h, (int)grid);
     return true;
 }
 
@@ -686,9 +695,26 @@ bool launch_fast(const ConvArgs &g, hipStream_t st) {
     return launch_tile<K, S, CCH, WVEC, 32, 2>(g, st);
 }
 
+// Layers whose reduction is short (at most 64 products per result: a 1 x 1 layer of up to 64 channels, the 3 x 3
+// first layer of an image classifier): 1 x 2 blocks per wavefront, four workgroups per CU (see FastTile) --
+// 64 channels x 4 pixel blocks, or 128 channels x 2 pixel blocks where the layer has that many channels (the
+// patch is then read once instead of twice).  Measured against 2 x 2 blocks: 1 x 1 64 -> 128 107 -> 96-99 us,
+// 1 x 1 32 -> 64 49 -> 41 us, 3 x 3 3 -> 64 45 -> 39-41 us; one block per wavefront was no faster than two.
+template <int K, int S, int CCH, bool WVEC>
+bool launch_brief(const ConvArgs &g, hipStream_t st) {
+    if ((g.Wo - 1) % 32 < 16) return launch_tile<K, S, CCH, WVEC, 16, 2, 1, 2>(g, st);
+    if ((g.Co - 1) % 128 >= 64) return launch_tile<K, S, CCH, WVEC, 32, 4, 1, 2>(g, st);
+    return launch_tile<K, S, CCH, WVEC, 32, 2, 1, 2>(g, st);
+}
+
 // The straight-line instantiation for this layer, if there is one: 3 x 3 at stride 1 or 2, 1 x 1, 5 x 5.
 bool dispatch_fast(const ConvArgs &g, bool wvec, hipStream_t st) {
     const int key = g.K * 10 + g.S;
+    const bool brief = g.Ci * g.K * g.K <= 64 && faith::tune_get(FAITH_TUNE_CONV_VARIANT) != 3;
+    if (brief) {
+        if (key == 11) return wvec ? launch_brief<1, 1, 16, true>(g, st) : launch_brief<1, 1, 16, false>(g, st);
+        if (key == 31 && !wvec) return launch_brief<3, 1, 4, false>(g, st);
+    }
     if (wvec) {
         switch (key) {
             case 31: return launch_fast<3, 1, 4, true>(g, st);      // layers that fill 128 x (4 x 32) tiles take the kernel above

@@ -60,7 +60,7 @@ int faith_version(void);
 #define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split GEMM: 1 = 64x64, 2 = 128x128, 3 = 128x64, 4 = 64x128, 5 = 32x32 with K split over the wavefronts (dim_out % 32 == 0); 6 = faith_matmul_concretize_verification takes its one-launch kernel whenever the shape allows; 7 = it keeps layer and concretize apart; 8 = as 6, with 32x32 blocks also where the reduction is short enough for 16x16 blocks */
 #define FAITH_TUNE_DOT_VARIANT   2   /* dot product: 1 = 128x64 persistent tiles with run-time extents (also where the straight-line instantiations for reductions of 32 / 64 / 128 would be taken), 2 = one 32x32 block per wavefront (short sequences only), 3 = transposed layout: the vector-ALU kernel also where the MFMA kernels apply */
 #define FAITH_TUNE_DOT_COORDS    3   /* dot product, 32x32 kernel: perturbation coordinates per wavefront, 1..16 */
-#define FAITH_TUNE_CONV_VARIANT  4   /* convolution: 1 = the general kernel (run-time extents) for every layer; 2 = tiles in the plain order (not whole images per XCD) */
+#define FAITH_TUNE_CONV_VARIANT  4   /* convolution: 1 = the general kernel (run-time extents) for every layer; 2 = tiles in the plain order (not whole images per XCD); 3 = 2 x 2 blocks per wavefront also for short reductions */
 #define FAITH_TUNE_COUNT         5
 int faith_tune_set(int knob, int value);
 

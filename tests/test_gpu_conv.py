@@ -135,6 +135,34 @@ def test_straight_line_conv_kernels_equal_the_general_kernel(case):
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("case", [
+    (6, 64, 128, 32, 32, 1, 1, 0),     # 1x1, 128-channel tiles (four wavefronts over the channels)
+    (8, 32, 64, 32, 32, 1, 1, 0),      # 1x1, 64-channel tiles, whole images per XCD
+    (300, 3, 64, 32, 32, 3, 1, 1),     # first layer; 2400 tiles: more than four per CU, so workgroups walk several
+    (3, 20, 100, 30, 30, 1, 1, 0),     # ragged: channels, rows and columns past the last full tile
+    (4, 16, 48, 16, 16, 1, 1, 0),      # 16-column pixel blocks
+    (2, 3, 200, 9, 70, 3, 1, 1),       # first layer, wide and short image, several channel tiles
+])
+def test_short_reductions_on_small_wavefront_tiles_equal_the_large_ones(case):
+    """Layers with at most 64 products per result run with 1 x 2 MFMA blocks per wavefront (four workgroups per CU)
+    instead of 2 x 2; the reduction order per result is the same, so the results are the same bits.  And against
+    the oracle."""
+    from faith_amd import _lib, ops
+    D, Ci, Co, Hh, Ww, K, s_, p = case
+    g = torch.Generator().manual_seed(47)
+    x = make(g, D, Ci, Hh, Ww, ordered=False)
+    W = torch.randn(Co, Ci, K, K, generator=g) * (2.0 / (Ci * K * K)) ** 0.5
+    bias = torch.randn(Co, generator=g)
+    got = check(x, W, bias, s_, p, "small wavefront tiles")
+    _lib.call("faith_tune_set", 4, 3)
+    try:
+        large = ops.conv2d(*(t.cuda() for t in x.tensors()), W.cuda(), bias.cuda(), s_, p)
+    finally:
+        _lib.call("faith_tune_set", 4, 0)
+    for name, a_, b_ in zip(("lw", "lb", "uw", "ub"), got, large):
+        assert torch.equal(a_, b_), name
+
+
 def test_conv_config4_reduced():
     """Benchmark configuration 4 with D_in = 8 instead of 256 (64 -> 128 channels, 32 x 32, 3x3)."""
     from faith_amd import ops
