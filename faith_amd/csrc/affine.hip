@@ -289,6 +289,30 @@ __global__ void __launch_bounds__(256) rows_put2(const float *__restrict__ a, co
     }
 }
 
+// out [B, L, W] = t [B, P, W] at the rows the positions name, zero elsewhere; VEC floats per thread.
+template <int VEC>
+__global__ void __launch_bounds__(256) rows_spread(const float *__restrict__ t, const long long *__restrict__ pos,
+                                                   float *__restrict__ out, const int L, const int P, const size_t W,
+                                                   const size_t n) {          // W, n in units of VEC floats
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+        const size_t bl = e / W, w = e % W;
+        const size_t bb = bl / L;
+        const long long l = (long long)(bl % L);
+        int slot = -1;
+        for (int p = 0; p < P; ++p)
+            if (pos[bb * P + p] == l) slot = p;
+        const size_t src = (bb * P + (slot >= 0 ? slot : 0)) * W + w;
+        if (VEC == 4) {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (slot >= 0) v = reinterpret_cast<const float4 *>(t)[src];
+            reinterpret_cast<float4 *>(out)[e] = v;
+        } else {
+            out[e] = slot >= 0 ? t[src] : 0.f;
+        }
+    }
+}
+
 bool all_aligned16(std::initializer_list<const void *> ptrs) {
     for (const void *p : ptrs)
         if (p != nullptr && !faith::aligned(p, 16)) return false;
@@ -430,4 +454,25 @@ extern "C" int faith_rows_put(const float *a, const float *b, const float *rows_
                        static_cast<hipStream_t>(stream), a, b, rows_a, rows_b, positions, out_a, out_b, length, n_positions,
                        dim_out, n);
     return faith::check_launch("faith_rows_put");
+}
+
+extern "C" int faith_rows_spread(const float *rows, const long long *positions, float *out, int batch_size, int length,
+                                 int n_positions, long long row_floats, void *stream) {
+    FAITH_NOT_NULL(rows); FAITH_NOT_NULL(positions); FAITH_NOT_NULL(out);
+    FAITH_ALIGNED4(rows); FAITH_ALIGNED4(out);
+    FAITH_REQUIRE(faith::aligned(positions, 8), FAITH_ERR_ALIGN, "faith_rows_spread: positions is not 8-byte aligned");
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && n_positions > 0 && row_floats > 0, FAITH_ERR_SHAPE,
+                  "faith_rows_spread: batch=%d length=%d positions=%d row_floats=%lld must be positive", batch_size, length,
+                  n_positions, row_floats);
+    const bool vec = row_floats % 4 == 0 && faith::aligned(rows, 16) && faith::aligned(out, 16);
+    const size_t W = vec ? (size_t)row_floats / 4 : (size_t)row_floats;
+    const size_t n = (size_t)batch_size * length * W;
+    const size_t blocks = (n + 255) / 256;
+    const dim3 gd((unsigned)(blocks < 262144 ? blocks : 262144)), bd(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (vec)
+        hipLaunchKernelGGL(rows_spread<4>, gd, bd, 0, st, rows, positions, out, length, n_positions, W, n);
+    else
+        hipLaunchKernelGGL(rows_spread<1>, gd, bd, 0, st, rows, positions, out, length, n_positions, W, n);
+    return faith::check_launch("faith_rows_spread");
 }

@@ -394,20 +394,19 @@ def layer_norm(lw, lb, uw, ub, weight=None, bias=None, other=None):
 
 def spread_positions(t, positions, length):
     """[B, P, ...] -> [B, length, ...]: row positions[b, i] of batch element b holds t[b, i], every other row
-    is zero.  positions: int64 [B, P] on t's device, distinct within a batch element.  A fill and an indexed copy
-    (nothing is computed); neither waits for the device, so both can be captured in a HIP graph."""
+    is zero (a position outside 0 ... length-1 names no row).  positions: int64 [B, P] on t's device, distinct
+    within a batch element.  One launch that writes the whole result; nothing is computed and nothing waits for
+    the device."""
+    _check("t", t)
     B, P = positions.shape
     if t.shape[:2] != (B, P):
         raise ValueError(f"t {tuple(t.shape)} does not start with positions' shape {(B, P)}")
-    out = zeros(B, length, *t.shape[2:], device=t.device)
-    key = (B, str(t.device))
-    if key not in _BATCH_INDEX:
-        _BATCH_INDEX[key] = torch.arange(B, device=t.device)[:, None]
-    out[_BATCH_INDEX[key], positions] = t
+    if not (positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous()):
+        raise ValueError("positions: expected a contiguous int64 GPU tensor")
+    out = _empty(B, length, *t.shape[2:], device=t.device)
+    with _on(t.device):
+        _lib.call("faith_rows_spread", _ptr(t), _ptr(positions), _ptr(out), B, length, P, t.numel() // (B * P), _stream(t))
     return out
-
-
-_BATCH_INDEX = {}
 
 
 def zeros(*shape, device):

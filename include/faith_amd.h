@@ -220,12 +220,16 @@ int faith_rowmean_verification(const float *src_lb, const float *src_ub,
  * positions (zero for a position that names no row).  faith_rows_put: out_a, out_b [batch, length, dim_out] = a, b
  * with the rows at the positions replaced by rows_a, rows_b [batch, n_positions, dim_out].  Two tensors a launch:
  * the lower and the upper constants / intervals always travel together.  out_* must not overlap the inputs.
+ * faith_rows_spread: out [batch, length, row_floats] = rows [batch, n_positions, row_floats] at the positions and
+ * zero everywhere else -- the object with its zeros written out (row_floats = dim_in * dim_out for coefficient rows).
  */
 int faith_rows_gather(const float *a, const float *b, const long long *positions, float *out_a, float *out_b,
                       int batch_size, int length, int n_positions, int dim_out, void *stream);
 int faith_rows_put(const float *a, const float *b, const float *rows_a, const float *rows_b,
                    const long long *positions, float *out_a, float *out_b,
                    int batch_size, int length, int n_positions, int dim_out, void *stream);
+int faith_rows_spread(const float *rows, const long long *positions, float *out,
+                      int batch_size, int length, int n_positions, long long row_floats, void *stream);
 
 /*
  * The layer driver's own device work, one launch each where the reference evaluates three or four tensor

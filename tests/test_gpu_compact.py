@@ -498,3 +498,25 @@ def test_rows_of_a_compact_object_are_gathered_and_put_back_by_the_library():
                 fa[i, l], fb[i, l] = ra[i, j], rb[i, j]
     assert torch.equal(ga.cpu(), ea) and torch.equal(gb.cpu(), eb)
     assert torch.equal(pa.cpu(), fa) and torch.equal(pb.cpu(), fb)
+
+
+@pytest.mark.parametrize("shape", [(3, 2, 7, 5, 8), (2, 1, 4, 3, 6), (1, 3, 9, 2, 5)])
+def test_rows_are_spread_into_the_written_out_object_by_the_library(shape):
+    """faith_rows_spread against a fill and an indexed copy on the CPU (16-byte and 4-byte rows); a position outside
+    the sentence names no row."""
+    from faith_amd import ops
+    B, P, L, D, H = shape
+    g = torch.Generator().manual_seed(141)
+    t = torch.randn(B, P, D, H, generator=g)
+    positions = torch.stack([torch.randperm(L, generator=g)[:P] for _ in range(B)])
+    if B > 1:
+        positions[1, 0] = L + 3
+    got = ops.spread_positions(t.cuda(), positions.cuda(), L)
+    const = ops.spread_positions(t[:, :, 0].contiguous().cuda(), positions.cuda(), L)      # [B, P, H] rows
+    torch.cuda.synchronize()
+    want = torch.zeros(B, L, D, H)
+    for i in range(B):
+        for j in range(P):
+            if 0 <= int(positions[i, j]) < L:
+                want[i, int(positions[i, j])] = t[i, j]
+    assert torch.equal(got.cpu(), want) and torch.equal(const.cpu(), want[:, :, 0])
