@@ -518,7 +518,8 @@ constexpr int SB = 32;                         // block edge
 // Its y terms, sum_k b(i, k) y(k, m, j), then have one addend per such position: no y fragments, no P and Q
 // accumulators; the addends are formed from b in LDS and the lane's column of the compact rows when the block is stored.
 template <bool VP, bool RAGGED = false, bool COMPACT_Y = false>
-__global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mpw, const int heads_first, const int w_tiles) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(COMPACT_Y ? 4 : 3, COMPACT_Y ? 4 : 3)))
+dot_w_small(const DotArgs g, const int mpw, const int heads_first, const int w_tiles) {
     static_assert(VP || !RAGGED, "a ragged reduction exists on the context path only");
     static_assert(VP || !COMPACT_Y, "compact value operands exist on the context path only");
     extern __shared__ __align__(16) float sh[];   // six operands, each d/8 swizzled [32 x 8] pieces (or a constant-term tile)
@@ -674,8 +675,8 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
         }
         // register r is row 8*(r/4) + 4*(lane/32) + r%4 of the block, lanes run along j
         if (COMPACT_Y) {
-            // cp, cq (zero so far) take the y terms as 2 (b+ y_lw + b- y_uw) and 2 (b+ y_uw + b- y_lw) in the places
-            // of P + Q and P - Q: one addend per key position that has coefficients
+            // the y terms, b+ y_lw + b- y_uw and b+ y_uw + b- y_lw, have one addend per key position that has
+            // coefficients: b from the staged tile, the lane's column of the compact row; added to the x terms in place
             const int yb = t / g.oy.heads, yh = t - yb * g.oy.heads;
             for (int p = 0; p < g.yP; ++p) {
                 const long long kp = g.y_positions[(size_t)yb * g.yP + p];
@@ -683,30 +684,38 @@ __global__ void __launch_bounds__(256) dot_w_small(const DotArgs g, const int mp
                 const int kk = (int)kp;
                 const size_t o = (((size_t)yb * g.yP + p) * g.D + m) * g.oy.pitch + (size_t)yh * g.oy.width + jcol;
                 const float vl = g.ylw[o], vu = g.yuw[o];
+                // row 8*(r/4) + 4*fh + r%4 of piece kk/8: bit 2 of the row is fh, so the swizzle is the lane's own
+                const float *bsrc = s_bp + (kk / 8) * (SB * 8) + 32 * fh + 4 * (((kk % 8) / 4) ^ fh) + kk % 4;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int row = 8 * (r / 4) + 4 * fh + (r % 4);
-                    const float bt = s_bp[(kk / 8) * (SB * 8) + swz(row, (kk % 8) / 4) + kk % 4];
+                    const float bt = bsrc[(8 * (r / 4) + (r % 4)) * 8];
                     const float bp = fmaxf(bt, 0.f), bn = fminf(bt, 0.f);
-                    cp[r] += bp * vl + bn * vu;
-                    cq[r] += bp * vu + bn * vl;
+                    cl[r] += bp * vl + bn * vu;
+                    cu[r] += bp * vu + bn * vl;
                 }
             }
-        }
-        if (j0 + fi < g.Ly) {
+        } else {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int i = i0 + 8 * (r / 4) + 4 * fh + (r % 4);
-                if (i < g.Lx) {
-                    const size_t o = zw0 + ((size_t)i * g.D + m) * g.oz.pitch + j0 + fi;
-                    if (COMPACT_Y) {
-                        __builtin_nontemporal_store(cl[r] + cp[r], &g.zlw[o]);
-                        __builtin_nontemporal_store(cu[r] + cq[r], &g.zuw[o]);
-                    } else {
-                        __builtin_nontemporal_store(cl[r] + 0.5f * (cp[r] + cq[r]), &g.zlw[o]);
-                        __builtin_nontemporal_store(cu[r] + 0.5f * (cp[r] - cq[r]), &g.zuw[o]);
-                    }
-                }
+                const float pp = cp[r], qq_ = cq[r];
+                cl[r] += 0.5f * (pp + qq_);
+                cu[r] += 0.5f * (pp - qq_);
+            }
+        }
+        // Buffer stores: the window is this block's rows of z at coordinate m (it ends behind the last row that exists),
+        // a register's row is a wave-uniform offset, the lane's offset is fixed; a lane without a column is sent outside.
+        {
+            const size_t z0 = zw0 + ((size_t)i0 * g.D + m) * g.oz.pitch + j0;
+            const unsigned row_b = (unsigned)g.D * g.oz.pitch * 4u;                 // one row i, bytes
+            const int rows_here = min(SB, g.Lx - i0);
+            const unsigned bytes = (unsigned)(rows_here - 1) * row_b + (unsigned)min(SB, g.Ly - j0) * 4u;   // <= rows_here * row_b
+            const __amdgpu_buffer_rsrc_t wzl = window(g.zlw + z0, bytes), wzu = window(g.zuw + z0, bytes);
+            const unsigned vo = j0 + fi < g.Ly ? (unsigned)(4 * fh) * row_b + (unsigned)fi * 4u : 0x80000000u;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const unsigned so = (unsigned)(8 * (r / 4) + (r % 4)) * row_b;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cl[r]), wzl, vo, so, 2 /* non-temporal */);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(cu[r]), wzu, vo, so, 2);
             }
         }
     }
