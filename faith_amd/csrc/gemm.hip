@@ -152,7 +152,10 @@ __device__ __forceinline__ void signsplit_gemm_tile(const GemmArgs &g, float *sm
     // piece kq of rows r0 (and r0 + 64).  Offsets are relative to the first row of the tile (the entry
     // point checks that a tile's rows span less than 4 GB); rows past the end re-read the last row, their
     // products are never stored.
-    const int kq = tid % 4, r0 = tid / 4;
+    // (the two pieces of a row that belong to the K-step's second half are taken by the threads two rows away: the
+    // eight lanes whose 16-byte stores the LDS serves in one cycle then write rows 0, 1 of the first half and rows
+    // 2, 3 of the second -- eight different groups of banks -- instead of rows 0, 1 of both)
+    const int kq = tid % 4, r0 = (tid / 4) ^ (kq & 2);
     const __amdgpu_buffer_rsrc_t wal = window(g.Al + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
     const __amdgpu_buffer_rsrc_t wau = window(g.Au + (size_t)m0 * K, ((size_t)(M - m0) * K) * 4);
     const __amdgpu_buffer_rsrc_t ww = window(g.W + (size_t)n0 * K, ((size_t)(g.N - n0) * K) * 4);
