@@ -58,6 +58,19 @@ class Bounds:
     def _c(self):
         return (self.lw.contiguous(), self.lb.contiguous(), self.uw.contiguous(), self.ub.contiguous())
 
+    def first_position(self):
+        """The bounds of position 0 alone, [B, 1, ...] (what VerifierForward._bound_pooling, :269-287, slices out).
+        One batch element: views.  Several: the rows are strided, so they are gathered -- a launch per pair of
+        tensors instead of a strided copy per tensor."""
+        if self.batch_size == 1:
+            return self._like(self.lw[:, :1], self.lb[:, :1], self.uw[:, :1], self.ub[:, :1])
+        lw, lb, uw, ub = self._c()
+        B, L, D, H = lw.shape
+        at = ops.positions_tensor([[0]] * B, lw.device)
+        flw, fuw = ops.gather_positions(lw.view(B, L, D * H), uw.view(B, L, D * H), at)
+        flb, fub = ops.gather_positions(lb, ub, at)
+        return self._like(flw.view(B, 1, D, H), flb, fuw.view(B, 1, D, H), fub)
+
     def _interval(self, kind):
         """method "ibp": the operator applied to the concrete interval; coefficients are zero
         (the `if self.ibp` branches of Bounds.py:863-866, :896-898, :924-926, :973-975, :1030-1032, :1139-1143)."""

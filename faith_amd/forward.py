@@ -240,6 +240,9 @@ def bound_layer(bounds_input, layer, layer_norm="no_var", hidden_act="relu", wan
 
 def bound_pooling(bounds, pooler_dense, make_bounds):
     """VerifierForward._bound_pooling: first position, dense, tanh."""
+    own = getattr(bounds, "first_position", None)
+    if own is not None:
+        return own().dense(pooler_dense).tanh()
     first = make_bounds(bounds.p, bounds.eps, bounds.lw[:, :1], bounds.lb[:, :1], bounds.uw[:, :1], bounds.ub[:, :1])
     return first.dense(pooler_dense).tanh()
 
