@@ -20,12 +20,23 @@ What can be tuned (see the FAITH_TUNE_* knobs in include/faith_amd.h):
 Results are kept in a TuningTable keyed by (operator, shape); `use(table)` makes the wrappers in
 faith_amd.ops apply an entry around the matching launch.  Results never depend on the variant, only
 speed does.
+
+Beyond the variants the library ships, `autotune_generated` runs the reference's loop as it is: a variant of the
+GEMM's MFMA kernel -- tile shape, register budget, wavefront priority, i.e. what matmul_config.h holds there -- is
+GENERATED as macros, COMPILED with hipcc into a small library of its own (csrc/variants/gemm_variant.hip, a few
+seconds), loaded, checked against the shipped kernel bit for bit and measured; the table then names the compiled
+library and faith_amd.ops.linear sends the coefficient rows of that shape through it.
 """
 from __future__ import annotations
 
 import contextlib
+import ctypes
+import hashlib
 import json
+import os
 import random
+import shutil
+import subprocess
 from dataclasses import dataclass, field
 
 import numpy as np
@@ -311,6 +322,184 @@ def autotune(op, shape, run, heuristics=None, rounds=3, samples=3, measure=None,
     return result
 
 
+# ------------------------------------------------------------------------------------------
+# Generated variants: generate -> compile -> load -> measure (autotuner.py:99-147 with
+# utils.py's rewrite-and-rebuild step; here the rebuilt unit is one translation unit, not the extension)
+# ------------------------------------------------------------------------------------------
+_HERE = os.path.dirname(os.path.abspath(__file__))
+VARIANT_SOURCE = os.path.join(_HERE, "csrc", "variants", "gemm_variant.hip")
+
+
+@dataclass(frozen=True)
+class GemmVariantSpec:
+    """What one generated GEMM kernel is compiled with: 32 x 32 MFMA blocks per wavefront along M and N (the
+    macro-tile is 64 mbm x 64 mbn), wavefronts per SIMD the register budget is set for, raised wavefront priority
+    during a run of MFMAs."""
+    mbm: int
+    mbn: int
+    waves: int
+    setprio: int
+
+    def macros(self):
+        return {"FAITH_V_MBM": self.mbm, "FAITH_V_MBN": self.mbn, "FAITH_V_WAVES": self.waves,
+                "FAITH_GEMM_SETPRIO": self.setprio}
+
+    def lds_bytes(self):
+        return 2 * (4 * 64 * self.mbm * 8 + 4 * 64 * self.mbn * 8) * 4
+
+    def registers(self):
+        return 2 * 16 * self.mbm * self.mbn + 8 * (self.mbm + self.mbn) + 40     # accumulators, fragments, the rest
+
+    def name(self):
+        return f"gemm_{64 * self.mbm}x{64 * self.mbn}_w{self.waves}_p{self.setprio}"
+
+
+def gemm_variant_space(metafile=None):
+    """Every variant the tile code can express and the part can hold: the accumulators of both operands fit a
+    wavefront's share of the registers at the asked-for occupancy, the two LDS stages fit a workgroup."""
+    meta = dict(mi355x_metafile, **(metafile or {}))
+    out = []
+    for mbm in (1, 2, 3, 4):
+        for mbn in (1, 2, 3, 4):
+            if mbm * mbn > 4:
+                continue
+            for waves in (1, 2, 3, 4):
+                for setprio in (0, 1):
+                    v = GemmVariantSpec(mbm, mbn, waves, setprio)
+                    if v.lds_bytes() > meta["MAX_LDS_KB"] * 1024:
+                        continue
+                    if v.registers() > meta["MAX_NUM_REGISTER_PER_LANE"] // waves:
+                        continue
+                    out.append(v)
+    return out
+
+
+def compile_gemm_variant(spec, out_dir, hipcc="hipcc", arch="gfx950"):
+    """Compiles the variant into out_dir and returns the library's path (an existing build of the same source and
+    macros is reused).  Needs hipcc; a GPU is not needed to build."""
+    if shutil.which(hipcc) is None:
+        raise RuntimeError(f"{hipcc} not found: generated variants are compiled on the machine that tunes")
+    os.makedirs(out_dir, exist_ok=True)
+    src = open(VARIANT_SOURCE, "rb").read() + open(os.path.join(_HERE, "csrc", "gemm_tile.h"), "rb").read()
+    tag = hashlib.sha256(src + json.dumps(spec.macros(), sort_keys=True).encode()).hexdigest()[:12]
+    path = os.path.join(out_dir, f"libfaith_{spec.name()}_{tag}.so")
+    if os.path.exists(path):
+        return path
+    from .build import COMMON
+    cmd = [hipcc, *COMMON, *[f"-D{k}={v}" for k, v in spec.macros().items()], "-shared", VARIANT_SOURCE,
+           os.path.join(_HERE, "csrc", "common.hip"), "-o", path + ".tmp"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {spec.name()}:\n{r.stderr[-2000:]}")
+    os.replace(path + ".tmp", path)
+    return path
+
+
+class GeneratedGemm:
+    """A compiled variant, loaded.  coefficients(...) multiplies the coefficient rows of a layer; the constant
+    rows stay with the library's exact-accumulation kernel (faith_matmul_rows_verification with no coefficient
+    rows)."""
+
+    def __init__(self, path):
+        self.path = path
+        self.lib = ctypes.CDLL(path)
+        P, I = ctypes.c_void_p, ctypes.c_int
+        self.lib.faith_variant_matmul_coefficients.argtypes = [P] * 5 + [ctypes.c_longlong, I, I, P]
+        self.lib.faith_variant_matmul_coefficients.restype = I
+        self.lib.faith_last_error.restype = ctypes.c_char_p
+        self.lib.faith_variant_lds_bytes.restype = I
+
+    def coefficients(self, lw, uw, weight, olw, ouw, stream):
+        rows = lw.numel() // lw.shape[-1]
+        rc = self.lib.faith_variant_matmul_coefficients(lw.data_ptr(), uw.data_ptr(), weight.data_ptr(), olw.data_ptr(),
+                                                        ouw.data_ptr(), rows, lw.shape[-1], weight.shape[0], stream)
+        if rc != 0:
+            from ._lib import FaithError
+            raise FaithError("faith_variant_matmul_coefficients", rc, self.lib.faith_last_error().decode())
+
+
+_LOADED = {}
+
+
+def load_generated(path):
+    g = _LOADED.get(path)
+    if g is None:
+        g = _LOADED[path] = GeneratedGemm(path)
+    return g
+
+
+def autotune_generated(shape, lw, uw, weight, out_dir, specs=None, rounds=3, samples=4, measure=None, seed=0,
+                       compile_variant=compile_gemm_variant):
+    """The generate-and-recompile loop for the coefficient rows of `linear` at shape = (rows, K, N):
+    lw, uw [..., K] and weight [N, K] are the operands to measure on (GPU tensors).
+
+    Round 0 compiles and measures `samples` specs drawn at random, later rounds the `samples` unmeasured specs the
+    cost model (fitted on what has been measured) ranks fastest.  The shipped kernel is measured first and a
+    generated variant is only kept if it is faster AND reproduces the shipped kernel's coefficient rows bit for bit
+    (the order of summation does not depend on the tile).  Returns (TuningResult, path of the best library or
+    None if the shipped kernel stays)."""
+    import torch
+    from . import ops
+    measure = measure or measure_on_gpu
+    rng = random.Random(seed)
+    pool = list(specs) if specs is not None else gemm_variant_space()
+    rows, K, N = (int(v) for v in shape)
+    x_lw, x_uw = lw.reshape(1, 1, rows, K), uw.reshape(1, 1, rows, K)
+    zeros_b = torch.zeros(1, 1, K, device=lw.device)
+    ref = ops.linear(x_lw, zeros_b, x_uw, zeros_b, weight)
+    olw, ouw = torch.empty_like(ref[0]), torch.empty_like(ref[2])
+    stream = torch.cuda.current_stream(lw.device).cuda_stream
+    result = TuningResult("linear", (rows, K, N), None, float("inf"))
+    builtin = Candidate((), (("builtin", 1.0),))
+    out4 = (ref[0], ref[1], ref[2], ref[3])
+    shipped = lambda: ops.linear(x_lw, zeros_b, x_uw, zeros_b, weight, out=out4)
+    measure(shipped)                                    # discarded: clocks
+    result.best, result.best_us = builtin, measure(shipped)
+    result.measured.append((builtin, result.best_us))
+    best_path = None
+    seen = set()
+
+    def feats(v):
+        tiles = -(-rows // (64 * v.mbm)) * -(-N // (64 * v.mbn))
+        resident = max(1, min(v.waves, (160 * 1024) // v.lds_bytes())) * mi355x_metafile["COMPUTE_UNITS"]
+        return [1.0, v.mbm, v.mbn, v.mbm * v.mbn, v.waves, v.setprio, np.log(tiles), np.ceil(tiles / resident)]
+
+    def take(v):
+        nonlocal best_path
+        seen.add(v)
+        try:
+            g = load_generated(compile_variant(v, out_dir))
+            run = lambda: g.coefficients(x_lw, x_uw, weight, olw, ouw, stream)
+            run()
+            torch.cuda.synchronize(lw.device)
+            if not (torch.equal(olw, ref[0]) and torch.equal(ouw, ref[2])):
+                raise RuntimeError("results differ from the shipped kernel's")
+            us = measure(run)
+        except Exception:
+            result.skipped += 1
+            return
+        cand = _cand({}, **{k.lower(): float(val) for k, val in v.macros().items()})
+        result.measured.append((cand, us))
+        spec_of[cand] = v
+        if us < result.best_us:
+            result.best, result.best_us, best_path = cand, us, g.path
+
+    spec_of = {}
+    for r in range(rounds):
+        rest = [v for v in pool if v not in seen]
+        if not rest:
+            break
+        fitted = [(spec_of[c], us) for c, us in result.measured if c in spec_of]
+        if r == 0 or len(fitted) < 3:
+            chosen = rng.sample(rest, min(samples, len(rest)))
+        else:
+            model = CostModel().fit([feats(v) for v, _ in fitted], [us for _, us in fitted])
+            chosen = sorted(rest, key=lambda v: float(model.predict([feats(v)])[0]))[:samples]
+        for v in chosen:
+            take(v)
+    return result, best_path
+
+
 class TuningTable:
     """(operator, shape) -> knob settings; JSON on disk."""
 
@@ -327,9 +516,20 @@ class TuningTable:
             "microseconds": round(result.best_us, 2),
             "measured": len(result.measured)}
 
+    def record_generated(self, result, path):
+        """The outcome of autotune_generated: the compiled library for this shape, or the shipped kernel."""
+        self.entries[self.key(result.op, result.shape)] = {
+            "knobs": {}, "microseconds": round(result.best_us, 2), "measured": len(result.measured),
+            **({"generated": path} if path else {})}
+
     def lookup(self, op, shape):
         e = self.entries.get(self.key(op, shape))
         return None if e is None else {int(k): int(v) for k, v in e["knobs"].items()}
+
+    def generated(self, op, shape):
+        """Path of the compiled variant recorded for (op, shape), or None."""
+        e = self.entries.get(self.key(op, shape))
+        return None if e is None else e.get("generated")
 
     def save(self, path):
         with open(path, "w") as f:

@@ -78,5 +78,24 @@ def build(force: bool = False, verbose: bool = True) -> str:
     return LIB
 
 
+VARIANTS = os.path.join(HERE, "variants")
+# GEMM kernel variants built ahead of time for the generate-and-recompile tuner (faith_amd.autotune): tile shapes
+# the library does not ship -- (MFMA blocks per wavefront along M, along N, wavefronts per SIMD, raised priority) --
+# so that a tuning run on a machine without a compiler, or one that must not compile, still has generated variants
+# to measure; the tuner compiles any other point of its space on demand.
+PREBUILT_VARIANTS = [(4, 1, 2, 0), (1, 4, 2, 0), (3, 1, 2, 0), (1, 3, 2, 1), (2, 2, 2, 0), (2, 1, 3, 0), (1, 2, 3, 1), (1, 1, 4, 1)]
+
+
+def build_variants(verbose: bool = True):
+    """Compiles PREBUILT_VARIANTS into faith_amd/variants/ (existing builds of the same source are kept)."""
+    from .autotune import GemmVariantSpec, compile_gemm_variant
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        paths = list(ex.map(lambda v: compile_gemm_variant(GemmVariantSpec(*v), VARIANTS), PREBUILT_VARIANTS))
+    if verbose:
+        print(f"built {len(paths)} GEMM variants in {VARIANTS}")
+    return paths
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
+    build_variants()

@@ -479,6 +479,16 @@ def linear(lw, lb, uw, ub, weight, bias=None, out=None):
         olw, olb, ouw, oub = out
         _check("out lw", olw, (B, L, D, N)); _check("out uw", ouw, (B, L, D, N))
         _check("out lb", olb, (B, L, N)); _check("out ub", oub, (B, L, N))
+    if autotune._ACTIVE is not None:
+        generated = autotune._ACTIVE.generated("linear", (B * L * D, H, N))
+        if generated is not None:
+            # a variant compiled by the tuner for this shape takes the coefficient rows; the constant rows stay with
+            # the library's exact-accumulation kernel
+            with _on(lw.device):
+                autotune.load_generated(generated).coefficients(lw, uw, weight, olw, ouw, _stream(lw))
+                _lib.call("faith_matmul_rows_verification", _ptr(lb), _ptr(ub), None, None, _ptr(weight), _ptr(bias),
+                          _ptr(olb), _ptr(oub), None, None, 0, B * L, H, N, _stream(lw))
+            return olw, olb, ouw, oub
     with _on(lw.device, "linear", (B * L * D, H, weight.shape[0])):
         _lib.call("faith_matmul_verification", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(weight), _ptr(bias),
                   _ptr(olb), _ptr(oub), _ptr(olw), _ptr(ouw), B, L, D, H, N, _stream(lw))

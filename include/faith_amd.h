@@ -395,6 +395,9 @@ int faith_matmul_group_verification(const float *x_lb, const float *x_ub,
  * [rows_w, dim_y_out]; x_lb, x_ub [rows_b, dim_out] -> y_lb, y_ub [rows_b, dim_y_out].  An ordinary
  * object has rows_w = rows_b * dim_in; one that keeps the coefficients of a few positions only
  * (VerifierForward.py:127-156 builds such an input: zero rows everywhere else) has fewer.
+ * faith_matmul_rows_verification with rows_w = 0 multiplies the constant rows alone (x_lw, x_uw, y_lw, y_uw are
+ * then not read and may be NULL): for a caller whose coefficient rows go through a kernel variant of its own
+ * (faith_amd.autotune's generated variants).
  */
 int faith_matmul_rows_verification(const float *x_lb, const float *x_ub,
                                    const float *x_lw, const float *x_uw,

@@ -194,3 +194,108 @@ def test_dot_variants_agree_and_tuning_is_never_slower_than_the_default():
         A.use(None)
     for a, b in zip(tuned, base):
         assert close(a, b, rtol=1e-5, atol=2e-6)
+
+
+# ------------------------------------------------------------------ generated variants (generate -> compile -> measure)
+def _prebuilt_only(spec, out_dir):
+    """compile_variant stand-in for GPU runs: the library built ahead of time, never a compiler run."""
+    import glob
+    import os
+    found = glob.glob(os.path.join(out_dir, f"libfaith_{spec.name()}_*.so"))
+    if not found:
+        raise FileNotFoundError(spec.name())
+    return found[0]
+
+
+def test_generated_variant_space_respects_registers_and_lds():
+    space = A.gemm_variant_space()
+    assert len(space) == len(set(space)) and len(space) > 30
+    for v in space:
+        assert v.mbm * v.mbn <= 4 and v.lds_bytes() <= 160 * 1024
+        assert v.registers() * v.waves <= 512
+    names = {v.name() for v in space}
+    assert "gemm_256x64_w2_p0" in names and "gemm_64x256_w2_p1" in names      # shapes the library does not ship
+    assert "gemm_128x128_w3_p0" not in names                                    # 128 accumulators + the rest: two per SIMD
+    # a part with a quarter of the LDS loses the large tiles
+    small = A.gemm_variant_space({"MAX_LDS_KB": 40})
+    assert {(v.mbm, v.mbn) for v in small} == {(1, 1)}
+
+
+def test_a_generated_variant_compiles_loads_and_validates_without_a_gpu(tmp_path):
+    """The compile step of the loop: macros -> hipcc -> a library of its own (reused when the source and the macros
+    are unchanged) whose entry point validates like the library's (status codes, nothing launched)."""
+    import ctypes
+    import os
+    import shutil
+    if shutil.which("hipcc") is None:
+        pytest.skip("no hipcc")
+    from faith_amd import build as B
+    spec = A.GemmVariantSpec(*B.PREBUILT_VARIANTS[0])
+    path = A.compile_gemm_variant(spec, B.VARIANTS)
+    assert os.path.exists(path) and A.compile_gemm_variant(spec, B.VARIANTS) == path
+    g = A.load_generated(path)
+    assert g.lib.faith_variant_lds_bytes() == spec.lds_bytes()
+    buf = (ctypes.c_float * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    f = g.lib.faith_variant_matmul_coefficients
+    assert f(None, p, p, p, p, 4, 16, 16, None) == -1
+    assert f(p, p, p, p, p, 0, 16, 16, None) == -2
+    assert f(p, p, p, p, p, 4, 6, 16, None) == -3 and b"dim_out" in g.lib.faith_last_error()
+    # a different macro set is a different library
+    other = A.GemmVariantSpec(spec.mbm, spec.mbn, spec.waves, 1 - spec.setprio)
+    assert other.name() != spec.name() and other.macros() != spec.macros()
+
+
+def test_tuning_table_keeps_generated_entries(tmp_path):
+    res = A.TuningResult("linear", (8192, 256, 192), A.Candidate((), (("builtin", 1.0),)), 12.5, [(None, 12.5)] * 3)
+    t = A.TuningTable()
+    t.record_generated(res, "/somewhere/libfaith_gemm_256x64_w2_p0_abc.so")
+    t.record_generated(A.TuningResult("linear", (64, 64, 64), None, 3.0), None)       # the shipped kernel stayed
+    t.save(tmp_path / "t.json")
+    back = A.TuningTable.load(tmp_path / "t.json")
+    assert back.generated("linear", (8192, 256, 192)).endswith("_abc.so")
+    assert back.generated("linear", (64, 64, 64)) is None and back.generated("linear", (1, 2, 3)) is None
+    assert back.lookup("linear", (8192, 256, 192)) == {}
+
+
+@pytest.mark.gpu
+def test_generate_compile_measure_loop_for_the_gemm():
+    """The reference's loop on this part: generated variants of the GEMM kernel (built ahead of time here: a GPU run
+    does not compile) are loaded, held to the shipped kernel's coefficient rows bit for bit and measured; the
+    table entry then routes ops.linear through the chosen library."""
+    from faith_amd import build as B, ops
+    from tests.helpers import close
+    x, W, bias = _linear_case(77, 64, 128, 256, 192)                  # 8192 coefficient rows, K = 256, N = 192
+    lw, lb, uw, ub = x
+    base = ops.linear(lw, lb, uw, ub, W, bias)
+    specs = [A.GemmVariantSpec(*v) for v in B.PREBUILT_VARIANTS]
+    res, path = A.autotune_generated((64 * 128, 256, 192), lw, uw, W, B.VARIANTS, specs=specs, rounds=2, samples=4,
+                                     compile_variant=_prebuilt_only)
+    print(f"[case] generated GEMM variants: shipped {res.measured[0][1]:.1f} us, best {res.best_us:.1f} us "
+          f"({'shipped' if path is None else path.split('/')[-1]}), {len(res.measured) - 1} variants measured", flush=True)
+    assert res.skipped == 0 and len(res.measured) == 9                 # the shipped kernel + eight variants
+    assert res.best_us <= res.measured[0][1]
+    # every variant through the table, whether or not it won
+    for spec in specs:
+        table = A.TuningTable()
+        table.record_generated(res, _prebuilt_only(spec, B.VARIANTS))
+        A.use(table)
+        try:
+            got = ops.linear(lw, lb, uw, ub, W, bias)
+        finally:
+            A.use(None)
+        assert torch.equal(got[0], base[0]) and torch.equal(got[2], base[2]), spec.name()
+        # constant rows: the exact-accumulation kernel alone instead of its tiles inside the MFMA launch
+        assert close(got[1], base[1].cpu(), rtol=1e-6, atol=1e-7) and close(got[3], base[3].cpu(), rtol=1e-6, atol=1e-7)
+    # a reduction that is no multiple of 16, ragged rows and columns
+    x2, W2, b2 = _linear_case(78, 3, 50, 36, 72)
+    base2 = ops.linear(*x2, W2, b2)
+    for spec in specs[:3]:
+        table = A.TuningTable()
+        table.record_generated(A.TuningResult("linear", (150, 36, 72), None, 1.0), _prebuilt_only(spec, B.VARIANTS))
+        A.use(table)
+        try:
+            got = ops.linear(*x2, W2, b2)
+        finally:
+            A.use(None)
+        assert torch.equal(got[0], base2[0]) and torch.equal(got[2], base2[2]), spec.name()
