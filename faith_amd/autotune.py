@@ -435,11 +435,12 @@ def autotune_generated(shape, lw, uw, weight, out_dir, specs=None, rounds=3, sam
 
     Round 0 compiles and measures `samples` specs drawn at random, later rounds the `samples` unmeasured specs the
     cost model (fitted on what has been measured) ranks fastest.  The shipped kernel is measured first and a
-    generated variant is only kept if it is faster AND reproduces the shipped kernel's coefficient rows bit for bit
-    (the order of summation does not depend on the tile).  Returns (TuningResult, path of the best library or
+    generated variant is only kept if it is faster -- measured as ops.linear would run it, the launch for the
+    constant rows included -- AND reproduces the shipped kernel's coefficient rows bit for bit (the order of
+    summation does not depend on the tile).  Returns (TuningResult, path of the best library or
     None if the shipped kernel stays)."""
     import torch
-    from . import ops
+    from . import _lib, ops
     measure = measure or measure_on_gpu
     rng = random.Random(seed)
     pool = list(specs) if specs is not None else gemm_variant_space()
@@ -469,7 +470,11 @@ def autotune_generated(shape, lw, uw, weight, out_dir, specs=None, rounds=3, sam
         seen.add(v)
         try:
             g = load_generated(compile_variant(v, out_dir))
-            run = lambda: g.coefficients(x_lw, x_uw, weight, olw, ouw, stream)
+
+            def run():      # what ops.linear does with a generated entry: the variant, then the constant rows
+                g.coefficients(x_lw, x_uw, weight, olw, ouw, stream)
+                _lib.call("faith_matmul_rows_verification", zeros_b.data_ptr(), zeros_b.data_ptr(), None, None,
+                          weight.data_ptr(), None, ref[1].data_ptr(), ref[3].data_ptr(), None, None, 0, 1, K, N, stream)
             run()
             torch.cuda.synchronize(lw.device)
             if not (torch.equal(olw, ref[0]) and torch.equal(ouw, ref[2])):
