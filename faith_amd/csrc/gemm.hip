@@ -227,9 +227,21 @@ __global__ void __launch_bounds__(256) signsplit_gemm_simple(const GemmArgs g) {
 // that serve many rows there 16 - 70 us slower: a quarter of the workgroups, each a four times longer chain with
 // nothing beside it.)
 // False if the grid would be too large.
+// Few rows (the machine far from full): the 8 x 8 tiles with the split reduction instead -- a 16 x 16 tile alone is a
+// chain of K / 16 staged steps (14 us at K = 256), the split one a quarter of that.
+__global__ void __launch_bounds__(256) signsplit_gemm_sliced(const GemmArgs g) {
+    __shared__ __align__(16) float sm[3 * 8 * 65 + 2 * 4 * 64 * 2];
+    const int tiles_n = (g.N + 7) / 8;
+    sliced_tile(g, blockIdx.x / tiles_n, blockIdx.x % tiles_n, sm);
+}
 static bool launch_constant_rows(const GemmArgs &g, hipStream_t st) {
     GemmArgs gb = g;
     gb.Mw = 0;
+    if ((long long)g.Mb * g.N <= 64LL * faith::compute_units()) {           // at most one 8 x 8 tile per CU
+        const long long grids = ((long long)(g.Mb + 7) / 8) * ((g.N + 7) / 8);
+        hipLaunchKernelGGL(signsplit_gemm_sliced, dim3((unsigned)grids), dim3(256), 0, st, gb);
+        return true;
+    }
     const long long gridb = ((long long)(g.Mb + 15) / 16) * ((g.N + 15) / 16);
     if (gridb > 0x7fffffffLL) return false;
     hipLaunchKernelGGL(signsplit_gemm_simple, dim3((unsigned)gridb), dim3(256), 0, st, gb);
