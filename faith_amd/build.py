@@ -91,6 +91,9 @@ def build_variants(verbose: bool = True):
     from .autotune import GemmVariantSpec, compile_gemm_variant
     with ThreadPoolExecutor(max_workers=8) as ex:
         paths = list(ex.map(lambda v: compile_gemm_variant(GemmVariantSpec(*v), VARIANTS), PREBUILT_VARIANTS))
+    for name in os.listdir(VARIANTS):                      # builds of an earlier state of the sources
+        if os.path.join(VARIANTS, name) not in paths:
+            os.remove(os.path.join(VARIANTS, name))
     if verbose:
         print(f"built {len(paths)} GEMM variants in {VARIANTS}")
     return paths
