@@ -35,6 +35,7 @@ SIGNATURES = {
     "faith_rows_gather": [_P] * 5 + [_I] * 4 + [_P],
     "faith_rows_put": [_P] * 7 + [_I] * 4 + [_P],
     "faith_rows_spread": [_P] * 3 + [_I] * 3 + [ctypes.c_longlong, _P],
+    "faith_concretize_rows": [_P] * 7 + [_I] * 5 + [_F, _I, _I, _P],
     "faith_input_coefficients": [_P] * 3 + [_F] + [_I] * 5 + [_P],
     "faith_flag_below": [_P, _P, _I, ctypes.c_longlong, _F, _I, _P],
     "faith_verdict": [_P] * 4 + [_I, ctypes.c_longlong, _I, _P],

@@ -517,11 +517,9 @@ class CompactBounds:
     def concrete_intervals(self):
         """(l, u) [B, L, H], as concretize() of the dense form gives them (computed once)."""
         if self._intervals is None:
-            lb, ub = self._lb.contiguous(), self._ub.contiguous()
-            rows_lb, rows_ub = ops.gather_positions(lb, ub, self.positions)
-            l, u = ops.concretize(self._lw.contiguous(), rows_lb, self._uw.contiguous(), rows_ub,
-                                  self.p, self.eps, self.perturbed_words)
-            self._intervals = ops.put_positions(lb, ub, self.positions, l, u)
+            self._intervals = ops.concretize_positions(self._lw.contiguous(), self._lb.contiguous(), self._uw.contiguous(),
+                                                       self._ub.contiguous(), self.positions, self.p, self.eps,
+                                                       self.perturbed_words)
         return self._intervals
 
     # ---- VerifierForward.py:208-229 + Bounds.py:833-841 for two objects with coefficients at the same positions

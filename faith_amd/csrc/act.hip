@@ -1006,7 +1006,113 @@ int run(const char *who, ActArgs a, int q, int layout, void *stream) {
     return faith::check_launch(who);
 }
 
+// ------------------------------------------------------------------ concrete interval of a compact object
+// An object that keeps the coefficient rows of P positions per batch element only (zero elsewhere: the input of a
+// query, VerifierForward.py:127-156, and what layer norm and dense layers make of it): its interval is the constant
+// terms everywhere and lb -/+ eps * ||rows|| (Bounds.py:311-326) at those positions.  One launch: the first `norm_wgs`
+// workgroups take one (batch element, position, 64 neurons) each -- four wavefronts over the dim_in rows of every
+// word's block, partial norms through LDS, the words added in the reference's order --, the others copy the
+// constants of the positions that have no coefficients.  A position outside 0 .. L-1 names no row.
+struct RowsArgs {
+    const float *lb, *ub, *lw, *uw;       // [B, L, H]; [B, P, D, H]
+    const long long *positions;           // [B, P]
+    float *l, *u;                         // [B, L, H]
+    int B, L, P, D, H, words;
+    float eps, qv;
+};
+template <int Q>
+__global__ void __launch_bounds__(256) concretize_rows_kernel(const RowsArgs a, const int norm_wgs) {
+    __shared__ float part[16 * 4 * 2 * 64];                 // [word][row group][l, u][column]
+    const int tid = threadIdx.x;
+    if ((int)blockIdx.x >= norm_wgs) {
+        // constants of the other positions, 4 bytes per thread and step
+        const size_t n = (size_t)a.B * a.L * a.H, stride = (size_t)(gridDim.x - norm_wgs) * 256;
+        for (size_t e = (size_t)(blockIdx.x - norm_wgs) * 256 + tid; e < n; e += stride) {
+            const size_t bl = e / a.H;
+            const size_t bb = bl / a.L;
+            const long long l = (long long)(bl % a.L);
+            bool mine = true;
+            for (int p = 0; p < a.P; ++p) mine = mine && a.positions[bb * a.P + p] != l;
+            if (mine) {
+                a.l[e] = a.lb[e];
+                a.u[e] = a.ub[e];
+            }
+        }
+        return;
+    }
+    const int tiles = (a.H + 63) / 64;
+    const int bp = blockIdx.x / tiles, col = (blockIdx.x % tiles) * 64 + tid % 64, rg = tid / 64;
+    const long long at = a.positions[bp];
+    if (at < 0 || at >= a.L) return;                        // uniform over the workgroup
+    const bool col_ok = col < a.H;
+    const int blk = a.D / a.words;
+    const float *lw = a.lw + (size_t)bp * a.D * a.H + col, *uw = a.uw + (size_t)bp * a.D * a.H + col;
+    for (int w = 0; w < a.words; ++w) {
+        float nl = 0.f, nu = 0.f;
+        if (col_ok) {
+#pragma unroll 4
+            for (int d = w * blk + rg; d < (w + 1) * blk; d += 4) {
+                nl = nacc<Q>(nl, lw[(size_t)d * a.H], a.qv);
+                nu = nacc<Q>(nu, uw[(size_t)d * a.H], a.qv);
+            }
+        }
+        part[((w * 4 + rg) * 2 + 0) * 64 + tid % 64] = nl;
+        part[((w * 4 + rg) * 2 + 1) * 64 + tid % 64] = nu;
+    }
+    __syncthreads();
+    if (rg == 0 && col_ok) {
+        const size_t o = ((size_t)(bp / a.P) * a.L + (size_t)at) * a.H + col;
+        float l = a.lb[o], u = a.ub[o];
+        for (int w = 0; w < a.words; ++w) {
+            float nl = 0.f, nu = 0.f;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                nl = ncomb<Q>(nl, part[((w * 4 + g) * 2 + 0) * 64 + tid]);
+                nu = ncomb<Q>(nu, part[((w * 4 + g) * 2 + 1) * 64 + tid]);
+            }
+            l += (-a.eps) * nfin<Q>(nl, a.qv);
+            u += a.eps * nfin<Q>(nu, a.qv);
+        }
+        a.l[o] = l;
+        a.u[o] = u;
+    }
+}
+
 }  // namespace
+
+extern "C" int faith_concretize_rows(const float *lb, const float *ub, const float *lw, const float *uw,
+                                     const long long *positions, float *l, float *u, int batch_size, int length,
+                                     int n_positions, int dim_in, int dim_out, float eps, int q, int words, void *stream) {
+    const char *who = "faith_concretize_rows";
+    FAITH_NOT_NULL(lb); FAITH_NOT_NULL(ub); FAITH_NOT_NULL(lw); FAITH_NOT_NULL(uw); FAITH_NOT_NULL(positions);
+    FAITH_NOT_NULL(l); FAITH_NOT_NULL(u);
+    FAITH_ALIGNED4(lb); FAITH_ALIGNED4(ub); FAITH_ALIGNED4(lw); FAITH_ALIGNED4(uw); FAITH_ALIGNED4(l); FAITH_ALIGNED4(u);
+    FAITH_REQUIRE(faith::aligned(positions, 8), FAITH_ERR_ALIGN, "%s: positions is not 8-byte aligned", who);
+    FAITH_REQUIRE(batch_size > 0 && length > 0 && n_positions > 0 && dim_in > 0 && dim_out > 0, FAITH_ERR_SHAPE,
+                  "%s: batch=%d length=%d positions=%d dim_in=%d dim_out=%d must be positive", who, batch_size, length,
+                  n_positions, dim_in, dim_out);
+    FAITH_REQUIRE(words >= 1 && words <= 16 && dim_in % words == 0, FAITH_ERR_SHAPE,
+                  "%s: words=%d must be in 1..16 and divide dim_in=%d", who, words, dim_in);
+    RowsArgs a{lb, ub, lw, uw, positions, l, u, batch_size, length, n_positions, dim_in, dim_out, words, eps, 0.f};
+    if (!faith::dual_exponent(q, &a.qv)) {
+        faith::set_error("%s: q=%d is neither FAITH_Q_1 / FAITH_Q_2 / FAITH_Q_INF nor the bits of an exponent in (1, inf)", who, q);
+        return FAITH_ERR_UNSUPPORTED;
+    }
+    const long long norm_wgs = (long long)batch_size * n_positions * ((dim_out + 63) / 64);
+    const long long elems = (long long)batch_size * length * dim_out;
+    long long copy_wgs = (elems + 255) / 256;
+    if (copy_wgs > 4096) copy_wgs = 4096;
+    FAITH_REQUIRE(norm_wgs + copy_wgs <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
+    const dim3 gd((unsigned)(norm_wgs + copy_wgs)), bd(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (q) {
+        case FAITH_Q_1: hipLaunchKernelGGL(concretize_rows_kernel<FAITH_Q_1>, gd, bd, 0, st, a, (int)norm_wgs); break;
+        case FAITH_Q_2: hipLaunchKernelGGL(concretize_rows_kernel<FAITH_Q_2>, gd, bd, 0, st, a, (int)norm_wgs); break;
+        case FAITH_Q_INF: hipLaunchKernelGGL(concretize_rows_kernel<FAITH_Q_INF>, gd, bd, 0, st, a, (int)norm_wgs); break;
+        default: hipLaunchKernelGGL(concretize_rows_kernel<Q_GENERAL>, gd, bd, 0, st, a, (int)norm_wgs); break;
+    }
+    return faith::check_launch(who);
+}
 
 // Concretizes two bound objects of equal dim_in in ONE launch (the dot product needs the intervals
 // of both operands before it can start).  Natural layout.

@@ -1268,6 +1268,130 @@ __global__ void __launch_bounds__(256) scores_compact(const CompactArgs g) {
     }
 }
 
+// The HEAVY launch on the matrix unit (L and D multiples of 32, head size 32 or 64): for a row i in S the x terms
+// are a matrix product with rows m -- [D x size] coefficient rows of x against the [size x L] intervals of the key,
+// split by sign --, so a wavefront takes 32 coordinates m and, in turn, every block of 32 columns j: its x fragments
+// and the key's intervals come straight from global memory in MFMA layout (lane (row, half) holds k = 8 s + 4 half
+// .. + 3 of its row), four products per K-pair as in dot_w_small.  The vector-ALU version above walks the reduction
+// with a global load per four k in every lane's chain (32 us for one query's four heads); this one has its loads
+// in flight together and 128 MFMAs per block.  A workgroup is four such wavefronts (128 coordinates) and first
+// forms the column values of its coordinates (the y terms) as the other launch does.
+template <int NS>                                                     // NS = head size / 8: K-steps
+__global__ void __launch_bounds__(256) scores_compact_heavy_mfma(const CompactArgs g) {
+    extern __shared__ __align__(16) float cs[];
+    constexpr int size = 8 * NS;
+    const int L = g.L, P = g.P, pitch = g.heads * size;
+    float *col_l = cs, *col_u = cs + P * CS_MC;                       // [P][CS_MC]
+    int pid = blockIdx.x;
+    const int c = pid % g.chunks;  pid /= g.chunks;
+    const int pi = pid % P;  pid /= P;
+    const int t = pid, b = t / g.heads, h = t - b * g.heads;
+    const long long *pos = g.positions + (size_t)b * P;
+    const long long at = pos[pi];
+    if (at < 0 || at >= L) return;                                    // no such row (uniform over the workgroup)
+    const int i = (int)at;
+    const int m0 = c * CS_MC, tid = threadIdx.x;
+    const int lane = tid % 64, wv = tid / 64;
+    const int fi = lane % 32, fh = lane / 32;
+    const int mb = m0 + 32 * wv;                                      // this wavefront's 32 coordinates
+    const bool active = mb < g.D;
+
+    // ---- the wavefront's x fragments (they serve every block of columns) and the key's intervals of the first block:
+    // asked for before anything else, so that they arrive under the column values
+    const size_t xrow = (((size_t)b * P + pi) * g.D + (active ? mb + fi : 0)) * pitch + (size_t)h * size + 4 * fh;
+    float4 xl[NS], xu[NS], al[NS], au[NS];
+    auto fetch_a = [&](int j0) __attribute__((always_inline)) {
+        const size_t arow = ((size_t)b * L + j0 + fi) * pitch + (size_t)h * size + 4 * fh;
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {
+            al[s_] = *reinterpret_cast<const float4 *>(g.y_l + arow + 8 * s_);
+            au[s_] = *reinterpret_cast<const float4 *>(g.y_u + arow + 8 * s_);
+        }
+    };
+    if (active) {
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {
+            xl[s_] = *reinterpret_cast<const float4 *>(g.xlw + xrow + 8 * s_);
+            xu[s_] = *reinterpret_cast<const float4 *>(g.xuw + xrow + 8 * s_);
+        }
+        fetch_a(0);
+    }
+
+    // ---- column values: b(i, :) against the key's rows of S; the loads of a dot product's quarter go out together
+    const float *beta = g.x_l + ((size_t)b * L + i) * pitch + (size_t)h * size;
+    for (int e = tid; e < 4 * P * CS_MC; e += 256) {
+        const int part = e % 4, ml = (e / 4) % CS_MC, p = e / (4 * CS_MC);
+        float sl = 0.f, su = 0.f;
+        if (m0 + ml < g.D) {
+            const size_t row = (((size_t)b * P + p) * g.D + m0 + ml) * pitch + (size_t)h * size;
+            constexpr int NQ = (size + 15) / 16;
+            float4 bt[NQ], yl[NQ], yu[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const int k = 4 * part + 16 * q;
+                const bool in = k < size;
+                const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+                bt[q] = in ? *reinterpret_cast<const float4 *>(beta + k) : zero;
+                yl[q] = in ? *reinterpret_cast<const float4 *>(g.ylw + row + k) : zero;
+                yu[q] = in ? *reinterpret_cast<const float4 *>(g.yuw + row + k) : zero;
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+#define FAITH_TERM(F)                                                        \
+    {                                                                        \
+        const float bp = fmaxf(bt[q].F, 0.f), bn = fminf(bt[q].F, 0.f);      \
+        sl += bp * yl[q].F + bn * yu[q].F;                                   \
+        su += bp * yu[q].F + bn * yl[q].F;                                   \
+    }
+                FAITH_TERM(x) FAITH_TERM(y) FAITH_TERM(z) FAITH_TERM(w)
+#undef FAITH_TERM
+            }
+        }
+        sl += __shfl_xor(sl, 1);  su += __shfl_xor(su, 1);
+        sl += __shfl_xor(sl, 2);  su += __shfl_xor(su, 2);
+        if (part == 0) { col_l[p * CS_MC + ml] = sl;  col_u[p * CS_MC + ml] = su; }
+    }
+    __syncthreads();
+    if (!active) return;
+
+    for (int j0 = 0; j0 < L; j0 += 32) {
+        floatx16 cl, cu;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) cl[r] = cu[r] = 0.f;
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {
+#define FAITH_STEP(F)                                                 \
+    cl = mfma(xl[s_].F, fmaxf(al[s_].F, 0.f), cl);                    \
+    cu = mfma(xu[s_].F, fmaxf(au[s_].F, 0.f), cu);                    \
+    cl = mfma(xu[s_].F, fminf(al[s_].F, 0.f), cl);                    \
+    cu = mfma(xl[s_].F, fminf(au[s_].F, 0.f), cu);
+            FAITH_STEP(x) FAITH_STEP(y) FAITH_STEP(z) FAITH_STEP(w)
+#undef FAITH_STEP
+        }
+        const int jcol = j0 + fi;
+        if (j0 + 32 < L) fetch_a(j0 + 32);                            // the next block's intervals under this block's stores
+        // register r is coordinate 8 (r / 4) + 4 fh + r % 4 of the block, lanes run along j; the column of a key
+        // position of S takes its column value on top
+        for (int p = 0; p < P; ++p) {
+            if (pos[p] == (long long)jcol) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int ml = 32 * wv + 8 * (r / 4) + 4 * fh + (r % 4);
+                    cl[r] += col_l[p * CS_MC + ml];
+                    cu[r] += col_u[p * CS_MC + ml];
+                }
+            }
+        }
+        const size_t z0 = (((size_t)t * L + i) * g.D + mb) * L + jcol;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const size_t o = z0 + (size_t)(8 * (r / 4) + 4 * fh + (r % 4)) * L;
+            g.zlw[o] = cl[r];
+            g.zuw[o] = cu[r];
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int faith_dot_product_verification_QK(float *x_l, float *y_l, float *x_u, float *y_u, const float *x_lb,
@@ -1436,7 +1560,16 @@ extern "C" int faith_attention_scores_compact(const float *x_l, const float *y_l
     FAITH_REQUIRE(light <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
     const long long b_tiles = B * ((length + BT_T - 1) / BT_T) * ((length + BT_T - 1) / BT_T);
     FAITH_REQUIRE(b_tiles <= 0x7fffffffLL, FAITH_ERR_SHAPE, "%s: grid too large", who);
-    hipLaunchKernelGGL(scores_compact<true>, dim3((unsigned)heavy), dim3(256), lds, st, c);
+    // rows of S: on the matrix unit where the blocks are whole (knob value 4 keeps the vector-ALU kernel)
+    const bool on_mfma = length % 32 == 0 && dim_in % 32 == 0 && (head_size == 32 || head_size == 64) &&
+                         faith::tune_get(FAITH_TUNE_DOT_VARIANT) != 4;
+    const size_t col_lds = (size_t)2 * n_positions * CS_MC * sizeof(float);
+    if (on_mfma && head_size == 64)
+        hipLaunchKernelGGL(scores_compact_heavy_mfma<8>, dim3((unsigned)heavy), dim3(256), col_lds, st, c);
+    else if (on_mfma)
+        hipLaunchKernelGGL(scores_compact_heavy_mfma<4>, dim3((unsigned)heavy), dim3(256), col_lds, st, c);
+    else
+        hipLaunchKernelGGL(scores_compact<true>, dim3((unsigned)heavy), dim3(256), lds, st, c);
     hipLaunchKernelGGL(scores_compact<false>, dim3((unsigned)light), dim3(256), (size_t)2 * n_positions * CS_MC * sizeof(float), st, c);
     // constant terms: the dense kernel (it reads constants and intervals only)
     DotArgs g{nullptr, nullptr, nullptr, nullptr, x_lb, x_ub, y_lb, y_ub, x_l, y_l, y_u, nullptr, nullptr, z_lb, z_ub,

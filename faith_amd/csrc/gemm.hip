@@ -281,16 +281,16 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_small(const GemmArgs 
 // (i, h) holds k = 8 s + 4 h .. + 3 of row i: the same K pairing as the LDS fragments above), so there is
 // no staging and no barrier in the loop; the four partial blocks meet in LDS and are added in a fixed
 // order.  K % 32 == 0.  The first `b_tiles` workgroups take the constant-term rows, as above.
-__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs g, const int b_tiles) {
-    __shared__ __align__(16) float sm[4 * 2 * 16 * 64];          // 32 KB: [wavefront][l, u][register][lane]
-    if ((int)blockIdx.x < b_tiles) {
+// `block`: the workgroup's number within its problem; sm: 32 KB ([wavefront][l, u][register][lane]).
+__device__ __forceinline__ void ksplit_body(const GemmArgs &g, const int b_tiles, const int block, float *sm) {
+    if (block < b_tiles) {
         const int tiles_n = (g.N + 7) / 8;
-        const int m_blk = blockIdx.x / tiles_n;
-        if (m_blk < (g.Mb + 7) / 8) sliced_tile(g, m_blk, blockIdx.x % tiles_n, sm);
+        const int m_blk = block / tiles_n;
+        if (m_blk < (g.Mb + 7) / 8) sliced_tile(g, m_blk, block % tiles_n, sm);
         return;
     }
     constexpr int CH = 4;                                        // K-steps of 8 fetched ahead
-    const int pid = blockIdx.x - b_tiles;
+    const int pid = block - b_tiles;
     const int tiles_n = (g.N + 31) / 32;
     const int m0 = (pid / tiles_n) * 32, n0 = (pid % tiles_n) * 32;
     const int lane = threadIdx.x % 64, wv = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -369,6 +369,10 @@ __global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs
         }
     }
 }
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit(const GemmArgs g, const int b_tiles) {
+    __shared__ __align__(16) float sm[4 * 2 * 16 * 64];
+    ksplit_body(g, b_tiles, blockIdx.x, sm);
+}
 
 
 // Up to three GEMMs that share their left operand (the query, key and value layers of an attention block:
@@ -388,6 +392,13 @@ __device__ __forceinline__ GemmArgs group_of(const GroupArgs &G, const int grp) 
         h.Cl = G.Cl[i];  h.Cu = G.Cu[i];  h.Dl = G.Dl[i];  h.Du = G.Du[i];
     }
     return h;
+}
+// Tiny problems that share their operand (the query, key and value layers on the coefficient rows of one perturbed
+// position): `per` workgroups of signsplit_gemm_ksplit per group, one launch.
+__global__ void __launch_bounds__(NTHREADS) signsplit_gemm_ksplit_grouped(const GroupArgs G, const int b_tiles, const int per) {
+    __shared__ __align__(16) float sm[4 * 2 * 16 * 64];
+    const GemmArgs h = group_of(G, blockIdx.x / per);
+    ksplit_body(h, b_tiles, blockIdx.x % per, sm);
 }
 // b_tiles constant-term tiles per group first (all groups), then `w_tiles` MFMA tiles per group; both are
 // multiples of 8, so a tile keeps the XCD its number within the group gives it.
@@ -569,11 +580,28 @@ static int matmul_group_rows(const float *x_lb, const float *x_ub, const float *
     // one launch where the small tiles are the choice for the three problems taken together and no single
     // one of them is a tiny problem (those have a kernel of their own); otherwise one launch each
     int tm = 0, tn = 0;
+    if (fast && dim_out % 32 == 0 && dim_out >= 128 && 4 * tiles(64, 64) / groups <= cus) {
+        // tiny problems: the kernel that splits the reduction over a workgroup's wavefronts, all groups in one launch
+        GroupArgs G{};
+        G.g = GemmArgs{x_lw, x_uw, x_lb, x_ub, W[0], bias ? bias[0] : nullptr, y_lw[0], y_uw[0], y_lb[0], y_ub[0], (int)mw, (int)rows,
+                       dim_y_out, dim_out};
+        for (int i = 1; i < groups; ++i) {
+            G.W[i - 1] = W[i];  G.bias[i - 1] = bias ? bias[i] : nullptr;
+            G.Cl[i - 1] = y_lw[i];  G.Cu[i - 1] = y_uw[i];  G.Dl[i - 1] = y_lb[i];  G.Du[i - 1] = y_ub[i];
+        }
+        G.groups = groups;
+        const long long gridb = ((rows + 7) / 8) * ((dim_y_out + 7) / 8);
+        const long long per = gridb + ((mw + 31) / 32) * ((dim_y_out + 31) / 32);
+        FAITH_REQUIRE(per * groups <= 0x7fffffffLL, FAITH_ERR_SHAPE, "faith_matmul_group_verification: grid too large");
+        hipLaunchKernelGGL(signsplit_gemm_ksplit_grouped, dim3((unsigned)(per * groups)), dim3(NTHREADS), 0,
+                           static_cast<hipStream_t>(stream), G, (int)gridb, (int)per);
+        return faith::check_launch("faith_matmul_group_verification");
+    }
     if (fast) {
         if (tiles(64, 64) <= cus) { tm = 64; tn = 64; }
         else if (tiles(128, 64) <= 2 * cus) { tm = 128; tn = 64; }
         else if (tiles(128, 128) < 8 * cus) { tm = 64; tn = 64; }
-        if (tm == 0 || (dim_out % 32 == 0 && dim_out >= 128 && 4 * tiles(64, 64) / groups <= cus)) fast = false;
+        if (tm == 0) fast = false;
     }
     if (!fast) {
         for (int i = 0; i < groups; ++i) {

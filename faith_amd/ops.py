@@ -939,6 +939,27 @@ def verdict(l, u, flags, label, host=False):
     return safe
 
 
+def concretize_positions(lw, lb, uw, ub, positions, p, eps, words=1):
+    """Concrete interval [B, L, H] of an object whose coefficients lw, uw [B, P, D, H] exist at `positions` [B, P] only
+    (lb, ub [B, L, H]): the constants where there are no coefficients, lb - eps ||lw||, ub + eps ||uw|| at the
+    positions.  One launch."""
+    _check("lw", lw); _check("uw", uw, lw.shape); _check("lb", lb); _check("ub", ub, lb.shape)
+    if lw.dim() != 4 or lb.dim() != 3:
+        raise ValueError(f"lw {tuple(lw.shape)} must be [B, P, dim_in, H] and lb {tuple(lb.shape)} [B, L, H]")
+    B, P, D, H = lw.shape
+    if lb.shape[0] != B or lb.shape[2] != H:
+        raise ValueError(f"lw {tuple(lw.shape)} and lb {tuple(lb.shape)} disagree in batch or width")
+    L = lb.shape[1]
+    if not (positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous()
+            and tuple(positions.shape) == (B, P)):
+        raise ValueError(f"positions: expected a contiguous int64 GPU tensor of shape {(B, P)}")
+    l, u = _empty_like(lb), _empty_like(ub)
+    with _on(lw.device):
+        _lib.call("faith_concretize_rows", _ptr(lb), _ptr(ub), _ptr(lw), _ptr(uw), _ptr(positions), _ptr(l), _ptr(u),
+                  B, L, P, D, H, float(eps), q_code(p), int(words), _stream(lw))
+    return l, u
+
+
 def attention_scores_compact_fits(length, n_positions, head_size, dim_in):
     """True if attention_scores_compact takes operands of this shape (16-byte aligned tensors assumed)."""
     return (dim_in > 1 and length % 4 == 0 and head_size % 4 == 0

@@ -58,7 +58,7 @@ int faith_version(void);
  */
 #define FAITH_TUNE_ACT_VARIANT   0   /* tile shape of the natural-layout relaxation kernels; 8 / 12 / 7 force the one-tile register-resident kernel with four wavefronts / sixteen wavefronts / sixteen wavefronts and non-temporal loads, 15 the persistent two-tile kernel; 0: eight wavefronts, two workgroups per CU (three for tanh), whole rows of the object dealt to the XCDs; 11 / 13 the four-wavefront shapes of concretize */
 #define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split GEMM: 1 = 64x64, 2 = 128x128, 3 = 128x64, 4 = 64x128, 5 = 32x32 with K split over the wavefronts (dim_out % 32 == 0); 6 = faith_matmul_concretize_verification takes its one-launch kernel whenever the shape allows; 7 = it keeps layer and concretize apart; 8 = as 6, with 32x32 blocks also where the reduction is short enough for 16x16 blocks */
-#define FAITH_TUNE_DOT_VARIANT   2   /* dot product: 1 = 128x64 persistent tiles with run-time extents (also where the straight-line instantiations for reductions of 32 / 64 / 128 would be taken), 2 = one 32x32 block per wavefront (short sequences only), 3 = transposed layout: the vector-ALU kernel also where the MFMA kernels apply */
+#define FAITH_TUNE_DOT_VARIANT   2   /* dot product: 1 = 128x64 persistent tiles with run-time extents (also where the straight-line instantiations for reductions of 32 / 64 / 128 would be taken), 2 = one 32x32 block per wavefront (short sequences only), 3 = transposed layout: the vector-ALU kernel also where the MFMA kernels apply; 4 = compact scores: the rows of the perturbed positions on the vector-ALU kernel also where the matrix-unit kernel takes them */
 #define FAITH_TUNE_DOT_COORDS    3   /* dot product, 32x32 kernel: perturbation coordinates per wavefront, 1..16 */
 #define FAITH_TUNE_CONV_VARIANT  4   /* convolution: 1 = the general kernel (run-time extents) for every layer; 2 = tiles in the plain order (not whole images per XCD); 3 = 2 x 2 blocks per wavefront also for short reductions */
 #define FAITH_TUNE_COUNT         5
@@ -230,6 +230,18 @@ int faith_rows_put(const float *a, const float *b, const float *rows_a, const fl
                    int batch_size, int length, int n_positions, int dim_out, void *stream);
 int faith_rows_spread(const float *rows, const long long *positions, float *out,
                       int batch_size, int length, int n_positions, long long row_floats, void *stream);
+
+/*
+ * Concrete interval (Bounds.concretize, Bounds.py:311-326) of an object that keeps the coefficient rows of
+ * n_positions positions per batch element only: lw, uw [batch, n_positions, dim_in, dim_out], lb, ub
+ * [batch, length, dim_out], positions int64 [batch, n_positions] -> l, u [batch, length, dim_out]: the constants
+ * where there are no coefficients, lb - eps * ||lw rows||_q and ub + eps * ||uw rows||_q at the positions (per word
+ * block, as faith_concretize).  One launch where gathering the constants, faith_concretize on the rows and putting
+ * the results back were three.  l, u must not overlap the inputs.
+ */
+int faith_concretize_rows(const float *lb, const float *ub, const float *lw, const float *uw,
+                          const long long *positions, float *l, float *u, int batch_size, int length,
+                          int n_positions, int dim_in, int dim_out, float eps, int q, int words, void *stream);
 
 /*
  * The layer driver's own device work, one launch each where the reference evaluates three or four tensor

@@ -74,6 +74,9 @@ def test_null_and_shape_errors_are_status_codes(lib):
     assert L.faith_input_coefficients(p, None, None, 1.0, 1, 4, 1, 8, 1, None) == -2     # compact: one row per word
     assert L.faith_flag_below(p, p, 0, 4, 0.0, 1, None) == -2
     assert L.faith_verdict(p, p, None, None, 1, 1, 0, None) == -1
+    assert L.faith_concretize_rows(p, p, p, p, None, p, p, 1, 4, 1, 8, 8, 0.1, lib.Q_2, 1, None) == -1
+    assert L.faith_concretize_rows(p, p, p, p, p, p, p, 1, 4, 1, 8, 8, 0.1, lib.Q_2, 3, None) == -2   # words divide dim_in
+    assert L.faith_concretize_rows(p, p, p, p, p, p, p, 1, 4, 1, 8, 8, 0.1, 7, 1, None) == -3
     # the allocation-free dot product refuses what its 4 MiB array cannot hold, before touching the GPU
     assert L.faith_static_scratch_bytes() == 4 << 20
     assert L.faith_dot_product_verification_QK_static(p, p, p, p, p, p, p, p, p, p, p, p,

@@ -520,3 +520,85 @@ def test_rows_are_spread_into_the_written_out_object_by_the_library(shape):
             if 0 <= int(positions[i, j]) < L:
                 want[i, int(positions[i, j])] = t[i, j]
     assert torch.equal(got.cpu(), want) and torch.equal(const.cpu(), want[:, :, 0])
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 64, 4, 64, 32), (2, 2, 256, 4, 64, 32), (3, 1, 128, 2, 32, 32), (1, 2, 64, 1, 32, 64)])
+@pytest.mark.parametrize("p", [2.0, float("inf"), 1.0])
+def test_rows_of_the_perturbed_positions_on_the_matrix_unit(shape, p):
+    """Where length and dim_in are multiples of 32 and a head is 32 or 64 wide the score rows of the perturbed
+    positions come from the matrix-unit kernel; knob 4 of the dot product's variant sends them to the vector-ALU
+    kernel.  Both sum the same head_size products, in different orders."""
+    from faith_amd import _lib
+    B, P, D, heads, size, L = shape
+    words = 2 if P == 2 else 1
+    print(f"[case] compact scores, matrix unit against vector ALU B={B} P={P} D={D} heads={heads} size={size} L={L} p={p}", flush=True)
+    cq, dq = compact_and_dense(51, B, P, D, heads * size, L, words=words, p=p)
+    ck, dk = compact_and_dense(52, B, P, D, heads * size, L, words=words, p=p, positions=cq.positions)
+    got = cq.attention_scores(ck, heads)
+    _lib.call("faith_tune_set", 2, 4)
+    try:
+        want = cq.attention_scores(ck, heads)
+        torch.cuda.synchronize()
+    finally:
+        _lib.call("faith_tune_set", 2, 0)
+    tw, tb = score_terms(dq, dk, heads)
+    for name, terms in (("lw", tw), ("uw", tw), ("lb", tb), ("ub", tb)):
+        x, y = getattr(got, name), getattr(want, name)
+        tol = ATOL + RTOL * y.double().abs().cpu() + 2 * KAPPA * U32 * terms
+        over = float(((x.double() - y.double()).abs().cpu() / tol).max())
+        assert over <= 1.0, f"scores.{name}: {over:.2f} of the accumulation-aware bar"
+    # the constants and the rows without coefficients do not go through the matrix unit: same bits
+    assert torch.equal(got.lb, want.lb) and torch.equal(got.ub, want.ub)
+    assert torch.equal(got.lw == 0, want.lw == 0) and torch.equal(got.uw == 0, want.uw == 0)
+
+
+@pytest.mark.parametrize("shape", [(3, 2, 10, 24, 5, 1), (2, 2, 64, 100, 9, 2), (1, 1, 256, 256, 32, 1), (4, 3, 33, 70, 6, 3),
+                                   (2, 1, 7, 130, 300, 1)])
+@pytest.mark.parametrize("p", [2.0, float("inf"), 1.0, 3.0])
+def test_concrete_interval_of_a_compact_object_in_one_launch(shape, p):
+    """faith_concretize_rows against its three-launch equivalent (constants gathered, faith_concretize on the rows,
+    results put back) and against faith_concretize on the object with the zeros written out."""
+    from faith_amd import ops
+    B, P, D, H, L, words = shape
+    print(f"[case] concretize rows B={B} P={P} D={D} H={H} L={L} words={words} p={p}", flush=True)
+    c, d = compact_and_dense(61, B, P, D, H, L, words=words, p=p)
+    l, u = ops.concretize_positions(c._lw, c._lb, c._uw, c._ub, c.positions, p, 0.1, words)
+    rows_lb, rows_ub = ops.gather_positions(c._lb, c._ub, c.positions)
+    rl, ru = ops.concretize(c._lw, rows_lb, c._uw, rows_ub, p, 0.1, words)
+    l3, u3 = ops.put_positions(c._lb, c._ub, c.positions, rl, ru)
+    dl, du = ops.concretize(d.lw, d.lb, d.uw, d.ub, p, 0.1, words)
+    torch.cuda.synchronize()
+    has = torch.zeros(B, L, dtype=torch.bool)
+    has[torch.arange(B)[:, None], c.positions.cpu()] = True
+    # no coefficients: the constants themselves
+    assert torch.equal(l.cpu()[~has], c._lb.cpu()[~has]) and torch.equal(u.cpu()[~has], c._ub.cpu()[~has])
+    for name, x, ys in (("l", l, (l3, dl)), ("u", u, (u3, du))):
+        for y in ys:
+            err, of_bar = worst(x, y)
+            assert of_bar <= 1.0, f"{name}: max err {err:.3g}, {of_bar:.2f} of the bar"
+    assert bool((l <= u).all())
+
+
+def test_concrete_interval_of_a_compact_object_skips_a_position_outside_the_sentence():
+    from faith_amd import ops
+    B, P, D, H, L = 2, 2, 12, 40, 6
+    g = torch.Generator().manual_seed(62)
+    positions = torch.tensor([[1, L + 3], [-1, 4]])
+    lw = torch.randn(B, P, D, H, generator=g)
+    uw = lw + 0.05 * torch.rand(B, P, D, H, generator=g)
+    lb = torch.randn(B, L, H, generator=g)
+    ub = lb + 0.3 * torch.rand(B, L, H, generator=g)
+    l, u = ops.concretize_positions(lw.cuda(), lb.cuda(), uw.cuda(), ub.cuda(), positions.cuda(), 2.0, 0.1, 1)
+    torch.cuda.synchronize()
+    want_l, want_u = lb.clone(), ub.clone()
+    for b, j, at in ((0, 0, 1), (1, 1, 4)):
+        want_l[b, at] = lb[b, at] - 0.1 * lw[b, j].double().norm(dim=0).float()
+        want_u[b, at] = ub[b, at] + 0.1 * uw[b, j].double().norm(dim=0).float()
+    for x, y in ((l, want_l), (u, want_u)):
+        assert worst(x.cpu(), y)[1] <= 1.0
+    keep = torch.ones(B, L, dtype=torch.bool); keep[0, 1] = keep[1, 4] = False
+    assert torch.equal(l.cpu()[keep], lb[keep]) and torch.equal(u.cpu()[keep], ub[keep])
+    with pytest.raises(ValueError):
+        ops.concretize_positions(lw.cuda(), lb.cuda(), uw.cuda(), ub.cuda(), positions.int().cuda(), 2.0, 0.1, 1)
+    with pytest.raises(Exception, match="words"):
+        ops.concretize_positions(lw.cuda(), lb.cuda(), uw.cuda(), ub.cuda(), positions.cuda(), 2.0, 0.1, 5)
