@@ -98,12 +98,16 @@ def _checked_positions(groups, length):
     return out
 
 
-def _compact_maker(make_bounds, batch, length, dim_in, dim_out):
+def _compact_maker(make_bounds, batch, length, dim_in, dim_out, captured=False):
     """make_bounds.compact if the maker has one (faith_amd.BoundsMaker) and finds that leaving out the zero
-    coefficient rows pays for an object of this shape, else None."""
+    coefficient rows pays for an object of this shape, else None.  captured: the propagation is replayed from a
+    graph, where a launch costs the device's time only."""
     compact = getattr(make_bounds, "compact", None)
     pays = getattr(make_bounds, "compact_pays", None)
-    if compact is None or (pays is not None and not pays(batch, length, dim_in, dim_out)):
+    if compact is None:
+        return None
+    if pays is not None and not (pays(batch, length, dim_in, dim_out, captured=True) if captured else
+                                 pays(batch, length, dim_in, dim_out)):
         return None
     return compact
 
@@ -410,7 +414,7 @@ class CapturedVerifier:
         dev = embeddings.device
         self.batch, self.label, self.dim, self.length, self.make_bounds = batch, label, dim, length, make_bounds
         self.b = embeddings[0].unsqueeze(0).expand(batch, length, dim).contiguous()
-        compact = _compact_maker(make_bounds, batch, length, dim, dim)
+        compact = _compact_maker(make_bounds, batch, length, dim, dim, captured=True)
         if compact is not None:
             # the graph reads the perturbed positions and the scaled identities from these two
             self.at = torch.zeros((batch, 1), dtype=torch.int64, device=dev)

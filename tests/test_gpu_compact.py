@@ -474,6 +474,18 @@ def test_captured_graph_on_the_compact_input_follows_new_positions_and_radii(len
         assert got == want, (idx, radii, got, want)
         seen.update(got)
     assert len(seen) == 2 or length != LENGTH                 # at the test network's own length both verdicts occur
+    # a maker that would write a propagation this small out keeps the compact form for the graph, where the extra
+    # launches cost the device's time only; one query per replay, against the written-out eager propagation
+    default, plain = BoundsMaker(), (lambda p_, e_, lw, lb, uw, ub: BoundsMaker()(p_, e_, lw, lb, uw, ub))
+    assert not default.compact_pays(1, length, HIDDEN, HIDDEN) and default.compact_pays(1, length, HIDDEN, HIDDEN, captured=True)
+    assert not BoundsMaker(SimpleNamespace(method="ibp")).compact_pays(1, length, HIDDEN, HIDDEN, captured=True)
+    one = F.CapturedVerifier(default, gnet, ge, 1, label, 2.0)
+    assert one.at is not None
+    for idx, radius in ((1, 0.004), (3, 0.3), (2, 0.0005), (1, 0.004)):
+        got = one([idx], [radius])
+        want = F.verify_safety(plain, gnet, ge, idx, radius, label, 2.0)
+        torch.cuda.synchronize()
+        assert got == [bool(want)], (idx, radius, got, want)
 
 
 def test_rows_of_a_compact_object_are_gathered_and_put_back_by_the_library():
