@@ -51,36 +51,40 @@ __device__ __forceinline__ TanhAt tanh_at(float x) {
     return {(t - 1.0) * r, 4.0 * t * r * r};
 }
 
-// Tangent point search of Bounds.py:1065-1075 (lower = true) and :1082-1092 (lower = false).
-// `anchor` is the far end of the interval (u for the lower line, l for the upper line).
-// v > 0 is decided on (tanh difference) - sech^2(d) * (distance), which has the sign of the
-// reference's quotient form because the distance (+1e-12) is positive; the line through the point
-// found is then formed in double.
+// Tangent point search of Bounds.py:1065-1075 (lower = true) and :1082-1092 (lower = false): the ten bisection
+// steps, in fp32 as the reference takes them on its fp32 tensors.  `anchor` is the far end of the interval (u for
+// the lower line, l for the upper line).  The reference asks whether (tanh difference) / (distance) - sech^2(d) is
+// positive; the distance (+1e-12) is positive, and so is (t + 1)^2 with t = exp(2 d), tanh d = (t - 1) / (t + 1),
+// sech^2 d = 4 t / (t + 1)^2, so the sign is that of
+//     (tanh(anchor) (t + 1) - (t - 1)) (t + 1) - 4 t distance          (lower; the upper line with the first factor negated)
+// -- no division, one exponential, fourteen instructions a step: the chain of ten dependent steps is what a tile
+// waits for.  A sign that differs from the quotient form's can only occur where the quantity is within rounding of
+// zero, i.e. at the tangent point itself, where the slope of the line is stationary.
 template <bool LOWER>
-__device__ __forceinline__ Line tanh_tangent_line(float l, float u) {
-    const float anchor = LOWER ? u : l;
-    const double ta = tanh_at(anchor).th;
-    const float ta32 = (float)ta;
+__device__ __forceinline__ float tanh_tangent_point(float l, float u) {
+    constexpr float TWO_LOG2E = 2.885390081777926815f;
+    const float ea = __builtin_amdgcn_exp2f(__builtin_amdgcn_fmed3f(LOWER ? u : l, -20.f, 20.f) * TWO_LOG2E);
+    const float ta = (ea - 1.f) / (ea + 1.f);
     float d = (LOWER ? l : u) / 2, a = LOWER ? l : 0.f, b = LOWER ? 0.f : u;
+#pragma unroll
     for (int it = 0; it < 10; ++it) {
-        // the sign test in fp32, as the reference takes it (torch.tanh / cosh on fp32 tensors): the chain of
-        // ten dependent evaluations is what a tile waits for, and in double it is four times as long
-        const float t = __expf(2.f * fminf(fmaxf(d, -20.f), 20.f));
-        const float r = 1.f / (t + 1.f);
-        const float th = (t - 1.f) * r, s2 = 4.f * t * r * r;
-        bool go;
-        if (LOWER)
-            go = (ta32 - th) - s2 * ((u - d) + TINY) > 0.f;
-        else
-            go = (th - ta32) - s2 * ((d - l) + TINY) > 0.f;
-        if (LOWER == go) {   // lower & v>0, or upper & v<=0: move right
+        const float t = __builtin_amdgcn_exp2f(__builtin_amdgcn_fmed3f(d, -20.f, 20.f) * TWO_LOG2E);
+        const float p = t + 1.f, tm1 = t - 1.f;
+        const float c4 = __builtin_fmaf(LOWER ? u - d : d - l, 4.f, 4.f * TINY);
+        const float q = LOWER ? __builtin_fmaf(ta, p, -tm1) : __builtin_fmaf(-ta, p, tm1);
+        const bool go = __builtin_fmaf(q, p, -(t * c4)) > 0.f;
+        if (LOWER == go)     // lower & v > 0, or upper & v <= 0: move right
             a = d;
-            d = (d + b) / 2;
-        } else {             // move left
+        else                 // move left
             b = d;
-            d = (d + a) / 2;
-        }
+        d = (a + b) / 2;     // the end that moved is d: (d + b) / 2 or (d + a) / 2
     }
+    return d;
+}
+
+// The line through the tangent point found and the anchor, formed in double; `ta` = tanh(anchor).
+template <bool LOWER>
+__device__ __forceinline__ Line tanh_tangent_line(float l, float u, float d, double ta) {
     const double td = tanh_at(d).th;
     if (LOWER) return {(float)((td - ta) / (double)((d - u) + TINY)), d, (float)td};
     return {(float)((td - ta) / (double)((d - l) + TINY)), d, (float)td};
@@ -103,16 +107,21 @@ __device__ __forceinline__ void tanh_pure_lines(float l, float u, Line &lo, Line
 }
 
 // tanh lines of the TH neurons of a tile whose concrete intervals are in s_lu ([2][TH]), entered by
-// every thread after a barrier: three wavefronts share the per-neuron work, lane = neuron.  Slopes end
-// up in s_ln[0 .. TH) and s_ln[3 TH .. 4 TH) (complete once the barrier inside has been passed), the
+// every thread after a barrier: four wavefronts share the per-neuron work, lane = neuron.  Slopes end
+// up in s_ln[0 .. TH) and s_ln[3 TH .. 4 TH) (complete once the barriers inside have been passed), the
 // constant terms in olb / oub.
 template <int TH>
 __device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, float *s_ln, float lb, float ub, size_t bi,
                                            bool n_ok, int lane, int wv) {
-    // three wavefronts share the per-neuron work: 0 = lower tangent search, 1 = upper tangent
-    // search (straddling neurons), 2 = tangent / chord of one-signed neurons
-    if (wv < 3 && n_ok) {
-        const float l = s_lu[lane], u = s_lu[TH + lane];
+    // 0 = lower tangent search, 1 = upper tangent search (straddling neurons), 2 = tangent / chord of one-signed
+    // neurons, 3 = tanh of both ends in double, which the lines of the straddling neurons pass through: the
+    // searches do not wait for it
+    __shared__ double s_anchor[2 * TH];
+    float l = 0.f, u = 0.f, d = 0.f;
+    bool searched = false;
+    if (wv < 4 && n_ok) {
+        l = s_lu[lane];
+        u = s_lu[TH + lane];
         const bool pure = (u < 0.f || l > 0.f);
         if (wv == 2) {
             if (pure) {
@@ -122,13 +131,23 @@ __device__ __forceinline__ void tanh_stage(const ActArgs &a, const float *s_lu, 
                 s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
             }
         } else if (!pure) {
-            if (wv == 0) {
-                const Line lo = tanh_tangent_line<true>(l, u);
-                s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
+            if (wv == 3) {
+                s_anchor[lane] = tanh_at(u).th;
+                s_anchor[TH + lane] = tanh_at(l).th;
             } else {
-                const Line up = tanh_tangent_line<false>(l, u);
-                s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
+                searched = true;
+                d = wv == 0 ? tanh_tangent_point<true>(l, u) : tanh_tangent_point<false>(l, u);
             }
+        }
+    }
+    __syncthreads();
+    if (searched) {
+        if (wv == 0) {
+            const Line lo = tanh_tangent_line<true>(l, u, d, s_anchor[lane]);
+            s_ln[lane] = lo.k; s_ln[TH + lane] = lo.x0; s_ln[2 * TH + lane] = lo.y0;
+        } else {
+            const Line up = tanh_tangent_line<false>(l, u, d, s_anchor[TH + lane]);
+            s_ln[3 * TH + lane] = up.k; s_ln[4 * TH + lane] = up.x0; s_ln[5 * TH + lane] = up.y0;
         }
     }
     __syncthreads();
@@ -597,8 +616,8 @@ __device__ __forceinline__ void relax_any(float l, float u, float lb, float ub, 
         if (u < 0.f || l > 0.f) {
             tanh_pure_lines(l, u, lo, up);
         } else {
-            lo = tanh_tangent_line<true>(l, u);
-            up = tanh_tangent_line<false>(l, u);
+            lo = tanh_tangent_line<true>(l, u, tanh_tangent_point<true>(l, u), tanh_at(u).th);
+            up = tanh_tangent_line<false>(l, u, tanh_tangent_point<false>(l, u), tanh_at(l).th);
         }
         klo = lo.k;
         kup = up.k;
@@ -910,14 +929,15 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         //   4 wavefronts x 8 rows, 4 workgroups per CU (256 KB in flight)   relu 39.9 | 56.0   tanh 40.5 | 59.3
         //   4 wavefronts x 8 rows, 3 per CU                                 relu 40.9 | 53.9   tanh 42.1 | 55.0
         //   4 wavefronts x 8 rows, 2 per CU                                 relu 42.9 | 52.7   tanh 45.2 | 56.6
-        //   8 wavefronts x 4 rows, 3 per CU (192 KB)                        relu 41.3 | 54.0   tanh 41.6 | 55.0
-        //   8 wavefronts x 4 rows, 2 per CU (128 KB)                        relu 41.3 | 51.9   tanh 43.1 | 53.2
+        //   8 wavefronts x 4 rows, 3 per CU (192 KB)                        relu 40.8 | 53.8   tanh 40.7 | 54.4
+        //   8 wavefronts x 4 rows, 2 per CU (128 KB)                        relu 41.4 | 51.9   tanh 42.7 | 52.7
         //   16 wavefronts x 2 rows, 2 per CU                                relu 44.5 | 52.7   tanh 48.0 | 53.6
         //   the same with non-temporal loads                                relu 50.2 | 51.3   tanh 51.3 | 52.5
         //   persistent, two tiles in registers, 2 per CU (plain order)      relu 41.5 | 57.3   tanh 43.8 | 59.9
+        //   the same with whole rows per XCD, 4 / 8 wavefronts              relu 41.8 | 58.2, 42.3 | 59.4   tanh 42.1 | 60.6, 43.2 | 62.4
         // From the cache more tiles in flight are better, from HBM fewer; the library cannot know which it will be, so
         // the default is the shape that is within 4 % of the best in both: eight wavefronts, two workgroups per CU --
-        // three for tanh, whose per-neuron stage (ten dependent bisection steps on three of the wavefronts) wants a
+        // three for tanh, whose per-neuron stage (ten dependent bisection steps on two of the wavefronts) wants a
         // third workgroup to run meanwhile.  Objects whose traffic is beyond 9/4 of the cache cannot be resident in it:
         // sixteen wavefronts and non-temporal loads ([B, 32, 256, 512], 404 MB ... 2 GB: the order flips near 600 MB).
         // Knob values 8 / 12 / 7 force the one-tile shapes of four / sixteen / sixteen wavefronts with non-temporal loads
