@@ -43,7 +43,8 @@ int compute_units() {
     return cached[dev];
 }
 
-static int g_tune[FAITH_TUNE_COUNT] = {0};
+// per calling thread: a tuning table applied around one thread's launch does not steer another thread's
+static thread_local int g_tune[FAITH_TUNE_COUNT] = {0};
 
 int tune_get(int knob) { return (knob >= 0 && knob < FAITH_TUNE_COUNT) ? g_tune[knob] : 0; }
 

@@ -54,7 +54,9 @@ int faith_version(void);
 /*
  * Kernel-variant selection for tuning runs (no counterpart in the reference, whose tile sizes
  * are compile-time: HandTunedKernels/matmul_config.h).  value 0 restores the built-in choice.
- * Process-wide, not thread-safe; results never depend on it, only speed.
+ * Kept per calling thread: a value set by one thread selects the variants of that thread's later calls only, so
+ * threads that tune, or that apply a tuning table around their launches, do not disturb each other.  Every variant
+ * of an operator meets the same tolerance; variants that sum in another order differ in the last bits.
  */
 #define FAITH_TUNE_ACT_VARIANT   0   /* tile shape of the natural-layout relaxation kernels; 8 / 12 / 7 force the one-tile register-resident kernel with four wavefronts / sixteen wavefronts / sixteen wavefronts and non-temporal loads, 15 the persistent two-tile kernel; 0: eight wavefronts, two workgroups per CU (three for tanh), whole rows of the object dealt to the XCDs; 11 / 13 the four-wavefront shapes of concretize */
 #define FAITH_TUNE_GEMM_VARIANT  1   /* macro-tile of the sign-split GEMM: 1 = 64x64, 2 = 128x128, 3 = 128x64, 4 = 64x128, 5 = 32x32 with K split over the wavefronts (dim_out % 32 == 0); 6 = faith_matmul_concretize_verification takes its one-launch kernel whenever the shape allows; 7 = it keeps layer and concretize apart; 8 = as 6, with 32x32 blocks also where the reduction is short enough for 16x16 blocks */

@@ -86,6 +86,31 @@ def test_null_and_shape_errors_are_status_codes(lib):
                                                       1, 0, 4, 4, 4, 0.1, lib.Q_1, 1, 0, None) == -2
 
 
+def test_tuning_knobs_are_kept_per_thread():
+    """Concurrent setters never fail, and what a thread that has ended did -- its knob values, the message of its
+    refused call -- is not the main thread's (tests/test_gpu_act.py checks on the GPU that a knob set in one thread
+    selects that thread's kernels only)."""
+    import threading
+    from faith_amd import _lib as lib
+    L = lib.lib
+    codes = []
+
+    def worker(i):
+        for _ in range(200):
+            codes.append(L.faith_tune_set(i % 5, i))
+        codes.append(L.faith_tune_set(99, 1))          # the unknown knob's message stays in this thread
+
+    L.faith_tune_set(0, 0)
+    before = L.faith_last_error()
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert codes.count(0) == 8 * 200 and codes.count(-3) == 8
+    assert L.faith_last_error() == before
+
+
 def test_python_wrappers_refuse_cpu_tensors():
     import torch
     from faith_amd import ops

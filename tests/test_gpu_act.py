@@ -107,6 +107,43 @@ def test_thread_shape_for_hbm_streams_gives_the_same_values(kind, p):
         assert close(a, b.cpu())
 
 
+def test_a_knob_set_by_one_thread_selects_that_threads_kernels_only():
+    """The tuning knobs are kept per calling thread.  Knob 8 (four wavefronts a tile) groups a column's partial norms
+    differently from the default shape, so its results differ in the last bits of some values: a worker thread that
+    sets it gets those bits, the main thread keeps getting the default's."""
+    import threading
+    from faith_amd import _lib, ops
+    g = torch.Generator(device="cuda").manual_seed(21)
+    shape = (1, 40, 256, 1024)
+    lw = torch.empty(shape, device="cuda").normal_(0, 0.05, generator=g)
+    uw = torch.empty(shape, device="cuda").normal_(0, 0.005, generator=g).abs_().add_(lw)
+    lb = torch.empty((1, 40, 1024), device="cuda").normal_(0, 1, generator=g)
+    ub = torch.empty((1, 40, 1024), device="cuda").normal_(0, 0.5, generator=g).abs_().add_(lb)
+    run = lambda: [t.clone() for t in ops.relu(lw, lb, uw, ub, 2.0, 0.01, 2, return_interval=True)]
+    ref = run()
+    _lib.call("faith_tune_set", 0, 8)
+    try:
+        forced = run()
+    finally:
+        _lib.call("faith_tune_set", 0, 0)
+    torch.cuda.synchronize()
+    assert not all(torch.equal(a, b) for a, b in zip(ref, forced)), "the two shapes gave the same bits: nothing to observe"
+    seen = {}
+
+    def worker():
+        _lib.call("faith_tune_set", 0, 8)          # never reset: the value ends with the thread
+        seen["forced"] = run()
+        torch.cuda.synchronize()
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    after = run()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(seen["forced"], forced))
+    assert all(torch.equal(a, b) for a, b in zip(after, ref))
+
+
 @pytest.mark.parametrize("kind,p", [("relu", 2.0), ("relu", INF), ("exp", 1.0), ("sqr", 2.0), ("tanh", 2.0)])
 @pytest.mark.parametrize("rows", [40, 43])
 def test_persistent_two_tile_kernel_gives_the_one_tile_kernels_bits(kind, p, rows):
