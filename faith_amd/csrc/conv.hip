@@ -697,12 +697,19 @@ bool launch_fast(const ConvArgs &g, hipStream_t st) {
 
 // Layers whose reduction is short (at most 64 products per result: a 1 x 1 layer of up to 64 channels, the 3 x 3
 // first layer of an image classifier): 1 x 2 blocks per wavefront, four workgroups per CU (see FastTile) --
-// 64 channels x 4 pixel blocks, or 128 channels x 2 pixel blocks where the layer has that many channels (the
-// patch is then read once instead of twice).  Measured against 2 x 2 blocks: 1 x 1 64 -> 128 107 -> 96-99 us,
+// 64 channels x 4 pixel blocks, 128 channels x 2 pixel blocks where the layer has that many channels (the
+// patch is then read once instead of twice), or 32 channels x 8 pixel blocks (below).  Measured against 2 x 2 blocks: 1 x 1 64 -> 128 107 -> 96-99 us,
 // 1 x 1 32 -> 64 49 -> 41 us, 3 x 3 3 -> 64 45 -> 39-41 us; one block per wavefront was no faster than two.
 template <int K, int S, int CCH, bool WVEC>
 bool launch_brief(const ConvArgs &g, hipStream_t st) {
     if ((g.Wo - 1) % 32 < 16) return launch_tile<K, S, CCH, WVEC, 16, 2, 1, 2>(g, st);
+    // 3 x 3 first layers whose last (or only) 64 channels would be at most half there: 32 channels x 8 pixel
+    // blocks, the four wavefronts side by side over the image rows (3 -> 32: 35 -> 23 us, 3 -> 96: 73 -> 53 us,
+    // 3 -> 64 the same either way).  Not for 1 x 1 layers, whose patch of 8 rows x 16 channels a chunk would leave
+    // room for two workgroups on a CU instead of four (1 x 1 64 -> 128 on it: 165 against 96 us).
+    if constexpr (K == 3) {
+        if ((g.Co - 1) % 64 < 32) return launch_tile<K, S, CCH, WVEC, 32, 1, 1, 2>(g, st);
+    }
     if ((g.Co - 1) % 128 >= 64) return launch_tile<K, S, CCH, WVEC, 32, 4, 1, 2>(g, st);
     return launch_tile<K, S, CCH, WVEC, 32, 2, 1, 2>(g, st);
 }

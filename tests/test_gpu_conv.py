@@ -142,6 +142,9 @@ def test_straight_line_conv_kernels_equal_the_general_kernel(case):
     (3, 20, 100, 30, 30, 1, 1, 0),     # ragged: channels, rows and columns past the last full tile
     (4, 16, 48, 16, 16, 1, 1, 0),      # 16-column pixel blocks
     (2, 3, 200, 9, 70, 3, 1, 1),       # first layer, wide and short image, several channel tiles
+    (40, 3, 32, 32, 32, 3, 1, 1),      # first layer of 32 channels: 32-channel tiles of eight image rows
+    (5, 3, 96, 28, 28, 3, 1, 1),       # 96 = three 32-channel tiles; rows and columns past the last full tile
+    (3, 1, 16, 28, 28, 3, 1, 1),       # one input channel, half a channel tile
 ])
 def test_short_reductions_on_small_wavefront_tiles_equal_the_large_ones(case):
     """Layers with at most 64 products per result run with 1 x 2 MFMA blocks per wavefront (four workgroups per CU)
