@@ -406,7 +406,9 @@ struct FastTile {
     static constexpr int RPB = 32 / TCB;                 // image rows of one pixel block
     static constexpr int NPB = MB * (4 / WM);            // pixel blocks of a workgroup
     static constexpr int ROWS = NPB * RPB, CHANNELS = 32 * MA * WM;
-    static constexpr int WAVES = MA * MB == 4 ? 2 : 4;   // wavefronts per SIMD the register budget is set for
+    // wavefronts per SIMD the register budget is set for: two with 128 accumulators, four with 64 -- three where the
+    // patch of a strided or 5 x 5 layer needs more than 128 registers beside them
+    static constexpr int WAVES = MA * MB == 4 ? 2 : (S > 1 || K >= 5) ? 3 : 4;
     static constexpr int KK = K * K, PROW = (ROWS - 1) * S + K, PCOL = (TCB - 1) * S + K, PP = PROW * PCOL;
     static constexpr int WS = (CCH * KK) | 1;
     static constexpr size_t LDS = ((size_t)4 * CCH * PP + (size_t)2 * CHANNELS * WS) * sizeof(float);
@@ -463,10 +465,11 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     const size_t w_bytes = (size_t)(g.Co - co0) * g.Ci * KK * 4;
 
     // ---- staging plan, fixed for the whole reduction: byte offsets inside a chunk of channels
-    // (a 5 x 5 layer has no registers to spare for the plan beside its weight slab, nor has a stride-2 layer with
-    // 64-channel tiles, whose patch is 18 elements per thread: they work each offset out again where it is used,
-    // a dozen integer operations per element against hundreds of MFMAs per chunk)
-    constexpr bool KEEP_PLAN = K < 5 && NP <= 12;
+    // (kept in registers by the 1 x 1 layers and by the 3 x 3 stride-1 layers with 128 accumulators; 4 x 4 and
+    // 5 x 5 layers have no registers to spare for it beside their weight slab, nor have strided layers, whose patch
+    // is up to 18 elements per thread, nor tiles with a budget of 128 registers: they work each offset out again
+    // where it is used, a dozen integer operations per element against hundreds of MFMAs per chunk)
+    constexpr bool KEEP_PLAN = K < 4 && S == 1 && NP <= 12 && !(T::WAVES == 4 && K > 1);
     auto patch_offset = [&](int u, int tid_) -> unsigned {
         const int e = tid_ + u * NTHREADS;
         const int ci = e / PP, r2 = e % PP, pr = r2 / PCOL, pc = r2 % PCOL;
@@ -689,6 +692,17 @@ bool launch_tile(const ConvArgs &g, hipStream_t st) {
 template <int K, int S, int CCH, bool WVEC>
 bool launch_fast(const ConvArgs &g, hipStream_t st) {
     const bool narrow = (g.Wo - 1) % 32 < 16, few = (g.Co - 1) % 128 < 64;
+    // at most 32 output channels: 32 channels x 8 pixel blocks, one channel block per wavefront (a 64-channel tile
+    // would multiply zeros for half of its rows: 3 x 3 16 -> 32 92 -> 52 us, 32 -> 32 171 -> 104 us, 5 x 5 16 -> 32
+    // 227 -> 126 us on 256 images of 32 x 32; with 1 x 4 blocks per wavefront instead of 1 x 2: no better).  Layers
+    // of 65 ... 96 channels keep the 64-channel tiles: three 32-channel tiles read the patch three times and measured
+    // slower (3 x 3 stride 2 32 -> 96: 121 against 98 us).
+    if (g.Co <= 32) return narrow ? launch_tile<K, S, CCH, WVEC, 16, 1, 1, 2>(g, st) : launch_tile<K, S, CCH, WVEC, 32, 1, 1, 2>(g, st);
+    // results of at most 8 x 8 pixels (the last layers of a small classifier): pixel blocks of 8 columns x 4 rows, two
+    // of them a tile -- the whole image --, under 128 or 64 channels (against 16-column blocks, which such an image
+    // fills by half: 3 x 3 64 -> 128 110 -> 76 us, 128 -> 128 208 -> 145 us, 4 x 4 stride 2 32 -> 64 102 -> 50 us)
+    if (g.Wo <= 8 && g.Ho <= 8)
+        return g.Co > 64 ? launch_tile<K, S, CCH, WVEC, 8, 4, 1, 2>(g, st) : launch_tile<K, S, CCH, WVEC, 8, 2, 1, 1>(g, st);
     if (narrow && few) return launch_tile<K, S, CCH, WVEC, 16, 1>(g, st);
     if (narrow) return launch_tile<K, S, CCH, WVEC, 16, 2>(g, st);
     if (few) return launch_tile<K, S, CCH, WVEC, 32, 1>(g, st);
@@ -728,6 +742,8 @@ bool dispatch_fast(const ConvArgs &g, bool wvec, hipStream_t st) {
             case 32: return launch_fast<3, 2, 4, true>(g, st);
             case 11: return launch_fast<1, 1, 16, true>(g, st);
             case 51: return launch_fast<5, 1, 4, true>(g, st);
+            case 42: return launch_fast<4, 2, 4, true>(g, st);      // the 4 x 4 stride-2 layers of the small image classifiers
+            case 41: return launch_fast<4, 1, 4, true>(g, st);
             default: return false;
         }
     }
@@ -735,6 +751,9 @@ bool dispatch_fast(const ConvArgs &g, bool wvec, hipStream_t st) {
         case 31: return launch_fast<3, 1, 4, false>(g, st);
         case 32: return launch_fast<3, 2, 4, false>(g, st);
         case 11: return launch_fast<1, 1, 16, false>(g, st);
+        case 51: return launch_fast<5, 1, 4, false>(g, st);
+        case 42: return launch_fast<4, 2, 4, false>(g, st);
+        case 41: return launch_fast<4, 1, 4, false>(g, st);
         default: return false;
     }
 }

@@ -74,6 +74,25 @@ def check(x, W, bias, stride, pad, what="", ratio_ceiling=None):
     (2, 16, 24, 7, 12, 1, 1, 0),       # 1x1: both small
     (1, 8, 32, 10, 10, 5, 1, 2),       # 5x5: both small
     (3, 3, 32, 16, 16, 3, 1, 1),       # C_in = 3, both small
+    # at most 32 output channels: 32-channel tiles of eight pixel blocks, one channel block per wavefront
+    (3, 16, 32, 32, 32, 3, 1, 1),
+    (2, 16, 16, 20, 20, 3, 1, 1),      # half a channel block, ragged rows and columns
+    (2, 8, 24, 33, 33, 3, 2, 1),       # stride 2, 16-column blocks
+    (2, 16, 32, 14, 40, 5, 1, 2),      # 5x5
+    (2, 32, 20, 9, 9, 1, 1, 0),        # 1x1
+    # 4x4 kernels (the strided layers of the small image classifiers), with and without 16-byte weight rows
+    (3, 3, 32, 32, 32, 4, 2, 1),
+    (2, 32, 128, 16, 16, 4, 2, 1),
+    (2, 16, 40, 15, 19, 4, 1, 1),
+    (2, 6, 70, 12, 36, 4, 2, 0),
+    (2, 1, 16, 28, 28, 5, 1, 2),       # 5x5 on one input channel (4-byte weight rows)
+    # results of at most 8 x 8 pixels: pixel blocks of 8 columns x 4 rows
+    (3, 64, 128, 8, 8, 3, 1, 1),
+    (3, 32, 64, 16, 16, 4, 2, 1),
+    (2, 16, 200, 7, 6, 3, 1, 1),       # ragged: 7 x 6 pixels, 128 + 72 channels
+    (2, 20, 48, 16, 13, 3, 2, 1),      # 8 x 7 results from stride 2, half a channel tile
+    (2, 64, 128, 8, 8, 1, 1, 0),
+    (2, 16, 64, 8, 8, 5, 1, 2),
 ])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_conv_shapes(case, with_bias):
