@@ -428,7 +428,9 @@ static void choose_tile(long long mw, int dim_out, int dim_y_out, int *tm, int *
     // the reduction length: 2 - 5 % at 131072 ... 245760 rows with K and N of 256 ... 768 (the batched propagation of
     // a sentence's positions), level at 8 tiles per CU, behind below that, where the pro- and epilogues of five
     // small co-resident workgroups overlap better than those of two large ones
-    if (tiles(64, 64) <= cus) { *tm = 64; *tn = 64; }
+    // (fewer 128 x 64 tiles than CUs would each run alone, one wavefront per SIMD: twice as many 64 x 64 tiles,
+    // two on a CU, finish in the time of one -- 2560 rows, K = N = 768: 118 -> 75 us, K = 3072: 451 -> 251 us)
+    if (tiles(64, 64) <= cus || tiles(128, 64) < cus) { *tm = 64; *tn = 64; }
     else if (tiles(128, 64) <= 2 * cus) { *tm = 128; *tn = 64; }
     else if (tiles(128, 128) >= 12 * cus) { *tm = 128; *tn = 128; }
     // many column tiles re-read every block of rows from L2: the large tile halves that (3 - 5 % at
