@@ -86,6 +86,9 @@ struct Vec<4> {
         const v4f t = {v.x, v.y, v.z, v.w};
         __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
     }
+    // through the L2 as an ordinary store: for rows that do not start on 64-byte boundaries, where neighbouring tiles
+    // write parts of the same 64 bytes and the cache puts them together before they go to memory
+    __device__ __forceinline__ void store_cached(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
     __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
     __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
     __device__ __forceinline__ void set(int i, float f) {
@@ -100,6 +103,7 @@ struct Vec<1> {
     float v;
     __device__ __forceinline__ void load(const float *p) { v = *p; }
     __device__ __forceinline__ void store(float *p) const { __builtin_nontemporal_store(v, p); }
+    __device__ __forceinline__ void store_cached(float *p) const { *p = v; }
     __device__ __forceinline__ void zero() { v = 0.f; }
     __device__ __forceinline__ float get(int) const { return v; }
     __device__ __forceinline__ void set(int, float f) { v = f; }
