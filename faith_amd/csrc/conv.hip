@@ -465,11 +465,12 @@ conv_signsplit_fast(const ConvArgs g, const int total_tiles) {
     const size_t w_bytes = (size_t)(g.Co - co0) * g.Ci * KK * 4;
 
     // ---- staging plan, fixed for the whole reduction: byte offsets inside a chunk of channels
-    // (kept in registers by the 1 x 1 layers and by the 3 x 3 stride-1 layers with 128 accumulators; 4 x 4 and
-    // 5 x 5 layers have no registers to spare for it beside their weight slab, nor have strided layers, whose patch
-    // is up to 18 elements per thread, nor tiles with a budget of 128 registers: they work each offset out again
-    // where it is used, a dozen integer operations per element against hundreds of MFMAs per chunk)
-    constexpr bool KEEP_PLAN = K < 4 && S == 1 && NP <= 12 && !(T::WAVES == 4 && K > 1);
+    // (kept in registers by the 1 x 1 layers and by the 3 x 3 layers with 128 accumulators and at most 12 patch
+    // elements per thread -- stride 2, 64 -> 128: 183 us with the plan, 197 us without; 4 x 4 and 5 x 5 layers have
+    // no registers to spare for it beside their weight slab, nor have the stride-2 tiles of 64 channels, whose patch
+    // is 18 elements per thread, nor tiles with a smaller register budget: they work each offset out again where it
+    // is used, a dozen integer operations per element against hundreds of MFMAs per chunk)
+    constexpr bool KEEP_PLAN = K < 4 && NP <= 12 && (T::WAVES == 2 || K == 1);
     auto patch_offset = [&](int u, int tid_) -> unsigned {
         const int e = tid_ + u * NTHREADS;
         const int ci = e / PP, r2 = e % PP, pr = r2 / PCOL, pc = r2 % PCOL;
