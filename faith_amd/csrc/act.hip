@@ -762,42 +762,79 @@ void launch_pipelined(const ActArgs &a, hipStream_t st) {
                        smem, st, a, n_tiles);
 }
 
-// Transposed layout, D_in = 256 V (V = 1, 2), 16-byte aligned: a wavefront owns 8 / V neurons, one
-// 16-byte load per lane covers 256 coefficients of a neuron's contiguous row, and everything a
-// wavefront reads (64 values per thread) stays in registers between the norm and the scaling: one
-// read, one write, no LDS and no barrier.  The norms of a neuron end up in every lane of its
-// wavefront (butterfly); lane i then derives the lines of the wavefront's i-th neuron, and the slopes
-// travel back by cross-lane reads.
-template <int MODE, int Q, int V>
+// Butterflies over groups of F lanes (F = 8, 16, 32 side by side in a wavefront), every lane ends with its group's
+// total: the steps of wave_sum / wave_max up to distance F / 2.
+template <int F>
+__device__ __forceinline__ float group_sum(float v) {
+    v += lane_permute<0xB1>(v);
+    v += lane_permute<0x4E>(v);
+    v += lane_permute<0x141>(v);
+    if constexpr (F >= 16) v += lane_permute<0x140>(v);
+    if constexpr (F >= 32) v += __shfl_xor(v, 16, WAVE);
+    if constexpr (F >= 64) v += __shfl_xor(v, 32, WAVE);
+    return v;
+}
+template <int F>
+__device__ __forceinline__ float group_max(float v) {
+    v = fmaxf(v, lane_permute<0xB1>(v));
+    v = fmaxf(v, lane_permute<0x4E>(v));
+    v = fmaxf(v, lane_permute<0x141>(v));
+    if constexpr (F >= 16) v = fmaxf(v, lane_permute<0x140>(v));
+    if constexpr (F >= 32) v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+    if constexpr (F >= 64) v = fmaxf(v, __shfl_xor(v, 32, WAVE));
+    return v;
+}
+
+// Transposed layout, D_in a multiple of 4 up to 1024, 16-byte aligned: a neuron's D_in coefficients are one
+// contiguous row, which the lanes of a wavefront read 16 bytes each -- V loads per lane for rows of more than 256
+// floats (V = ceil(D_in / 256); lanes past the end of the row hold zeros), G = 64 / (D_in / 4) neurons side by side
+// for rows of 128, 64 or 32 floats.  A wavefront owns R G neurons, and everything it reads (up to 64 values per
+// thread) stays in registers between the norm and the scaling: one read, one write, no LDS and no barrier.  The
+// norms of a neuron end up in every lane of its group (butterfly); lane j then derives the lines of the
+// wavefront's j-th neuron, and the slopes travel back by cross-lane reads.
+template <int MODE, int Q, int V, int G, int R>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) act_transposed_resident(const ActArgs a) {
-    constexpr int NPW = 8 / V;
+    static_assert(V == 1 || G == 1, "several loads per lane, or several neurons per row of lanes");
+    constexpr int NPW = R * G, F = WAVE / G;                           // neurons per wavefront; lanes per neuron
+    static_assert(4 * NPW <= WAVE, "the shared tanh stage takes one neuron per lane of a wavefront");
     const int lane = threadIdx.x % WAVE, wv = threadIdx.x / WAVE;
+    const int grp = G == 1 ? 0 : lane / F, fl = G == 1 ? lane : lane % F;
     const long long total = (long long)a.rows * a.H;
     const long long n0 = ((long long)blockIdx.x * 4 + wv) * NPW;      // first neuron of this wavefront
     const int blk = a.D / a.words;
-
-    Vec<4> dl[NPW][V], du[NPW][V];
+    bool ok[V];
 #pragma unroll
-    for (int i = 0; i < NPW; ++i) {
-        const long long n = n0 + i < total ? n0 + i : total - 1;      // a clamped neuron is never stored
-        const float *pl = a.lw + (size_t)n * a.D + lane * 4, *pu = a.uw + (size_t)n * a.D + lane * 4;
+    for (int v = 0; v < V; ++v) ok[v] = (v * WAVE + fl) * 4 < a.D;
+
+    Vec<4> dl[R][V], du[R][V];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const long long want = n0 + i * G + grp;
+        const long long n = want < total ? want : total - 1;          // a clamped neuron is never stored
+        const float *pl = a.lw + (size_t)n * a.D + fl * 4, *pu = a.uw + (size_t)n * a.D + fl * 4;
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            dl[i][v].load(pl + v * 256);
-            du[i][v].load(pu + v * 256);
+            if (ok[v]) {
+                dl[i][v].load(pl + v * 256);
+                du[i][v].load(pu + v * 256);
+            } else {
+                dl[i][v].zero();
+                du[i][v].zero();
+            }
         }
     }
-    float l[NPW], u[NPW];
+    float l[R], u[R];
 #pragma unroll
-    for (int i = 0; i < NPW; ++i) {
-        const long long n = n0 + i < total ? n0 + i : total - 1;
+    for (int i = 0; i < R; ++i) {
+        const long long want = n0 + i * G + grp;
+        const long long n = want < total ? want : total - 1;
         float li = a.lb[n], ui = a.ub[n];
         for (int w = 0; w < a.words; ++w) {
             float nl = 0.f, nu = 0.f;
 #pragma unroll
             for (int v = 0; v < V; ++v) {
-                const int k0 = v * 256 + lane * 4;                    // blk % 4 == 0: a float4 lies in one word
-                if (k0 >= w * blk && k0 < (w + 1) * blk) {
+                const int k0 = (v * WAVE + fl) * 4;                   // blk % 4 == 0: a float4 lies in one word
+                if (k0 >= w * blk && k0 < (w + 1) * blk) {            // (zeros past the end of the row belong to none)
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         nl = nacc<Q>(nl, dl[i][v].get(c), a.qv);
@@ -805,21 +842,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) a
                     }
                 }
             }
-            nl = Q == FAITH_Q_INF ? wave_max(nl) : wave_sum(nl);
-            nu = Q == FAITH_Q_INF ? wave_max(nu) : wave_sum(nu);
+            nl = Q == FAITH_Q_INF ? group_max<F>(nl) : group_sum<F>(nl);
+            nu = Q == FAITH_Q_INF ? group_max<F>(nu) : group_sum<F>(nu);
             li += (-a.eps) * nfin<Q>(nl, a.qv);
             ui += a.eps * nfin<Q>(nu, a.qv);
         }
         l[i] = li;
         u[i] = ui;
     }
-    // lane i takes the wavefront's i-th neuron
-    float myl = l[0], myu = u[0];
+    // lane j takes the wavefront's j-th neuron: row j / G of group j % G
+    float myl = 0.f, myu = 0.f;
 #pragma unroll
-    for (int i = 1; i < NPW; ++i) {
-        if (lane == i) {
-            myl = l[i];
-            myu = u[i];
+    for (int i = 0; i < R; ++i) {
+        const float tl = G == 1 ? l[i] : __shfl(l[i], (lane % G) * F, WAVE);
+        const float tu = G == 1 ? u[i] : __shfl(u[i], (lane % G) * F, WAVE);
+        if (lane / G == i) {
+            myl = tl;
+            myu = tu;
         }
     }
     float klo = 0.f, kup = 0.f;
@@ -836,7 +875,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) a
     }
     if (MODE == CONCRETIZE) return;
     if (MODE == TANH) {
-        // the search for the tangent points is long: gather the workgroup's neurons in LDS and let three
+        // the search for the tangent points is long: gather the workgroup's neurons in LDS and let four
         // wavefronts do it for all of them at once, one neuron per lane
         constexpr int NPB = 4 * NPW;
         __shared__ float s_lu[2 * NPB], s_ln[6 * NPB];
@@ -846,30 +885,33 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) a
         }
         __syncthreads();
         const long long first = (long long)blockIdx.x * NPB;
-        const bool mine = lane < NPB && first + lane < total;
-        const float lb0 = (wv == 0 && mine) ? a.lb[first + lane] : 0.f, ub0 = (wv == 0 && mine) ? a.ub[first + lane] : 0.f;
-        tanh_stage<NPB>(a, s_lu, s_ln, lb0, ub0, (size_t)(first + lane), mine, lane, wv);
+        const bool mine_ok = lane < NPB && first + lane < total;
+        const float lb0 = (wv == 0 && mine_ok) ? a.lb[first + lane] : 0.f, ub0 = (wv == 0 && mine_ok) ? a.ub[first + lane] : 0.f;
+        tanh_stage<NPB>(a, s_lu, s_ln, lb0, ub0, (size_t)(first + lane), mine_ok, lane, wv);
         if (lane < NPW) {
             klo = s_ln[wv * NPW + lane];
             kup = s_ln[3 * NPB + wv * NPW + lane];
         }
     }
 #pragma unroll
-    for (int i = 0; i < NPW; ++i) {
-        const float k_lo = __shfl(klo, i, WAVE), k_up = __shfl(kup, i, WAVE);
-        if (n0 + i < total) {
-            float *ql = a.olw + (size_t)(n0 + i) * a.D + lane * 4, *qu = a.ouw + (size_t)(n0 + i) * a.D + lane * 4;
+    for (int i = 0; i < R; ++i) {
+        const float k_lo = __shfl(klo, i * G + grp, WAVE), k_up = __shfl(kup, i * G + grp, WAVE);
+        const long long n = n0 + i * G + grp;
+        if (n < total) {
+            float *ql = a.olw + (size_t)n * a.D + fl * 4, *qu = a.ouw + (size_t)n * a.D + fl * 4;
 #pragma unroll
             for (int v = 0; v < V; ++v) {
-                Vec<4> ol, ou;
+                if (ok[v]) {
+                    Vec<4> ol, ou;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float xl = dl[i][v].get(c), xu = du[i][v].get(c);
-                    ol.set(c, (k_lo > 0.f ? xl : xu) * k_lo);
-                    ou.set(c, (k_up > 0.f ? xu : xl) * k_up);
+                    for (int c = 0; c < 4; ++c) {
+                        const float xl = dl[i][v].get(c), xu = du[i][v].get(c);
+                        ol.set(c, (k_lo > 0.f ? xl : xu) * k_lo);
+                        ou.set(c, (k_up > 0.f ? xu : xl) * k_up);
+                    }
+                    ol.store(ql + v * 256);
+                    ou.store(qu + v * 256);
                 }
-                ol.store(ql + v * 256);
-                ou.store(qu + v * 256);
             }
         }
     }
@@ -1005,10 +1047,22 @@ void dispatch_layout(const ActArgs &a, int layout, hipStream_t st) {
         const long long total = (long long)a.rows * a.H;
         const bool vec = (a.D / a.words) % 4 == 0 && faith::aligned(a.lw, 16) && faith::aligned(a.uw, 16) &&
                          (MODE == CONCRETIZE || (faith::aligned(a.olw, 16) && faith::aligned(a.ouw, 16)));
-        if (vec && a.D == 256)
-            hipLaunchKernelGGL((act_transposed_resident<MODE, Q, 1>), dim3((unsigned)((total + 31) / 32)), dim3(256), 0, st, a);
-        else if (vec && a.D == 512)
-            hipLaunchKernelGGL((act_transposed_resident<MODE, Q, 2>), dim3((unsigned)((total + 15) / 16)), dim3(256), 0, st, a);
+        // rows of up to 1024 floats stay in registers (see act_transposed_resident): V loads per lane, or G neurons
+        // side by side in a wavefront
+        auto resident = [&](auto v, auto g, auto r) {
+            constexpr int V = decltype(v)::value, G = decltype(g)::value, R = decltype(r)::value;
+            hipLaunchKernelGGL((act_transposed_resident<MODE, Q, V, G, R>), dim3((unsigned)((total + 4 * R * G - 1) / (4 * R * G))),
+                               dim3(256), 0, st, a);
+        };
+        using std::integral_constant;
+        const int f4 = a.D / 4;
+        if (vec && a.D == 128) resident(integral_constant<int, 1>{}, integral_constant<int, 2>{}, integral_constant<int, 8>{});
+        else if (vec && a.D == 64) resident(integral_constant<int, 1>{}, integral_constant<int, 4>{}, integral_constant<int, 4>{});
+        else if (vec && a.D == 32) resident(integral_constant<int, 1>{}, integral_constant<int, 8>{}, integral_constant<int, 2>{});
+        else if (vec && f4 <= 64) resident(integral_constant<int, 1>{}, integral_constant<int, 1>{}, integral_constant<int, 8>{});
+        else if (vec && f4 <= 128) resident(integral_constant<int, 2>{}, integral_constant<int, 1>{}, integral_constant<int, 4>{});
+        else if (vec && f4 <= 192) resident(integral_constant<int, 3>{}, integral_constant<int, 1>{}, integral_constant<int, 2>{});
+        else if (vec && f4 <= 256) resident(integral_constant<int, 4>{}, integral_constant<int, 1>{}, integral_constant<int, 2>{});
         else
             hipLaunchKernelGGL((act_transposed<MODE, Q>), dim3((unsigned)((total + 63) / 64)), dim3(256), 0, st, a);
     }

@@ -70,6 +70,20 @@ def test_activation_small_shapes(kind, p, layout):
         check(kind, x, p, 0.05, words, layout)
 
 
+@pytest.mark.parametrize("kind", ["relu", "tanh", "exp"])
+@pytest.mark.parametrize("p", [2.0, INF, 1.0, 3.0])
+def test_transposed_rows_of_any_length_stay_in_registers(kind, p):
+    """The transposed layout (what the reference's adapters hand over) keeps rows of up to 1024 coefficients in
+    registers: several neurons side by side in a wavefront for D_in = 32 / 64 / 128, one to four loads per lane
+    beyond, lanes past the end of a row idle (D_in = 192, 300, 516).  Neuron counts that do not fill the last
+    wavefront or workgroup; against the oracle."""
+    g = torch.Generator().manual_seed(16)
+    for (L, D, H, words) in [(5, 32, 50, 1), (3, 64, 70, 2), (7, 128, 33, 1), (2, 192, 40, 2), (2, 300, 24, 1),
+                             (2, 384, 40, 2), (3, 768, 23, 1), (1, 1024, 20, 2), (1, 516, 19, 3), (1, 16, 9, 1)]:
+        x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+        check(kind, x, p, 0.05, words, "transposed")
+
+
 @pytest.mark.parametrize("kind", ["concretize", "relu", "tanh"])
 @pytest.mark.parametrize("words", [8, 16])
 def test_many_perturbed_words_need_more_than_64_kb_of_lds(kind, words):
