@@ -1006,10 +1006,13 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
         ActArgs b = a;
         const long long n_tiles = (long long)a.rows * (a.H / 32);
         b.remap = (tv == 8 || tv == 12 || tv == 7) ? 0 : a.rows % 8 == 0 ? 2 : n_tiles % 8 == 0 ? 1 : 0;
+        // a step of the tile is NTHREADS / 8 rows, whole steps only: the shapes of eight and sixteen wavefronts take
+        // D_in that are multiples of 64 and of 128; 160 or 224 rows stay with four wavefronts (steps of 32 rows)
+        const bool steps64 = a.D % 64 == 0, steps128 = a.D % 128 == 0;
         if (a.D <= 128) launch_resident<MODE, Q, 8, 256, 4>(b, st);
-        else if (tv == 12) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(b, st);
-        else if (streams_from_hbm) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(b, st);
-        else if (tv == 8 || Q == Q_GENERAL || MODE == CONCRETIZE)
+        else if (tv == 12 && steps128) launch_resident<MODE, Q, 8, 1024, 2, 8, false>(b, st);
+        else if (streams_from_hbm && steps128) launch_resident<MODE, Q, 8, 1024, 2, 8, true>(b, st);
+        else if (tv == 8 || Q == Q_GENERAL || MODE == CONCRETIZE || !steps64)
             launch_resident<MODE, Q, 8, 256, 8, (Q == Q_GENERAL ? 3 : 4)>(b, st);     // a general exponent needs more registers than 128
         else if (MODE == TANH) launch_resident<MODE, Q, 8, 512, 4, 6, false, 6>(b, st);
         else launch_resident<MODE, Q, 8, 512, 4, 4, false, 4>(b, st);

@@ -71,6 +71,24 @@ def test_activation_small_shapes(kind, p, layout):
 
 
 @pytest.mark.parametrize("kind", ["relu", "tanh", "exp"])
+@pytest.mark.parametrize("knob", [0, 7, 12])
+def test_register_resident_tiles_take_whole_steps_of_rows_only(kind, knob):
+    """D_in between 128 and 256 that is a multiple of 32 but not of 64 (160, 224), or of 64 but not of 128 (192): a
+    step of the eight-wavefront tile is 64 rows and one of the sixteen-wavefront tile (knobs 7 and 12, and objects
+    beyond the memory-side cache) 128, and a tile must not reach into the rows of the next position.  Regression:
+    160 rows on the eight-wavefront tile read and overwrote 32 rows of the neighbouring position."""
+    from faith_amd import _lib
+    g = torch.Generator().manual_seed(17)
+    _lib.call("faith_tune_set", 0, knob)
+    try:
+        for (L, D, H, words) in [(3, 160, 64, 1), (5, 224, 96, 2), (2, 192, 64, 1), (4, 160, 32, 5), (3, 256, 64, 2)]:
+            x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+            check(kind, x, 2.0, 0.05, words)
+    finally:
+        _lib.call("faith_tune_set", 0, 0)
+
+
+@pytest.mark.parametrize("kind", ["relu", "tanh", "exp"])
 @pytest.mark.parametrize("p", [2.0, INF, 1.0, 3.0])
 def test_transposed_rows_of_any_length_stay_in_registers(kind, p):
     """The transposed layout (what the reference's adapters hand over) keeps rows of up to 1024 coefficients in
