@@ -37,6 +37,20 @@ def test_random_relaxation_shapes(seed):
     T_act.check(pick(rng, "relu", "tanh"), x, pick(rng, *PS), 0.05, words, pick(rng, "natural", "natural", "transposed"))
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_relaxation_shapes_on_the_register_resident_tiles(seed):
+    """D_in and H multiples of 32 (the register-resident kernels' territory, which uniformly drawn sizes rarely hit),
+    several positions, so that a tile that reaches past its own rows lands in a neighbour's."""
+    rng = random.Random(7000 + seed)
+    g = torch.Generator().manual_seed(8000 + seed)
+    D = dims(rng, 32, pick(rng, 256, 256, 512, 1024), 32)
+    words = pick(rng, 1, 1, 2, 4)
+    H = dims(rng, 32, 192, 32)
+    L = rng.randrange(2, 7)
+    x = rand_bounds(g, 1, L, D, H, ordered=True, sw=0.2, sb=1.0, gap_w=0.02, gap_b=0.5)
+    T_act.check(pick(rng, "relu", "tanh"), x, pick(rng, *PS), 0.05, words, pick(rng, "natural", "natural", "transposed"))
+
+
 @pytest.mark.parametrize("seed", range(20))
 def test_random_linear_shapes(seed):
     rng = random.Random(3000 + seed)
