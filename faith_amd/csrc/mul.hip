@@ -163,8 +163,13 @@ __global__ void __launch_bounds__(NTHREADS) mul_natural(const MulArgs a) {
                     ol.set(v, (al[v] > 0.f ? xl : xu) * al[v] + (bt[v] > 0.f ? yl : yu) * bt[v]);
                     ou.set(v, (au[v] > 0.f ? xu : xl) * au[v] + (bt[v] > 0.f ? yu : yl) * bt[v]);
                 }
-                ol.store(a.zlw + off);
-                ou.store(a.zuw + off);
+                if (VEC == 4 && a.H % 16 != 0) {     // rows that share 64-byte sectors with their neighbours: through the L2 (see Vec::store_cached; [128, 256, 300]: 76 -> 64 us)
+                    ol.store_cached(a.zlw + off);
+                    ou.store_cached(a.zuw + off);
+                } else {
+                    ol.store(a.zlw + off);
+                    ou.store(a.zuw + off);
+                }
             }
         }
     }
