@@ -970,6 +970,18 @@ void dispatch_natural(const ActArgs &a, hipStream_t st) {
     }
     // straight-line kernel for the common shape: 32-neuron tiles, 32 rows in flight, up to 8 rows a thread
     const int tv = faith::tune_get(FAITH_TUNE_ACT_VARIANT);
+    // 256 < D_in <= 1024 in whole steps of the tile (64 rows with eight wavefronts, 128 with sixteen; eight rows a
+    // thread): the same straight-line kernel, where the general one below walks its tile with row and column
+    // predicates -- same bits, [128, 512, 512] 110 -> 86 us, [32, 768, 768] 75 -> 50 us, [128, 1024, 512] 224 -> 203 us
+    // (knob 9 keeps the general kernel)
+    if constexpr (MODE != CONCRETIZE && Q != Q_GENERAL) {
+        if (tv == 0 && a.rows2 == 0 && a.H % 32 == 0 && a.D > 256 && a.D <= 1024) {
+            ActArgs b = a;
+            b.remap = a.rows % 8 == 0 ? 2 : 0;
+            if (a.D <= 512 && a.D % 64 == 0) { launch_resident<MODE, Q, 8, 512, 8, 4, false, 4>(b, st); return; }
+            if (a.D % 128 == 0) { launch_resident<MODE, Q, 8, 1024, 8, 4, false, 4>(b, st); return; }
+        }
+    }
     if (tv != 9 && a.rows2 == 0 && a.H % 32 == 0 && a.D % 32 == 0 && a.D <= 256) {
         // Tile order (ActArgs::remap): the hardware deals consecutive workgroups to the eight XCDs in turn, so with
         // tiles numbered along a row every XCD touches every row of the object at once; with whole rows dealt to the
