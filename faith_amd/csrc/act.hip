@@ -211,7 +211,7 @@ __global__ void __launch_bounds__(NTHREADS) act_natural(const ActArgs a) {
     constexpr int TH = TPR * VEC;
     constexpr int RG = NTHREADS / TPR;
     constexpr int NW = NTHREADS / WAVE;
-    static_assert(TH <= WAVE && TPR <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
+    static_assert(TH <= WAVE && TPR <= WAVE && NW >= 4, "per-neuron stages use one lane per neuron in wavefronts 0 ... 3");
     extern __shared__ float smem[];
     float *part = smem;                       // [words][NW][2][TH] per-wavefront partial norms
     float *s_lu = part + a.words * NW * 2 * TH;   // [2][TH] concrete interval
@@ -441,7 +441,7 @@ __device__ __forceinline__ void resident_partials(const ActArgs &a, const Vec<VE
 template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE = 4, bool NTL = false, int MAXW = 8>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE, MAXW))) act_resident(const ActArgs a) {
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
-    static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
+    static_assert(TH <= WAVE && NW >= 4, "per-neuron stages use one lane per neuron in wavefronts 0 ... 3");
     extern __shared__ float smem[];
     float *part = smem;                           // [words][NW][2][TH] per-wavefront partial norms
     float *s_lu = part + a.words * NW * 2 * TH;   // [2][TH] concrete interval
@@ -526,7 +526,7 @@ template <int MODE, int Q, int TPR, int NTHREADS, int RPT, int WPE>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(WPE))) act_pipelined(const ActArgs a, const int n_tiles) {
     static_assert(MODE != CONCRETIZE, "a read-only pass has no phases to overlap");
     constexpr int VEC = 4, TH = TPR * VEC, RG = NTHREADS / TPR, NW = NTHREADS / WAVE;
-    static_assert(TH <= WAVE && NW >= 3, "per-neuron stages use one lane per neuron in waves 0..2");
+    static_assert(TH <= WAVE && NW >= 4, "per-neuron stages use one lane per neuron in wavefronts 0 ... 3");
     extern __shared__ float smem[];
     float *part = smem;                           // [words][NW][2][TH] per-wavefront partial norms
     float *s_lu = part + a.words * NW * 2 * TH;   // [2][TH] concrete interval
